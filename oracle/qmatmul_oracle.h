@@ -1,0 +1,112 @@
+/*
+ * TEST INFRASTRUCTURE ONLY.  CPU restatement of the antfly inference engine's
+ * own CPU block-quantized matmul (GGUF Q4_0 / Q8_0 `linearNoBias`), used as the
+ * checker for the HIP path.  Nothing the product ships may call into this file:
+ * only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg load it.
+ *
+ * Reference files are cited as INF = zig/pkg/inference/src in the reference
+ * tree.  Every function here is pinned by the reference's own known-answer
+ * tests (re-encoded under tests/golden/) plus closed forms / brute force in
+ * tests/test_oracle_*.py; no function is "parity unpinned".
+ */
+#ifndef ANTFLY_QMATMUL_ORACLE_H
+#define ANTFLY_QMATMUL_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Block geometry, INF/gguf/tensor_types.zig:160-219. */
+enum { AFO_FMT_Q4_0 = 2, AFO_FMT_Q8_0 = 8 }; /* GGUF tensor-type ids */
+enum { AFO_BLOCK_VALUES = 32, AFO_Q4_0_BLOCK_BYTES = 18, AFO_Q8_0_BLOCK_BYTES = 34 };
+
+/* Which f32 association the Q4_0 activation-quantized apply uses for one term.
+ * The reference mixes both depending on row pairing and thread plan
+ * (INF/ops/native_compute.zig:23427-23775). */
+enum { AFO_ASSOC_PAIR = 0 /* (sx*sw)*dot */, AFO_ASSOC_SINGLE = 1 /* sx*(sw*dot + 0*sum) */ };
+
+size_t afo_block_bytes(int fmt);                     /* 18 / 34, 0 if unknown */
+size_t afo_byte_len(int fmt, size_t n_values);       /* tensor_types.byteLen */
+
+/* INF/gguf/quant_codec.zig:35-39 (decode) and the f32->f16 cast used by the
+ * weight quantizers (round-to-nearest-even, subnormals kept). */
+float    afo_fp16_to_f32(uint16_t bits);
+uint16_t afo_f32_to_fp16(float value);
+
+/* Weight quantizers, quant_codec.zig:601-623 (Q8_0), :895-910,:1261-1265 (Q4_0). */
+void afo_quantize_q8_0_block(const float *x32, uint8_t *out34);
+void afo_quantize_q4_0_block(const float *x32, uint8_t *out18);
+/* Dequantizers, quant_codec.zig:1877-1895 (Q8_0), :1918-1942 (Q4_0). */
+int afo_dequantize(int fmt, const uint8_t *raw, size_t n_blocks, float *out);
+
+/* Prepared int8 view of one weight block: Q8_0 -> the 32 int8 as stored,
+ * Q4_0 -> nibble-8 in ggml order (native_compute.zig:8408-8413,:8434-8457). */
+void afo_block_values_i8(int fmt, const uint8_t *raw_block, int8_t *out32, float *scale);
+
+/* Activation quantizer, native_compute.zig:11998-12028 and :23799-23832.
+ * q: rows*in_dim int8, scales: rows*(in_dim/32) f32, sums (may be NULL). */
+void afo_quantize_activation_rows(const float *x, size_t rows, size_t in_dim,
+                                  int8_t *q, float *scales, int32_t *sums);
+
+/* int32 block dot, native_compute.zig:12140-12151. */
+int32_t afo_dot_i8_block(const int8_t *a32, const int8_t *b32);
+
+/* All int32 block dots of the activation-quantized route:
+ * dots[(r*out_dim + o)*row_blocks + b].  Returns 0 on success. */
+int afo_block_dots(int fmt, const float *x, const uint8_t *w_raw, size_t rows,
+                   size_t in_dim, size_t out_dim, int32_t *dots);
+
+/* Route gate, native_compute.zig:3410-3419: activation quantization is used
+ * iff out_dim >= 512 && in_dim/32 >= 3. */
+int afo_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim);
+
+/* Route A (activation-quantized) applies over output columns [o0,o1).
+ * Q8_0: native_compute.zig:13304-13478.  Q4_0: :23427-23775 (use_mr4 = false). */
+int afo_linear_act_range(int fmt, const int8_t *qx, const float *sx, const int32_t *sums,
+                         const uint8_t *w_raw, float *y, size_t rows, size_t in_dim,
+                         size_t out_dim, size_t o0, size_t o1);
+/* Same but one fixed association for every term (test helper). */
+int afo_linear_act_assoc(int fmt, int assoc, const int8_t *qx, const float *sx,
+                         const uint8_t *w_raw, float *y, size_t rows, size_t in_dim,
+                         size_t out_dim);
+
+/* Route B (f32 activations), native_compute.zig:29919-29963, :11639-11672,
+ * :17472-17600. */
+int afo_linear_f32(int fmt, const float *x, const uint8_t *w_raw, float *y,
+                   size_t rows, size_t in_dim, size_t out_dim);
+
+/* The engine's op: picks route A or B with the reference gate, runs on
+ * `workers` threads with the reference's split policy
+ * (native_compute.zig:9756-9838; pool cap 8).  workers<=1 -> serial.
+ * Errors: -1 shape (in_dim%32), -2 unknown format. */
+int afo_linear_no_bias(int fmt, const float *x, const uint8_t *w_raw, float *y,
+                       size_t rows, size_t in_dim, size_t out_dim, int workers);
+
+/* Route A in double precision (no f32 rounding after the int dot); bounds the
+ * f32 accumulation error of any evaluation order. */
+int afo_linear_act_f64(int fmt, const float *x, const uint8_t *w_raw, double *y,
+                       size_t rows, size_t in_dim, size_t out_dim);
+
+/* Thread plan the reference would pick: returns worker count and sets
+ * *column_split (1 = split output columns, 0 = split rows). */
+int afo_thread_plan(size_t rows, size_t in_dim, size_t out_dim, int max_workers,
+                    int cpu_count, int *column_split);
+
+/* Timing path for the CPU baseline: weights unpacked once to int8 + f32 scale
+ * (what prepareNativeQuantizedStorage does at load time,
+ * native_compute.zig:8130-8204), then activation quantization + 2-row x 4-col
+ * register tiles + the reference's thread split on every call.  Every term uses
+ * (sx*sw)*dot; tests hold it to the faithful path above. */
+typedef struct afo_prepared afo_prepared;
+afo_prepared *afo_prepare(int fmt, const uint8_t *w_raw, size_t out_dim, size_t in_dim);
+void afo_prepared_free(afo_prepared *p);
+int afo_linear_prepared(const afo_prepared *p, const float *x, float *y, size_t rows,
+                        int workers);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,335 @@
+"""Pins the CPU oracle against the reference's known-answer vectors and against
+what the mathematics fixes (closed forms, brute force, invariants).  No GPU."""
+import numpy as np
+import pytest
+
+from antfly_amd import synth
+from oracle import oracle as O
+
+Q4, Q8 = O.FMT_Q4_0, O.FMT_Q8_0
+
+
+def smoke_row(fmt, scale, value):
+    """Same bytes as the reference's smoke-row writers (ops/cuda/kernels.zig:2516-2531)."""
+    hb = np.array([scale], dtype=np.float16).view(np.uint8)
+    if fmt == Q8:
+        return np.concatenate([hb, np.full(32, value, dtype=np.int8).view(np.uint8)])
+    nib = (value + 8) & 0xF
+    return np.concatenate([hb, np.full(16, nib | (nib << 4), dtype=np.uint8)])
+
+
+# ---------------------------------------------------------------- geometry / fp16
+
+def test_block_sizes(kats):
+    assert O.lib().afo_block_bytes(Q4) == kats["block_sizes"]["q4_0"]["bytes"] == 18
+    assert O.lib().afo_block_bytes(Q8) == kats["block_sizes"]["q8_0"]["bytes"] == 34
+    assert O.lib().afo_block_bytes(12) == 0
+    assert O.lib().afo_byte_len(Q4, 4096 * 14336) == 33030144
+    assert O.lib().afo_byte_len(Q8, 4096 * 4096) == 17825792
+    assert O.lib().afo_byte_len(Q8, 33) == 0
+
+
+def test_fp16_reference_constants(kats):
+    for bits, want in kats["fp16_constants"]["cases"]:
+        assert O.fp16_to_f32(bits) == want
+
+
+def test_fp16_decode_all_bit_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = np.array([O.fp16_to_f32(int(b)) for b in bits], dtype=np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+
+
+def test_fp16_encode_matches_ieee_rne():
+    rng = np.random.default_rng(7)
+    vals = np.concatenate([
+        rng.standard_normal(20000).astype(np.float32) * 10.0 ** rng.integers(-9, 5, 20000),
+        np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32),  # exact halves
+        np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e9, 5.96e-8, 2.98e-8, 2.99e-8, 6.1e-5], np.float32),
+    ])
+    vals = vals[np.isfinite(vals)]
+    # midpoints between adjacent halves exercise ties-to-even
+    h = np.arange(0, 0x7BFF, 37, dtype=np.uint16)
+    mid = (h.view(np.float16).astype(np.float64) + (h + 1).astype(np.uint16).view(np.float16).astype(np.float64)) / 2
+    vals = np.concatenate([vals, mid.astype(np.float32)])
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    got = np.array([O.f32_to_fp16(float(v)) for v in vals], dtype=np.uint16)
+    assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- block codecs
+
+def test_smoke_row_writer_layout(kats):
+    k = kats["smoke_row_writer"]
+    r8 = smoke_row(Q8, k["scale"], k["value"])
+    assert list(r8[:2]) == k["q8_0_bytes_head"] and set(r8[2:]) == {k["q8_0_fill"]} and r8.size == 34
+    r4 = smoke_row(Q4, k["scale"], k["value"])
+    assert list(r4[:2]) == k["q4_0_bytes_head"] and set(r4[2:]) == {k["q4_0_fill"]} and r4.size == 18
+
+
+def test_q4_0_nibble_order_and_offset(kats):
+    k = kats["q4_0_nibble_order"]
+    blk = np.full(18, k["fill_byte"], dtype=np.uint8)
+    blk[0:2] = np.array([k["scale_bits"]], dtype=np.uint16).view(np.uint8)
+    blk[2], blk[3] = k["qs0"], k["qs1"]
+    deq = O.dequantize(Q4, blk)
+    for idx, want in k["dequant"].items():
+        assert deq[int(idx)] == want
+    x = np.zeros((1, 32), dtype=np.float32)
+    x[0, k["input_ones_at"]] = 1.0
+    y = O.linear_f32(Q4, x, blk, 1, 32, 1)
+    assert abs(y[0, 0] - k["expected"]) <= k["tolerance_abs"]
+    v, s = O.block_values_i8(Q4, blk)
+    assert s == 1.0 and v[0] == -8 and v[1] == -6 and v[16] == -7 and v[17] == -5 and v[5] == 0
+
+
+@pytest.mark.parametrize("name,fmt", [("q8_0_direct", Q8), ("q4_0_direct", Q4)])
+def test_direct_matmul_kats(kats, name, fmt):
+    k = kats[name]
+    rows = []
+    for r in k["rows"]:
+        hb = np.array([r["scale_bits"]], dtype=np.uint16).view(np.uint8)
+        if fmt == Q8:
+            rows.append(np.concatenate([hb, np.full(32, r["q"], np.int8).view(np.uint8)]))
+        else:
+            rows.append(np.concatenate([hb, np.full(16, r["fill_byte"], np.uint8)]))
+    w = np.concatenate(rows)
+    x = np.full((1, 32), k["input_fill"], dtype=np.float32)
+    y = O.linear_f32(fmt, x, w, 1, 32, k["out_dim"])
+    assert np.allclose(y[0], k["expected"], atol=k["tolerance_abs"], rtol=0)
+    # the engine op takes the same (f32) route at this shape
+    assert not O.uses_activation_quant(1, 32, k["out_dim"])
+    assert np.array_equal(O.linear_no_bias(fmt, x, w, 1, 32, k["out_dim"]), y)
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_gpu_smoke_kat_on_oracle(kats, fmt):
+    k = kats["gpu_smoke"]
+    x = np.stack([np.arange(1, 33), -np.arange(1, 33)]).astype(np.float32)
+    w = np.concatenate([smoke_row(fmt, r["scale"], r["value"]) for r in k["weight_rows"]])
+    y = O.linear_no_bias(fmt, x, w, k["rows"], k["in_dim"], k["out_dim"])
+    assert np.allclose(y.reshape(-1), k["expected"], atol=k["tolerance_abs"], rtol=0)
+
+
+def test_weight_quantizers_closed_form(kats):
+    rng = np.random.default_rng(3)
+    for _ in range(50):
+        x = (rng.standard_normal(32) * rng.uniform(1e-3, 30)).astype(np.float32)
+        # Q8_0: scale = max|x|/127 stored as fp16, q = round-half-away(x * (1/scale)) clamped
+        raw = O.quantize_weights(Q8, x)
+        scale32 = np.float32(np.abs(x).max()) / np.float32(127.0)
+        assert raw[:2].view(np.float16)[0] == np.float16(scale32)
+        inv = np.float32(1.0) / scale32
+        t = x * inv
+        want = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int8)
+        assert np.array_equal(raw[2:].view(np.int8), want)
+        assert np.abs(want).max() == 127
+        # Q4_0: scale = max|x|/8 >= 0, q = clamp(round(x/scale) + 8, 0, 15), lo | hi<<4
+        raw4 = O.quantize_weights(Q4, x)
+        s4 = np.float32(np.abs(x).max()) / np.float32(8.0)
+        assert raw4[:2].view(np.float16)[0] == np.float16(s4)
+        t4 = x * (np.float32(1.0) / s4)
+        q4 = np.clip(np.sign(t4) * np.floor(np.abs(t4) + np.float32(0.5)) + 8, 0, 15).astype(np.uint8)
+        assert np.array_equal(raw4[2:], q4[:16] | (q4[16:] << 4))
+        deq = O.dequantize(Q4, raw4)
+        assert np.abs(deq - x).max() <= kats["quantizer_roundtrip"]["q4_0_tolerance"] * float(s4)
+    z = np.zeros(32, np.float32)
+    r8, r4 = O.quantize_weights(Q8, z), O.quantize_weights(Q4, z)
+    assert r8[:2].view(np.float16)[0] == 1.0 and not r8[2:].any()
+    assert r4[:2].view(np.float16)[0] == 1.0 and set(r4[2:]) == {0x88}
+    unit = np.concatenate([np.array([0x3C00], np.uint16).view(np.uint8), np.ones(32, np.uint8)])
+    assert np.array_equal(O.dequantize(Q8, unit), np.ones(32, np.float32))
+
+
+# ---------------------------------------------------------------- activation quantizer
+
+def test_activation_quantizer_invariants_and_rounding():
+    x = synth.activations(11, 3, 256)
+    x[1, 32:64] = 0.0  # zero block
+    q, s, sums = O.quantize_activation_rows(x, 3, 256)
+    blocks = x.reshape(3, 8, 32)
+    max_abs = np.abs(blocks).max(axis=2)
+    want_s = np.where(max_abs == 0, np.float32(1.0), max_abs / np.float32(127.0)).astype(np.float32)
+    assert np.array_equal(s, want_s)
+    assert np.abs(q).max() <= 127
+    qb = q.reshape(3, 8, 32)
+    assert np.all(np.abs(qb).max(axis=2)[max_abs > 0] == 127)
+    assert not qb[1, 1].any() and s[1, 1] == 1.0
+    assert np.array_equal(sums, qb.astype(np.int32).sum(axis=2))
+    inv = np.where(max_abs == 0, np.float32(0.0), np.float32(1.0) / want_s).astype(np.float32)
+    t = blocks * inv[:, :, None]
+    want_q = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int8)
+    assert np.array_equal(qb, want_q)
+    # ties round away from zero: max = 127 makes scale = 1 and inv = 1 exactly
+    blk = np.zeros((1, 32), np.float32)
+    blk[0, :7] = [127.0, 0.5, -0.5, 1.5, -1.5, 126.5, -2.5]
+    q2, s2, _ = O.quantize_activation_rows(blk, 1, 32)
+    assert s2[0, 0] == 1.0
+    assert list(q2[0, :7]) == [127, 1, -1, 2, -2, 127, -3]
+
+
+def test_i8_dot_reference_pattern_and_brute_force(kats):
+    i = np.arange(32)
+    x = ((i % 17) - 8).astype(np.int8)
+    w = (((5 * i + 3) % 19) - 9).astype(np.int8)
+    assert O.dot_i8_block(x, w) == int((x.astype(np.int64) * w.astype(np.int64)).sum())
+    rng = np.random.default_rng(5)
+    for _ in range(200):
+        a = rng.integers(-128, 128, 32).astype(np.int8)
+        b = rng.integers(-128, 128, 32).astype(np.int8)
+        assert O.dot_i8_block(a, b) == int((a.astype(np.int64) * b.astype(np.int64)).sum())
+    full = np.full(32, -127, np.int8)
+    assert O.dot_i8_block(full, full) == 516128  # largest |dot| the quantizers can produce
+
+
+# ---------------------------------------------------------------- matmuls
+
+def _numpy_route_a(fmt, x, w_raw, rows, in_dim, out_dim):
+    """float64 closed form: sum_b sx*sw*dot_b with the quantizers restated in numpy."""
+    kb = in_dim // 32
+    bb = O.BLOCK_BYTES[fmt]
+    wb = np.asarray(w_raw, np.uint8).reshape(out_dim, kb, bb)
+    sw = wb[:, :, :2].copy().view(np.float16).astype(np.float64).reshape(out_dim, kb)
+    if fmt == Q8:
+        qw = wb[:, :, 2:].view(np.int8).astype(np.int64)
+    else:
+        qs = wb[:, :, 2:]
+        qw = np.concatenate([(qs & 0xF).astype(np.int64) - 8, (qs >> 4).astype(np.int64) - 8], axis=2)
+    blocks = x.reshape(rows, kb, 32)
+    max_abs = np.abs(blocks).max(axis=2)
+    sx = np.where(max_abs == 0, np.float32(1), max_abs / np.float32(127)).astype(np.float32)
+    inv = np.where(max_abs == 0, np.float32(0), np.float32(1) / sx).astype(np.float32)
+    t = blocks * inv[:, :, None]
+    qx = np.clip(np.sign(t) * np.floor(np.abs(t) + np.float32(0.5)), -127, 127).astype(np.int64)
+    dots = np.einsum("rbk,obk->rob", qx, qw)
+    y = np.einsum("rob,rb,ob->ro", dots.astype(np.float64), sx.astype(np.float64), sw)
+    return dots, y
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+@pytest.mark.parametrize("rows", [1, 2, 3, 5])
+def test_route_a_matches_independent_numpy_closed_form(fmt, rows):
+    in_dim, out_dim = 160, 37
+    x = synth.activations(21 + rows, rows, in_dim)
+    w = synth.weights(fmt, 99, out_dim, in_dim)
+    dots_np, y_np = _numpy_route_a(fmt, x, w, rows, in_dim, out_dim)
+    assert np.array_equal(O.block_dots(fmt, x, w, rows, in_dim, out_dim), dots_np)
+    y64 = O.linear_act_f64(fmt, x, w, rows, in_dim, out_dim)
+    assert np.allclose(y64, y_np, rtol=1e-12, atol=0)
+    qx, sx, sums = O.quantize_activation_rows(x, rows, in_dim)
+    y = O.linear_act_range(fmt, qx, sx, sums, w, rows, in_dim, out_dim, 0, out_dim)
+    scale = np.abs(y_np).max()
+    assert np.abs(y - y_np).max() <= 2e-6 * scale
+    # every association / column range the reference can take agrees to f32 rounding
+    for assoc in (O.ASSOC_PAIR, O.ASSOC_SINGLE):
+        ya = O.linear_act_assoc(fmt, assoc, x, w, rows, in_dim, out_dim)
+        assert np.abs(ya - y_np).max() <= 2e-6 * scale
+    yr = np.zeros_like(y)
+    for o0, o1 in [(0, 5), (5, 18), (18, 37)]:
+        O.linear_act_range(fmt, qx, sx, sums, w, rows, in_dim, out_dim, o0, o1, y=yr)
+    assert np.abs(yr - y).max() <= 1e-6 * scale
+    if fmt == Q8:
+        assert np.array_equal(yr, y)  # Q8_0 has one association on every path
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_route_b_equals_dequantize_then_matmul(fmt, kats):
+    k = kats["q4_0_multirow_vs_dense"]
+    rows, in_dim, out_dim = k["rows"], k["in_dim"], k["out_dim"]
+    bb = O.BLOCK_BYTES[fmt]
+    n = out_dim * (in_dim // 32) * bb
+    w = ((37 * np.arange(n) + 11) & 0xFF).astype(np.uint8)
+    w.reshape(-1, bb)[:, 0] = 0x00
+    w.reshape(-1, bb)[:, 1] = 0x3C
+    x = (synth.uniform01(0x5EED1234, 0, rows * in_dim) * 2 - 1).astype(np.float32).reshape(rows, in_dim)
+    dense = O.dequantize(fmt, w).reshape(out_dim, in_dim).astype(np.float64)
+    want = x.astype(np.float64) @ dense.T
+    got = O.linear_f32(fmt, x, w, rows, in_dim, out_dim)
+    assert np.abs(got - want).max() <= k["tolerance_abs"]
+
+
+def test_activation_quant_route_stays_close_to_f32_route(kats):
+    k = kats["act_quant_vs_f32"]
+    rows, in_dim, out_dim = k["rows"], k["in_dim"], k["out_dim"]
+    x = (((np.arange(rows * in_dim) % 17) - 8) / np.float32(9.0)).astype(np.float32).reshape(rows, in_dim)
+    dense = (((np.arange(out_dim * in_dim) % 23) - 11) / np.float32(32.0)).astype(np.float32)
+    w = O.quantize_weights(Q8, dense)
+    exact = O.linear_f32(Q8, x, w, rows, in_dim, out_dim)
+    qx, sx, sums = O.quantize_activation_rows(x, rows, in_dim)
+    quant = O.linear_act_range(Q8, qx, sx, sums, w, rows, in_dim, out_dim, 0, out_dim)
+    assert np.abs(quant - exact).max() <= k["tolerance_abs"]
+    assert np.abs(quant - exact).max() > 0  # they are different computations
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_engine_op_route_gate_and_thread_plans(fmt):
+    # below the gate: f32 route
+    x = synth.activations(1, 2, 64)
+    w = synth.weights(fmt, 2, 600, 64)
+    assert not O.uses_activation_quant(2, 64, 600)
+    assert np.array_equal(O.linear_no_bias(fmt, x, w, 2, 64, 600), O.linear_f32(fmt, x, w, 2, 64, 600))
+    # at the gate: activation-quantized route, any thread plan within f32 rounding
+    rows, in_dim, out_dim = 5, 96, 640
+    x = synth.activations(4, rows, in_dim)
+    w = synth.weights(fmt, 5, out_dim, in_dim)
+    assert O.uses_activation_quant(rows, in_dim, out_dim)
+    y1 = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim, workers=1)
+    y8 = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim, workers=8)
+    y64 = O.linear_act_f64(fmt, x, w, rows, in_dim, out_dim)
+    scale = np.abs(y64).max()
+    assert np.abs(y1 - y64).max() <= 2e-6 * scale and np.abs(y8 - y64).max() <= 2e-6 * scale
+    if fmt == Q8:
+        assert np.array_equal(y1, y8)
+    for r in (1, 2):
+        ya = O.linear_no_bias(fmt, x[:r], w, r, in_dim, out_dim, workers=1)
+        yb = O.linear_no_bias(fmt, x[:r], w, r, in_dim, out_dim, workers=8)
+        assert np.abs(ya - yb).max() <= 1e-6 * scale
+    # errors
+    with pytest.raises(ValueError):
+        O.linear_no_bias(fmt, x, w, 1, 33, 4)
+    with pytest.raises(ValueError):
+        O.linear_no_bias(12, x, w, 1, 32, 4)
+
+
+def test_thread_plan_matches_reference_policy():
+    assert O.thread_plan(1, 4096, 14336) == (8, True)     # decode: 8 column chunks
+    assert O.thread_plan(2, 4096, 14336) == (8, True)
+    assert O.thread_plan(4, 4096, 14336) == (4, False)    # rows > 2: row split, min(8, rows)
+    assert O.thread_plan(5, 14336, 4096) == (5, False)
+    assert O.thread_plan(512, 4096, 4096) == (8, False)
+    assert O.thread_plan(1, 4096, 300) == (1, False)      # out < 512 and one row: serial
+    assert O.thread_plan(1, 4096, 576) == (8, True)       # 576/64 = 9 -> capped at 8
+    assert O.thread_plan(1, 4096, 512, max_workers=8, cpu_count=4) == (4, True)
+    assert O.thread_plan(1, 32, 100) == (1, False)        # below the 16384 work-unit floor
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_timing_path_matches_faithful_path(fmt):
+    rows, in_dim, out_dim = 5, 256, 515
+    x = synth.activations(8, rows, in_dim)
+    w = synth.weights(fmt, 9, out_dim, in_dim)
+    p = O.Prepared(fmt, w, out_dim, in_dim)
+    want = O.linear_act_assoc(fmt, O.ASSOC_PAIR, x, w, rows, in_dim, out_dim)
+    for workers in (1, 8):
+        assert np.array_equal(p.linear(x, rows, workers=workers), want)
+    assert np.array_equal(p.linear(x[:1], 1, workers=8), want[:1])
+    p.close()
+
+
+def test_synth_is_chunk_invariant_and_in_range():
+    a = synth.splitmix64(42, 0, 1000)
+    b = np.concatenate([synth.splitmix64(42, 0, 333), synth.splitmix64(42, 333, 667)])
+    assert np.array_equal(a, b)
+    w8 = synth.weights(Q8, 1, 8, 64).reshape(-1, 34)
+    q = w8[:, 2:].view(np.int8)
+    assert q.min() >= -127 and q.max() <= 127
+    s = w8[:, :2].copy().view(np.float16).astype(np.float32)
+    assert (s >= 0).all() and s.max() < 0.02 * 6 / 127
+    w4 = synth.weights(Q4, 1, 8, 64)
+    assert w4.size == synth.weight_bytes(Q4, 8, 64) == 8 * 2 * 18
+    x = synth.activations(3, 64, 512)
+    assert abs(float(x.mean())) < 0.02 and abs(float(x.std()) - 1.0) < 0.02
