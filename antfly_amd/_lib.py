@@ -1,0 +1,201 @@
+"""Loads libantfly_hip_qmatmul.so and declares its C ABI (include/antfly_hip_qmatmul.h).
+
+There is no fallback: if the library is missing, import fails loudly.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "lib", "libantfly_hip_qmatmul.so")
+
+# enum afhip_error
+OK = 0
+ERR_INVALID_STATE = -1
+ERR_UNSUPPORTED_TENSOR_TYPE = -2
+ERR_INVALID_SHAPE = -3
+ERR_WEIGHT_NOT_FOUND = -4
+ERR_OP_UNSUPPORTED = -5
+ERR_INVALID_PARTITION_PLAN = -6
+ERR_UNAVAILABLE = -7
+ERR_NO_DEVICES = -8
+ERR_OUT_OF_MEMORY = -9
+ERR_INVALID_ARGUMENT = -10
+ERR_SMOKE_MISMATCH = -11
+
+TYPE_F32, TYPE_Q4_0, TYPE_Q8_0 = 0, 2, 8
+LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
+DTYPE_F32, DTYPE_U8 = 0, 1
+
+
+class Buffer(C.Structure):
+    """afhip_buffer: a device allocation (ptr, len)."""
+
+    _fields_ = [("ptr", C.c_uint64), ("len", C.c_size_t)]
+
+
+class QuantPlan(C.Structure):
+    _fields_ = [
+        ("dispatch", C.c_uint8),
+        ("primitive", C.c_uint8),
+        ("op", C.c_uint8),
+        ("row_bucket", C.c_uint8),
+        ("format", C.c_uint16),
+        ("rows", C.c_size_t),
+        ("in_dim", C.c_size_t),
+        ("out_dim", C.c_size_t),
+    ]
+
+
+class OperatorPlan(C.Structure):
+    _fields_ = [("kind", C.c_int), ("quant_matmul", QuantPlan)]
+
+
+class PlannedRequest(C.Structure):
+    _fields_ = [
+        ("input", C.c_void_p),
+        ("weight", C.c_void_p),
+        ("rows", C.c_size_t),
+        ("in_dim", C.c_size_t),
+        ("out_dim", C.c_size_t),
+        ("operator_plan", OperatorPlan),
+    ]
+
+
+class DebugStats(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in (
+        "h2d_bytes", "d2h_bytes", "resident_weight_bytes", "pooled_buffers", "device_allocs",
+        "launches_mmv", "launches_small_batch", "launches_mm", "launches_f32_route",
+        "launches_activation_quant", "launches_prepare", "scratch_bytes")]
+
+
+# name -> (restype, argtypes); the loader test checks every one is exported.
+_sz, _vp, _i, _st = C.c_size_t, C.c_void_p, C.c_int, C.c_int
+SIGNATURES = {
+    "afhip_status_string": (C.c_char_p, [_st]),
+    "afhip_quant_matmul_select": (_i, [_sz, _sz, _sz, _i]),
+    "afhip_quant_matmul_plan": (None, [_sz, _sz, _sz, _i, C.POINTER(QuantPlan)]),
+    "afhip_quant_row_bucket": (_i, [_sz]),
+    "afhip_quant_format_from_tensor_type": (_i, [_i]),
+    "afhip_uses_activation_quant": (_i, [_sz, _sz, _sz]),
+    "afhip_linear_workspace_bytes": (_sz, [_i, _sz, _sz, _sz]),
+    "afhip_launch_linear_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_linear_q8_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
+    "afhip_launch_linear_q4_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
+    "afhip_launch_prepare_weight": (_st, [_vp, _i, Buffer, Buffer, _sz, _sz]),
+    "afhip_launch_quantize_activations": (_st, [_vp, Buffer, _sz, _sz, Buffer, Buffer, Buffer]),
+    "afhip_launch_block_dots": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
+    "afhip_compute_create": (_st, [C.POINTER(_vp)]),
+    "afhip_compute_destroy": (None, [_vp]),
+    "afhip_compute_backend_kind": (_i, [_vp]),
+    "afhip_compute_stream": (_vp, [_vp]),
+    "afhip_compute_synchronize": (_st, [_vp]),
+    "afhip_compute_device_name": (_st, [_vp, C.c_char_p, _sz]),
+    "afhip_compute_insert_weight_from_loaded": (_st, [_vp, C.c_char_p, _i, _vp, _sz, C.POINTER(C.c_int64), _sz, _i]),
+    "afhip_compute_insert_weight_f32": (_st, [_vp, C.c_char_p, _vp, C.POINTER(C.c_int64), _sz]),
+    "afhip_compute_get_weight": (_st, [_vp, C.c_char_p, C.POINTER(_vp)]),
+    "afhip_compute_from_float32": (_st, [_vp, _vp, _sz, C.POINTER(C.c_int32), _sz, C.POINTER(_vp)]),
+    "afhip_compute_to_float32": (_st, [_vp, _vp, _vp, _sz]),
+    "afhip_compute_wrap_device_f32": (_st, [_vp, C.c_uint64, C.POINTER(C.c_int64), _sz, C.POINTER(_vp)]),
+    "afhip_compute_free_tensor": (None, [_vp, _vp]),
+    "afhip_compute_eval_tensor": (_st, [_vp, _vp]),
+    "afhip_tensor_dtype": (_i, [_vp]),
+    "afhip_tensor_quant_type": (_i, [_vp]),
+    "afhip_tensor_layout": (_i, [_vp]),
+    "afhip_tensor_elem_count": (_sz, [_vp]),
+    "afhip_tensor_rank": (_sz, [_vp]),
+    "afhip_tensor_shape": (_st, [_vp, C.POINTER(C.c_int64), _sz]),
+    "afhip_tensor_device_ptr": (C.c_uint64, [_vp]),
+    "afhip_tensor_byte_len": (_sz, [_vp]),
+    "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "afhip_compute_linear_no_bias_planned": (_st, [_vp, C.POINTER(PlannedRequest), C.POINTER(_vp)]),
+    "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
+    "afhip_smoke_q8_0": (_st, []),
+    "afhip_smoke_q4_0": (_st, []),
+}
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is missing: build it with `make -C antfly_amd/csrc` "
+                "(or __graft_entry__.build()); there is no CPU fallback")
+        L = C.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(L, name)  # AttributeError if the library does not export it
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = L
+    return _lib
+
+
+class HipError(Exception):
+    """An error union member of the backend (negative) or a hipError_t (positive)."""
+
+    def __init__(self, status: int):
+        self.status = status
+        try:
+            self.name = lib().afhip_status_string(status).decode()
+        except Exception:  # pragma: no cover
+            self.name = str(status)
+        super().__init__(f"error.{self.name} ({status})")
+
+
+class InvalidHipState(HipError):
+    pass
+
+
+class UnsupportedTensorType(HipError):
+    pass
+
+
+class InvalidShape(HipError):
+    pass
+
+
+class WeightNotFound(HipError):
+    pass
+
+
+class HipOpUnsupported(HipError):
+    pass
+
+
+class InvalidPartitionPlan(HipError):
+    pass
+
+
+class HipUnavailable(HipError):
+    pass
+
+
+class NoHipDevices(HipError):
+    pass
+
+
+class HipSmokeMismatch(HipError):
+    pass
+
+
+_ERRORS = {
+    ERR_INVALID_STATE: InvalidHipState,
+    ERR_UNSUPPORTED_TENSOR_TYPE: UnsupportedTensorType,
+    ERR_INVALID_SHAPE: InvalidShape,
+    ERR_WEIGHT_NOT_FOUND: WeightNotFound,
+    ERR_OP_UNSUPPORTED: HipOpUnsupported,
+    ERR_INVALID_PARTITION_PLAN: InvalidPartitionPlan,
+    ERR_UNAVAILABLE: HipUnavailable,
+    ERR_NO_DEVICES: NoHipDevices,
+    ERR_SMOKE_MISMATCH: HipSmokeMismatch,
+}
+
+
+def check(status: int) -> None:
+    if status != OK:
+        raise _ERRORS.get(status, HipError)(status)

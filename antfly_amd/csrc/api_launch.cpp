@@ -1,0 +1,315 @@
+// C ABI, part 1: dispatch vocabulary (graph/quant_matmul.zig) and the
+// stream-ordered launchers (ops/cuda/kernels.zig:1221-1289).
+#include <hip/hip_runtime_api.h>
+
+#include <limits>
+
+#include "antfly_hip_qmatmul.h"
+#include "api_internal.h"
+#include "qmatmul_launch.h"
+
+namespace afhip {
+
+bool checked_mul(size_t a, size_t b, size_t* out) { return !__builtin_mul_overflow(a, b, out); }
+
+size_t block_bytes(int tensor_type) {
+    if (tensor_type == AFHIP_TYPE_Q4_0) return 18;
+    if (tensor_type == AFHIP_TYPE_Q8_0) return 34;
+    return 0;
+}
+
+static bool fits_u32(size_t v) { return v <= std::numeric_limits<uint32_t>::max(); }  // toU32, kernels.zig:2558-2563
+
+// Scratch layout: [qx int8 rows*in_dim | pad to 256][sx f32 rows*kb][sums i32 rows*kb]
+struct WorkspaceView {
+    int8_t* qx;
+    float* sx;
+    int* sums;
+    size_t bytes;
+};
+static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
+    const size_t kb = in_dim / 32;
+    const size_t q_bytes = (rows * in_dim + 255) / 256 * 256;
+    WorkspaceView v;
+    v.qx = reinterpret_cast<int8_t*>(base);
+    v.sx = reinterpret_cast<float*>(base + q_bytes);
+    v.sums = reinterpret_cast<int*>(base + q_bytes + rows * kb * 4);
+    v.bytes = q_bytes + rows * kb * 8;
+    return v;
+}
+
+// LDS the fused GEMV may use per workgroup; gfx950 has 160 KiB per CU.
+constexpr size_t kGemvLdsBudget = 96 * 1024;
+
+static int gemv_row_chunk(size_t rows, size_t in_dim) {
+    int chunk = rows < 8 ? static_cast<int>(rows) : 8;
+    while (chunk > 0 && gemv_fused_lds_bytes(chunk, static_cast<int>(in_dim)) > kGemvLdsBudget) --chunk;
+    return chunk;
+}
+
+static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t out_dim) {
+    (void)tensor_type;
+    (void)out_dim;
+    GemvTuning t;
+    const size_t lds = gemv_fused_lds_bytes(rows, static_cast<int>(in_dim));
+    t.threads = lds > 32 * 1024 ? 1024 : 512;
+    t.max_workgroups = lds > 64 * 1024 ? 256 : 512;
+    return t;
+}
+
+afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                         afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                         int dispatch, afhip_buffer dots, LaunchCounters* counters) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const size_t bb = block_bytes(tensor_type);
+    if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    const size_t kb = in_dim / 32;
+    size_t out_count, in_count, w_blocks, w_bytes, bytes;
+    if (!checked_mul(rows, out_dim, &out_count) || !checked_mul(rows, in_dim, &in_count) ||
+        !checked_mul(out_dim, kb, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes))
+        return AFHIP_ERR_INVALID_STATE;
+    const bool want_dots = dots.ptr != 0;
+    if (!want_dots) {
+        if (!checked_mul(out_count, 4, &bytes) || bytes > dst.len) return AFHIP_ERR_INVALID_STATE;
+    } else {
+        size_t n;
+        if (!checked_mul(out_count, kb, &n) || !checked_mul(n, 4, &bytes) || bytes > dots.len) return AFHIP_ERR_INVALID_STATE;
+    }
+    if (!checked_mul(in_count, 4, &bytes) || bytes > input.len) return AFHIP_ERR_INVALID_STATE;
+    if (w_bytes > weight.len) return AFHIP_ERR_INVALID_STATE;
+    if (out_count == 0) return AFHIP_OK;
+    if (!fits_u32(rows) || !fits_u32(in_dim) || !fits_u32(out_dim) || in_dim > 0x7fffffff || out_dim > 0x7fffffff ||
+        rows > 0x7fffffff)
+        return AFHIP_ERR_INVALID_STATE;
+    if ((!want_dots && dst.ptr == 0) || input.ptr == 0 || weight.ptr == 0) return AFHIP_ERR_INVALID_STATE;
+    // 128-bit activation loads; prepared weights are read with 128-bit loads, raw GGUF bytes with 16-bit loads
+    if (input.ptr % 16 != 0 || dst.ptr % 4 != 0 || dots.ptr % 4 != 0) return AFHIP_ERR_INVALID_STATE;
+    if (weight.ptr % (layout == AFHIP_LAYOUT_PREPARED ? 16 : 2) != 0) return AFHIP_ERR_INVALID_STATE;
+
+    float* y = reinterpret_cast<float*>(dst.ptr);
+    int* dot_out = reinterpret_cast<int*>(dots.ptr);
+    const float* x = reinterpret_cast<const float*>(input.ptr);
+    const uint8_t* w = reinterpret_cast<const uint8_t*>(weight.ptr);
+
+    // The block dots only exist on the activation-quantized route.
+    const bool route_a = want_dots || afhip_uses_activation_quant(rows, in_dim, out_dim);
+    if (!route_a) {
+        if (counters) counters->f32_route++;
+        hipError_t e = launch_linear_generic(stream, tensor_type, layout, false, y, nullptr, x, nullptr, nullptr, w,
+                                             static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
+
+    int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim,
+                                                                    afhip_quant_format_from_tensor_type(tensor_type));
+    const int chunk = gemv_row_chunk(rows, in_dim);
+    const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR;
+    if (fused_ok) {
+        // mmv / small_batch: rows <= 8 in one launch.  mm (rows >= 9): same kernel
+        // over 8-row slices until the MFMA GEMM takes over.
+        if (counters) {
+            if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+            else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+            else counters->mm++;
+        }
+        for (size_t r0 = 0; r0 < rows; r0 += static_cast<size_t>(chunk)) {
+            const int nr = rows - r0 < static_cast<size_t>(chunk) ? static_cast<int>(rows - r0) : chunk;
+            const GemvTuning tune = gemv_tuning(tensor_type, nr, in_dim, out_dim);
+            hipError_t e = launch_gemv_fused(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
+                                             want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, w, nr,
+                                             static_cast<int>(in_dim), static_cast<int>(out_dim), tune);
+            if (e != hipSuccess) return static_cast<afhip_status>(e);
+        }
+        return AFHIP_OK;
+    }
+
+    // Generic activation-quantized path: quantize into the caller's scratch first.
+    const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
+    if (workspace.ptr == 0 || workspace.len < ws.bytes || workspace.ptr % 16 != 0) return AFHIP_ERR_INVALID_STATE;
+    if (counters) {
+        counters->activation_quant++;
+        if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+        else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+        else counters->mm++;
+    }
+    hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx, ws.sx,
+                                               ws.sums);
+    if (e != hipSuccess) return static_cast<afhip_status>(e);
+    e = launch_linear_generic(stream, tensor_type, layout, true, want_dots ? nullptr : y, dot_out, nullptr, ws.qx, ws.sx,
+                              w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+}  // namespace afhip
+
+using namespace afhip;
+
+extern "C" {
+
+const char* afhip_status_string(afhip_status status) {
+    switch (status) {
+        case AFHIP_OK: return "ok";
+        case AFHIP_ERR_INVALID_STATE: return "InvalidHipState";
+        case AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE: return "UnsupportedTensorType";
+        case AFHIP_ERR_INVALID_SHAPE: return "InvalidShape";
+        case AFHIP_ERR_WEIGHT_NOT_FOUND: return "WeightNotFound";
+        case AFHIP_ERR_OP_UNSUPPORTED: return "HipOpUnsupported";
+        case AFHIP_ERR_INVALID_PARTITION_PLAN: return "InvalidPartitionPlan";
+        case AFHIP_ERR_UNAVAILABLE: return "HipUnavailable";
+        case AFHIP_ERR_NO_DEVICES: return "NoHipDevices";
+        case AFHIP_ERR_OUT_OF_MEMORY: return "OutOfMemory";
+        case AFHIP_ERR_INVALID_ARGUMENT: return "InvalidArgument";
+        case AFHIP_ERR_SMOKE_MISMATCH: return "HipSmokeMismatch";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorName(static_cast<hipError_t>(status));
+    return "unknown";
+}
+
+// ---- graph/quant_matmul.zig
+
+static size_t format_values_per_block(int format) {
+    switch (format) {  // Format.valuesPerBlock, :84-117
+        case AFHIP_FORMAT_Q4_0:
+        case AFHIP_FORMAT_Q8_0: return 32;
+        case AFHIP_FORMAT_F32: return 1;
+        default: return 0;
+    }
+}
+
+static bool valid_shape(size_t rows, size_t in_dim, size_t out_dim, int format) {  // validShape, :566-576
+    if (rows == 0 || in_dim == 0 || out_dim == 0) return false;
+    const size_t vpb = format_values_per_block(format);
+    if (vpb == 0) return false;
+    return in_dim % vpb == 0;
+}
+
+int afhip_quant_matmul_select(size_t rows, size_t in_dim, size_t out_dim, int format) {  // select, :263-268
+    if (!valid_shape(rows, in_dim, out_dim, format)) return AFHIP_DISPATCH_SCALAR;
+    if (rows >= 2 && rows <= 8) return AFHIP_DISPATCH_SMALL_BATCH;
+    if (rows >= 9) return AFHIP_DISPATCH_MM;
+    return AFHIP_DISPATCH_MMV;
+}
+
+int afhip_quant_row_bucket(size_t rows) {  // rowBucket, :558-564
+    if (rows == 0) return AFHIP_ROWS_0;
+    if (rows == 1) return AFHIP_ROWS_1;
+    if (rows <= 8) return AFHIP_ROWS_2_8;
+    if (rows <= 64) return AFHIP_ROWS_9_64;
+    return AFHIP_ROWS_65_PLUS;
+}
+
+void afhip_quant_matmul_plan(size_t rows, size_t in_dim, size_t out_dim, int format, afhip_quant_plan* out) {
+    if (!out) return;
+    const int d = afhip_quant_matmul_select(rows, in_dim, out_dim, format);
+    out->dispatch = static_cast<uint8_t>(d);
+    // primitiveForDispatch, :270-277
+    static const uint8_t prim[4] = {AFHIP_PRIM_SCALAR, AFHIP_PRIM_MAT_VEC, AFHIP_PRIM_MAT_VEC_EXT, AFHIP_PRIM_MAT_MAT};
+    out->primitive = prim[d];
+    // operatorForDispatch, :279-287: every format known here supports mul_mv / mul_mv_ext / mul_mm
+    const bool known = format == AFHIP_FORMAT_Q4_0 || format == AFHIP_FORMAT_Q8_0 || format == AFHIP_FORMAT_F32;
+    static const uint8_t op[4] = {AFHIP_OP_FALLBACK, AFHIP_OP_MUL_MV, AFHIP_OP_MUL_MV_EXT, AFHIP_OP_MUL_MM};
+    out->op = known ? op[d] : static_cast<uint8_t>(AFHIP_OP_FALLBACK);
+    out->row_bucket = static_cast<uint8_t>(afhip_quant_row_bucket(rows));
+    out->format = static_cast<uint16_t>(format);
+    out->rows = rows;
+    out->in_dim = in_dim;
+    out->out_dim = out_dim;
+}
+
+int afhip_quant_format_from_tensor_type(int tensor_type) {  // backend_contracts.zig:199-236
+    switch (tensor_type) {
+        case AFHIP_TYPE_Q4_0: return AFHIP_FORMAT_Q4_0;
+        case AFHIP_TYPE_Q8_0: return AFHIP_FORMAT_Q8_0;
+        case AFHIP_TYPE_F32: return AFHIP_FORMAT_F32;
+        default: return AFHIP_FORMAT_UNKNOWN;
+    }
+}
+
+int afhip_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim) {
+    (void)rows;
+    return out_dim >= 512 && in_dim / 32 >= 3;
+}
+
+// ---- launchers
+
+size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;
+    return workspace_view(0, rows, in_dim).bytes;
+}
+
+afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                                     afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim,
+                                     afhip_buffer workspace, int dispatch) {
+    return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr);
+}
+
+afhip_status afhip_launch_linear_q8_0_f32(void* stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight_raw,
+                                          size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace) {
+    return linear_impl(stream, AFHIP_TYPE_Q8_0, AFHIP_LAYOUT_RAW, dst, input, weight_raw, rows, in_dim, out_dim,
+                       workspace, -1, afhip_buffer{0, 0}, nullptr);
+}
+
+afhip_status afhip_launch_linear_q4_0_f32(void* stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight_raw,
+                                          size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace) {
+    return linear_impl(stream, AFHIP_TYPE_Q4_0, AFHIP_LAYOUT_RAW, dst, input, weight_raw, rows, in_dim, out_dim,
+                       workspace, -1, afhip_buffer{0, 0}, nullptr);
+}
+
+afhip_status afhip_launch_block_dots(void* stream, int tensor_type, int layout, afhip_buffer dots, afhip_buffer input,
+                                     afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim,
+                                     afhip_buffer workspace, int dispatch) {
+    if (dots.ptr == 0) return AFHIP_ERR_INVALID_STATE;
+    return linear_impl(stream, tensor_type, layout, afhip_buffer{0, 0}, input, weight, rows, in_dim, out_dim, workspace,
+                       dispatch, dots, nullptr);
+}
+
+afhip_status afhip_launch_prepare_weight(void* stream, int tensor_type, afhip_buffer dst, afhip_buffer src,
+                                         size_t out_dim, size_t in_dim) {
+    const size_t bb = block_bytes(tensor_type);
+    if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    size_t blocks, bytes;
+    if (!checked_mul(out_dim, in_dim / 32, &blocks) || !checked_mul(blocks, bb, &bytes)) return AFHIP_ERR_INVALID_STATE;
+    if (bytes > src.len || bytes > dst.len) return AFHIP_ERR_INVALID_STATE;
+    if (blocks == 0) return AFHIP_OK;
+    if (dst.ptr == 0 || src.ptr == 0 || dst.ptr % 16 != 0 || src.ptr % 2 != 0) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_prepare_weight(static_cast<hipStream_t>(stream), tensor_type,
+                                         reinterpret_cast<uint8_t*>(dst.ptr), reinterpret_cast<const uint8_t*>(src.ptr),
+                                         blocks);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_launch_quantize_activations(void* stream, afhip_buffer input, size_t rows, size_t in_dim,
+                                               afhip_buffer q, afhip_buffer scales, afhip_buffer sums) {
+    if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    size_t count, bytes;
+    if (!checked_mul(rows, in_dim, &count) || !checked_mul(count, 4, &bytes)) return AFHIP_ERR_INVALID_STATE;
+    const size_t nb = count / 32;
+    if (bytes > input.len || count > q.len || nb * 4 > scales.len) return AFHIP_ERR_INVALID_STATE;
+    if (sums.ptr != 0 && nb * 4 > sums.len) return AFHIP_ERR_INVALID_STATE;
+    if (count == 0) return AFHIP_OK;
+    if (rows > 0x7fffffff || in_dim > 0x7fffffff || input.ptr == 0 || q.ptr == 0 || scales.ptr == 0 ||
+        input.ptr % 16 != 0 || q.ptr % 4 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_quantize_activations(static_cast<hipStream_t>(stream),
+                                               reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
+                                               static_cast<int>(in_dim), reinterpret_cast<int8_t*>(q.ptr),
+                                               reinterpret_cast<float*>(scales.ptr), reinterpret_cast<int*>(sums.ptr));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {
+    if (n * 4 > dst.len || n * 2 > src.len) return AFHIP_ERR_INVALID_STATE;
+    if (n == 0) return AFHIP_OK;
+    if (dst.ptr == 0 || src.ptr == 0) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_decode_fp16(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr),
+                                      reinterpret_cast<const uint16_t*>(src.ptr), n);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+}  // extern "C"

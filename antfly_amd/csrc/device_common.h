@@ -1,0 +1,200 @@
+// Device-side building blocks shared by the gfx950 quantized-matmul kernels.
+// Wavefronts are 64 wide; every helper here assumes that.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace afhip {
+
+constexpr int kWave = 64;
+constexpr int kBlockValues = 32;  // weights per quant block (gguf/tensor_types.zig:160-219)
+constexpr int kQ4BlockBytes = 18;
+constexpr int kQ8BlockBytes = 34;
+
+// ---- fp16 scale decode (gguf/quant_codec.zig:35-39).  v_cvt_f32_f16 is exact
+// for every half, subnormals included.
+__device__ __forceinline__ float half_bits_to_f32(uint16_t bits) {
+    _Float16 h;
+    __builtin_memcpy(&h, &bits, 2);
+    return static_cast<float>(h);
+}
+
+// ---- signed 4 x int8 dot with int32 accumulate (v_dot4_i32_i8).
+__device__ __forceinline__ int dot4(int a, int b, int acc) {
+    return __builtin_amdgcn_sdot4(a, b, acc, false);
+}
+
+// ---- DPP lane exchanges.  Controls: quad_perm encodes four 2-bit selectors,
+// 0x140 = row_mirror, 0x141 = row_half_mirror (rows are 16 lanes).
+template <int kCtrl>
+__device__ __forceinline__ int dpp_move(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, kCtrl, 0xF, 0xF, true);
+}
+template <int kCtrl>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, dpp_move<kCtrl>(__builtin_bit_cast(int, v)));
+}
+constexpr int kDppXor1 = 0xB1;  // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;  // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141;
+constexpr int kDppRowMirror = 0x140;
+
+// Sum over the 8 lanes that share (lane >> 3); every lane gets the result.
+template <typename T>
+__device__ __forceinline__ T sum_over_8(T v) {
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    return v;
+}
+__device__ __forceinline__ float max_over_8(float v) {
+    v = fmaxf(v, dpp_move<kDppXor1>(v));
+    v = fmaxf(v, dpp_move<kDppXor2>(v));
+    v = fmaxf(v, dpp_move<kDppHalfMirror>(v));
+    return v;
+}
+
+// Sum over the whole wavefront, result uniform.  Fixed order, so deterministic.
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_move<kDppXor1>(v);
+    v += dpp_move<kDppXor2>(v);
+    v += dpp_move<kDppHalfMirror>(v);
+    v += dpp_move<kDppRowMirror>(v);  // every lane now holds its 16-lane row sum
+    int bits = __builtin_bit_cast(int, v);
+    float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+    float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+    float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+    float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+    return (r0 + r1) + (r2 + r3);
+}
+
+// ---- activation quantizer for one value, given its block's max |x|
+// (ops/native_compute.zig:11998-12028): f32 scale, one reciprocal, round half
+// away from zero, clamp to +-127.
+__device__ __forceinline__ float act_scale(float max_abs) {
+    return max_abs == 0.0f ? 1.0f : max_abs / 127.0f;
+}
+__device__ __forceinline__ int act_quant(float x, float inv_scale) {
+    float r = roundf(x * inv_scale);
+    r = fminf(fmaxf(r, -127.0f), 127.0f);
+    return static_cast<int>(r);
+}
+
+// Quantizes `rows * in_dim` activations into shared memory with every thread of
+// the workgroup: 8 consecutive lanes own one 32-value block (one float4 each).
+//   q     int8  [rows][in_dim]
+//   scale f32   [rows][in_dim/32]
+//   sum   int32 [rows][in_dim/32]   (sum of the block's int8 values)
+__device__ __forceinline__ void quantize_rows_to_lds(const float* __restrict__ x, int rows, int in_dim,
+                                                     int8_t* q, float* scale, int* sum) {
+    const int units = rows * (in_dim >> 2);  // float4 units; in_dim % 32 == 0
+    for (int u = threadIdx.x; u < units; u += blockDim.x) {
+        float4 v = reinterpret_cast<const float4*>(x)[u];
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        const float s = act_scale(m);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
+        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+        const int packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        reinterpret_cast<int*>(q)[u] = packed;
+        const int total = sum_over_8(q0 + q1 + q2 + q3);
+        if ((u & 7) == 0) {
+            scale[u >> 3] = s;
+            sum[u >> 3] = total;
+        }
+    }
+}
+
+// ---- weight block readers.  A "block view" yields the 32 weights of block
+// (row n, block b) as eight int32 of packed int8 in element order plus the f32
+// scale.  Q4_0 values are nibble-8 with low nibbles = elements 0..15 and high
+// nibbles = 16..31 (gguf/quant_codec.zig:1918-1942).
+struct BlockI8 {
+    int q[8];
+    float d;
+};
+
+__device__ __forceinline__ void unpack_q4(const uint32_t packed[4], int out[8]) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = packed[j] & 0x0F0F0F0Fu;
+        const uint32_t hi = (packed[j] >> 4) & 0x0F0F0F0Fu;
+        // per-byte nibble-8: bytes never borrow across lanes because we bias by
+        // 0x80 first ((n | 0x80) - 8 keeps bit 7 set), then flip bit 7 back.
+        out[j] = static_cast<int>((((lo | 0x80808080u) - 0x08080808u) ^ 0x80808080u));
+        out[4 + j] = static_cast<int>((((hi | 0x80808080u) - 0x08080808u) ^ 0x80808080u));
+    }
+}
+
+template <int kType>
+struct RawWeights;  // GGUF bytes, 2-byte aligned blocks
+
+template <>
+struct RawWeights<2> {  // Q4_0
+    const uint8_t* base;
+    __device__ __forceinline__ BlockI8 load(size_t block_index) const {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(base + block_index * kQ4BlockBytes);
+        BlockI8 r;
+        r.d = half_bits_to_f32(p[0]);
+        uint32_t packed[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) packed[j] = static_cast<uint32_t>(p[1 + 2 * j]) | (static_cast<uint32_t>(p[2 + 2 * j]) << 16);
+        unpack_q4(packed, r.q);
+        return r;
+    }
+};
+
+template <>
+struct RawWeights<8> {  // Q8_0
+    const uint8_t* base;
+    __device__ __forceinline__ BlockI8 load(size_t block_index) const {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(base + block_index * kQ8BlockBytes);
+        BlockI8 r;
+        r.d = half_bits_to_f32(p[0]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) r.q[j] = static_cast<int>(static_cast<uint32_t>(p[1 + 2 * j]) | (static_cast<uint32_t>(p[2 + 2 * j]) << 16));
+        return r;
+    }
+};
+
+template <int kType>
+struct PreparedWeights;  // quant bytes region then fp16 scale region
+
+template <>
+struct PreparedWeights<2> {
+    const uint4* qs;      // [blocks] 16 B
+    const uint16_t* d;    // [blocks]
+    __device__ __forceinline__ BlockI8 load(size_t block_index) const {
+        const uint4 v = qs[block_index];
+        BlockI8 r;
+        r.d = half_bits_to_f32(d[block_index]);
+        const uint32_t packed[4] = {v.x, v.y, v.z, v.w};
+        unpack_q4(packed, r.q);
+        return r;
+    }
+};
+
+template <>
+struct PreparedWeights<8> {
+    const uint4* qs;      // [blocks][2] 32 B
+    const uint16_t* d;
+    __device__ __forceinline__ BlockI8 load(size_t block_index) const {
+        const uint4 a = qs[2 * block_index], b = qs[2 * block_index + 1];
+        BlockI8 r;
+        r.d = half_bits_to_f32(d[block_index]);
+        r.q[0] = a.x; r.q[1] = a.y; r.q[2] = a.z; r.q[3] = a.w;
+        r.q[4] = b.x; r.q[5] = b.y; r.q[6] = b.z; r.q[7] = b.w;
+        return r;
+    }
+};
+
+__device__ __forceinline__ int dot32(const int w[8], const int a[8]) {
+    int acc = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc = dot4(w[j], a[j], acc);
+    return acc;
+}
+
+}  // namespace afhip

@@ -1,0 +1,407 @@
+// gfx950 kernels and stream-ordered launchers for the Q4_0 / Q8_0 quantized
+// matmul Y[rows,out] = X[rows,in] * W[out,in]^T.  Replaces
+// termite_linear_q8_0_f32 / termite_linear_q4_0_f32
+// (ops/cuda/artifacts/inference_cuda_kernels.cu:873-927) and their launchers
+// (ops/cuda/kernels.zig:1221-1289).
+//
+// Two numeric routes, chosen exactly like the CPU engine does
+// (ops/native_compute.zig:3410-3419):
+//   A  activations quantized to int8 per 32-block (f32 scale), int32 block dots,
+//      y += (sx*sw)*f32(dot)            -- out_dim >= 512 and in_dim/32 >= 3
+//   B  f32 activations times dequantized weights             -- otherwise
+#include "qmatmul_launch.h"
+
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+
+namespace afhip {
+
+// =====================================================================
+// Generic kernels: any in_dim % 32 == 0, any layout.  One wavefront per output
+// column, lanes stride over the row's blocks.  Correctness path for raw GGUF
+// buffers, odd shapes and the f32 route; the tuned kernels are further down.
+// =====================================================================
+
+// Route B.  grid = (out_dim, rows), block = 64.
+template <typename Weights>
+__global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict__ dst,
+                                                              const float* __restrict__ input, Weights w,
+                                                              int rows, int in_dim, int out_dim) {
+    const int o = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    const int kb = in_dim >> 5;
+    const float* x = input + static_cast<size_t>(r) * in_dim;
+    float acc = 0.0f;
+    for (int b = lane; b < kb; b += kWave) {
+        const BlockI8 blk = w.load(static_cast<size_t>(o) * kb + b);
+        const float* xb = x + b * 32;
+        float part = 0.0f;  // sum_i x_i * f32(q_i), then one multiply by d
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float4 xv = reinterpret_cast<const float4*>(xb)[j];
+            const int packed = blk.q[j];
+            part += xv.x * static_cast<float>(static_cast<int8_t>(packed & 0xFF));
+            part += xv.y * static_cast<float>(static_cast<int8_t>((packed >> 8) & 0xFF));
+            part += xv.z * static_cast<float>(static_cast<int8_t>((packed >> 16) & 0xFF));
+            part += xv.w * static_cast<float>(static_cast<int8_t>((packed >> 24) & 0xFF));
+        }
+        acc += blk.d * part;
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) dst[static_cast<size_t>(r) * out_dim + o] = acc;
+}
+
+// Route A from pre-quantized activations.  grid = (out_dim, rows), block = 64.
+// dots (optional): int32 [rows][out_dim][kb].
+template <typename Weights>
+__global__ __launch_bounds__(64) void linear_act_generic_kernel(float* __restrict__ dst, int* __restrict__ dots,
+                                                                const int8_t* __restrict__ qx,
+                                                                const float* __restrict__ sx, Weights w,
+                                                                int rows, int in_dim, int out_dim) {
+    const int o = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    const int kb = in_dim >> 5;
+    float acc = 0.0f;
+    for (int b = lane; b < kb; b += kWave) {
+        const BlockI8 blk = w.load(static_cast<size_t>(o) * kb + b);
+        const int4* ap = reinterpret_cast<const int4*>(qx + static_cast<size_t>(r) * in_dim + b * 32);
+        const int4 a0 = ap[0], a1 = ap[1];
+        const int a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+        const int dot = dot32(blk.q, a);
+        if (dots) dots[(static_cast<size_t>(r) * out_dim + o) * kb + b] = dot;
+        const float t = sx[static_cast<size_t>(r) * kb + b] * blk.d;
+        acc += t * static_cast<float>(dot);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0 && dst) dst[static_cast<size_t>(r) * out_dim + o] = acc;
+}
+
+// Stand-alone activation quantizer (ops/native_compute.zig:11998-12028,
+// :23799-23832).  8 lanes per block, grid-stride over float4 units.
+__global__ __launch_bounds__(256) void quantize_activations_kernel(const float* __restrict__ x, int rows, int in_dim,
+                                                                    int8_t* __restrict__ q, float* __restrict__ scale,
+                                                                    int* __restrict__ sum) {
+    const size_t units = static_cast<size_t>(rows) * (in_dim >> 2);
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const float4 v = reinterpret_cast<const float4*>(x)[u];
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        const float s = act_scale(m);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
+        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+        reinterpret_cast<int*>(q)[u] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        const int total = sum_over_8(q0 + q1 + q2 + q3);
+        if ((u & 7) == 0) {
+            scale[u >> 3] = s;
+            if (sum) sum[u >> 3] = total;
+        }
+    }
+}
+
+// RAW -> PREPARED repack, one thread per block.
+template <int kType>
+__global__ __launch_bounds__(256) void prepare_weight_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
+                                                             size_t blocks) {
+    constexpr int kQuantBytes = kType == 2 ? 16 : 32;
+    constexpr int kRawBytes = kQuantBytes + 2;
+    const size_t b = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+    if (b >= blocks) return;
+    const uint16_t* s = reinterpret_cast<const uint16_t*>(src + b * kRawBytes);
+    uint16_t* dq = reinterpret_cast<uint16_t*>(dst + b * kQuantBytes);
+    uint16_t* dd = reinterpret_cast<uint16_t*>(dst + blocks * kQuantBytes) + b;
+    *dd = s[0];
+#pragma unroll
+    for (int j = 0; j < kQuantBytes / 2; ++j) dq[j] = s[1 + j];
+}
+
+__global__ __launch_bounds__(256) void decode_fp16_kernel(float* __restrict__ dst, const uint16_t* __restrict__ src,
+                                                          size_t n) {
+    const size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
+    if (i < n) dst[i] = half_bits_to_f32(src[i]);
+}
+
+// =====================================================================
+// Fused-quant GEMV on the PREPARED layout, rows = kRows in 1..8 (decode and
+// speculative-verify).  HBM-bound: every weight byte is read once with 128-bit
+// loads, 1 KiB contiguous per wavefront instruction.
+//
+// Workgroup prologue: all threads quantize X[kRows, in_dim] into LDS (int8,
+// f32 scales, int32 block sums) while the first weight loads are in flight.
+// Main loop: one wavefront owns kCols output columns at a time; lane l owns
+// blocks l, l+64, ... of each of them.  Per-lane f32 partial sums are reduced
+// across the wavefront with DPP at the end of each column group.
+// =====================================================================
+
+template <int kType>
+struct GemvLane;
+
+// Q4_0: one lane = one block (16 B of nibbles).  Nibbles stay unsigned:
+// dot(qx, n-8) = dot(qx, n) - 8*sum(qx), with sum(qx) from the prologue.
+template <>
+struct GemvLane<2> {
+    static constexpr int kLanesPerBlock = 1;
+    uint32_t lo[4], hi[4];
+    float d;
+    __device__ __forceinline__ void load(const uint4* qs, const uint16_t* ds, size_t block_index, int /*half*/) {
+        const uint4 v = qs[block_index];
+        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            lo[j] = p[j] & 0x0F0F0F0Fu;
+            hi[j] = (p[j] >> 4) & 0x0F0F0F0Fu;
+        }
+        d = half_bits_to_f32(ds[block_index]);
+    }
+    // a: this block's 32 int8 activations (8 dwords), sum: their int32 sum
+    __device__ __forceinline__ int dot(const int8_t* a_lds, int sum, int /*half*/) const {
+        const int4 a0 = reinterpret_cast<const int4*>(a_lds)[0];
+        const int4 a1 = reinterpret_cast<const int4*>(a_lds)[1];
+        int acc = -8 * sum;
+        acc = dot4(static_cast<int>(lo[0]), a0.x, acc);
+        acc = dot4(static_cast<int>(lo[1]), a0.y, acc);
+        acc = dot4(static_cast<int>(lo[2]), a0.z, acc);
+        acc = dot4(static_cast<int>(lo[3]), a0.w, acc);
+        acc = dot4(static_cast<int>(hi[0]), a1.x, acc);
+        acc = dot4(static_cast<int>(hi[1]), a1.y, acc);
+        acc = dot4(static_cast<int>(hi[2]), a1.z, acc);
+        acc = dot4(static_cast<int>(hi[3]), a1.w, acc);
+        return acc;
+    }
+};
+
+// Q8_0: two lanes = one block (16 B of int8 each); halves are added with one DPP.
+template <>
+struct GemvLane<8> {
+    static constexpr int kLanesPerBlock = 2;
+    int q[4];
+    float d;
+    __device__ __forceinline__ void load(const uint4* qs, const uint16_t* ds, size_t block_index, int half) {
+        const uint4 v = qs[2 * block_index + half];
+        q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
+        d = half_bits_to_f32(ds[block_index]);
+    }
+    __device__ __forceinline__ int dot(const int8_t* a_lds, int /*sum*/, int half) const {
+        const int4 a = reinterpret_cast<const int4*>(a_lds)[half];
+        int acc = dot4(q[0], a.x, 0);
+        acc = dot4(q[1], a.y, acc);
+        acc = dot4(q[2], a.z, acc);
+        acc = dot4(q[3], a.w, acc);
+        acc += dpp_move<kDppXor1>(acc);  // both lanes of the pair now hold the block dot
+        return acc;
+    }
+};
+
+template <int kType, int kRows, int kCols, bool kWriteDots>
+__global__ void gemv_fused_kernel(float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input,
+                                  const uint8_t* __restrict__ weight, int in_dim, int out_dim) {
+    using Lane = GemvLane<kType>;
+    constexpr int kLpb = Lane::kLanesPerBlock;
+    constexpr int kBlocksPerStep = kWave / kLpb;
+    constexpr int kQuantBytes = kType == 2 ? 16 : 32;
+
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int kb = in_dim >> 5;
+    int8_t* qx = reinterpret_cast<int8_t*>(lds);                        // [kRows][in_dim]
+    float* sx = reinterpret_cast<float*>(lds + static_cast<size_t>(kRows) * in_dim);  // [kRows][kb]
+    int* sumx = reinterpret_cast<int*>(sx + kRows * kb);                // [kRows][kb]
+
+    const size_t blocks = static_cast<size_t>(out_dim) * kb;
+    const uint4* qs = reinterpret_cast<const uint4*>(weight);
+    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * kQuantBytes);
+
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int waves_per_wg = blockDim.x >> 6;
+    const int half = lane & (kLpb - 1);
+    const int lane_block = lane / kLpb;
+
+    const int groups = (out_dim + kCols - 1) / kCols;
+    const int wave_global = blockIdx.x * waves_per_wg + wave;
+    const int wave_stride = gridDim.x * waves_per_wg;
+
+    quantize_rows_to_lds(input, kRows, in_dim, qx, sx, sumx);
+    __syncthreads();
+
+    for (int g = wave_global; g < groups; g += wave_stride) {
+        const int o0 = g * kCols;
+        float acc[kRows][kCols];
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) acc[r][c] = 0.0f;
+
+        for (int b = lane_block; b < kb; b += kBlocksPerStep) {
+            Lane w[kCols];
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) {
+                const int o = min(o0 + c, out_dim - 1);  // clamp: tail columns recompute the last one
+                w[c].load(qs, ds, static_cast<size_t>(o) * kb + b, half);
+            }
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                const int8_t* a = qx + static_cast<size_t>(r) * in_dim + b * 32;
+                const float s = sx[r * kb + b];
+                const int sm = sumx[r * kb + b];
+#pragma unroll
+                for (int c = 0; c < kCols; ++c) {
+                    const int dot = w[c].dot(a, sm, half);
+                    if (kWriteDots) {
+                        if (half == 0 && o0 + c < out_dim)
+                            dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + b] = dot;
+                    }
+                    const float t = s * w[c].d;
+                    const float term = t * static_cast<float>(dot);
+                    acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < kRows; ++r)
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) {
+                const float total = wave_sum(acc[r][c]);
+                if (lane == 0 && o0 + c < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + c] = total;
+            }
+    }
+}
+
+// =====================================================================
+// Launchers
+// =====================================================================
+
+namespace {
+
+hipError_t launch_status() { return hipGetLastError(); }
+
+template <int kType, int kRows, bool kDots>
+hipError_t launch_gemv_rows(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight,
+                            int in_dim, int out_dim, const GemvTuning& tune) {
+    constexpr int kCols = kRows <= 2 ? 4 : 2;
+    const int kb = in_dim / 32;
+    const size_t lds = static_cast<size_t>(kRows) * in_dim + static_cast<size_t>(kRows) * kb * 8;
+    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
+    // Raising the dynamic-LDS limit is sticky per kernel: do it once, outside any
+    // stream capture a caller may have open later.
+    static size_t lds_limit = 64 * 1024;
+    if (lds > lds_limit) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        if (e != hipSuccess) return e;
+        lds_limit = 128 * 1024;
+    }
+    const int threads = tune.threads;
+    const int waves_per_wg = threads / 64;
+    const int groups = (out_dim + kCols - 1) / kCols;
+    int grid = (groups + waves_per_wg - 1) / waves_per_wg;
+    if (grid > tune.max_workgroups) grid = tune.max_workgroups;
+    if (grid < 1) grid = 1;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, dst, dots, input, weight, in_dim, out_dim);
+    return launch_status();
+}
+
+template <int kType, bool kDots>
+hipError_t launch_gemv(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight, int rows,
+                       int in_dim, int out_dim, const GemvTuning& tune) {
+    switch (rows) {
+        case 1: return launch_gemv_rows<kType, 1, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 2: return launch_gemv_rows<kType, 2, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 3: return launch_gemv_rows<kType, 3, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 4: return launch_gemv_rows<kType, 4, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 5: return launch_gemv_rows<kType, 5, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 6: return launch_gemv_rows<kType, 6, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 7: return launch_gemv_rows<kType, 7, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        case 8: return launch_gemv_rows<kType, 8, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+size_t gemv_fused_lds_bytes(int rows, int in_dim) {
+    return static_cast<size_t>(rows) * in_dim + static_cast<size_t>(rows) * (in_dim / 32) * 8;
+}
+
+hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
+                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
+                             const GemvTuning& tune) {
+    if (tensor_type == 2) {
+        return dots ? launch_gemv<2, true>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune)
+                    : launch_gemv<2, false>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
+    }
+    return dots ? launch_gemv<8, true>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune)
+                : launch_gemv<8, false>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
+}
+
+hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
+                                       float* scale, int* sum) {
+    const size_t units = static_cast<size_t>(rows) * (in_dim / 4);
+    size_t grid = (units + 255) / 256;
+    if (grid > 4096) grid = 4096;
+    if (grid == 0) return hipSuccess;
+    hipLaunchKernelGGL(quantize_activations_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, x, rows,
+                       in_dim, q, scale, sum);
+    return launch_status();
+}
+
+template <typename Weights>
+static hipError_t launch_generic(hipStream_t stream, bool route_a, float* dst, int* dots, const float* input,
+                                 const int8_t* qx, const float* sx, Weights w, int rows, int in_dim, int out_dim) {
+    dim3 grid(out_dim, rows);
+    if (route_a) {
+        hipLaunchKernelGGL(linear_act_generic_kernel<Weights>, grid, dim3(64), 0, stream, dst, dots, qx, sx, w, rows,
+                           in_dim, out_dim);
+    } else {
+        hipLaunchKernelGGL(linear_f32_route_kernel<Weights>, grid, dim3(64), 0, stream, dst, input, w, rows, in_dim,
+                           out_dim);
+    }
+    return launch_status();
+}
+
+hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout, bool route_a, float* dst, int* dots,
+                                 const float* input, const int8_t* qx, const float* sx, const uint8_t* weight,
+                                 int rows, int in_dim, int out_dim) {
+    const size_t blocks = static_cast<size_t>(out_dim) * (in_dim / 32);
+    // grid.y is limited to 65535 rows per launch
+    for (int r0 = 0; r0 < rows; r0 += 32768) {
+        const int nr = rows - r0 < 32768 ? rows - r0 : 32768;
+        float* d = dst ? dst + static_cast<size_t>(r0) * out_dim : nullptr;
+        int* dd = dots ? dots + static_cast<size_t>(r0) * out_dim * (in_dim / 32) : nullptr;
+        const float* in = input ? input + static_cast<size_t>(r0) * in_dim : nullptr;
+        const int8_t* q = qx ? qx + static_cast<size_t>(r0) * in_dim : nullptr;
+        const float* s = sx ? sx + static_cast<size_t>(r0) * (in_dim / 32) : nullptr;
+        hipError_t e;
+        if (layout == 0) {
+            if (tensor_type == 2) e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<2>{weight}, nr, in_dim, out_dim);
+            else e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<8>{weight}, nr, in_dim, out_dim);
+        } else {
+            const uint4* qs = reinterpret_cast<const uint4*>(weight);
+            if (tensor_type == 2) {
+                PreparedWeights<2> w{qs, reinterpret_cast<const uint16_t*>(weight + blocks * 16)};
+                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim);
+            } else {
+                PreparedWeights<8> w{qs, reinterpret_cast<const uint16_t*>(weight + blocks * 32)};
+                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim);
+            }
+        }
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
+                                 size_t blocks) {
+    if (blocks == 0) return hipSuccess;
+    const unsigned grid = static_cast<unsigned>((blocks + 255) / 256);
+    if (tensor_type == 2) hipLaunchKernelGGL(prepare_weight_kernel<2>, dim3(grid), dim3(256), 0, stream, dst, src, blocks);
+    else hipLaunchKernelGGL(prepare_weight_kernel<8>, dim3(grid), dim3(256), 0, stream, dst, src, blocks);
+    return launch_status();
+}
+
+hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(decode_fp16_kernel, dim3(static_cast<unsigned>((n + 255) / 256)), dim3(256), 0, stream, dst, src, n);
+    return launch_status();
+}
+
+}  // namespace afhip

@@ -1,0 +1,37 @@
+// Internal C++ interface between the kernel file and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace afhip {
+
+// Launch geometry of the fused GEMV; chosen host-side (ops/cuda/kernels.zig
+// does the same for its launch1d / launchBlocks helpers).
+struct GemvTuning {
+    int threads = 256;          // workgroup size, multiple of 64
+    int max_workgroups = 2048;  // persistent-grid cap
+};
+
+size_t gemv_fused_lds_bytes(int rows, int in_dim);
+
+// rows in 1..8, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
+hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
+                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
+                             const GemvTuning& tune);
+
+hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
+                                       float* scale, int* sum);
+
+// Any layout / shape.  route_a: uses qx/sx (pre-quantized), else f32 `input`.
+hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout, bool route_a, float* dst, int* dots,
+                                 const float* input, const int8_t* qx, const float* sx, const uint8_t* weight,
+                                 int rows, int in_dim, int out_dim);
+
+hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
+                                 size_t blocks);
+
+hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);
+
+}  // namespace afhip

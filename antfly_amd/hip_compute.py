@@ -1,0 +1,168 @@
+"""`HipCompute`: the backend object behind the engine's ComputeBackend op
+interface, mirroring ops/cuda/cuda_compute.zig of the reference (method names
+and error behaviour follow the vtable entries on the quantized-linear path:
+linearNoBias ops/ops.zig:890, linearNoBiasPlanned :895, fromFloat32, toFloat32,
+getWeight, freeTensor).  All work happens behind the C ABI."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib, quant_matmul
+from ._lib import check
+
+
+class HipTensor:
+    """Opaque tensor handle (CT).  Borrowed handles (weights) are not freed."""
+
+    def __init__(self, handle: int, borrowed: bool = False):
+        self.handle = handle
+        self.borrowed = borrowed
+
+    @property
+    def dtype(self) -> int:
+        return _lib.lib().afhip_tensor_dtype(self.handle)
+
+    @property
+    def quant_type(self):
+        q = _lib.lib().afhip_tensor_quant_type(self.handle)
+        return None if q < 0 else q
+
+    @property
+    def layout(self) -> int:
+        return _lib.lib().afhip_tensor_layout(self.handle)
+
+    @property
+    def elem_count(self) -> int:
+        return _lib.lib().afhip_tensor_elem_count(self.handle)
+
+    @property
+    def shape(self):
+        n = _lib.lib().afhip_tensor_rank(self.handle)
+        out = (C.c_int64 * max(n, 1))()
+        check(_lib.lib().afhip_tensor_shape(self.handle, out, n))
+        return [int(out[i]) for i in range(n)]
+
+    @property
+    def device_ptr(self) -> int:
+        return _lib.lib().afhip_tensor_device_ptr(self.handle)
+
+    @property
+    def byte_len(self) -> int:
+        return _lib.lib().afhip_tensor_byte_len(self.handle)
+
+
+class HipCompute:
+    def __init__(self):
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_create(C.byref(h)))
+        self._h = h
+
+    # -- lifecycle -----------------------------------------------------
+    def deinit(self) -> None:
+        if self._h:
+            _lib.lib().afhip_compute_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.deinit()
+
+    def __del__(self):
+        try:
+            self.deinit()
+        except Exception:
+            pass
+
+    def backendKind(self) -> str:
+        return "hip" if _lib.lib().afhip_compute_backend_kind(self._h) == 1 else "unknown"
+
+    @property
+    def stream(self) -> int:
+        return _lib.lib().afhip_compute_stream(self._h) or 0
+
+    def synchronize(self) -> None:
+        check(_lib.lib().afhip_compute_synchronize(self._h))
+
+    def deviceName(self) -> str:
+        buf = C.create_string_buffer(256)
+        check(_lib.lib().afhip_compute_device_name(self._h, buf, 256))
+        return buf.value.decode()
+
+    # -- weights ---------------------------------------------------------
+    def insertWeightFromLoaded(self, key: str, tensor_type: int, raw_bytes, shape, keep_raw_layout: bool = False) -> None:
+        raw = np.ascontiguousarray(raw_bytes, dtype=np.uint8)
+        shp = (C.c_int64 * max(len(shape), 1))(*shape)
+        check(_lib.lib().afhip_compute_insert_weight_from_loaded(self._h, key.encode(), tensor_type, raw.ctypes.data,
+                                                                 raw.size, shp, len(shape), int(keep_raw_layout)))
+
+    def insertWeightFromTensor(self, key: str, data, shape) -> None:
+        arr = np.ascontiguousarray(data, dtype=np.float32)
+        shp = (C.c_int64 * max(len(shape), 1))(*shape)
+        check(_lib.lib().afhip_compute_insert_weight_f32(self._h, key.encode(), arr.ctypes.data, shp, len(shape)))
+
+    def getWeight(self, name: str) -> HipTensor:
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_get_weight(self._h, name.encode(), C.byref(h)))
+        return HipTensor(h.value, borrowed=True)
+
+    # -- tensors ---------------------------------------------------------
+    def fromFloat32(self, data, shape=None) -> HipTensor:
+        arr = np.ascontiguousarray(data, dtype=np.float32)
+        if shape is None:
+            shape = [arr.size]
+        shp = (C.c_int32 * max(len(shape), 1))(*shape)
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_from_float32(self._h, arr.ctypes.data, arr.size, shp, len(shape), C.byref(h)))
+        return HipTensor(h.value)
+
+    def wrapDeviceFloat32(self, device_ptr: int, shape) -> HipTensor:
+        shp = (C.c_int64 * max(len(shape), 1))(*shape)
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_wrap_device_f32(self._h, device_ptr, shp, len(shape), C.byref(h)))
+        return HipTensor(h.value)
+
+    def toFloat32(self, tensor: HipTensor) -> np.ndarray:
+        out = np.empty(tensor.elem_count, dtype=np.float32)
+        check(_lib.lib().afhip_compute_to_float32(self._h, tensor.handle, out.ctypes.data, out.size))
+        return out
+
+    def evalTensor(self, tensor: HipTensor) -> None:
+        check(_lib.lib().afhip_compute_eval_tensor(self._h, tensor.handle))
+
+    def freeTensor(self, tensor: HipTensor) -> None:
+        if tensor is not None and tensor.handle:
+            _lib.lib().afhip_compute_free_tensor(self._h, tensor.handle)
+            if not tensor.borrowed:
+                tensor.handle = None
+
+    free = freeTensor
+
+    # -- the op ------------------------------------------------------------
+    def linearNoBias(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int) -> HipTensor:
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_no_bias(self._h, input.handle, weight.handle, rows, in_dim, out_dim,
+                                                      C.byref(h)))
+        return HipTensor(h.value)
+
+    def linearNoBiasPlanned(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int,
+                            operator_plan: "quant_matmul.OperatorPlan") -> HipTensor:
+        req = _lib.PlannedRequest(input.handle, weight.handle, rows, in_dim, out_dim, operator_plan.to_c())
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_no_bias_planned(self._h, C.byref(req), C.byref(h)))
+        return HipTensor(h.value)
+
+    def linearNoBiasWithPlan(self, input, weight, rows, in_dim, out_dim, op_plan=None) -> HipTensor:
+        """ops/ops.zig:1762-1784: planned op when a plan is given, eager op otherwise."""
+        if op_plan is not None:
+            return self.linearNoBiasPlanned(input, weight, rows, in_dim, out_dim, op_plan)
+        return self.linearNoBias(input, weight, rows, in_dim, out_dim)
+
+    # -- counters ------------------------------------------------------------
+    def debugStats(self) -> dict:
+        s = _lib.DebugStats()
+        check(_lib.lib().afhip_compute_debug_stats(self._h, C.byref(s)))
+        return {name: int(getattr(s, name)) for name, _ in s._fields_}

@@ -1,0 +1,247 @@
+/*
+ * antfly_hip_qmatmul -- C ABI of the MI355X (gfx950) block-quantized matmul
+ * backend: Y[rows, out_dim] = X[rows, in_dim] * Wq[out_dim, in_dim]^T with W in
+ * GGUF Q4_0 / Q8_0 blocks (32 weights, fp16 scale).
+ *
+ * These are the entry points a Zig `hip` backend binds in place of the
+ * reference's CUDA backend.  Reference paths below are relative to
+ * zig/pkg/inference/src in the antfly tree.
+ *
+ * Conventions: every function returns an afhip_status (0 = ok, > 0 = a
+ * hipError_t from the runtime, < 0 = one of enum afhip_error); nothing throws or
+ * aborts.  Device pointers are plain 64-bit addresses.  `stream` is a
+ * hipStream_t (NULL = the null stream); all launches are asynchronous on it.
+ * A backend instance is not thread-safe: one caller thread per instance
+ * (ops/cuda/context.zig:44-105 has the same rule).
+ */
+#ifndef ANTFLY_HIP_QMATMUL_H
+#define ANTFLY_HIP_QMATMUL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef int afhip_status;
+
+/* Error vocabulary of the reference backend (ops/cuda/driver.zig:32-38,
+ * ops/cuda/cuda_compute.zig:689-717, ops/native_compute.zig:5039-5050). */
+enum afhip_error {
+    AFHIP_OK = 0,
+    AFHIP_ERR_INVALID_STATE = -1,           /* error.InvalidCudaState: bad shape / short buffer at a launcher */
+    AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE = -2, /* error.UnsupportedTensorType */
+    AFHIP_ERR_INVALID_SHAPE = -3,           /* error.InvalidShape */
+    AFHIP_ERR_WEIGHT_NOT_FOUND = -4,        /* error.WeightNotFound */
+    AFHIP_ERR_OP_UNSUPPORTED = -5,          /* error.CudaOpUnsupported */
+    AFHIP_ERR_INVALID_PARTITION_PLAN = -6,  /* error.InvalidPartitionPlan */
+    AFHIP_ERR_UNAVAILABLE = -7,             /* error.CudaUnavailable: no usable HIP runtime */
+    AFHIP_ERR_NO_DEVICES = -8,              /* error.NoCudaDevices */
+    AFHIP_ERR_OUT_OF_MEMORY = -9,
+    AFHIP_ERR_INVALID_ARGUMENT = -10,       /* null pointer / unknown enum at the ABI itself */
+    AFHIP_ERR_SMOKE_MISMATCH = -11          /* error.CudaSmokeMismatch */
+};
+const char *afhip_status_string(afhip_status status);
+
+/* GGUF tensor-type ids (gguf/tensor_types.zig). */
+enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_0 = 8 };
+
+/* How a quantized weight sits in device memory.
+ * RAW       GGUF bytes as uploaded: [out][in/32] blocks of 18 / 34 bytes.
+ * PREPARED  device-side repack of the same bytes (same size): all quant bytes
+ *           first, 16 / 32 bytes per block in block order, then all fp16 scales.
+ *           16-byte aligned so one lane loads a block (Q4_0) or half a block
+ *           (Q8_0) with a single 128-bit load.  The CPU backend prepares its
+ *           layouts at load time in the same way (ops/native_compute.zig:8130-8204). */
+enum afhip_weight_layout { AFHIP_LAYOUT_RAW = 0, AFHIP_LAYOUT_PREPARED = 1 };
+
+/* A device allocation, ops/cuda/buffer.zig DeviceBuffer{ptr,len}. */
+typedef struct afhip_buffer {
+    uint64_t ptr;
+    size_t len;
+} afhip_buffer;
+
+/* ------------------------------------------------------------------------
+ * Dispatch vocabulary: graph/quant_matmul.zig:17-55 (enums), :241-287
+ * (plan/select), :558-576 (rowBucket, validShape).
+ * ---------------------------------------------------------------------- */
+enum afhip_dispatch_kind { AFHIP_DISPATCH_SCALAR = 0, AFHIP_DISPATCH_MMV = 1, AFHIP_DISPATCH_SMALL_BATCH = 2, AFHIP_DISPATCH_MM = 3 };
+enum afhip_primitive { AFHIP_PRIM_MAT_VEC = 0, AFHIP_PRIM_MAT_VEC_EXT = 1, AFHIP_PRIM_MAT_MAT = 2, AFHIP_PRIM_SCALAR = 3 };
+enum afhip_operator { AFHIP_OP_FALLBACK = 0, AFHIP_OP_MUL_MV = 1, AFHIP_OP_MUL_MV_EXT = 2, AFHIP_OP_MUL_MM = 3, AFHIP_OP_GET_ROWS = 4 };
+enum afhip_row_bucket { AFHIP_ROWS_0 = 0, AFHIP_ROWS_1 = 1, AFHIP_ROWS_2_8 = 2, AFHIP_ROWS_9_64 = 3, AFHIP_ROWS_65_PLUS = 4 };
+/* quant_matmul.Format values for the formats this backend knows. */
+enum afhip_quant_format { AFHIP_FORMAT_UNKNOWN = 0, AFHIP_FORMAT_Q4_0 = 1, AFHIP_FORMAT_Q8_0 = 5, AFHIP_FORMAT_F32 = 254 };
+
+typedef struct afhip_quant_plan { /* quant_matmul.Plan, :223-232 */
+    uint8_t dispatch;
+    uint8_t primitive;
+    uint8_t op;
+    uint8_t row_bucket;
+    uint16_t format;
+    size_t rows;
+    size_t in_dim;
+    size_t out_dim;
+} afhip_quant_plan;
+
+/* OperatorPlan union tag (graph/operator_plan.zig:24-38): only quant_matmul
+ * plans are valid for a linear op. */
+enum afhip_operator_plan_kind { AFHIP_PLAN_QUANT_MATMUL = 0, AFHIP_PLAN_QUANT_ROW = 1, AFHIP_PLAN_ATTENTION = 2 };
+typedef struct afhip_operator_plan {
+    int kind;
+    afhip_quant_plan quant_matmul;
+} afhip_operator_plan;
+
+int afhip_quant_matmul_select(size_t rows, size_t in_dim, size_t out_dim, int format);            /* select, :263-268 */
+void afhip_quant_matmul_plan(size_t rows, size_t in_dim, size_t out_dim, int format, afhip_quant_plan *out); /* plan, :241-252 */
+int afhip_quant_row_bucket(size_t rows);                                                          /* rowBucket, :558-564 */
+int afhip_quant_format_from_tensor_type(int tensor_type); /* graph/backend_contracts.zig:199-236 */
+/* Route gate of the CPU engine (ops/native_compute.zig:3410-3419): 1 when the op
+ * quantizes activations to int8 per 32-block, 0 when it multiplies f32
+ * activations by dequantized weights. */
+int afhip_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim);
+
+/* ------------------------------------------------------------------------
+ * Kernel launchers: ops/cuda/kernels.zig:1221-1289 (launchLinearQ8_0F32 /
+ * launchLinearQ4_0F32).  Same checks: in_dim must be a non-zero multiple of 32
+ * and every buffer long enough, else AFHIP_ERR_INVALID_STATE; rows*out_dim == 0
+ * is a successful no-op.
+ * ---------------------------------------------------------------------- */
+
+/* Bytes of device scratch a launch needs (quantized activations for the
+ * int8-MFMA GEMM and for unfused GEMV); 0 when the call needs none. */
+size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
+
+/* Y = X * W^T.  `layout` says how `weight` is stored; `dispatch` is -1 to let
+ * quant_matmul.select choose by rows, or an afhip_dispatch_kind to force a
+ * kernel family (what a validated OperatorPlan forwards). */
+afhip_status afhip_launch_linear_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                     afhip_buffer input, afhip_buffer weight, size_t rows,
+                                     size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                     int dispatch);
+/* Drop-ins with the reference launcher names: raw GGUF layout, automatic dispatch. */
+afhip_status afhip_launch_linear_q8_0_f32(void *stream, afhip_buffer dst, afhip_buffer input,
+                                          afhip_buffer weight_raw, size_t rows, size_t in_dim,
+                                          size_t out_dim, afhip_buffer workspace);
+afhip_status afhip_launch_linear_q4_0_f32(void *stream, afhip_buffer dst, afhip_buffer input,
+                                          afhip_buffer weight_raw, size_t rows, size_t in_dim,
+                                          size_t out_dim, afhip_buffer workspace);
+
+/* One-time device-side repack RAW -> PREPARED (dst.len >= src bytes). */
+afhip_status afhip_launch_prepare_weight(void *stream, int tensor_type, afhip_buffer dst_prepared,
+                                         afhip_buffer src_raw, size_t out_dim, size_t in_dim);
+
+/* Activation quantizer on its own (ops/native_compute.zig:11998-12028,
+ * :23799-23832): q int8 [rows][in_dim], scales f32 [rows][in_dim/32],
+ * sums int32 [rows][in_dim/32] (sums.ptr may be 0). */
+afhip_status afhip_launch_quantize_activations(void *stream, afhip_buffer input, size_t rows,
+                                               size_t in_dim, afhip_buffer q, afhip_buffer scales,
+                                               afhip_buffer sums);
+
+/* The int32 block dot products the activation-quantized route forms
+ * (ops/native_compute.zig:12140-12151), written as
+ * dots[(r*out_dim + o)*(in_dim/32) + b] by the same device code the matmul
+ * kernels use (`dispatch` picks the kernel family as above).  Debug / parity. */
+afhip_status afhip_launch_block_dots(void *stream, int tensor_type, int layout, afhip_buffer dots,
+                                     afhip_buffer input, afhip_buffer weight, size_t rows,
+                                     size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                     int dispatch);
+
+/* fp16 -> f32 of n little-endian halves with the device's conversion
+ * (gguf/quant_codec.zig:35-39).  Parity probe for subnormal scales. */
+afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_buffer src_u16, size_t n);
+
+/* ------------------------------------------------------------------------
+ * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
+ * vtable entries on this path).  Owns one device context, ONE stream, resident
+ * weights, a <= 256-entry best-fit pool of freed buffers (:193-223) and a
+ * grow-only scratch (ops/cuda/scratch.zig).
+ * ---------------------------------------------------------------------- */
+typedef struct afhip_compute afhip_compute;
+typedef struct afhip_tensor afhip_tensor; /* CudaTensor, cuda_compute.zig:29-38 */
+
+enum afhip_dtype { AFHIP_DTYPE_F32 = 0, AFHIP_DTYPE_U8 = 1 };
+enum afhip_backend_kind { AFHIP_BACKEND_HIP = 1 };
+
+afhip_status afhip_compute_create(afhip_compute **out);   /* CudaCompute.create, :60-66 */
+void afhip_compute_destroy(afhip_compute *self);          /* deinit, :68-83 */
+int afhip_compute_backend_kind(const afhip_compute *self);
+void *afhip_compute_stream(afhip_compute *self);          /* the instance's hipStream_t */
+afhip_status afhip_compute_synchronize(afhip_compute *self); /* ctx.synchronize, context.zig:105 */
+afhip_status afhip_compute_device_name(afhip_compute *self, char *out, size_t out_len);
+
+/* insertWeightFromLoaded, :88-137: copies raw GGUF bytes H2D, synchronizes, and
+ * (unless `keep_raw_layout`) repacks them on the device.  shape = [out, in].
+ * f32 weights go through afhip_compute_insert_weight_f32 (insertWeightFromTensor). */
+afhip_status afhip_compute_insert_weight_from_loaded(afhip_compute *self, const char *key,
+                                                     int tensor_type, const void *raw_bytes,
+                                                     size_t raw_len, const int64_t *shape,
+                                                     size_t shape_len, int keep_raw_layout);
+afhip_status afhip_compute_insert_weight_f32(afhip_compute *self, const char *key, const float *data,
+                                             const int64_t *shape, size_t shape_len);
+/* getWeight, :233-236: borrowed handle, never freed by the caller. */
+afhip_status afhip_compute_get_weight(afhip_compute *self, const char *key, afhip_tensor **out);
+
+/* fromFloat32Shape, :243-270: product(shape) must equal data_len, else AFHIP_ERR_INVALID_SHAPE. */
+afhip_status afhip_compute_from_float32(afhip_compute *self, const float *data, size_t data_len,
+                                        const int32_t *shape, size_t shape_len, afhip_tensor **out);
+afhip_status afhip_compute_to_float32(afhip_compute *self, const afhip_tensor *tensor, float *out,
+                                      size_t out_count);                            /* :272-281 */
+/* Wraps caller-owned device memory (not freed by free_tensor) as an f32 tensor. */
+afhip_status afhip_compute_wrap_device_f32(afhip_compute *self, uint64_t device_ptr,
+                                           const int64_t *shape, size_t shape_len, afhip_tensor **out);
+void afhip_compute_free_tensor(afhip_compute *self, afhip_tensor *tensor);          /* :225-231 */
+afhip_status afhip_compute_eval_tensor(afhip_compute *self, const afhip_tensor *tensor); /* :293-296 */
+int afhip_tensor_dtype(const afhip_tensor *tensor);
+int afhip_tensor_quant_type(const afhip_tensor *tensor); /* -1 when not quantized */
+int afhip_tensor_layout(const afhip_tensor *tensor);
+size_t afhip_tensor_elem_count(const afhip_tensor *tensor);
+size_t afhip_tensor_rank(const afhip_tensor *tensor);
+afhip_status afhip_tensor_shape(const afhip_tensor *tensor, int64_t *out, size_t out_len);
+uint64_t afhip_tensor_device_ptr(const afhip_tensor *tensor);
+size_t afhip_tensor_byte_len(const afhip_tensor *tensor);
+
+/* linearNoBias, ops/ops.zig:890 and cuda_compute.zig:689-717: new f32 tensor
+ * [rows, out_dim] owned by the caller.  Quantized weights other than
+ * Q4_0 / Q8_0 -> AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE; element-count mismatches ->
+ * AFHIP_ERR_INVALID_SHAPE; in_dim % 32 != 0 -> AFHIP_ERR_INVALID_STATE. */
+afhip_status afhip_compute_linear_no_bias(afhip_compute *self, const afhip_tensor *input,
+                                          const afhip_tensor *weight, size_t rows, size_t in_dim,
+                                          size_t out_dim, afhip_tensor **out);
+
+/* linearNoBiasPlanned, ops/ops.zig:895 (request struct :92-99).  The plan is
+ * validated like validateQuantLinearPlan (ops/native_compute.zig:5039-5050):
+ * anything but a quant_matmul plan whose rows / in_dim / out_dim / format match
+ * and whose operator is not `fallback` -> AFHIP_ERR_INVALID_PARTITION_PLAN.  A
+ * valid plan's dispatch kind selects the kernel family. */
+typedef struct afhip_linear_no_bias_planned_request {
+    const afhip_tensor *input;
+    const afhip_tensor *weight;
+    size_t rows;
+    size_t in_dim;
+    size_t out_dim;
+    afhip_operator_plan operator_plan;
+} afhip_linear_no_bias_planned_request;
+afhip_status afhip_compute_linear_no_bias_planned(afhip_compute *self,
+                                                  const afhip_linear_no_bias_planned_request *request,
+                                                  afhip_tensor **out);
+
+/* Counters a backend snapshot exposes (ops/ops.zig:649-713,1368;
+ * pkg/inference/CUDA.md:492-507). */
+typedef struct afhip_debug_stats {
+    uint64_t h2d_bytes, d2h_bytes, resident_weight_bytes, pooled_buffers, device_allocs;
+    uint64_t launches_mmv, launches_small_batch, launches_mm, launches_f32_route;
+    uint64_t launches_activation_quant, launches_prepare, scratch_bytes;
+} afhip_debug_stats;
+afhip_status afhip_compute_debug_stats(const afhip_compute *self, afhip_debug_stats *out);
+
+/* Known-answer smokes run entirely inside the library on device 0
+ * (ops/cuda/kernels.zig:2309-2399, driven by `cuda-info --smoke`,
+ * cuda_info.zig:57-82). */
+afhip_status afhip_smoke_q8_0(void);
+afhip_status afhip_smoke_q4_0(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

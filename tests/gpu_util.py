@@ -1,0 +1,61 @@
+"""Helpers for the GPU tests: torch is only the allocator and the stream."""
+import numpy as np
+import torch
+
+from antfly_amd import _lib, kernels
+from antfly_amd._lib import Buffer
+
+DEV = "cuda:0"
+
+
+def buf(t: torch.Tensor) -> Buffer:
+    return Buffer(t.data_ptr(), t.numel() * t.element_size())
+
+
+def stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def to_dev(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def prepare(fmt: int, w_raw: np.ndarray, out_dim: int, in_dim: int) -> torch.Tensor:
+    raw = to_dev(w_raw)
+    prepared = torch.empty_like(raw)
+    kernels.launchPrepareWeight(stream(), fmt, buf(prepared), buf(raw), out_dim, in_dim)
+    torch.cuda.synchronize()
+    return prepared
+
+
+def numpy_prepare(fmt: int, w_raw: np.ndarray) -> np.ndarray:
+    bb = 18 if fmt == _lib.TYPE_Q4_0 else 34
+    blocks = np.asarray(w_raw, np.uint8).reshape(-1, bb)
+    return np.concatenate([blocks[:, 2:].reshape(-1), blocks[:, :2].reshape(-1)])
+
+
+def linear(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1) -> np.ndarray:
+    xd = to_dev(x.astype(np.float32))
+    y = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    ws_bytes = kernels.workspaceBytes(fmt, rows, in_dim, out_dim)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=DEV)
+    kernels.launchLinearF32(stream(), fmt, layout, buf(y), buf(xd), buf(w_dev), rows, in_dim, out_dim, buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def block_dots(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1) -> np.ndarray:
+    xd = to_dev(x.astype(np.float32))
+    d = torch.full((rows, out_dim, in_dim // 32), -(2 ** 31), dtype=torch.int32, device=DEV)
+    ws_bytes = kernels.workspaceBytes(fmt, rows, in_dim, out_dim)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=DEV)
+    kernels.launchBlockDots(stream(), fmt, layout, buf(d), buf(xd), buf(w_dev), rows, in_dim, out_dim, buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return d.cpu().numpy()
+
+
+def max_rel_err(got: np.ndarray, want: np.ndarray) -> float:
+    """Largest |got - want| relative to the largest |want| of the same output row."""
+    scale = np.abs(want).max(axis=-1, keepdims=True)
+    scale = np.where(scale == 0, 1.0, scale)
+    return float((np.abs(got.astype(np.float64) - want) / scale).max())

@@ -1,0 +1,156 @@
+"""The backend object (HipCompute) through the C ABI: same op contract, ownership
+and error behaviour as the reference's CUDA backend (ops/cuda/cuda_compute.zig)
+and the native planned op (ops/native_compute.zig:42750-42831)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+pytest.importorskip("torch")
+
+from antfly_amd import _lib, quant_matmul as qm, synth  # noqa: E402
+from antfly_amd.hip_compute import HipCompute  # noqa: E402
+from oracle import oracle as O  # noqa: E402
+from tests import gpu_util as G  # noqa: E402
+
+Q4, Q8 = _lib.TYPE_Q4_0, _lib.TYPE_Q8_0
+
+
+@pytest.fixture()
+def cb():
+    c = HipCompute()
+    yield c
+    c.deinit()
+
+
+def test_backend_identity(cb):
+    assert cb.backendKind() == "hip"
+    assert "gfx950" in cb.deviceName()
+    assert cb.stream != 0
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+@pytest.mark.parametrize("keep_raw", [False, True])
+def test_linear_no_bias_matches_cpu_engine(cb, fmt, keep_raw):
+    rows, in_dim, out_dim = 5, 1024, 768
+    print(f"case: backend linearNoBias fmt={fmt} keep_raw={keep_raw}", flush=True)
+    w = synth.weights(fmt, 5, out_dim, in_dim)
+    x = synth.activations(6, rows, in_dim)
+    cb.insertWeightFromLoaded("blk.0.ffn_up.weight", fmt, w, [out_dim, in_dim], keep_raw_layout=keep_raw)
+    wt = cb.getWeight("blk.0.ffn_up.weight")
+    assert wt.dtype == _lib.DTYPE_U8 and wt.quant_type == fmt and wt.elem_count == out_dim * in_dim
+    assert wt.shape == [out_dim, in_dim] and wt.byte_len >= w.size
+    assert wt.layout == (_lib.LAYOUT_RAW if keep_raw else _lib.LAYOUT_PREPARED)
+    xt = cb.fromFloat32(x, [rows, in_dim])
+    yt = cb.linearNoBias(xt, wt, rows, in_dim, out_dim)
+    assert yt.shape == [rows, out_dim] and yt.dtype == _lib.DTYPE_F32 and yt.quant_type is None
+    y = cb.toFloat32(yt).reshape(rows, out_dim)
+    ref = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim, workers=8)
+    assert G.max_rel_err(y, ref.astype(np.float64)) <= 2e-5
+    # weights are borrowed: freeing the handle is a no-op and the weight stays usable
+    cb.freeTensor(wt)
+    yt2 = cb.linearNoBias(xt, cb.getWeight("blk.0.ffn_up.weight"), rows, in_dim, out_dim)
+    assert np.array_equal(cb.toFloat32(yt2).reshape(rows, out_dim), y)
+    stats = cb.debugStats()
+    assert stats["launches_small_batch"] == 2 and stats["resident_weight_bytes"] >= w.size
+    assert stats["launches_prepare"] == (0 if keep_raw else 1)
+    assert stats["launches_activation_quant"] == (2 if keep_raw else 0)
+    for t in (yt, yt2, xt):
+        cb.freeTensor(t)
+    assert cb.debugStats()["pooled_buffers"] >= 2
+
+
+def test_freed_buffers_are_reused(cb):
+    x = synth.activations(1, 4, 256)
+    a = cb.fromFloat32(x, [4, 256])
+    ptr = a.device_ptr
+    cb.freeTensor(a)
+    allocs = cb.debugStats()["device_allocs"]
+    b = cb.fromFloat32(x, [4, 256])
+    assert b.device_ptr == ptr and cb.debugStats()["device_allocs"] == allocs
+    cb.freeTensor(b)
+
+
+def test_op_errors(cb):
+    in_dim, out_dim = 256, 512
+    w = synth.weights(Q8, 1, out_dim, in_dim)
+    cb.insertWeightFromLoaded("w", Q8, w, [out_dim, in_dim])
+    cb.insertWeightFromLoaded("w_q4k", 12, np.zeros(144 * 2, np.uint8), [2, 256])  # resident, but no kernel here
+    cb.insertWeightFromTensor("w_dense", np.zeros((out_dim, in_dim), np.float32), [out_dim, in_dim])
+    x = cb.fromFloat32(synth.activations(2, 2, in_dim), [2, in_dim])
+    with pytest.raises(_lib.WeightNotFound):
+        cb.getWeight("missing")
+    with pytest.raises(_lib.InvalidShape):
+        cb.linearNoBias(x, cb.getWeight("w"), 3, in_dim, out_dim)        # input count mismatch
+    with pytest.raises(_lib.InvalidShape):
+        cb.linearNoBias(x, cb.getWeight("w"), 2, in_dim, out_dim + 1)    # weight count mismatch
+    with pytest.raises(_lib.UnsupportedTensorType):
+        cb.linearNoBias(cb.getWeight("w"), cb.getWeight("w"), 2, in_dim, out_dim)  # quantized input
+    with pytest.raises(_lib.UnsupportedTensorType):
+        cb.linearNoBias(cb.fromFloat32(np.zeros(2 * 256, np.float32), [2, 256]), cb.getWeight("w_q4k"), 2, 256, 2)
+    with pytest.raises(_lib.HipOpUnsupported):
+        cb.linearNoBias(x, cb.getWeight("w_dense"), 2, in_dim, out_dim)
+    with pytest.raises(_lib.InvalidShape):
+        cb.fromFloat32(np.zeros(8, np.float32), [3, 3])
+    with pytest.raises(_lib.InvalidShape):
+        cb.fromFloat32(np.zeros(8, np.float32), [-1, 8])
+    with pytest.raises(_lib.UnsupportedTensorType):
+        cb.toFloat32(cb.getWeight("w"))
+    # in_dim not a multiple of 32: the launcher rejects it (kernels.zig:1231)
+    cb.insertWeightFromLoaded("w_bad", Q8, np.zeros(34 * 4, np.uint8), [4, 33], keep_raw_layout=True)
+    xb = cb.fromFloat32(np.zeros(33, np.float32), [1, 33])
+    with pytest.raises(_lib.InvalidHipState):
+        cb.linearNoBias(xb, cb.getWeight("w_bad"), 1, 33, 4)
+    # zero rows: a valid empty result
+    empty = cb.fromFloat32(np.zeros(0, np.float32), [0, in_dim])
+    out = cb.linearNoBias(empty, cb.getWeight("w"), 0, in_dim, out_dim)
+    assert out.shape == [0, out_dim] and cb.toFloat32(out).size == 0
+
+
+def test_planned_op_follows_reference_test(cb, kats):
+    k = kats["planned_op"]
+    rows, in_dim, out_dim = k["rows"], k["in_dim"], k["out_dim"]
+
+    def fill(n, seed, scale):  # fillNativeQuantDispatchValues, native_compute.zig:42444-42449
+        idx = np.arange(n)
+        return ((((idx * 17 + seed * 31 + 7) % 67) - 33) * scale).astype(np.float32)
+
+    x = fill(rows * in_dim, rows, 0.015)
+    w = O.quantize_weights(Q8, fill(out_dim * in_dim, in_dim, 0.0125))
+    cb.insertWeightFromLoaded("planned_q8_0.weight", Q8, w, [out_dim, in_dim])
+    wt = cb.getWeight("planned_q8_0.weight")
+    xt = cb.fromFloat32(x, [rows, in_dim])
+    good = qm.OperatorPlan(qm.OperatorPlanKind.quant_matmul, qm.plan(qm.Shape(rows, in_dim, out_dim, qm.Format.q8_0)))
+    out = cb.linearNoBiasWithPlan(xt, wt, rows, in_dim, out_dim, good)
+    y = cb.toFloat32(out)
+    assert y.size == rows * out_dim and np.isfinite(y).all()
+    ref = O.linear_no_bias(Q8, x.reshape(rows, in_dim), w, rows, in_dim, out_dim)
+    assert G.max_rel_err(y.reshape(rows, out_dim), ref.astype(np.float64)) <= 2e-5
+    eager = cb.toFloat32(cb.linearNoBiasWithPlan(xt, wt, rows, in_dim, out_dim, None))
+    assert np.array_equal(eager, y)
+
+    bad_rows = qm.OperatorPlan(qm.OperatorPlanKind.quant_matmul, qm.plan(qm.Shape(rows + 1, in_dim, out_dim, qm.Format.q8_0)))
+    bad_fmt = qm.OperatorPlan(qm.OperatorPlanKind.quant_matmul, qm.plan(qm.Shape(rows, in_dim, out_dim, qm.Format.q4_0)))
+    fallback = qm.plan(qm.Shape(rows, in_dim, out_dim, qm.Format.q8_0))
+    fallback.operator = qm.Operator.fallback
+    row_plan = qm.OperatorPlan(qm.OperatorPlanKind.quant_row, None)
+    for bad in (bad_rows, bad_fmt, qm.OperatorPlan(qm.OperatorPlanKind.quant_matmul, fallback), row_plan):
+        with pytest.raises(_lib.InvalidPartitionPlan):
+            cb.linearNoBiasWithPlan(xt, wt, rows, in_dim, out_dim, bad)
+
+
+def test_torch_memory_can_be_wrapped(cb):
+    import torch
+
+    rows, in_dim, out_dim = 2, 512, 512
+    w = synth.weights(Q4, 3, out_dim, in_dim)
+    x = synth.activations(4, rows, in_dim)
+    cb.insertWeightFromLoaded("w", Q4, w, [out_dim, in_dim])
+    xd = torch.from_numpy(x).to("cuda:0")
+    torch.cuda.synchronize()
+    xt = cb.wrapDeviceFloat32(xd.data_ptr(), [rows, in_dim])
+    y = cb.toFloat32(cb.linearNoBias(xt, cb.getWeight("w"), rows, in_dim, out_dim)).reshape(rows, out_dim)
+    ref = O.linear_no_bias(Q4, x, w, rows, in_dim, out_dim)
+    assert G.max_rel_err(y, ref.astype(np.float64)) <= 2e-5
+    cb.freeTensor(xt)  # does not free torch's memory
+    assert torch.equal(xd.cpu(), torch.from_numpy(x))

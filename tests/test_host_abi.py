@@ -1,0 +1,96 @@
+"""CPU-only checks of the C ABI: the library loads, exports every declared
+symbol, and the host logic (dispatch vocabulary, launcher argument checks, plan
+validation) behaves like the reference's.  No kernel is launched."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from antfly_amd import _lib, kernels, quant_matmul as qm
+from antfly_amd._lib import Buffer
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "antfly_hip_qmatmul.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)  # drop comments
+    declared = set(re.findall(r"\b(afhip_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 40
+    L = C.CDLL(_lib.LIB_PATH)
+    missing = [name for name in sorted(declared) if not hasattr(L, name)]
+    assert not missing, missing
+    # the Python binding declares exactly the header's functions
+    assert declared == set(_lib.SIGNATURES)
+
+
+def test_status_strings():
+    L = _lib.lib()
+    assert L.afhip_status_string(0) == b"ok"
+    assert L.afhip_status_string(_lib.ERR_INVALID_PARTITION_PLAN) == b"InvalidPartitionPlan"
+    assert L.afhip_status_string(_lib.ERR_UNSUPPORTED_TENSOR_TYPE) == b"UnsupportedTensorType"
+
+
+def test_dispatch_buckets_match_reference(kats):
+    k = kats["dispatch"]
+    for case in k["select"]:
+        shape = qm.Shape(case["rows"], case["in_dim"], case["out_dim"], qm.Format[case["format"]])
+        assert qm.select(shape).name == case["dispatch"], case
+    for case in k["plan"]:
+        p = qm.plan(qm.Shape(case["rows"], case["in_dim"], case["out_dim"], qm.Format[case["format"]]))
+        assert p.primitive.name == case["primitive"] and p.operator.name == case["operator"], case
+    for rows, name in k["row_buckets"]:
+        assert qm.rowBucket(rows).name == name
+    # K must be a multiple of the 32-value block for both formats
+    for fmt in (qm.Format.q4_0, qm.Format.q8_0):
+        assert qm.select(qm.Shape(1, 48, 64, fmt)) == qm.DispatchKind.scalar
+        assert qm.select(qm.Shape(1, 64, 64, fmt)) == qm.DispatchKind.mmv
+        assert qm.select(qm.Shape(1, 0, 64, fmt)) == qm.DispatchKind.scalar
+        assert qm.select(qm.Shape(1, 64, 0, fmt)) == qm.DispatchKind.scalar
+    p = qm.plan(qm.Shape(5, 14336, 4096, qm.Format.q4_0))
+    assert (p.dispatch, p.row_bucket, p.rows, p.in_dim, p.out_dim) == (qm.DispatchKind.small_batch, qm.RowBucket.rows_2_8, 5, 14336, 4096)
+    assert qm.formatFromTensorType(2) == qm.Format.q4_0 and qm.formatFromTensorType(8) == qm.Format.q8_0
+    assert qm.formatFromTensorType(12) == qm.Format.unknown
+
+
+def test_route_gate_matches_cpu_engine():
+    L = _lib.lib()
+    assert L.afhip_uses_activation_quant(1, 4096, 14336) == 1
+    assert L.afhip_uses_activation_quant(1, 4096, 511) == 0
+    assert L.afhip_uses_activation_quant(1, 64, 4096) == 0   # two blocks per row
+    assert L.afhip_uses_activation_quant(1, 96, 512) == 1
+
+
+def test_launcher_argument_checks_before_any_launch():
+    big = Buffer(0x1000, 1 << 40)
+    # in_dim not a multiple of 32, or zero -> InvalidHipState (kernels.zig:1231,1266)
+    for fn in (kernels.launchLinearQ8_0F32, kernels.launchLinearQ4_0F32):
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, big, big, big, 1, 33, 8)
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, big, big, big, 1, 0, 8)
+        # short output / input / weight buffers
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, Buffer(0x1000, 4 * 8 - 1), big, big, 1, 32, 8)
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, big, Buffer(0x1000, 4 * 32 - 1), big, 1, 32, 8)
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, big, big, Buffer(0x1000, 8 * 18 - 1), 1, 32, 8)
+        # rows * out_dim == 0 is a successful no-op
+        fn(None, big, big, big, 0, 32, 8)
+        fn(None, big, big, big, 4, 32, 0)
+        # dimension overflow
+        with pytest.raises(_lib.InvalidHipState):
+            fn(None, big, big, big, 1 << 62, 32, 1 << 10)
+    with pytest.raises(_lib.UnsupportedTensorType):
+        kernels.launchLinearF32(None, 12, 0, big, big, big, 1, 256, 8)  # Q4_K is another operator
+    # raw-layout activation-quantized route needs the caller's scratch
+    assert kernels.workspaceBytes(2, 5, 14336, 4096) >= 5 * 14336 + 5 * 448 * 8
+    assert kernels.workspaceBytes(2, 0, 14336, 4096) == 0
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchLinearQ4_0F32(None, big, big, big, 1, 4096, 4096)
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchPrepareWeight(None, 2, Buffer(0x1000, 17), Buffer(0x2000, 18), 1, 32)
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchQuantizeActivations(None, big, 1, 48, big, big)
