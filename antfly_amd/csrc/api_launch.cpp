@@ -2,6 +2,7 @@
 // stream-ordered launchers (ops/cuda/kernels.zig:1221-1289).
 #include <hip/hip_runtime_api.h>
 
+#include <cstdlib>
 #include <limits>
 
 #include "antfly_hip_qmatmul.h"
@@ -47,13 +48,23 @@ static int gemv_row_chunk(size_t rows, size_t in_dim) {
     return chunk;
 }
 
+// Launch geometry of the fused GEMV.  AFHIP_GEMV_THREADS overrides it for tuning runs (the CPU engine exposes TERMITE_QUANT_* knobs the
+// same way, ops/native_compute.zig:2902-2945).
+static int env_int(const char* name) {
+    const char* v = std::getenv(name);
+    return v && *v ? std::atoi(v) : 0;
+}
+
 static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t out_dim) {
     (void)tensor_type;
     (void)out_dim;
+    static const int env_threads = env_int("AFHIP_GEMV_THREADS");
     GemvTuning t;
-    const size_t lds = gemv_fused_lds_bytes(rows, static_cast<int>(in_dim));
-    t.threads = lds > 32 * 1024 ? 1024 : 512;
-    t.max_workgroups = lds > 64 * 1024 ? 256 : 512;
+    // every workgroup quantizes all of X, so large workgroups share that work best
+    t.threads = 1024;
+    if (env_threads >= 64 && env_threads <= 1024 && env_threads % 64 == 0) t.threads = env_threads;
+    static const int env_wide = env_int("AFHIP_GEMV_WIDE");
+    t.wide = env_wide != 0;
     return t;
 }
 
@@ -106,7 +117,8 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim,
                                                                     afhip_quant_format_from_tensor_type(tensor_type));
     const int chunk = gemv_row_chunk(rows, in_dim);
-    const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR;
+    const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR &&
+                          in_dim <= static_cast<size_t>(gemv_fused_max_in_dim());
     if (fused_ok) {
         // mmv / small_batch: rows <= 8 in one launch.  mm (rows >= 9): same kernel
         // over 8-row slices until the MFMA GEMM takes over.

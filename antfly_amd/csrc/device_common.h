@@ -76,9 +76,16 @@ __device__ __forceinline__ float act_scale(float max_abs) {
     return max_abs == 0.0f ? 1.0f : max_abs / 127.0f;
 }
 __device__ __forceinline__ int act_quant(float x, float inv_scale) {
-    float r = roundf(x * inv_scale);
-    r = fminf(fmaxf(r, -127.0f), 127.0f);
-    return static_cast<int>(r);
+    // clamp(round_half_away(t), -127, 127) in three VALU operations:
+    //   t + copysign(h, t), h = the largest float below 0.5, truncated toward zero,
+    // is round-half-away for every |t| < 2^22: a fraction >= 0.5 pushes the sum to
+    // the next integer (the sum is within 2^-25 of it and rounds onto it), a smaller
+    // fraction leaves it at least half an ulp short, and |t| < 0.5 gives |sum| < 1.
+    // Clamping the sum to +-127.75 before truncating equals clamping the rounded
+    // integer to +-127.
+    const float t = x * inv_scale;
+    const float u = t + __builtin_copysignf(0x1.fffffep-2f, t);
+    return static_cast<int>(__builtin_amdgcn_fmed3f(u, -127.75f, 127.75f));
 }
 
 // Quantizes `rows * in_dim` activations into shared memory with every thread of

@@ -122,151 +122,6 @@ __global__ __launch_bounds__(256) void decode_fp16_kernel(float* __restrict__ ds
 }
 
 // =====================================================================
-// Fused-quant GEMV on the PREPARED layout, rows = kRows in 1..8 (decode and
-// speculative-verify).  HBM-bound: every weight byte is read once with 128-bit
-// loads, 1 KiB contiguous per wavefront instruction.
-//
-// Workgroup prologue: all threads quantize X[kRows, in_dim] into LDS (int8,
-// f32 scales, int32 block sums) while the first weight loads are in flight.
-// Main loop: one wavefront owns kCols output columns at a time; lane l owns
-// blocks l, l+64, ... of each of them.  Per-lane f32 partial sums are reduced
-// across the wavefront with DPP at the end of each column group.
-// =====================================================================
-
-template <int kType>
-struct GemvLane;
-
-// Q4_0: one lane = one block (16 B of nibbles).  Nibbles stay unsigned:
-// dot(qx, n-8) = dot(qx, n) - 8*sum(qx), with sum(qx) from the prologue.
-template <>
-struct GemvLane<2> {
-    static constexpr int kLanesPerBlock = 1;
-    uint32_t lo[4], hi[4];
-    float d;
-    __device__ __forceinline__ void load(const uint4* qs, const uint16_t* ds, size_t block_index, int /*half*/) {
-        const uint4 v = qs[block_index];
-        const uint32_t p[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            lo[j] = p[j] & 0x0F0F0F0Fu;
-            hi[j] = (p[j] >> 4) & 0x0F0F0F0Fu;
-        }
-        d = half_bits_to_f32(ds[block_index]);
-    }
-    // a: this block's 32 int8 activations (8 dwords), sum: their int32 sum
-    __device__ __forceinline__ int dot(const int8_t* a_lds, int sum, int /*half*/) const {
-        const int4 a0 = reinterpret_cast<const int4*>(a_lds)[0];
-        const int4 a1 = reinterpret_cast<const int4*>(a_lds)[1];
-        int acc = -8 * sum;
-        acc = dot4(static_cast<int>(lo[0]), a0.x, acc);
-        acc = dot4(static_cast<int>(lo[1]), a0.y, acc);
-        acc = dot4(static_cast<int>(lo[2]), a0.z, acc);
-        acc = dot4(static_cast<int>(lo[3]), a0.w, acc);
-        acc = dot4(static_cast<int>(hi[0]), a1.x, acc);
-        acc = dot4(static_cast<int>(hi[1]), a1.y, acc);
-        acc = dot4(static_cast<int>(hi[2]), a1.z, acc);
-        acc = dot4(static_cast<int>(hi[3]), a1.w, acc);
-        return acc;
-    }
-};
-
-// Q8_0: two lanes = one block (16 B of int8 each); halves are added with one DPP.
-template <>
-struct GemvLane<8> {
-    static constexpr int kLanesPerBlock = 2;
-    int q[4];
-    float d;
-    __device__ __forceinline__ void load(const uint4* qs, const uint16_t* ds, size_t block_index, int half) {
-        const uint4 v = qs[2 * block_index + half];
-        q[0] = v.x; q[1] = v.y; q[2] = v.z; q[3] = v.w;
-        d = half_bits_to_f32(ds[block_index]);
-    }
-    __device__ __forceinline__ int dot(const int8_t* a_lds, int /*sum*/, int half) const {
-        const int4 a = reinterpret_cast<const int4*>(a_lds)[half];
-        int acc = dot4(q[0], a.x, 0);
-        acc = dot4(q[1], a.y, acc);
-        acc = dot4(q[2], a.z, acc);
-        acc = dot4(q[3], a.w, acc);
-        acc += dpp_move<kDppXor1>(acc);  // both lanes of the pair now hold the block dot
-        return acc;
-    }
-};
-
-template <int kType, int kRows, int kCols, bool kWriteDots>
-__global__ void gemv_fused_kernel(float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input,
-                                  const uint8_t* __restrict__ weight, int in_dim, int out_dim) {
-    using Lane = GemvLane<kType>;
-    constexpr int kLpb = Lane::kLanesPerBlock;
-    constexpr int kBlocksPerStep = kWave / kLpb;
-    constexpr int kQuantBytes = kType == 2 ? 16 : 32;
-
-    extern __shared__ __align__(16) unsigned char lds[];
-    const int kb = in_dim >> 5;
-    int8_t* qx = reinterpret_cast<int8_t*>(lds);                        // [kRows][in_dim]
-    float* sx = reinterpret_cast<float*>(lds + static_cast<size_t>(kRows) * in_dim);  // [kRows][kb]
-    int* sumx = reinterpret_cast<int*>(sx + kRows * kb);                // [kRows][kb]
-
-    const size_t blocks = static_cast<size_t>(out_dim) * kb;
-    const uint4* qs = reinterpret_cast<const uint4*>(weight);
-    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * kQuantBytes);
-
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x >> 6;
-    const int waves_per_wg = blockDim.x >> 6;
-    const int half = lane & (kLpb - 1);
-    const int lane_block = lane / kLpb;
-
-    const int groups = (out_dim + kCols - 1) / kCols;
-    const int wave_global = blockIdx.x * waves_per_wg + wave;
-    const int wave_stride = gridDim.x * waves_per_wg;
-
-    quantize_rows_to_lds(input, kRows, in_dim, qx, sx, sumx);
-    __syncthreads();
-
-    for (int g = wave_global; g < groups; g += wave_stride) {
-        const int o0 = g * kCols;
-        float acc[kRows][kCols];
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int c = 0; c < kCols; ++c) acc[r][c] = 0.0f;
-
-        for (int b = lane_block; b < kb; b += kBlocksPerStep) {
-            Lane w[kCols];
-#pragma unroll
-            for (int c = 0; c < kCols; ++c) {
-                const int o = min(o0 + c, out_dim - 1);  // clamp: tail columns recompute the last one
-                w[c].load(qs, ds, static_cast<size_t>(o) * kb + b, half);
-            }
-#pragma unroll
-            for (int r = 0; r < kRows; ++r) {
-                const int8_t* a = qx + static_cast<size_t>(r) * in_dim + b * 32;
-                const float s = sx[r * kb + b];
-                const int sm = sumx[r * kb + b];
-#pragma unroll
-                for (int c = 0; c < kCols; ++c) {
-                    const int dot = w[c].dot(a, sm, half);
-                    if (kWriteDots) {
-                        if (half == 0 && o0 + c < out_dim)
-                            dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + b] = dot;
-                    }
-                    const float t = s * w[c].d;
-                    const float term = t * static_cast<float>(dot);
-                    acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
-                }
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int c = 0; c < kCols; ++c) {
-                const float total = wave_sum(acc[r][c]);
-                if (lane == 0 && o0 + c < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + c] = total;
-            }
-    }
-}
-
-// =====================================================================
 // Launchers
 // =====================================================================
 
@@ -274,64 +129,7 @@ namespace {
 
 hipError_t launch_status() { return hipGetLastError(); }
 
-template <int kType, int kRows, bool kDots>
-hipError_t launch_gemv_rows(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight,
-                            int in_dim, int out_dim, const GemvTuning& tune) {
-    constexpr int kCols = kRows <= 2 ? 4 : 2;
-    const int kb = in_dim / 32;
-    const size_t lds = static_cast<size_t>(kRows) * in_dim + static_cast<size_t>(kRows) * kb * 8;
-    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
-    // Raising the dynamic-LDS limit is sticky per kernel: do it once, outside any
-    // stream capture a caller may have open later.
-    static size_t lds_limit = 64 * 1024;
-    if (lds > lds_limit) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-        if (e != hipSuccess) return e;
-        lds_limit = 128 * 1024;
-    }
-    const int threads = tune.threads;
-    const int waves_per_wg = threads / 64;
-    const int groups = (out_dim + kCols - 1) / kCols;
-    int grid = (groups + waves_per_wg - 1) / waves_per_wg;
-    if (grid > tune.max_workgroups) grid = tune.max_workgroups;
-    if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, dst, dots, input, weight, in_dim, out_dim);
-    return launch_status();
-}
-
-template <int kType, bool kDots>
-hipError_t launch_gemv(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight, int rows,
-                       int in_dim, int out_dim, const GemvTuning& tune) {
-    switch (rows) {
-        case 1: return launch_gemv_rows<kType, 1, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 2: return launch_gemv_rows<kType, 2, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 3: return launch_gemv_rows<kType, 3, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 4: return launch_gemv_rows<kType, 4, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 5: return launch_gemv_rows<kType, 5, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 6: return launch_gemv_rows<kType, 6, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 7: return launch_gemv_rows<kType, 7, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 8: return launch_gemv_rows<kType, 8, kDots>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        default: return hipErrorInvalidValue;
-    }
-}
-
 }  // namespace
-
-size_t gemv_fused_lds_bytes(int rows, int in_dim) {
-    return static_cast<size_t>(rows) * in_dim + static_cast<size_t>(rows) * (in_dim / 32) * 8;
-}
-
-hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
-                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
-                             const GemvTuning& tune) {
-    if (tensor_type == 2) {
-        return dots ? launch_gemv<2, true>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune)
-                    : launch_gemv<2, false>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
-    }
-    return dots ? launch_gemv<8, true>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune)
-                : launch_gemv<8, false>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
-}
 
 hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
                                        float* scale, int* sum) {

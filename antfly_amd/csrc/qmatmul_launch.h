@@ -10,11 +10,12 @@ namespace afhip {
 // Launch geometry of the fused GEMV; chosen host-side (ops/cuda/kernels.zig
 // does the same for its launch1d / launchBlocks helpers).
 struct GemvTuning {
-    int threads = 256;          // workgroup size, multiple of 64
-    int max_workgroups = 2048;  // persistent-grid cap
+    int threads = 256;  // workgroup size, multiple of 64 (rounded to whole column groups)
+    bool wide = false;  // rows <= 2: twice the output columns per wavefront
 };
 
 size_t gemv_fused_lds_bytes(int rows, int in_dim);
+int gemv_fused_max_in_dim();
 
 // rows in 1..8, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,

@@ -80,6 +80,18 @@ def test_activation_quantizer_bit_exact(rows, in_dim):
     if in_dim >= 64:
         x[rows - 1, 32:64] = [127.0, 0.5, -0.5, 1.5, -1.5, 126.5, -2.5] + [0.25] * 25  # ties
         x[rows - 1, -32:] *= 1e-30        # tiny magnitudes
+    if in_dim >= 4096:
+        # every half-integer and its two float neighbours, both signs: block max 127 makes
+        # the scale and its reciprocal exactly 1, so these hit the rounding rule directly
+        k = np.arange(0, 127, dtype=np.float32) + np.float32(0.5)
+        edge = np.concatenate([k, np.nextafter(k, np.float32(0)), np.nextafter(k, np.float32(200)),
+                               [0.49999997, 0.25, 126.99999, 127.0]]).astype(np.float32)
+        edge = np.concatenate([edge, -edge])
+        nblk = (edge.size + 30) // 31
+        pad = np.zeros(nblk * 31, np.float32)
+        pad[: edge.size] = edge
+        blocks = np.concatenate([np.full((nblk, 1), 127.0, np.float32), pad.reshape(nblk, 31)], axis=1)
+        x[0, 64 : 64 + blocks.size] = blocks.reshape(-1)
     qw, sw, sumw = O.quantize_activation_rows(x, rows, in_dim)
     xd = G.to_dev(x)
     q = torch.empty(rows * in_dim, dtype=torch.int8, device=G.DEV)
