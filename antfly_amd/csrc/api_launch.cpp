@@ -39,11 +39,17 @@ static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
     return v;
 }
 
+// From this many rows on, activations are quantized by a separate kernel.
+constexpr size_t kGemvPrequantizeRows = 3;
+
 // LDS the fused GEMV may use per workgroup; gfx950 has 160 KiB per CU.
 constexpr size_t kGemvLdsBudget = 96 * 1024;
 
+// Rows one GEMV launch takes: as many as fit the LDS budget (1-2 rows quantize
+// in the kernel's own prologue, more use separately quantized activations).
+constexpr int kGemvMaxRowsPerLaunch = 16;
 static int gemv_row_chunk(size_t rows, size_t in_dim) {
-    int chunk = rows < 8 ? static_cast<int>(rows) : 8;
+    int chunk = rows < kGemvMaxRowsPerLaunch ? static_cast<int>(rows) : kGemvMaxRowsPerLaunch;
     while (chunk > 0 && gemv_fused_lds_bytes(chunk, static_cast<int>(in_dim)) > kGemvLdsBudget) --chunk;
     return chunk;
 }
@@ -63,8 +69,6 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
     // every workgroup quantizes all of X, so large workgroups share that work best
     t.threads = 1024;
     if (env_threads >= 64 && env_threads <= 1024 && env_threads % 64 == 0) t.threads = env_threads;
-    static const int env_wide = env_int("AFHIP_GEMV_WIDE");
-    t.wide = env_wide != 0;
     return t;
 }
 
@@ -122,17 +126,36 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     if (fused_ok) {
         // mmv / small_batch: rows <= 8 in one launch.  mm (rows >= 9): same kernel
         // over 8-row slices until the MFMA GEMM takes over.
+        // One or two rows: the GEMV quantizes X in its own prologue (one launch).
+        // More rows: every workgroup would repeat that work, so X is quantized once
+        // by its own kernel into the caller's scratch.
+        const bool prequantize = rows >= kGemvPrequantizeRows;
+        const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
+        if (prequantize && (workspace.ptr == 0 || workspace.len < ws.bytes || workspace.ptr % 16 != 0))
+            return AFHIP_ERR_INVALID_STATE;
         if (counters) {
             if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
             else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
             else counters->mm++;
+            if (prequantize) counters->activation_quant++;
+        }
+        if (prequantize) {
+            hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx,
+                                                       ws.sx, ws.sums);
+            if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         for (size_t r0 = 0; r0 < rows; r0 += static_cast<size_t>(chunk)) {
             const int nr = rows - r0 < static_cast<size_t>(chunk) ? static_cast<int>(rows - r0) : chunk;
             const GemvTuning tune = gemv_tuning(tensor_type, nr, in_dim, out_dim);
+            GemvActivations pre;
+            if (prequantize) {
+                pre.q = ws.qx + r0 * in_dim;
+                pre.scale = ws.sx + r0 * kb;
+                pre.sum = ws.sums + r0 * kb;
+            }
             hipError_t e = launch_gemv_fused(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
-                                             want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, w, nr,
-                                             static_cast<int>(in_dim), static_cast<int>(out_dim), tune);
+                                             want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, pre, w,
+                                             nr, static_cast<int>(in_dim), static_cast<int>(out_dim), tune);
             if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         return AFHIP_OK;

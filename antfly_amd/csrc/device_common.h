@@ -69,6 +69,44 @@ __device__ __forceinline__ float wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// Reduces kCount per-lane values across the wavefront at once ("transposed"
+// reduction): every exchange step halves the number of live values instead of
+// running one full butterfly per value.  kCount must be a power of two <= 16.
+// On return lane l holds in v[0] the wavefront total of value (l % kCount).
+// Exchanges: quad_perm xor 1, quad_perm xor 2, row rotate by 4, row rotate by 8
+// inside a 16-lane row (all keep the lane's low bits, which select the values it
+// keeps), then ds_swizzle xor 16 and a 64-lane permute for the four rows.
+constexpr int kDppRor4 = 0x124;  // row_ror:4
+constexpr int kDppRor8 = 0x128;  // row_ror:8
+
+template <int kCtrl, int kLive>
+__device__ __forceinline__ void halve_step(float* v, bool keep_odd) {
+#pragma unroll
+    for (int i = 0; i < kLive / 2; ++i) {
+        const float keep = keep_odd ? v[2 * i + 1] : v[2 * i];
+        const float send = keep_odd ? v[2 * i] : v[2 * i + 1];
+        v[i] = keep + dpp_move<kCtrl>(send);
+    }
+}
+
+template <int kCount>
+__device__ __forceinline__ void wave_sum_transposed(float* v, int lane) {
+    static_assert(kCount == 1 || kCount == 2 || kCount == 4 || kCount == 8 || kCount == 16, "power of two <= 16");
+    if (kCount >= 2) halve_step<kDppXor1, kCount>(v, (lane & 1) != 0);
+    else v[0] += dpp_move<kDppXor1>(v[0]);
+    if (kCount >= 4) halve_step<kDppXor2, kCount / 2>(v, (lane & 2) != 0);
+    else v[0] += dpp_move<kDppXor2>(v[0]);
+    if (kCount >= 8) halve_step<kDppRor4, kCount / 4>(v, (lane & 4) != 0);
+    else v[0] += dpp_move<kDppRor4>(v[0]);
+    if (kCount >= 16) halve_step<kDppRor8, kCount / 8>(v, (lane & 8) != 0);
+    else v[0] += dpp_move<kDppRor8>(v[0]);
+    // rows: xor 16 inside each half (ds_swizzle bit mode: and 0x1f, or 0, xor 0x10), then xor 32
+    float t = v[0];
+    t += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, t), 0x401F));
+    t += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, t)));
+    v[0] = t;
+}
+
 // ---- activation quantizer for one value, given its block's max |x|
 // (ops/native_compute.zig:11998-12028): f32 scale, one reciprocal, round half
 // away from zero, clamp to +-127.
@@ -86,32 +124,6 @@ __device__ __forceinline__ int act_quant(float x, float inv_scale) {
     const float t = x * inv_scale;
     const float u = t + __builtin_copysignf(0x1.fffffep-2f, t);
     return static_cast<int>(__builtin_amdgcn_fmed3f(u, -127.75f, 127.75f));
-}
-
-// Quantizes `rows * in_dim` activations into shared memory with every thread of
-// the workgroup: 8 consecutive lanes own one 32-value block (one float4 each).
-//   q     int8  [rows][in_dim]
-//   scale f32   [rows][in_dim/32]
-//   sum   int32 [rows][in_dim/32]   (sum of the block's int8 values)
-__device__ __forceinline__ void quantize_rows_to_lds(const float* __restrict__ x, int rows, int in_dim,
-                                                     int8_t* q, float* scale, int* sum) {
-    const int units = rows * (in_dim >> 2);  // float4 units; in_dim % 32 == 0
-    for (int u = threadIdx.x; u < units; u += blockDim.x) {
-        float4 v = reinterpret_cast<const float4*>(x)[u];
-        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        m = max_over_8(m);
-        const float s = act_scale(m);
-        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
-        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
-        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
-        const int packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-        reinterpret_cast<int*>(q)[u] = packed;
-        const int total = sum_over_8(q0 + q1 + q2 + q3);
-        if ((u & 7) == 0) {
-            scale[u >> 3] = s;
-            sum[u >> 3] = total;
-        }
-    }
 }
 
 // ---- weight block readers.  A "block view" yields the 32 weights of block

@@ -83,13 +83,16 @@ __device__ __forceinline__ void quantize_block_to_lds(const float4 (&v)[8], int 
     sum_row[block] = total;
 }
 
-// Workgroups hold at most 1024 threads for 1-2 rows and 512 beyond that (more
-// registers per lane for the extra accumulators).
-constexpr int gemv_max_threads(int rows) { return rows <= 2 ? 1024 : 512; }
+constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
-template <int kType, int kRows, int kCols, bool kWriteDots>
-__global__ __launch_bounds__(gemv_max_threads(kRows)) void gemv_fused_kernel(float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input,
-                                  const uint8_t* __restrict__ weight, int in_dim, int out_dim, int slices) {
+// kFused: quantize f32 `input` in the prologue.  Otherwise the activations were
+// quantized by quantize_activations_kernel (natural order: pre_q [rows][in_dim]
+// int8, pre_scale / pre_sum [rows][in_dim/32]) and the prologue only copies them.
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kFused>
+__global__ __launch_bounds__(1024) void gemv_fused_kernel(
+    float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input, const int4* __restrict__ pre_q,
+    const float* __restrict__ pre_scale, const int* __restrict__ pre_sum, const uint8_t* __restrict__ weight, int in_dim,
+    int out_dim, int slices) {
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
     constexpr int kBlocksPerStep = kWave / kLpb;
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(gemv_max_threads(kRows)) void gemv_fused_kernel(flo
     // ---- 1. first activation requests, then every weight byte this wavefront needs
     const int x_blocks = kRows * kb;  // one thread quantizes one block
     float4 xpre[8];
-    {
+    if (kFused) {
         const int xb = tid < x_blocks ? tid : 0;
 #pragma unroll
         for (int i = 0; i < 8; ++i) xpre[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
@@ -152,17 +155,33 @@ __global__ __launch_bounds__(gemv_max_threads(kRows)) void gemv_fused_kernel(flo
         }
     }
 
-    // ---- 2. quantize X into LDS, one thread per block
-    if (tid < x_blocks) {
-        const int r = tid / kb, b = tid - r * kb;
-        quantize_block_to_lds<kType>(xpre, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-    }
-    for (int xb = tid + static_cast<int>(blockDim.x); xb < x_blocks; xb += blockDim.x) {
-        float4 v[8];
+    // ---- 2. quantized X into LDS
+    if (kFused) {  // one thread per block
+        if (tid < x_blocks) {
+            const int r = tid / kb, b = tid - r * kb;
+            quantize_block_to_lds<kType>(xpre, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+        }
+        for (int xb = tid + static_cast<int>(blockDim.x); xb < x_blocks; xb += blockDim.x) {
+            float4 v[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
-        const int r = xb / kb, b = xb - r * kb;
-        quantize_block_to_lds<kType>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+            for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
+            const int r = xb / kb, b = xb - r * kb;
+            quantize_block_to_lds<kType>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+        }
+    } else {  // coalesced copy, 16 bytes (half a block) per thread
+        const int row_int4 = in_dim >> 4;
+        for (int u = tid; u < kRows * row_int4; u += blockDim.x) {
+            int idx = u;
+            if (kType == 2) {
+                const int r = u / row_int4, w = u - r * row_int4;
+                idx = r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
+            }
+            reinterpret_cast<int4*>(qx)[idx] = pre_q[u];
+        }
+        for (int u = tid; u < x_blocks; u += blockDim.x) {
+            sx[u] = pre_scale[u];
+            sumx[u] = pre_sum[u];
+        }
     }
     __syncthreads();
 
@@ -219,38 +238,202 @@ __global__ __launch_bounds__(gemv_max_threads(kRows)) void gemv_fused_kernel(flo
                 const float term = tscale * static_cast<float>(dot);
                 acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
             }
-            // keep one row's activations live at a time: without this fence the
-            // scheduler hoists every row's LDS reads and spills registers
-            if (kRows > 2) __builtin_amdgcn_sched_barrier(0);
         }
     }
 
-    // ---- 4. wavefront reduction, then K-slices in slice order
+    // ---- 4. wavefront reduction (all rows x columns at once), then K-slices in slice order
+    constexpr int kCells = kRows * kCols;
+    constexpr int kPadded = pow2_at_least(kCells);
+    static_assert(kCells <= 16, "at most 16 accumulators per lane");
+    float red[kPadded];
+#pragma unroll
+    for (int i = 0; i < kPadded; ++i) red[i] = i < kCells ? acc[i / kCols][i % kCols] : 0.0f;
+    wave_sum_transposed<kPadded>(red, lane);
+    const int cell = lane & (kPadded - 1);  // this lane holds the total of accumulator `cell`
+    const int cr = cell / kCols, cc = cell - cr * kCols;
     if (slices == 1) {
-#pragma unroll
-        for (int r = 0; r < kRows; ++r)
-#pragma unroll
-            for (int c = 0; c < kCols; ++c) {
-                const float total = wave_sum(acc[r][c]);
-                if (lane == 0 && o0 + c < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + c] = total;
-            }
+        if (lane < kPadded && cell < kCells && o0 + cc < out_dim && dst)
+            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
         return;
     }
-#pragma unroll
-    for (int r = 0; r < kRows; ++r)
-#pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            const float total = wave_sum(acc[r][c]);
-            if (lane == 0) partial[wave * (kRows * kCols) + r * kCols + c] = total;
-        }
+    if (lane < kPadded && cell < kCells) partial[wave * kCells + cell] = red[0];
     __syncthreads();
-    const int cells = groups_per_wg * kRows * kCols;
-    for (int i = threadIdx.x; i < cells; i += blockDim.x) {
-        const int gi = i / (kRows * kCols), rc = i - gi * (kRows * kCols);
+    const int cells = groups_per_wg * kCells;
+    for (int i = tid; i < cells; i += blockDim.x) {
+        const int gi = i / kCells, rc = i - gi * kCells;
         const int r = rc / kCols, c = rc - r * kCols;
         const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
         float total = 0.0f;
-        for (int s = 0; s < slices; ++s) total += partial[(gi * slices + s) * (kRows * kCols) + rc];
+        for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
+        if (o < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o] = total;
+    }
+}
+
+// =====================================================================
+// Same work decomposition for 3 or more rows, activations quantized beforehand
+// by quantize_activations_kernel.  The wavefront keeps its weights (unpacked
+// once) in registers and walks the rows two at a time, so register use does not
+// grow with the row count; `rows` is a run-time value bounded only by LDS.
+// =====================================================================
+template <int kType, int kCols, bool kWriteDots>
+__global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ dst, int* __restrict__ dots,
+                                                            const int4* __restrict__ pre_q,
+                                                            const float* __restrict__ pre_scale,
+                                                            const int* __restrict__ pre_sum,
+                                                            const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                            int out_dim, int slices) {
+    using F = GemvFormat<kType>;
+    constexpr int kLpb = F::kLanesPerBlock;
+    constexpr int kBlocksPerStep = kWave / kLpb;
+    constexpr int kSteps = F::kSteps;
+    constexpr int kWords = kType == 2 ? 8 : 4;  // int8x4 words of weights per lane per step
+
+    extern __shared__ __align__(16) unsigned char lds[];
+    const int kb = in_dim >> 5;
+    const int row_dwords = in_dim >> 2;
+    int* qx = reinterpret_cast<int*>(lds);                                          // [rows][in_dim] bytes
+    float* sx = reinterpret_cast<float*>(lds + static_cast<size_t>(rows) * in_dim);  // [rows][kb]
+    int* sumx = reinterpret_cast<int*>(sx + rows * kb);                              // [rows][kb]
+    float* partial = reinterpret_cast<float*>(sumx + rows * kb);                     // [waves][rows*kCols]
+
+    const size_t blocks = static_cast<size_t>(out_dim) * kb;
+    const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
+    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int waves = blockDim.x >> 6;
+    const int half = lane & (kLpb - 1);
+    const int lane_block = lane / kLpb;
+    const int slice = wave % slices;
+    const int groups_per_wg = waves / slices;
+    const int group = blockIdx.x * groups_per_wg + wave / slices;
+    const int o0 = group * kCols;
+    const bool active = o0 < out_dim;
+
+    // ---- 1. every weight byte this wavefront needs
+    int wv[kSteps][kCols][kWords];
+    float wd[kSteps][kCols];
+    int blk[kSteps];
+    bool ok[kSteps];
+#pragma unroll
+    for (int j = 0; j < kSteps; ++j) {
+        const int b = slice * kSliceBlocks + j * kBlocksPerStep + lane_block;
+        ok[j] = active && b < kb;
+        blk[j] = b < kb ? b : kb - 1;
+    }
+    {
+        u32x4 raw[kSteps][kCols];
+        uint16_t rawd[kSteps][kCols];
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) {
+            const int o = min(o0 + c, out_dim - 1);
+            const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
+            const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
+#pragma unroll
+            for (int j = 0; j < kSteps; ++j) {
+                raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+                rawd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
+            }
+        }
+
+        // ---- 2. quantized X into LDS: coalesced copy, 16 bytes (half a block) per thread
+        const int row_int4 = in_dim >> 4;
+        for (int u = tid; u < rows * row_int4; u += blockDim.x) {
+            int idx = u;
+            if (kType == 2) {
+                const int r = u / row_int4, w = u - r * row_int4;
+                idx = r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
+            }
+            reinterpret_cast<int4*>(qx)[idx] = pre_q[u];
+        }
+        for (int u = tid; u < rows * kb; u += blockDim.x) {
+            sx[u] = pre_scale[u];
+            sumx[u] = pre_sum[u];
+        }
+
+        // unpack once; lanes that own no block get a zero scale
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j)
+#pragma unroll
+            for (int c = 0; c < kCols; ++c) {
+                const u32x4 w = raw[j][c];
+                if (kType == 2) {
+                    wv[j][c][0] = w.x & 0x0F0F0F0Fu; wv[j][c][1] = w.y & 0x0F0F0F0Fu;
+                    wv[j][c][2] = w.z & 0x0F0F0F0Fu; wv[j][c][3] = w.w & 0x0F0F0F0Fu;
+                    wv[j][c][4] = (w.x >> 4) & 0x0F0F0F0Fu; wv[j][c][5] = (w.y >> 4) & 0x0F0F0F0Fu;
+                    wv[j][c][6] = (w.z >> 4) & 0x0F0F0F0Fu; wv[j][c][7] = (w.w >> 4) & 0x0F0F0F0Fu;
+                } else {
+                    wv[j][c][0] = w.x; wv[j][c][1] = w.y; wv[j][c][2] = w.z; wv[j][c][3] = w.w;
+                }
+                wd[j][c] = (ok[j] && (kLpb == 1 || half == 0)) ? half_bits_to_f32(rawd[j][c]) : 0.0f;
+            }
+    }
+    __syncthreads();
+
+    // ---- 3. two rows per pass
+    const int cells = rows * kCols;
+    for (int r0 = 0; r0 < rows; r0 += 2) {
+        const int r1 = r0 + 1 < rows ? r0 + 1 : r0;  // odd row count: the last pass repeats its row
+        float acc[2][kCols];
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) acc[0][c] = acc[1][c] = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int b = blk[j];
+#pragma unroll
+            for (int rr = 0; rr < 2; ++rr) {
+                const int r = rr == 0 ? r0 : r1;
+                const float s = sx[r * kb + b];
+                int a[8];
+                int sm = 0;
+                if (kType == 2) {
+                    const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b];
+                    const int4 a1 = reinterpret_cast<const int4*>(qx + r * row_dwords + (row_dwords >> 1))[b];
+                    a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
+                    a[4] = a1.x; a[5] = a1.y; a[6] = a1.z; a[7] = a1.w;
+                    sm = sumx[r * kb + b];
+                } else {
+                    const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b * 2 + half];
+                    a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
+                }
+#pragma unroll
+                for (int c = 0; c < kCols; ++c) {
+                    int dot = kType == 2 ? -8 * sm : 0;  // unsigned nibbles: dot(qx, n - 8) = dot(qx, n) - 8 sum(qx)
+#pragma unroll
+                    for (int i = 0; i < kWords; ++i) dot = dot4(wv[j][c][i], a[i], dot);
+                    if (kLpb == 2) dot += dpp_move<kDppXor1>(dot);
+                    if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim && (rr == 0 || r1 != r0))
+                        dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + b] = dot;
+                    const float tscale = s * wd[j][c];
+                    acc[rr][c] += tscale * static_cast<float>(dot);
+                }
+            }
+        }
+        constexpr int kPadded = pow2_at_least(2 * kCols);
+        float red[kPadded];
+#pragma unroll
+        for (int i = 0; i < kPadded; ++i) red[i] = i < 2 * kCols ? acc[i / kCols][i % kCols] : 0.0f;
+        wave_sum_transposed<kPadded>(red, lane);
+        const int cell = lane & (kPadded - 1);
+        const int rr = cell / kCols, cc = cell - rr * kCols;
+        const bool mine = lane < kPadded && cell < 2 * kCols && (rr == 0 || r1 != r0);
+        const int r = rr == 0 ? r0 : r1;
+        if (slices == 1) {
+            if (mine && o0 + cc < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + cc] = red[0];
+        } else if (mine) {
+            partial[wave * cells + r * kCols + cc] = red[0];
+        }
+    }
+    if (slices == 1) return;
+    __syncthreads();
+    for (int i = tid; i < groups_per_wg * cells; i += blockDim.x) {
+        const int gi = i / cells, rc = i - gi * cells;
+        const int r = rc / kCols, c = rc - r * kCols;
+        const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
+        float total = 0.0f;
+        for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * cells + rc];
         if (o < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o] = total;
     }
 }
@@ -259,76 +442,95 @@ __global__ __launch_bounds__(gemv_max_threads(kRows)) void gemv_fused_kernel(flo
 
 namespace {
 
-template <int kType, int kRows, int kCols>
-hipError_t launch_gemv_cols(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight,
-                            int in_dim, int out_dim, const GemvTuning& tune) {
-    const int kb = in_dim / 32;
-    const int slices = (kb + kSliceBlocks - 1) / kSliceBlocks;
-    if (slices > 16) return hipErrorInvalidValue;  // callers route in_dim > 65536 elsewhere
-    int waves = (tune.threads < gemv_max_threads(kRows) ? tune.threads : gemv_max_threads(kRows)) / 64;
+int workgroup_waves(int requested_threads, int max_threads, int slices) {
+    int waves = (requested_threads < max_threads ? requested_threads : max_threads) / 64;
     if (waves < slices) waves = slices;
-    waves = waves / slices * slices;  // whole column groups per workgroup
+    return waves / slices * slices;  // whole column groups per workgroup
+}
+
+// Raising the dynamic-LDS limit is sticky per kernel: done once per kernel, outside
+// any stream capture a caller may open later.
+template <typename Kernel>
+hipError_t allow_large_lds(Kernel kernel, size_t lds, size_t* limit) {
+    if (lds <= *limit) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       128 * 1024);
+    if (e == hipSuccess) *limit = 128 * 1024;
+    return e;
+}
+
+template <int kType, int kRows, bool kDots>
+hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight, int in_dim,
+                        int out_dim, const GemvTuning& tune) {
+    constexpr int kCols = kType == 2 ? 4 : 2;
+    const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
+    const int waves = workgroup_waves(tune.threads, 1024, slices);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
-    auto kernel = dots ? gemv_fused_kernel<kType, kRows, kCols, true> : gemv_fused_kernel<kType, kRows, kCols, false>;
-    // Raising the dynamic-LDS limit is sticky per kernel: do it once, outside any
-    // stream capture a caller may open later.
+    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots, true>;
     static size_t lds_limit = 64 * 1024;
-    if (lds > lds_limit) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-        if (e != hipSuccess) return e;
-        lds_limit = 128 * 1024;
-    }
+    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int groups = (out_dim + kCols - 1) / kCols;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, weight, in_dim, out_dim,
-                       slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, nullptr, nullptr, nullptr,
+                       weight, in_dim, out_dim, slices);
     return hipGetLastError();
 }
 
-template <int kType, int kRows>
-hipError_t launch_gemv_rows(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight,
-                            int in_dim, int out_dim, const GemvTuning& tune) {
-    constexpr int kCols = kType == 2 ? (kRows <= 4 ? 4 : 2) : 2;
-    if constexpr (kRows <= 2) {
-        if (tune.wide)
-            return launch_gemv_cols<kType, kRows, 2 * kCols>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-    }
-    return launch_gemv_cols<kType, kRows, kCols>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+template <int kType, bool kDots>
+hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const GemvActivations& pre, const uint8_t* weight,
+                       int rows, int in_dim, int out_dim, const GemvTuning& tune) {
+    constexpr int kCols = kType == 2 ? 4 : 2;
+    const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
+    const int waves = workgroup_waves(tune.threads, 512, slices);
+    const int groups_per_wg = waves / slices;
+    const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
+    auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
+    static size_t lds_limit = 64 * 1024;
+    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
+    const int groups = (out_dim + kCols - 1) / kCols;
+    const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, reinterpret_cast<const int4*>(pre.q),
+                       pre.scale, pre.sum, weight, rows, in_dim, out_dim, slices);
+    return hipGetLastError();
 }
 
 template <int kType>
-hipError_t launch_gemv(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight, int rows,
-                       int in_dim, int out_dim, const GemvTuning& tune) {
-    switch (rows) {
-        case 1: return launch_gemv_rows<kType, 1>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 2: return launch_gemv_rows<kType, 2>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 3: return launch_gemv_rows<kType, 3>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 4: return launch_gemv_rows<kType, 4>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 5: return launch_gemv_rows<kType, 5>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 6: return launch_gemv_rows<kType, 6>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 7: return launch_gemv_rows<kType, 7>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        case 8: return launch_gemv_rows<kType, 8>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
-        default: return hipErrorInvalidValue;
+hipError_t launch_gemv_type(hipStream_t stream, float* dst, int* dots, const float* input, const GemvActivations& pre,
+                            const uint8_t* weight, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
+    if (pre.q != nullptr) {
+        return dots ? launch_rows<kType, true>(stream, dst, dots, pre, weight, rows, in_dim, out_dim, tune)
+                    : launch_rows<kType, false>(stream, dst, dots, pre, weight, rows, in_dim, out_dim, tune);
     }
+    if (rows == 1) {
+        return dots ? launch_fused<kType, 1, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
+                    : launch_fused<kType, 1, false>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+    }
+    if (rows == 2) {
+        return dots ? launch_fused<kType, 2, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
+                    : launch_fused<kType, 2, false>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+    }
+    return hipErrorInvalidValue;  // three or more rows need pre-quantized activations
 }
 
 }  // namespace
 
-// quantized X (int8 + f32 scale + i32 sum per block) plus one partial-sum slot
-// of up to 8 rows x 4 columns for each of up to 16 wavefronts
+// quantized X (int8 + f32 scale + i32 sum per block) plus, for each of up to 16
+// wavefronts, one partial-sum slot per (row, column) it owns (at most 4 columns)
 size_t gemv_fused_lds_bytes(int rows, int in_dim) {
-    return static_cast<size_t>(rows) * in_dim + static_cast<size_t>(rows) * (in_dim / 32) * 8 + 16 * 64 * 4;
+    return static_cast<size_t>(rows) * in_dim + static_cast<size_t>(rows) * (in_dim / 32) * 8 +
+           static_cast<size_t>(16) * (rows < 4 ? 4 : rows) * 4 * 4;
 }
 
 int gemv_fused_max_in_dim() { return 16 * kSliceBlocks * 32; }
 
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
-                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
-                             const GemvTuning& tune) {
-    if (tensor_type == 2) return launch_gemv<2>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
-    return launch_gemv<8>(stream, dst, dots, input, weight_prepared, rows, in_dim, out_dim, tune);
+                             const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
+                             int out_dim, const GemvTuning& tune) {
+    if (in_dim > gemv_fused_max_in_dim()) return hipErrorInvalidValue;
+    if (tensor_type == 2)
+        return launch_gemv_type<2>(stream, dst, dots, input, pre, weight_prepared, rows, in_dim, out_dim, tune);
+    return launch_gemv_type<8>(stream, dst, dots, input, pre, weight_prepared, rows, in_dim, out_dim, tune);
 }
 
 }  // namespace afhip

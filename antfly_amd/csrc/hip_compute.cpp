@@ -162,7 +162,7 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
     s = alloc_device_buffer(self, out_bytes, &device);
     if (s != AFHIP_OK) return s;
     afhip_buffer scratch{0, 0};
-    if (weight->layout == AFHIP_LAYOUT_RAW && afhip_uses_activation_quant(rows, in_dim, out_dim)) {
+    if (afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
         s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);
         if (s != AFHIP_OK) {
             release_device_buffer(self, &device);

@@ -11,16 +11,23 @@ namespace afhip {
 // does the same for its launch1d / launchBlocks helpers).
 struct GemvTuning {
     int threads = 256;  // workgroup size, multiple of 64 (rounded to whole column groups)
-    bool wide = false;  // rows <= 2: twice the output columns per wavefront
 };
 
 size_t gemv_fused_lds_bytes(int rows, int in_dim);
 int gemv_fused_max_in_dim();
 
+// Activations already quantized by launch_quantize_activations (natural order);
+// q == nullptr makes the GEMV quantize `input` itself in its prologue.
+struct GemvActivations {
+    const int8_t* q = nullptr;   // [rows][in_dim]
+    const float* scale = nullptr;  // [rows][in_dim/32]
+    const int* sum = nullptr;      // [rows][in_dim/32]
+};
+
 // rows in 1..8, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
-                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
-                             const GemvTuning& tune);
+                             const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
+                             int out_dim, const GemvTuning& tune);
 
 hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
                                        float* scale, int* sum);
