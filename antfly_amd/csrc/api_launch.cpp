@@ -123,9 +123,23 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     const int chunk = gemv_row_chunk(rows, in_dim);
     const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR &&
                           in_dim <= static_cast<size_t>(gemv_fused_max_in_dim());
+    if (layout == AFHIP_LAYOUT_PREPARED && kind == AFHIP_DISPATCH_MM) {
+        // rows >= 9 (or a plan that asks for mul_mm): quantize X once, then the int8-MFMA GEMM
+        const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
+        if (workspace.ptr == 0 || workspace.len < ws.bytes || workspace.ptr % 16 != 0) return AFHIP_ERR_INVALID_STATE;
+        if (counters) {
+            counters->mm++;
+            counters->activation_quant++;
+        }
+        hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx,
+                                                   ws.sx, ws.sums);
+        if (e != hipSuccess) return static_cast<afhip_status>(e);
+        e = launch_gemm_i8(stream, tensor_type, want_dots ? nullptr : y, dot_out, ws.qx, ws.sx, w, static_cast<int>(rows),
+                           static_cast<int>(in_dim), static_cast<int>(out_dim));
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     if (fused_ok) {
-        // mmv / small_batch: rows <= 8 in one launch.  mm (rows >= 9): same kernel
-        // over 8-row slices until the MFMA GEMM takes over.
+        // mmv / small_batch (also when a plan forces them on more rows: 16-row slices).
         // One or two rows: the GEMV quantizes X in its own prologue (one launch).
         // More rows: every workgroup would repeat that work, so X is quantized once
         // by its own kernel into the caller's scratch.

@@ -29,6 +29,11 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
                              const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
                              int out_dim, const GemvTuning& tune);
 
+// Int8-MFMA GEMM on pre-quantized activations (natural order) and PREPARED
+// weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set.
+hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
+                          const uint8_t* weight_prepared, int rows, int in_dim, int out_dim);
+
 hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
                                        float* scale, int* sum);
 

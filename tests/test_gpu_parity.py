@@ -115,6 +115,7 @@ def test_prepare_weight_is_a_pure_repack(fmt):
 SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (1, 4096, 512), (2, 96, 515), (3, 2048, 640), (4, 4096, 1024), (5, 1120, 513),
     (6, 256, 600), (7, 160, 777), (8, 4096, 512), (9, 256, 512), (17, 512, 530),
+    (33, 96, 513), (64, 1056, 640), (130, 256, 1030), (257, 512, 512),
 ]
 
 
@@ -178,6 +179,8 @@ def test_forced_dispatch_kinds_agree(fmt):
 
 FULL = [
     ("C1", Q8, [1], 4096, 4096),
+    ("C4", Q8, [128, 512], 4096, 4096),
+    ("C4-q4", Q4, [128], 4096, 4096),
     ("C2", Q4, [1, 2, 4, 8], 4096, 14336),
     ("C3", Q4, [1, 5], 14336, 4096),
 ]
@@ -195,10 +198,13 @@ def test_full_size_decode_configs(name, fmt, row_list, in_dim, out_dim):
         ref = prepared.linear(x, rows, workers=8)
         err = G.max_rel_err(y, ref.astype(np.float64))
         assert err <= TOL and err <= TIGHT, err
-        # block dots on a slice of output columns (full tensor would be 1.8M x rows ints)
-        sub = 64
-        dots = G.block_dots(fmt, PREP, x, wd, rows, in_dim, out_dim)[:, :sub]
-        assert np.array_equal(dots, O.block_dots(fmt, x, w[: sub * (in_dim // 32) * O.BLOCK_BYTES[fmt]], rows, in_dim, sub))
+        # block dots on a slice of output columns and rows (the full tensor is rows x out x in/32 ints)
+        sub, rsub = 64, min(rows, 40)
+        wsub = w[: sub * (in_dim // 32) * O.BLOCK_BYTES[fmt]]
+        wsub_d = G.prepare(fmt, wsub, sub, in_dim)
+        dots = G.block_dots(fmt, PREP, x[:rsub], wsub_d, rsub, in_dim, sub,
+                            dispatch=-1 if rows <= 8 else 3)  # rows >= 9: the MFMA kernel
+        assert np.array_equal(dots, O.block_dots(fmt, x[:rsub], wsub, rsub, in_dim, sub))
         # linearity in X is NOT a property of this op (activations are re-quantized);
         # scaling X by a power of two is: scales double, int8 values stay.
         y2 = G.linear(fmt, PREP, x * 2.0, wd, rows, in_dim, out_dim)
