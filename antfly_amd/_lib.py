@@ -87,6 +87,7 @@ SIGNATURES = {
     "afhip_launch_quantize_activations": (_st, [_vp, Buffer, _sz, _sz, Buffer, Buffer, Buffer]),
     "afhip_launch_block_dots": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
+    "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),
     "afhip_compute_destroy": (None, [_vp]),
     "afhip_compute_backend_kind": (_i, [_vp]),

@@ -352,6 +352,15 @@ afhip_status afhip_launch_quantize_activations(void* stream, afhip_buffer input,
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_stream_read(void* stream, afhip_buffer src, afhip_buffer sink) {
+    if (src.len / 16 > 0xffffffffull * 256) return AFHIP_ERR_INVALID_STATE;
+    if (src.len < 16) return AFHIP_OK;
+    if (src.ptr == 0 || src.ptr % 16 != 0 || sink.ptr == 0 || sink.len < 4) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_stream_read(static_cast<hipStream_t>(stream), reinterpret_cast<const uint8_t*>(src.ptr),
+                                      reinterpret_cast<uint32_t*>(sink.ptr), src.len);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {
     if (n * 4 > dst.len || n * 2 > src.len) return AFHIP_ERR_INVALID_STATE;
     if (n == 0) return AFHIP_OK;

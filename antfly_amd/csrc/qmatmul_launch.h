@@ -45,6 +45,8 @@ hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout
 hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
                                  size_t blocks);
 
+hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
+
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);
 
 }  // namespace afhip

@@ -48,6 +48,10 @@ def launchDecodeFp16(stream, dst_f32: Buffer, src_u16: Buffer, n: int) -> None:
     check(_lib.lib().afhip_launch_decode_fp16(stream, dst_f32, src_u16, n))
 
 
+def launchStreamRead(stream, src: Buffer, sink: Buffer) -> None:
+    check(_lib.lib().afhip_launch_stream_read(stream, src, sink))
+
+
 def smokeQ8_0() -> None:
     check(_lib.lib().afhip_smoke_q8_0())
 

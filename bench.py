@@ -151,6 +151,40 @@ def main() -> int:
     # ---- other configurations ---------------------------------------------------------
     if not args.no_extra:
         extra = {}
+
+        def time_stream_read(nbytes_read, steps, copies):
+            """A kernel that only reads `nbytes_read` bytes, launched like the GEMV above."""
+            srcs = [torch.full((nbytes_read,), 1, dtype=torch.uint8, device=dev) for _ in range(copies)]
+            sink = torch.zeros(4, dtype=torch.int32, device=dev)
+            read = _lib.lib().afhip_launch_stream_read
+            bufs = [buf(t) for t in srcs]
+            for i in range(20):
+                read(stream, bufs[i % copies], buf(sink))
+            torch.cuda.synchronize()
+            chunk = max(d for d in range(1, min(steps, 256) + 1) if steps % d == 0)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for i in range(chunk):
+                    read(cs, bufs[i % copies], buf(sink))
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps // chunk):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / steps
+
+        w_bytes = out_dim * (in_dim // 32) * 18
+        t_small = time_stream_read(w_bytes, max(64, args.steps // 4), args.copies)
+        t_large = time_stream_read(8 * w_bytes, 64, 4)
+        extra["stream_read_only"] = {
+            "what": "kernel that only reads N bytes (16 B per lane, all loads at once), same launch pattern",
+            "33MB_us": round(t_small * 1e6, 3), "33MB_GBps": round(w_bytes / t_small / 1e9, 1),
+            "264MB_us": round(t_large * 1e6, 3), "264MB_GBps": round(8 * w_bytes / t_large / 1e9, 1),
+        }
         small_steps = max(50, args.steps // 4)
         for name, fmt, r, k, n in [
             ("q8_gemv_m1_k4096_n4096", Q8, 1, 4096, 4096),

@@ -151,6 +151,12 @@ afhip_status afhip_launch_block_dots(void *stream, int tensor_type, int layout, 
  * (gguf/quant_codec.zig:35-39).  Parity probe for subnormal scales. */
 afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_buffer src_u16, size_t n);
 
+/* Diagnostic with no counterpart in the reference: reads src.len bytes (16 per
+ * lane, every load issued at once) and does nothing else.  bench.py times it
+ * beside the GEMV as "what one launch of this size can draw from HBM", and it is
+ * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
+afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
+
 /* ------------------------------------------------------------------------
  * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
  * vtable entries on this path).  Owns one device context, ONE stream, resident
