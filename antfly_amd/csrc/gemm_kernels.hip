@@ -1,7 +1,7 @@
 // Prefill GEMM (rows >= 9) on CDNA4 int8 MFMA, activation-quantized route
 // (ops/native_compute.zig:13304-13478 for Q8_0, :23427-23775 for Q4_0):
 //   dot[m][n][b] = sum_i qx[m][32b+i] * qw[n][32b+i]            (int32, exact)
-//   y[m][n]      = sum_b (sx[m][b] * sw[n][b]) * f32(dot[m][n][b]), b ascending
+//   y[m][n]      = sum_b (sx[m][b] * sw[n][b]) * f32(dot[m][n][b])
 //
 // Per 32x32 output tile and per pair of blocks (b, b+1) a wavefront issues
 //   2 x v_mfma_i32_32x32x32_i8     the int32 dots of block b and of block b+1
@@ -10,16 +10,28 @@
 //                                  is the correctly rounded f32 product)
 // and then one int->float conversion and one fused multiply-add per element and
 // block on the vector ALU.  All three results share the 32x32 MFMA register
-// layout, so the epilogue is element-wise.  The vector ALU work (2 operations per
-// (m, n, block)) is what bounds this kernel, not the MFMA pipe.
+// layout, so the epilogue is element-wise.  On this chip the vector ALU and the
+// matrix pipe of a SIMD do not run these two halves side by side, so a pair costs
+// their sum; everything else (global loads, LDS traffic, barriers) is arranged to
+// hide behind that.
 //
-// Workgroup tile = (32*kWavesM) rows x (32*kWavesN) columns, one 32x32 tile per
-// wavefront.  The K loop moves in stages of four blocks (128 values): while one
-// stage is consumed from LDS the next is in flight from global memory to
-// registers (double-buffered LDS, one barrier per stage).  LDS keeps operands in
-// MFMA fragment order -- [block][half][row][16 bytes] -- so fragment reads are
-// unit-stride 128-bit reads; Q4_0 nibbles are expanded to int8 once, on the way
-// into LDS.
+// Workgroup = kWavesM x kWavesN output tiles of 32x32, times kSplit wavefronts per
+// tile that share the K loop: a stage holds 2*kSplit blocks and wavefront ks of a
+// tile takes pair ks of every stage.  The kSplit partial sums of a tile are added
+// in LDS at the end, in ks order (so y is a fixed-order sum of kSplit block-ascending
+// partial sums).  Sixteen wavefronts per workgroup put four on every SIMD.
+//
+// Operands reach LDS without passing through registers: activations and Q8_0 weight
+// bytes are fetched with global_load_lds_dwordx4 into a ring of kRing stages (4, or
+// 3 for the widest stages), kRing - 1 stages ahead of the one being consumed.  One
+// such load moves 64 x 16 bytes: whole 128-byte lines of kRowsPerLoad rows, with
+// consecutive lanes on the chunks of one line (one cache-line lookup per eight
+// lanes).  LDS holds a stage row-major with the 16-byte chunk index XOR-swizzled by
+// the row, so that the MFMA fragment reads (one row per lane, same chunk column) of 16
+// consecutive lanes hit 16 different bank groups.  Block scales arrive the same way
+// (f32 activation scales as they are, fp16 weight scales zero-extended to 32 bits
+// and converted when read).  Q4_0 nibble chunks land in a staging area of the slot
+// and are expanded to int8 fragments by the wavefront that fetched them.
 //
 // MFMA operands: A = activations (row = lane % 32 -> m), B = weights (column =
 // lane % 32 -> n); lane / 32 selects bytes [16*(lane/32), +16) of the block.
@@ -37,260 +49,400 @@ namespace afhip {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v32f __attribute__((ext_vector_type(32)));
+typedef float v16f __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kStageBlocks = 4;  // 128 K-values per LDS stage
-constexpr int kPrefetch = 2;     // stages in flight from global memory (even)
-
-// One LDS stage.  Operand planes are [block][half] x rows of 16 bytes; a plane is
-// padded by two rows so that the 16 lanes of a 128-bit store phase (2 rows x 8
-// planes, or 4 rows x 4 plane pairs for Q4_0) fall into 16 different bank groups.
-// Scale planes are padded by 16 floats for the same reason.
-template <int kTM, int kTN>
-struct GemmLds {
-    static constexpr int kPlaneA = kTM + 2, kPlaneB = kTN + 2;
-    static constexpr int kScaleA = kTM + 16, kScaleB = kTN + 16;
-    int4 a[kStageBlocks * 2 * kPlaneA];
-    int4 b[kStageBlocks * 2 * kPlaneB];
-    float sx[kStageBlocks * kScaleA];
-    float sw[kStageBlocks * kScaleB];
+template <int kWavesM, int kWavesN, int kSplit, bool kQ4>
+struct GemmShape {
+    static constexpr int kTiles = kWavesM * kWavesN;
+    static constexpr int kWaves = kTiles * kSplit;
+    static constexpr int kThreads = 64 * kWaves;
+    static constexpr int kTM = 32 * kWavesM, kTN = 32 * kWavesN;
+    static constexpr int kStageBlocks = 2 * kSplit;              // one pair per wavefront and stage
+    static constexpr int kChunksPerRow = 2 * kStageBlocks;       // 16-byte chunks of int8 per row and stage
+    static constexpr int kRowsPerLoad = 64 / kChunksPerRow;      // rows one 64-lane LDS load covers
+    static constexpr int kGroupsA = kTM / kRowsPerLoad, kGroupsB = kTN / kRowsPerLoad;
+    static constexpr int kABytes = kTM * kChunksPerRow * 16, kBBytes = kTN * kChunksPerRow * 16;
+    // LDS keeps a stage of an operand row-major, [row][chunk], with the chunk index
+    // XOR-swizzled by the row so that 16 consecutive rows reading the same chunk
+    // column hit 16 different 16-byte bank groups (a row is 16 * kChunksPerRow bytes,
+    // the banks wrap every 256 bytes).
+    static constexpr int kRowsPerWrap = 16 / kChunksPerRow > 0 ? 16 / kChunksPerRow : 1;
+    __device__ static constexpr int chunk_pos(int row, int chunk) {
+        return row * kChunksPerRow + (chunk ^ ((row / kRowsPerWrap) % kChunksPerRow));
+    }
+    static_assert(kChunksPerRow == 4 || kChunksPerRow == 8 || kChunksPerRow == 16, "swizzle covers rows of 64..256 bytes");
+    static constexpr int kSxBytes = kTM * kStageBlocks * 4, kSwBytes = kTN * kStageBlocks * 4;
+    static constexpr int kRawBytes = kQ4 ? kTN * kStageBlocks * 16 : 0;  // Q4_0 nibble chunks as fetched
+    static constexpr int kStageBytes = kABytes + kBBytes + kSxBytes + kSwBytes + kRawBytes;
+    static constexpr int kReduceBytes = kSplit > 1 ? kSplit * kTM * kTN * 4 : 0;
+    // LDS stages: loads run kRing - 1 stages ahead of the consumer
+    static constexpr int kRing = 4 * kStageBytes <= 160 * 1024 ? 4 : 3;
+    static constexpr int kLdsBytes = kRing * kStageBytes > kReduceBytes ? kRing * kStageBytes : kReduceBytes;
+    static_assert(kSplit == 1 || kSplit == 2 || kSplit == 4 || kSplit == 8, "kSplit");
+    static_assert(kThreads <= 1024, "workgroup size");
+    static_assert(kTM % kRowsPerLoad == 0 && kTN % kRowsPerLoad == 0, "tile rows per load");
+    static_assert(kLdsBytes <= 160 * 1024, "LDS");
 };
 
-template <int kType, int kWavesM, int kWavesN, bool kWriteDots>
-__global__ __launch_bounds__(64 * kWavesM * kWavesN) void gemm_i8_kernel(
+// s_waitcnt for "at most n vector memory operations outstanding" (nothing else waited
+// for).  n is wave-uniform; the instruction needs an immediate.
+__device__ __forceinline__ void wait_vm_outstanding(int n) {
+    // simm16: vmcnt[3:0] | expcnt << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14
+#define AFHIP_WAIT_VM(N) __builtin_amdgcn_s_waitcnt(((N) & 15) | (7 << 4) | (15 << 8) | (((N) >> 4) << 14))
+    switch (n) {
+        case 1: AFHIP_WAIT_VM(1); break;
+        case 2: AFHIP_WAIT_VM(2); break;
+        case 3: AFHIP_WAIT_VM(3); break;
+        case 4: AFHIP_WAIT_VM(4); break;
+        case 5: AFHIP_WAIT_VM(5); break;
+        case 6: AFHIP_WAIT_VM(6); break;
+        case 8: AFHIP_WAIT_VM(8); break;
+        case 10: AFHIP_WAIT_VM(10); break;
+        case 12: AFHIP_WAIT_VM(12); break;
+        default: AFHIP_WAIT_VM(0); break;  // 0, or a count not listed: waiting for everything is always safe
+    }
+#undef AFHIP_WAIT_VM
+}
+
+// One 64-lane load from global memory straight into LDS: lane l's `bytes` at
+// base + voff land at lds_addr + l * max(bytes, 4) (a 2-byte element is zero-extended
+// to 4).  Issued as inline assembly on purpose: the compiler would otherwise make
+// every later LDS read wait for all such loads in flight, which defeats the ring.
+// Completion is tracked with wait_vm_outstanding(); base and lds_addr are wave-uniform.
+// M0 is written without being declared (it is reserved to the compiler, which has no
+// use for it in this kernel: no LDS-direct builtins, no relative register moves).
+__device__ __forceinline__ void lds_load16(const void* base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_load4(const void* base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+__device__ __forceinline__ void lds_load2(const void* base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+}
+
+extern __shared__ __align__(16) unsigned char gemm_lds[];
+
+template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots>
+__global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles) {
-    constexpr int kThreads = 64 * kWavesM * kWavesN;
-    constexpr int kTM = 32 * kWavesM;
-    constexpr int kTN = 32 * kWavesN;
-    using Lds = GemmLds<kTM, kTN>;
+    using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
+    constexpr int kWaves = S::kWaves, kSB = S::kStageBlocks, kRPL = S::kRowsPerLoad, kCPR = S::kChunksPerRow;
+    constexpr int kTM = S::kTM, kTN = S::kTN, kRing = S::kRing;
     constexpr int kQuantBytes = kType == 2 ? 16 : 32;
-    constexpr int kAChunks = kTM * 8;                        // 16-byte chunks of activations per stage
-    constexpr int kBChunks = kTN * (kType == 2 ? 4 : 8);     // 16-byte chunks of weight bytes per stage
-    constexpr int kALoads = (kAChunks + kThreads - 1) / kThreads;
-    constexpr int kBLoads = (kBChunks + kThreads - 1) / kThreads;
-
-    __shared__ GemmLds<kTM, kTN> lds[2];
+    constexpr bool kQ4 = kType == 2;
+    // units of 64 lanes per stage, by kind
+    constexpr int kUnitsA = S::kGroupsA;                          // LDS loads of activation bytes
+    constexpr int kUnitsB = kQ4 ? kTN * kSB / 64 : S::kGroupsB;   // Q8_0: LDS loads; Q4_0: register loads of 16-byte nibble chunks
+    constexpr int kUnitsSx = kTM * kSB / 64, kUnitsSw = kTN * kSB / 64;
+    constexpr int kPerA = (kUnitsA + kWaves - 1) / kWaves, kPerB = (kUnitsB + kWaves - 1) / kWaves;
+    constexpr int kPerSx = (kUnitsSx + kWaves - 1) / kWaves, kPerSw = (kUnitsSw + kWaves - 1) / kWaves;
+    // each kind starts its round-robin over the wavefronts where the previous one stopped
+    constexpr int kStartB = kUnitsA % kWaves, kStartSx = (kStartB + kUnitsB) % kWaves, kStartSw = (kStartSx + kUnitsSx) % kWaves;
 
     const int kb = in_dim >> 5;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / kWavesN, wn = wave % kWavesN;
+    const int ks = wave / S::kTiles, tile = wave % S::kTiles;
+    const int wm = tile / kWavesN, wn = tile % kWavesN;
     const int lj = lane & 31, lh = lane >> 5;
 
     // Workgroups that share a weight tile (same n tile, different m tiles) sit on
     // the same XCD (consecutive workgroup ids go round-robin over the 8 XCDs), so
     // each L2 reads every weight byte once.
     const int id = blockIdx.x;
-    const int xcd = id & 7, slot = id >> 3;
-    const int m_tile = slot % m_tiles;
-    const int n_tile = (slot / m_tiles) * 8 + xcd;
+    const int xcd = id & 7, slot_id = id >> 3;
+    const int m_tile = slot_id % m_tiles;
+    const int n_tile = (slot_id / m_tiles) * 8 + xcd;
     if (n_tile >= n_tiles) return;
     const int m0 = m_tile * kTM, n0 = n_tile * kTN;
 
     const size_t blocks = static_cast<size_t>(out_dim) * kb;
-    const uint8_t* wq = weight;
-    const uint16_t* wd = reinterpret_cast<const uint16_t*>(weight + blocks * kQuantBytes);
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(qx) + static_cast<size_t>(m0) * in_dim;
+    const uint8_t* b_base = weight + static_cast<size_t>(n0) * kb * kQuantBytes;
+    const uint8_t* sx_base = reinterpret_cast<const uint8_t*>(sx + static_cast<size_t>(m0) * kb);
+    const uint8_t* sw_base = weight + blocks * kQuantBytes + static_cast<size_t>(n0) * kb * 2;
 
-    // ---- staging registers
-    constexpr int kSxLoads = (kStageBlocks * kTM + kThreads - 1) / kThreads;
-    constexpr int kSwLoads = (kStageBlocks * kTN + kThreads - 1) / kThreads;
-    // kPrefetch stages are in flight from global memory at any time (the latency of
-    // one stage's loads is several stages of compute); nothing may consume a staged
-    // value before store_stage.
-    u32x4 ra[kPrefetch][kALoads], rb[kPrefetch][kBLoads];
-    float rsx[kPrefetch][kSxLoads];
-    uint16_t rsw[kPrefetch][kSwLoads];  // raw fp16 bits
+    const int stages = (kb + kSB - 1) / kSB;
+    const int last_blocks = kb - (stages - 1) * kSB;  // blocks in the last stage, 1..kSB
 
-    auto load_stage = [&](int set, int kb0) {
+    // first unit of each kind this wavefront handles (then every kWaves-th)
+    const int ua0 = wave;
+    const int ub0 = (wave + kWaves - kStartB) % kWaves;
+    const int usx0 = (wave + kWaves - kStartSx) % kWaves;
+    const int usw0 = (wave + kWaves - kStartSw) % kWaves;
+    int loads_per_stage = 0;
 #pragma unroll
-        for (int i = 0; i < kALoads; ++i) {
-            const int q = tid + i * kThreads;
-            if (kAChunks % kThreads == 0 || q < kAChunks) {
-                const int r = q >> 3, c = q & 7;
-                const int m = min(m0 + r, rows - 1);
-                const int blk = min(kb0 + (c >> 1), kb - 1);
-                ra[set][i] = *reinterpret_cast<const u32x4*>(qx + static_cast<size_t>(m) * in_dim + blk * 32 + (c & 1) * 16);
-            }
+    for (int i = 0; i < kPerA; ++i) loads_per_stage += ua0 + i * kWaves < kUnitsA;
+#pragma unroll
+    for (int i = 0; i < kPerB; ++i) loads_per_stage += ub0 + i * kWaves < kUnitsB;
+#pragma unroll
+    for (int i = 0; i < kPerSx; ++i) loads_per_stage += usx0 + i * kWaves < kUnitsSx;
+#pragma unroll
+    for (int i = 0; i < kPerSw; ++i) loads_per_stage += usw0 + i * kWaves < kUnitsSw;
+
+    // Per-lane byte offsets of the loads, for a full stage ([0]) and for the last
+    // stage ([1], block indices clamped to the last valid block: nothing is read past
+    // a row's end; the scales of the clamped blocks are written as zero).
+    // LDS position p = lane of a 64-lane load is chunk slot p % kCPR of row p / kCPR:
+    // eight (or more) consecutive lanes read one 128-byte line, in swizzled order.
+    const int dma_r = lane / kCPR, dma_slot = lane % kCPR;
+    uint32_t off_a[kPerA][2], off_b[kPerB][2], off_sx[kPerSx][2], off_sw[kPerSw][2];
+    int lds_b4[kPerB][2];  // Q4_0: LDS chunk positions of the low- and high-nibble halves
+    auto dma_chunk_last = [&](int c) { return min(c >> 1, last_blocks - 1) * 2 + (c & 1); };
+#pragma unroll
+    for (int i = 0; i < kPerA; ++i) {
+        const int r = min((ua0 + i * kWaves) * kRPL + dma_r, kTM - 1);
+        const int c = dma_slot ^ ((r / S::kRowsPerWrap) % kCPR);
+        const uint32_t rowoff = static_cast<uint32_t>(min(m0 + r, rows - 1) - m0) * static_cast<uint32_t>(in_dim);
+        off_a[i][0] = rowoff + c * 16;
+        off_a[i][1] = rowoff + dma_chunk_last(c) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < kPerB; ++i) {
+        if (kQ4) {
+            const int q = min((ub0 + i * kWaves) * 64 + lane, kTN * kSB - 1);
+            const int r = q / kSB, blk = q % kSB;
+            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb) * 16u;
+            off_b[i][0] = rowoff + blk * 16;
+            off_b[i][1] = rowoff + min(blk, last_blocks - 1) * 16;
+            lds_b4[i][0] = S::chunk_pos(r, 2 * blk);
+            lds_b4[i][1] = S::chunk_pos(r, 2 * blk + 1);
+        } else {
+            const int r = min((ub0 + i * kWaves) * kRPL + dma_r, kTN - 1);
+            const int c = dma_slot ^ ((r / S::kRowsPerWrap) % kCPR);
+            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb) * 32u;
+            off_b[i][0] = rowoff + c * 16;
+            off_b[i][1] = rowoff + dma_chunk_last(c) * 16;
+            lds_b4[i][0] = lds_b4[i][1] = 0;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kPerSx; ++i) {
+        const int q = min((usx0 + i * kWaves) * 64 + lane, kTM * kSB - 1);
+        const int r = q / kSB, blk = q % kSB;
+        const uint32_t rowoff = static_cast<uint32_t>(min(m0 + r, rows - 1) - m0) * static_cast<uint32_t>(kb);
+        off_sx[i][0] = (rowoff + blk) * 4;
+        off_sx[i][1] = (rowoff + min(blk, last_blocks - 1)) * 4;
+    }
+#pragma unroll
+    for (int i = 0; i < kPerSw; ++i) {
+        const int q = min((usw0 + i * kWaves) * 64 + lane, kTN * kSB - 1);
+        const int r = q / kSB, blk = q % kSB;
+        const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb);
+        off_sw[i][0] = (rowoff + blk) * 2;
+        off_sw[i][1] = (rowoff + min(blk, last_blocks - 1)) * 2;
+    }
+
+    const uint32_t lds_base = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(gemm_lds)));
+    constexpr int kOffB = S::kABytes, kOffSx = kOffB + S::kBBytes, kOffSw = kOffSx + S::kSxBytes, kOffRaw = kOffSw + S::kSwBytes;
+    auto stage_ptr = [&](int slot) { return gemm_lds + slot * S::kStageBytes; };
+
+    // Issues every load of stage `st` (clamped to the last stage) towards ring slot `slot`.
+    auto issue_loads = [&](int slot, int st) {
+        const int se = min(st, stages - 1);
+        const int sel = se == stages - 1 ? 1 : 0;
+        const uint32_t sp = lds_base + slot * S::kStageBytes;
+#pragma unroll
+        for (int i = 0; i < kPerA; ++i) {
+            const int u = ua0 + i * kWaves;
+            if (u < kUnitsA) lds_load16(a_base + static_cast<size_t>(se) * (kSB * 32), off_a[i][sel], sp + u * 1024);
         }
 #pragma unroll
-        for (int i = 0; i < kBLoads; ++i) {
-            const int q = tid + i * kThreads;
-            if (kBChunks % kThreads == 0 || q < kBChunks) {
-                if (kType == 2) {
-                    const int r = q >> 2, c = q & 3;
-                    const int n = min(n0 + r, out_dim - 1);
-                    const int blk = min(kb0 + c, kb - 1);
-                    rb[set][i] = *reinterpret_cast<const u32x4*>(wq + (static_cast<size_t>(n) * kb + blk) * 16);
-                } else {
-                    const int r = q >> 3, c = q & 7;
-                    const int n = min(n0 + r, out_dim - 1);
-                    const int blk = min(kb0 + (c >> 1), kb - 1);
-                    rb[set][i] = *reinterpret_cast<const u32x4*>(wq + (static_cast<size_t>(n) * kb + blk) * 32 + (c & 1) * 16);
-                }
-            }
-        }
-        // block scales, one (row, block) per load (clamped addresses; blocks past the
-        // end are zeroed when the stage is written to LDS)
-#pragma unroll
-        for (int i = 0; i < kSxLoads; ++i) {
-            const int t = min(tid + i * kThreads, kStageBlocks * kTM - 1);
-            const int m = min(m0 + (t >> 2), rows - 1);
-            rsx[set][i] = sx[static_cast<size_t>(m) * kb + min(kb0 + (t & 3), kb - 1)];
+        for (int i = 0; i < kPerB; ++i) {
+            const int u = ub0 + i * kWaves;
+            if (u < kUnitsB)
+                lds_load16(b_base + static_cast<size_t>(se) * (kSB * kQuantBytes), off_b[i][sel],
+                           sp + (kQ4 ? kOffRaw + u * 1024 : kOffB + u * 1024));
         }
 #pragma unroll
-        for (int i = 0; i < kSwLoads; ++i) {
-            const int t = min(tid + i * kThreads, kStageBlocks * kTN - 1);
-            const int n = min(n0 + (t >> 2), out_dim - 1);
-            rsw[set][i] = wd[static_cast<size_t>(n) * kb + min(kb0 + (t & 3), kb - 1)];
+        for (int i = 0; i < kPerSx; ++i) {
+            const int u = usx0 + i * kWaves;
+            if (u < kUnitsSx) lds_load4(sx_base + static_cast<size_t>(se) * (kSB * 4), off_sx[i][sel], sp + kOffSx + u * 256);
+        }
+#pragma unroll
+        for (int i = 0; i < kPerSw; ++i) {
+            const int u = usw0 + i * kWaves;
+            if (u < kUnitsSw) lds_load2(sw_base + static_cast<size_t>(se) * (kSB * 2), off_sw[i][sel], sp + kOffSw + u * 256);
         }
     };
 
-    auto store_stage = [&](int set, int stage_kb0, GemmLds<kTM, kTN>& s) {
+    // Q4_0: expands the nibble chunks this wavefront fetched for ring slot `slot` into
+    // int8 fragments (its own loads have landed: no other wavefront is involved).
+    auto expand_q4 = [&](int slot) {
+        if (!kQ4) return;
+        unsigned char* sp = stage_ptr(slot);
+        const int4* raw = reinterpret_cast<const int4*>(sp + kOffRaw);
+        int4* bs = reinterpret_cast<int4*>(sp + kOffB);
 #pragma unroll
-        for (int i = 0; i < kALoads; ++i) {
-            const int q = tid + i * kThreads;
-            if (kAChunks % kThreads == 0 || q < kAChunks) {
-                const int r = q >> 3, c = q & 7;
-                s.a[c * Lds::kPlaneA + r] = make_int4(ra[set][i].x, ra[set][i].y, ra[set][i].z, ra[set][i].w);
+        for (int i = 0; i < kPerB; ++i) {
+            const int u = ub0 + i * kWaves;
+            if (u < kUnitsB) {
+                const int4 r = raw[u * 64 + lane];
+                const uint32_t p[4] = {static_cast<uint32_t>(r.x), static_cast<uint32_t>(r.y), static_cast<uint32_t>(r.z), static_cast<uint32_t>(r.w)};
+                int v[8];
+                unpack_q4(p, v);  // low nibbles = values 0..15 (half 0), high nibbles = 16..31 (half 1)
+                bs[lds_b4[i][0]] = make_int4(v[0], v[1], v[2], v[3]);
+                bs[lds_b4[i][1]] = make_int4(v[4], v[5], v[6], v[7]);
             }
-        }
-#pragma unroll
-        for (int i = 0; i < kBLoads; ++i) {
-            const int q = tid + i * kThreads;
-            if (kBChunks % kThreads == 0 || q < kBChunks) {
-                if (kType == 2) {
-                    const int r = q >> 2, c = q & 3;
-                    const uint32_t p[4] = {rb[set][i].x, rb[set][i].y, rb[set][i].z, rb[set][i].w};
-                    int v[8];
-                    unpack_q4(p, v);  // low nibbles = values 0..15 (half 0), high nibbles = 16..31 (half 1)
-                    s.b[(c * 2 + 0) * Lds::kPlaneB + r] = make_int4(v[0], v[1], v[2], v[3]);
-                    s.b[(c * 2 + 1) * Lds::kPlaneB + r] = make_int4(v[4], v[5], v[6], v[7]);
-                } else {
-                    const int r = q >> 3, c = q & 7;
-                    s.b[c * Lds::kPlaneB + r] = make_int4(rb[set][i].x, rb[set][i].y, rb[set][i].z, rb[set][i].w);
-                }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < kSxLoads; ++i) {
-            const int t = tid + i * kThreads;
-            if (t < kStageBlocks * kTM) s.sx[(t & 3) * Lds::kScaleA + (t >> 2)] = stage_kb0 + (t & 3) < kb ? rsx[set][i] : 0.0f;
-        }
-#pragma unroll
-        for (int i = 0; i < kSwLoads; ++i) {
-            const int t = tid + i * kThreads;
-            if (t < kStageBlocks * kTN)
-                s.sw[(t & 3) * Lds::kScaleB + (t >> 2)] = stage_kb0 + (t & 3) < kb ? half_bits_to_f32(rsw[set][i]) : 0.0f;
         }
     };
 
-    float acc[16];
-#pragma unroll
-    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+    // this lane's fragment positions (loop-invariant; only the ring slot changes)
+    const int row = wm * 32 + lj;  // activation row (A operand) inside the tile
+    const int col = wn * 32 + lj;  // weight column (B operand) inside the tile
+    const int b0 = 2 * ks;         // first block of this wavefront's pair inside a stage
+    const int frag_a0 = S::chunk_pos(row, 2 * b0 + lh), frag_a1 = S::chunk_pos(row, 2 * b0 + 2 + lh);
+    const int frag_b0 = S::chunk_pos(col, 2 * b0 + lh), frag_b1 = S::chunk_pos(col, 2 * b0 + 2 + lh);
+    const int frag_sx = row * kSB + b0 + lh;  // lanes 0-31 carry block b0, lanes 32-63 block b0 + 1
+    const int frag_sw = col * kSB + b0 + lh;
 
-    const int stages = (kb + kStageBlocks - 1) / kStageBlocks;
-    // Loads are never predicated: past the last stage they re-read clamped addresses
-    // and their scales are written as zero, so the loop body is straight-line code and
-    // the compiler can wait for exactly the one stage it is about to store.
+    v16f acc = {};
+
+    // ---- prologue: stages 0 .. kRing-2 in flight, stage 0 landed
 #pragma unroll
-    for (int d = 0; d < kPrefetch; ++d) load_stage(d, d * kStageBlocks);
-    store_stage(0, 0, lds[0]);
+    for (int d = 0; d < kRing - 1; ++d) issue_loads(d, d);
+    // A stage has landed for this wavefront once at most (kRing - 2) stages' worth of
+    // its later loads are outstanding (loads complete in order).
+    wait_vm_outstanding(loads_per_stage * (kRing - 2));
+    expand_q4(0);
     __syncthreads();
 
-    const int row = wm * 32 + lj;  // this lane's activation row (A operand) inside the tile
-    const int col = wn * 32 + lj;  // this lane's weight column (B operand) inside the tile
-    for (int st0 = 0; st0 < stages; st0 += kPrefetch) {
+    for (int st0 = 0; st0 < stages; st0 += kRing) {
 #pragma unroll
-        for (int d = 0; d < kPrefetch; ++d) {
+        for (int d = 0; d < kRing; ++d) {
             const int st = st0 + d;  // may run past `stages` in the last round: zero scales, no effect
-            const GemmLds<kTM, kTN>& cur = lds[d & 1];  // kPrefetch is even: stage st sits in buffer st & 1 == d & 1
-            // register set d has just been written to LDS: refill it with the stage kPrefetch ahead
-            load_stage(d, (st + kPrefetch) * kStageBlocks);
-            __builtin_amdgcn_sched_barrier(0);
+            // the slot of stage st - 1 is free (everyone passed the barrier): refill it, kRing - 1 stages ahead
+            issue_loads((d + kRing - 1) % kRing, st + kRing - 1);
 
-            // a real loop: one pair's MFMA results live at a time
-#pragma unroll 1
-            for (int pair = 0; pair < kStageBlocks / 2; ++pair) {
-                const int b0 = 2 * pair, b1 = b0 + 1;
-                const int4 a0v = cur.a[(b0 * 2 + lh) * Lds::kPlaneA + row], a1v = cur.a[(b1 * 2 + lh) * Lds::kPlaneA + row];
-                const int4 w0v = cur.b[(b0 * 2 + lh) * Lds::kPlaneB + col], w1v = cur.b[(b1 * 2 + lh) * Lds::kPlaneB + col];
-                // scale operands: lanes 0-31 carry block b0, lanes 32-63 block b1
-                const float ta = cur.sx[(b0 + lh) * Lds::kScaleA + row];
-                const float tb = cur.sw[(b0 + lh) * Lds::kScaleB + col];
-                const v4i a0 = {a0v.x, a0v.y, a0v.z, a0v.w}, a1 = {a1v.x, a1v.y, a1v.z, a1v.w};
-                const v4i w0 = {w0v.x, w0v.y, w0v.z, w0v.w}, w1 = {w1v.x, w1v.y, w1v.z, w1v.w};
-                v16i c0 = {}, c1 = {};
-                v32f t = {};
-                c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, c0, 0, 0, 0);
-                c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, c1, 0, 0, 0);
-                t = __builtin_amdgcn_mfma_f32_32x32x1f32(ta, tb, t, 0, 0, 0);
-                if (kWriteDots) {
-                    const int blk = st * kStageBlocks + b0;
-                    const int n = n0 + col;
+            const unsigned char* sp = stage_ptr(d);
+            const int4* as = reinterpret_cast<const int4*>(sp);
+            const int4* bs = reinterpret_cast<const int4*>(sp + kOffB);
+            const float* sxs = reinterpret_cast<const float*>(sp + kOffSx);
+            const uint32_t* sws = reinterpret_cast<const uint32_t*>(sp + kOffSw);  // fp16 bits
+            const int4 a0v = as[frag_a0], a1v = as[frag_a1];
+            const int4 w0v = bs[frag_b0], w1v = bs[frag_b1];
+            // blocks past the end of K (clamped re-reads of the last block) get scale 0
+            const bool live = st * kSB + b0 + lh < kb;
+            float ta_raw = sxs[frag_sx];
+            uint32_t tb_raw = sws[frag_sw];
+            asm volatile("" : "+v"(ta_raw), "+v"(tb_raw));  // plain loads, then selects: no branch around the reads
+            const float ta = live ? ta_raw : 0.0f;
+            const float tb = live ? half_bits_to_f32(static_cast<uint16_t>(tb_raw)) : 0.0f;
+            const v4i a0 = {a0v.x, a0v.y, a0v.z, a0v.w}, a1 = {a1v.x, a1v.y, a1v.z, a1v.w};
+            const v4i w0 = {w0v.x, w0v.y, w0v.z, w0v.w}, w1 = {w1v.x, w1v.y, w1v.z, w1v.w};
+            const v16i zi = {};
+            const v32f zf = {};
+            const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, zi, 0, 0, 0);
+            const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, zi, 0, 0, 0);
+            const v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(ta, tb, zf, 0, 0, 0);
+            if (kWriteDots) {
+                const int blk = st * kSB + b0;
+                const int n = n0 + col;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                        if (m < rows && n < out_dim) {
-                            int* dp = dots + (static_cast<size_t>(m) * out_dim + n) * kb;
-                            if (blk < kb) dp[blk] = c0[v];
-                            if (blk + 1 < kb) dp[blk + 1] = c1[v];
-                        }
+                for (int v = 0; v < 16; ++v) {
+                    const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+                    if (m < rows && n < out_dim) {
+                        int* dp = dots + (static_cast<size_t>(m) * out_dim + n) * kb;
+                        if (blk < kb) dp[blk] = c0[v];
+                        if (blk + 1 < kb) dp[blk + 1] = c1[v];
                     }
                 }
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[v]);
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[v]);
             }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[v]);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[v]);
 
-            store_stage((d + 1) % kPrefetch, (st + 1) * kStageBlocks, lds[(d + 1) & 1]);
+            // Program-order fence for the compiler (no instruction): the stage's arithmetic
+            // is emitted here and not carried, with its 64 result registers, into later stages.
+            asm volatile("" : "+v"(acc) : : "memory");
+
+            // stage st + 1: its loads were issued kRing - 2 stages ago
+            wait_vm_outstanding(loads_per_stage * (kRing - 2));
+            expand_q4((d + 1) % kRing);
             __syncthreads();
         }
     }
 
-    if (dst == nullptr) return;
+    // Loads still in flight target ring slots nobody reads again; they must land before
+    // the ring is reused for the reduction (and before the workgroup ends).
+    wait_vm_outstanding(0);
     const int n = n0 + col;
+    if (kSplit > 1) {
+        // ---- the kSplit partial sums of a tile meet in LDS
+        __syncthreads();
+        float* red = reinterpret_cast<float*>(gemm_lds);  // [ks][tile][v][lane]
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-        if (m < rows && n < out_dim) dst[static_cast<size_t>(m) * out_dim + n] = acc[v];
+        for (int v = 0; v < 16; ++v) red[((ks * S::kTiles + tile) * 16 + v) * 64 + lane] = acc[v];
+        __syncthreads();
+        if (dst == nullptr) return;
+        constexpr int kPer = 16 / kSplit;
+#pragma unroll
+        for (int j = 0; j < kPer; ++j) {
+            const int v = ks * kPer + j;
+            float sum = red[(tile * 16 + v) * 64 + lane];
+#pragma unroll
+            for (int k2 = 1; k2 < kSplit; ++k2) sum += red[((k2 * S::kTiles + tile) * 16 + v) * 64 + lane];
+            const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < rows && n < out_dim) dst[static_cast<size_t>(m) * out_dim + n] = sum;
+        }
+    } else {
+        if (dst == nullptr) return;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
+            if (m < rows && n < out_dim) dst[static_cast<size_t>(m) * out_dim + n] = acc[v];
+        }
     }
 }
 
 namespace {
 
-template <int kType, int kWavesM, int kWavesN>
+template <int kType, int kWavesM, int kWavesN, int kSplit>
 hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
                        const uint8_t* weight, int rows, int in_dim, int out_dim) {
-    constexpr int kTM = 32 * kWavesM, kTN = 32 * kWavesN;
-    const int m_tiles = (rows + kTM - 1) / kTM;
-    const int n_tiles = (out_dim + kTN - 1) / kTN;
+    using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
+    const int m_tiles = (rows + S::kTM - 1) / S::kTM;
+    const int n_tiles = (out_dim + S::kTN - 1) / S::kTN;
     const int n_groups = (n_tiles + 7) / 8;
     const long long grid = static_cast<long long>(n_groups) * m_tiles * 8;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    dim3 g(static_cast<unsigned>(grid)), b(64 * kWavesM * kWavesN);
+    // per-lane load offsets are 32-bit, relative to the workgroup's first row
+    if (static_cast<long long>(S::kTM > S::kTN ? S::kTM : S::kTN) * in_dim > 0x7fffffffLL) return hipErrorInvalidValue;
+    dim3 g(static_cast<unsigned>(grid)), b(S::kThreads);
+    auto kernel_f32 = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, false>;
+    auto kernel_dots = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, true>;
+    // more than 64 KB of LDS has to be asked for once per kernel
+    static const hipError_t attr = [&]() {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_f32),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes);
+        if (e != hipSuccess) return e;
+        return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_dots), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                   S::kLdsBytes);
+    }();
+    if (attr != hipSuccess) return attr;
     if (dots)
-        hipLaunchKernelGGL((gemm_i8_kernel<kType, kWavesM, kWavesN, true>), g, b, 0, stream, dst, dots, qx, sx, weight,
-                           rows, in_dim, out_dim, m_tiles, n_tiles);
+        hipLaunchKernelGGL(kernel_dots, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
+                           m_tiles, n_tiles);
     else
-        hipLaunchKernelGGL((gemm_i8_kernel<kType, kWavesM, kWavesN, false>), g, b, 0, stream, dst, dots, qx, sx, weight,
-                           rows, in_dim, out_dim, m_tiles, n_tiles);
+        hipLaunchKernelGGL(kernel_f32, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
+                           m_tiles, n_tiles);
     return hipGetLastError();
 }
 
 template <int kType>
 hipError_t launch_type(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
                        const uint8_t* weight, int rows, int in_dim, int out_dim) {
-    // 64 x 128 tiles (8 wavefronts) when they still give every CU a workgroup, 32 x 128 otherwise
+    // 64 x 128 tiles while they still give every CU a workgroup, 32 x 64 with a deeper K split otherwise
     const long long big = static_cast<long long>((rows + 63) / 64) * ((out_dim + 127) / 128);
-    static const char* force = std::getenv("AFHIP_GEMM_TILE");  // tuning: "L" = 64x128, "S" = 32x128
+    static const char* force = std::getenv("AFHIP_GEMM_TILE");  // tuning: "L" = 64x128, "S" = 32x64
     const bool use_big = force ? force[0] == 'L' : big >= 256;
-    if (force && force[0] == 'M') return launch_tile<kType, 2, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
-    if (force && force[0] == 'N') return launch_tile<kType, 1, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
-    if (use_big) return launch_tile<kType, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
-    return launch_tile<kType, 1, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
+    if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
+    return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
 }
 
 }  // namespace
