@@ -302,69 +302,93 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
 
     v16f acc = {};
 
-    // ---- prologue: stages 0 .. kRing-2 in flight, stage 0 landed
+    // MFMA operands of one stage as read from LDS (scales still raw)
+    struct Frag {
+        int4 a0, a1, w0, w1;
+        float ta;
+        uint32_t tb;  // fp16 bits
+    };
+    auto read_frag = [&](int slot, Frag& f) {
+        const unsigned char* sp = stage_ptr(slot);
+        const int4* as = reinterpret_cast<const int4*>(sp);
+        const int4* bs = reinterpret_cast<const int4*>(sp + kOffB);
+        f.a0 = as[frag_a0];
+        f.a1 = as[frag_a1];
+        f.w0 = bs[frag_b0];
+        f.w1 = bs[frag_b1];
+        f.ta = reinterpret_cast<const float*>(sp + kOffSx)[frag_sx];
+        f.tb = reinterpret_cast<const uint32_t*>(sp + kOffSw)[frag_sw];
+    };
+    // One pair of blocks, first block `blk` (absolute index): MFMAs of block blk and of
+    // the scale products, vector-ALU work of block blk, then the same for block blk + 1 in
+    // the registers block blk's dots have left (the two halves of a wavefront's work do
+    // not overlap anyway, and 16 registers fewer are live).  `between` runs after the
+    // last MFMA has been issued: the operand registers are free from there on.
+    auto pair_step = [&](const Frag& f, int blk, auto&& between) {
+        // blocks past the end of K (clamped re-reads of the last block) get scale 0
+        const bool live = blk + lh < kb;
+        const float ta = live ? f.ta : 0.0f;
+        const float tb = live ? half_bits_to_f32(static_cast<uint16_t>(f.tb)) : 0.0f;
+        const v4i a0 = {f.a0.x, f.a0.y, f.a0.z, f.a0.w}, a1 = {f.a1.x, f.a1.y, f.a1.z, f.a1.w};
+        const v4i w0 = {f.w0.x, f.w0.y, f.w0.z, f.w0.w}, w1 = {f.w1.x, f.w1.y, f.w1.z, f.w1.w};
+        const v16i zi = {};
+        const v32f zf = {};
+        const int n = n0 + col;
+        v16i c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, zi, 0, 0, 0);
+        v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(ta, tb, zf, 0, 0, 0);
 #pragma unroll
-    for (int d = 0; d < kRing - 1; ++d) issue_loads(d, d);
-    // A stage has landed for this wavefront once at most (kRing - 2) stages' worth of
-    // its later loads are outstanding (loads complete in order).
-    wait_vm_outstanding(loads_per_stage * (kRing - 2));
-    expand_q4(0);
-    __syncthreads();
-
-    for (int st0 = 0; st0 < stages; st0 += kRing) {
-#pragma unroll
-        for (int d = 0; d < kRing; ++d) {
-            const int st = st0 + d;  // may run past `stages` in the last round: zero scales, no effect
-            // the slot of stage st - 1 is free (everyone passed the barrier): refill it, kRing - 1 stages ahead
-            issue_loads((d + kRing - 1) % kRing, st + kRing - 1);
-
-            const unsigned char* sp = stage_ptr(d);
-            const int4* as = reinterpret_cast<const int4*>(sp);
-            const int4* bs = reinterpret_cast<const int4*>(sp + kOffB);
-            const float* sxs = reinterpret_cast<const float*>(sp + kOffSx);
-            const uint32_t* sws = reinterpret_cast<const uint32_t*>(sp + kOffSw);  // fp16 bits
-            const int4 a0v = as[frag_a0], a1v = as[frag_a1];
-            const int4 w0v = bs[frag_b0], w1v = bs[frag_b1];
-            // blocks past the end of K (clamped re-reads of the last block) get scale 0
-            const bool live = st * kSB + b0 + lh < kb;
-            float ta_raw = sxs[frag_sx];
-            uint32_t tb_raw = sws[frag_sw];
-            asm volatile("" : "+v"(ta_raw), "+v"(tb_raw));  // plain loads, then selects: no branch around the reads
-            const float ta = live ? ta_raw : 0.0f;
-            const float tb = live ? half_bits_to_f32(static_cast<uint16_t>(tb_raw)) : 0.0f;
-            const v4i a0 = {a0v.x, a0v.y, a0v.z, a0v.w}, a1 = {a1v.x, a1v.y, a1v.z, a1v.w};
-            const v4i w0 = {w0v.x, w0v.y, w0v.z, w0v.w}, w1 = {w1v.x, w1v.y, w1v.z, w1v.w};
-            const v16i zi = {};
-            const v32f zf = {};
-            const v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a0, w0, zi, 0, 0, 0);
-            const v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, zi, 0, 0, 0);
-            const v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(ta, tb, zf, 0, 0, 0);
-            if (kWriteDots) {
-                const int blk = st * kSB + b0;
-                const int n = n0 + col;
+        for (int h = 0; h < 2; ++h) {
+            if (kWriteDots && blk + h < kb) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                    if (m < rows && n < out_dim) {
-                        int* dp = dots + (static_cast<size_t>(m) * out_dim + n) * kb;
-                        if (blk < kb) dp[blk] = c0[v];
-                        if (blk + 1 < kb) dp[blk + 1] = c1[v];
-                    }
+                    if (m < rows && n < out_dim) dots[(static_cast<size_t>(m) * out_dim + n) * kb + blk + h] = c[v];
                 }
             }
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[v]);
+            for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[16 * h + v], static_cast<float>(c[v]), acc[v]);
+            if (h == 0) {
+                // compiler fence (no instruction): block blk is finished before block blk + 1 starts
+                asm volatile("" : "+v"(acc), "+v"(t) : : "memory");
+                c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a1, w1, zi, 0, 0, 0);
+                between();
+            }
+        }
+    };
+    // Program-order fence for the compiler (it emits no instruction): a stage's arithmetic
+    // is emitted before it.  Without it the optimizer gathers the MFMAs of several stages
+    // in one place and spills their results.
+    auto pin_acc = [&]() { asm volatile("" : "+v"(acc) : : "memory"); };
+
+    // ---- prologue: stages 0 .. kRing-2 in flight, stages 0 and 1 landed, stage 0 in registers
+    static_assert(kRing == 4, "the loop reads stage st + 1 while stage st + 2 lands and stage st + 3 is issued");
 #pragma unroll
-            for (int v = 0; v < 16; ++v) acc[v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[v]);
-
-            // Program-order fence for the compiler (no instruction): the stage's arithmetic
-            // is emitted here and not carried, with its 64 result registers, into later stages.
-            asm volatile("" : "+v"(acc) : : "memory");
-
-            // stage st + 1: its loads were issued kRing - 2 stages ago
-            wait_vm_outstanding(loads_per_stage * (kRing - 2));
-            expand_q4((d + 1) % kRing);
-            __syncthreads();
+    for (int d = 0; d < kRing - 1; ++d) issue_loads(d, d);
+    // Loads complete in order: a stage has landed for this wavefront once at most the
+    // loads of the stages issued after it are outstanding.
+    wait_vm_outstanding(loads_per_stage);
+    expand_q4(0);
+    expand_q4(1);
+    __syncthreads();
+    {
+        // The next stage's operands are read from LDS while this stage's arithmetic runs.
+        Frag frag[2];
+        read_frag(0, frag[0]);
+        for (int st0 = 0; st0 < stages; st0 += kRing) {
+#pragma unroll
+            for (int d = 0; d < kRing; ++d) {
+                const int st = st0 + d;  // may run past `stages` in the last round: zero scales, no effect
+                // the slot of stage st - 1 is free (its fragments were read a stage ago): refill it, kRing - 1 stages ahead
+                issue_loads((d + kRing - 1) % kRing, st + kRing - 1);
+                // the next stage's operands landed before the last barrier
+                pair_step(frag[d & 1], st * kSB + b0, [&]() { read_frag((d + 1) % kRing, frag[(d + 1) & 1]); });
+                pin_acc();
+                // stage st + 2 (issued two stages ago) has to be complete before the barrier:
+                // the next stage reads its operands
+                wait_vm_outstanding(loads_per_stage);
+                expand_q4((d + 2) % kRing);
+                __syncthreads();
+            }
         }
     }
 
@@ -440,7 +464,7 @@ hipError_t launch_type(hipStream_t stream, float* dst, int* dots, const int8_t* 
     // 64 x 128 tiles while they still give every CU a workgroup, 32 x 64 with a deeper K split otherwise
     const long long big = static_cast<long long>((rows + 63) / 64) * ((out_dim + 127) / 128);
     static const char* force = std::getenv("AFHIP_GEMM_TILE");  // tuning: "L" = 64x128, "S" = 32x64
-    const bool use_big = force ? force[0] == 'L' : big >= 256;
+    const bool use_big = force ? force[0] != 'S' : big >= 256;
     if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
     return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim);
 }
