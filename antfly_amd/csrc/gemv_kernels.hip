@@ -85,13 +85,11 @@ __device__ __forceinline__ void quantize_block_to_lds(const float4 (&v)[8], int 
 
 constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
-// kFused: quantize f32 `input` in the prologue.  Otherwise the activations were
-// quantized by quantize_activations_kernel (natural order: pre_q [rows][in_dim]
-// int8, pre_scale / pre_sum [rows][in_dim/32]) and the prologue only copies them.
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kFused>
+// One or two rows of f32 activations, quantized in the prologue of every workgroup.
+template <int kType, int kRows, int kCols, bool kWriteDots>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
-    float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input, const int4* __restrict__ pre_q,
-    const float* __restrict__ pre_scale, const int* __restrict__ pre_sum, const uint8_t* __restrict__ weight, int in_dim,
+    float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input,
+    const uint8_t* __restrict__ weight, int in_dim,
     int out_dim, int slices) {
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
@@ -124,15 +122,11 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const int o0 = group * kCols;
     const bool active = o0 < out_dim;
 
-    // ---- 1. first activation requests, then every weight byte this wavefront needs
-    const int x_blocks = kRows * kb;  // one thread quantizes one block
-    float4 xpre[8];
-    if (kFused) {
-        const int xb = tid < x_blocks ? tid : 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) xpre[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
-    }
-
+    // ---- 1. requests: first the activations (wavefronts that quantize a block per
+    // thread), then every weight byte this wavefront needs.  Loads complete in order, so
+    // the activation requests have to be the older ones: quantizing X -- which the whole
+    // workgroup waits for at the barrier -- must not wait for the weights.
+    const int x_blocks = kRows * kb;
     u32x4 wq[kSteps][kCols];
     uint16_t wd[kSteps][kCols];
     int blk[kSteps];
@@ -143,45 +137,37 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         ok[j] = active && b < kb;
         blk[j] = b < kb ? b : kb - 1;  // lanes past the row end re-read its last block and contribute nothing
     }
+    auto request_weights = [&]() {
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) {
-        const int o = min(o0 + c, out_dim - 1);  // likewise for columns past the end
-        const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
-        const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
+        for (int c = 0; c < kCols; ++c) {
+            const int o = min(o0 + c, out_dim - 1);  // likewise for columns past the end
+            const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
+            const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
 #pragma unroll
-        for (int j = 0; j < kSteps; ++j) {
-            wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
-            wd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
-        }
-    }
-
-    // ---- 2. quantized X into LDS
-    if (kFused) {  // one thread per block
-        if (tid < x_blocks) {
-            const int r = tid / kb, b = tid - r * kb;
-            quantize_block_to_lds<kType>(xpre, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-        }
-        for (int xb = tid + static_cast<int>(blockDim.x); xb < x_blocks; xb += blockDim.x) {
-            float4 v[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
-            const int r = xb / kb, b = xb - r * kb;
-            quantize_block_to_lds<kType>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-        }
-    } else {  // coalesced copy, 16 bytes (half a block) per thread
-        const int row_int4 = in_dim >> 4;
-        for (int u = tid; u < kRows * row_int4; u += blockDim.x) {
-            int idx = u;
-            if (kType == 2) {
-                const int r = u / row_int4, w = u - r * row_int4;
-                idx = r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
+            for (int j = 0; j < kSteps; ++j) {
+                wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+                wd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
             }
-            reinterpret_cast<int4*>(qx)[idx] = pre_q[u];
         }
-        for (int u = tid; u < x_blocks; u += blockDim.x) {
-            sx[u] = pre_scale[u];
-            sumx[u] = pre_sum[u];
+    };
+    if (wave * kWave < x_blocks) {  // wave-uniform
+        const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
+        float4 v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
+        __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
+        request_weights();
+        __builtin_amdgcn_sched_barrier(0);
+        const int r = xb / kb, b = xb - r * kb;
+        quantize_block_to_lds<kType>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+        for (int xb2 = tid + static_cast<int>(blockDim.x); xb2 < x_blocks; xb2 += blockDim.x) {  // more blocks than threads
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb2 * 8 + i];
+            const int r2 = xb2 / kb, b2 = xb2 - r2 * kb;
+            quantize_block_to_lds<kType>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
         }
+    } else {
+        request_weights();
     }
     __syncthreads();
 
@@ -192,31 +178,45 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
 #pragma unroll
         for (int c = 0; c < kCols; ++c) acc[r][c] = 0.0f;
 
+    // The activations of this lane's blocks go to registers once; the weights are then
+    // consumed column by column, in the order their loads were issued, so the arithmetic
+    // of a column runs while the later columns are still arriving.
+    float sxr[kSteps][kRows];
+    int ar[kSteps][kRows][kType == 2 ? 8 : 4];
+    int smr[kSteps][kRows];
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
         const int b = blk[j];
 #pragma unroll
         for (int r = 0; r < kRows; ++r) {
-            const float s = ok[j] ? sx[r * kb + b] : 0.0f;
-            int a[8];
-            int sm = 0;
+            sxr[j][r] = ok[j] ? sx[r * kb + b] : 0.0f;
+            smr[j][r] = 0;
             if (kType == 2) {
                 const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b];
                 const int4 a1 = reinterpret_cast<const int4*>(qx + r * row_dwords + (row_dwords >> 1))[b];
-                a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
-                a[4] = a1.x; a[5] = a1.y; a[6] = a1.z; a[7] = a1.w;
-                sm = sumx[r * kb + b];
+                ar[j][r][0] = a0.x; ar[j][r][1] = a0.y; ar[j][r][2] = a0.z; ar[j][r][3] = a0.w;
+                ar[j][r][4] = a1.x; ar[j][r][5] = a1.y; ar[j][r][6] = a1.z; ar[j][r][7] = a1.w;
+                smr[j][r] = sumx[r * kb + b];
             } else {
                 const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b * 2 + half];
-                a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
+                ar[j][r][0] = a0.x; ar[j][r][1] = a0.y; ar[j][r][2] = a0.z; ar[j][r][3] = a0.w;
             }
+        }
+    }
 #pragma unroll
-            for (int c = 0; c < kCols; ++c) {
-                const u32x4 w = wq[j][c];
+    for (int c = 0; c < kCols; ++c) {
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+            const int b = blk[j];
+            const u32x4 w = wq[j][c];
+            const float dw = half_bits_to_f32(wd[j][c]);
+#pragma unroll
+            for (int r = 0; r < kRows; ++r) {
+                const int* a = ar[j][r];
                 int dot;
                 if (kType == 2) {
                     // nibbles stay unsigned: dot(qx, n - 8) = dot(qx, n) - 8 * sum(qx)
-                    dot = -8 * sm;
+                    dot = -8 * smr[j][r];
                     dot = dot4(static_cast<int>(w.x & 0x0F0F0F0Fu), a[0], dot);
                     dot = dot4(static_cast<int>(w.y & 0x0F0F0F0Fu), a[1], dot);
                     dot = dot4(static_cast<int>(w.z & 0x0F0F0F0Fu), a[2], dot);
@@ -234,7 +234,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
                 }
                 if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim)
                     dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + b] = dot;
-                const float tscale = s * half_bits_to_f32(wd[j][c]);
+                const float tscale = sxr[j][r] * dw;
                 const float term = tscale * static_cast<float>(dot);
                 acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
             }
@@ -312,7 +312,32 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     const int o0 = group * kCols;
     const bool active = o0 < out_dim;
 
-    // ---- 1. every weight byte this wavefront needs
+    // ---- 1. requests for the quantized X (coalesced, 16 bytes = half a block per thread)
+    // go out before the weight requests: loads complete in order, and the copy into LDS
+    // (and with it the barrier) must not wait for every weight byte of the wavefront.
+    // kXPre units per thread are requested up front (all of X for up to 8 rows of 4096
+    // values with 512 threads); larger inputs copy the rest after the weight requests.
+    constexpr int kXPre = 4;
+    const int row_int4 = in_dim >> 4;
+    const int x_units = rows * row_int4;
+    auto x_lds_index = [&](int u) {
+        if (kType != 2) return u;
+        const int r = u / row_int4, w = u - r * row_int4;
+        return r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
+    };
+    int4 xq[kXPre];
+    int xu[kXPre];
+#pragma unroll
+    for (int i = 0; i < kXPre; ++i) {
+        xu[i] = min(tid + i * static_cast<int>(blockDim.x), x_units - 1);  // spare threads repeat the last unit
+        xq[i] = pre_q[xu[i]];
+    }
+    const int su = min(tid, rows * kb - 1);
+    const float xs0 = pre_scale[su];
+    const int xm0 = pre_sum[su];
+    __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
+
+    // ---- 2. every weight byte this wavefront needs
     int wv[kSteps][kCols][kWords];
     float wd[kSteps][kCols];
     int blk[kSteps];
@@ -338,17 +363,14 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
             }
         }
 
-        // ---- 2. quantized X into LDS: coalesced copy, 16 bytes (half a block) per thread
-        const int row_int4 = in_dim >> 4;
-        for (int u = tid; u < rows * row_int4; u += blockDim.x) {
-            int idx = u;
-            if (kType == 2) {
-                const int r = u / row_int4, w = u - r * row_int4;
-                idx = r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
-            }
-            reinterpret_cast<int4*>(qx)[idx] = pre_q[u];
-        }
-        for (int u = tid; u < rows * kb; u += blockDim.x) {
+        // ---- 3. quantized X into LDS (waits for the X requests only)
+#pragma unroll
+        for (int i = 0; i < kXPre; ++i) reinterpret_cast<int4*>(qx)[x_lds_index(xu[i])] = xq[i];
+        sx[su] = xs0;
+        sumx[su] = xm0;
+        for (int u = tid + kXPre * static_cast<int>(blockDim.x); u < x_units; u += blockDim.x)
+            reinterpret_cast<int4*>(qx)[x_lds_index(u)] = pre_q[u];
+        for (int u = tid + static_cast<int>(blockDim.x); u < rows * kb; u += blockDim.x) {
             sx[u] = pre_scale[u];
             sumx[u] = pre_sum[u];
         }
@@ -467,13 +489,13 @@ hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* 
     const int waves = workgroup_waves(tune.threads, 1024, slices);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
-    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots, true>;
+    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int groups = (out_dim + kCols - 1) / kCols;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, nullptr, nullptr, nullptr,
-                       weight, in_dim, out_dim, slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, weight, in_dim, out_dim,
+                       slices);
     return hipGetLastError();
 }
 
