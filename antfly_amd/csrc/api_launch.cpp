@@ -68,7 +68,10 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
     GemvTuning t;
     // every workgroup quantizes all of X, so large workgroups share that work best
     t.threads = 1024;
-    if (env_threads >= 64 && env_threads <= 1024 && env_threads % 64 == 0) t.threads = env_threads;
+    if (env_threads >= 64 && env_threads <= 1024 && env_threads % 64 == 0) {
+        t.threads = env_threads;
+        t.exact = true;
+    }
     return t;
 }
 

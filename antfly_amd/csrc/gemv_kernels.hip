@@ -464,10 +464,39 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
 
 namespace {
 
-int workgroup_waves(int requested_threads, int max_threads, int slices) {
-    int waves = (requested_threads < max_threads ? requested_threads : max_threads) / 64;
-    if (waves < slices) waves = slices;
-    return waves / slices * slices;  // whole column groups per workgroup
+int compute_units() {
+    static const int cus = []() {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return cus;
+}
+
+// Wavefronts per workgroup: a multiple of `slices` (whole column groups), at most the
+// requested size, chosen so that the workgroups spread evenly over the compute units:
+// the busiest unit's share, ceil(grid / units) workgroups of `waves` wavefronts, is
+// smallest (ties go to the larger workgroup, which repeats the prologue less often).
+// `exact` takes the requested size as it is (tuning runs).
+int workgroup_waves(int requested_threads, int max_threads, int slices, int groups, bool exact) {
+    int limit = (requested_threads < max_threads ? requested_threads : max_threads) / 64;
+    if (limit < slices) limit = slices;
+    limit = limit / slices * slices;
+    if (exact) return limit;
+    const int units = compute_units();
+    int best = limit;
+    long best_cost = -1;
+    for (int waves = limit; waves >= slices && waves * 2 > limit; waves -= slices) {  // down to half the limit
+        const int groups_per_wg = waves / slices;
+        const long grid = (groups + groups_per_wg - 1) / groups_per_wg;
+        const long cost = (grid + units - 1) / units * waves;
+        if (best_cost < 0 || cost < best_cost) {
+            best_cost = cost;
+            best = waves;
+        }
+    }
+    return best;
 }
 
 // Raising the dynamic-LDS limit is sticky per kernel: done once per kernel, outside
@@ -486,13 +515,13 @@ hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* 
                         int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
-    const int waves = workgroup_waves(tune.threads, 1024, slices);
+    const int groups = (out_dim + kCols - 1) / kCols;
+    const int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
     auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
-    const int groups = (out_dim + kCols - 1) / kCols;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, weight, in_dim, out_dim,
                        slices);
@@ -504,13 +533,13 @@ hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const GemvActi
                        int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
-    const int waves = workgroup_waves(tune.threads, 512, slices);
+    const int groups = (out_dim + kCols - 1) / kCols;
+    const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);  // several of these workgroups share a unit: no balancing
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
     auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
-    const int groups = (out_dim + kCols - 1) / kCols;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, reinterpret_cast<const int4*>(pre.q),
                        pre.scale, pre.sum, weight, rows, in_dim, out_dim, slices);

@@ -10,7 +10,8 @@ namespace afhip {
 // Launch geometry of the fused GEMV; chosen host-side (ops/cuda/kernels.zig
 // does the same for its launch1d / launchBlocks helpers).
 struct GemvTuning {
-    int threads = 256;  // workgroup size, multiple of 64 (rounded to whole column groups)
+    int threads = 256;   // largest workgroup size, multiple of 64 (rounded to whole column groups)
+    bool exact = false;  // use `threads` as it is instead of balancing the grid over the compute units
 };
 
 size_t gemv_fused_lds_bytes(int rows, int in_dim);
