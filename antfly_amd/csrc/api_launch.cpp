@@ -39,8 +39,9 @@ static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
     return v;
 }
 
-// From this many rows on, activations are quantized by a separate kernel.
-constexpr size_t kGemvPrequantizeRows = 3;
+// The GEMV quantizes X in its own prologue (every workgroup repeats that work) as long
+// as X has at most this many 32-value blocks; beyond, a separate kernel quantizes X once.
+constexpr size_t kGemvFusedQuantBlocks = 512;
 
 // LDS the fused GEMV may use per workgroup; gfx950 has 160 KiB per CU.
 constexpr size_t kGemvLdsBudget = 96 * 1024;
@@ -143,10 +144,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     }
     if (fused_ok) {
         // mmv / small_batch (also when a plan forces them on more rows: 16-row slices).
-        // One or two rows: the GEMV quantizes X in its own prologue (one launch).
-        // More rows: every workgroup would repeat that work, so X is quantized once
-        // by its own kernel into the caller's scratch.
-        const bool prequantize = rows >= kGemvPrequantizeRows;
+        // Small X (one to four rows of 4096 values): the GEMV quantizes it in its own
+        // prologue, one launch.  Larger X: every workgroup would repeat too much of that
+        // work, so X is quantized once by its own kernel into the caller's scratch.
+        const bool prequantize = rows > 2 && rows * kb > kGemvFusedQuantBlocks;
         const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
         if (prequantize && (workspace.ptr == 0 || workspace.len < ws.bytes || workspace.ptr % 16 != 0))
             return AFHIP_ERR_INVALID_STATE;

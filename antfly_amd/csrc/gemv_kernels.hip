@@ -270,13 +270,19 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
 }
 
 // =====================================================================
-// Same work decomposition for 3 or more rows, activations quantized beforehand
-// by quantize_activations_kernel.  The wavefront keeps its weights (unpacked
-// once) in registers and walks the rows two at a time, so register use does not
-// grow with the row count; `rows` is a run-time value bounded only by LDS.
+// Same work decomposition for 3 or more rows.  The wavefront keeps its weights
+// (unpacked once) in registers and walks the rows two at a time, so register use
+// does not grow with the row count; `rows` is a run-time value bounded only by LDS.
+// kFusedX: the workgroup quantizes the f32 `input` itself -- its first wavefronts
+// (half of them at most) do that, a block per thread and pass, and ask for their
+// weights afterwards, while the other wavefronts have their weight requests out from
+// the start.  Otherwise the activations were quantized beforehand by
+// quantize_activations_kernel (natural order: pre_q [rows][in_dim] int8, pre_scale /
+// pre_sum [rows][in_dim/32]) and are copied into LDS.
 // =====================================================================
-template <int kType, int kCols, bool kWriteDots>
+template <int kType, int kCols, bool kWriteDots, bool kFusedX>
 __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ dst, int* __restrict__ dots,
+                                                            const float* __restrict__ input,
                                                             const int4* __restrict__ pre_q,
                                                             const float* __restrict__ pre_scale,
                                                             const int* __restrict__ pre_sum,
@@ -312,32 +318,6 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     const int o0 = group * kCols;
     const bool active = o0 < out_dim;
 
-    // ---- 1. requests for the quantized X (coalesced, 16 bytes = half a block per thread)
-    // go out before the weight requests: loads complete in order, and the copy into LDS
-    // (and with it the barrier) must not wait for every weight byte of the wavefront.
-    // kXPre units per thread are requested up front (all of X for up to 8 rows of 4096
-    // values with 512 threads); larger inputs copy the rest after the weight requests.
-    constexpr int kXPre = 4;
-    const int row_int4 = in_dim >> 4;
-    const int x_units = rows * row_int4;
-    auto x_lds_index = [&](int u) {
-        if (kType != 2) return u;
-        const int r = u / row_int4, w = u - r * row_int4;
-        return r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
-    };
-    int4 xq[kXPre];
-    int xu[kXPre];
-#pragma unroll
-    for (int i = 0; i < kXPre; ++i) {
-        xu[i] = min(tid + i * static_cast<int>(blockDim.x), x_units - 1);  // spare threads repeat the last unit
-        xq[i] = pre_q[xu[i]];
-    }
-    const int su = min(tid, rows * kb - 1);
-    const float xs0 = pre_scale[su];
-    const int xm0 = pre_sum[su];
-    __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
-
-    // ---- 2. every weight byte this wavefront needs
     int wv[kSteps][kCols][kWords];
     float wd[kSteps][kCols];
     int blk[kSteps];
@@ -351,29 +331,94 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     {
         u32x4 raw[kSteps][kCols];
         uint16_t rawd[kSteps][kCols];
+        auto request_weights = [&]() {
 #pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            const int o = min(o0 + c, out_dim - 1);
-            const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
-            const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
+            for (int c = 0; c < kCols; ++c) {
+                const int o = min(o0 + c, out_dim - 1);
+                const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
+                const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
 #pragma unroll
-            for (int j = 0; j < kSteps; ++j) {
-                raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
-                rawd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
+                for (int j = 0; j < kSteps; ++j) {
+                    raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+                    rawd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
+                }
+            }
+        };
+
+        if (kFusedX) {
+            // ---- 1a. Loads complete in order, so whoever quantizes X asks for X first and
+            // for its weights afterwards; the barrier below must not wait for weight bytes.
+            const int x_blocks = rows * kb;
+            const int q_waves = min(max(waves >> 1, 1), (x_blocks + kWave - 1) / kWave);
+            if (wave < q_waves) {
+                const int stride = q_waves * kWave;
+                auto load_block = [&](int xb, float4 (&v)[8]) {
+                    const int b = min(xb, x_blocks - 1);  // spare lanes repeat the last block
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[b * 8 + i];
+                };
+                auto quantize = [&](int xb, const float4 (&v)[8]) {
+                    const int b = min(xb, x_blocks - 1);
+                    const int r = b / kb, bb = b - r * kb;
+                    quantize_block_to_lds<kType>(v, bb, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+                };
+                // two blocks in flight per thread
+                float4 va[8], vb[8];
+                int xb = tid;
+                load_block(xb, va);
+                for (; xb < x_blocks; xb += 2 * stride) {
+                    if (xb + stride < x_blocks) load_block(xb + stride, vb);
+                    quantize(xb, va);
+                    if (xb + stride < x_blocks) {
+                        if (xb + 2 * stride < x_blocks) load_block(xb + 2 * stride, va);
+                        quantize(xb + stride, vb);
+                    }
+                }
+                request_weights();
+            } else {
+                request_weights();
+            }
+        } else {
+            // ---- 1b. requests for the quantized X (coalesced, 16 bytes = half a block per
+            // thread) go out before the weight requests: loads complete in order, and the copy
+            // into LDS (and with it the barrier) must not wait for every weight byte of the
+            // wavefront.  kXPre units per thread are requested up front (all of X for up to 8
+            // rows of 4096 values with 512 threads); larger inputs copy the rest afterwards.
+            constexpr int kXPre = 4;
+            const int row_int4 = in_dim >> 4;
+            const int x_units = rows * row_int4;
+            auto x_lds_index = [&](int u) {
+                if (kType != 2) return u;
+                const int r = u / row_int4, w = u - r * row_int4;
+                return r * row_int4 + (w & 1) * (row_int4 >> 1) + (w >> 1);  // plane (w & 1), block (w >> 1)
+            };
+            int4 xq[kXPre];
+            int xu[kXPre];
+#pragma unroll
+            for (int i = 0; i < kXPre; ++i) {
+                xu[i] = min(tid + i * static_cast<int>(blockDim.x), x_units - 1);  // spare threads repeat the last unit
+                xq[i] = pre_q[xu[i]];
+            }
+            const int su = min(tid, rows * kb - 1);
+            const float xs0 = pre_scale[su];
+            const int xm0 = pre_sum[su];
+            __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
+            request_weights();
+#pragma unroll
+            for (int i = 0; i < kXPre; ++i) reinterpret_cast<int4*>(qx)[x_lds_index(xu[i])] = xq[i];
+            sx[su] = xs0;
+            sumx[su] = xm0;
+            for (int u = tid + kXPre * static_cast<int>(blockDim.x); u < x_units; u += blockDim.x)
+                reinterpret_cast<int4*>(qx)[x_lds_index(u)] = pre_q[u];
+            for (int u = tid + static_cast<int>(blockDim.x); u < rows * kb; u += blockDim.x) {
+                sx[u] = pre_scale[u];
+                sumx[u] = pre_sum[u];
             }
         }
 
-        // ---- 3. quantized X into LDS (waits for the X requests only)
-#pragma unroll
-        for (int i = 0; i < kXPre; ++i) reinterpret_cast<int4*>(qx)[x_lds_index(xu[i])] = xq[i];
-        sx[su] = xs0;
-        sumx[su] = xm0;
-        for (int u = tid + kXPre * static_cast<int>(blockDim.x); u < x_units; u += blockDim.x)
-            reinterpret_cast<int4*>(qx)[x_lds_index(u)] = pre_q[u];
-        for (int u = tid + static_cast<int>(blockDim.x); u < rows * kb; u += blockDim.x) {
-            sx[u] = pre_scale[u];
-            sumx[u] = pre_sum[u];
-        }
+        // X is complete in LDS once every wavefront is here; none of them has had to wait
+        // for its weights yet
+        __syncthreads();
 
         // unpack once; lanes that own no block get a zero scale
 #pragma unroll
@@ -392,7 +437,6 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
                 wd[j][c] = (ok[j] && (kLpb == 1 || half == 0)) ? half_bits_to_f32(rawd[j][c]) : 0.0f;
             }
     }
-    __syncthreads();
 
     // ---- 3. two rows per pass
     const int cells = rows * kCols;
@@ -528,21 +572,21 @@ hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* 
     return hipGetLastError();
 }
 
-template <int kType, bool kDots>
-hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const GemvActivations& pre, const uint8_t* weight,
-                       int rows, int in_dim, int out_dim, const GemvTuning& tune) {
+template <int kType, bool kDots, bool kFusedX>
+hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const float* input, const GemvActivations& pre,
+                       const uint8_t* weight, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
     const int groups = (out_dim + kCols - 1) / kCols;
     const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);  // several of these workgroups share a unit: no balancing
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
-    auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
+    auto kernel = gemv_rows_kernel<kType, kCols, kDots, kFusedX>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, reinterpret_cast<const int4*>(pre.q),
-                       pre.scale, pre.sum, weight, rows, in_dim, out_dim, slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input,
+                       reinterpret_cast<const int4*>(pre.q), pre.scale, pre.sum, weight, rows, in_dim, out_dim, slices);
     return hipGetLastError();
 }
 
@@ -550,8 +594,8 @@ template <int kType>
 hipError_t launch_gemv_type(hipStream_t stream, float* dst, int* dots, const float* input, const GemvActivations& pre,
                             const uint8_t* weight, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     if (pre.q != nullptr) {
-        return dots ? launch_rows<kType, true>(stream, dst, dots, pre, weight, rows, in_dim, out_dim, tune)
-                    : launch_rows<kType, false>(stream, dst, dots, pre, weight, rows, in_dim, out_dim, tune);
+        return dots ? launch_rows<kType, true, false>(stream, dst, dots, nullptr, pre, weight, rows, in_dim, out_dim, tune)
+                    : launch_rows<kType, false, false>(stream, dst, dots, nullptr, pre, weight, rows, in_dim, out_dim, tune);
     }
     if (rows == 1) {
         return dots ? launch_fused<kType, 1, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
@@ -561,7 +605,8 @@ hipError_t launch_gemv_type(hipStream_t stream, float* dst, int* dots, const flo
         return dots ? launch_fused<kType, 2, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
                     : launch_fused<kType, 2, false>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
     }
-    return hipErrorInvalidValue;  // three or more rows need pre-quantized activations
+    return dots ? launch_rows<kType, true, true>(stream, dst, dots, input, pre, weight, rows, in_dim, out_dim, tune)
+                : launch_rows<kType, false, true>(stream, dst, dots, input, pre, weight, rows, in_dim, out_dim, tune);
 }
 
 }  // namespace

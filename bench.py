@@ -46,6 +46,9 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
+                         "read kernel over the same number of bytes and of the Q8_0 M=512 GEMM, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -120,6 +123,80 @@ def main() -> int:
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
         return wall, e0.elapsed_time(e1) * 1e-3
+
+    def decode_sweep(layers=32, token_steps=20):
+        """Matmuls of one Llama-3-8B-shaped decode step (Q4_0, 32 layers of QKV, O, gate, up,
+        down), every layer with its own weight memory, as one HIP graph per token."""
+        shapes = [("qkv", 6144, 4096), ("o", 4096, 4096), ("gate", 14336, 4096), ("up", 14336, 4096),
+                  ("down", 4096, 14336)]
+        launch = _lib.lib().afhip_launch_linear_f32
+        # one layer of synthetic weights, repacked into `layers` separate device buffers
+        per_layer = []
+        for li, (_, n, k) in enumerate(shapes):
+            per_layer.append(prepared_copies(Q4, n, k, layers, 500 + li))
+        weight_bytes = layers * sum(n * (k // 32) * 18 for _, n, k in shapes)
+        out = {"what": "32 layers x (QKV 6144x4096, O 4096x4096, gate and up 14336x4096, down 4096x14336), Q4_0, "
+                       "one set of random weights repacked into 32 distinct device copies; matmuls only",
+               "weight_bytes_per_token": weight_bytes}
+        for m in (1, 5):
+            xs = {k: torch.from_numpy(synth.activations(900 + k, m, k)).to(dev) for k in (4096, 14336)}
+            ys = {n: torch.empty((m, n), dtype=torch.float32, device=dev) for n in (6144, 4096, 14336)}
+            wsb = max(kernels.workspaceBytes(Q4, m, k, n) for _, n, k in shapes)
+            scratch = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
+
+            def token(st):
+                for layer in range(layers):
+                    for li, (_, n, k) in enumerate(shapes):
+                        rc = launch(st, Q4, _lib.LAYOUT_PREPARED, buf(ys[n]), buf(xs[k]), buf(per_layer[li][layer]), m, k, n,
+                                    buf(scratch), -1)
+                        if rc != 0:
+                            raise RuntimeError(f"launch failed: {rc}")
+
+            token(stream)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                token(torch.cuda.current_stream().cuda_stream)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(token_steps):
+                graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            t = e0.elapsed_time(e1) * 1e-3 / token_steps
+            out[f"m{m}"] = {"us_per_step": round(t * 1e6, 1), "steps_per_s": round(1.0 / t, 1),
+                            "tokens_per_s": round(m / t, 1), "weight_GBps": round(weight_bytes / t / 1e9, 1),
+                            "frac_hbm_peak": round(weight_bytes / t / HBM_PEAK_BPS, 4)}
+        return out
+
+    if args.counter_probe:
+        n_launch, copies = 40, 8
+        launch = _lib.lib().afhip_launch_linear_f32
+        ws = prepared_copies(Q4, 14336, 4096, copies, 2024)
+        x = torch.from_numpy(synth.activations(2025, 1, 4096)).to(dev)
+        y = torch.empty((1, 14336), dtype=torch.float32, device=dev)
+        scratch = torch.empty(max(kernels.workspaceBytes(Q4, 1, 4096, 14336), 16), dtype=torch.uint8, device=dev)
+        for i in range(n_launch):
+            launch(stream, Q4, _lib.LAYOUT_PREPARED, buf(y), buf(x), buf(ws[i % copies]), 1, 4096, 14336, buf(scratch), -1)
+        torch.cuda.synchronize()
+        w_bytes = 14336 * 128 * 18
+        srcs = [torch.full((w_bytes,), 1, dtype=torch.uint8, device=dev) for _ in range(copies)]
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        for i in range(n_launch):
+            _lib.lib().afhip_launch_stream_read(stream, buf(srcs[i % copies]), buf(sink))
+        torch.cuda.synchronize()
+        wg = prepared_copies(Q8, 4096, 4096, 2, 7)
+        xg = torch.from_numpy(synth.activations(8, 512, 4096)).to(dev)
+        yg = torch.empty((512, 4096), dtype=torch.float32, device=dev)
+        sg = torch.empty(kernels.workspaceBytes(Q8, 512, 4096, 4096), dtype=torch.uint8, device=dev)
+        for i in range(n_launch):
+            launch(stream, Q8, _lib.LAYOUT_PREPARED, buf(yg), buf(xg), buf(wg[i % 2]), 512, 4096, 4096, buf(sg), -1)
+        torch.cuda.synchronize()
+        print(json.dumps({"counter_probe": {"launches_each": n_launch, "gemv_bytes": gemv_bytes(Q4, 1, 4096, 14336),
+                                            "stream_read_bytes": w_bytes}}))
+        return 0
 
     # ---- headline: Q4_0 decode GEMV, M=1, K=4096, N=14336 --------------------------
     rows, in_dim, out_dim = 1, 4096, 14336
@@ -201,12 +278,14 @@ def main() -> int:
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
         for m in (128, 512, 2048):
-            gsteps = 20
-            w_s, e_s = time_config(Q8, m, 4096, 4096, gsteps, 3, 4, 7)
+            gsteps = 200
+            w_s, e_s = time_config(Q8, m, 4096, 4096, gsteps, 20, 4, 7)
             ops = 2.0 * m * 4096 * 4096
-            extra[f"q8_gemm_m{m}_k4096_n4096"] = {"us_per_call": round(e_s / gsteps * 1e6, 3),
+            extra[f"q8_gemm_m{m}_k4096_n4096"] = {"what": "activation quantizer + int8-MFMA GEMM kernel, per call",
+                                                 "us_per_call": round(e_s / gsteps * 1e6, 3),
                                                  "TOPS": round(ops * gsteps / e_s / 1e12, 3),
                                                  "frac_int8_mfma_peak": round(ops * gsteps / e_s / INT8_MFMA_PEAK_OPS, 5)}
+        extra["llama3_8b_decode_matmuls"] = decode_sweep()
         result["extra"] = extra
 
     # ---- CPU baseline: the engine's CPU route restated in C, on this host --------------

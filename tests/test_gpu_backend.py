@@ -54,7 +54,9 @@ def test_linear_no_bias_matches_cpu_engine(cb, fmt, keep_raw):
     stats = cb.debugStats()
     assert stats["launches_small_batch"] == 2 and stats["resident_weight_bytes"] >= w.size
     assert stats["launches_prepare"] == (0 if keep_raw else 1)
-    assert stats["launches_activation_quant"] == 2  # five rows: activations are quantized by their own kernel
+    # a small X on repacked weights: the GEMV quantizes it in its own prologue; the
+    # generic kernels (raw GGUF layout) read activations quantized by a separate kernel
+    assert stats["launches_activation_quant"] == (2 if keep_raw else 0)
     for t in (yt, yt2, xt):
         cb.freeTensor(t)
     assert cb.debugStats()["pooled_buffers"] >= 2

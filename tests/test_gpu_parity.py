@@ -161,9 +161,10 @@ def test_f32_route_matches_oracle(fmt, layout, rows, in_dim, out_dim):
 
 
 @pytest.mark.parametrize("fmt", [Q8, Q4])
-def test_forced_dispatch_kinds_agree(fmt):
+@pytest.mark.parametrize("rows", [6, 12])  # 12 rows forced onto the GEMV kernels: activations quantized by their own kernel
+def test_forced_dispatch_kinds_agree(fmt, rows):
     """A plan may force any kernel family; all of them compute the same op."""
-    rows, in_dim, out_dim = 6, 512, 640
+    in_dim, out_dim = 512, 640
     x = synth.activations(77, rows, in_dim)
     w = synth.weights(fmt, 78, out_dim, in_dim)
     wd = G.prepare(fmt, w, out_dim, in_dim)
