@@ -25,6 +25,15 @@ __device__ __forceinline__ int dot4(int a, int b, int acc) {
     return __builtin_amdgcn_sdot4(a, b, acc, false);
 }
 
+// ---- 8 x 4-bit dots with 32-bit accumulate: signed x signed (v_dot8_i32_i4) and
+// unsigned x unsigned (v_dot8_u32_u4, wraps modulo 2^32).  Nibble i of a meets nibble i of b.
+__device__ __forceinline__ int dot8_i4(int a, int b, int acc) {
+    return __builtin_amdgcn_sdot8(a, b, acc, false);
+}
+__device__ __forceinline__ uint32_t dot8_u4(uint32_t a, uint32_t b, uint32_t acc) {
+    return __builtin_amdgcn_udot8(a, b, acc, false);
+}
+
 // ---- DPP lane exchanges.  Controls: quad_perm encodes four 2-bit selectors,
 // 0x140 = row_mirror, 0x141 = row_half_mirror (rows are 16 lanes).
 template <int kCtrl>

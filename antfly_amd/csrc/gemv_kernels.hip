@@ -52,7 +52,13 @@ constexpr int kSliceBlocks = 128;  // 4096 values
 // Quantizes one 32-value block held by one thread (8 float4) and stores it.
 // Same arithmetic as ops/native_compute.zig:23799-23832: f32 scale = max|x|/127,
 // one reciprocal, round half away from zero, clamp to +-127, zero block -> scale 1.
-template <int kType>
+// kNibblePlanes (Q4_0 only): instead of int8 values, LDS gets the high nibbles h = q >> 4
+// (signed, -8..7) and the low nibbles l = q & 15 (unsigned) of the block, each packed
+// eight to a word in the order of the weight nibbles (bits 8t..8t+3 = value 4d+t, bits
+// 8t+4..8t+7 = value 16+4d+t of word d), and sum_row gets -8 * sum(l): with weight
+// nibbles n (value n - 8, which is n ^ 8 read as a signed nibble)
+//   dot(q, n - 8) = 16 * dot_i4(h, n ^ 8) + dot_u4(l, n) - 8 * sum(l).
+template <int kType, bool kNibblePlanes = false>
 __device__ __forceinline__ void quantize_block_to_lds(const float4 (&v)[8], int block, int kb, int* q_row,
                                                       float* scale_row, int* sum_row) {
     float m = 0.0f;
@@ -69,6 +75,22 @@ __device__ __forceinline__ void quantize_block_to_lds(const float4 (&v)[8], int 
         const int q2 = act_quant(v[i].z, inv), q3 = act_quant(v[i].w, inv);
         p[i] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
         total = dot4(p[i], 0x01010101, total);
+    }
+    if (kType == 2 && kNibblePlanes) {
+        int h[4], l[4];
+        uint32_t lsum = 0;
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            const uint32_t a = static_cast<uint32_t>(p[d]), b = static_cast<uint32_t>(p[4 + d]);
+            l[d] = static_cast<int>((a & 0x0F0F0F0Fu) | ((b & 0x0F0F0F0Fu) << 4));
+            h[d] = static_cast<int>(((a >> 4) & 0x0F0F0F0Fu) | (b & 0xF0F0F0F0u));
+            lsum = dot8_u4(static_cast<uint32_t>(l[d]), 0x11111111u, lsum);
+        }
+        reinterpret_cast<int4*>(q_row)[block] = make_int4(h[0], h[1], h[2], h[3]);
+        reinterpret_cast<int4*>(q_row + kb * 4)[block] = make_int4(l[0], l[1], l[2], l[3]);
+        scale_row[block] = s;
+        sum_row[block] = -8 * static_cast<int>(lsum);
+        return;
     }
     const int4 lo = make_int4(p[0], p[1], p[2], p[3]), hi = make_int4(p[4], p[5], p[6], p[7]);
     if (kType == 2) {
@@ -159,12 +181,12 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         request_weights();
         __builtin_amdgcn_sched_barrier(0);
         const int r = xb / kb, b = xb - r * kb;
-        quantize_block_to_lds<kType>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+        quantize_block_to_lds<kType, true>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
         for (int xb2 = tid + static_cast<int>(blockDim.x); xb2 < x_blocks; xb2 += blockDim.x) {  // more blocks than threads
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb2 * 8 + i];
             const int r2 = xb2 / kb, b2 = xb2 - r2 * kb;
-            quantize_block_to_lds<kType>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
+            quantize_block_to_lds<kType, true>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
         }
     } else {
         request_weights();
@@ -215,16 +237,18 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
                 const int* a = ar[j][r];
                 int dot;
                 if (kType == 2) {
-                    // nibbles stay unsigned: dot(qx, n - 8) = dot(qx, n) - 8 * sum(qx)
-                    dot = -8 * smr[j][r];
-                    dot = dot4(static_cast<int>(w.x & 0x0F0F0F0Fu), a[0], dot);
-                    dot = dot4(static_cast<int>(w.y & 0x0F0F0F0Fu), a[1], dot);
-                    dot = dot4(static_cast<int>(w.z & 0x0F0F0F0Fu), a[2], dot);
-                    dot = dot4(static_cast<int>(w.w & 0x0F0F0F0Fu), a[3], dot);
-                    dot = dot4(static_cast<int>((w.x >> 4) & 0x0F0F0F0Fu), a[4], dot);
-                    dot = dot4(static_cast<int>((w.y >> 4) & 0x0F0F0F0Fu), a[5], dot);
-                    dot = dot4(static_cast<int>((w.z >> 4) & 0x0F0F0F0Fu), a[6], dot);
-                    dot = dot4(static_cast<int>((w.w >> 4) & 0x0F0F0F0Fu), a[7], dot);
+                    // 4-bit dots on the packed nibbles, nothing is unpacked: a[0..3] = high
+                    // nibbles of the activations (signed), a[4..7] = low nibbles (unsigned),
+                    // smr = -8 * sum(low nibbles); see quantize_block_to_lds
+                    int hi = dot8_i4(static_cast<int>(w.x ^ 0x88888888u), a[0], 0);
+                    hi = dot8_i4(static_cast<int>(w.y ^ 0x88888888u), a[1], hi);
+                    hi = dot8_i4(static_cast<int>(w.z ^ 0x88888888u), a[2], hi);
+                    hi = dot8_i4(static_cast<int>(w.w ^ 0x88888888u), a[3], hi);
+                    uint32_t lo = dot8_u4(w.x, static_cast<uint32_t>(a[4]), static_cast<uint32_t>(smr[j][r]));
+                    lo = dot8_u4(w.y, static_cast<uint32_t>(a[5]), lo);
+                    lo = dot8_u4(w.z, static_cast<uint32_t>(a[6]), lo);
+                    lo = dot8_u4(w.w, static_cast<uint32_t>(a[7]), lo);
+                    dot = (hi << 4) + static_cast<int>(lo);
                 } else {
                     dot = dot4(static_cast<int>(w.x), a[0], 0);
                     dot = dot4(static_cast<int>(w.y), a[1], dot);
