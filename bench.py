@@ -31,6 +31,21 @@ Q4, Q8 = 2, 8
 BLOCK_BYTES = {Q4: 18, Q8: 34}
 
 
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel from the committed counter summary
+    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-probe`, each scaled
+    by a kernel of known traffic in the same run), or None when that file is not there."""
+    path = os.path.join(ROOT, "profiles", "gemv_q4_0_m1_and_gemm_q8_0_m512_counters.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch_gemv_q4_0_m1:"):
+                    return int(float(line.split(":", 1)[1]))
+    except OSError:
+        pass
+    return None
+
+
 def gemv_bytes(fmt, rows, in_dim, out_dim):
     """Algorithmic bytes of one call: weights once + f32 activations + f32 outputs."""
     return out_dim * (in_dim // 32) * BLOCK_BYTES[fmt] + 4 * rows * in_dim + 4 * rows * out_dim
@@ -221,7 +236,7 @@ def main() -> int:
                    "rows": rows, "in_dim": in_dim, "out_dim": out_dim, "weight_copies": args.copies,
                    "bytes_per_step": nbytes},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK_BPS, 4), "traffic": None,
+                     "frac": round(achieved * 1e9 / HBM_PEAK_BPS, 4), "traffic": measured_traffic(),
                      "kernel": "gemv_fused_kernel<Q4_0, rows=1>", "us_per_launch": round(ev / args.steps * 1e6, 3)},
     }
 
