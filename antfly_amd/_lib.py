@@ -81,6 +81,7 @@ SIGNATURES = {
     "afhip_uses_activation_quant": (_i, [_sz, _sz, _sz]),
     "afhip_linear_workspace_bytes": (_sz, [_i, _sz, _sz, _sz]),
     "afhip_launch_linear_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_linear_pair_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_q8_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_linear_q4_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_prepare_weight": (_st, [_vp, _i, Buffer, Buffer, _sz, _sz]),
@@ -111,6 +112,7 @@ SIGNATURES = {
     "afhip_tensor_device_ptr": (C.c_uint64, [_vp]),
     "afhip_tensor_byte_len": (_sz, [_vp]),
     "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "afhip_compute_linear_no_bias_pair": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_planned": (_st, [_vp, C.POINTER(PlannedRequest), C.POINTER(_vp)]),
     "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
     "afhip_smoke_q8_0": (_st, []),

@@ -17,8 +17,11 @@ size_t block_bytes(int tensor_type);
 
 // The op behind every linear launcher.  dots.ptr != 0 switches to "write the
 // int32 block dots instead of Y".
+// weight_b.ptr != 0 adds a second matrix of the same shape and layout that shares the
+// input (result in dst_b; not together with dots).
 afhip_status linear_impl(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
-                         int dispatch, afhip_buffer dots, LaunchCounters* counters);
+                         int dispatch, afhip_buffer dots, LaunchCounters* counters,
+                         afhip_buffer dst_b = afhip_buffer{0, 0}, afhip_buffer weight_b = afhip_buffer{0, 0});
 
 }  // namespace afhip

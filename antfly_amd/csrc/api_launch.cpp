@@ -78,8 +78,10 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
 
 afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
-                         int dispatch, afhip_buffer dots, LaunchCounters* counters) {
+                         int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
+                         afhip_buffer weight_b) {
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -99,6 +101,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     }
     if (!checked_mul(in_count, 4, &bytes) || bytes > input.len) return AFHIP_ERR_INVALID_STATE;
     if (w_bytes > weight.len) return AFHIP_ERR_INVALID_STATE;
+    if (pair) {
+        if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;
+        if (!checked_mul(out_count, 4, &bytes) || bytes > dst_b.len || w_bytes > weight_b.len) return AFHIP_ERR_INVALID_STATE;
+    }
     if (out_count == 0) return AFHIP_OK;
     if (!fits_u32(rows) || !fits_u32(in_dim) || !fits_u32(out_dim) || in_dim > 0x7fffffff || out_dim > 0x7fffffff ||
         rows > 0x7fffffff)
@@ -107,8 +113,13 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     // 128-bit activation loads; prepared weights are read with 128-bit loads, raw GGUF bytes with 16-bit loads
     if (input.ptr % 16 != 0 || dst.ptr % 4 != 0 || dots.ptr % 4 != 0) return AFHIP_ERR_INVALID_STATE;
     if (weight.ptr % (layout == AFHIP_LAYOUT_PREPARED ? 16 : 2) != 0) return AFHIP_ERR_INVALID_STATE;
+    if (pair && (dst_b.ptr == 0 || weight_b.ptr == 0 || dst_b.ptr % 4 != 0 ||
+                 weight_b.ptr % (layout == AFHIP_LAYOUT_PREPARED ? 16 : 2) != 0))
+        return AFHIP_ERR_INVALID_STATE;
 
     float* y = reinterpret_cast<float*>(dst.ptr);
+    float* y_b = reinterpret_cast<float*>(dst_b.ptr);
+    const uint8_t* w_b = reinterpret_cast<const uint8_t*>(weight_b.ptr);
     int* dot_out = reinterpret_cast<int*>(dots.ptr);
     const float* x = reinterpret_cast<const float*>(input.ptr);
     const uint8_t* w = reinterpret_cast<const uint8_t*>(weight.ptr);
@@ -119,6 +130,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         if (counters) counters->f32_route++;
         hipError_t e = launch_linear_generic(stream, tensor_type, layout, false, y, nullptr, x, nullptr, nullptr, w,
                                              static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+        if (e == hipSuccess && pair) {
+            if (counters) counters->f32_route++;
+            e = launch_linear_generic(stream, tensor_type, layout, false, y_b, nullptr, x, nullptr, nullptr, w_b,
+                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+        }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
 
@@ -140,6 +156,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         if (e != hipSuccess) return static_cast<afhip_status>(e);
         e = launch_gemm_i8(stream, tensor_type, want_dots ? nullptr : y, dot_out, ws.qx, ws.sx, w, static_cast<int>(rows),
                            static_cast<int>(in_dim), static_cast<int>(out_dim));
+        if (e == hipSuccess && pair) {  // the second matrix reuses the quantized activations
+            if (counters) counters->mm++;
+            e = launch_gemm_i8(stream, tensor_type, y_b, nullptr, ws.qx, ws.sx, w_b, static_cast<int>(rows),
+                               static_cast<int>(in_dim), static_cast<int>(out_dim));
+        }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     if (fused_ok) {
@@ -171,9 +192,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                 pre.scale = ws.sx + r0 * kb;
                 pre.sum = ws.sums + r0 * kb;
             }
+            // a pair is one launch over the columns of both matrices
             hipError_t e = launch_gemv_fused(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
                                              want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, pre, w,
-                                             nr, static_cast<int>(in_dim), static_cast<int>(out_dim), tune);
+                                             nr, static_cast<int>(in_dim), static_cast<int>(out_dim), tune,
+                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr);
             if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         return AFHIP_OK;
@@ -193,6 +216,9 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     if (e != hipSuccess) return static_cast<afhip_status>(e);
     e = launch_linear_generic(stream, tensor_type, layout, true, want_dots ? nullptr : y, dot_out, nullptr, ws.qx, ws.sx,
                               w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+    if (e == hipSuccess && pair)
+        e = launch_linear_generic(stream, tensor_type, layout, true, y_b, nullptr, nullptr, ws.qx, ws.sx, w_b,
+                                  static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
@@ -299,6 +325,15 @@ afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, 
                                      afhip_buffer workspace, int dispatch) {
     return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
                        afhip_buffer{0, 0}, nullptr);
+}
+
+afhip_status afhip_launch_linear_pair_f32(void* stream, int tensor_type, int layout, afhip_buffer dst_a,
+                                          afhip_buffer dst_b, afhip_buffer input, afhip_buffer weight_a,
+                                          afhip_buffer weight_b, size_t rows, size_t in_dim, size_t out_dim,
+                                          afhip_buffer workspace, int dispatch) {
+    if (weight_b.ptr == 0 || (dst_b.ptr == 0 && rows != 0 && out_dim != 0)) return AFHIP_ERR_INVALID_STATE;
+    return linear_impl(stream, tensor_type, layout, dst_a, input, weight_a, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr, dst_b, weight_b);
 }
 
 afhip_status afhip_launch_linear_q8_0_f32(void* stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight_raw,

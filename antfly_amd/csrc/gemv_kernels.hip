@@ -105,14 +105,24 @@ __device__ __forceinline__ void quantize_block_to_lds(const float4 (&v)[8], int 
     sum_row[block] = total;
 }
 
+// Where a GEMV launch reads its weights and writes its results: one matrix, or two of
+// the same shape that share X (the engine's linearNoBiasPair, ops/ops.zig:909).  Column
+// groups [0, groups_each) belong to the first matrix, [groups_each, 2*groups_each) to
+// the second.
+struct GemvTargets {
+    float* dst_a;
+    float* dst_b;
+    const uint8_t* weight_a;
+    const uint8_t* weight_b;  // null: one matrix
+    int groups_each;
+};
+
 constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
 // One or two rows of f32 activations, quantized in the prologue of every workgroup.
 template <int kType, int kRows, int kCols, bool kWriteDots>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
-    float* __restrict__ dst, int* __restrict__ dots, const float* __restrict__ input,
-    const uint8_t* __restrict__ weight, int in_dim,
-    int out_dim, int slices) {
+    GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices) {
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
     constexpr int kBlocksPerStep = kWave / kLpb;
@@ -127,8 +137,6 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     float* partial = reinterpret_cast<float*>(sumx + kRows * kb);                     // [waves][kRows*kCols]
 
     const size_t blocks = static_cast<size_t>(out_dim) * kb;
-    const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
-    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -140,9 +148,16 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const int lane_block = lane / kLpb;
     const int slice = wave % slices;
     const int groups_per_wg = waves / slices;
-    const int group = blockIdx.x * groups_per_wg + wave / slices;
+    // column group -> matrix (wave-uniform), columns o0 .. o0 + kCols - 1 of it
+    const int group_all = blockIdx.x * groups_per_wg + wave / slices;
+    const bool second = tg.weight_b != nullptr && group_all >= tg.groups_each;
+    const int group = second ? group_all - tg.groups_each : group_all;
+    const uint8_t* weight = second ? tg.weight_b : tg.weight_a;
+    float* dst = second ? tg.dst_b : tg.dst_a;
+    const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
+    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
     const int o0 = group * kCols;
-    const bool active = o0 < out_dim;
+    const bool active = group < tg.groups_each && o0 < out_dim;
 
     // ---- 1. requests: first the activations (wavefronts that quantize a block per
     // thread), then every weight byte this wavefront needs.  Loads complete in order, so
@@ -276,7 +291,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const int cell = lane & (kPadded - 1);  // this lane holds the total of accumulator `cell`
     const int cr = cell / kCols, cc = cell - cr * kCols;
     if (slices == 1) {
-        if (lane < kPadded && cell < kCells && o0 + cc < out_dim && dst)
+        if (active && lane < kPadded && cell < kCells && o0 + cc < out_dim && dst)
             dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
         return;
     }
@@ -286,10 +301,14 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     for (int i = tid; i < cells; i += blockDim.x) {
         const int gi = i / kCells, rc = i - gi * kCells;
         const int r = rc / kCols, c = rc - r * kCols;
-        const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
+        const int ga = blockIdx.x * groups_per_wg + gi;
+        const bool sec = tg.weight_b != nullptr && ga >= tg.groups_each;
+        const int g = sec ? ga - tg.groups_each : ga;
+        float* d = sec ? tg.dst_b : tg.dst_a;
+        const int o = g * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
-        if (o < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o] = total;
+        if (g < tg.groups_each && o < out_dim && d) d[static_cast<size_t>(r) * out_dim + o] = total;
     }
 }
 
@@ -305,12 +324,11 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
 // pre_sum [rows][in_dim/32]) and are copied into LDS.
 // =====================================================================
 template <int kType, int kCols, bool kWriteDots, bool kFusedX>
-__global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ dst, int* __restrict__ dots,
+__global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* __restrict__ dots,
                                                             const float* __restrict__ input,
                                                             const int4* __restrict__ pre_q,
                                                             const float* __restrict__ pre_scale,
-                                                            const int* __restrict__ pre_sum,
-                                                            const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                            const int* __restrict__ pre_sum, int rows, int in_dim,
                                                             int out_dim, int slices) {
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
@@ -327,8 +345,6 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     float* partial = reinterpret_cast<float*>(sumx + rows * kb);                     // [waves][rows*kCols]
 
     const size_t blocks = static_cast<size_t>(out_dim) * kb;
-    const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
-    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -338,9 +354,16 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     const int lane_block = lane / kLpb;
     const int slice = wave % slices;
     const int groups_per_wg = waves / slices;
-    const int group = blockIdx.x * groups_per_wg + wave / slices;
+    // column group -> matrix (wave-uniform), columns o0 .. o0 + kCols - 1 of it
+    const int group_all = blockIdx.x * groups_per_wg + wave / slices;
+    const bool second = tg.weight_b != nullptr && group_all >= tg.groups_each;
+    const int group = second ? group_all - tg.groups_each : group_all;
+    const uint8_t* weight = second ? tg.weight_b : tg.weight_a;
+    float* dst = second ? tg.dst_b : tg.dst_a;
+    const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
+    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
     const int o0 = group * kCols;
-    const bool active = o0 < out_dim;
+    const bool active = group < tg.groups_each && o0 < out_dim;
 
     int wv[kSteps][kCols][kWords];
     float wd[kSteps][kCols];
@@ -511,7 +534,7 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
         const bool mine = lane < kPadded && cell < 2 * kCols && (rr == 0 || r1 != r0);
         const int r = rr == 0 ? r0 : r1;
         if (slices == 1) {
-            if (mine && o0 + cc < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + cc] = red[0];
+            if (active && mine && o0 + cc < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o0 + cc] = red[0];
         } else if (mine) {
             partial[wave * cells + r * kCols + cc] = red[0];
         }
@@ -521,10 +544,14 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(float* __restrict__ d
     for (int i = tid; i < groups_per_wg * cells; i += blockDim.x) {
         const int gi = i / cells, rc = i - gi * cells;
         const int r = rc / kCols, c = rc - r * kCols;
-        const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
+        const int ga = blockIdx.x * groups_per_wg + gi;
+        const bool sec = tg.weight_b != nullptr && ga >= tg.groups_each;
+        const int g = sec ? ga - tg.groups_each : ga;
+        float* d = sec ? tg.dst_b : tg.dst_a;
+        const int o = g * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * cells + rc];
-        if (o < out_dim && dst) dst[static_cast<size_t>(r) * out_dim + o] = total;
+        if (g < tg.groups_each && o < out_dim && d) d[static_cast<size_t>(r) * out_dim + o] = total;
     }
 }
 
@@ -579,11 +606,13 @@ hipError_t allow_large_lds(Kernel kernel, size_t lds, size_t* limit) {
 }
 
 template <int kType, int kRows, bool kDots>
-hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* input, const uint8_t* weight, int in_dim,
+hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, const float* input, int in_dim,
                         int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
-    const int groups = (out_dim + kCols - 1) / kCols;
+    GemvTargets tg = tg0;
+    tg.groups_each = (out_dim + kCols - 1) / kCols;
+    const int groups = tg.groups_each * (tg.weight_b ? 2 : 1);
     const int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
@@ -591,17 +620,18 @@ hipError_t launch_fused(hipStream_t stream, float* dst, int* dots, const float* 
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input, weight, in_dim, out_dim,
-                       slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices);
     return hipGetLastError();
 }
 
 template <int kType, bool kDots, bool kFusedX>
-hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const float* input, const GemvActivations& pre,
-                       const uint8_t* weight, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
+hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, const float* input, const GemvActivations& pre,
+                       int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
-    const int groups = (out_dim + kCols - 1) / kCols;
+    GemvTargets tg = tg0;
+    tg.groups_each = (out_dim + kCols - 1) / kCols;
+    const int groups = tg.groups_each * (tg.weight_b ? 2 : 1);
     const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);  // several of these workgroups share a unit: no balancing
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
@@ -609,28 +639,28 @@ hipError_t launch_rows(hipStream_t stream, float* dst, int* dots, const float* i
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, dots, input,
-                       reinterpret_cast<const int4*>(pre.q), pre.scale, pre.sum, weight, rows, in_dim, out_dim, slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input,
+                       reinterpret_cast<const int4*>(pre.q), pre.scale, pre.sum, rows, in_dim, out_dim, slices);
     return hipGetLastError();
 }
 
 template <int kType>
-hipError_t launch_gemv_type(hipStream_t stream, float* dst, int* dots, const float* input, const GemvActivations& pre,
-                            const uint8_t* weight, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
+hipError_t launch_gemv_type(hipStream_t stream, const GemvTargets& tg, int* dots, const float* input,
+                            const GemvActivations& pre, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     if (pre.q != nullptr) {
-        return dots ? launch_rows<kType, true, false>(stream, dst, dots, nullptr, pre, weight, rows, in_dim, out_dim, tune)
-                    : launch_rows<kType, false, false>(stream, dst, dots, nullptr, pre, weight, rows, in_dim, out_dim, tune);
+        return dots ? launch_rows<kType, true, false>(stream, tg, dots, nullptr, pre, rows, in_dim, out_dim, tune)
+                    : launch_rows<kType, false, false>(stream, tg, dots, nullptr, pre, rows, in_dim, out_dim, tune);
     }
     if (rows == 1) {
-        return dots ? launch_fused<kType, 1, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
-                    : launch_fused<kType, 1, false>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        return dots ? launch_fused<kType, 1, true>(stream, tg, dots, input, in_dim, out_dim, tune)
+                    : launch_fused<kType, 1, false>(stream, tg, dots, input, in_dim, out_dim, tune);
     }
     if (rows == 2) {
-        return dots ? launch_fused<kType, 2, true>(stream, dst, dots, input, weight, in_dim, out_dim, tune)
-                    : launch_fused<kType, 2, false>(stream, dst, dots, input, weight, in_dim, out_dim, tune);
+        return dots ? launch_fused<kType, 2, true>(stream, tg, dots, input, in_dim, out_dim, tune)
+                    : launch_fused<kType, 2, false>(stream, tg, dots, input, in_dim, out_dim, tune);
     }
-    return dots ? launch_rows<kType, true, true>(stream, dst, dots, input, pre, weight, rows, in_dim, out_dim, tune)
-                : launch_rows<kType, false, true>(stream, dst, dots, input, pre, weight, rows, in_dim, out_dim, tune);
+    return dots ? launch_rows<kType, true, true>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune)
+                : launch_rows<kType, false, true>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
 
 }  // namespace
@@ -646,11 +676,12 @@ int gemv_fused_max_in_dim() { return 16 * kSliceBlocks * 32; }
 
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
                              const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
-                             int out_dim, const GemvTuning& tune) {
+                             int out_dim, const GemvTuning& tune, float* dst_b, const uint8_t* weight_b_prepared) {
     if (in_dim > gemv_fused_max_in_dim()) return hipErrorInvalidValue;
-    if (tensor_type == 2)
-        return launch_gemv_type<2>(stream, dst, dots, input, pre, weight_prepared, rows, in_dim, out_dim, tune);
-    return launch_gemv_type<8>(stream, dst, dots, input, pre, weight_prepared, rows, in_dim, out_dim, tune);
+    if (weight_b_prepared != nullptr && dots != nullptr) return hipErrorInvalidValue;  // block dots: one matrix at a time
+    const GemvTargets tg{dst, dst_b, weight_prepared, weight_b_prepared, 0};
+    if (tensor_type == 2) return launch_gemv_type<2>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
+    return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
 
 }  // namespace afhip

@@ -140,41 +140,8 @@ void free_tensor_storage(afhip_compute* self, afhip_tensor* t) {
 
 bool is_f32(const afhip_tensor* t) { return t->dtype == AFHIP_DTYPE_F32 && t->quant_type < 0; }  // ensureF32
 
-afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
-                                 size_t rows, size_t in_dim, size_t out_dim, int dispatch, afhip_tensor** out) {
-    // cuda_compute.zig:689-717
-    if (!self || !input || !weight || !out) return AFHIP_ERR_INVALID_ARGUMENT;
-    *out = nullptr;
-    if (!is_f32(input)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
-    if (weight->quant_type < 0 && !is_f32(weight)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
-    size_t in_count, w_count, out_count, out_bytes;
-    if (!checked_mul(rows, in_dim, &in_count) || !checked_mul(out_dim, in_dim, &w_count) ||
-        !checked_mul(rows, out_dim, &out_count) || !checked_mul(out_count, 4, &out_bytes))
-        return AFHIP_ERR_INVALID_SHAPE;
-    if (input->elem_count != in_count || weight->elem_count != w_count) return AFHIP_ERR_INVALID_SHAPE;
-    if (weight->quant_type < 0) return AFHIP_ERR_OP_UNSUPPORTED;  // dense f32 linear is another operator
-    if (weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0)
-        return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
-
-    afhip_status s = make_current(self);
-    if (s != AFHIP_OK) return s;
-    afhip_buffer device;
-    s = alloc_device_buffer(self, out_bytes, &device);
-    if (s != AFHIP_OK) return s;
-    afhip_buffer scratch{0, 0};
-    if (afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
-        s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);
-        if (s != AFHIP_OK) {
-            release_device_buffer(self, &device);
-            return s;
-        }
-    }
-    s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows, in_dim,
-                    out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters);
-    if (s != AFHIP_OK) {
-        release_device_buffer(self, &device);
-        return s;
-    }
+afhip_status make_f32_result(afhip_compute* self, afhip_buffer device, size_t rows, size_t out_dim, size_t out_count,
+                             afhip_tensor** out) {
     afhip_tensor* t = new (std::nothrow) afhip_tensor();
     if (!t) {
         release_device_buffer(self, &device);
@@ -186,6 +153,85 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
     t->elem_count = out_count;
     *out = t;
     return AFHIP_OK;
+}
+
+// weight_b / out_b null: one linear; otherwise two linears of the same shape that share
+// the input (the weights must have the same format and layout to share one launch).
+afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
+                                 size_t rows, size_t in_dim, size_t out_dim, int dispatch, afhip_tensor** out,
+                                 const afhip_tensor* weight_b = nullptr, afhip_tensor** out_b = nullptr) {
+    // cuda_compute.zig:689-717
+    const bool pair = weight_b != nullptr || out_b != nullptr;
+    if (!self || !input || !weight || !out || (pair && (!weight_b || !out_b))) return AFHIP_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (pair) *out_b = nullptr;
+    if (!is_f32(input)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    const afhip_tensor* ws[2] = {weight, weight_b};
+    size_t in_count, w_count, out_count, out_bytes;
+    if (!checked_mul(rows, in_dim, &in_count) || !checked_mul(out_dim, in_dim, &w_count) ||
+        !checked_mul(rows, out_dim, &out_count) || !checked_mul(out_count, 4, &out_bytes))
+        return AFHIP_ERR_INVALID_SHAPE;
+    if (input->elem_count != in_count) return AFHIP_ERR_INVALID_SHAPE;
+    for (int i = 0; i < (pair ? 2 : 1); ++i) {
+        const afhip_tensor* w = ws[i];
+        if (w->quant_type < 0 && !is_f32(w)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+        if (w->elem_count != w_count) return AFHIP_ERR_INVALID_SHAPE;
+        if (w->quant_type < 0) return AFHIP_ERR_OP_UNSUPPORTED;  // dense f32 linear is another operator
+        if (w->quant_type != AFHIP_TYPE_Q4_0 && w->quant_type != AFHIP_TYPE_Q8_0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    }
+    if (pair && (weight_b->quant_type != weight->quant_type || weight_b->layout != weight->layout)) {
+        // nothing to share: two independent ops, as the engine's wrapper does (ops/ops.zig:1828-1849)
+        afhip_status s = linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, dispatch, out);
+        if (s != AFHIP_OK) return s;
+        s = linear_no_bias_impl(self, input, weight_b, rows, in_dim, out_dim, dispatch, out_b);
+        if (s != AFHIP_OK) {
+            free_tensor_storage(self, *out);
+            delete *out;
+            *out = nullptr;
+        }
+        return s;
+    }
+
+    afhip_status s = make_current(self);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer device, device_b{0, 0};
+    s = alloc_device_buffer(self, out_bytes, &device);
+    if (s != AFHIP_OK) return s;
+    if (pair) {
+        s = alloc_device_buffer(self, out_bytes, &device_b);
+        if (s != AFHIP_OK) {
+            release_device_buffer(self, &device);
+            return s;
+        }
+    }
+    afhip_buffer scratch{0, 0};
+    if (afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
+        s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);
+    }
+    if (s == AFHIP_OK) {
+        s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows,
+                        in_dim, out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
+                        pair ? weight_b->buffer : afhip_buffer{0, 0});
+    }
+    if (s != AFHIP_OK) {
+        release_device_buffer(self, &device);
+        if (pair) release_device_buffer(self, &device_b);
+        return s;
+    }
+    s = make_f32_result(self, device, rows, out_dim, out_count, out);
+    if (s != AFHIP_OK) {
+        if (pair) release_device_buffer(self, &device_b);
+        return s;
+    }
+    if (pair) {
+        s = make_f32_result(self, device_b, rows, out_dim, out_count, out_b);
+        if (s != AFHIP_OK) {
+            free_tensor_storage(self, *out);
+            delete *out;
+            *out = nullptr;
+        }
+    }
+    return s;
 }
 
 }  // namespace
@@ -443,6 +489,14 @@ size_t afhip_tensor_byte_len(const afhip_tensor* t) { return t ? t->buffer.len :
 afhip_status afhip_compute_linear_no_bias(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
                                           size_t rows, size_t in_dim, size_t out_dim, afhip_tensor** out) {
     return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out);
+}
+
+afhip_status afhip_compute_linear_no_bias_pair(afhip_compute* self, const afhip_tensor* input,
+                                               const afhip_tensor* weight_a, const afhip_tensor* weight_b, size_t rows,
+                                               size_t in_dim, size_t out_dim, afhip_tensor** out_first,
+                                               afhip_tensor** out_second) {
+    if (!weight_b || !out_second) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_no_bias_impl(self, input, weight_a, rows, in_dim, out_dim, -1, out_first, weight_b, out_second);
 }
 
 afhip_status afhip_compute_linear_no_bias_planned(afhip_compute* self,

@@ -25,10 +25,13 @@ struct GemvActivations {
     const int* sum = nullptr;      // [rows][in_dim/32]
 };
 
-// rows in 1..8, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
+// rows in 1..16, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
+// weight_b_prepared / dst_b (optional): a second matrix of the same shape that shares X,
+// computed by the same launch (not together with dots).
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
                              const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
-                             int out_dim, const GemvTuning& tune);
+                             int out_dim, const GemvTuning& tune, float* dst_b = nullptr,
+                             const uint8_t* weight_b_prepared = nullptr);
 
 // Int8-MFMA GEMM on pre-quantized activations (natural order) and PREPARED
 // weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set.

@@ -148,6 +148,14 @@ class HipCompute:
                                                       C.byref(h)))
         return HipTensor(h.value)
 
+    def linearNoBiasPair(self, input: HipTensor, weight_a: HipTensor, weight_b: HipTensor, rows: int, in_dim: int,
+                         out_dim: int):
+        """ops/ops.zig:909, :1828-1849: (first, second) = (X @ Wa^T, X @ Wb^T)."""
+        ha, hb = C.c_void_p(), C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_no_bias_pair(self._h, input.handle, weight_a.handle, weight_b.handle, rows,
+                                                           in_dim, out_dim, C.byref(ha), C.byref(hb)))
+        return HipTensor(ha.value), HipTensor(hb.value)
+
     def linearNoBiasPlanned(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int,
                             operator_plan: "quant_matmul.OperatorPlan") -> HipTensor:
         req = _lib.PlannedRequest(input.handle, weight.handle, rows, in_dim, out_dim, operator_plan.to_c())

@@ -19,6 +19,14 @@ def launchLinearF32(stream, tensor_type, layout, dst: Buffer, input: Buffer, wei
                                              workspace, dispatch))
 
 
+def launchLinearPairF32(stream, tensor_type, layout, dst_a: Buffer, dst_b: Buffer, input: Buffer, weight_a: Buffer,
+                        weight_b: Buffer, rows, in_dim, out_dim, workspace: Buffer = NO_BUFFER,
+                        dispatch: int = -1) -> None:
+    """Two matmuls of one shape that share X (gate + up): X is quantized once."""
+    check(_lib.lib().afhip_launch_linear_pair_f32(stream, tensor_type, layout, dst_a, dst_b, input, weight_a, weight_b,
+                                                  rows, in_dim, out_dim, workspace, dispatch))
+
+
 def launchLinearQ8_0F32(stream, dst: Buffer, input: Buffer, weight_raw: Buffer, rows, in_dim, out_dim,
                         workspace: Buffer = NO_BUFFER) -> None:
     check(_lib.lib().afhip_launch_linear_q8_0_f32(stream, dst, input, weight_raw, rows, in_dim, out_dim, workspace))

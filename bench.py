@@ -145,25 +145,35 @@ def main() -> int:
         shapes = [("qkv", 6144, 4096), ("o", 4096, 4096), ("gate", 14336, 4096), ("up", 14336, 4096),
                   ("down", 4096, 14336)]
         launch = _lib.lib().afhip_launch_linear_f32
+        launch_pair = _lib.lib().afhip_launch_linear_pair_f32  # gate + up share X: the engine's linearNoBiasPair
         # one layer of synthetic weights, repacked into `layers` separate device buffers
         per_layer = []
         for li, (_, n, k) in enumerate(shapes):
             per_layer.append(prepared_copies(Q4, n, k, layers, 500 + li))
         weight_bytes = layers * sum(n * (k // 32) * 18 for _, n, k in shapes)
         out = {"what": "32 layers x (QKV 6144x4096, O 4096x4096, gate and up 14336x4096, down 4096x14336), Q4_0, "
-                       "one set of random weights repacked into 32 distinct device copies; matmuls only",
+                       "one set of random weights repacked into 32 distinct device copies; matmuls only, gate and up as "
+                       "one pair call (shared X)",
                "weight_bytes_per_token": weight_bytes}
         for m in (1, 5):
             xs = {k: torch.from_numpy(synth.activations(900 + k, m, k)).to(dev) for k in (4096, 14336)}
             ys = {n: torch.empty((m, n), dtype=torch.float32, device=dev) for n in (6144, 4096, 14336)}
+            y_up = torch.empty((m, 14336), dtype=torch.float32, device=dev)
             wsb = max(kernels.workspaceBytes(Q4, m, k, n) for _, n, k in shapes)
             scratch = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
 
             def token(st):
                 for layer in range(layers):
-                    for li, (_, n, k) in enumerate(shapes):
-                        rc = launch(st, Q4, _lib.LAYOUT_PREPARED, buf(ys[n]), buf(xs[k]), buf(per_layer[li][layer]), m, k, n,
-                                    buf(scratch), -1)
+                    for li, (name, n, k) in enumerate(shapes):
+                        if name == "up":
+                            continue  # computed with "gate"
+                        if name == "gate":
+                            rc = launch_pair(st, Q4, _lib.LAYOUT_PREPARED, buf(ys[n]), buf(y_up), buf(xs[k]),
+                                             buf(per_layer[li][layer]), buf(per_layer[li + 1][layer]), m, k, n,
+                                             buf(scratch), -1)
+                        else:
+                            rc = launch(st, Q4, _lib.LAYOUT_PREPARED, buf(ys[n]), buf(xs[k]), buf(per_layer[li][layer]), m,
+                                        k, n, buf(scratch), -1)
                         if rc != 0:
                             raise RuntimeError(f"launch failed: {rc}")
 

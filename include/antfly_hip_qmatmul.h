@@ -119,6 +119,15 @@ afhip_status afhip_launch_linear_f32(void *stream, int tensor_type, int layout, 
                                      afhip_buffer input, afhip_buffer weight, size_t rows,
                                      size_t in_dim, size_t out_dim, afhip_buffer workspace,
                                      int dispatch);
+/* Two matmuls of the same shape, format and layout that share X (what the engine's
+ * linearNoBiasPair computes for gate + up, ops/ops.zig:909, CPU op
+ * ops/native_compute.zig:6262-6307): Ya = X * Wa^T, Yb = X * Wb^T.  Each result is
+ * exactly what afhip_launch_linear_f32 gives for that matrix; X is quantized once,
+ * and up to 8 rows both matrices are served by one kernel launch. */
+afhip_status afhip_launch_linear_pair_f32(void *stream, int tensor_type, int layout, afhip_buffer dst_a,
+                                          afhip_buffer dst_b, afhip_buffer input, afhip_buffer weight_a,
+                                          afhip_buffer weight_b, size_t rows, size_t in_dim,
+                                          size_t out_dim, afhip_buffer workspace, int dispatch);
 /* Drop-ins with the reference launcher names: raw GGUF layout, automatic dispatch. */
 afhip_status afhip_launch_linear_q8_0_f32(void *stream, afhip_buffer dst, afhip_buffer input,
                                           afhip_buffer weight_raw, size_t rows, size_t in_dim,
@@ -214,6 +223,16 @@ size_t afhip_tensor_byte_len(const afhip_tensor *tensor);
 afhip_status afhip_compute_linear_no_bias(afhip_compute *self, const afhip_tensor *input,
                                           const afhip_tensor *weight, size_t rows, size_t in_dim,
                                           size_t out_dim, afhip_tensor **out);
+
+/* linearNoBiasPair, ops/ops.zig:909 (wrapper :1828-1849, CPU op
+ * ops/native_compute.zig:6262-6307): two no-bias linears that share the input and
+ * the shape; two new f32 tensors [rows, out_dim] owned by the caller.  Weights of
+ * different format or layout are served as two independent ops, as the engine's
+ * wrapper does; errors as for afhip_compute_linear_no_bias. */
+afhip_status afhip_compute_linear_no_bias_pair(afhip_compute *self, const afhip_tensor *input,
+                                               const afhip_tensor *weight_a, const afhip_tensor *weight_b,
+                                               size_t rows, size_t in_dim, size_t out_dim,
+                                               afhip_tensor **out_first, afhip_tensor **out_second);
 
 /* linearNoBiasPlanned, ops/ops.zig:895 (request struct :92-99).  The plan is
  * validated like validateQuantLinearPlan (ops/native_compute.zig:5039-5050):

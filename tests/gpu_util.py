@@ -44,6 +44,18 @@ def linear(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_di
     return y.cpu().numpy()
 
 
+def linear_pair(fmt, layout, x: np.ndarray, wa_dev: torch.Tensor, wb_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1):
+    xd = to_dev(x.astype(np.float32))
+    ya = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    yb = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    ws_bytes = kernels.workspaceBytes(fmt, rows, in_dim, out_dim)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=DEV)
+    kernels.launchLinearPairF32(stream(), fmt, layout, buf(ya), buf(yb), buf(xd), buf(wa_dev), buf(wb_dev), rows, in_dim,
+                                out_dim, buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return ya.cpu().numpy(), yb.cpu().numpy()
+
+
 def block_dots(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1) -> np.ndarray:
     xd = to_dev(x.astype(np.float32))
     d = torch.full((rows, out_dim, in_dim // 32), -(2 ** 31), dtype=torch.int32, device=DEV)

@@ -62,6 +62,32 @@ def test_linear_no_bias_matches_cpu_engine(cb, fmt, keep_raw):
     assert cb.debugStats()["pooled_buffers"] >= 2
 
 
+@pytest.mark.parametrize("rows", [1, 5, 24])
+def test_linear_no_bias_pair(cb, rows):
+    """linearNoBiasPair (ops/ops.zig:909): (X @ Wa^T, X @ Wb^T), both equal to the single op."""
+    in_dim, out_dim = 1024, 768
+    print(f"case: backend linearNoBiasPair rows={rows}", flush=True)
+    x = synth.activations(16, rows, in_dim)
+    wa, wb = synth.weights(Q4, 17, out_dim, in_dim), synth.weights(Q4, 18, out_dim, in_dim)
+    cb.insertWeightFromLoaded("gate", Q4, wa, [out_dim, in_dim])
+    cb.insertWeightFromLoaded("up", Q4, wb, [out_dim, in_dim])
+    cb.insertWeightFromLoaded("up_raw", Q4, wb, [out_dim, in_dim], keep_raw_layout=True)
+    xt = cb.fromFloat32(x, [rows, in_dim])
+    first, second = cb.linearNoBiasPair(xt, cb.getWeight("gate"), cb.getWeight("up"), rows, in_dim, out_dim)
+    assert first.shape == [rows, out_dim] and second.shape == [rows, out_dim]
+    ya, yb = cb.toFloat32(first), cb.toFloat32(second)
+    assert np.array_equal(ya, cb.toFloat32(cb.linearNoBias(xt, cb.getWeight("gate"), rows, in_dim, out_dim)))
+    assert np.array_equal(yb, cb.toFloat32(cb.linearNoBias(xt, cb.getWeight("up"), rows, in_dim, out_dim)))
+    ref = O.linear_no_bias(Q4, x, wb, rows, in_dim, out_dim, workers=8)
+    assert G.max_rel_err(yb.reshape(rows, out_dim), ref.astype(np.float64)) <= 2e-5
+    # different layouts: served as two independent ops, same results
+    f2, s2 = cb.linearNoBiasPair(xt, cb.getWeight("gate"), cb.getWeight("up_raw"), rows, in_dim, out_dim)
+    assert np.array_equal(cb.toFloat32(f2), ya)
+    assert G.max_rel_err(cb.toFloat32(s2).reshape(rows, out_dim), ref.astype(np.float64)) <= 2e-5
+    with pytest.raises(_lib.InvalidShape):
+        cb.linearNoBiasPair(xt, cb.getWeight("gate"), cb.getWeight("up"), rows, in_dim, out_dim + 1)
+
+
 def test_freed_buffers_are_reused(cb):
     x = synth.activations(1, 4, 256)
     a = cb.fromFloat32(x, [4, 256])

@@ -176,6 +176,33 @@ def test_forced_dispatch_kinds_agree(fmt, rows):
         assert G.max_rel_err(y, base.astype(np.float64)) <= TIGHT
 
 
+# ---- two matmuls that share X (linearNoBiasPair, ops/ops.zig:909) ----------------
+
+PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K slices, ragged columns, MFMA GEMM, f32 route
+    (1, 4096, 1024), (2, 512, 514), (4, 2048, 640), (5, 8224, 513), (8, 4096, 512), (12, 256, 530), (40, 512, 640),
+    (3, 64, 100),
+]
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+@pytest.mark.parametrize("layout", [RAW, PREP])
+@pytest.mark.parametrize("rows,in_dim,out_dim", PAIR_SHAPES)
+def test_pair_equals_two_single_ops(fmt, layout, rows, in_dim, out_dim):
+    """Each half of a pair is bit-identical to the single op on that matrix (and so to the
+    oracle within the single op's bound); the op is the engine's two-call fallback fused."""
+    print(f"case: pair fmt={fmt} layout={layout} rows={rows} in={in_dim} out={out_dim}", flush=True)
+    x = synth.activations(510 + rows, rows, in_dim)
+    wa = synth.weights(fmt, 511, out_dim, in_dim)
+    wb = synth.weights(fmt, 512, out_dim, in_dim)
+    da = G.prepare(fmt, wa, out_dim, in_dim) if layout == PREP else G.to_dev(wa)
+    db = G.prepare(fmt, wb, out_dim, in_dim) if layout == PREP else G.to_dev(wb)
+    ya, yb = G.linear_pair(fmt, layout, x, da, db, rows, in_dim, out_dim)
+    assert np.array_equal(ya, G.linear(fmt, layout, x, da, rows, in_dim, out_dim))
+    assert np.array_equal(yb, G.linear(fmt, layout, x, db, rows, in_dim, out_dim))
+    ref_b = O.linear_no_bias(fmt, x, wb, rows, in_dim, out_dim, workers=8)
+    assert G.max_rel_err(yb, ref_b.astype(np.float64)) <= TIGHT
+
+
 # ---- the benchmark configurations at full size ---------------------------------
 
 FULL = [
