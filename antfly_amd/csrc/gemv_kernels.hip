@@ -4,21 +4,23 @@
 //
 // The kernel is bound by HBM, and at these sizes (one call streams 18-33 MB in a
 // few microseconds) by how early the bytes are requested.  So it is "single
-// shot": a wavefront requests every weight byte it will ever use as its first
-// instructions, and only then does anything else.
+// shot": a wavefront requests every weight byte it will ever use before it
+// touches any of them.
 //
 //   * work unit: kCols consecutive output columns x one K-slice of 4096 values.
 //     A slice is kSteps wavefront-wide steps of 16 bytes per lane (Q4_0: lane =
 //     block, 2 steps; Q8_0: lane = half block, 4 steps), 1 KiB contiguous per
 //     load instruction.
 //   * a workgroup is kGroups x slices wavefronts; slices = ceil(in_dim / 4096).
-//   * prologue (after the weight requests are out): the workgroup quantizes
-//     X[rows, in_dim] into LDS -- the activation quantizer of
-//     ops/native_compute.zig:23799-23832, fused.  The first activation loads are
-//     issued before the weight loads so that they return first.
-//   * each lane accumulates (sx*sw)*f32(dot) for its blocks in f32; the
-//     wavefront reduces with DPP; K-slices are combined through LDS in slice
-//     order.  The summation order is fixed, so results are run-to-run identical.
+//   * prologue: the workgroup quantizes X[rows, in_dim] into LDS -- the activation
+//     quantizer of ops/native_compute.zig:23799-23832, fused.  Loads complete in
+//     order, so a wavefront that quantizes asks for X before its weights: the
+//     barrier after the prologue never waits for weight bytes.
+//   * each lane accumulates (sx*sw)*f32(dot) for its blocks in f32, consuming its
+//     weights in the order they were requested; the wavefront reduces with DPP;
+//     K-slices are combined through LDS in slice order.  The summation order is
+//     fixed, so results are run-to-run identical.
+//   * a launch may serve two matrices of the same shape that share X (GemvTargets).
 #include <hip/hip_runtime.h>
 
 #include "device_common.h"
@@ -47,7 +49,8 @@ constexpr int kSliceBlocks = 128;  // 4096 values
 // LDS image of the quantized activations.
 //   Q4_0: two planes per row so that a lane's two 16-byte reads are unit-stride
 //         across lanes: plane 0 holds values 0..15 of every block, plane 1 holds
-//         values 16..31 (matching low / high nibbles).
+//         values 16..31 (matching low / high nibbles) -- or, with kNibblePlanes,
+//         the high nibbles and the low nibbles of all 32 values (see below).
 //   Q8_0: natural order; lane (block, half) reads 16 bytes at 16*lane.
 // Quantizes one 32-value block held by one thread (8 float4) and stores it.
 // Same arithmetic as ops/native_compute.zig:23799-23832: f32 scale = max|x|/127,
