@@ -116,6 +116,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (1, 4096, 512), (2, 96, 515), (3, 2048, 640), (4, 4096, 1024), (5, 1120, 513),
     (6, 256, 600), (7, 160, 777), (8, 4096, 512), (9, 256, 512), (17, 512, 530),
     (33, 96, 513), (64, 1056, 640), (130, 256, 1030), (257, 512, 512),
+    (16, 14336, 512), (70, 8224, 520),  # long K on the MFMA kernel: many ring stages, a one-block last stage
 ]
 
 
