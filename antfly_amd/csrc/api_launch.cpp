@@ -43,13 +43,17 @@ static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
 // as X has at most this many 32-value blocks; beyond, a separate kernel quantizes X once.
 constexpr size_t kGemvFusedQuantBlocks = 512;
 
-// LDS the fused GEMV may use per workgroup; gfx950 has 160 KiB per CU.
+// LDS the GEMV may use per workgroup; gfx950 has 160 KiB per CU.  The larger figure is
+// for up to eight rows of a long K (8 x 14336): one workgroup per CU then, but the
+// weights are read once instead of once per slice of rows.
 constexpr size_t kGemvLdsBudget = 96 * 1024;
+constexpr size_t kGemvLdsBudgetFewRows = 152 * 1024;
 
-// Rows one GEMV launch takes: as many as fit the LDS budget (1-2 rows quantize
-// in the kernel's own prologue, more use separately quantized activations).
+// Rows one GEMV launch takes: as many as fit the LDS budget.
 constexpr int kGemvMaxRowsPerLaunch = 16;
 static int gemv_row_chunk(size_t rows, size_t in_dim) {
+    if (rows <= 8 && gemv_fused_lds_bytes(static_cast<int>(rows), static_cast<int>(in_dim)) <= kGemvLdsBudgetFewRows)
+        return static_cast<int>(rows);
     int chunk = rows < kGemvMaxRowsPerLaunch ? static_cast<int>(rows) : kGemvMaxRowsPerLaunch;
     while (chunk > 0 && gemv_fused_lds_bytes(chunk, static_cast<int>(in_dim)) > kGemvLdsBudget) --chunk;
     return chunk;

@@ -603,8 +603,8 @@ template <typename Kernel>
 hipError_t allow_large_lds(Kernel kernel, size_t lds, size_t* limit) {
     if (lds <= *limit) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       128 * 1024);
-    if (e == hipSuccess) *limit = 128 * 1024;
+                                       160 * 1024);
+    if (e == hipSuccess) *limit = 160 * 1024;
     return e;
 }
 

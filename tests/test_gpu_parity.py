@@ -117,6 +117,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (6, 256, 600), (7, 160, 777), (8, 4096, 512), (9, 256, 512), (17, 512, 530),
     (33, 96, 513), (64, 1056, 640), (130, 256, 1030), (257, 512, 512),
     (16, 14336, 512), (70, 8224, 520),  # long K on the MFMA kernel: many ring stages, a one-block last stage
+    (8, 14336, 516), (7, 9216, 512),    # small batch with a long K: one launch with more than 128 KB of LDS
 ]
 
 
