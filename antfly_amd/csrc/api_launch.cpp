@@ -39,8 +39,9 @@ static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
     return v;
 }
 
-// The GEMV quantizes X in its own prologue (every workgroup repeats that work) as long
-// as X has at most this many 32-value blocks; beyond, a separate kernel quantizes X once.
+// The GEMV quantizes X in its own prologue (every workgroup repeats that work) for one or
+// two rows of any length, and for three or four rows of Q4_0 up to this many 32-value
+// blocks of X; beyond, a separate kernel quantizes X once.
 constexpr size_t kGemvFusedQuantBlocks = 512;
 
 // LDS the GEMV may use per workgroup; gfx950 has 160 KiB per CU.  The larger figure is
@@ -169,10 +170,13 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     }
     if (fused_ok) {
         // mmv / small_batch (also when a plan forces them on more rows: 16-row slices).
-        // Small X (one to four rows of 4096 values): the GEMV quantizes it in its own
-        // prologue, one launch.  Larger X: every workgroup would repeat too much of that
-        // work, so X is quantized once by its own kernel into the caller's scratch.
-        const bool prequantize = rows > 2 && rows * kb > kGemvFusedQuantBlocks;
+        // Few rows: the GEMV quantizes X in its own prologue, one launch.  More: every
+        // workgroup would repeat too much of that work, so X is quantized once by its own
+        // kernel into the caller's scratch.  (AFHIP_GEMV_FUSED_ROWS caps the rows for tuning runs.)
+        static const int env_fused_rows = env_int("AFHIP_GEMV_FUSED_ROWS");
+        const size_t type_rows = tensor_type == AFHIP_TYPE_Q4_0 ? 4 : 2;
+        const size_t fused_rows = env_fused_rows >= 1 && env_fused_rows <= 4 ? size_t(env_fused_rows) : type_rows;
+        const bool prequantize = rows > fused_rows || (rows > 2 && rows * kb > kGemvFusedQuantBlocks);
         const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
         if (prequantize && (workspace.ptr == 0 || workspace.len < ws.bytes || workspace.ptr % 16 != 0))
             return AFHIP_ERR_INVALID_STATE;

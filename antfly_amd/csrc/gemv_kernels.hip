@@ -122,7 +122,7 @@ struct GemvTargets {
 
 constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
-// One or two rows of f32 activations, quantized in the prologue of every workgroup.
+// One to four rows of f32 activations, quantized in the prologue of every workgroup.
 template <int kType, int kRows, int kCols, bool kWriteDots>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices) {
@@ -177,30 +177,45 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         ok[j] = active && b < kb;
         blk[j] = b < kb ? b : kb - 1;  // lanes past the row end re-read its last block and contribute nothing
     }
+    // Request order = consumption order: column by column for one or two rows, K step by
+    // K step for more (the activations of a step are then in registers for all columns).
+    constexpr bool kStepMajor = kRows > 2;
     auto request_weights = [&]() {
 #pragma unroll
-        for (int c = 0; c < kCols; ++c) {
-            const int o = min(o0 + c, out_dim - 1);  // likewise for columns past the end
+        for (int u = 0; u < kCols * kSteps; ++u) {
+            const int c = kStepMajor ? u % kCols : u / kSteps;
+            const int j = kStepMajor ? u / kCols : u % kSteps;
+            const int o = min(o0 + c, out_dim - 1);  // columns past the end re-read the last one
             const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
             const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
-#pragma unroll
-            for (int j = 0; j < kSteps; ++j) {
-                wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
-                wd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
-            }
+            wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+            wd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
         }
     };
     if (wave * kWave < x_blocks) {  // wave-uniform
+        const int threads = static_cast<int>(blockDim.x);
         const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
-        float4 v[8];
+        const bool two = x_blocks > threads;                 // uniform: a second block per thread
+        const int xb1 = min(tid + threads, x_blocks - 1);
+        float4 v[8], v1[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
+        if (two) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v1[i] = reinterpret_cast<const float4*>(input)[xb1 * 8 + i];
+        }
         __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
         request_weights();
         __builtin_amdgcn_sched_barrier(0);
         const int r = xb / kb, b = xb - r * kb;
         quantize_block_to_lds<kType, true>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-        for (int xb2 = tid + static_cast<int>(blockDim.x); xb2 < x_blocks; xb2 += blockDim.x) {  // more blocks than threads
+        if (two) {
+            const int r1 = xb1 / kb, b1 = xb1 - r1 * kb;
+            quantize_block_to_lds<kType, true>(v1, b1, kb, qx + r1 * row_dwords, sx + r1 * kb, sumx + r1 * kb);
+        }
+        // more than two blocks per thread (not a shape the host sends here): these requests
+        // queue behind the weights
+        for (int xb2 = tid + 2 * threads; xb2 < x_blocks; xb2 += threads) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb2 * 8 + i];
             const int r2 = xb2 / kb, b2 = xb2 - r2 * kb;
@@ -211,94 +226,113 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     }
     __syncthreads();
 
-    // ---- 3. block dots and scaled accumulation
+    // ---- 3. block dots and scaled accumulation (the weights stay packed in registers)
+    static_assert(kRows <= 4, "the accumulators of all rows and columns live in registers");
+    constexpr int kWords = kType == 2 ? 8 : 4;
+    constexpr int kCells = kRows * kCols;
+    // one block of one column against one row's activations
+    auto block_dot = [&](const u32x4& w, const int (&a)[kWords], int sm) {
+        int dot;
+        if (kType == 2) {
+            // 4-bit dots on the packed nibbles, nothing is unpacked: a[0..3] = high
+            // nibbles of the activations (signed), a[4..7] = low nibbles (unsigned),
+            // sm = -8 * sum(low nibbles); see quantize_block_to_lds
+            int hi = dot8_i4(static_cast<int>(w.x ^ 0x88888888u), a[0], 0);
+            hi = dot8_i4(static_cast<int>(w.y ^ 0x88888888u), a[1], hi);
+            hi = dot8_i4(static_cast<int>(w.z ^ 0x88888888u), a[2], hi);
+            hi = dot8_i4(static_cast<int>(w.w ^ 0x88888888u), a[3], hi);
+            uint32_t lo = dot8_u4(w.x, static_cast<uint32_t>(a[4 % kWords]), static_cast<uint32_t>(sm));
+            lo = dot8_u4(w.y, static_cast<uint32_t>(a[5 % kWords]), lo);
+            lo = dot8_u4(w.z, static_cast<uint32_t>(a[6 % kWords]), lo);
+            lo = dot8_u4(w.w, static_cast<uint32_t>(a[7 % kWords]), lo);
+            dot = (hi << 4) + static_cast<int>(lo);
+        } else {
+            dot = dot4(static_cast<int>(w.x), a[0], 0);
+            dot = dot4(static_cast<int>(w.y), a[1], dot);
+            dot = dot4(static_cast<int>(w.z), a[2], dot);
+            dot = dot4(static_cast<int>(w.w), a[3], dot);
+            dot += dpp_move<kDppXor1>(dot);  // both lanes of the pair hold the block dot
+        }
+        return dot;
+    };
+    // this lane's activations of block blk[j], row r: words, scale, -8 * sum(low nibbles)
+    auto load_x = [&](int j, int r, int (&a)[kWords], float& s, int& sm) {
+        const int b = blk[j];
+        s = ok[j] ? sx[r * kb + b] : 0.0f;
+        sm = 0;
+        if (kType == 2) {
+            const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b];
+            const int4 a1 = reinterpret_cast<const int4*>(qx + r * row_dwords + (row_dwords >> 1))[b];
+            a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
+            a[4 % kWords] = a1.x; a[5 % kWords] = a1.y; a[6 % kWords] = a1.z; a[7 % kWords] = a1.w;
+            sm = sumx[r * kb + b];
+        } else {
+            const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b * 2 + half];
+            a[0] = a0.x; a[1] = a0.y; a[2] = a0.z; a[3] = a0.w;
+        }
+    };
     float acc[kRows][kCols];
 #pragma unroll
     for (int r = 0; r < kRows; ++r)
 #pragma unroll
         for (int c = 0; c < kCols; ++c) acc[r][c] = 0.0f;
-
-    // The activations of this lane's blocks go to registers once; the weights are then
-    // consumed column by column, in the order their loads were issued, so the arithmetic
-    // of a column runs while the later columns are still arriving.
-    float sxr[kSteps][kRows];
-    int ar[kSteps][kRows][kType == 2 ? 8 : 4];
-    int smr[kSteps][kRows];
+    auto accumulate = [&](int j, int c, int r, const int (&a)[kWords], float s, int sm) {
+        const int dot = block_dot(wq[j][c], a, sm);
+        if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim)
+            dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + blk[j]] = dot;
+        const float tscale = s * half_bits_to_f32(wd[j][c]);
+        const float term = tscale * static_cast<float>(dot);
+        acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
+    };
+    if (!kStepMajor) {
+        // one or two rows: all activations of this lane's blocks go to registers, then the
+        // weights are consumed column by column, in the order their loads were issued
+        float sxr[kSteps][kRows];
+        int ar[kSteps][kRows][kWords];
+        int smr[kSteps][kRows];
 #pragma unroll
-    for (int j = 0; j < kSteps; ++j) {
-        const int b = blk[j];
+        for (int j = 0; j < kSteps; ++j)
 #pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-            sxr[j][r] = ok[j] ? sx[r * kb + b] : 0.0f;
-            smr[j][r] = 0;
-            if (kType == 2) {
-                const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b];
-                const int4 a1 = reinterpret_cast<const int4*>(qx + r * row_dwords + (row_dwords >> 1))[b];
-                ar[j][r][0] = a0.x; ar[j][r][1] = a0.y; ar[j][r][2] = a0.z; ar[j][r][3] = a0.w;
-                ar[j][r][4] = a1.x; ar[j][r][5] = a1.y; ar[j][r][6] = a1.z; ar[j][r][7] = a1.w;
-                smr[j][r] = sumx[r * kb + b];
-            } else {
-                const int4 a0 = reinterpret_cast<const int4*>(qx + r * row_dwords)[b * 2 + half];
-                ar[j][r][0] = a0.x; ar[j][r][1] = a0.y; ar[j][r][2] = a0.z; ar[j][r][3] = a0.w;
-            }
-        }
-    }
+            for (int r = 0; r < kRows; ++r) load_x(j, r, ar[j][r], sxr[j][r], smr[j][r]);
 #pragma unroll
-    for (int c = 0; c < kCols; ++c) {
+        for (int c = 0; c < kCols; ++c)
+#pragma unroll
+            for (int j = 0; j < kSteps; ++j)
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) accumulate(j, c, r, ar[j][r], sxr[j][r], smr[j][r]);
+    } else {
+        // three or four rows: K step by K step (the order of the requests), the step's
+        // activations of all rows in registers for all columns
 #pragma unroll
         for (int j = 0; j < kSteps; ++j) {
-            const int b = blk[j];
-            const u32x4 w = wq[j][c];
-            const float dw = half_bits_to_f32(wd[j][c]);
+            float sxr[kRows];
+            int ar[kRows][kWords];
+            int smr[kRows];
 #pragma unroll
-            for (int r = 0; r < kRows; ++r) {
-                const int* a = ar[j][r];
-                int dot;
-                if (kType == 2) {
-                    // 4-bit dots on the packed nibbles, nothing is unpacked: a[0..3] = high
-                    // nibbles of the activations (signed), a[4..7] = low nibbles (unsigned),
-                    // smr = -8 * sum(low nibbles); see quantize_block_to_lds
-                    int hi = dot8_i4(static_cast<int>(w.x ^ 0x88888888u), a[0], 0);
-                    hi = dot8_i4(static_cast<int>(w.y ^ 0x88888888u), a[1], hi);
-                    hi = dot8_i4(static_cast<int>(w.z ^ 0x88888888u), a[2], hi);
-                    hi = dot8_i4(static_cast<int>(w.w ^ 0x88888888u), a[3], hi);
-                    uint32_t lo = dot8_u4(w.x, static_cast<uint32_t>(a[4]), static_cast<uint32_t>(smr[j][r]));
-                    lo = dot8_u4(w.y, static_cast<uint32_t>(a[5]), lo);
-                    lo = dot8_u4(w.z, static_cast<uint32_t>(a[6]), lo);
-                    lo = dot8_u4(w.w, static_cast<uint32_t>(a[7]), lo);
-                    dot = (hi << 4) + static_cast<int>(lo);
-                } else {
-                    dot = dot4(static_cast<int>(w.x), a[0], 0);
-                    dot = dot4(static_cast<int>(w.y), a[1], dot);
-                    dot = dot4(static_cast<int>(w.z), a[2], dot);
-                    dot = dot4(static_cast<int>(w.w), a[3], dot);
-                    dot += dpp_move<kDppXor1>(dot);  // both lanes of the pair hold the block dot
-                }
-                if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim)
-                    dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + b] = dot;
-                const float tscale = sxr[j][r] * dw;
-                const float term = tscale * static_cast<float>(dot);
-                acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
-            }
+            for (int r = 0; r < kRows; ++r) load_x(j, r, ar[r], sxr[r], smr[r]);
+#pragma unroll
+            for (int c = 0; c < kCols; ++c)
+#pragma unroll
+                for (int r = 0; r < kRows; ++r) accumulate(j, c, r, ar[r], sxr[r], smr[r]);
         }
     }
 
-    // ---- 4. wavefront reduction (all rows x columns at once), then K-slices in slice order
-    constexpr int kCells = kRows * kCols;
+    // ---- 4. wavefront reduction (all rows x columns at once)
     constexpr int kPadded = pow2_at_least(kCells);
-    static_assert(kCells <= 16, "at most 16 accumulators per lane");
+    static_assert(kCells <= 16, "at most 16 accumulators per lane and reduction");
     float red[kPadded];
 #pragma unroll
     for (int i = 0; i < kPadded; ++i) red[i] = i < kCells ? acc[i / kCols][i % kCols] : 0.0f;
     wave_sum_transposed<kPadded>(red, lane);
     const int cell = lane & (kPadded - 1);  // this lane holds the total of accumulator `cell`
-    const int cr = cell / kCols, cc = cell - cr * kCols;
+    const int cr = cell / kCols, cc = cell % kCols;
+    const bool mine = lane < kPadded && cell < kCells;
     if (slices == 1) {
-        if (active && lane < kPadded && cell < kCells && o0 + cc < out_dim && dst)
-            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
+        if (active && mine && o0 + cc < out_dim && dst) dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
         return;
     }
-    if (lane < kPadded && cell < kCells) partial[wave * kCells + cell] = red[0];
+    if (mine) partial[wave * kCells + cell] = red[0];
+    // K-slices are combined in slice order
     __syncthreads();
     const int cells = groups_per_wg * kCells;
     for (int i = tid; i < cells; i += blockDim.x) {
@@ -316,19 +350,14 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
 }
 
 // =====================================================================
-// Same work decomposition for 3 or more rows.  The wavefront keeps its weights
-// (unpacked once) in registers and walks the rows two at a time, so register use
-// does not grow with the row count; `rows` is a run-time value bounded only by LDS.
-// kFusedX: the workgroup quantizes the f32 `input` itself -- its first wavefronts
-// (half of them at most) do that, a block per thread and pass, and ask for their
-// weights afterwards, while the other wavefronts have their weight requests out from
-// the start.  Otherwise the activations were quantized beforehand by
-// quantize_activations_kernel (natural order: pre_q [rows][in_dim] int8, pre_scale /
-// pre_sum [rows][in_dim/32]) and are copied into LDS.
+// Same work decomposition for any number of rows whose activations were quantized
+// beforehand by quantize_activations_kernel (natural order: pre_q [rows][in_dim] int8,
+// pre_scale / pre_sum [rows][in_dim/32]); they are copied into LDS.  The wavefront keeps
+// its weights (unpacked once) in registers and walks the rows two at a time, so register
+// use does not grow with the row count; `rows` is a run-time value bounded only by LDS.
 // =====================================================================
-template <int kType, int kCols, bool kWriteDots, bool kFusedX>
+template <int kType, int kCols, bool kWriteDots>
 __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* __restrict__ dots,
-                                                            const float* __restrict__ input,
                                                             const int4* __restrict__ pre_q,
                                                             const float* __restrict__ pre_scale,
                                                             const int* __restrict__ pre_sum, int rows, int in_dim,
@@ -395,41 +424,8 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
             }
         };
 
-        if (kFusedX) {
-            // ---- 1a. Loads complete in order, so whoever quantizes X asks for X first and
-            // for its weights afterwards; the barrier below must not wait for weight bytes.
-            const int x_blocks = rows * kb;
-            const int q_waves = min(max(waves >> 1, 1), (x_blocks + kWave - 1) / kWave);
-            if (wave < q_waves) {
-                const int stride = q_waves * kWave;
-                auto load_block = [&](int xb, float4 (&v)[8]) {
-                    const int b = min(xb, x_blocks - 1);  // spare lanes repeat the last block
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[b * 8 + i];
-                };
-                auto quantize = [&](int xb, const float4 (&v)[8]) {
-                    const int b = min(xb, x_blocks - 1);
-                    const int r = b / kb, bb = b - r * kb;
-                    quantize_block_to_lds<kType>(v, bb, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-                };
-                // two blocks in flight per thread
-                float4 va[8], vb[8];
-                int xb = tid;
-                load_block(xb, va);
-                for (; xb < x_blocks; xb += 2 * stride) {
-                    if (xb + stride < x_blocks) load_block(xb + stride, vb);
-                    quantize(xb, va);
-                    if (xb + stride < x_blocks) {
-                        if (xb + 2 * stride < x_blocks) load_block(xb + 2 * stride, va);
-                        quantize(xb + stride, vb);
-                    }
-                }
-                request_weights();
-            } else {
-                request_weights();
-            }
-        } else {
-            // ---- 1b. requests for the quantized X (coalesced, 16 bytes = half a block per
+        {
+            // ---- 1. requests for the quantized X (coalesced, 16 bytes = half a block per
             // thread) go out before the weight requests: loads complete in order, and the copy
             // into LDS (and with it the barrier) must not wait for every weight byte of the
             // wavefront.  kXPre units per thread are requested up front (all of X for up to 8
@@ -616,7 +612,10 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     GemvTargets tg = tg0;
     tg.groups_each = (out_dim + kCols - 1) / kCols;
     const int groups = tg.groups_each * (tg.weight_b ? 2 : 1);
-    const int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact);
+    int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact);
+    // the prologue quantizes up to two blocks of X per thread ahead of the weight requests
+    const int x_blocks = kRows * (in_dim / 32);
+    if (x_blocks > 2 * waves * 64 && !tune.exact) waves = workgroup_waves(1024, 1024, slices, groups, true);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
     auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
@@ -627,8 +626,8 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     return hipGetLastError();
 }
 
-template <int kType, bool kDots, bool kFusedX>
-hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, const float* input, const GemvActivations& pre,
+template <int kType, bool kDots>
+hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, const GemvActivations& pre,
                        int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
@@ -638,11 +637,11 @@ hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, co
     const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);  // several of these workgroups share a unit: no balancing
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
-    auto kernel = gemv_rows_kernel<kType, kCols, kDots, kFusedX>;
+    auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input,
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots,
                        reinterpret_cast<const int4*>(pre.q), pre.scale, pre.sum, rows, in_dim, out_dim, slices);
     return hipGetLastError();
 }
@@ -651,19 +650,21 @@ template <int kType>
 hipError_t launch_gemv_type(hipStream_t stream, const GemvTargets& tg, int* dots, const float* input,
                             const GemvActivations& pre, int rows, int in_dim, int out_dim, const GemvTuning& tune) {
     if (pre.q != nullptr) {
-        return dots ? launch_rows<kType, true, false>(stream, tg, dots, nullptr, pre, rows, in_dim, out_dim, tune)
-                    : launch_rows<kType, false, false>(stream, tg, dots, nullptr, pre, rows, in_dim, out_dim, tune);
+        return dots ? launch_rows<kType, true>(stream, tg, dots, pre, rows, in_dim, out_dim, tune)
+                    : launch_rows<kType, false>(stream, tg, dots, pre, rows, in_dim, out_dim, tune);
     }
-    if (rows == 1) {
-        return dots ? launch_fused<kType, 1, true>(stream, tg, dots, input, in_dim, out_dim, tune)
-                    : launch_fused<kType, 1, false>(stream, tg, dots, input, in_dim, out_dim, tune);
+    switch (rows) {  // up to four rows: activations quantized in the kernel's own prologue
+#define AFHIP_FUSED_ROWS(R)                                                                          \
+    case R:                                                                                          \
+        return dots ? launch_fused<kType, R, true>(stream, tg, dots, input, in_dim, out_dim, tune)   \
+                    : launch_fused<kType, R, false>(stream, tg, dots, input, in_dim, out_dim, tune);
+        AFHIP_FUSED_ROWS(1)
+        AFHIP_FUSED_ROWS(2)
+        AFHIP_FUSED_ROWS(3)
+        AFHIP_FUSED_ROWS(4)
+#undef AFHIP_FUSED_ROWS
+        default: return hipErrorInvalidValue;  // more rows arrive quantized
     }
-    if (rows == 2) {
-        return dots ? launch_fused<kType, 2, true>(stream, tg, dots, input, in_dim, out_dim, tune)
-                    : launch_fused<kType, 2, false>(stream, tg, dots, input, in_dim, out_dim, tune);
-    }
-    return dots ? launch_rows<kType, true, true>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune)
-                : launch_rows<kType, false, true>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
 
 }  // namespace

@@ -54,9 +54,15 @@ def test_linear_no_bias_matches_cpu_engine(cb, fmt, keep_raw):
     stats = cb.debugStats()
     assert stats["launches_small_batch"] == 2 and stats["resident_weight_bytes"] >= w.size
     assert stats["launches_prepare"] == (0 if keep_raw else 1)
-    # a small X on repacked weights: the GEMV quantizes it in its own prologue; the
-    # generic kernels (raw GGUF layout) read activations quantized by a separate kernel
-    assert stats["launches_activation_quant"] == (2 if keep_raw else 0)
+    # five rows: a separate kernel quantizes the activations, once per op
+    assert stats["launches_activation_quant"] == 2
+    # two rows on repacked weights: the GEMV quantizes them in its own prologue; the
+    # generic kernels (raw GGUF layout) always read activations quantized beforehand
+    x2t = cb.fromFloat32(x[:2], [2, in_dim])
+    y2 = cb.toFloat32(cb.linearNoBias(x2t, wt, 2, in_dim, out_dim)).reshape(2, out_dim)
+    ref2 = O.linear_no_bias(fmt, x[:2], w, 2, in_dim, out_dim, workers=8)
+    assert G.max_rel_err(y2, ref2.astype(np.float64)) <= 2e-5
+    assert cb.debugStats()["launches_activation_quant"] == (3 if keep_raw else 2)
     for t in (yt, yt2, xt):
         cb.freeTensor(t)
     assert cb.debugStats()["pooled_buffers"] >= 2
