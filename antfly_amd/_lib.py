@@ -87,6 +87,10 @@ SIGNATURES = {
     "afhip_launch_prepare_weight": (_st, [_vp, _i, Buffer, Buffer, _sz, _sz]),
     "afhip_launch_quantize_activations": (_st, [_vp, Buffer, _sz, _sz, Buffer, Buffer, Buffer]),
     "afhip_launch_block_dots": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_argmax_workspace_bytes": (_sz, [_sz]),
+    "afhip_launch_argmax_last_row_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, Buffer]),
+    "afhip_linear_argmax_workspace_bytes": (_sz, [_i, _sz, _sz]),
+    "afhip_launch_linear_argmax_last_row_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),
@@ -113,6 +117,10 @@ SIGNATURES = {
     "afhip_tensor_byte_len": (_sz, [_vp]),
     "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_pair": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
+    "afhip_compute_linear_no_bias_grouped": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32), _sz, C.POINTER(_vp)]),
+    "afhip_compute_argmax_last_row": (_st, [_vp, _vp, _sz, _sz, C.POINTER(C.c_uint32)]),
+    "afhip_compute_linear_no_bias_argmax_last_row": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32)]),
+    "afhip_compute_linear_no_bias_argmax_last_row_tensor": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_planned": (_st, [_vp, C.POINTER(PlannedRequest), C.POINTER(_vp)]),
     "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
     "afhip_smoke_q8_0": (_st, []),

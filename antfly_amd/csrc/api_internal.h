@@ -24,4 +24,14 @@ afhip_status linear_impl(void* stream, int tensor_type, int layout, afhip_buffer
                          int dispatch, afhip_buffer dots, LaunchCounters* counters,
                          afhip_buffer dst_b = afhip_buffer{0, 0}, afhip_buffer weight_b = afhip_buffer{0, 0});
 
+// argmax over the last row of f32 [rows, dim]; `workspace` (optional) lets several workgroups scan a long row.
+afhip_status argmax_last_row_impl(void* stream, afhip_buffer token_u32, afhip_buffer token_f32, afhip_buffer input,
+                                  size_t rows, size_t dim, afhip_buffer workspace);
+
+// argmax(X[rows-1] * W^T): one GEMV over the last row whose workgroups keep the best of their
+// columns (repacked weights), or logits into `workspace` and the argmax kernels.
+afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip_buffer token_u32,
+                                afhip_buffer token_f32, afhip_buffer input, afhip_buffer weight, size_t rows,
+                                size_t in_dim, size_t out_dim, afhip_buffer workspace, LaunchCounters* counters);
+
 }  // namespace afhip

@@ -230,6 +230,89 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+static size_t argmax_logits_bytes(size_t out_dim) { return (out_dim * 4 + 255) / 256 * 256; }
+static size_t argmax_keys_bytes(size_t dim) {
+    if (dim > 0x7fffffff) return 0;
+    const int groups = argmax_row_workgroups(static_cast<int>(dim));
+    return groups > 1 ? (static_cast<size_t>(groups) * 8 + 255) / 256 * 256 : 0;
+}
+
+afhip_status argmax_last_row_impl(void* stream, afhip_buffer token_u32, afhip_buffer token_f32, afhip_buffer input,
+                                  size_t rows, size_t dim, afhip_buffer workspace) {
+    if (rows == 0 || dim == 0) return AFHIP_ERR_INVALID_SHAPE;  // error.InvalidTensorShape, native_compute.zig:37903
+    size_t count, bytes;
+    if (!checked_mul(rows, dim, &count) || !checked_mul(count, 4, &bytes)) return AFHIP_ERR_INVALID_SHAPE;
+    if (bytes > input.len) return AFHIP_ERR_INVALID_SHAPE;
+    if (dim > 0x7fffffff || input.ptr == 0 || input.ptr % 4 != 0) return AFHIP_ERR_INVALID_STATE;
+    if (token_u32.ptr == 0 && token_f32.ptr == 0) return AFHIP_ERR_INVALID_STATE;
+    if ((token_u32.ptr != 0 && (token_u32.len < 4 || token_u32.ptr % 4 != 0)) ||
+        (token_f32.ptr != 0 && (token_f32.len < 4 || token_f32.ptr % 4 != 0)))
+        return AFHIP_ERR_INVALID_STATE;
+    // a long row is scanned by several workgroups when the caller lends room for their keys
+    unsigned long long* keys = nullptr;
+    if (workspace.ptr != 0 && workspace.ptr % 8 == 0 && argmax_keys_bytes(dim) != 0 && workspace.len >= argmax_keys_bytes(dim))
+        keys = reinterpret_cast<unsigned long long*>(workspace.ptr);
+    hipError_t e = launch_argmax_row(static_cast<hipStream_t>(stream),
+                                     reinterpret_cast<const float*>(input.ptr) + (rows - 1) * dim, static_cast<int>(dim),
+                                     keys, reinterpret_cast<uint32_t*>(token_u32.ptr),
+                                     reinterpret_cast<float*>(token_f32.ptr));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+// Workspace: [keys or logits: out_dim f32, padded to 256][scratch of a one-row linear][keys of the argmax over logits]
+afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip_buffer token_u32,
+                                afhip_buffer token_f32, afhip_buffer input, afhip_buffer weight, size_t rows,
+                                size_t in_dim, size_t out_dim, afhip_buffer workspace, LaunchCounters* counters) {
+    const size_t bb = block_bytes(tensor_type);
+    if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (rows == 0 || in_dim == 0 || out_dim == 0) return AFHIP_ERR_INVALID_SHAPE;
+    if (in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    size_t count, bytes, w_blocks, w_bytes;
+    if (!checked_mul(rows, in_dim, &count) || !checked_mul(count, 4, &bytes) || bytes > input.len)
+        return AFHIP_ERR_INVALID_STATE;
+    if (!checked_mul(out_dim, in_dim / 32, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes) || w_bytes > weight.len)
+        return AFHIP_ERR_INVALID_STATE;
+    if (in_dim > 0x7fffffff || out_dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || weight.ptr == 0)
+        return AFHIP_ERR_INVALID_STATE;
+    if ((token_u32.ptr == 0 && token_f32.ptr == 0) ||
+        (token_u32.ptr != 0 && (token_u32.len < 4 || token_u32.ptr % 4 != 0)) ||
+        (token_f32.ptr != 0 && (token_f32.len < 4 || token_f32.ptr % 4 != 0)))
+        return AFHIP_ERR_INVALID_STATE;
+    const size_t logits_bytes = argmax_logits_bytes(out_dim);
+    if (workspace.ptr == 0 || workspace.ptr % 256 != 0 ||
+        workspace.len < afhip_linear_argmax_workspace_bytes(tensor_type, in_dim, out_dim))
+        return AFHIP_ERR_INVALID_STATE;
+    // only the last row's logits matter: one GEMV whatever `rows` is
+    const afhip_buffer last_row{input.ptr + (rows - 1) * in_dim * 4, in_dim * 4};
+
+    if (layout == AFHIP_LAYOUT_PREPARED && weight.ptr % 16 == 0 && afhip_uses_activation_quant(1, in_dim, out_dim) &&
+        in_dim <= static_cast<size_t>(gemv_fused_max_in_dim()) && gemv_row_chunk(1, in_dim) > 0) {
+        // the GEMV's workgroups keep the best of their own columns; no logits are written
+        unsigned long long* keys = reinterpret_cast<unsigned long long*>(workspace.ptr);  // at most (out_dim + 1) / 2 of them
+        int key_count = 0;
+        if (counters) counters->mmv++;
+        hipError_t e = launch_gemv_argmax_keys(static_cast<hipStream_t>(stream), tensor_type, keys, &key_count,
+                                               reinterpret_cast<const float*>(last_row.ptr),
+                                               reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(in_dim),
+                                               static_cast<int>(out_dim), gemv_tuning(tensor_type, 1, in_dim, out_dim));
+        if (e == hipSuccess)
+            e = launch_argmax_keys(static_cast<hipStream_t>(stream), keys, key_count,
+                                   reinterpret_cast<uint32_t*>(token_u32.ptr), reinterpret_cast<float*>(token_f32.ptr));
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
+
+    const afhip_buffer logits{workspace.ptr, out_dim * 4};
+    const size_t linear_bytes = workspace_view(0, 1, in_dim).bytes;
+    const afhip_buffer linear_ws{workspace.ptr + logits_bytes, linear_bytes};
+    const size_t keys_offset = logits_bytes + (linear_bytes + 255) / 256 * 256;
+    const afhip_buffer keys_ws{workspace.ptr + keys_offset, workspace.len - keys_offset};
+    afhip_status s = linear_impl(stream, tensor_type, layout, logits, last_row, weight, 1, in_dim, out_dim, linear_ws,
+                                 -1, afhip_buffer{0, 0}, counters);
+    if (s != AFHIP_OK) return s;
+    return argmax_last_row_impl(stream, token_u32, token_f32, logits, 1, out_dim, keys_ws);
+}
+
 }  // namespace afhip
 
 using namespace afhip;
@@ -415,6 +498,28 @@ afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buff
     hipError_t e = launch_decode_fp16(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr),
                                       reinterpret_cast<const uint16_t*>(src.ptr), n);
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+// ---- lm_head: argmax over the last row
+
+size_t afhip_argmax_workspace_bytes(size_t dim) { return argmax_keys_bytes(dim); }
+
+afhip_status afhip_launch_argmax_last_row_f32(void* stream, afhip_buffer token_u32, afhip_buffer token_f32,
+                                              afhip_buffer input, size_t rows, size_t dim, afhip_buffer workspace) {
+    return argmax_last_row_impl(stream, token_u32, token_f32, input, rows, dim, workspace);
+}
+
+size_t afhip_linear_argmax_workspace_bytes(int tensor_type, size_t in_dim, size_t out_dim) {
+    if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || in_dim == 0 || out_dim == 0) return 0;
+    return argmax_logits_bytes(out_dim) + (workspace_view(0, 1, in_dim).bytes + 255) / 256 * 256 + argmax_keys_bytes(out_dim);
+}
+
+afhip_status afhip_launch_linear_argmax_last_row_f32(void* stream, int tensor_type, int layout, afhip_buffer token_u32,
+                                                     afhip_buffer token_f32, afhip_buffer input, afhip_buffer weight,
+                                                     size_t rows, size_t in_dim, size_t out_dim,
+                                                     afhip_buffer workspace) {
+    return linear_argmax_impl(stream, tensor_type, layout, token_u32, token_f32, input, weight, rows, in_dim, out_dim,
+                              workspace, nullptr);
 }
 
 }  // extern "C"

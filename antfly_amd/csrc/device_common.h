@@ -116,6 +116,60 @@ __device__ __forceinline__ void wave_sum_transposed(float* v, int lane) {
     v[0] = t;
 }
 
+// ---- argmax keys (backends/activations.zig:350-357: the largest value, the lowest
+// index among equal values, -0 equals +0, NaNs never win).  key = (value mapped to an
+// unsigned that orders like the float) : (~index); larger key wins; 0 = no candidate.
+__device__ __forceinline__ unsigned long long argmax_key(float v, uint32_t index) {
+    uint32_t bits = __builtin_bit_cast(uint32_t, v);
+    if ((bits << 1) == 0) bits = 0;  // -0 -> +0
+    const uint32_t ordered = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+    const unsigned long long k = (static_cast<unsigned long long>(ordered) << 32) | (0xFFFFFFFFu - index);
+    return v == v ? k : 0ull;
+}
+
+__device__ __forceinline__ uint32_t argmax_key_index(unsigned long long key) {
+    return key == 0 ? 0u : 0xFFFFFFFFu - static_cast<uint32_t>(key & 0xFFFFFFFFu);
+}
+
+template <int kCtrl>
+__device__ __forceinline__ unsigned long long max_key_step(unsigned long long key) {
+    const unsigned long long other =
+        (static_cast<unsigned long long>(static_cast<uint32_t>(dpp_move<kCtrl>(static_cast<int>(key >> 32)))) << 32) |
+        static_cast<uint32_t>(dpp_move<kCtrl>(static_cast<int>(key & 0xFFFFFFFFu)));
+    return other > key ? other : key;
+}
+
+// Largest key of each 16-lane row, in all of its lanes (register exchanges only).
+__device__ __forceinline__ unsigned long long row_max_key(unsigned long long key) {
+    key = max_key_step<kDppXor1>(key);
+    key = max_key_step<kDppXor2>(key);
+    key = max_key_step<kDppHalfMirror>(key);
+    return max_key_step<kDppRowMirror>(key);
+}
+
+// Largest key of the workgroup (at most 16 wavefronts), valid on thread 0.  `slots` = one
+// LDS word per wavefront.  kLiveLanes: only lanes [0, kLiveLanes) of a wavefront hold
+// candidates (at most 16: one row).
+template <int kLiveLanes = 64>
+__device__ __forceinline__ unsigned long long workgroup_max_key(unsigned long long key, unsigned long long* slots) {
+    key = row_max_key(key);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    if (kLiveLanes > 16) {  // the four rows of the wavefront
+        const unsigned long long r1 = __shfl(key, 16), r2 = __shfl(key, 32), r3 = __shfl(key, 48);
+        key = key > r1 ? key : r1;
+        key = key > r2 ? key : r2;
+        key = key > r3 ? key : r3;
+    }
+    if (lane == 0) slots[tid >> 6] = key;
+    __syncthreads();
+    if (tid < 16) {  // one row of the first wavefront: a slot per lane
+        key = tid < static_cast<int>(blockDim.x >> 6) ? slots[tid] : 0ull;
+        key = row_max_key(key);
+    }
+    return key;
+}
+
 // ---- activation quantizer for one value, given its block's max |x|
 // (ops/native_compute.zig:11998-12028): f32 scale, one reciprocal, round half
 // away from zero, clamp to +-127.

@@ -123,9 +123,13 @@ struct GemvTargets {
 constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
 // One to four rows of f32 activations, quantized in the prologue of every workgroup.
-template <int kType, int kRows, int kCols, bool kWriteDots>
+// kArgmax (one row, one matrix): no Y is written; the workgroup leaves the argmax key of
+// its output columns in keys[blockIdx.x] instead.
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
-    GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices) {
+    GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices,
+    unsigned long long* __restrict__ keys = nullptr) {
+    static_assert(!kArgmax || (kRows == 1 && !kWriteDots), "argmax keys: one row, no block dots");
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
     constexpr int kBlocksPerStep = kWave / kLpb;
@@ -328,6 +332,14 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const int cr = cell / kCols, cc = cell % kCols;
     const bool mine = lane < kPadded && cell < kCells;
     if (slices == 1) {
+        if (kArgmax) {
+            // (`partial` is free here: one word per wavefront)
+            const bool live = active && mine && o0 + cc < out_dim;
+            const unsigned long long key = workgroup_max_key<kPadded>(
+                live ? argmax_key(red[0], static_cast<uint32_t>(o0 + cc)) : 0ull, reinterpret_cast<unsigned long long*>(partial));
+            if (tid == 0) keys[blockIdx.x] = key;
+            return;
+        }
         if (active && mine && o0 + cc < out_dim && dst) dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
         return;
     }
@@ -335,6 +347,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     // K-slices are combined in slice order
     __syncthreads();
     const int cells = groups_per_wg * kCells;
+    unsigned long long key = 0;
     for (int i = tid; i < cells; i += blockDim.x) {
         const int gi = i / kCells, rc = i - gi * kCells;
         const int r = rc / kCols, c = rc - r * kCols;
@@ -345,7 +358,19 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         const int o = g * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
-        if (g < tg.groups_each && o < out_dim && d) d[static_cast<size_t>(r) * out_dim + o] = total;
+        if (kArgmax) {
+            if (g < tg.groups_each && o < out_dim) {
+                const unsigned long long k = argmax_key(total, static_cast<uint32_t>(o));
+                if (k > key) key = k;
+            }
+        } else if (g < tg.groups_each && o < out_dim && d) {
+            d[static_cast<size_t>(r) * out_dim + o] = total;
+        }
+    }
+    if (kArgmax) {
+        __syncthreads();  // every total has been read: the partial sums' memory becomes the key slots
+        key = workgroup_max_key(key, reinterpret_cast<unsigned long long*>(partial));
+        if (tid == 0) keys[blockIdx.x] = key;
     }
 }
 
@@ -604,9 +629,9 @@ hipError_t allow_large_lds(Kernel kernel, size_t lds, size_t* limit) {
     return e;
 }
 
-template <int kType, int kRows, bool kDots>
+template <int kType, int kRows, bool kDots, bool kArgmax = false>
 hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, const float* input, int in_dim,
-                        int out_dim, const GemvTuning& tune) {
+                        int out_dim, const GemvTuning& tune, unsigned long long* keys = nullptr, int* key_count = nullptr) {
     constexpr int kCols = kType == 2 ? 4 : 2;
     const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
     GemvTargets tg = tg0;
@@ -616,13 +641,19 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     // the prologue quantizes up to two blocks of X per thread ahead of the weight requests
     const int x_blocks = kRows * (in_dim / 32);
     if (x_blocks > 2 * waves * 64 && !tune.exact) waves = workgroup_waves(1024, 1024, slices, groups, true);
+    // A matrix that takes several rounds of workgroups (a vocabulary): half-size workgroups,
+    // two to a compute unit, so that one streams weights while the other is in its prologue.
+    if (!tune.exact && waves > 8 && slices <= 8 && x_blocks <= 512 &&
+        (groups + waves / slices - 1) / (waves / slices) > compute_units() * 3 / 2)
+        waves = workgroup_waves(512, 512, slices, groups, true);  // many rounds: nothing to balance
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
-    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots>;
+    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax>;
     static size_t lds_limit = 64 * 1024;
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices);
+    if (key_count) *key_count = grid;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices, keys);
     return hipGetLastError();
 }
 
@@ -686,6 +717,16 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
     const GemvTargets tg{dst, dst_b, weight_prepared, weight_b_prepared, 0};
     if (tensor_type == 2) return launch_gemv_type<2>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
     return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
+}
+
+hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned long long* keys, int* key_count,
+                                   const float* input, const uint8_t* weight_prepared, int in_dim, int out_dim,
+                                   const GemvTuning& tune) {
+    if (in_dim > gemv_fused_max_in_dim() || keys == nullptr || key_count == nullptr) return hipErrorInvalidValue;
+    const GemvTargets tg{nullptr, nullptr, weight_prepared, nullptr, 0};
+    if (tensor_type == 2)
+        return launch_fused<2, 1, false, true>(stream, tg, nullptr, input, in_dim, out_dim, tune, keys, key_count);
+    return launch_fused<8, 1, false, true>(stream, tg, nullptr, input, in_dim, out_dim, tune, keys, key_count);
 }
 
 }  // namespace afhip

@@ -499,6 +499,109 @@ afhip_status afhip_compute_linear_no_bias_pair(afhip_compute* self, const afhip_
     return linear_no_bias_impl(self, input, weight_a, rows, in_dim, out_dim, -1, out_first, weight_b, out_second);
 }
 
+afhip_status afhip_compute_linear_no_bias_grouped(afhip_compute* self, const afhip_tensor* input,
+                                                  const afhip_tensor* weight, size_t rows, size_t in_dim, size_t out_dim,
+                                                  const uint32_t* projection_out_dims, size_t num_projections,
+                                                  afhip_tensor** out) {
+    if (!out) return AFHIP_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (num_projections == 0 || !projection_out_dims) return AFHIP_ERR_INVALID_SHAPE;
+    size_t total = 0;
+    for (size_t i = 0; i < num_projections; ++i) {
+        if (projection_out_dims[i] == 0) return AFHIP_ERR_INVALID_SHAPE;
+        total += projection_out_dims[i];
+    }
+    if (total != out_dim) return AFHIP_ERR_INVALID_SHAPE;
+    // the projections are rows [o0, o1) of one concatenated matrix: one linear serves them all
+    return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out);
+}
+
+afhip_status afhip_compute_argmax_last_row(afhip_compute* self, const afhip_tensor* tensor, size_t rows, size_t dim,
+                                           uint32_t* token) {
+    if (!self || !tensor || !token) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (!is_f32(tensor)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    size_t count;
+    if (rows == 0 || dim == 0 || !checked_mul(rows, dim, &count) || tensor->elem_count != count)
+        return AFHIP_ERR_INVALID_SHAPE;
+    afhip_status s = make_current(self);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer id;
+    s = alloc_device_buffer(self, 4, &id);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer scratch{0, 0};
+    s = acquire_scratch(self, afhip_argmax_workspace_bytes(dim), &scratch);
+    if (s == AFHIP_OK)
+        s = afhip_launch_argmax_last_row_f32(self->stream, id, afhip_buffer{0, 0}, tensor->buffer, rows, dim, scratch);
+    if (s == AFHIP_OK) s = copy_to_host(self, token, id, 4);
+    if (s == AFHIP_OK) s = from_hip(hipStreamSynchronize(self->stream));
+    release_device_buffer(self, &id);
+    return s;
+}
+
+namespace {
+
+// token_host: the id is copied back and the stream synchronized; token_tensor: a new f32 [1] tensor.
+afhip_status linear_argmax(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight, size_t rows,
+                           size_t in_dim, size_t out_dim, uint32_t* token_host, afhip_tensor** token_tensor) {
+    if (!self || !input || !weight) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (!is_f32(input)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    size_t in_count, w_count;
+    if (rows == 0 || in_dim == 0 || out_dim == 0 || !checked_mul(rows, in_dim, &in_count) ||
+        !checked_mul(out_dim, in_dim, &w_count) || input->elem_count != in_count || weight->elem_count != w_count)
+        return AFHIP_ERR_INVALID_SHAPE;
+    if (weight->quant_type < 0) return is_f32(weight) ? AFHIP_ERR_OP_UNSUPPORTED : AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    afhip_status s = make_current(self);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer id;  // [f32 id][u32 id]
+    s = alloc_device_buffer(self, 8, &id);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer scratch{0, 0};
+    s = acquire_scratch(self, afhip_linear_argmax_workspace_bytes(weight->quant_type, in_dim, out_dim), &scratch);
+    const afhip_buffer id_f32{id.ptr, 4};
+    const afhip_buffer id_u32{id.ptr + 4, 4};
+    if (s == AFHIP_OK)
+        s = linear_argmax_impl(self->stream, weight->quant_type, weight->layout, id_u32, id_f32, input->buffer,
+                               weight->buffer, rows, in_dim, out_dim, scratch, &self->counters);
+    if (s == AFHIP_OK && token_host) {
+        s = copy_to_host(self, token_host, id_u32, 4);
+        if (s == AFHIP_OK) s = from_hip(hipStreamSynchronize(self->stream));
+    }
+    if (s != AFHIP_OK || !token_tensor) {
+        release_device_buffer(self, &id);
+        return s;
+    }
+    // the f32 copy of the id (first word) is the tensor's one element; the buffer goes with the tensor
+    afhip_tensor* t = new (std::nothrow) afhip_tensor();
+    if (!t) {
+        release_device_buffer(self, &id);
+        return AFHIP_ERR_OUT_OF_MEMORY;
+    }
+    t->buffer = id;
+    t->dtype = AFHIP_DTYPE_F32;
+    t->shape = {1};
+    t->elem_count = 1;
+    *token_tensor = t;
+    return AFHIP_OK;
+}
+
+}  // namespace
+
+afhip_status afhip_compute_linear_no_bias_argmax_last_row(afhip_compute* self, const afhip_tensor* input,
+                                                          const afhip_tensor* weight, size_t rows, size_t in_dim,
+                                                          size_t out_dim, uint32_t* token) {
+    if (!token) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_argmax(self, input, weight, rows, in_dim, out_dim, token, nullptr);
+}
+
+afhip_status afhip_compute_linear_no_bias_argmax_last_row_tensor(afhip_compute* self, const afhip_tensor* input,
+                                                                 const afhip_tensor* weight, size_t rows, size_t in_dim,
+                                                                 size_t out_dim, afhip_tensor** out) {
+    if (!out) return AFHIP_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    return linear_argmax(self, input, weight, rows, in_dim, out_dim, nullptr, out);
+}
+
 afhip_status afhip_compute_linear_no_bias_planned(afhip_compute* self,
                                                   const afhip_linear_no_bias_planned_request* request,
                                                   afhip_tensor** out) {

@@ -137,6 +137,86 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4* __
 // Launchers
 // =====================================================================
 
+// argmax of one f32 row (backends/activations.zig:350-357).  Workgroup g scans
+// row[g*chunk, (g+1)*chunk) with eight 16-byte loads in flight per thread.  With
+// `keys` it leaves its best key there (argmax_keys_kernel finishes); without (one
+// workgroup) it writes the token itself, as u32 and / or as f32 (the engine's token
+// tensors are f32, architectures/gpt.zig:859-868).
+__global__ __launch_bounds__(1024) void argmax_row_kernel(const float* __restrict__ row_all, int dim_all, int chunk,
+                                                           unsigned long long* __restrict__ keys,
+                                                           uint32_t* __restrict__ token_u32,
+                                                           float* __restrict__ token_f32) {
+    constexpr int kInFlight = 8;
+    __shared__ unsigned long long slots[16];
+    const int tid = threadIdx.x, threads = blockDim.x;
+    const int first = blockIdx.x * chunk;
+    const float* row = row_all + first;
+    const int dim = min(chunk, dim_all - first);
+    unsigned long long key = 0;
+    auto take = [&](float v, int i) {
+        const unsigned long long k = argmax_key(v, static_cast<uint32_t>(first + i));
+        if (k > key) key = k;
+    };
+    // the row starts anywhere (last row of a [rows, dim] tensor): scalar head up to 16-byte alignment
+    const int head = min(dim, static_cast<int>(((16 - (reinterpret_cast<uintptr_t>(row) & 15)) & 15) >> 2));
+    if (tid < head) take(row[tid], tid);
+    const float4* row4 = reinterpret_cast<const float4*>(row + head);
+    const int n4 = (dim - head) >> 2;
+    for (int base = 0; base < n4; base += threads * kInFlight) {
+        float4 v[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) v[u] = row4[min(base + u * threads + tid, n4 - 1)];  // past the end: re-read the last one
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            const int i4 = base + u * threads + tid;
+            if (i4 < n4) {
+                const int i = head + 4 * i4;
+                take(v[u].x, i);
+                take(v[u].y, i + 1);
+                take(v[u].z, i + 2);
+                take(v[u].w, i + 3);
+            }
+        }
+    }
+    const int tail = head + 4 * n4 + tid;
+    if (tail < dim) take(row[tail], tail);
+
+    key = workgroup_max_key(key, slots);
+    if (tid == 0) {
+        if (keys) {
+            keys[blockIdx.x] = key;
+        } else {
+            const uint32_t token = argmax_key_index(key);
+            if (token_u32) *token_u32 = token;
+            if (token_f32) *token_f32 = static_cast<float>(token);
+        }
+    }
+}
+
+// Best of n keys (one per workgroup of argmax_row_kernel or of the GEMV) -> token.
+__global__ __launch_bounds__(1024) void argmax_keys_kernel(const unsigned long long* __restrict__ keys, int n,
+                                                            uint32_t* __restrict__ token_u32,
+                                                            float* __restrict__ token_f32) {
+    constexpr int kInFlight = 8;
+    __shared__ unsigned long long slots[16];
+    const int tid = threadIdx.x, threads = blockDim.x;
+    unsigned long long key = 0;
+    for (int base = 0; base < n; base += threads * kInFlight) {
+        unsigned long long k[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) k[u] = keys[min(base + u * threads + tid, n - 1)];  // past the end: the last one again
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u)
+            if (k[u] > key) key = k[u];
+    }
+    key = workgroup_max_key(key, slots);
+    if (tid == 0) {
+        const uint32_t token = argmax_key_index(key);
+        if (token_u32) *token_u32 = token;
+        if (token_f32) *token_f32 = static_cast<float>(token);
+    }
+}
+
 namespace {
 
 hipError_t launch_status() { return hipGetLastError(); }
@@ -213,6 +293,31 @@ hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* 
     if (n16 == 0) return hipSuccess;
     hipLaunchKernelGGL(stream_read_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0, stream,
                        reinterpret_cast<const stream_u32x4*>(src), sink, n16);
+    return launch_status();
+}
+
+int argmax_row_workgroups(int dim) {
+    if (dim <= kArgmaxOneWorkgroup) return 1;
+    return (dim + kArgmaxChunk - 1) / kArgmaxChunk;
+}
+
+hipError_t launch_argmax_row(hipStream_t stream, const float* row, int dim, unsigned long long* keys, uint32_t* token_u32,
+                             float* token_f32) {
+    const int groups = keys ? argmax_row_workgroups(dim) : 1;
+    if (groups == 1) {
+        hipLaunchKernelGGL(argmax_row_kernel, dim3(1), dim3(1024), 0, stream, row, dim, dim, nullptr, token_u32,
+                           token_f32);
+        return launch_status();
+    }
+    hipLaunchKernelGGL(argmax_row_kernel, dim3(groups), dim3(256), 0, stream, row, dim, kArgmaxChunk, keys, nullptr,
+                       nullptr);
+    if (hipError_t e = launch_status(); e != hipSuccess) return e;
+    return launch_argmax_keys(stream, keys, groups, token_u32, token_f32);
+}
+
+hipError_t launch_argmax_keys(hipStream_t stream, const unsigned long long* keys, int n, uint32_t* token_u32,
+                              float* token_f32) {
+    hipLaunchKernelGGL(argmax_keys_kernel, dim3(1), dim3(n > 2048 ? 1024 : 256), 0, stream, keys, n, token_u32, token_f32);
     return launch_status();
 }
 

@@ -33,6 +33,13 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
                              int out_dim, const GemvTuning& tune, float* dst_b = nullptr,
                              const uint8_t* weight_b_prepared = nullptr);
 
+// One row, no Y: every workgroup leaves the argmax key (see argmax_key) of its output
+// columns in keys[workgroup]; *key_count receives the number of workgroups, which is at
+// most (out_dim + 1) / 2.  launch_argmax_keys turns the keys into the token.
+hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned long long* keys, int* key_count,
+                                   const float* input, const uint8_t* weight_prepared, int in_dim, int out_dim,
+                                   const GemvTuning& tune);
+
 // Int8-MFMA GEMM on pre-quantized activations (natural order) and PREPARED
 // weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set.
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
@@ -52,5 +59,17 @@ hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* d
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);
+
+// argmax of row[0..dim): token_u32 and / or token_f32 (either may be null) receive the
+// index.  Rows longer than kArgmaxOneWorkgroup are scanned by argmax_row_workgroups(dim)
+// workgroups that leave one key each in `keys`, and a second launch picks the best; with
+// keys == nullptr one workgroup does everything.
+constexpr int kArgmaxOneWorkgroup = 16384;
+constexpr int kArgmaxChunk = 8192;  // 256 threads x 8 loads x 4 values
+int argmax_row_workgroups(int dim);
+hipError_t launch_argmax_row(hipStream_t stream, const float* row, int dim, unsigned long long* keys, uint32_t* token_u32,
+                             float* token_f32);
+hipError_t launch_argmax_keys(hipStream_t stream, const unsigned long long* keys, int n, uint32_t* token_u32,
+                              float* token_f32);
 
 }  // namespace afhip

@@ -156,6 +156,38 @@ class HipCompute:
                                                            in_dim, out_dim, C.byref(ha), C.byref(hb)))
         return HipTensor(ha.value), HipTensor(hb.value)
 
+    def linearNoBiasGrouped(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int,
+                            projection_out_dims, num_projections: int) -> HipTensor:
+        """ops/ops.zig:901, :1786-1800: `weight` is the concatenation of the projections along the output axis."""
+        dims = (C.c_uint32 * max(len(projection_out_dims), 1))(*projection_out_dims)
+        if num_projections > len(projection_out_dims):
+            raise _lib.InvalidShape(_lib.ERR_INVALID_SHAPE)
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_no_bias_grouped(self._h, input.handle, weight.handle, rows, in_dim,
+                                                              out_dim, dims, num_projections, C.byref(h)))
+        return HipTensor(h.value)
+
+    def argmaxLastRow(self, tensor: HipTensor, rows: int, dim: int) -> int:
+        """ops/ops.zig:1282, :2551: token id from the last row of a [rows, dim] tensor."""
+        token = C.c_uint32()
+        check(_lib.lib().afhip_compute_argmax_last_row(self._h, tensor.handle, rows, dim, C.byref(token)))
+        return int(token.value)
+
+    def linearNoBiasArgmaxLastRow(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int) -> int:
+        """ops/ops.zig:1292, :2565: argmax(input @ weight^T) for the last input row."""
+        token = C.c_uint32()
+        check(_lib.lib().afhip_compute_linear_no_bias_argmax_last_row(self._h, input.handle, weight.handle, rows, in_dim,
+                                                                      out_dim, C.byref(token)))
+        return int(token.value)
+
+    def linearNoBiasArgmaxLastRowTensor(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int,
+                                        out_dim: int) -> HipTensor:
+        """ops/ops.zig:1297, :2572: the token id as an f32 [1] backend tensor."""
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_no_bias_argmax_last_row_tensor(self._h, input.handle, weight.handle, rows,
+                                                                             in_dim, out_dim, C.byref(h)))
+        return HipTensor(h.value)
+
     def linearNoBiasPlanned(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int,
                             operator_plan: "quant_matmul.OperatorPlan") -> HipTensor:
         req = _lib.PlannedRequest(input.handle, weight.handle, rows, in_dim, out_dim, operator_plan.to_c())

@@ -52,6 +52,28 @@ def launchBlockDots(stream, tensor_type, layout, dots: Buffer, input: Buffer, we
                                              workspace, dispatch))
 
 
+def argmaxWorkspaceBytes(dim: int) -> int:
+    return _lib.lib().afhip_argmax_workspace_bytes(dim)
+
+
+def launchArgmaxLastRowF32(stream, token_u32: Buffer, token_f32: Buffer, input: Buffer, rows, dim,
+                           workspace: Buffer = NO_BUFFER) -> None:
+    """Token id of the last row of f32 [rows, dim]: as u32 and / or as f32 (either buffer may be NO_BUFFER).
+    With a workspace of argmaxWorkspaceBytes(dim) a long row is scanned by many workgroups."""
+    check(_lib.lib().afhip_launch_argmax_last_row_f32(stream, token_u32, token_f32, input, rows, dim, workspace))
+
+
+def linearArgmaxWorkspaceBytes(tensor_type: int, in_dim: int, out_dim: int) -> int:
+    return _lib.lib().afhip_linear_argmax_workspace_bytes(tensor_type, in_dim, out_dim)
+
+
+def launchLinearArgmaxLastRowF32(stream, tensor_type, layout, token_u32: Buffer, token_f32: Buffer, input: Buffer,
+                                 weight: Buffer, rows, in_dim, out_dim, workspace: Buffer) -> None:
+    """argmax(X[rows-1] @ W^T) without the logits matrix (lm_head of a greedy decode step)."""
+    check(_lib.lib().afhip_launch_linear_argmax_last_row_f32(stream, tensor_type, layout, token_u32, token_f32, input,
+                                                             weight, rows, in_dim, out_dim, workspace))
+
+
 def launchDecodeFp16(stream, dst_f32: Buffer, src_u16: Buffer, n: int) -> None:
     check(_lib.lib().afhip_launch_decode_fp16(stream, dst_f32, src_u16, n))
 

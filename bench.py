@@ -139,6 +139,40 @@ def main() -> int:
         wall = time.perf_counter() - t0
         return wall, e0.elapsed_time(e1) * 1e-3
 
+    def time_lm_head(out_dim=128256, in_dim=4096, steps=40, copies=2):
+        """argmax(x @ W^T) over a Llama-3 vocabulary, Q4_0: GEMV into scratch + argmax kernel per call."""
+        ws = prepared_copies(Q4, out_dim, in_dim, copies, 31)
+        x = torch.from_numpy(synth.activations(32, 1, in_dim)).to(dev)
+        scratch = torch.empty(kernels.linearArgmaxWorkspaceBytes(Q4, in_dim, out_dim), dtype=torch.uint8, device=dev)
+        token = torch.zeros(2, dtype=torch.int32, device=dev)
+        bx, bs, bt = buf(x), buf(scratch), buf(token[:1])
+        bws = [buf(w) for w in ws]
+
+        def step(i, st):
+            kernels.launchLinearArgmaxLastRowF32(st, Q4, _lib.LAYOUT_PREPARED, bt, kernels.NO_BUFFER, bx, bws[i % copies],
+                                                 1, in_dim, out_dim, bs)
+
+        for i in range(4):
+            step(i, stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cs = torch.cuda.current_stream().cuda_stream
+            for i in range(steps):
+                step(i, cs)
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        sec = e0.elapsed_time(e1) * 1e-3 / steps
+        b = gemv_bytes(Q4, 1, in_dim, out_dim)
+        return {"what": "greedy lm_head: Q4_0 GEMV over a 128256-token vocabulary into scratch, then the argmax kernel",
+                "us_per_call": round(sec * 1e6, 3), "GBps": round(b / sec / 1e9, 1),
+                "frac_hbm_peak": round(b / sec / HBM_PEAK_BPS, 4)}
+
     def decode_sweep(layers=32, token_steps=20):
         """Matmuls of one Llama-3-8B-shaped decode step (Q4_0, 32 layers of QKV, O, gate, up,
         down), every layer with its own weight memory, as one HIP graph per token."""
@@ -310,6 +344,7 @@ def main() -> int:
                                                  "us_per_call": round(e_s / gsteps * 1e6, 3),
                                                  "TOPS": round(ops * gsteps / e_s / 1e12, 3),
                                                  "frac_int8_mfma_peak": round(ops * gsteps / e_s / INT8_MFMA_PEAK_OPS, 5)}
+        extra["q4_lm_head_argmax_k4096_n128256"] = time_lm_head()
         extra["llama3_8b_decode_matmuls"] = decode_sweep()
         result["extra"] = extra
 

@@ -136,6 +136,30 @@ afhip_status afhip_launch_linear_q4_0_f32(void *stream, afhip_buffer dst, afhip_
                                           afhip_buffer weight_raw, size_t rows, size_t in_dim,
                                           size_t out_dim, afhip_buffer workspace);
 
+/* argmaxLastRow, ops/ops.zig:1282 (CPU op ops/native_compute.zig:37901-37907, argmax
+ * backends/activations.zig:350-357): index of the largest value of the last row of an
+ * f32 [rows, dim] tensor -- the lowest index among equal values, NaNs never win, 0 for
+ * an all-NaN row.  Written as u32 to token_u32 and / or as f32 to token_f32 (the engine's
+ * token tensors are f32 [1], architectures/gpt.zig:859-868); either .ptr may be 0.
+ * rows == 0 or dim == 0 -> AFHIP_ERR_INVALID_SHAPE.  `workspace` is optional
+ * (.ptr 0): with afhip_argmax_workspace_bytes(dim) bytes, 8-byte aligned, a long row is
+ * scanned by many workgroups (two launches) instead of one. */
+size_t afhip_argmax_workspace_bytes(size_t dim);
+afhip_status afhip_launch_argmax_last_row_f32(void *stream, afhip_buffer token_u32, afhip_buffer token_f32,
+                                              afhip_buffer input, size_t rows, size_t dim,
+                                              afhip_buffer workspace);
+/* linearNoBiasArgmaxLastRow / ...Tensor, ops/ops.zig:1292,1297 (caller
+ * architectures/gpt.zig:859-872): argmax(X[rows-1] * W^T) without the [rows, out_dim]
+ * logits: one GEMV over the last row.  On repacked weights its workgroups keep only
+ * the best of their own columns and a second small launch picks the token; otherwise
+ * the row of logits goes to the workspace and the argmax above runs on it.
+ * `workspace` (256-byte aligned) holds afhip_linear_argmax_workspace_bytes bytes. */
+size_t afhip_linear_argmax_workspace_bytes(int tensor_type, size_t in_dim, size_t out_dim);
+afhip_status afhip_launch_linear_argmax_last_row_f32(void *stream, int tensor_type, int layout,
+                                                     afhip_buffer token_u32, afhip_buffer token_f32,
+                                                     afhip_buffer input, afhip_buffer weight, size_t rows,
+                                                     size_t in_dim, size_t out_dim, afhip_buffer workspace);
+
 /* One-time device-side repack RAW -> PREPARED (dst.len >= src bytes). */
 afhip_status afhip_launch_prepare_weight(void *stream, int tensor_type, afhip_buffer dst_prepared,
                                          afhip_buffer src_raw, size_t out_dim, size_t in_dim);
@@ -233,6 +257,32 @@ afhip_status afhip_compute_linear_no_bias_pair(afhip_compute *self, const afhip_
                                                const afhip_tensor *weight_a, const afhip_tensor *weight_b,
                                                size_t rows, size_t in_dim, size_t out_dim,
                                                afhip_tensor **out_first, afhip_tensor **out_second);
+
+/* linearNoBiasGrouped, ops/ops.zig:901 (wrapper :1786-1800): `weight` is already the
+ * concatenation of `num_projections` matrices along the output axis, so this is one
+ * linear over out_dim; projection_out_dims must be non-zero and add up to out_dim,
+ * else AFHIP_ERR_INVALID_SHAPE (ops/metal_compute.zig:7859-7883). */
+afhip_status afhip_compute_linear_no_bias_grouped(afhip_compute *self, const afhip_tensor *input,
+                                                  const afhip_tensor *weight, size_t rows, size_t in_dim,
+                                                  size_t out_dim, const uint32_t *projection_out_dims,
+                                                  size_t num_projections, afhip_tensor **out);
+
+/* argmaxLastRow, ops/ops.zig:1282,2551: token id of the last row of an f32 tensor with
+ * rows*dim elements (else AFHIP_ERR_INVALID_SHAPE); synchronizes the stream. */
+afhip_status afhip_compute_argmax_last_row(afhip_compute *self, const afhip_tensor *tensor, size_t rows,
+                                           size_t dim, uint32_t *token);
+/* linearNoBiasArgmaxLastRow, ops/ops.zig:1292,2565: the token id on the host
+ * (synchronizes); ...Tensor, ops/ops.zig:1297,2572: a new f32 [1] tensor that holds the
+ * id, stream-ordered, for decode loops that feed it back without a host round trip.
+ * Errors as for afhip_compute_linear_no_bias. */
+afhip_status afhip_compute_linear_no_bias_argmax_last_row(afhip_compute *self, const afhip_tensor *input,
+                                                          const afhip_tensor *weight, size_t rows,
+                                                          size_t in_dim, size_t out_dim, uint32_t *token);
+afhip_status afhip_compute_linear_no_bias_argmax_last_row_tensor(afhip_compute *self,
+                                                                 const afhip_tensor *input,
+                                                                 const afhip_tensor *weight, size_t rows,
+                                                                 size_t in_dim, size_t out_dim,
+                                                                 afhip_tensor **out);
 
 /* linearNoBiasPlanned, ops/ops.zig:895 (request struct :92-99).  The plan is
  * validated like validateQuantLinearPlan (ops/native_compute.zig:5039-5050):

@@ -57,6 +57,10 @@ def lib() -> C.CDLL:
         L.afo_linear_act_assoc.argtypes = [i32, i32, vp, vp, vp, vp, sz, sz, sz]
         L.afo_linear_f32.argtypes = [i32, vp, vp, vp, sz, sz, sz]
         L.afo_linear_no_bias.argtypes = [i32, vp, vp, vp, sz, sz, sz, i32]
+        L.afo_argmax.restype = sz
+        L.afo_argmax.argtypes = [vp, sz]
+        L.afo_argmax_last_row.restype = C.c_long
+        L.afo_argmax_last_row.argtypes = [vp, sz, sz]
         L.afo_linear_act_f64.argtypes = [i32, vp, vp, vp, sz, sz, sz]
         L.afo_thread_plan.argtypes = [sz, sz, sz, i32, i32, vp]
         L.afo_prepare.restype = vp
@@ -194,6 +198,21 @@ def linear_act_f64(fmt, x, w_raw, rows, in_dim, out_dim) -> np.ndarray:
     if rc != 0:
         raise ValueError(f"afo_linear_act_f64 rc={rc}")
     return y
+
+
+def argmax(data) -> int:
+    d = _f32(data).reshape(-1)
+    return int(lib().afo_argmax(_p(d), d.size))
+
+
+def argmax_last_row(data, rows: int, dim: int) -> int:
+    """Token id of the last row; ValueError for an empty shape (error.InvalidTensorShape)."""
+    d = _f32(data).reshape(-1)
+    assert d.size == rows * dim
+    r = lib().afo_argmax_last_row(_p(d), rows, dim)
+    if r < 0:
+        raise ValueError("InvalidTensorShape")
+    return int(r)
 
 
 def thread_plan(rows, in_dim, out_dim, max_workers=8, cpu_count=8):

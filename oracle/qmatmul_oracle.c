@@ -622,3 +622,24 @@ int afo_linear_prepared(const afo_prepared *p, const float *x, float *y, size_t 
     free(sx);
     return 0;
 }
+
+/* ---- greedy token pick: INF/backends/activations.zig:331-357 ---- */
+
+size_t afo_argmax(const float *data, size_t n) {
+    if (n == 0) return 0;
+    /* vectorMax: @max over vectors = maxnum, a NaN operand loses */
+    float max_val = data[0];
+    for (size_t i = 1; i < n; ++i) {
+        if (max_val != max_val || data[i] > max_val) max_val = data[i];
+    }
+    /* argmax: first index whose value equals the maximum (a NaN equals nothing) */
+    for (size_t i = 0; i < n; ++i)
+        if (data[i] == max_val) return i;
+    return 0;
+}
+
+long afo_argmax_last_row(const float *data, size_t rows, size_t dim) {
+    /* INF/ops/native_compute.zig:37901-37907 */
+    if (rows == 0 || dim == 0) return -1;
+    return (long)afo_argmax(data + (rows - 1) * dim, dim);
+}

@@ -106,6 +106,17 @@ void afo_prepared_free(afo_prepared *p);
 int afo_linear_prepared(const afo_prepared *p, const float *x, float *y, size_t rows,
                         int workers);
 
+/* Greedy token pick, INF/backends/activations.zig:331-357 (vectorMax + argmax) as used
+ * by argmaxLastRow (INF/ops/native_compute.zig:37901-37907): the largest value's
+ * index, the first one among equal values (-0 == +0), 0 for an empty slice.  NaNs: the
+ * reference's vector maximum drops them (its scalar tail, whose length depends on the
+ * build's vector width, does not replace a NaN it started from); here a NaN never
+ * wins and an all-NaN slice gives 0, which is what the reference gives whenever the
+ * slice is at least one vector long. */
+size_t afo_argmax(const float *data, size_t n);
+/* Last row of [rows, dim]; -1 when rows or dim is 0 (error.InvalidTensorShape). */
+long afo_argmax_last_row(const float *data, size_t rows, size_t dim);
+
 #ifdef __cplusplus
 }
 #endif

@@ -188,3 +188,51 @@ def test_torch_memory_can_be_wrapped(cb):
     assert G.max_rel_err(y, ref.astype(np.float64)) <= 2e-5
     cb.freeTensor(xt)  # does not free torch's memory
     assert torch.equal(xd.cpu(), torch.from_numpy(x))
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_lm_head_ops(cb, fmt, kats):
+    """argmaxLastRow, linearNoBiasArgmaxLastRow(+Tensor) and linearNoBiasGrouped on the backend object."""
+    rows, in_dim, out_dim = 3, 512, 2048
+    print(f"case: backend lm_head ops fmt={fmt}", flush=True)
+    lr = kats["argmax"]["last_row"]
+    t = cb.fromFloat32(np.array(lr["data"], np.float32), [lr["rows"], lr["dim"]])
+    assert cb.argmaxLastRow(t, lr["rows"], lr["dim"]) == lr["expect"]
+    with pytest.raises(_lib.InvalidShape):
+        cb.argmaxLastRow(t, 0, 3)
+    with pytest.raises(_lib.InvalidShape):
+        cb.argmaxLastRow(t, 2, 4)
+    cb.freeTensor(t)
+
+    w = synth.weights(fmt, 21, out_dim, in_dim)
+    x = synth.activations(22, rows, in_dim)
+    cb.insertWeightFromLoaded("lm_head.weight", fmt, w, [out_dim, in_dim])
+    wt = cb.getWeight("lm_head.weight")
+    xt = cb.fromFloat32(x, [rows, in_dim])
+    logits = cb.linearNoBias(xt, wt, rows, in_dim, out_dim)
+    want = cb.argmaxLastRow(logits, rows, out_dim)
+    assert want == int(np.argmax(cb.toFloat32(logits).reshape(rows, out_dim)[-1]))
+    before = cb.debugStats()["launches_mmv"]
+    assert cb.linearNoBiasArgmaxLastRow(xt, wt, rows, in_dim, out_dim) == want
+    assert cb.debugStats()["launches_mmv"] == before + 1  # one GEMV over the last row, whatever `rows` is
+    tt = cb.linearNoBiasArgmaxLastRowTensor(xt, wt, rows, in_dim, out_dim)
+    assert tt.shape == [1] and tt.dtype == _lib.DTYPE_F32
+    assert cb.toFloat32(tt).tolist() == [float(want)]
+    cb.freeTensor(tt)
+    ref = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim, workers=8)
+    ref_token = O.argmax_last_row(ref, rows, out_dim)
+    assert want == ref_token or ref[-1, ref_token] - ref[-1, want] <= 2e-5 * np.abs(ref[-1]).max()
+    with pytest.raises(_lib.InvalidShape):
+        cb.linearNoBiasArgmaxLastRow(xt, wt, rows, in_dim, out_dim + 1)
+
+    # grouped: the weight is the concatenation of the projections, one linear serves them
+    y = cb.toFloat32(logits)
+    g = cb.linearNoBiasGrouped(xt, wt, rows, in_dim, out_dim, [1024, 512, 512], 3)
+    assert g.shape == [rows, out_dim] and np.array_equal(cb.toFloat32(g), y)
+    cb.freeTensor(g)
+    for dims, n in (([1024, 512], 2), ([1024, 0, 1024], 3), ([2048], 0)):
+        with pytest.raises(_lib.InvalidShape):
+            cb.linearNoBiasGrouped(xt, wt, rows, in_dim, out_dim, dims, n)
+    for t in (logits, xt):
+        cb.freeTensor(t)
+

@@ -320,6 +320,29 @@ def test_timing_path_matches_faithful_path(fmt):
     p.close()
 
 
+# ---------------------------------------------------------------- greedy token pick
+
+def test_argmax_reference_vectors_and_properties(kats):
+    for case in kats["argmax"]["cases"]:
+        assert O.argmax(case["data"]) == case["expect"]
+    lr = kats["argmax"]["last_row"]
+    assert O.argmax_last_row(lr["data"], lr["rows"], lr["dim"]) == lr["expect"]
+    with pytest.raises(ValueError):
+        O.argmax_last_row([], 0, 3)
+    # against numpy (first index of the maximum) on random rows with many ties
+    rng = np.random.default_rng(5)
+    for n in (1, 7, 64, 1000):
+        v = rng.integers(-3, 4, size=n).astype(np.float32)
+        assert O.argmax(v) == int(np.argmax(v))
+    # equal values: the first one; -0 equals +0; infinities order; NaNs never win
+    assert O.argmax([1.0, 5.0, 5.0, 2.0]) == 1
+    assert O.argmax([-1.0, -0.0, 0.0]) == 1
+    assert O.argmax([-np.inf, -np.inf]) == 0
+    assert O.argmax([1.0, np.inf, np.nan, np.inf]) == 1
+    assert O.argmax([np.nan, -2.0, np.nan, -1.0]) == 3
+    assert O.argmax([np.nan, np.nan]) == 0
+
+
 def test_synth_is_chunk_invariant_and_in_range():
     a = synth.splitmix64(42, 0, 1000)
     b = np.concatenate([synth.splitmix64(42, 0, 333), synth.splitmix64(42, 333, 667)])
