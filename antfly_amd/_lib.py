@@ -23,6 +23,7 @@ ERR_NO_DEVICES = -8
 ERR_OUT_OF_MEMORY = -9
 ERR_INVALID_ARGUMENT = -10
 ERR_SMOKE_MISMATCH = -11
+ERR_INVALID_TOKEN_ID = -12
 
 TYPE_F32, TYPE_Q4_0, TYPE_Q8_0 = 0, 2, 8
 LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
@@ -91,6 +92,9 @@ SIGNATURES = {
     "afhip_launch_argmax_last_row_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, Buffer]),
     "afhip_linear_argmax_workspace_bytes": (_sz, [_i, _sz, _sz]),
     "afhip_launch_linear_argmax_last_row_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
+    "afhip_launch_embedding_lookup_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
+    "afhip_launch_dequantize_f32": (_st, [_vp, _i, _i, Buffer, Buffer, _sz, _sz]),
+    "afhip_launch_quantize_rows": (_st, [_vp, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),
@@ -115,6 +119,7 @@ SIGNATURES = {
     "afhip_tensor_shape": (_st, [_vp, C.POINTER(C.c_int64), _sz]),
     "afhip_tensor_device_ptr": (C.c_uint64, [_vp]),
     "afhip_tensor_byte_len": (_sz, [_vp]),
+    "afhip_compute_embedding_lookup": (_st, [_vp, _vp, C.POINTER(C.c_int64), _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_pair": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_grouped": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32), _sz, C.POINTER(_vp)]),
@@ -194,6 +199,10 @@ class HipSmokeMismatch(HipError):
     pass
 
 
+class InvalidTokenId(HipError):
+    pass
+
+
 _ERRORS = {
     ERR_INVALID_STATE: InvalidHipState,
     ERR_UNSUPPORTED_TENSOR_TYPE: UnsupportedTensorType,
@@ -204,6 +213,7 @@ _ERRORS = {
     ERR_UNAVAILABLE: HipUnavailable,
     ERR_NO_DEVICES: NoHipDevices,
     ERR_SMOKE_MISMATCH: HipSmokeMismatch,
+    ERR_INVALID_TOKEN_ID: InvalidTokenId,
 }
 
 

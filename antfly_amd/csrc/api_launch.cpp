@@ -333,6 +333,7 @@ const char* afhip_status_string(afhip_status status) {
         case AFHIP_ERR_OUT_OF_MEMORY: return "OutOfMemory";
         case AFHIP_ERR_INVALID_ARGUMENT: return "InvalidArgument";
         case AFHIP_ERR_SMOKE_MISMATCH: return "HipSmokeMismatch";
+        case AFHIP_ERR_INVALID_TOKEN_ID: return "InvalidTokenId";
         default: break;
     }
     if (status > 0) return hipGetErrorName(static_cast<hipError_t>(status));
@@ -520,6 +521,72 @@ afhip_status afhip_launch_linear_argmax_last_row_f32(void* stream, int tensor_ty
                                                      afhip_buffer workspace) {
     return linear_argmax_impl(stream, tensor_type, layout, token_u32, token_f32, input, weight, rows, in_dim, out_dim,
                               workspace, nullptr);
+}
+
+// ---- row operators: get_rows / cpy_q_to_f32 / cpy_f32_to_q / set_rows
+
+static afhip_status dequantize_rows(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer weight,
+                                    afhip_buffer ids, bool gather, size_t rows, size_t dim, size_t weight_rows) {
+    const bool dense = tensor_type == AFHIP_TYPE_F32;
+    const size_t bb = block_bytes(tensor_type);
+    if (!dense && bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (dim == 0 || (!dense && dim % 32 != 0) || (dense && !gather)) return AFHIP_ERR_INVALID_STATE;
+    size_t out_count, out_bytes, w_count, w_bytes, id_bytes;
+    if (!checked_mul(rows, dim, &out_count) || !checked_mul(out_count, 4, &out_bytes) ||
+        !checked_mul(weight_rows, dim, &w_count) || !checked_mul(rows, 8, &id_bytes))
+        return AFHIP_ERR_INVALID_STATE;
+    if (dense) {
+        if (!checked_mul(w_count, 4, &w_bytes)) return AFHIP_ERR_INVALID_STATE;
+    } else if (!checked_mul(w_count / 32, bb, &w_bytes)) {
+        return AFHIP_ERR_INVALID_STATE;
+    }
+    if (out_bytes > dst.len || w_bytes > weight.len || (gather && id_bytes > ids.len)) return AFHIP_ERR_INVALID_STATE;
+    if (out_count == 0) return AFHIP_OK;
+    if (dim > 0x7fffffff || dst.ptr == 0 || weight.ptr == 0 || dst.ptr % 16 != 0 ||
+        weight.ptr % (dense ? 4 : (layout == AFHIP_LAYOUT_PREPARED ? 16 : 2)) != 0 ||
+        (gather && (ids.ptr == 0 || ids.ptr % 8 != 0)))
+        return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_dequantize_rows(static_cast<hipStream_t>(stream), tensor_type, layout,
+                                          reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
+                                          gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows,
+                                          static_cast<int>(dim), weight_rows);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_launch_embedding_lookup_f32(void* stream, int tensor_type, int layout, afhip_buffer dst,
+                                               afhip_buffer weight, afhip_buffer ids_i64, size_t total, size_t dim,
+                                               size_t vocab) {
+    return dequantize_rows(stream, tensor_type, layout, dst, weight, ids_i64, true, total, dim, vocab);
+}
+
+afhip_status afhip_launch_dequantize_f32(void* stream, int tensor_type, int layout, afhip_buffer dst,
+                                         afhip_buffer weight, size_t rows, size_t dim) {
+    return dequantize_rows(stream, tensor_type, layout, dst, weight, afhip_buffer{0, 0}, false, rows, dim, rows);
+}
+
+afhip_status afhip_launch_quantize_rows(void* stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
+                                        afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows) {
+    const size_t bb = block_bytes(tensor_type);
+    if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (dim == 0 || dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    const bool scatter = row_ids_i64.ptr != 0;
+    if (!scatter && dst_rows != rows) return AFHIP_ERR_INVALID_STATE;
+    size_t in_count, in_bytes, d_count, d_bytes, id_bytes;
+    if (!checked_mul(rows, dim, &in_count) || !checked_mul(in_count, 4, &in_bytes) ||
+        !checked_mul(dst_rows, dim, &d_count) || !checked_mul(d_count / 32, bb, &d_bytes) ||
+        !checked_mul(rows, 8, &id_bytes))
+        return AFHIP_ERR_INVALID_STATE;
+    if (in_bytes > input.len || d_bytes > dst_raw.len || (scatter && id_bytes > row_ids_i64.len)) return AFHIP_ERR_INVALID_STATE;
+    if (in_count == 0) return AFHIP_OK;
+    if (dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || dst_raw.ptr == 0 || dst_raw.ptr % 2 != 0 ||
+        (scatter && row_ids_i64.ptr % 8 != 0))
+        return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_quantize_rows(static_cast<hipStream_t>(stream), tensor_type,
+                                        reinterpret_cast<uint8_t*>(dst_raw.ptr), reinterpret_cast<const float*>(input.ptr),
+                                        scatter ? reinterpret_cast<const long long*>(row_ids_i64.ptr) : nullptr, rows,
+                                        static_cast<int>(dim));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
 }  // extern "C"

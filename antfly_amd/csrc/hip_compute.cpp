@@ -486,6 +486,41 @@ afhip_status afhip_tensor_shape(const afhip_tensor* t, int64_t* out, size_t out_
 uint64_t afhip_tensor_device_ptr(const afhip_tensor* t) { return t ? t->buffer.ptr : 0; }
 size_t afhip_tensor_byte_len(const afhip_tensor* t) { return t ? t->buffer.len : 0; }
 
+afhip_status afhip_compute_embedding_lookup(afhip_compute* self, const afhip_tensor* weight, const int64_t* ids,
+                                            size_t ids_len, size_t total, size_t dim, afhip_tensor** out) {
+    // cuda_compute.zig:405-435
+    if (!self || !weight || !out || (!ids && ids_len != 0)) return AFHIP_ERR_INVALID_ARGUMENT;
+    *out = nullptr;
+    if (weight->quant_type < 0 && !is_f32(weight)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (ids_len != total) return AFHIP_ERR_INVALID_SHAPE;
+    if (dim == 0 || weight->elem_count % dim != 0) return AFHIP_ERR_INVALID_SHAPE;
+    const size_t vocab = weight->elem_count / dim;
+    for (size_t i = 0; i < total; ++i)
+        if (ids[i] < 0 || static_cast<uint64_t>(ids[i]) >= vocab) return AFHIP_ERR_INVALID_TOKEN_ID;
+    if (weight->quant_type >= 0 && weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0)
+        return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    size_t out_count, out_bytes;
+    if (!checked_mul(total, dim, &out_count) || !checked_mul(out_count, 4, &out_bytes)) return AFHIP_ERR_INVALID_SHAPE;
+    afhip_status s = make_current(self);
+    if (s != AFHIP_OK) return s;
+    afhip_buffer ids_device, device;
+    s = alloc_device_buffer(self, total * 8, &ids_device);  // uploadTempI64
+    if (s != AFHIP_OK) return s;
+    s = alloc_device_buffer(self, out_bytes, &device);
+    if (s == AFHIP_OK) s = copy_from_host(self, ids_device, ids, total * 8);
+    if (s == AFHIP_OK)
+        s = afhip_launch_embedding_lookup_f32(self->stream, weight->quant_type < 0 ? AFHIP_TYPE_F32 : weight->quant_type,
+                                              weight->layout, device, weight->buffer, ids_device, total, dim, vocab);
+    // the ids were read from pageable host memory: the copy has completed on return, and the
+    // kernel that reads the device copy is ordered before any later use of the pooled buffer
+    release_device_buffer(self, &ids_device);
+    if (s != AFHIP_OK) {
+        release_device_buffer(self, &device);
+        return s;
+    }
+    return make_f32_result(self, device, total, dim, out_count, out);
+}
+
 afhip_status afhip_compute_linear_no_bias(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
                                           size_t rows, size_t in_dim, size_t out_dim, afhip_tensor** out) {
     return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out);

@@ -115,6 +115,111 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(uint8_t* __restrict
     for (int j = 0; j < kQuantBytes / 2; ++j) dq[j] = s[1 + j];
 }
 
+// get_rows / cpy_q_to_f32: dst[t][:] = dequantized row ids[t] of a [*, dim] weight
+// (w = d * f32(q), gguf/quant_codec.zig:1877-1895, :1918-1942); ids == nullptr copies rows
+// 0 .. rows-1 in order.  Eight lanes per block, four values (one 16-byte store) per lane,
+// so a wavefront writes 1 KB of contiguous output.  `blocks_total` = blocks of the whole
+// weight (where the scales of the repacked layout start).
+template <int kType, bool kPrepared>
+__global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict__ dst, const uint8_t* __restrict__ weight,
+                                                              const long long* __restrict__ ids, size_t rows, int dim,
+                                                              size_t blocks_total) {
+    constexpr int kQuantBytes = kType == 2 ? 16 : 32;
+    const size_t kb = static_cast<size_t>(dim >> 5);
+    const size_t units = rows * kb * 8;
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const int j = static_cast<int>(u & 7);  // values 4j .. 4j+3 of the block
+        const size_t tb = u >> 3;
+        const size_t t = tb / kb, b = tb - t * kb;
+        const size_t block = static_cast<size_t>(ids ? ids[t] : static_cast<long long>(t)) * kb + b;
+        const uint8_t* quants = kPrepared ? weight + block * kQuantBytes : weight + block * (kQuantBytes + 2) + 2;
+        const uint16_t scale_bits = kPrepared ? reinterpret_cast<const uint16_t*>(weight + blocks_total * kQuantBytes)[block]
+                                              : *reinterpret_cast<const uint16_t*>(weight + block * (kQuantBytes + 2));
+        const float d = half_bits_to_f32(scale_bits);
+        // four quant bytes: Q8_0 values 4j..4j+3; Q4_0 bytes 4(j%4).. whose low (j < 4) or high nibbles are the values
+        const uint16_t* two = reinterpret_cast<const uint16_t*>(quants + 4 * (kType == 2 ? (j & 3) : j));
+        const uint32_t packed = two[0] | (static_cast<uint32_t>(two[1]) << 16);
+        float4 out;
+        if (kType == 2) {
+            const uint32_t n = (j < 4 ? packed : packed >> 4) & 0x0F0F0F0Fu;
+            out.x = d * static_cast<float>(static_cast<int>(n & 0xFF) - 8);
+            out.y = d * static_cast<float>(static_cast<int>((n >> 8) & 0xFF) - 8);
+            out.z = d * static_cast<float>(static_cast<int>((n >> 16) & 0xFF) - 8);
+            out.w = d * static_cast<float>(static_cast<int>(n >> 24) - 8);
+        } else {
+            out.x = d * static_cast<float>(static_cast<int8_t>(packed & 0xFF));
+            out.y = d * static_cast<float>(static_cast<int8_t>((packed >> 8) & 0xFF));
+            out.z = d * static_cast<float>(static_cast<int8_t>((packed >> 16) & 0xFF));
+            out.w = d * static_cast<float>(static_cast<int8_t>(packed >> 24));
+        }
+        reinterpret_cast<float4*>(dst)[u] = out;
+    }
+}
+
+// Dense f32 table: dst[t][:] = weight[ids[t]][:] (embedding lookup on an unquantized table).
+__global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict__ dst, const float* __restrict__ weight,
+                                                              const long long* __restrict__ ids, size_t rows, int dim) {
+    const size_t total = rows * static_cast<size_t>(dim);
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t t = i / dim, c = i - t * dim;
+        dst[i] = weight[static_cast<size_t>(ids[t]) * dim + c];
+    }
+}
+
+// set_rows / cpy_f32_to_q: rows of f32 -> GGUF blocks (raw layout) at row ids[t] of the
+// destination (ids == nullptr: rows in order).  The weight quantizers of
+// gguf/quant_codec.zig: Q8_0 :601-623 (scale = max|x| / 127, q = clamp(round_half_away(x / scale), +-127)),
+// Q4_0 :895-910, :1261-1265 (scale = max|x| / 8, nibble = clamp(round_half_away(x / scale) + 8, 0, 15),
+// byte i = value i | value i+16 << 4); the stored scale is f16(scale), an all-zero
+// block has scale 1.  Eight lanes per block.
+template <int kType>
+__global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
+                                                            const long long* __restrict__ ids, size_t rows, int dim) {
+    constexpr int kRawBytes = kType == 2 ? 18 : 34;
+    const size_t kb = static_cast<size_t>(dim >> 5);
+    const size_t units = rows * kb * 8;
+    for (size_t u0 = blockIdx.x * static_cast<size_t>(blockDim.x); u0 < units; u0 += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t u = u0 + threadIdx.x;        // units is a multiple of 8: a block's eight lanes are live together
+        const bool live = u < units;
+        const float4 v = live ? reinterpret_cast<const float4*>(x)[u] : float4{0.0f, 0.0f, 0.0f, 0.0f};
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        const float scale = m == 0.0f ? 1.0f : m / (kType == 2 ? 8.0f : 127.0f);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / scale;
+        const int j = static_cast<int>(u & 7);
+        const size_t tb = u >> 3;
+        const size_t t = live ? tb / kb : 0, b = live ? tb - t * kb : 0;
+        const size_t block = static_cast<size_t>(ids && live ? ids[t] : static_cast<long long>(t)) * kb + b;
+        uint8_t* out = dst + block * kRawBytes;
+        uint32_t packed;
+        if (kType == 2) {
+            // round_half_away(x * inv) + 8 clamped to 0..15 (an all-zero block: inv = 0 -> 8)
+            auto nib = [&](float a) {
+                const float tq = a * inv;
+                const float r = tq + __builtin_copysignf(0x1.fffffep-2f, tq);
+                return static_cast<uint32_t>(min(max(static_cast<int>(r) + 8, 0), 15));
+            };
+            const uint32_t mine = nib(v.x) | (nib(v.y) << 8) | (nib(v.z) << 16) | (nib(v.w) << 24);
+            // lane j < 4 holds values 4j..4j+3 (low nibbles), lane j+4 the matching high nibbles
+            const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(mine), 4));
+            packed = mine | (other << 4);  // meaningful on lanes j < 4 (other = lane j+4)
+        } else {
+            const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv), q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+            packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+        }
+        if (!live) continue;
+        // blocks are 2-byte aligned: 16-bit stores
+        if (j == 0) *reinterpret_cast<uint16_t*>(out) = __builtin_bit_cast(uint16_t, static_cast<_Float16>(scale));
+        if (kType != 2 || j < 4) {
+            uint16_t* q = reinterpret_cast<uint16_t*>(out + 2 + 4 * j);
+            q[0] = static_cast<uint16_t>(packed & 0xFFFF);
+            q[1] = static_cast<uint16_t>(packed >> 16);
+        }
+    }
+}
+
 __global__ __launch_bounds__(256) void decode_fp16_kernel(float* __restrict__ dst, const uint16_t* __restrict__ src,
                                                           size_t n) {
     const size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
@@ -293,6 +398,41 @@ hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* 
     if (n16 == 0) return hipSuccess;
     hipLaunchKernelGGL(stream_read_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0, stream,
                        reinterpret_cast<const stream_u32x4*>(src), sink, n16);
+    return launch_status();
+}
+
+static unsigned grid_for(size_t units) {
+    size_t grid = (units + 255) / 256;
+    return static_cast<unsigned>(grid > 65536 ? 65536 : (grid == 0 ? 1 : grid));
+}
+
+hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layout, float* dst, const uint8_t* weight,
+                                  const long long* ids, size_t rows, int dim, size_t weight_rows) {
+    if (rows == 0 || dim == 0) return hipSuccess;
+    if (tensor_type == 0) {
+        if (ids == nullptr) return hipErrorInvalidValue;  // a plain copy is not this kernel's job
+        hipLaunchKernelGGL(gather_rows_f32_kernel, dim3(grid_for(rows * dim)), dim3(256), 0, stream, dst,
+                           reinterpret_cast<const float*>(weight), ids, rows, dim);
+        return launch_status();
+    }
+    const size_t blocks_total = weight_rows * static_cast<size_t>(dim >> 5);
+    const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
+    if (tensor_type == 2) {
+        if (layout == 0) hipLaunchKernelGGL((dequantize_rows_kernel<2, false>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+        else hipLaunchKernelGGL((dequantize_rows_kernel<2, true>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+    } else {
+        if (layout == 0) hipLaunchKernelGGL((dequantize_rows_kernel<8, false>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+        else hipLaunchKernelGGL((dequantize_rows_kernel<8, true>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+    }
+    return launch_status();
+}
+
+hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
+                                size_t rows, int dim) {
+    if (rows == 0 || dim == 0) return hipSuccess;
+    const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
+    if (tensor_type == 2) hipLaunchKernelGGL(quantize_rows_kernel<2>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim);
+    else hipLaunchKernelGGL(quantize_rows_kernel<8>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim);
     return launch_status();
 }
 

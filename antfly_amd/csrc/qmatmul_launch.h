@@ -56,6 +56,15 @@ hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout
 hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
                                  size_t blocks);
 
+// get_rows / cpy_q_to_f32: dst f32 [rows][dim] = rows ids[t] (ids == nullptr: rows in order) of a
+// weight with weight_rows rows; tensor_type 0 = dense f32 table (ids required).
+hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layout, float* dst, const uint8_t* weight,
+                                  const long long* ids, size_t rows, int dim, size_t weight_rows);
+
+// set_rows / cpy_f32_to_q: f32 [rows][dim] -> raw GGUF blocks at rows ids[t] of dst_raw (ids == nullptr: in order).
+hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
+                                size_t rows, int dim);
+
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);

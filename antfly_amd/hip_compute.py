@@ -141,6 +141,15 @@ class HipCompute:
 
     free = freeTensor
 
+    def embeddingLookup(self, weight: HipTensor, ids, total: int, dim: int) -> HipTensor:
+        """ops/ops.zig:824, :1673: weight[ids[i]] for each i as f32 [total, dim] (f32, Q4_0 or Q8_0 table)."""
+        arr = np.ascontiguousarray(ids, dtype=np.int64)
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_embedding_lookup(self._h, weight.handle,
+                                                        arr.ctypes.data_as(C.POINTER(C.c_int64)), arr.size, total, dim,
+                                                        C.byref(h)))
+        return HipTensor(h.value)
+
     # -- the op ------------------------------------------------------------
     def linearNoBias(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int) -> HipTensor:
         h = C.c_void_p()

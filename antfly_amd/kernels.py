@@ -74,6 +74,25 @@ def launchLinearArgmaxLastRowF32(stream, tensor_type, layout, token_u32: Buffer,
                                                              weight, rows, in_dim, out_dim, workspace))
 
 
+def launchEmbeddingLookupF32(stream, tensor_type, layout, dst: Buffer, weight: Buffer, ids_i64: Buffer, total, dim,
+                             vocab) -> None:
+    """get_rows: dst f32 [total, dim] = dequantized rows ids[t] of a [vocab, dim] table (ids: int64 on the device)."""
+    check(_lib.lib().afhip_launch_embedding_lookup_f32(stream, tensor_type, layout, dst, weight, ids_i64, total, dim,
+                                                       vocab))
+
+
+def launchDequantizeF32(stream, tensor_type, layout, dst: Buffer, weight: Buffer, rows, dim) -> None:
+    """cpy_q_to_f32: the whole [rows, dim] tensor as f32."""
+    check(_lib.lib().afhip_launch_dequantize_f32(stream, tensor_type, layout, dst, weight, rows, dim))
+
+
+def launchQuantizeRows(stream, tensor_type, dst_raw: Buffer, input: Buffer, rows, dim, row_ids_i64: Buffer = NO_BUFFER,
+                       dst_rows=None) -> None:
+    """cpy_f32_to_q (no ids) / set_rows (row t of input -> row ids[t] of the destination): f32 -> raw GGUF blocks."""
+    check(_lib.lib().afhip_launch_quantize_rows(stream, tensor_type, dst_raw, input, row_ids_i64, rows, dim,
+                                                rows if dst_rows is None else dst_rows))
+
+
 def launchDecodeFp16(stream, dst_f32: Buffer, src_u16: Buffer, n: int) -> None:
     check(_lib.lib().afhip_launch_decode_fp16(stream, dst_f32, src_u16, n))
 

@@ -40,7 +40,8 @@ enum afhip_error {
     AFHIP_ERR_NO_DEVICES = -8,              /* error.NoCudaDevices */
     AFHIP_ERR_OUT_OF_MEMORY = -9,
     AFHIP_ERR_INVALID_ARGUMENT = -10,       /* null pointer / unknown enum at the ABI itself */
-    AFHIP_ERR_SMOKE_MISMATCH = -11          /* error.CudaSmokeMismatch */
+    AFHIP_ERR_SMOKE_MISMATCH = -11,         /* error.CudaSmokeMismatch */
+    AFHIP_ERR_INVALID_TOKEN_ID = -12        /* error.InvalidTokenId, ops/cuda/cuda_compute.zig:412-416 */
 };
 const char *afhip_status_string(afhip_status status);
 
@@ -160,6 +161,29 @@ afhip_status afhip_launch_linear_argmax_last_row_f32(void *stream, int tensor_ty
                                                      afhip_buffer input, afhip_buffer weight, size_t rows,
                                                      size_t in_dim, size_t out_dim, afhip_buffer workspace);
 
+/* Row operators on quantized tensors (planner vocabulary get_rows / set_rows /
+ * cpy_q_to_f32 / cpy_f32_to_q, graph/quant_matmul.zig:35-47,334-353).
+ *
+ * Embedding lookup = get_rows (launcher ops/cuda/kernels.zig launchEmbeddingLookupF32 /
+ * ...Q4KF32, op ops/cuda/cuda_compute.zig:405-435): dst f32 [total, dim] =
+ * dequantized rows ids[t] of a [vocab, dim] table, w = d * f32(q)
+ * (gguf/quant_codec.zig:1877-1895, :1918-1942).  tensor_type AFHIP_TYPE_F32 gathers
+ * from a dense table.  ids_i64: `total` little-endian int64 on the device, every one
+ * in [0, vocab) -- the backend op checks them on the host as the reference does; the
+ * launcher cannot.  dim % 32 != 0 for a quantized table -> AFHIP_ERR_INVALID_STATE. */
+afhip_status afhip_launch_embedding_lookup_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                               afhip_buffer weight, afhip_buffer ids_i64, size_t total,
+                                               size_t dim, size_t vocab);
+/* cpy_q_to_f32: the whole [rows, dim] tensor, dequantized in order. */
+afhip_status afhip_launch_dequantize_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                         afhip_buffer weight, size_t rows, size_t dim);
+/* cpy_f32_to_q (row_ids_i64.ptr == 0: rows in order, dst_rows == rows) and set_rows
+ * (row t of `input` becomes row row_ids[t] of the [dst_rows, dim] destination): f32 ->
+ * raw GGUF blocks with the engine's weight quantizers (gguf/quant_codec.zig:601-623
+ * Q8_0, :895-910 and :1261-1265 Q4_0).  dst_raw must be 2-byte aligned. */
+afhip_status afhip_launch_quantize_rows(void *stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
+                                        afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows);
+
 /* One-time device-side repack RAW -> PREPARED (dst.len >= src bytes). */
 afhip_status afhip_launch_prepare_weight(void *stream, int tensor_type, afhip_buffer dst_prepared,
                                          afhip_buffer src_raw, size_t out_dim, size_t in_dim);
@@ -239,6 +263,14 @@ size_t afhip_tensor_rank(const afhip_tensor *tensor);
 afhip_status afhip_tensor_shape(const afhip_tensor *tensor, int64_t *out, size_t out_len);
 uint64_t afhip_tensor_device_ptr(const afhip_tensor *tensor);
 size_t afhip_tensor_byte_len(const afhip_tensor *tensor);
+
+/* embeddingLookup, ops/ops.zig:824,1673 (ops/cuda/cuda_compute.zig:405-435): new f32
+ * tensor [total, dim] = rows ids[i] of `weight` (f32, Q4_0 or Q8_0, [vocab, dim]).
+ * ids_len != total, dim == 0 or elem_count % dim != 0 -> AFHIP_ERR_INVALID_SHAPE; an id
+ * outside [0, vocab) -> AFHIP_ERR_INVALID_TOKEN_ID; other quantized types ->
+ * AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE. */
+afhip_status afhip_compute_embedding_lookup(afhip_compute *self, const afhip_tensor *weight, const int64_t *ids,
+                                            size_t ids_len, size_t total, size_t dim, afhip_tensor **out);
 
 /* linearNoBias, ops/ops.zig:890 and cuda_compute.zig:689-717: new f32 tensor
  * [rows, out_dim] owned by the caller.  Quantized weights other than
