@@ -24,6 +24,12 @@ ERR_OUT_OF_MEMORY = -9
 ERR_INVALID_ARGUMENT = -10
 ERR_SMOKE_MISMATCH = -11
 ERR_INVALID_TOKEN_ID = -12
+ERR_GGUF_INVALID_MAGIC = -13
+ERR_GGUF_UNEXPECTED_EOF = -14
+ERR_GGUF_UNSUPPORTED_METADATA = -15
+ERR_GGUF_NESTED_ARRAY = -16
+ERR_TENSOR_NOT_FOUND = -17
+ERR_IO = -18
 
 TYPE_F32, TYPE_Q4_0, TYPE_Q8_0 = 0, 2, 8
 LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
@@ -69,6 +75,27 @@ class DebugStats(C.Structure):
         "h2d_bytes", "d2h_bytes", "resident_weight_bytes", "pooled_buffers", "device_allocs",
         "launches_mmv", "launches_small_batch", "launches_mm", "launches_f32_route",
         "launches_activation_quant", "launches_prepare", "scratch_bytes")]
+
+
+GGUF_MAX_DIMS = 8
+
+
+class GgufSummary(C.Structure):
+    _fields_ = [("version", C.c_uint32), ("tensor_count", C.c_uint64), ("metadata_count", C.c_uint64),
+                ("alignment", C.c_uint64), ("data_region_offset", C.c_uint64), ("file_len", C.c_uint64)]
+
+
+class GgufTensorInfo(C.Structure):
+    _fields_ = [("name", C.c_void_p), ("name_len", C.c_size_t), ("n_dimensions", C.c_uint32),
+                ("dimensions", C.c_uint64 * GGUF_MAX_DIMS), ("tensor_type", C.c_uint32), ("type_name", C.c_char_p),
+                ("is_quantized", C.c_int), ("offset", C.c_uint64), ("data_offset", C.c_uint64),
+                ("byte_len", C.c_uint64)]
+
+
+class GgufMetadata(C.Structure):
+    _fields_ = [("key", C.c_void_p), ("key_len", C.c_size_t), ("value_type", C.c_uint32),
+                ("element_type", C.c_uint32), ("count", C.c_uint64), ("u64", C.c_uint64), ("i64", C.c_int64),
+                ("f64", C.c_double), ("str", C.c_void_p), ("str_len", C.c_size_t)]
 
 
 # name -> (restype, argtypes); the loader test checks every one is exported.
@@ -127,6 +154,18 @@ SIGNATURES = {
     "afhip_compute_linear_no_bias_argmax_last_row": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32)]),
     "afhip_compute_linear_no_bias_argmax_last_row_tensor": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_planned": (_st, [_vp, C.POINTER(PlannedRequest), C.POINTER(_vp)]),
+    "afhip_gguf_parse": (_st, [_vp, _sz, C.POINTER(_vp)]),
+    "afhip_gguf_open": (_st, [C.c_char_p, C.POINTER(_vp)]),
+    "afhip_gguf_close": (None, [_vp]),
+    "afhip_gguf_get_summary": (_st, [_vp, C.POINTER(GgufSummary)]),
+    "afhip_gguf_tensor_at": (_st, [_vp, _sz, C.POINTER(GgufTensorInfo)]),
+    "afhip_gguf_find_tensor": (_st, [_vp, C.c_char_p, C.POINTER(GgufTensorInfo)]),
+    "afhip_gguf_tensor_data": (_st, [_vp, C.POINTER(GgufTensorInfo), C.POINTER(_vp), C.POINTER(_sz)]),
+    "afhip_gguf_tensor_byte_len": (C.c_uint64, [C.c_uint32, _i, C.POINTER(C.c_uint64), _sz]),
+    "afhip_gguf_metadata_at": (_st, [_vp, _sz, C.POINTER(GgufMetadata)]),
+    "afhip_gguf_find_metadata": (_st, [_vp, C.c_char_p, C.POINTER(GgufMetadata)]),
+    "afhip_compute_insert_weight_from_gguf": (_st, [_vp, _vp, C.c_char_p, C.c_char_p, _i]),
+    "afhip_compute_load_gguf": (_st, [_vp, _vp, _i, C.POINTER(_sz), C.POINTER(_sz)]),
     "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
     "afhip_smoke_q8_0": (_st, []),
     "afhip_smoke_q4_0": (_st, []),
@@ -203,6 +242,30 @@ class InvalidTokenId(HipError):
     pass
 
 
+class InvalidGgufMagic(HipError):
+    pass
+
+
+class UnexpectedEndOfFile(HipError):
+    pass
+
+
+class UnsupportedMetadataType(HipError):
+    pass
+
+
+class UnsupportedNestedMetadataArray(HipError):
+    pass
+
+
+class TensorNotFound(HipError):
+    pass
+
+
+class FileNotAccessible(HipError):
+    pass
+
+
 _ERRORS = {
     ERR_INVALID_STATE: InvalidHipState,
     ERR_UNSUPPORTED_TENSOR_TYPE: UnsupportedTensorType,
@@ -214,6 +277,12 @@ _ERRORS = {
     ERR_NO_DEVICES: NoHipDevices,
     ERR_SMOKE_MISMATCH: HipSmokeMismatch,
     ERR_INVALID_TOKEN_ID: InvalidTokenId,
+    ERR_GGUF_INVALID_MAGIC: InvalidGgufMagic,
+    ERR_GGUF_UNEXPECTED_EOF: UnexpectedEndOfFile,
+    ERR_GGUF_UNSUPPORTED_METADATA: UnsupportedMetadataType,
+    ERR_GGUF_NESTED_ARRAY: UnsupportedNestedMetadataArray,
+    ERR_TENSOR_NOT_FOUND: TensorNotFound,
+    ERR_IO: FileNotAccessible,
 }
 
 

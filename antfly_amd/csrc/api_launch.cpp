@@ -334,6 +334,12 @@ const char* afhip_status_string(afhip_status status) {
         case AFHIP_ERR_INVALID_ARGUMENT: return "InvalidArgument";
         case AFHIP_ERR_SMOKE_MISMATCH: return "HipSmokeMismatch";
         case AFHIP_ERR_INVALID_TOKEN_ID: return "InvalidTokenId";
+        case AFHIP_ERR_GGUF_INVALID_MAGIC: return "InvalidGgufMagic";
+        case AFHIP_ERR_GGUF_UNEXPECTED_EOF: return "UnexpectedEndOfFile";
+        case AFHIP_ERR_GGUF_UNSUPPORTED_METADATA: return "UnsupportedMetadataType";
+        case AFHIP_ERR_GGUF_NESTED_ARRAY: return "UnsupportedNestedMetadataArray";
+        case AFHIP_ERR_TENSOR_NOT_FOUND: return "TensorNotFound";
+        case AFHIP_ERR_IO: return "FileNotAccessible";
         default: break;
     }
     if (status > 0) return hipGetErrorName(static_cast<hipError_t>(status));

@@ -104,6 +104,19 @@ class HipCompute:
         shp = (C.c_int64 * max(len(shape), 1))(*shape)
         check(_lib.lib().afhip_compute_insert_weight_f32(self._h, key.encode(), arr.ctypes.data, shp, len(shape)))
 
+    def insertWeightFromGguf(self, file, tensor_name: str, key: str = None, keep_raw_layout: bool = False) -> None:
+        """One tensor of an open gguf.File becomes a resident weight (models/tensor_store.zig:370-392)."""
+        check(_lib.lib().afhip_compute_insert_weight_from_gguf(self._h, file.handle, tensor_name.encode(),
+                                                               key.encode() if key is not None else None,
+                                                               int(keep_raw_layout)))
+
+    def loadGguf(self, file, keep_raw_layout: bool = False):
+        """Every F32 / Q4_0 / Q8_0 tensor of the file, under its own name; returns (loaded, skipped)."""
+        loaded, skipped = C.c_size_t(), C.c_size_t()
+        check(_lib.lib().afhip_compute_load_gguf(self._h, file.handle, int(keep_raw_layout), C.byref(loaded),
+                                                 C.byref(skipped)))
+        return int(loaded.value), int(skipped.value)
+
     def getWeight(self, name: str) -> HipTensor:
         h = C.c_void_p()
         check(_lib.lib().afhip_compute_get_weight(self._h, name.encode(), C.byref(h)))

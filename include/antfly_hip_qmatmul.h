@@ -41,7 +41,13 @@ enum afhip_error {
     AFHIP_ERR_OUT_OF_MEMORY = -9,
     AFHIP_ERR_INVALID_ARGUMENT = -10,       /* null pointer / unknown enum at the ABI itself */
     AFHIP_ERR_SMOKE_MISMATCH = -11,         /* error.CudaSmokeMismatch */
-    AFHIP_ERR_INVALID_TOKEN_ID = -12        /* error.InvalidTokenId, ops/cuda/cuda_compute.zig:412-416 */
+    AFHIP_ERR_INVALID_TOKEN_ID = -12,       /* error.InvalidTokenId, ops/cuda/cuda_compute.zig:412-416 */
+    AFHIP_ERR_GGUF_INVALID_MAGIC = -13,     /* error.InvalidGgufMagic, gguf/format.zig:165 */
+    AFHIP_ERR_GGUF_UNEXPECTED_EOF = -14,    /* error.UnexpectedEndOfFile, gguf/format.zig:282 */
+    AFHIP_ERR_GGUF_UNSUPPORTED_METADATA = -15, /* error.UnsupportedMetadataType, gguf/format.zig:179 */
+    AFHIP_ERR_GGUF_NESTED_ARRAY = -16,      /* error.UnsupportedNestedMetadataArray, gguf/format.zig:199 */
+    AFHIP_ERR_TENSOR_NOT_FOUND = -17,       /* error.TensorNotFound, models/tensor_store.zig:370 */
+    AFHIP_ERR_IO = -18                      /* the file could not be opened or mapped */
 };
 const char *afhip_status_string(afhip_status status);
 
@@ -332,6 +338,79 @@ typedef struct afhip_linear_no_bias_planned_request {
 afhip_status afhip_compute_linear_no_bias_planned(afhip_compute *self,
                                                   const afhip_linear_no_bias_planned_request *request,
                                                   afhip_tensor **out);
+
+/* ------------------------------------------------------------------------
+ * GGUF container: gguf/format.zig (parse, :113-161), gguf/tensor_types.zig
+ * (type ids :17-56, block geometry :160-219, byteLen :238-260),
+ * gguf/tensor_catalog.zig (find), and the path from the file to a resident device
+ * weight (models/tensor_store.zig:370-392 -> insertWeightFromLoaded).  Host code;
+ * strings returned here live as long as the afhip_gguf they came from.
+ * ---------------------------------------------------------------------- */
+typedef struct afhip_gguf afhip_gguf; /* format.File + the bytes it describes */
+enum { AFHIP_GGUF_MAX_DIMS = 8 };
+
+/* Parses a GGUF image the caller keeps alive (format.parse). */
+afhip_status afhip_gguf_parse(const void *bytes, size_t len, afhip_gguf **out);
+/* Maps the file read-only and parses it; tensor bytes are used in place
+ * (raw_mmap_backed, models/tensor_store.zig:389). */
+afhip_status afhip_gguf_open(const char *path, afhip_gguf **out);
+void afhip_gguf_close(afhip_gguf *file);
+
+typedef struct afhip_gguf_summary { /* format.Header + File.alignment / data_region_offset */
+    uint32_t version;
+    uint64_t tensor_count, metadata_count, alignment, data_region_offset, file_len;
+} afhip_gguf_summary;
+afhip_status afhip_gguf_get_summary(const afhip_gguf *file, afhip_gguf_summary *out);
+
+typedef struct afhip_gguf_tensor_info { /* format.TensorInfo, :85-96 */
+    const char *name;
+    size_t name_len;
+    uint32_t n_dimensions;
+    uint64_t dimensions[AFHIP_GGUF_MAX_DIMS]; /* as stored: fastest-varying first */
+    uint32_t tensor_type;  /* raw GGUF id */
+    const char *type_name; /* "Q4_0", ...; "TL2" for id 39 in a BitNet file; "UNKNOWN" */
+    int is_quantized;      /* TensorType.isQuantized */
+    uint64_t offset;       /* relative to the data region */
+    uint64_t data_offset;  /* absolute in the file */
+    uint64_t byte_len;     /* tensor_types.byteLen; 0 when the type's size rule is unknown */
+} afhip_gguf_tensor_info;
+/* index >= tensor_count / unknown name -> AFHIP_ERR_TENSOR_NOT_FOUND. */
+afhip_status afhip_gguf_tensor_at(const afhip_gguf *file, size_t index, afhip_gguf_tensor_info *out);
+afhip_status afhip_gguf_find_tensor(const afhip_gguf *file, const char *name, afhip_gguf_tensor_info *out);
+/* The tensor's bytes inside the image, bounds-checked against the file. */
+afhip_status afhip_gguf_tensor_data(const afhip_gguf *file, const afhip_gguf_tensor_info *info,
+                                    const void **data, size_t *len);
+/* tensor_types.byteLen; bitnet_dialect != 0 reads id 39 as TL2 (fromRawForDialect, :73-75).
+ * 0 = unknown type or overflow. */
+uint64_t afhip_gguf_tensor_byte_len(uint32_t tensor_type, int bitnet_dialect, const uint64_t *dimensions,
+                                    size_t n_dimensions);
+
+typedef struct afhip_gguf_metadata { /* format.MetadataEntry; value_type as format.MetadataValueType */
+    const char *key;
+    size_t key_len;
+    uint32_t value_type;   /* 0 u8 1 i8 2 u16 3 i16 4 u32 5 i32 6 f32 7 bool 8 string 9 array 10 u64 11 i64 12 f64 */
+    uint32_t element_type; /* arrays */
+    uint64_t count;        /* arrays: number of elements (the elements themselves are not kept) */
+    uint64_t u64;          /* unsigned and bool values */
+    int64_t i64;           /* signed values */
+    double f64;            /* float values (and integers, converted) */
+    const char *str;       /* string values */
+    size_t str_len;
+} afhip_gguf_metadata;
+afhip_status afhip_gguf_metadata_at(const afhip_gguf *file, size_t index, afhip_gguf_metadata *out);
+afhip_status afhip_gguf_find_metadata(const afhip_gguf *file, const char *key, afhip_gguf_metadata *out);
+
+/* One tensor of the file becomes a resident weight under `key` (null: its own name):
+ * Q4_0 / Q8_0 through insertWeightFromLoaded with shape = reversed GGUF dimensions
+ * (normalizedShapeFromDims, models/tensor_store.zig:654-658), F32 through
+ * insertWeightFromTensor; other types -> AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE. */
+afhip_status afhip_compute_insert_weight_from_gguf(afhip_compute *self, const afhip_gguf *file,
+                                                   const char *tensor_name, const char *key,
+                                                   int keep_raw_layout);
+/* Every F32 / Q4_0 / Q8_0 tensor of the file under its own name; tensors of other
+ * types are counted in *skipped (either counter may be null). */
+afhip_status afhip_compute_load_gguf(afhip_compute *self, const afhip_gguf *file, int keep_raw_layout,
+                                     size_t *loaded, size_t *skipped);
 
 /* Counters a backend snapshot exposes (ops/ops.zig:649-713,1368;
  * pkg/inference/CUDA.md:492-507). */

@@ -236,3 +236,44 @@ def test_lm_head_ops(cb, fmt, kats):
     for t in (logits, xt):
         cb.freeTensor(t)
 
+
+
+def test_gguf_file_to_device_weights(cb, tmp_path):
+    """A GGUF file on disk -> mapped -> resident weights -> the same results as weights inserted from memory."""
+    from antfly_amd import gguf
+    from tests import gguf_util as W
+
+    in_dim, out_dim, rows = 512, 768, 3
+    w4 = synth.weights(Q4, 31, out_dim, in_dim)
+    w8 = synth.weights(Q8, 32, out_dim, in_dim)
+    norm = synth.activations(33, 1, in_dim)[0]
+    img = W.build([("general.architecture", gguf.STRING, "llama"), ("llama.block_count", gguf.U32, 1)],
+                  [("blk.0.ffn_gate.weight", [in_dim, out_dim], Q4, w4.tobytes()),
+                   ("blk.0.ffn_up.weight", [in_dim, out_dim], Q8, w8.tobytes()),
+                   ("blk.0.ffn_norm.weight", [in_dim], 0, norm.tobytes()),
+                   ("blk.0.attn_q.weight", [256, 2], 12, bytes(288))])  # Q4_K: not a format this backend computes on
+    path = tmp_path / "model.gguf"
+    path.write_bytes(img)
+    x = synth.activations(34, rows, in_dim)
+    with gguf.File.open(str(path)) as f:
+        print("case: backend loadGguf", flush=True)
+        assert cb.loadGguf(f) == (3, 1)
+        with pytest.raises(_lib.UnsupportedTensorType):
+            cb.insertWeightFromGguf(f, "blk.0.attn_q.weight")
+        with pytest.raises(_lib.TensorNotFound):
+            cb.insertWeightFromGguf(f, "blk.9.missing")
+        cb.insertWeightFromGguf(f, "blk.0.ffn_up.weight", key="raw_up", keep_raw_layout=True)
+    # the file is closed and unmapped: the weights live on the device
+    xt = cb.fromFloat32(x, [rows, in_dim])
+    for name, fmt, w in (("blk.0.ffn_gate.weight", Q4, w4), ("blk.0.ffn_up.weight", Q8, w8), ("raw_up", Q8, w8)):
+        wt = cb.getWeight(name)
+        assert wt.quant_type == fmt and wt.shape == [out_dim, in_dim]
+        cb.insertWeightFromLoaded("direct", fmt, w, [out_dim, in_dim], keep_raw_layout=(name == "raw_up"))
+        y = cb.toFloat32(cb.linearNoBias(xt, wt, rows, in_dim, out_dim))
+        y_direct = cb.toFloat32(cb.linearNoBias(xt, cb.getWeight("direct"), rows, in_dim, out_dim))
+        assert np.array_equal(y, y_direct)
+        ref = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim, workers=8)
+        assert G.max_rel_err(y.reshape(rows, out_dim), ref.astype(np.float64)) <= 2e-5
+    nt = cb.getWeight("blk.0.ffn_norm.weight")
+    assert nt.dtype == _lib.DTYPE_F32 and nt.shape == [in_dim]
+    assert np.array_equal(cb.toFloat32(nt), norm)
