@@ -138,8 +138,14 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict_
                                               : *reinterpret_cast<const uint16_t*>(weight + block * (kQuantBytes + 2));
         const float d = half_bits_to_f32(scale_bits);
         // four quant bytes: Q8_0 values 4j..4j+3; Q4_0 bytes 4(j%4).. whose low (j < 4) or high nibbles are the values
-        const uint16_t* two = reinterpret_cast<const uint16_t*>(quants + 4 * (kType == 2 ? (j & 3) : j));
-        const uint32_t packed = two[0] | (static_cast<uint32_t>(two[1]) << 16);
+        const uint8_t* four = quants + 4 * (kType == 2 ? (j & 3) : j);
+        uint32_t packed;
+        if (kPrepared) {  // 16-byte aligned blocks
+            packed = *reinterpret_cast<const uint32_t*>(four);
+        } else {          // GGUF blocks are only 2-byte aligned
+            const uint16_t* two = reinterpret_cast<const uint16_t*>(four);
+            packed = two[0] | (static_cast<uint32_t>(two[1]) << 16);
+        }
         float4 out;
         if (kType == 2) {
             const uint32_t n = (j < 4 ? packed : packed >> 4) & 0x0F0F0F0Fu;

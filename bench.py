@@ -173,6 +173,52 @@ def main() -> int:
                 "us_per_call": round(sec * 1e6, 3), "GBps": round(b / sec / 1e9, 1),
                 "frac_hbm_peak": round(b / sec / HBM_PEAK_BPS, 4)}
 
+    def time_row_ops(rows=14336, dim=4096, steps=20):
+        """cpy_q_to_f32 / cpy_f32_to_q over one FFN matrix and an embedding lookup: HBM-bound copies."""
+        def timed(fn):
+            for _ in range(3):
+                fn(stream)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for _ in range(steps):
+                    fn(cs)
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e-3 / steps
+
+        out = {}
+        f32_bytes = rows * dim * 4
+        dense = torch.empty((rows, dim), dtype=torch.float32, device=dev)
+        for name, fmt, bb in (("q4_0", Q4, 18), ("q8_0", Q8, 34)):
+            w = prepared_copies(fmt, rows, dim, 1, 41)[0]
+            q_bytes = rows * dim // 32 * bb
+            sec = timed(lambda st: kernels.launchDequantizeF32(st, fmt, _lib.LAYOUT_PREPARED, buf(dense), buf(w), rows, dim))
+            out[f"cpy_{name}_to_f32"] = {"us_per_call": round(sec * 1e6, 2),
+                                        "GBps": round((q_bytes + f32_bytes) / sec / 1e9, 1),
+                                        "frac_hbm_peak": round((q_bytes + f32_bytes) / sec / HBM_PEAK_BPS, 4)}
+            raw = torch.empty(q_bytes, dtype=torch.uint8, device=dev)
+            sec = timed(lambda st: kernels.launchQuantizeRows(st, fmt, buf(raw), buf(dense), rows, dim))
+            out[f"cpy_f32_to_{name}"] = {"us_per_call": round(sec * 1e6, 2),
+                                        "GBps": round((q_bytes + f32_bytes) / sec / 1e9, 1),
+                                        "frac_hbm_peak": round((q_bytes + f32_bytes) / sec / HBM_PEAK_BPS, 4)}
+            tokens = 512
+            ids = torch.randint(0, rows, (tokens,), dtype=torch.int64, device=dev)
+            emb = torch.empty((tokens, dim), dtype=torch.float32, device=dev)
+            sec = timed(lambda st: kernels.launchEmbeddingLookupF32(st, fmt, _lib.LAYOUT_PREPARED, buf(emb), buf(w), buf(ids),
+                                                                   tokens, dim, rows))
+            moved = tokens * dim // 32 * bb + tokens * dim * 4
+            out[f"get_rows_{name}_512_tokens"] = {"us_per_call": round(sec * 1e6, 2), "GBps": round(moved / sec / 1e9, 1)}
+        out["what"] = (f"row operators on a {rows} x {dim} tensor: dequantize all of it, quantize all of it "
+                       "(bytes = quantized + f32 side), embedding lookup of 512 rows")
+        return out
+
     def decode_sweep(layers=32, token_steps=20):
         """Matmuls of one Llama-3-8B-shaped decode step (Q4_0, 32 layers of QKV, O, gate, up,
         down), every layer with its own weight memory, as one HIP graph per token."""
@@ -345,6 +391,7 @@ def main() -> int:
                                                  "TOPS": round(ops * gsteps / e_s / 1e12, 3),
                                                  "frac_int8_mfma_peak": round(ops * gsteps / e_s / INT8_MFMA_PEAK_OPS, 5)}
         extra["q4_lm_head_argmax_k4096_n128256"] = time_lm_head()
+        extra["row_ops_14336x4096"] = time_row_ops()
         extra["llama3_8b_decode_matmuls"] = decode_sweep()
         result["extra"] = extra
 
