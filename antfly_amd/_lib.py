@@ -31,7 +31,7 @@ ERR_GGUF_NESTED_ARRAY = -16
 ERR_TENSOR_NOT_FOUND = -17
 ERR_IO = -18
 
-TYPE_F32, TYPE_Q4_0, TYPE_Q8_0 = 0, 2, 8
+TYPE_F32, TYPE_Q4_0, TYPE_Q8_0, TYPE_Q4_K = 0, 2, 8, 12
 LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
 DTYPE_F32, DTYPE_U8 = 0, 1
 

@@ -81,12 +81,53 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
     return t;
 }
 
+// Q4_K: f32 activations against the dequantized weights, one kernel family for any row count.
+static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
+                                    size_t rows, size_t in_dim, size_t out_dim, int dispatch, bool want_dots,
+                                    LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b) {
+    const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
+    if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // this format has no integer route
+    if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || in_dim % 256 != 0) return AFHIP_ERR_INVALID_STATE;
+    size_t out_count, in_count, w_blocks, w_bytes, bytes;
+    if (!checked_mul(rows, out_dim, &out_count) || !checked_mul(rows, in_dim, &in_count) ||
+        !checked_mul(out_dim, in_dim / 256, &w_blocks) || !checked_mul(w_blocks, 144, &w_bytes))
+        return AFHIP_ERR_INVALID_STATE;
+    if (!checked_mul(out_count, 4, &bytes) || bytes > dst.len || (pair && bytes > dst_b.len)) return AFHIP_ERR_INVALID_STATE;
+    if (!checked_mul(in_count, 4, &bytes) || bytes > input.len) return AFHIP_ERR_INVALID_STATE;
+    if (w_bytes > weight.len || (pair && w_bytes > weight_b.len)) return AFHIP_ERR_INVALID_STATE;
+    if (out_count == 0) return AFHIP_OK;
+    if (rows > 0x7fffffff || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
+    if (in_dim > static_cast<size_t>(gemv_q4k_max_in_dim())) return AFHIP_ERR_OP_UNSUPPORTED;
+    if (dst.ptr == 0 || input.ptr == 0 || weight.ptr == 0 || dst.ptr % 4 != 0 || input.ptr % 16 != 0 || weight.ptr % 16 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    if (pair && (dst_b.ptr == 0 || weight_b.ptr == 0 || dst_b.ptr % 4 != 0 || weight_b.ptr % 16 != 0))
+        return AFHIP_ERR_INVALID_STATE;
+    const int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim, AFHIP_FORMAT_Q4_K);
+    for (int i = 0; i < (pair ? 2 : 1); ++i) {
+        if (counters) {
+            if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+            else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+            else counters->mm++;
+        }
+        hipError_t e = launch_gemv_q4k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
+                                       reinterpret_cast<const float*>(input.ptr),
+                                       reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
+                                       static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+        if (e != hipSuccess) return static_cast<afhip_status>(e);
+    }
+    return AFHIP_OK;
+}
+
 afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
                          int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
                          afhip_buffer weight_b) {
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
+    if (tensor_type == AFHIP_TYPE_Q4_K)
+        return linear_q4k_impl(stream, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters, dst_b,
+                               weight_b);
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -263,15 +304,17 @@ afhip_status argmax_last_row_impl(void* stream, afhip_buffer token_u32, afhip_bu
 afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip_buffer token_u32,
                                 afhip_buffer token_f32, afhip_buffer input, afhip_buffer weight, size_t rows,
                                 size_t in_dim, size_t out_dim, afhip_buffer workspace, LaunchCounters* counters) {
-    const size_t bb = block_bytes(tensor_type);
+    const bool q4k = tensor_type == AFHIP_TYPE_Q4_K;
+    const size_t bb = q4k ? 144 : block_bytes(tensor_type);
+    const size_t block_values = q4k ? 256 : 32;
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
     if (rows == 0 || in_dim == 0 || out_dim == 0) return AFHIP_ERR_INVALID_SHAPE;
-    if (in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    if (in_dim % block_values != 0) return AFHIP_ERR_INVALID_STATE;
     size_t count, bytes, w_blocks, w_bytes;
     if (!checked_mul(rows, in_dim, &count) || !checked_mul(count, 4, &bytes) || bytes > input.len)
         return AFHIP_ERR_INVALID_STATE;
-    if (!checked_mul(out_dim, in_dim / 32, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes) || w_bytes > weight.len)
+    if (!checked_mul(out_dim, in_dim / block_values, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes) || w_bytes > weight.len)
         return AFHIP_ERR_INVALID_STATE;
     if (in_dim > 0x7fffffff || out_dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || weight.ptr == 0)
         return AFHIP_ERR_INVALID_STATE;
@@ -286,7 +329,7 @@ afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip
     // only the last row's logits matter: one GEMV whatever `rows` is
     const afhip_buffer last_row{input.ptr + (rows - 1) * in_dim * 4, in_dim * 4};
 
-    if (layout == AFHIP_LAYOUT_PREPARED && weight.ptr % 16 == 0 && afhip_uses_activation_quant(1, in_dim, out_dim) &&
+    if (!q4k && layout == AFHIP_LAYOUT_PREPARED && weight.ptr % 16 == 0 && afhip_uses_activation_quant(1, in_dim, out_dim) &&
         in_dim <= static_cast<size_t>(gemv_fused_max_in_dim()) && gemv_row_chunk(1, in_dim) > 0) {
         // the GEMV's workgroups keep the best of their own columns; no logits are written
         unsigned long long* keys = reinterpret_cast<unsigned long long*>(workspace.ptr);  // at most (out_dim + 1) / 2 of them
@@ -303,7 +346,7 @@ afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip
     }
 
     const afhip_buffer logits{workspace.ptr, out_dim * 4};
-    const size_t linear_bytes = workspace_view(0, 1, in_dim).bytes;
+    const size_t linear_bytes = q4k ? 256 : workspace_view(0, 1, in_dim).bytes;
     const afhip_buffer linear_ws{workspace.ptr + logits_bytes, linear_bytes};
     const size_t keys_offset = logits_bytes + (linear_bytes + 255) / 256 * 256;
     const afhip_buffer keys_ws{workspace.ptr + keys_offset, workspace.len - keys_offset};
@@ -352,6 +395,7 @@ static size_t format_values_per_block(int format) {
     switch (format) {  // Format.valuesPerBlock, :84-117
         case AFHIP_FORMAT_Q4_0:
         case AFHIP_FORMAT_Q8_0: return 32;
+        case AFHIP_FORMAT_Q4_K: return 256;
         case AFHIP_FORMAT_F32: return 1;
         default: return 0;
     }
@@ -387,7 +431,8 @@ void afhip_quant_matmul_plan(size_t rows, size_t in_dim, size_t out_dim, int for
     static const uint8_t prim[4] = {AFHIP_PRIM_SCALAR, AFHIP_PRIM_MAT_VEC, AFHIP_PRIM_MAT_VEC_EXT, AFHIP_PRIM_MAT_MAT};
     out->primitive = prim[d];
     // operatorForDispatch, :279-287: every format known here supports mul_mv / mul_mv_ext / mul_mm
-    const bool known = format == AFHIP_FORMAT_Q4_0 || format == AFHIP_FORMAT_Q8_0 || format == AFHIP_FORMAT_F32;
+    const bool known = format == AFHIP_FORMAT_Q4_0 || format == AFHIP_FORMAT_Q8_0 || format == AFHIP_FORMAT_Q4_K ||
+                       format == AFHIP_FORMAT_F32;
     static const uint8_t op[4] = {AFHIP_OP_FALLBACK, AFHIP_OP_MUL_MV, AFHIP_OP_MUL_MV_EXT, AFHIP_OP_MUL_MM};
     out->op = known ? op[d] : static_cast<uint8_t>(AFHIP_OP_FALLBACK);
     out->row_bucket = static_cast<uint8_t>(afhip_quant_row_bucket(rows));
@@ -401,6 +446,7 @@ int afhip_quant_format_from_tensor_type(int tensor_type) {  // backend_contracts
     switch (tensor_type) {
         case AFHIP_TYPE_Q4_0: return AFHIP_FORMAT_Q4_0;
         case AFHIP_TYPE_Q8_0: return AFHIP_FORMAT_Q8_0;
+        case AFHIP_TYPE_Q4_K: return AFHIP_FORMAT_Q4_K;
         case AFHIP_TYPE_F32: return AFHIP_FORMAT_F32;
         default: return AFHIP_FORMAT_UNKNOWN;
     }
@@ -517,6 +563,8 @@ afhip_status afhip_launch_argmax_last_row_f32(void* stream, afhip_buffer token_u
 }
 
 size_t afhip_linear_argmax_workspace_bytes(int tensor_type, size_t in_dim, size_t out_dim) {
+    if (tensor_type == AFHIP_TYPE_Q4_K)
+        return in_dim == 0 || in_dim % 256 != 0 || out_dim == 0 ? 0 : argmax_logits_bytes(out_dim) + 256 + argmax_keys_bytes(out_dim);
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || in_dim == 0 || out_dim == 0) return 0;
     return argmax_logits_bytes(out_dim) + (workspace_view(0, 1, in_dim).bytes + 255) / 256 * 256 + argmax_keys_bytes(out_dim);
 }
@@ -534,25 +582,34 @@ afhip_status afhip_launch_linear_argmax_last_row_f32(void* stream, int tensor_ty
 static afhip_status dequantize_rows(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer weight,
                                     afhip_buffer ids, bool gather, size_t rows, size_t dim, size_t weight_rows) {
     const bool dense = tensor_type == AFHIP_TYPE_F32;
-    const size_t bb = block_bytes(tensor_type);
+    const bool q4k = tensor_type == AFHIP_TYPE_Q4_K;
+    const size_t bb = q4k ? 144 : block_bytes(tensor_type);
+    const size_t block_values = q4k ? 256 : 32;
     if (!dense && bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
-    if (dim == 0 || (!dense && dim % 32 != 0) || (dense && !gather)) return AFHIP_ERR_INVALID_STATE;
+    if (dim == 0 || (!dense && dim % block_values != 0) || (dense && !gather)) return AFHIP_ERR_INVALID_STATE;
     size_t out_count, out_bytes, w_count, w_bytes, id_bytes;
     if (!checked_mul(rows, dim, &out_count) || !checked_mul(out_count, 4, &out_bytes) ||
         !checked_mul(weight_rows, dim, &w_count) || !checked_mul(rows, 8, &id_bytes))
         return AFHIP_ERR_INVALID_STATE;
     if (dense) {
         if (!checked_mul(w_count, 4, &w_bytes)) return AFHIP_ERR_INVALID_STATE;
-    } else if (!checked_mul(w_count / 32, bb, &w_bytes)) {
+    } else if (!checked_mul(w_count / block_values, bb, &w_bytes)) {
         return AFHIP_ERR_INVALID_STATE;
     }
     if (out_bytes > dst.len || w_bytes > weight.len || (gather && id_bytes > ids.len)) return AFHIP_ERR_INVALID_STATE;
     if (out_count == 0) return AFHIP_OK;
     if (dim > 0x7fffffff || dst.ptr == 0 || weight.ptr == 0 || dst.ptr % 16 != 0 ||
-        weight.ptr % (dense ? 4 : (layout == AFHIP_LAYOUT_PREPARED ? 16 : 2)) != 0 ||
+        weight.ptr % (dense ? 4 : (q4k || layout == AFHIP_LAYOUT_PREPARED ? 16 : 2)) != 0 ||
         (gather && (ids.ptr == 0 || ids.ptr % 8 != 0)))
         return AFHIP_ERR_INVALID_STATE;
+    if (q4k) {
+        hipError_t e = launch_dequantize_q4k_rows(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr),
+                                                  reinterpret_cast<const uint8_t*>(weight.ptr),
+                                                  gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows,
+                                                  static_cast<int>(dim));
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     hipError_t e = launch_dequantize_rows(static_cast<hipStream_t>(stream), tensor_type, layout,
                                           reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
                                           gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows,

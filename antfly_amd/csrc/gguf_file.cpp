@@ -421,7 +421,8 @@ afhip_status afhip_compute_insert_weight_from_gguf(afhip_compute* self, const af
         if (reinterpret_cast<uintptr_t>(data) % 4 != 0) return AFHIP_ERR_INVALID_STATE;
         return afhip_compute_insert_weight_f32(self, name, static_cast<const float*>(data), shape, rank);
     }
-    if (t->raw_type != AFHIP_TYPE_Q4_0 && t->raw_type != AFHIP_TYPE_Q8_0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (t->raw_type != AFHIP_TYPE_Q4_0 && t->raw_type != AFHIP_TYPE_Q8_0 && t->raw_type != AFHIP_TYPE_Q4_K)
+        return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     return afhip_compute_insert_weight_from_loaded(self, name, static_cast<int>(t->raw_type), data, len, shape, rank,
                                                    keep_raw_layout);
 }
@@ -431,7 +432,8 @@ afhip_status afhip_compute_load_gguf(afhip_compute* self, const afhip_gguf* g, i
     if (!self || !g) return AFHIP_ERR_INVALID_ARGUMENT;
     size_t n_loaded = 0, n_skipped = 0;
     for (const TensorInfo& t : g->tensors) {
-        const bool supported = t.raw_type == AFHIP_TYPE_F32 || t.raw_type == AFHIP_TYPE_Q4_0 || t.raw_type == AFHIP_TYPE_Q8_0;
+        const bool supported = t.raw_type == AFHIP_TYPE_F32 || t.raw_type == AFHIP_TYPE_Q4_0 || t.raw_type == AFHIP_TYPE_Q8_0 ||
+                               t.raw_type == AFHIP_TYPE_Q4_K;
         if (!supported) {
             ++n_skipped;
             continue;

@@ -177,7 +177,8 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         if (w->quant_type < 0 && !is_f32(w)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
         if (w->elem_count != w_count) return AFHIP_ERR_INVALID_SHAPE;
         if (w->quant_type < 0) return AFHIP_ERR_OP_UNSUPPORTED;  // dense f32 linear is another operator
-        if (w->quant_type != AFHIP_TYPE_Q4_0 && w->quant_type != AFHIP_TYPE_Q8_0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+        if (w->quant_type != AFHIP_TYPE_Q4_0 && w->quant_type != AFHIP_TYPE_Q8_0 && w->quant_type != AFHIP_TYPE_Q4_K)
+            return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     }
     if (pair && (weight_b->quant_type != weight->quant_type || weight_b->layout != weight->layout)) {
         // nothing to share: two independent ops, as the engine's wrapper does (ops/ops.zig:1828-1849)
@@ -205,7 +206,7 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         }
     }
     afhip_buffer scratch{0, 0};
-    if (afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
+    if (weight->quant_type != AFHIP_TYPE_Q4_K && afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
         s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);
     }
     if (s == AFHIP_OK) {
@@ -497,7 +498,8 @@ afhip_status afhip_compute_embedding_lookup(afhip_compute* self, const afhip_ten
     const size_t vocab = weight->elem_count / dim;
     for (size_t i = 0; i < total; ++i)
         if (ids[i] < 0 || static_cast<uint64_t>(ids[i]) >= vocab) return AFHIP_ERR_INVALID_TOKEN_ID;
-    if (weight->quant_type >= 0 && weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0)
+    if (weight->quant_type >= 0 && weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0 &&
+        weight->quant_type != AFHIP_TYPE_Q4_K)
         return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     size_t out_count, out_bytes;
     if (!checked_mul(total, dim, &out_count) || !checked_mul(out_count, 4, &out_bytes)) return AFHIP_ERR_INVALID_SHAPE;
@@ -585,7 +587,8 @@ afhip_status linear_argmax(afhip_compute* self, const afhip_tensor* input, const
         !checked_mul(out_dim, in_dim, &w_count) || input->elem_count != in_count || weight->elem_count != w_count)
         return AFHIP_ERR_INVALID_SHAPE;
     if (weight->quant_type < 0) return is_f32(weight) ? AFHIP_ERR_OP_UNSUPPORTED : AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
-    if (weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    if (weight->quant_type != AFHIP_TYPE_Q4_0 && weight->quant_type != AFHIP_TYPE_Q8_0 && weight->quant_type != AFHIP_TYPE_Q4_K)
+        return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     afhip_status s = make_current(self);
     if (s != AFHIP_OK) return s;
     afhip_buffer id;  // [f32 id][u32 id]

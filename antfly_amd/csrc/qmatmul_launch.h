@@ -65,6 +65,15 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
 hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
                                 size_t rows, int dim);
 
+// Q4_K (raw GGUF layout, 16-byte aligned): Y = X * W^T on f32 activations, any number of rows
+// (two per launch), in_dim a multiple of 256 up to gemv_q4k_max_in_dim(); and its get_rows /
+// cpy_q_to_f32.
+int gemv_q4k_max_in_dim();
+hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                           int out_dim);
+hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
+                                      size_t rows, int dim);
+
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);

@@ -43,6 +43,7 @@ class Format(enum.IntEnum):
     unknown = 0
     q4_0 = 1
     q8_0 = 5
+    q4_k = 9
     f32 = 254
 
 

@@ -9,6 +9,9 @@ Shapes and distributions follow the benchmark definition:
   Q8_0 W     32 int8 uniform in [-127, 127] per block, scale fp16(|N(0, 0.02)| / 127)
   Q4_0 W     16 bytes of two uniform nibbles 0..15 (value = nibble - 8, low nibbles
              are elements 0..15 and high nibbles 16..31), scale fp16(|N(0, 0.02)| / 7)
+  Q4_K W     144-byte super-blocks of 256 weights: d = fp16(|N(0, 0.02)| / 240),
+             dmin = fp16(|N(0, 0.02)| / 64), 12 uniform bytes of packed 6-bit scales and
+             mins, 128 uniform bytes of nibbles
 Block layouts are GGUF's: [fp16 scale, little endian][quants], 34 / 18 bytes.
 """
 from __future__ import annotations
@@ -17,8 +20,10 @@ import numpy as np
 
 Q4_0 = 2  # GGUF tensor-type ids
 Q8_0 = 8
+Q4_K = 12
 BLOCK_VALUES = 32
 BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
+Q4_K_BLOCK_VALUES, Q4_K_BLOCK_BYTES = 256, 144
 
 _GOLDEN = np.uint64(0x9E3779B97F4A7C15)
 _M1 = np.uint64(0xBF58476D1CE4E5B9)
@@ -51,8 +56,25 @@ def activations(seed: int, rows: int, in_dim: int) -> np.ndarray:
     return normal(seed, rows * in_dim).astype(np.float32).reshape(rows, in_dim)
 
 
+def weights_q4_k(seed: int, out_dim: int, in_dim: int) -> np.ndarray:
+    """Raw GGUF Q4_K bytes for W[out_dim, in_dim], flat uint8."""
+    if in_dim % Q4_K_BLOCK_VALUES:
+        raise ValueError("in_dim must be a multiple of 256")
+    nb = out_dim * (in_dim // Q4_K_BLOCK_VALUES)
+    out = np.empty((nb, Q4_K_BLOCK_BYTES), dtype=np.uint8)
+    d = (np.abs(normal(seed ^ 0x5CA1E, nb)) * 0.02 / 240.0).astype(np.float16)
+    dmin = (np.abs(normal(seed ^ 0xD317, nb)) * 0.02 / 64.0).astype(np.float16)
+    out[:, 0:2] = d.view(np.uint8).reshape(nb, 2)
+    out[:, 2:4] = dmin.view(np.uint8).reshape(nb, 2)
+    raw = splitmix64(seed, 0, nb * 18)  # 140 of the 144 random bytes per block are used
+    out[:, 4:] = raw.view(np.uint8).reshape(nb, 144)[:, :140]
+    return out.reshape(-1)
+
+
 def weights(fmt: int, seed: int, out_dim: int, in_dim: int) -> np.ndarray:
     """Raw GGUF block bytes for W[out_dim, in_dim], flat uint8."""
+    if fmt == Q4_K:
+        return weights_q4_k(seed, out_dim, in_dim)
     if in_dim % BLOCK_VALUES:
         raise ValueError("in_dim must be a multiple of 32")
     nb = out_dim * (in_dim // BLOCK_VALUES)

@@ -52,7 +52,13 @@ enum afhip_error {
 const char *afhip_status_string(afhip_status status);
 
 /* GGUF tensor-type ids (gguf/tensor_types.zig). */
-enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_0 = 8 };
+enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_0 = 8, AFHIP_TYPE_Q4_K = 12 };
+/* Q4_K (144-byte super-blocks of 256 weights) is computed on f32 activations against the
+ * dequantized weights, as the engine does on the CPU (ops/native_compute.zig:31075-31144)
+ * and in its CUDA backend (ops/cuda/cuda_compute.zig:708): no activation quantizer, no
+ * block dots, no repack (the raw layout is used, 16-byte aligned; `layout` is ignored),
+ * no workspace; in_dim must be a multiple of 256.  Served by the linear launchers and
+ * ops, the pair op, the argmax ops, embedding lookup and cpy_q_to_f32. */
 
 /* How a quantized weight sits in device memory.
  * RAW       GGUF bytes as uploaded: [out][in/32] blocks of 18 / 34 bytes.
@@ -78,7 +84,7 @@ enum afhip_primitive { AFHIP_PRIM_MAT_VEC = 0, AFHIP_PRIM_MAT_VEC_EXT = 1, AFHIP
 enum afhip_operator { AFHIP_OP_FALLBACK = 0, AFHIP_OP_MUL_MV = 1, AFHIP_OP_MUL_MV_EXT = 2, AFHIP_OP_MUL_MM = 3, AFHIP_OP_GET_ROWS = 4 };
 enum afhip_row_bucket { AFHIP_ROWS_0 = 0, AFHIP_ROWS_1 = 1, AFHIP_ROWS_2_8 = 2, AFHIP_ROWS_9_64 = 3, AFHIP_ROWS_65_PLUS = 4 };
 /* quant_matmul.Format values for the formats this backend knows. */
-enum afhip_quant_format { AFHIP_FORMAT_UNKNOWN = 0, AFHIP_FORMAT_Q4_0 = 1, AFHIP_FORMAT_Q8_0 = 5, AFHIP_FORMAT_F32 = 254 };
+enum afhip_quant_format { AFHIP_FORMAT_UNKNOWN = 0, AFHIP_FORMAT_Q4_0 = 1, AFHIP_FORMAT_Q8_0 = 5, AFHIP_FORMAT_Q4_K = 9, AFHIP_FORMAT_F32 = 254 };
 
 typedef struct afhip_quant_plan { /* quant_matmul.Plan, :223-232 */
     uint8_t dispatch;

@@ -16,7 +16,9 @@ LIB_PATH = os.path.join(HERE, "libqmatmul_oracle.so")
 
 FMT_Q4_0 = 2
 FMT_Q8_0 = 8
-BLOCK_BYTES = {FMT_Q4_0: 18, FMT_Q8_0: 34}
+FMT_Q4_K = 12
+BLOCK_BYTES = {FMT_Q4_0: 18, FMT_Q8_0: 34, FMT_Q4_K: 144}
+BLOCK_VALUES = {FMT_Q4_0: 32, FMT_Q8_0: 32, FMT_Q4_K: 256}
 ASSOC_PAIR = 0
 ASSOC_SINGLE = 1
 
@@ -57,6 +59,10 @@ def lib() -> C.CDLL:
         L.afo_linear_act_assoc.argtypes = [i32, i32, vp, vp, vp, vp, sz, sz, sz]
         L.afo_linear_f32.argtypes = [i32, vp, vp, vp, sz, sz, sz]
         L.afo_linear_no_bias.argtypes = [i32, vp, vp, vp, sz, sz, sz, i32]
+        L.afo_q4k_unpack_scale_mins.argtypes = [vp, vp, vp]
+        L.afo_dequantize_q4_k.argtypes = [vp, sz, vp]
+        L.afo_linear_q4_k.argtypes = [vp, vp, vp, sz, sz, sz]
+        L.afo_linear_q4_k_f64.argtypes = [vp, vp, vp, sz, sz, sz]
         L.afo_argmax.restype = sz
         L.afo_argmax.argtypes = [vp, sz]
         L.afo_argmax_last_row.restype = C.c_long
@@ -197,6 +203,32 @@ def linear_act_f64(fmt, x, w_raw, rows, in_dim, out_dim) -> np.ndarray:
     rc = lib().afo_linear_act_f64(fmt, _p(x), _p(w_raw), _p(y), rows, in_dim, out_dim)
     if rc != 0:
         raise ValueError(f"afo_linear_act_f64 rc={rc}")
+    return y
+
+
+def q4k_unpack_scale_mins(scales12):
+    sc = _u8(scales12)
+    assert sc.size == 12
+    scs, mins = np.zeros(8, np.uint8), np.zeros(8, np.uint8)
+    lib().afo_q4k_unpack_scale_mins(_p(sc), _p(scs), _p(mins))
+    return scs, mins
+
+
+def dequantize_q4_k(raw) -> np.ndarray:
+    r = _u8(raw)
+    assert r.size % 144 == 0
+    out = np.zeros(r.size // 144 * 256, np.float32)
+    lib().afo_dequantize_q4_k(_p(r), r.size // 144, _p(out))
+    return out
+
+
+def linear_q4_k(x, w_raw, rows, in_dim, out_dim, f64=False) -> np.ndarray:
+    xx, w = _f32(x), _u8(w_raw)
+    assert xx.size == rows * in_dim and w.size == out_dim * (in_dim // 256) * 144
+    y = np.zeros((rows, out_dim), np.float64 if f64 else np.float32)
+    rc = (lib().afo_linear_q4_k_f64 if f64 else lib().afo_linear_q4_k)(_p(xx), _p(w), _p(y), rows, in_dim, out_dim)
+    if rc != 0:
+        raise ValueError("InvalidQuantizedLinearShape")
     return y
 
 

@@ -643,3 +643,75 @@ long afo_argmax_last_row(const float *data, size_t rows, size_t dim) {
     if (rows == 0 || dim == 0) return -1;
     return (long)afo_argmax(data + (rows - 1) * dim, dim);
 }
+
+/* ---- Q4_K ---- */
+
+void afo_q4k_unpack_scale_mins(const uint8_t *scales, uint8_t *scs, uint8_t *mins) {
+    /* native_compute.zig:33745-33754 */
+    for (int j = 0; j < 4; j++) {
+        scs[j] = scales[j] & 63;
+        mins[j] = scales[j + 4] & 63;
+    }
+    for (int j = 4; j < 8; j++) {
+        scs[j] = (uint8_t)((scales[j + 4] & 0x0F) | ((scales[j - 4] >> 6) << 4));
+        mins[j] = (uint8_t)((scales[j + 4] >> 4) | ((scales[j] >> 6) << 4));
+    }
+}
+
+void afo_dequantize_q4_k(const uint8_t *raw, size_t n_blocks, float *out) {
+    /* quant_codec.zig:2624-2663 */
+    for (size_t b = 0; b < n_blocks; b++) {
+        const uint8_t *blk = raw + b * AFO_Q4_K_BLOCK_BYTES;
+        float d = afo_fp16_to_f32((uint16_t)(blk[0] | (blk[1] << 8)));
+        float dmin = afo_fp16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+        uint8_t scs[8], mins[8];
+        afo_q4k_unpack_scale_mins(blk + 4, scs, mins);
+        const uint8_t *qs = blk + 16;
+        float *o = out + b * AFO_Q4_K_BLOCK_VALUES;
+        for (int chunk = 0; chunk < 4; chunk++) {
+            int sub = chunk * 2;
+            float dsc0 = d * (float)scs[sub], dmn0 = dmin * (float)mins[sub];
+            float dsc1 = d * (float)scs[sub + 1], dmn1 = dmin * (float)mins[sub + 1];
+            for (int i = 0; i < 32; i++) o[chunk * 64 + i] = dsc0 * (float)(qs[chunk * 32 + i] & 0x0F) - dmn0;
+            for (int i = 0; i < 32; i++) o[chunk * 64 + 32 + i] = dsc1 * (float)(qs[chunk * 32 + i] >> 4) - dmn1;
+        }
+    }
+}
+
+int afo_linear_q4_k(const float *x, const uint8_t *w, float *y, size_t rows, size_t in_dim, size_t out_dim) {
+    if (in_dim % AFO_Q4_K_BLOCK_VALUES != 0) return -1;
+    size_t kb = in_dim / AFO_Q4_K_BLOCK_VALUES;
+    float wf[AFO_Q4_K_BLOCK_VALUES];
+    for (size_t o = 0; o < out_dim; o++) {
+        for (size_t r = 0; r < rows; r++) y[r * out_dim + o] = 0.0f;
+        for (size_t b = 0; b < kb; b++) {
+            afo_dequantize_q4_k(w + (o * kb + b) * AFO_Q4_K_BLOCK_BYTES, 1, wf);
+            for (size_t r = 0; r < rows; r++) {
+                const float *xb = x + r * in_dim + b * AFO_Q4_K_BLOCK_VALUES;
+                float acc = 0.0f; /* dotQ4_KBlock with one lane */
+                for (int i = 0; i < AFO_Q4_K_BLOCK_VALUES; i++) acc += xb[i] * wf[i];
+                y[r * out_dim + o] += acc;
+            }
+        }
+    }
+    return 0;
+}
+
+int afo_linear_q4_k_f64(const float *x, const uint8_t *w, double *y, size_t rows, size_t in_dim, size_t out_dim) {
+    if (in_dim % AFO_Q4_K_BLOCK_VALUES != 0) return -1;
+    size_t kb = in_dim / AFO_Q4_K_BLOCK_VALUES;
+    float wf[AFO_Q4_K_BLOCK_VALUES];
+    for (size_t o = 0; o < out_dim; o++) {
+        for (size_t r = 0; r < rows; r++) y[r * out_dim + o] = 0.0;
+        for (size_t b = 0; b < kb; b++) {
+            afo_dequantize_q4_k(w + (o * kb + b) * AFO_Q4_K_BLOCK_BYTES, 1, wf);
+            for (size_t r = 0; r < rows; r++) {
+                const float *xb = x + r * in_dim + b * AFO_Q4_K_BLOCK_VALUES;
+                double acc = 0.0;
+                for (int i = 0; i < AFO_Q4_K_BLOCK_VALUES; i++) acc += (double)xb[i] * (double)wf[i];
+                y[r * out_dim + o] += acc;
+            }
+        }
+    }
+    return 0;
+}

@@ -106,6 +106,27 @@ void afo_prepared_free(afo_prepared *p);
 int afo_linear_prepared(const afo_prepared *p, const float *x, float *y, size_t rows,
                         int workers);
 
+/* ---- Q4_K: 144-byte super-blocks of 256 weights (INF/gguf/tensor_types.zig:160-219):
+ * fp16 d, fp16 dmin, 12 bytes of packed 6-bit (scale, min) pairs for 8 sub-blocks of
+ * 32, 128 bytes of nibbles.  The CPU engine multiplies f32 activations by the
+ * dequantized weights; there is no integer route for this format. */
+enum { AFO_FMT_Q4_K = 12, AFO_Q4_K_BLOCK_VALUES = 256, AFO_Q4_K_BLOCK_BYTES = 144 };
+/* unpackQ4KScaleMinsU8, INF/ops/native_compute.zig:33745-33754 (= quant_codec.zig:2742-2751). */
+void afo_q4k_unpack_scale_mins(const uint8_t *scales12, uint8_t *scs8, uint8_t *mins8);
+/* dequantizeQ4K, INF/gguf/quant_codec.zig:2624-2663: w = (d*sc)*f32(q) - (dmin*m), low
+ * nibbles of a 32-byte chunk = sub-block 2c, high nibbles = sub-block 2c+1. */
+void afo_dequantize_q4_k(const uint8_t *raw, size_t n_blocks, float *out);
+/* y[r][o] = sum_b dot(x block, dequantized block) in f32, values in natural order
+ * (dotQ4_KBlock, INF/ops/native_compute.zig:31075-31113, with one accumulator lane:
+ * the engine's lane count, and with it the order of the f32 sums, is a build
+ * parameter, so its outputs are only defined up to that reordering).
+ * -1 when in_dim is not a multiple of 256. */
+int afo_linear_q4_k(const float *x, const uint8_t *w_raw, float *y, size_t rows, size_t in_dim,
+                    size_t out_dim);
+/* The same sum in double precision over the f32 dequantized weights. */
+int afo_linear_q4_k_f64(const float *x, const uint8_t *w_raw, double *y, size_t rows, size_t in_dim,
+                        size_t out_dim);
+
 /* Greedy token pick, INF/backends/activations.zig:331-357 (vectorMax + argmax) as used
  * by argmaxLastRow (INF/ops/native_compute.zig:37901-37907): the largest value's
  * index, the first one among equal values (-0 == +0), 0 for an empty slice.  NaNs: the

@@ -109,7 +109,7 @@ def test_op_errors(cb):
     in_dim, out_dim = 256, 512
     w = synth.weights(Q8, 1, out_dim, in_dim)
     cb.insertWeightFromLoaded("w", Q8, w, [out_dim, in_dim])
-    cb.insertWeightFromLoaded("w_q4k", 12, np.zeros(144 * 2, np.uint8), [2, 256])  # resident, but no kernel here
+    cb.insertWeightFromLoaded("w_q6k", 14, np.zeros(210 * 2, np.uint8), [2, 256])  # resident, but no kernel here
     cb.insertWeightFromTensor("w_dense", np.zeros((out_dim, in_dim), np.float32), [out_dim, in_dim])
     x = cb.fromFloat32(synth.activations(2, 2, in_dim), [2, in_dim])
     with pytest.raises(_lib.WeightNotFound):
@@ -121,7 +121,7 @@ def test_op_errors(cb):
     with pytest.raises(_lib.UnsupportedTensorType):
         cb.linearNoBias(cb.getWeight("w"), cb.getWeight("w"), 2, in_dim, out_dim)  # quantized input
     with pytest.raises(_lib.UnsupportedTensorType):
-        cb.linearNoBias(cb.fromFloat32(np.zeros(2 * 256, np.float32), [2, 256]), cb.getWeight("w_q4k"), 2, 256, 2)
+        cb.linearNoBias(cb.fromFloat32(np.zeros(2 * 256, np.float32), [2, 256]), cb.getWeight("w_q6k"), 2, 256, 2)
     with pytest.raises(_lib.HipOpUnsupported):
         cb.linearNoBias(x, cb.getWeight("w_dense"), 2, in_dim, out_dim)
     with pytest.raises(_lib.InvalidShape):
@@ -251,7 +251,7 @@ def test_gguf_file_to_device_weights(cb, tmp_path):
                   [("blk.0.ffn_gate.weight", [in_dim, out_dim], Q4, w4.tobytes()),
                    ("blk.0.ffn_up.weight", [in_dim, out_dim], Q8, w8.tobytes()),
                    ("blk.0.ffn_norm.weight", [in_dim], 0, norm.tobytes()),
-                   ("blk.0.attn_q.weight", [256, 2], 12, bytes(288))])  # Q4_K: not a format this backend computes on
+                   ("blk.0.attn_q.weight", [256, 2], 14, bytes(420))])  # Q6_K: not a format this backend computes on
     path = tmp_path / "model.gguf"
     path.write_bytes(img)
     x = synth.activations(34, rows, in_dim)

@@ -1,0 +1,145 @@
+"""GPU parity for GGUF Q4_K (144-byte super-blocks), through the C ABI, against the CPU
+oracle.  The engine computes this format in f32 on the dequantized weights and its own
+outputs depend on its vector width, so the matmul is held to a tolerance: max-relative
+error <= 1e-3 stated, <= 2e-5 in practice (against the oracle's f32 sum and its f64 sum).
+Dequantization (get_rows, cpy_q_to_f32) is bit-exact."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from antfly_amd import _lib, kernels, synth  # noqa: E402
+from antfly_amd.hip_compute import HipCompute  # noqa: E402
+from oracle import oracle as O  # noqa: E402
+from tests import gpu_util as G  # noqa: E402
+
+Q4K = _lib.TYPE_Q4_K
+RAW = _lib.LAYOUT_RAW
+TOL, TIGHT = 1e-3, 2e-5
+
+
+def q4k_block(d_bits, dmin_bits, scales12, qs128):
+    return np.concatenate([np.array([d_bits, dmin_bits], np.uint16).view(np.uint8), np.asarray(scales12, np.uint8),
+                           np.asarray(qs128, np.uint8)])
+
+
+def test_reference_vectors(kats):
+    k = kats["q4_k"]
+    u = k["uniform_block"]
+    scales = [u["scales_first4"]] * 4 + [0] * 4 + [u["scales_last4"]] * 4
+    m = k["direct_matmul"]
+    print("case: q4_k direct matmul kat", flush=True)
+    w = np.concatenate([q4k_block(15360, 0, scales, [f] * 128) for f in m["row_qs_fill"]])
+    x = np.full((1, m["in_dim"]), m["input_fill"], np.float32)
+    y = G.linear(Q4K, RAW, x, G.to_dev(w), 1, m["in_dim"], m["out_dim"])
+    assert np.abs(y[0] - np.array(m["expected"])).max() <= m["tolerance_abs"]
+    h = k["header_packing"]
+    print("case: q4_k header packing kat", flush=True)
+    raw = np.array(h["header"] + h["qs_32"] * 4, np.uint8)
+    out = torch.empty(256, dtype=torch.float32, device=G.DEV)
+    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(out), G.buf(G.to_dev(raw)), 1, 256)
+    torch.cuda.synchronize()
+    want = np.array([h["scs"][sub] * (i % 16) - h["mins"][sub] for sub in range(8) for i in range(32)], np.float32)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 256), (5, 1024), (3, 4096)])
+def test_dequantize_and_get_rows_bit_exact(rows, dim):
+    print(f"case: q4_k cpy_q_to_f32 / get_rows rows={rows} dim={dim}", flush=True)
+    vocab = rows + 7
+    w = synth.weights(Q4K, 2, vocab, dim).copy()
+    w[0:4] = np.array([0x0001, 0x7BFF], np.uint16).view(np.uint8)  # subnormal d, largest finite dmin
+    wd = G.to_dev(w)
+    table = O.dequantize_q4_k(w).reshape(vocab, dim)
+    out = torch.empty((vocab, dim), dtype=torch.float32, device=G.DEV)
+    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(out), G.buf(wd), vocab, dim)
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), table.view(np.uint32))
+    ids = np.array([vocab - 1, 0, 3, 3][:rows + 1], dtype=np.int64)
+    idd = G.to_dev(ids)
+    emb = torch.empty((len(ids), dim), dtype=torch.float32, device=G.DEV)
+    kernels.launchEmbeddingLookupF32(G.stream(), Q4K, RAW, G.buf(emb), G.buf(wd), G.buf(idd), len(ids), dim, vocab)
+    torch.cuda.synchronize()
+    assert np.array_equal(emb.cpu().numpy().view(np.uint32), table[ids].view(np.uint32))
+
+
+SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130), (3, 1024, 40), (5, 4096, 96),
+          (1, 14336, 48), (2, 14336, 20), (9, 2048, 24), (1, 32768, 8)]
+
+
+@pytest.mark.parametrize("rows,in_dim,out_dim", SHAPES)
+def test_linear_matches_oracle(rows, in_dim, out_dim):
+    print(f"case: q4_k linear rows={rows} in={in_dim} out={out_dim}", flush=True)
+    w = synth.weights(Q4K, 11, out_dim, in_dim)
+    x = synth.activations(12, rows, in_dim)
+    y = G.linear(Q4K, RAW, x, G.to_dev(w), rows, in_dim, out_dim)
+    ref64 = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+    ref32 = O.linear_q4_k(x, w, rows, in_dim, out_dim)
+    err64, err32 = G.max_rel_err(y, ref64), G.max_rel_err(y, ref32.astype(np.float64))
+    assert err64 <= TOL and err64 <= TIGHT, err64
+    assert err32 <= TOL and err32 <= TIGHT, err32
+
+
+def test_linear_argument_checks():
+    w = G.to_dev(synth.weights(Q4K, 1, 4, 256))
+    x = G.to_dev(synth.activations(2, 1, 256))
+    y = torch.empty((1, 4), dtype=torch.float32, device=G.DEV)
+    ws = kernels.NO_BUFFER
+    with pytest.raises(_lib.InvalidHipState):  # K must be whole super-blocks
+        kernels.launchLinearF32(G.stream(), Q4K, RAW, G.buf(y), G.buf(x), G.buf(w), 1, 128, 4, ws)
+    with pytest.raises(_lib.InvalidHipState):  # short weight buffer
+        kernels.launchLinearF32(G.stream(), Q4K, RAW, G.buf(y), G.buf(x), G.buf(w), 1, 256, 5, ws)
+    d = torch.empty(4, dtype=torch.int32, device=G.DEV)
+    with pytest.raises(_lib.HipError):  # no integer route, so no block dots
+        kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
+    assert kernels.workspaceBytes(Q4K, 8, 4096, 4096) == 0
+
+
+def test_full_size_ffn_matrix_and_pair():
+    """Llama-3-8B FFN shapes in Q4_K (33 MB per matrix, as Q4_0): decode rows, a pair, scaling property."""
+    in_dim, out_dim = 4096, 14336
+    wa, wb = synth.weights(Q4K, 21, out_dim, in_dim), synth.weights(Q4K, 22, out_dim, in_dim)
+    da, db = G.to_dev(wa), G.to_dev(wb)
+    for rows in (1, 2, 4):
+        print(f"case: q4_k full size rows={rows}", flush=True)
+        x = synth.activations(30 + rows, rows, in_dim)
+        y = G.linear(Q4K, RAW, x, da, rows, in_dim, out_dim)
+        ref = O.linear_q4_k(x, wa, rows, in_dim, out_dim, f64=True)
+        err = G.max_rel_err(y, ref)
+        assert err <= TOL and err <= TIGHT, err
+        ya, yb = G.linear_pair(Q4K, RAW, x, da, db, rows, in_dim, out_dim)
+        assert np.array_equal(ya, y)
+        assert np.array_equal(yb, G.linear(Q4K, RAW, x, db, rows, in_dim, out_dim))
+        # every product scales exactly with a power of two
+        assert np.array_equal(G.linear(Q4K, RAW, x * 4.0, da, rows, in_dim, out_dim), y * 4.0)
+    # down projection: K = 14336
+    wd_ = synth.weights(Q4K, 23, 4096, 14336)
+    x = synth.activations(40, 1, 14336)
+    y = G.linear(Q4K, RAW, x, G.to_dev(wd_), 1, 14336, 4096)
+    assert G.max_rel_err(y, O.linear_q4_k(x, wd_, 1, 14336, 4096, f64=True)) <= TIGHT
+
+
+def test_backend_ops_on_q4_k():
+    in_dim, out_dim, rows = 512, 1000, 3
+    w = synth.weights(Q4K, 51, out_dim, in_dim)
+    x = synth.activations(52, rows, in_dim)
+    with HipCompute() as cb:
+        print("case: backend q4_k ops", flush=True)
+        cb.insertWeightFromLoaded("output.weight", Q4K, w, [out_dim, in_dim])
+        wt = cb.getWeight("output.weight")
+        assert wt.quant_type == Q4K and wt.layout == _lib.LAYOUT_RAW and wt.shape == [out_dim, in_dim]
+        xt = cb.fromFloat32(x, [rows, in_dim])
+        y = cb.toFloat32(cb.linearNoBias(xt, wt, rows, in_dim, out_dim)).reshape(rows, out_dim)
+        ref = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+        assert G.max_rel_err(y, ref) <= TIGHT
+        stats = cb.debugStats()
+        assert stats["launches_small_batch"] == 1 and stats["launches_activation_quant"] == 0 and stats["launches_prepare"] == 0
+        token = cb.linearNoBiasArgmaxLastRow(xt, wt, rows, in_dim, out_dim)
+        assert token == int(np.argmax(y[-1]))
+        assert token == O.argmax(ref[-1].astype(np.float32)) or ref[-1].max() - ref[-1][token] <= TIGHT * np.abs(ref[-1]).max()
+        emb = cb.toFloat32(cb.embeddingLookup(wt, [999, 0], 2, in_dim)).reshape(2, in_dim)
+        assert np.array_equal(emb.view(np.uint32), O.dequantize_q4_k(w).reshape(out_dim, in_dim)[[999, 0]].view(np.uint32))
+        with pytest.raises(_lib.InvalidHipState):
+            cb.linearNoBias(cb.fromFloat32(x[:, :128].copy(), [rows, 128]), wt, rows, 128, out_dim * 4)  # K not whole super-blocks

@@ -79,7 +79,7 @@ def test_embedding_lookup_dense_table_and_checks():
     with pytest.raises(_lib.InvalidHipState):  # short id buffer
         kernels.launchEmbeddingLookupF32(G.stream(), Q8, RAW, G.buf(o), G.buf(w), G.buf(idd[:1]), 2, 64, 4)
     with pytest.raises(_lib.UnsupportedTensorType):
-        kernels.launchEmbeddingLookupF32(G.stream(), 12, RAW, G.buf(o), G.buf(w), G.buf(idd), 2, 64, 4)
+        kernels.launchEmbeddingLookupF32(G.stream(), 14, RAW, G.buf(o), G.buf(w), G.buf(idd), 2, 64, 4)
 
 
 def rows_for_quantizer(seed, rows, dim):

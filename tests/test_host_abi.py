@@ -51,7 +51,10 @@ def test_dispatch_buckets_match_reference(kats):
     p = qm.plan(qm.Shape(5, 14336, 4096, qm.Format.q4_0))
     assert (p.dispatch, p.row_bucket, p.rows, p.in_dim, p.out_dim) == (qm.DispatchKind.small_batch, qm.RowBucket.rows_2_8, 5, 14336, 4096)
     assert qm.formatFromTensorType(2) == qm.Format.q4_0 and qm.formatFromTensorType(8) == qm.Format.q8_0
-    assert qm.formatFromTensorType(12) == qm.Format.unknown
+    assert qm.formatFromTensorType(12) == qm.Format.q4_k and qm.formatFromTensorType(14) == qm.Format.unknown
+    # Q4_K: K must be whole 256-value super-blocks
+    assert qm.select(qm.Shape(1, 128, 64, qm.Format.q4_k)) == qm.DispatchKind.scalar
+    assert qm.select(qm.Shape(3, 512, 64, qm.Format.q4_k)) == qm.DispatchKind.small_batch
 
 
 def test_route_gate_matches_cpu_engine():
@@ -84,7 +87,11 @@ def test_launcher_argument_checks_before_any_launch():
         with pytest.raises(_lib.InvalidHipState):
             fn(None, big, big, big, 1 << 62, 32, 1 << 10)
     with pytest.raises(_lib.UnsupportedTensorType):
-        kernels.launchLinearF32(None, 12, 0, big, big, big, 1, 256, 8)  # Q4_K is another operator
+        kernels.launchLinearF32(None, 14, 0, big, big, big, 1, 256, 8)  # Q6_K is another operator
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchLinearF32(None, 12, 0, big, big, big, 1, 128, 8)  # Q4_K: K must be whole super-blocks
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchLinearF32(None, 12, 0, big, big, Buffer(0x1000, 8 * 144 - 1), 1, 256, 8)
     # raw-layout activation-quantized route needs the caller's scratch
     assert kernels.workspaceBytes(2, 5, 14336, 4096) >= 5 * 14336 + 5 * 448 * 8
     assert kernels.workspaceBytes(2, 0, 14336, 4096) == 0

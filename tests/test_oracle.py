@@ -320,6 +320,70 @@ def test_timing_path_matches_faithful_path(fmt):
     p.close()
 
 
+# ---------------------------------------------------------------- Q4_K
+
+def q4k_block(d_bits, dmin_bits, scales12, qs128):
+    return np.concatenate([np.array([d_bits, dmin_bits], np.uint16).view(np.uint8), np.asarray(scales12, np.uint8),
+                           np.asarray(qs128, np.uint8)])
+
+
+def test_q4_k_reference_vectors(kats):
+    k = kats["q4_k"]
+    u = k["uniform_block"]
+    scales = [u["scales_first4"]] * 4 + [0] * 4 + [u["scales_last4"]] * 4
+    blk = q4k_block(u["d_bits"], 0, scales, [u["qs_fill"]] * 128)
+    assert np.abs(O.dequantize_q4_k(blk) - u["expect_all"]).max() <= u["tolerance_abs"]
+    m = k["direct_matmul"]
+    w = np.concatenate([q4k_block(15360, 0, scales, [f] * 128) for f in m["row_qs_fill"]])
+    x = np.full((1, m["in_dim"]), m["input_fill"], np.float32)
+    y = O.linear_q4_k(x, w, 1, m["in_dim"], m["out_dim"])
+    assert np.abs(y[0] - np.array(m["expected"])).max() <= m["tolerance_abs"]
+    # the reference's quantizer test fixes the bytes of a block whose values are scs*q - mins with d = dmin = 1:
+    # decoding those bytes must give the values back exactly (a wrong bit in the 6-bit unpack fails here)
+    h = k["header_packing"]
+    scs, mins = O.q4k_unpack_scale_mins(h["header"][4:16])
+    assert scs.tolist() == h["scs"] and mins.tolist() == h["mins"]
+    raw = np.array(h["header"] + h["qs_32"] * 4, np.uint8)
+    want = np.array([h["scs"][sub] * (i % 16) - h["mins"][sub] for sub in range(8) for i in range(32)], np.float32)
+    assert np.array_equal(O.dequantize_q4_k(raw), want)
+
+
+def numpy_dequantize_q4_k(raw):
+    """Independent restatement: published ggml Q4_K layout, vectorised."""
+    b = np.asarray(raw, np.uint8).reshape(-1, 144)
+    d = b[:, 0:2].copy().view(np.float16).astype(np.float32)[:, 0]
+    dmin = b[:, 2:4].copy().view(np.float16).astype(np.float32)[:, 0]
+    s = b[:, 4:16].astype(np.uint8)
+    sc = np.empty((b.shape[0], 8), np.uint8)
+    mn = np.empty((b.shape[0], 8), np.uint8)
+    sc[:, :4], mn[:, :4] = s[:, 0:4] & 63, s[:, 4:8] & 63
+    sc[:, 4:] = (s[:, 8:12] & 0x0F) | ((s[:, 0:4] >> 6) << 4)
+    mn[:, 4:] = (s[:, 8:12] >> 4) | ((s[:, 4:8] >> 6) << 4)
+    qs = b[:, 16:].reshape(-1, 4, 32)
+    q = np.stack([qs & 0x0F, qs >> 4], axis=2).reshape(-1, 8, 32).astype(np.float32)   # sub-blocks 2c, 2c+1
+    dsc = (d[:, None] * sc.astype(np.float32)).astype(np.float32)
+    dmn = (dmin[:, None] * mn.astype(np.float32)).astype(np.float32)
+    return ((dsc[:, :, None] * q).astype(np.float32) - dmn[:, :, None]).astype(np.float32).reshape(-1)
+
+
+def test_q4_k_against_independent_numpy_form():
+    w = synth.weights(synth.Q4_K, 3, 6, 512)
+    w[0:4] = np.array([0x0001, 0x7BFF], np.uint16).view(np.uint8)  # subnormal d, largest finite dmin
+    deq = O.dequantize_q4_k(w)
+    assert np.array_equal(deq.view(np.uint32), numpy_dequantize_q4_k(w).view(np.uint32))
+    x = synth.activations(4, 5, 512)
+    wf = np.nan_to_num(deq.reshape(6, 512).astype(np.float64), posinf=0, neginf=0)
+    w2 = synth.weights(synth.Q4_K, 5, 6, 512)
+    wf2 = O.dequantize_q4_k(w2).reshape(6, 512).astype(np.float64)
+    y64 = O.linear_q4_k(x, w2, 5, 512, 6, f64=True)
+    assert np.abs(y64 - x.astype(np.float64) @ wf2.T).max() <= 1e-12 * np.abs(y64).max() + 1e-15
+    y = O.linear_q4_k(x, w2, 5, 512, 6)
+    assert np.abs(y - y64).max() <= 2e-6 * np.abs(y64).max()
+    with pytest.raises(ValueError):
+        O.linear_q4_k(np.zeros((1, 128), np.float32), np.zeros(0, np.uint8), 1, 128, 0)
+    del wf
+
+
 # ---------------------------------------------------------------- greedy token pick
 
 def test_argmax_reference_vectors_and_properties(kats):
