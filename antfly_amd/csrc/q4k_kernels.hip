@@ -22,28 +22,33 @@ constexpr int kQ4kBlockValues = 256;
 
 typedef uint32_t q4k_u32x4 __attribute__((ext_vector_type(4)));
 
-// Byte k (0..11) of the 12 scale bytes held in header words 1..3.
-__device__ __forceinline__ uint32_t scale_byte(const q4k_u32x4& header, int k) {
-    const uint32_t word = k < 4 ? header.y : (k < 8 ? header.z : header.w);
-    return (word >> ((k & 3) * 8)) & 0xFFu;
-}
-
 // 6-bit scale and min of sub-block `sub` (unpackQ4KScaleMinsU8, ops/native_compute.zig:33745-33754).
+// With k = sub % 4 and a, b, c = bytes k, k + 4, k + 8 of the 12 scale bytes (byte k of
+// header words 1, 2, 3): sub < 4 -> (a & 63, b & 63); else -> ((c & 15) | (a >> 6) << 4,
+// (c >> 4) | (b >> 6) << 4).  No branches: `sub` differs from lane to lane.
 __device__ __forceinline__ void q4k_scale_min(const q4k_u32x4& header, int sub, float* sc, float* mn) {
-    uint32_t s, m;
-    if (sub < 4) {
-        s = scale_byte(header, sub) & 63u;
-        m = scale_byte(header, sub + 4) & 63u;
-    } else {
-        s = (scale_byte(header, sub + 4) & 0x0Fu) | ((scale_byte(header, sub - 4) >> 6) << 4);
-        m = (scale_byte(header, sub + 4) >> 4) | ((scale_byte(header, sub) >> 6) << 4);
-    }
+    const int shift = (sub & 3) * 8;
+    const uint32_t a = (header.y >> shift) & 0xFFu, b = (header.z >> shift) & 0xFFu, c = (header.w >> shift) & 0xFFu;
+    const bool low = sub < 4;
+    const uint32_t s = low ? (a & 63u) : ((c & 0x0Fu) | ((a >> 6) << 4));
+    const uint32_t m = low ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
     *sc = static_cast<float>(s);
     *mn = static_cast<float>(m);
 }
 
-__device__ __forceinline__ float byte_to_f32(uint32_t word, int index) {
-    return static_cast<float>((word >> (index * 8)) & 0xFFu);  // v_cvt_f32_ubyte0..3
+// Byte `kIndex` of `word` as a float: one v_cvt_f32_ubyteN (written out, because the
+// compiler extracts the byte with a separate instruction first).
+// Volatile, so that a value is converted where it is used instead of all of them up front;
+// `pass` tells conversions of different passes over the same weights apart (a second pass
+// with other rows converts again instead of keeping the first pass's values in registers).
+template <int kIndex>
+__device__ __forceinline__ float byte_to_f32(uint32_t word, int pass = 0) {
+    float out;
+    if (kIndex == 0) asm volatile("v_cvt_f32_ubyte0 %0, %1" : "=v"(out) : "v"(word), "n"(0), "s"(pass));
+    else if (kIndex == 1) asm volatile("v_cvt_f32_ubyte1 %0, %1" : "=v"(out) : "v"(word), "n"(0), "s"(pass));
+    else if (kIndex == 2) asm volatile("v_cvt_f32_ubyte2 %0, %1" : "=v"(out) : "v"(word), "n"(0), "s"(pass));
+    else asm volatile("v_cvt_f32_ubyte3 %0, %1" : "=v"(out) : "v"(word), "n"(0), "s"(pass));
+    return out;
 }
 
 }  // namespace
@@ -74,38 +79,46 @@ __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restr
         const float dsc = half_bits_to_f32(static_cast<uint16_t>(header.x & 0xFFFFu)) * sc;
         const float dmn = half_bits_to_f32(static_cast<uint16_t>(header.x >> 16)) * mn;
         float4 out;
-        out.x = dsc * byte_to_f32(nib, 0) - dmn;
-        out.y = dsc * byte_to_f32(nib, 1) - dmn;
-        out.z = dsc * byte_to_f32(nib, 2) - dmn;
-        out.w = dsc * byte_to_f32(nib, 3) - dmn;
+        out.x = dsc * byte_to_f32<0>(nib) - dmn;
+        out.y = dsc * byte_to_f32<1>(nib) - dmn;
+        out.z = dsc * byte_to_f32<2>(nib) - dmn;
+        out.w = dsc * byte_to_f32<3>(nib) - dmn;
         reinterpret_cast<float4*>(dst)[u] = out;
     }
 }
 
 // Y[r][o] = sum over K of x[r][k] * w[o][k] for kRows rows of f32 activations.
-// A wavefront owns kCols consecutive output columns and one K-slice of 16 super-blocks
-// (4096 values, two steps of 8 super-blocks); eight lanes share a super-block, each
-// with one 16-byte run of nibbles: 16 values of sub-block 2c (low nibbles) and the 16
-// values at the same positions of sub-block 2c+1 (high nibbles).  Per run the lane forms
+// A wavefront owns kCols consecutive output columns and one K-slice of 8 super-blocks
+// (2048 values); eight lanes share a super-block, each with one 16-byte run of nibbles:
+// 16 values of sub-block 2c (low nibbles) and the 16 values at the same positions of
+// sub-block 2c+1 (high nibbles).  Per run the lane forms
 //   dsc * sum(x * q) - dmn * sum(x)
-// which is the sum of x * (dsc * q - dmn) up to f32 rounding.  The weights of all
-// columns are requested at once, the activations (L2 hits) before them, so the
-// arithmetic of a column can run while later columns are still arriving.  K-slices meet
-// in LDS in slice order.  One or two rows per launch.
+// which is the sum of x * (dsc * q - dmn) up to f32 rounding.
+// The workgroup copies X into LDS first (coalesced); a lane then reads its 2 x 64 bytes
+// per row from LDS.  16-byte unit u of a row sits at (u & ~15) | ((u + (u >> 4 & 3) + 8 * (u >> 6 & 1)) & 15):
+// the 16 lanes of a read phase (two super-blocks x four chunks x two halves, same unit
+// within their runs) then hit 16 different bank groups.  The weights of all columns are
+// requested at once and consumed column by column in that order, so the arithmetic of
+// a column runs while later columns are still arriving.  K-slices meet in LDS in slice order.
+__device__ __forceinline__ int q4k_x_unit(int u) { return (u & ~15) | ((u + ((u >> 4) & 3) + 8 * ((u >> 6) & 1)) & 15); }
+
 template <int kRows, int kCols>
-__global__ __launch_bounds__(512) void gemv_q4k_kernel(float* __restrict__ dst, const float* __restrict__ x,
-                                                       const uint8_t* __restrict__ weight, int in_dim, int out_dim,
-                                                       int slices) {
-    constexpr int kSteps = 2;
+__global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void gemv_q4k_kernel(float* __restrict__ dst, const float* __restrict__ x,
+                                                                          const uint8_t* __restrict__ weight, int in_dim,
+                                                                          int out_dim, int slices) {
     constexpr int kCells = kRows * kCols;
-    static_assert(kRows <= 2, "the activations of both steps live in registers");
-    __shared__ float partial[8 * kCells];
+    constexpr int kXPre = 2;  // 16-byte units of a row of X a thread has in flight at once
+    extern __shared__ __align__(16) unsigned char lds[];
+    float4* xs = reinterpret_cast<float4*>(lds);                                   // [kRows][in_dim / 4], swizzled
+    float* partial = reinterpret_cast<float*>(xs + static_cast<size_t>(kRows) * (in_dim >> 2));  // [waves][kCells]
 
     const int kb = in_dim / kQ4kBlockValues;
+    const int row_units = in_dim >> 2;
     const int tid = threadIdx.x;
+    const int threads = blockDim.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int waves = blockDim.x >> 6;
+    const int waves = threads >> 6;
     const int slice = wave % slices;
     const int groups_per_wg = waves / slices;
     const int group = blockIdx.x * groups_per_wg + wave / slices;
@@ -113,108 +126,126 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(float* __restrict__ dst, 
     const bool active = o0 < out_dim;
     const int part = lane & 7;            // which 16-byte run of the super-block
     const int chunk = part >> 1;          // 64 values: sub-blocks 2c and 2c+1
-    const int run = (part & 1) * 16;      // first or second half of the chunk's 32 bytes
 
-    int sb[kSteps];
-    bool ok[kSteps];
+    const int b = slice * 8 + (lane >> 3);
+    const bool ok = active && b < kb;
+    const int sb = b < kb ? b : kb - 1;  // lanes past the row end re-read its last super-block and contribute nothing
+
+    // ---- 1. X into LDS (this thread's share; L2 hits after the first workgroups), then the
+    // requests for every weight byte of the wavefront.  Loads complete in order, so X is
+    // not requested behind the weights; other workgroups of the compute unit stream
+    // their weights while this one waits for X.
 #pragma unroll
-    for (int j = 0; j < kSteps; ++j) {
-        const int b = slice * (kSteps * 8) + j * 8 + (lane >> 3);
-        ok[j] = active && b < kb;
-        sb[j] = b < kb ? b : kb - 1;  // lanes past the row end re-read its last super-block and contribute nothing
+    for (int r = 0; r < kRows; ++r) {  // row by row: no division to find a unit's row
+        const float4* src = reinterpret_cast<const float4*>(x) + static_cast<size_t>(r) * row_units;
+        float4* dst_row = xs + r * row_units;
+        float4 xq[kXPre];
+#pragma unroll
+        for (int i = 0; i < kXPre; ++i) xq[i] = src[min(tid + i * threads, row_units - 1)];  // spare threads repeat the last unit
+#pragma unroll
+        for (int i = 0; i < kXPre; ++i) dst_row[q4k_x_unit(min(tid + i * threads, row_units - 1))] = xq[i];
+        for (int u = tid + kXPre * threads; u < row_units; u += threads) dst_row[q4k_x_unit(u)] = src[u];
     }
-
-    // this lane's activations: x[r][sb*256 + chunk*64 + run + 0..15] (with the low nibbles)
-    // and the same 16 positions 32 values further on (with the high nibbles)
-    float4 xv[kSteps][kRows][8];
-    auto load_x = [&](int j, float4 (&out)[kRows][8]) {
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-            const float4* p = reinterpret_cast<const float4*>(x + static_cast<size_t>(r) * in_dim + sb[j] * kQ4kBlockValues +
-                                                              chunk * 64 + run);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                out[r][i] = p[i];
-                out[r][4 + i] = p[8 + i];
-            }
-        }
-    };
-#pragma unroll
-    for (int j = 0; j < kSteps; ++j) load_x(j, xv[j]);
-    __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
-
-    q4k_u32x4 header[kSteps][kCols], quants[kSteps][kCols];
+    __builtin_amdgcn_sched_barrier(0);
+    q4k_u32x4 header[kCols], quants[kCols];
 #pragma unroll
     for (int c = 0; c < kCols; ++c) {
         const int o = min(o0 + c, out_dim - 1);  // columns past the end re-read the last one
-#pragma unroll
-        for (int j = 0; j < kSteps; ++j) {
-            const uint8_t* base = weight + (static_cast<size_t>(o) * kb + sb[j]) * kQ4kBlockBytes;
-            header[j][c] = __builtin_nontemporal_load(reinterpret_cast<const q4k_u32x4*>(base));
-            quants[j][c] = __builtin_nontemporal_load(reinterpret_cast<const q4k_u32x4*>(base + 16 + part * 16));
-        }
+        const uint8_t* base = weight + (static_cast<size_t>(o) * kb + sb) * kQ4kBlockBytes;
+        header[c] = __builtin_nontemporal_load(reinterpret_cast<const q4k_u32x4*>(base));
+        quants[c] = __builtin_nontemporal_load(reinterpret_cast<const q4k_u32x4*>(base + 16 + part * 16));
     }
+    __builtin_amdgcn_sched_barrier(0);
+    __syncthreads();
 
+    // ---- 2. column by column, two rows at a time
     float acc[kRows][kCols];
 #pragma unroll
     for (int r = 0; r < kRows; ++r)
 #pragma unroll
         for (int c = 0; c < kCols; ++c) acc[r][c] = 0.0f;
+    // this lane's activations: x[r][sb*256 + chunk*64 + (part&1)*16 + 0..15] (with the low
+    // nibbles) and the same 16 positions 32 values further on (with the high nibbles)
+    const int first_unit = sb * 64 + chunk * 16 + (part & 1) * 4;
 
-    auto consume = [&](int j, int c, const float4 (&xs)[kRows][8], const float (&xsum)[kRows][2]) {
-        const q4k_u32x4 h = header[j][c];
-        float sc0, mn0, sc1, mn1;
-        q4k_scale_min(h, chunk * 2, &sc0, &mn0);
-        q4k_scale_min(h, chunk * 2 + 1, &sc1, &mn1);
-        const float d = ok[j] ? half_bits_to_f32(static_cast<uint16_t>(h.x & 0xFFFFu)) : 0.0f;
-        const float dmin = ok[j] ? half_bits_to_f32(static_cast<uint16_t>(h.x >> 16)) : 0.0f;
-        const float dsc0 = d * sc0, dmn0 = dmin * mn0, dsc1 = d * sc1, dmn1 = dmin * mn1;
-        const uint32_t w[4] = {quants[j][c].x, quants[j][c].y, quants[j][c].z, quants[j][c].w};
-        float lo[16], hi[16];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t l = w[i] & 0x0F0F0F0Fu, hgh = (w[i] >> 4) & 0x0F0F0F0Fu;
+    for (int r0 = 0; r0 < kRows; r0 += 2) {
+        constexpr int kPairMax = 2;
+        const int pair = kRows - r0 < kPairMax ? kRows - r0 : kPairMax;  // compile-time after unrolling
+        float4 xv[kPairMax][8];
+        float xsum[kPairMax][2];
 #pragma unroll
-            for (int b = 0; b < 4; ++b) {
-                lo[4 * i + b] = byte_to_f32(l, b);
-                hi[4 * i + b] = byte_to_f32(hgh, b);
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-            float s0 = 0.0f, s1 = 0.0f;
+        for (int rr = 0; rr < kPairMax; ++rr) {
+            if (rr >= pair) continue;
+            const float4* row = xs + (r0 + rr) * row_units;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                s0 += xs[r][i].x * lo[4 * i] + xs[r][i].y * lo[4 * i + 1] + xs[r][i].z * lo[4 * i + 2] + xs[r][i].w * lo[4 * i + 3];
-                s1 += xs[r][4 + i].x * hi[4 * i] + xs[r][4 + i].y * hi[4 * i + 1] + xs[r][4 + i].z * hi[4 * i + 2] +
-                      xs[r][4 + i].w * hi[4 * i + 3];
+                xv[rr][i] = row[q4k_x_unit(first_unit + i)];
+                xv[rr][4 + i] = row[q4k_x_unit(first_unit + 8 + i)];
             }
-            acc[r][c] += (dsc0 * s0 - dmn0 * xsum[r][0]) + (dsc1 * s1 - dmn1 * xsum[r][1]);
-        }
-    };
-    auto sums_of = [&](const float4 (&xs)[kRows][8], float (&xsum)[kRows][2]) {
-#pragma unroll
-        for (int r = 0; r < kRows; ++r) {
-            float a = 0.0f, b = 0.0f;
+            float a = 0.0f, bsum = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                a += (xs[r][i].x + xs[r][i].y) + (xs[r][i].z + xs[r][i].w);
-                b += (xs[r][4 + i].x + xs[r][4 + i].y) + (xs[r][4 + i].z + xs[r][4 + i].w);
+                a += (xv[rr][i].x + xv[rr][i].y) + (xv[rr][i].z + xv[rr][i].w);
+                bsum += (xv[rr][4 + i].x + xv[rr][4 + i].y) + (xv[rr][4 + i].z + xv[rr][4 + i].w);
             }
-            xsum[r][0] = a;
-            xsum[r][1] = b;
+            xsum[rr][0] = a;
+            xsum[rr][1] = bsum;
         }
-    };
+#pragma unroll
+        for (int c = 0; c < kCols; ++c) {  // the order the weight loads were issued in
+            const q4k_u32x4 h = header[c];
+            // every lane of the super-block's eight unpacks one sub-block (its own index) and
+            // takes the pair it needs, 2 * chunk and 2 * chunk + 1, from its neighbour
+            float sc, mn;
+            q4k_scale_min(h, part, &sc, &mn);
+            const float d = ok ? half_bits_to_f32(static_cast<uint16_t>(h.x & 0xFFFFu)) : 0.0f;
+            const float dmin = ok ? half_bits_to_f32(static_cast<uint16_t>(h.x >> 16)) : 0.0f;
+            const float dsc = d * sc, dmn = dmin * mn;
+            const float dsc_other = dpp_move<kDppXor1>(dsc), dmn_other = dpp_move<kDppXor1>(dmn);
+            const bool odd = (part & 1) != 0;
+            const float dsc0 = odd ? dsc_other : dsc, dsc1 = odd ? dsc : dsc_other;
+            const float dmn0 = odd ? dmn_other : dmn, dmn1 = odd ? dmn : dmn_other;
+            const uint32_t w[4] = {quants[c].x, quants[c].y, quants[c].z, quants[c].w};
+            // fused multiply-adds, four independent chains per half run (the engine's own sums
+            // are only defined up to rounding order)
+            float s0[kPairMax][4], s1[kPairMax][4];
+#pragma unroll
+            for (int rr = 0; rr < kPairMax; ++rr)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) s0[rr][k] = s1[rr][k] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // four bytes at a time: eight converted values live
+                const uint32_t l = w[i] & 0x0F0F0F0Fu, hgh = (w[i] >> 4) & 0x0F0F0F0Fu;
+                const float l0 = byte_to_f32<0>(l, r0), l1 = byte_to_f32<1>(l, r0), l2 = byte_to_f32<2>(l, r0), l3 = byte_to_f32<3>(l, r0);
+                const float h0 = byte_to_f32<0>(hgh, r0), h1 = byte_to_f32<1>(hgh, r0), h2 = byte_to_f32<2>(hgh, r0),
+                            h3 = byte_to_f32<3>(hgh, r0);
+#pragma unroll
+                for (int rr = 0; rr < kPairMax; ++rr) {
+                    if (rr >= pair) continue;
+                    s0[rr][0] = __builtin_fmaf(xv[rr][i].x, l0, s0[rr][0]);
+                    s0[rr][1] = __builtin_fmaf(xv[rr][i].y, l1, s0[rr][1]);
+                    s0[rr][2] = __builtin_fmaf(xv[rr][i].z, l2, s0[rr][2]);
+                    s0[rr][3] = __builtin_fmaf(xv[rr][i].w, l3, s0[rr][3]);
+                    s1[rr][0] = __builtin_fmaf(xv[rr][4 + i].x, h0, s1[rr][0]);
+                    s1[rr][1] = __builtin_fmaf(xv[rr][4 + i].y, h1, s1[rr][1]);
+                    s1[rr][2] = __builtin_fmaf(xv[rr][4 + i].z, h2, s1[rr][2]);
+                    s1[rr][3] = __builtin_fmaf(xv[rr][4 + i].w, h3, s1[rr][3]);
+                }
+            }
+#pragma unroll
+            for (int rr = 0; rr < kPairMax; ++rr) {
+                if (rr >= pair) continue;
+                const float t0 = (s0[rr][0] + s0[rr][1]) + (s0[rr][2] + s0[rr][3]);
+                const float t1 = (s1[rr][0] + s1[rr][1]) + (s1[rr][2] + s1[rr][3]);
+                acc[r0 + rr][c] += (dsc0 * t0 - dmn0 * xsum[rr][0]) + (dsc1 * t1 - dmn1 * xsum[rr][1]);
+            }
+            // nothing of the next column is to move up here: it would wait for that column's bytes
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
 
-    float xsum[kSteps][kRows][2];
-#pragma unroll
-    for (int j = 0; j < kSteps; ++j) sums_of(xv[j], xsum[j]);
-#pragma unroll
-    for (int c = 0; c < kCols; ++c)  // the order the weight loads were issued in
-#pragma unroll
-        for (int j = 0; j < kSteps; ++j) consume(j, c, xv[j], xsum[j]);
-
-    // wavefront reduction of all rows x columns at once
+    // ---- 3. wavefront reduction of all rows x columns at once
     constexpr int kPadded = kCells <= 1 ? 1 : (kCells <= 2 ? 2 : (kCells <= 4 ? 4 : (kCells <= 8 ? 8 : 16)));
     static_assert(kCells <= 16, "at most 16 accumulators per lane");
     float red[kPadded];
@@ -231,7 +262,7 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(float* __restrict__ dst, 
     if (mine) partial[wave * kCells + cell] = red[0];
     __syncthreads();
     const int cells = groups_per_wg * kCells;
-    for (int i = tid; i < cells; i += blockDim.x) {
+    for (int i = tid; i < cells; i += threads) {
         const int gi = i / kCells, rc = i - gi * kCells;
         const int r = rc / kCols, c = rc - r * kCols;
         const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
@@ -243,34 +274,83 @@ __global__ __launch_bounds__(512) void gemv_q4k_kernel(float* __restrict__ dst, 
 
 namespace {
 
+int compute_unit_count() {
+    static const int units = []() {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return units;
+}
+
+constexpr int kQ4kMaxSlices = 8;  // 8 x 2048 values
+
+size_t q4k_lds_bytes(int rows, int in_dim) { return static_cast<size_t>(rows) * in_dim * 4 + 16 * 16 * 4; }
+
 template <int kRows>
 hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int in_dim, int out_dim) {
-    constexpr int kCols = 4;
+    constexpr int kCols = 2;
     const int kb = in_dim / kQ4kBlockValues;
-    const int slices = (kb + 15) / 16;
-    if (slices > 8) return hipErrorInvalidValue;
-    const int waves = 8 / slices * slices;
-    const int groups_per_wg = waves / slices;
     const int groups = (out_dim + kCols - 1) / kCols;
+    const int slices = (kb + 7) / 8;
+    if (slices > kQ4kMaxSlices) return hipErrorInvalidValue;
+    // 8 wavefronts a workgroup (one row: two workgroups share a compute unit, so that one computes
+    // while the other waits for its weights); among the sizes down to half of that, the one whose
+    // grid leaves the busiest compute unit the least work
+    constexpr int kMaxWaves = 8;
+    int limit = kMaxWaves / slices * slices;
+    if (limit == 0) limit = slices;  // a long K: one column group per workgroup
+    if (limit > kMaxWaves) return hipErrorInvalidValue;
+    const int units = compute_unit_count();
+    int waves = limit;
+    long best = -1;
+    for (int w = limit; w >= slices && 2 * w > limit; w -= slices) {
+        const long g = (groups + w / slices - 1) / (w / slices);
+        const long cost = (g + units - 1) / units * w;
+        if (best < 0 || cost < best) {
+            best = cost;
+            waves = w;
+        }
+    }
+    const int groups_per_wg = waves / slices;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
-    hipLaunchKernelGGL((gemv_q4k_kernel<kRows, kCols>), dim3(grid), dim3(waves * 64), 0, stream, dst, x, weight, in_dim,
-                       out_dim, slices);
+    const size_t lds = q4k_lds_bytes(kRows, in_dim);
+    auto kernel = gemv_q4k_kernel<kRows, kCols>;
+    static bool large_lds = false;  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    if (lds > 64 * 1024 && !large_lds) {
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            e != hipSuccess)
+            return e;
+        large_lds = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, in_dim, out_dim, slices);
     return hipGetLastError();
 }
 
 }  // namespace
 
-int gemv_q4k_max_in_dim() { return 8 * 16 * kQ4kBlockValues; }
+// 8 wavefronts a workgroup, one slice of 2048 values each at most.
+int gemv_q4k_max_in_dim() { return 8 * 8 * kQ4kBlockValues; }
 
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                            int out_dim) {
     if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
-    // two rows per launch; more rows walk the weights again (from the Infinity Cache when the matrix fits)
-    for (int r0 = 0; r0 < rows; r0 += 2) {
+    // up to four rows per launch while X fits LDS; more rows walk the weights again (from the
+    // Infinity Cache when the matrix fits)
+    int per_launch = 4;
+    while (per_launch > 1 && q4k_lds_bytes(per_launch, in_dim) > 144 * 1024) --per_launch;
+    for (int r0 = 0; r0 < rows; r0 += per_launch) {
+        const int nr = rows - r0 < per_launch ? rows - r0 : per_launch;
         float* d = dst + static_cast<size_t>(r0) * out_dim;
         const float* xr = x + static_cast<size_t>(r0) * in_dim;
-        const hipError_t e = rows - r0 >= 2 ? launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim)
-                                            : launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim);
+        hipError_t e;
+        switch (nr) {
+            case 1: e = launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim); break;
+            case 2: e = launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim); break;
+            case 3: e = launch_q4k_rows<3>(stream, d, xr, weight, in_dim, out_dim); break;
+            default: e = launch_q4k_rows<4>(stream, d, xr, weight, in_dim, out_dim); break;
+        }
         if (e != hipSuccess) return e;
     }
     return hipSuccess;

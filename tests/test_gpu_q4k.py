@@ -66,7 +66,7 @@ def test_dequantize_and_get_rows_bit_exact(rows, dim):
 
 
 SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130), (3, 1024, 40), (5, 4096, 96),
-          (1, 14336, 48), (2, 14336, 20), (9, 2048, 24), (1, 32768, 8)]
+          (1, 14336, 48), (2, 14336, 20), (9, 2048, 24), (1, 16384, 8), (3, 16384, 12), (4, 14336, 8)]
 
 
 @pytest.mark.parametrize("rows,in_dim,out_dim", SHAPES)
@@ -95,6 +95,10 @@ def test_linear_argument_checks():
     with pytest.raises(_lib.HipError):  # no integer route, so no block dots
         kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
     assert kernels.workspaceBytes(Q4K, 8, 4096, 4096) == 0
+    big_w = torch.zeros(4 * 128 * 144, dtype=torch.uint8, device=G.DEV)
+    big_x = torch.zeros(32768, dtype=torch.float32, device=G.DEV)
+    with pytest.raises(_lib.HipOpUnsupported):  # K beyond what one workgroup's slices cover
+        kernels.launchLinearF32(G.stream(), Q4K, RAW, G.buf(y), G.buf(big_x), G.buf(big_w), 1, 32768, 4, ws)
 
 
 def test_full_size_ffn_matrix_and_pair():
