@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_BPS = 8.0e12           # MI355X HBM3E
 INT8_MFMA_PEAK_OPS = 5.0e15     # MI355X dense int8 MFMA
-Q4, Q8 = 2, 8
+Q4, Q8, Q4K = 2, 8, 12
 BLOCK_BYTES = {Q4: 18, Q8: 34}
 
 
@@ -89,7 +89,10 @@ def main() -> int:
         out = []
         for _ in range(copies):
             p = torch.empty_like(raw)
-            kernels.launchPrepareWeight(stream, fmt, buf(p), buf(raw), out_dim, in_dim)
+            if fmt == Q4K:
+                p.copy_(raw)  # Q4_K is computed on the raw layout
+            else:
+                kernels.launchPrepareWeight(stream, fmt, buf(p), buf(raw), out_dim, in_dim)
             out.append(p)
         torch.cuda.synchronize()
         return out
@@ -380,6 +383,14 @@ def main() -> int:
             w_s, e_s = time_config(fmt, r, k, n, small_steps, 20, copies, 99)
             b = gemv_bytes(fmt, r, k, n)
             extra[name] = {"us_per_call": round(e_s / small_steps * 1e6, 3),
+                           "GBps": round(b * small_steps / e_s / 1e9, 1),
+                           "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
+        for name, r, k, n in [("q4k_gemv_m1_k4096_n14336", 1, 4096, 14336), ("q4k_gemv_m2_k4096_n14336", 2, 4096, 14336),
+                              ("q4k_gemv_m1_k14336_n4096", 1, 14336, 4096)]:
+            w_s, e_s = time_config(Q4K, r, k, n, small_steps, 20, args.copies, 77)
+            b = n * (k // 256) * 144 + 4 * r * (k + n)
+            extra[name] = {"what": "Q4_K (144-byte super-blocks), f32 activations against the dequantized weights",
+                           "us_per_call": round(e_s / small_steps * 1e6, 3),
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
         for m in (128, 512, 2048):
