@@ -110,6 +110,8 @@ SIGNATURES = {
     "afhip_linear_workspace_bytes": (_sz, [_i, _sz, _sz, _sz]),
     "afhip_launch_linear_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_pair_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_linear_bias_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_linear_pair_bias_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_q8_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_linear_q4_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_prepare_weight": (_st, [_vp, _i, Buffer, Buffer, _sz, _sz]),
@@ -149,6 +151,9 @@ SIGNATURES = {
     "afhip_compute_embedding_lookup": (_st, [_vp, _vp, C.POINTER(C.c_int64), _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_pair": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
+    "afhip_compute_linear": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "afhip_compute_linear_pair": (_st, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
+    "afhip_compute_linear_triple": (_st, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_grouped": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32), _sz, C.POINTER(_vp)]),
     "afhip_compute_argmax_last_row": (_st, [_vp, _vp, _sz, _sz, C.POINTER(C.c_uint32)]),
     "afhip_compute_linear_no_bias_argmax_last_row": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32)]),

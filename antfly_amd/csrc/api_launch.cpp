@@ -84,7 +84,8 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
 // Q4_K: f32 activations against the dequantized weights, one kernel family for any row count.
 static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                     size_t rows, size_t in_dim, size_t out_dim, int dispatch, bool want_dots,
-                                    LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b) {
+                                    LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b,
+                                    afhip_buffer bias, afhip_buffer bias_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // this format has no integer route
     if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -113,7 +114,8 @@ static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_
         hipError_t e = launch_gemv_q4k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
                                        reinterpret_cast<const float*>(input.ptr),
                                        reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
-                                       static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+                                       static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
+                                       reinterpret_cast<const float*>(i ? bias_b.ptr : bias.ptr));
         if (e != hipSuccess) return static_cast<afhip_status>(e);
     }
     return AFHIP_OK;
@@ -122,12 +124,21 @@ static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_
 afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
                          int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
-                         afhip_buffer weight_b) {
+                         afhip_buffer weight_b, afhip_buffer bias, afhip_buffer bias_b) {
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
+    // biases: f32 [out_dim]; the second one only with a second matrix, none with the block dots
+    if ((bias_b.ptr != 0 && !pair) || ((bias.ptr != 0 || bias_b.ptr != 0) && dots.ptr != 0)) return AFHIP_ERR_INVALID_ARGUMENT;
+    for (const afhip_buffer& b : {bias, bias_b}) {
+        size_t need;
+        if (b.ptr == 0) continue;
+        if (b.ptr % 4 != 0 || !checked_mul(out_dim, 4, &need) || b.len < need) return AFHIP_ERR_INVALID_STATE;
+    }
+    const float* add = reinterpret_cast<const float*>(bias.ptr);
+    const float* add_b = reinterpret_cast<const float*>(bias_b.ptr);
     if (tensor_type == AFHIP_TYPE_Q4_K)
         return linear_q4k_impl(stream, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters, dst_b,
-                               weight_b);
+                               weight_b, bias, bias_b);
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -175,11 +186,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     if (!route_a) {
         if (counters) counters->f32_route++;
         hipError_t e = launch_linear_generic(stream, tensor_type, layout, false, y, nullptr, x, nullptr, nullptr, w,
-                                             static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+                                             static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add);
         if (e == hipSuccess && pair) {
             if (counters) counters->f32_route++;
             e = launch_linear_generic(stream, tensor_type, layout, false, y_b, nullptr, x, nullptr, nullptr, w_b,
-                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
@@ -201,11 +212,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                                                    ws.sx, ws.sums);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
         e = launch_gemm_i8(stream, tensor_type, want_dots ? nullptr : y, dot_out, ws.qx, ws.sx, w, static_cast<int>(rows),
-                           static_cast<int>(in_dim), static_cast<int>(out_dim));
+                           static_cast<int>(in_dim), static_cast<int>(out_dim), add);
         if (e == hipSuccess && pair) {  // the second matrix reuses the quantized activations
             if (counters) counters->mm++;
             e = launch_gemm_i8(stream, tensor_type, y_b, nullptr, ws.qx, ws.sx, w_b, static_cast<int>(rows),
-                               static_cast<int>(in_dim), static_cast<int>(out_dim));
+                               static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
@@ -245,7 +256,7 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
             hipError_t e = launch_gemv_fused(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
                                              want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, pre, w,
                                              nr, static_cast<int>(in_dim), static_cast<int>(out_dim), tune,
-                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr);
+                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr, add, add_b);
             if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         return AFHIP_OK;
@@ -264,10 +275,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                                                ws.sums);
     if (e != hipSuccess) return static_cast<afhip_status>(e);
     e = launch_linear_generic(stream, tensor_type, layout, true, want_dots ? nullptr : y, dot_out, nullptr, ws.qx, ws.sx,
-                              w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+                              w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add);
     if (e == hipSuccess && pair)
         e = launch_linear_generic(stream, tensor_type, layout, true, y_b, nullptr, nullptr, ws.qx, ws.sx, w_b,
-                                  static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+                                  static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
@@ -478,6 +489,25 @@ afhip_status afhip_launch_linear_pair_f32(void* stream, int tensor_type, int lay
     if (weight_b.ptr == 0 || (dst_b.ptr == 0 && rows != 0 && out_dim != 0)) return AFHIP_ERR_INVALID_STATE;
     return linear_impl(stream, tensor_type, layout, dst_a, input, weight_a, rows, in_dim, out_dim, workspace, dispatch,
                        afhip_buffer{0, 0}, nullptr, dst_b, weight_b);
+}
+
+afhip_status afhip_launch_linear_bias_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                                          afhip_buffer weight, afhip_buffer bias, size_t rows, size_t in_dim,
+                                          size_t out_dim, afhip_buffer workspace, int dispatch) {
+    if (bias.ptr == 0 && out_dim != 0) return AFHIP_ERR_INVALID_STATE;
+    return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr, afhip_buffer{0, 0}, afhip_buffer{0, 0}, bias);
+}
+
+afhip_status afhip_launch_linear_pair_bias_f32(void* stream, int tensor_type, int layout, afhip_buffer dst_a,
+                                               afhip_buffer dst_b, afhip_buffer input, afhip_buffer weight_a,
+                                               afhip_buffer bias_a, afhip_buffer weight_b, afhip_buffer bias_b,
+                                               size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                               int dispatch) {
+    if (weight_b.ptr == 0 || (dst_b.ptr == 0 && rows != 0 && out_dim != 0)) return AFHIP_ERR_INVALID_STATE;
+    if ((bias_a.ptr == 0 || bias_b.ptr == 0) && out_dim != 0) return AFHIP_ERR_INVALID_STATE;
+    return linear_impl(stream, tensor_type, layout, dst_a, input, weight_a, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr, dst_b, weight_b, bias_a, bias_b);
 }
 
 afhip_status afhip_launch_linear_q8_0_f32(void* stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight_raw,

@@ -159,13 +159,20 @@ afhip_status make_f32_result(afhip_compute* self, afhip_buffer device, size_t ro
 // the input (the weights must have the same format and layout to share one launch).
 afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
                                  size_t rows, size_t in_dim, size_t out_dim, int dispatch, afhip_tensor** out,
-                                 const afhip_tensor* weight_b = nullptr, afhip_tensor** out_b = nullptr) {
-    // cuda_compute.zig:689-717
+                                 const afhip_tensor* weight_b = nullptr, afhip_tensor** out_b = nullptr,
+                                 const afhip_tensor* bias = nullptr, const afhip_tensor* bias_b = nullptr) {
+    // cuda_compute.zig:689-717; with biases (f32 [out_dim], added to every row): linear :544-575, linearPair :799-815
     const bool pair = weight_b != nullptr || out_b != nullptr;
-    if (!self || !input || !weight || !out || (pair && (!weight_b || !out_b))) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (!self || !input || !weight || !out || (pair && (!weight_b || !out_b)) || (bias_b && !pair))
+        return AFHIP_ERR_INVALID_ARGUMENT;
     *out = nullptr;
     if (pair) *out_b = nullptr;
     if (!is_f32(input)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+    for (const afhip_tensor* b : {bias, bias_b}) {
+        if (!b) continue;
+        if (!is_f32(b)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
+        if (b->elem_count != out_dim) return AFHIP_ERR_INVALID_SHAPE;
+    }
     const afhip_tensor* ws[2] = {weight, weight_b};
     size_t in_count, w_count, out_count, out_bytes;
     if (!checked_mul(rows, in_dim, &in_count) || !checked_mul(out_dim, in_dim, &w_count) ||
@@ -182,9 +189,9 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
     }
     if (pair && (weight_b->quant_type != weight->quant_type || weight_b->layout != weight->layout)) {
         // nothing to share: two independent ops, as the engine's wrapper does (ops/ops.zig:1828-1849)
-        afhip_status s = linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, dispatch, out);
+        afhip_status s = linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, dispatch, out, nullptr, nullptr, bias);
         if (s != AFHIP_OK) return s;
-        s = linear_no_bias_impl(self, input, weight_b, rows, in_dim, out_dim, dispatch, out_b);
+        s = linear_no_bias_impl(self, input, weight_b, rows, in_dim, out_dim, dispatch, out_b, nullptr, nullptr, bias_b);
         if (s != AFHIP_OK) {
             free_tensor_storage(self, *out);
             delete *out;
@@ -212,7 +219,8 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
     if (s == AFHIP_OK) {
         s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows,
                         in_dim, out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
-                        pair ? weight_b->buffer : afhip_buffer{0, 0});
+                        pair ? weight_b->buffer : afhip_buffer{0, 0}, bias ? bias->buffer : afhip_buffer{0, 0},
+                        bias_b ? bias_b->buffer : afhip_buffer{0, 0});
     }
     if (s != AFHIP_OK) {
         release_device_buffer(self, &device);
@@ -534,6 +542,45 @@ afhip_status afhip_compute_linear_no_bias_pair(afhip_compute* self, const afhip_
                                                afhip_tensor** out_second) {
     if (!weight_b || !out_second) return AFHIP_ERR_INVALID_ARGUMENT;
     return linear_no_bias_impl(self, input, weight_a, rows, in_dim, out_dim, -1, out_first, weight_b, out_second);
+}
+
+afhip_status afhip_compute_linear(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
+                                  const afhip_tensor* bias, size_t rows, size_t in_dim, size_t out_dim,
+                                  afhip_tensor** out) {
+    if (!bias) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out, nullptr, nullptr, bias);
+}
+
+afhip_status afhip_compute_linear_pair(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight_a,
+                                       const afhip_tensor* bias_a, const afhip_tensor* weight_b,
+                                       const afhip_tensor* bias_b, size_t rows, size_t in_dim, size_t out_dim,
+                                       afhip_tensor** out_first, afhip_tensor** out_second) {
+    if (!weight_b || !out_second || !bias_a || !bias_b) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_no_bias_impl(self, input, weight_a, rows, in_dim, out_dim, -1, out_first, weight_b, out_second, bias_a,
+                               bias_b);
+}
+
+afhip_status afhip_compute_linear_triple(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight_a,
+                                         const afhip_tensor* bias_a, const afhip_tensor* weight_b,
+                                         const afhip_tensor* bias_b, const afhip_tensor* weight_c,
+                                         const afhip_tensor* bias_c, size_t rows, size_t in_dim, size_t out_dim,
+                                         afhip_tensor** out_first, afhip_tensor** out_second,
+                                         afhip_tensor** out_third) {
+    // Q/K/V with separate weights: the first two share one launch where a pair does, the third follows
+    if (!out_third || !weight_c || !bias_c) return AFHIP_ERR_INVALID_ARGUMENT;
+    *out_third = nullptr;
+    afhip_status s = afhip_compute_linear_pair(self, input, weight_a, bias_a, weight_b, bias_b, rows, in_dim, out_dim,
+                                               out_first, out_second);
+    if (s != AFHIP_OK) return s;
+    s = afhip_compute_linear(self, input, weight_c, bias_c, rows, in_dim, out_dim, out_third);
+    if (s != AFHIP_OK) {
+        for (afhip_tensor** t : {out_first, out_second}) {
+            free_tensor_storage(self, *t);
+            delete *t;
+            *t = nullptr;
+        }
+    }
+    return s;
 }
 
 afhip_status afhip_compute_linear_no_bias_grouped(afhip_compute* self, const afhip_tensor* input,

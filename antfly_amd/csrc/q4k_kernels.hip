@@ -105,7 +105,8 @@ __device__ __forceinline__ int q4k_x_unit(int u) { return (u & ~15) | ((u + ((u 
 template <int kRows, int kCols>
 __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void gemv_q4k_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                                           const uint8_t* __restrict__ weight, int in_dim,
-                                                                          int out_dim, int slices) {
+                                                                          int out_dim, int slices,
+                                                                          const float* __restrict__ bias) {
     constexpr int kCells = kRows * kCols;
     constexpr int kXPre = 2;  // 16-byte units of a row of X a thread has in flight at once
     extern __shared__ __align__(16) unsigned char lds[];
@@ -256,7 +257,8 @@ __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void ge
     const int cr = cell / kCols, cc = cell % kCols;
     const bool mine = lane < kPadded && cell < kCells;
     if (slices == 1) {
-        if (active && mine && o0 + cc < out_dim) dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = red[0];
+        if (active && mine && o0 + cc < out_dim)
+            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = bias != nullptr ? red[0] + bias[o0 + cc] : red[0];
         return;
     }
     if (mine) partial[wave * kCells + cell] = red[0];
@@ -268,7 +270,7 @@ __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void ge
         const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
-        if (o < out_dim) dst[static_cast<size_t>(r) * out_dim + o] = total;
+        if (o < out_dim) dst[static_cast<size_t>(r) * out_dim + o] = bias != nullptr ? total + bias[o] : total;
     }
 }
 
@@ -289,7 +291,8 @@ constexpr int kQ4kMaxSlices = 8;  // 8 x 2048 values
 size_t q4k_lds_bytes(int rows, int in_dim) { return static_cast<size_t>(rows) * in_dim * 4 + 16 * 16 * 4; }
 
 template <int kRows>
-hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int in_dim, int out_dim) {
+hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int in_dim, int out_dim,
+                           const float* bias) {
     constexpr int kCols = 2;
     const int kb = in_dim / kQ4kBlockValues;
     const int groups = (out_dim + kCols - 1) / kCols;
@@ -324,7 +327,7 @@ hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const
             return e;
         large_lds = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, in_dim, out_dim, slices);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, in_dim, out_dim, slices, bias);
     return hipGetLastError();
 }
 
@@ -334,7 +337,7 @@ hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const
 int gemv_q4k_max_in_dim() { return 8 * 8 * kQ4kBlockValues; }
 
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                           int out_dim) {
+                           int out_dim, const float* bias) {
     if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
     // up to four rows per launch while X fits LDS; more rows walk the weights again (from the
     // Infinity Cache when the matrix fits)
@@ -346,10 +349,10 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
         const float* xr = x + static_cast<size_t>(r0) * in_dim;
         hipError_t e;
         switch (nr) {
-            case 1: e = launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim); break;
-            case 2: e = launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim); break;
-            case 3: e = launch_q4k_rows<3>(stream, d, xr, weight, in_dim, out_dim); break;
-            default: e = launch_q4k_rows<4>(stream, d, xr, weight, in_dim, out_dim); break;
+            case 1: e = launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim, bias); break;
+            case 2: e = launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim, bias); break;
+            case 3: e = launch_q4k_rows<3>(stream, d, xr, weight, in_dim, out_dim, bias); break;
+            default: e = launch_q4k_rows<4>(stream, d, xr, weight, in_dim, out_dim, bias); break;
         }
         if (e != hipSuccess) return e;
     }

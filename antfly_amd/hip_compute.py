@@ -178,6 +178,31 @@ class HipCompute:
                                                            in_dim, out_dim, C.byref(ha), C.byref(hb)))
         return HipTensor(ha.value), HipTensor(hb.value)
 
+    def linear(self, input: HipTensor, weight: HipTensor, bias: HipTensor, rows: int, in_dim: int,
+               out_dim: int) -> HipTensor:
+        """ops/ops.zig:1728: Y = X @ W^T + bias, bias an f32 tensor of out_dim elements."""
+        h = C.c_void_p()
+        check(_lib.lib().afhip_compute_linear(self._h, input.handle, weight.handle, bias.handle, rows, in_dim, out_dim,
+                                              C.byref(h)))
+        return HipTensor(h.value)
+
+    def linearPair(self, input: HipTensor, weight_a: HipTensor, bias_a: HipTensor, weight_b: HipTensor,
+                   bias_b: HipTensor, rows: int, in_dim: int, out_dim: int):
+        """ops/ops.zig:915, :1846-1885: (first, second) = (X @ Wa^T + ba, X @ Wb^T + bb)."""
+        ha, hb = C.c_void_p(), C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_pair(self._h, input.handle, weight_a.handle, bias_a.handle, weight_b.handle,
+                                                   bias_b.handle, rows, in_dim, out_dim, C.byref(ha), C.byref(hb)))
+        return HipTensor(ha.value), HipTensor(hb.value)
+
+    def linearTriple(self, input: HipTensor, weight_a: HipTensor, bias_a: HipTensor, weight_b: HipTensor,
+                     bias_b: HipTensor, weight_c: HipTensor, bias_c: HipTensor, rows: int, in_dim: int, out_dim: int):
+        """ops/ops.zig:921, :1887-1910: the three biased Q/K/V projections of one input."""
+        ha, hb, hc = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        check(_lib.lib().afhip_compute_linear_triple(self._h, input.handle, weight_a.handle, bias_a.handle,
+                                                     weight_b.handle, bias_b.handle, weight_c.handle, bias_c.handle, rows,
+                                                     in_dim, out_dim, C.byref(ha), C.byref(hb), C.byref(hc)))
+        return HipTensor(ha.value), HipTensor(hb.value), HipTensor(hc.value)
+
     def linearNoBiasGrouped(self, input: HipTensor, weight: HipTensor, rows: int, in_dim: int, out_dim: int,
                             projection_out_dims, num_projections: int) -> HipTensor:
         """ops/ops.zig:901, :1786-1800: `weight` is the concatenation of the projections along the output axis."""

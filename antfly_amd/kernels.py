@@ -27,6 +27,21 @@ def launchLinearPairF32(stream, tensor_type, layout, dst_a: Buffer, dst_b: Buffe
                                                   rows, in_dim, out_dim, workspace, dispatch))
 
 
+def launchLinearBiasF32(stream, tensor_type, layout, dst: Buffer, input: Buffer, weight: Buffer, bias: Buffer, rows, in_dim,
+                        out_dim, workspace: Buffer = NO_BUFFER, dispatch: int = -1) -> None:
+    """Y = X @ W^T + bias (f32 [out_dim]), the bias added by the kernel that writes Y."""
+    check(_lib.lib().afhip_launch_linear_bias_f32(stream, tensor_type, layout, dst, input, weight, bias, rows, in_dim,
+                                                  out_dim, workspace, dispatch))
+
+
+def launchLinearPairBiasF32(stream, tensor_type, layout, dst_a: Buffer, dst_b: Buffer, input: Buffer, weight_a: Buffer,
+                            bias_a: Buffer, weight_b: Buffer, bias_b: Buffer, rows, in_dim, out_dim,
+                            workspace: Buffer = NO_BUFFER, dispatch: int = -1) -> None:
+    """Two biased matmuls of one shape that share X."""
+    check(_lib.lib().afhip_launch_linear_pair_bias_f32(stream, tensor_type, layout, dst_a, dst_b, input, weight_a, bias_a,
+                                                       weight_b, bias_b, rows, in_dim, out_dim, workspace, dispatch))
+
+
 def launchLinearQ8_0F32(stream, dst: Buffer, input: Buffer, weight_raw: Buffer, rows, in_dim, out_dim,
                         workspace: Buffer = NO_BUFFER) -> None:
     check(_lib.lib().afhip_launch_linear_q8_0_f32(stream, dst, input, weight_raw, rows, in_dim, out_dim, workspace))

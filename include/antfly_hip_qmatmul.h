@@ -141,6 +141,23 @@ afhip_status afhip_launch_linear_pair_f32(void *stream, int tensor_type, int lay
                                           afhip_buffer dst_b, afhip_buffer input, afhip_buffer weight_a,
                                           afhip_buffer weight_b, size_t rows, size_t in_dim,
                                           size_t out_dim, afhip_buffer workspace, int dispatch);
+/* Y = X * W^T + bias: the matmul above with an f32 bias [out_dim] added to every row by the
+ * kernel that writes Y (the engine's `linear`, ops/ops.zig:1728; the CUDA backend's biased
+ * launchers, ops/cuda/kernels.zig:339ff and cuda_compute.zig:544-575; the CPU op adds the
+ * bias rows after the no-bias product, ops/native_compute.zig:5065-5077 and :5197-5203).
+ * Each element is exactly afhip_launch_linear_f32's value plus its bias in f32. */
+afhip_status afhip_launch_linear_bias_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                          afhip_buffer input, afhip_buffer weight, afhip_buffer bias,
+                                          size_t rows, size_t in_dim, size_t out_dim,
+                                          afhip_buffer workspace, int dispatch);
+/* Two biased matmuls that share X (linearPair, ops/ops.zig:915, wrapper :1846-1885; CPU op
+ * ops/native_compute.zig:6513ff): afhip_launch_linear_pair_f32 with bias_a / bias_b added. */
+afhip_status afhip_launch_linear_pair_bias_f32(void *stream, int tensor_type, int layout,
+                                               afhip_buffer dst_a, afhip_buffer dst_b, afhip_buffer input,
+                                               afhip_buffer weight_a, afhip_buffer bias_a,
+                                               afhip_buffer weight_b, afhip_buffer bias_b, size_t rows,
+                                               size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                               int dispatch);
 /* Drop-ins with the reference launcher names: raw GGUF layout, automatic dispatch. */
 afhip_status afhip_launch_linear_q8_0_f32(void *stream, afhip_buffer dst, afhip_buffer input,
                                           afhip_buffer weight_raw, size_t rows, size_t in_dim,
@@ -301,6 +318,35 @@ afhip_status afhip_compute_linear_no_bias_pair(afhip_compute *self, const afhip_
                                                const afhip_tensor *weight_a, const afhip_tensor *weight_b,
                                                size_t rows, size_t in_dim, size_t out_dim,
                                                afhip_tensor **out_first, afhip_tensor **out_second);
+
+/* linear, ops/ops.zig:1728 (CUDA backend cuda_compute.zig:544-575, CPU op
+ * ops/native_compute.zig:5143-5183): Y = X * W^T + bias with an f32 bias tensor of out_dim
+ * elements (other dtypes -> AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE, other counts ->
+ * AFHIP_ERR_INVALID_SHAPE); otherwise as afhip_compute_linear_no_bias. */
+afhip_status afhip_compute_linear(afhip_compute *self, const afhip_tensor *input,
+                                  const afhip_tensor *weight, const afhip_tensor *bias, size_t rows,
+                                  size_t in_dim, size_t out_dim, afhip_tensor **out);
+
+/* linearPair, ops/ops.zig:915 (wrapper :1846-1885, CUDA backend cuda_compute.zig:799-815):
+ * two biased linears that share the input; as afhip_compute_linear_no_bias_pair with the
+ * biases added. */
+afhip_status afhip_compute_linear_pair(afhip_compute *self, const afhip_tensor *input,
+                                       const afhip_tensor *weight_a, const afhip_tensor *bias_a,
+                                       const afhip_tensor *weight_b, const afhip_tensor *bias_b,
+                                       size_t rows, size_t in_dim, size_t out_dim,
+                                       afhip_tensor **out_first, afhip_tensor **out_second);
+
+/* linearTriple, ops/ops.zig:921 (wrapper :1887-1910, CUDA backend cuda_compute.zig:719ff):
+ * the Q/K/V projections of a model with separate weights: three biased linears that share
+ * the input.  The first two are served as a pair, the third as a single op; on an error no
+ * tensor is returned. */
+afhip_status afhip_compute_linear_triple(afhip_compute *self, const afhip_tensor *input,
+                                         const afhip_tensor *weight_a, const afhip_tensor *bias_a,
+                                         const afhip_tensor *weight_b, const afhip_tensor *bias_b,
+                                         const afhip_tensor *weight_c, const afhip_tensor *bias_c,
+                                         size_t rows, size_t in_dim, size_t out_dim,
+                                         afhip_tensor **out_first, afhip_tensor **out_second,
+                                         afhip_tensor **out_third);
 
 /* linearNoBiasGrouped, ops/ops.zig:901 (wrapper :1786-1800): `weight` is already the
  * concatenation of `num_projections` matrices along the output axis, so this is one

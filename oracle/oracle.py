@@ -67,6 +67,8 @@ def lib() -> C.CDLL:
         L.afo_argmax.argtypes = [vp, sz]
         L.afo_argmax_last_row.restype = C.c_long
         L.afo_argmax_last_row.argtypes = [vp, sz, sz]
+        L.afo_add_linear_bias_rows.restype = None
+        L.afo_add_linear_bias_rows.argtypes = [vp, vp, sz, sz]
         L.afo_linear_act_f64.argtypes = [i32, vp, vp, vp, sz, sz, sz]
         L.afo_thread_plan.argtypes = [sz, sz, sz, i32, i32, vp]
         L.afo_prepare.restype = vp
@@ -195,6 +197,20 @@ def linear_no_bias(fmt, x, w_raw, rows, in_dim, out_dim, workers=1) -> np.ndarra
     if rc != 0:
         raise ValueError(f"afo_linear_no_bias rc={rc}")
     return y
+
+
+def add_linear_bias_rows(y, bias, rows, out_dim) -> np.ndarray:
+    """y[r][o] + bias[o] in f32 (a new array)."""
+    out = np.array(_f32(y), dtype=np.float32).reshape(rows, out_dim).copy()
+    bias = _f32(bias)
+    assert bias.size == out_dim
+    lib().afo_add_linear_bias_rows(_p(out), _p(bias), rows, out_dim)
+    return out
+
+
+def linear(fmt, x, w_raw, bias, rows, in_dim, out_dim, workers=1) -> np.ndarray:
+    """The engine's biased `linear` on a quantized weight: the no-bias op, then the bias rows."""
+    return add_linear_bias_rows(linear_no_bias(fmt, x, w_raw, rows, in_dim, out_dim, workers), bias, rows, out_dim)
 
 
 def linear_act_f64(fmt, x, w_raw, rows, in_dim, out_dim) -> np.ndarray:

@@ -453,6 +453,12 @@ int afo_linear_no_bias(int fmt, const float *x, const uint8_t *w, float *y, size
     return 0;
 }
 
+void afo_add_linear_bias_rows(float *y, const float *bias, size_t rows, size_t out_dim) {
+    /* native_compute.zig:5197-5203 */
+    for (size_t r = 0; r < rows; r++)
+        for (size_t o = 0; o < out_dim; o++) y[r * out_dim + o] += bias[o];
+}
+
 int afo_linear_act_f64(int fmt, const float *x, const uint8_t *w, double *y, size_t rows,
                        size_t in_dim, size_t out_dim) {
     size_t bb = afo_block_bytes(fmt);

@@ -87,6 +87,11 @@ int afo_linear_no_bias(int fmt, const float *x, const uint8_t *w_raw, float *y,
 
 /* Route A in double precision (no f32 rounding after the int dot); bounds the
  * f32 accumulation error of any evaluation order. */
+/* addLinearBiasRows, ops/native_compute.zig:5197-5203: y[r][o] += bias[o].  The engine's
+ * biased `linear` on a quantized weight is the no-bias product followed by this
+ * (dispatchQuantizedLinear .single_bias, :5065-5077; .pair_bias falls back to it, :5110-5111). */
+void afo_add_linear_bias_rows(float *y, const float *bias, size_t rows, size_t out_dim);
+
 int afo_linear_act_f64(int fmt, const float *x, const uint8_t *w_raw, double *y,
                        size_t rows, size_t in_dim, size_t out_dim);
 

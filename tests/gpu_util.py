@@ -56,6 +56,29 @@ def linear_pair(fmt, layout, x: np.ndarray, wa_dev: torch.Tensor, wb_dev: torch.
     return ya.cpu().numpy(), yb.cpu().numpy()
 
 
+def linear_bias(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, bias: np.ndarray, rows, in_dim, out_dim,
+                dispatch=-1) -> np.ndarray:
+    xd, bd = to_dev(x.astype(np.float32)), to_dev(bias.astype(np.float32))
+    y = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    ws = torch.empty(max(kernels.workspaceBytes(fmt, rows, in_dim, out_dim), 16), dtype=torch.uint8, device=DEV)
+    kernels.launchLinearBiasF32(stream(), fmt, layout, buf(y), buf(xd), buf(w_dev), buf(bd), rows, in_dim, out_dim,
+                                buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+def linear_pair_bias(fmt, layout, x: np.ndarray, wa_dev, ba: np.ndarray, wb_dev, bb: np.ndarray, rows, in_dim, out_dim,
+                     dispatch=-1):
+    xd, bad, bbd = to_dev(x.astype(np.float32)), to_dev(ba.astype(np.float32)), to_dev(bb.astype(np.float32))
+    ya = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    yb = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=DEV)
+    ws = torch.empty(max(kernels.workspaceBytes(fmt, rows, in_dim, out_dim), 16), dtype=torch.uint8, device=DEV)
+    kernels.launchLinearPairBiasF32(stream(), fmt, layout, buf(ya), buf(yb), buf(xd), buf(wa_dev), buf(bad), buf(wb_dev),
+                                    buf(bbd), rows, in_dim, out_dim, buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return ya.cpu().numpy(), yb.cpu().numpy()
+
+
 def block_dots(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1) -> np.ndarray:
     xd = to_dev(x.astype(np.float32))
     d = torch.full((rows, out_dim, in_dim // 32), -(2 ** 31), dtype=torch.int32, device=DEV)

@@ -407,6 +407,28 @@ def test_argmax_reference_vectors_and_properties(kats):
     assert O.argmax([np.nan, np.nan]) == 0
 
 
+def test_biased_linear_is_the_no_bias_op_plus_bias_rows():
+    """The reference's own biased Q8_0 test inputs (ops/native_compute.zig:39163-39223): small
+    integers and scale 1.0, so the expected values are exact; and the general definition
+    (:5065-5077, :5197-5203) against numpy broadcasting."""
+    rows, in_dim, out_dim = 3, 32, 2
+    x = np.array([(i % 7) - 3 for i in range(rows * in_dim)], np.float32).reshape(rows, in_dim)
+    q = np.array([(i % 5) - 2 for i in range(32)], np.int8)
+    w = np.concatenate([np.concatenate([np.array([0x00, 0x3C], np.uint8), q.view(np.uint8)])] * out_dim)
+    bias = np.array([0.25, -0.5], np.float32)
+    want = (x.astype(np.int64) @ np.tile(q.astype(np.int64), (out_dim, 1)).T).astype(np.float32) + bias
+    assert np.array_equal(O.linear(Q8, x, w, bias, rows, in_dim, out_dim), want)
+    assert want[0, 0] != want[0, 1] and want[0, 0] - bias[0] == want[0, 1] - bias[1]  # same weights, different bias
+
+    rows, in_dim, out_dim = 5, 512, 700
+    x = synth.activations(71, rows, in_dim)
+    bias = synth.activations(72, 1, out_dim)[0]
+    for fmt in (Q4, Q8):
+        w = synth.weights(fmt, 73, out_dim, in_dim)
+        plain = O.linear_no_bias(fmt, x, w, rows, in_dim, out_dim)
+        assert np.array_equal(O.linear(fmt, x, w, bias, rows, in_dim, out_dim), plain + bias[None, :])
+
+
 def test_synth_is_chunk_invariant_and_in_range():
     a = synth.splitmix64(42, 0, 1000)
     b = np.concatenate([synth.splitmix64(42, 0, 333), synth.splitmix64(42, 333, 667)])
