@@ -123,6 +123,52 @@ def test_parser_errors():
             f.tensorData("nope")
 
 
+def test_truncated_and_corrupted_images_fail_cleanly():
+    """Every prefix of a valid image and seeded byte corruptions of its header region either
+    parse (and then every tensor / metadata accessor works or reports an error) or raise one
+    of the library's errors; nothing reads outside the image."""
+    rng = np.random.default_rng(7)
+    img = W.build([("general.architecture", gguf.STRING, "llama"), ("n", gguf.U32, 7),
+                   ("toks", gguf.ARRAY, (gguf.STRING, ["a", "bc", "def"]))],
+                  [("a.weight", [64, 4], 2, bytes(4 * 2 * 18)), ("b.weight", [64, 4], 8, bytes(4 * 2 * 34)),
+                   ("n.weight", [64], 0, bytes(256))])
+    header = len(img) - (4 * 2 * 18 + 4 * 2 * 34 + 256)
+
+    def walk(image):
+        try:
+            with gguf.File.parse(image) as f:
+                for t in f.tensors:
+                    try:
+                        data = f.tensorData(t.name)
+                        assert len(data) == t.byte_len
+                    except _lib.HipError:
+                        pass
+                assert len(f.metadata) == f.header.metadata_count
+            return True
+        except _lib.HipError:
+            return False
+
+    assert walk(img)
+    results = [walk(img[:cut]) for cut in range(header)]  # a cut anywhere is an error or a parse, never a crash
+    infos_end = results.index(True) if True in results else header
+    assert infos_end > header - gguf.DEFAULT_ALIGNMENT  # only cuts inside the alignment padding still parse
+    assert all(results[infos_end:])
+    parsed = 0
+    for _ in range(3000):
+        b = bytearray(img)
+        for _ in range(int(rng.integers(1, 4))):
+            pos = int(rng.integers(0, header))
+            kind = int(rng.integers(0, 3))
+            if kind == 0:
+                b[pos] = int(rng.integers(0, 256))
+            elif kind == 1:
+                b[pos] ^= 1 << int(rng.integers(0, 8))
+            else:
+                b[pos:pos + 8] = int(rng.choice([0, 2 ** 64 - 1, 2 ** 63, 2 ** 32 - 1, 2 ** 31])).to_bytes(8, "little")[:len(b) - pos]
+        parsed += walk(bytes(b))
+    assert 0 < parsed < 3000
+
+
 def test_open_maps_a_file(tmp_path):
     blocks = np.arange(2 * 2 * 34, dtype=np.uint8)
     img = W.build([("general.architecture", gguf.STRING, "llama")],
