@@ -19,6 +19,16 @@ DEFAULT_ALIGNMENT = 32
 U8, I8, U16, I16, U32, I32, F32, BOOL, STRING, ARRAY, U64, I64, F64 = range(13)
 
 
+def _text(raw: bytes) -> str:
+    """Names and strings are byte strings in the file (format.zig keeps them as []const u8);
+    bytes that are not UTF-8 survive a round trip through str as surrogate escapes."""
+    return raw.decode("utf-8", "surrogateescape")
+
+
+def _raw(text: str) -> bytes:
+    return text.encode("utf-8", "surrogateescape")
+
+
 @dataclass
 class Header:
     version: int
@@ -110,7 +120,7 @@ class File:
     @staticmethod
     def _tensor(info: _lib.GgufTensorInfo) -> TensorInfo:
         return TensorInfo(
-            name=C.string_at(info.name, info.name_len).decode(),
+            name=_text(C.string_at(info.name, info.name_len)),
             dimensions=[int(info.dimensions[i]) for i in range(min(info.n_dimensions, _lib.GGUF_MAX_DIMS))],
             tensor_type=int(info.tensor_type), type_name=info.type_name.decode(),
             is_quantized=bool(info.is_quantized), offset=int(info.offset), data_offset=int(info.data_offset),
@@ -129,9 +139,9 @@ class File:
     def _entry(m: _lib.GgufMetadata) -> MetadataEntry:
         t = int(m.value_type)
         if t == STRING:
-            value = C.string_at(m.str, m.str_len).decode()
+            value = _text(C.string_at(m.str, m.str_len))
         elif t == ARRAY:
-            return MetadataEntry(C.string_at(m.key, m.key_len).decode(), t, int(m.count), int(m.element_type))
+            return MetadataEntry(_text(C.string_at(m.key, m.key_len)), t, int(m.count), int(m.element_type))
         elif t in (F32, F64):
             value = float(m.f64)
         elif t == BOOL:
@@ -140,7 +150,7 @@ class File:
             value = int(m.i64)
         else:
             value = int(m.u64)
-        return MetadataEntry(C.string_at(m.key, m.key_len).decode(), t, value)
+        return MetadataEntry(_text(C.string_at(m.key, m.key_len)), t, value)
 
     @property
     def metadata(self) -> List[MetadataEntry]:
@@ -153,7 +163,7 @@ class File:
 
     def findMetadata(self, key: str) -> Optional[MetadataEntry]:
         m = _lib.GgufMetadata()
-        rc = _lib.lib().afhip_gguf_find_metadata(self._h, key.encode(), C.byref(m))
+        rc = _lib.lib().afhip_gguf_find_metadata(self._h, _raw(key), C.byref(m))
         if rc == _lib.ERR_TENSOR_NOT_FOUND:
             return None
         check(rc)
@@ -162,7 +172,7 @@ class File:
     def tensorData(self, name: str) -> np.ndarray:
         """The tensor's raw bytes, copied out of the image (ErrTensorNotFound / UnexpectedEndOfFile as the C ABI)."""
         info = _lib.GgufTensorInfo()
-        check(_lib.lib().afhip_gguf_find_tensor(self._h, name.encode(), C.byref(info)))
+        check(_lib.lib().afhip_gguf_find_tensor(self._h, _raw(name), C.byref(info)))
         ptr, n = C.c_void_p(), C.c_size_t()
         check(_lib.lib().afhip_gguf_tensor_data(self._h, C.byref(info), C.byref(ptr), C.byref(n)))
         return np.frombuffer(C.string_at(ptr.value, n.value), dtype=np.uint8)
@@ -179,7 +189,7 @@ class Catalog:
 
     def find(self, name: str) -> Optional[TensorInfo]:
         info = _lib.GgufTensorInfo()
-        rc = _lib.lib().afhip_gguf_find_tensor(self.file.handle, name.encode(), C.byref(info))
+        rc = _lib.lib().afhip_gguf_find_tensor(self.file.handle, _raw(name), C.byref(info))
         if rc == _lib.ERR_TENSOR_NOT_FOUND:
             return None
         check(rc)
