@@ -604,11 +604,14 @@ int compute_units() {
 }
 
 // Wavefronts per workgroup: a multiple of `slices` (whole column groups), at most the
-// requested size, chosen so that the workgroups spread evenly over the compute units:
-// the busiest unit's share, ceil(grid / units) workgroups of `waves` wavefronts, is
-// smallest (ties go to the larger workgroup, which repeats the prologue less often).
-// `exact` takes the requested size as it is (tuning runs).
-int workgroup_waves(int requested_threads, int max_threads, int slices, int groups, bool exact) {
+// requested size, chosen so that the workgroups spread evenly over the compute units.
+// The busiest unit runs ceil(grid / units) workgroups, each `waves` wavefronts of weight
+// streaming plus a prologue (X is quantized by every workgroup) that costs about as much
+// as kPrologueWaves more; the size (of at least min_waves wavefronts) with the smallest
+// such share wins, ties go to the larger workgroup.  A small matrix therefore gets small workgroups (one per unit), a
+// large one gets large ones.  `exact` takes the requested size as it is (tuning runs).
+int workgroup_waves(int requested_threads, int max_threads, int slices, int groups, bool exact, int min_waves = 1) {
+    constexpr int kPrologueWaves = 2;
     int limit = (requested_threads < max_threads ? requested_threads : max_threads) / 64;
     if (limit < slices) limit = slices;
     limit = limit / slices * slices;
@@ -616,10 +619,11 @@ int workgroup_waves(int requested_threads, int max_threads, int slices, int grou
     const int units = compute_units();
     int best = limit;
     long best_cost = -1;
-    for (int waves = limit; waves >= slices && waves * 2 > limit; waves -= slices) {  // down to half the limit
+    if (min_waves < 2) min_waves = 2;  // a lone wavefront per workgroup measured slower than two
+    for (int waves = limit; waves >= slices && waves >= min_waves; waves -= slices) {
         const int groups_per_wg = waves / slices;
         const long grid = (groups + groups_per_wg - 1) / groups_per_wg;
-        const long cost = (grid + units - 1) / units * waves;
+        const long cost = (grid + units - 1) / units * (waves + kPrologueWaves);
         if (best_cost < 0 || cost < best_cost) {
             best_cost = cost;
             best = waves;
@@ -647,14 +651,13 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     GemvTargets tg = tg0;
     tg.groups_each = (out_dim + kCols - 1) / kCols;
     const int groups = tg.groups_each * (tg.weight_b ? 2 : 1);
-    int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact);
     // the prologue quantizes up to two blocks of X per thread ahead of the weight requests
     const int x_blocks = kRows * (in_dim / 32);
-    if (x_blocks > 2 * waves * 64 && !tune.exact) waves = workgroup_waves(1024, 1024, slices, groups, true);
+    int waves = workgroup_waves(tune.threads, 1024, slices, groups, tune.exact, (x_blocks + 127) / 128);
     // A matrix that takes several rounds of workgroups (a vocabulary): half-size workgroups,
     // two to a compute unit, so that one streams weights while the other is in its prologue.
     if (!tune.exact && waves > 8 && slices <= 8 && x_blocks <= 512 &&
-        (groups + waves / slices - 1) / (waves / slices) > compute_units() * 3 / 2)
+        (groups + waves / slices - 1) / (waves / slices) > compute_units() * 3)
         waves = workgroup_waves(512, 512, slices, groups, true);  // many rounds: nothing to balance
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
@@ -675,7 +678,8 @@ hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, co
     GemvTargets tg = tg0;
     tg.groups_each = (out_dim + kCols - 1) / kCols;
     const int groups = tg.groups_each * (tg.weight_b ? 2 : 1);
-    const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);  // several of these workgroups share a unit: no balancing
+    // 8 wavefronts; several of these workgroups share a unit, and smaller ones for small matrices measured no better
+    const int waves = workgroup_waves(tune.threads, 512, slices, groups, true);
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
     auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
