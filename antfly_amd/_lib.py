@@ -32,6 +32,7 @@ ERR_TENSOR_NOT_FOUND = -17
 ERR_IO = -18
 
 TYPE_F32, TYPE_Q4_0, TYPE_Q8_0, TYPE_Q4_K = 0, 2, 8, 12
+ACTIVATION_NONE, ACTIVATION_RELU, ACTIVATION_QUICK_GELU, ACTIVATION_GELU = 0, 1, 2, 3
 LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
 DTYPE_F32, DTYPE_U8 = 0, 1
 
@@ -111,6 +112,7 @@ SIGNATURES = {
     "afhip_launch_linear_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_pair_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_bias_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
+    "afhip_launch_linear_epilogue_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, _i, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_pair_bias_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_q8_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_linear_q4_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
@@ -152,6 +154,8 @@ SIGNATURES = {
     "afhip_compute_linear_no_bias": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_pair": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear": (_st, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "afhip_compute_linear_activation": (_st, [_vp, _vp, _vp, _vp, _i, _sz, _sz, _sz, C.POINTER(_vp)]),
+    "afhip_compute_linear_add": (_st, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp)]),
     "afhip_compute_linear_pair": (_st, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear_triple": (_st, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(_vp), C.POINTER(_vp), C.POINTER(_vp)]),
     "afhip_compute_linear_no_bias_grouped": (_st, [_vp, _vp, _vp, _sz, _sz, _sz, C.POINTER(C.c_uint32), _sz, C.POINTER(_vp)]),

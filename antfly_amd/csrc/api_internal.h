@@ -19,12 +19,18 @@ size_t block_bytes(int tensor_type);
 // int32 block dots instead of Y".
 // weight_b.ptr != 0 adds a second matrix of the same shape and layout that shares the
 // input (result in dst_b; not together with dots).
-// bias / bias_b (.ptr != 0): f32 [out_dim] added to every row of dst / dst_b (not together with dots).
+// extras: what the kernel that writes Y adds to the plain product (not together with dots).
+struct LinearExtras {
+    afhip_buffer bias{0, 0};      // f32 [out_dim], added to every row of dst
+    afhip_buffer bias_b{0, 0};    // the same for dst_b
+    afhip_buffer residual{0, 0};  // f32 [rows][out_dim], added last (one matrix only)
+    int activation = AFHIP_ACTIVATION_NONE;  // applied after the bias (one matrix only)
+};
 afhip_status linear_impl(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
                          int dispatch, afhip_buffer dots, LaunchCounters* counters,
                          afhip_buffer dst_b = afhip_buffer{0, 0}, afhip_buffer weight_b = afhip_buffer{0, 0},
-                         afhip_buffer bias = afhip_buffer{0, 0}, afhip_buffer bias_b = afhip_buffer{0, 0});
+                         const LinearExtras& extras = LinearExtras{});
 
 // argmax over the last row of f32 [rows, dim]; `workspace` (optional) lets several workgroups scan a long row.
 afhip_status argmax_last_row_impl(void* stream, afhip_buffer token_u32, afhip_buffer token_f32, afhip_buffer input,

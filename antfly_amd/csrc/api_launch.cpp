@@ -85,7 +85,7 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
 static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                     size_t rows, size_t in_dim, size_t out_dim, int dispatch, bool want_dots,
                                     LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b,
-                                    afhip_buffer bias, afhip_buffer bias_b) {
+                                    const Epilogue& ep, const Epilogue& ep_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // this format has no integer route
     if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -115,7 +115,7 @@ static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_
                                        reinterpret_cast<const float*>(input.ptr),
                                        reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
                                        static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
-                                       reinterpret_cast<const float*>(i ? bias_b.ptr : bias.ptr));
+                                       i ? ep_b : ep);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
     }
     return AFHIP_OK;
@@ -124,21 +124,35 @@ static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_
 afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
                          int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
-                         afhip_buffer weight_b, afhip_buffer bias, afhip_buffer bias_b) {
+                         afhip_buffer weight_b, const LinearExtras& extras) {
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
-    // biases: f32 [out_dim]; the second one only with a second matrix, none with the block dots
-    if ((bias_b.ptr != 0 && !pair) || ((bias.ptr != 0 || bias_b.ptr != 0) && dots.ptr != 0)) return AFHIP_ERR_INVALID_ARGUMENT;
-    for (const afhip_buffer& b : {bias, bias_b}) {
+    // biases: f32 [out_dim], the second one only with a second matrix; activation and residual
+    // (f32 [rows][out_dim]) only with one matrix; none of them with the block dots
+    const bool any_extra = extras.bias.ptr != 0 || extras.bias_b.ptr != 0 || extras.residual.ptr != 0 ||
+                           extras.activation != AFHIP_ACTIVATION_NONE;
+    if ((extras.bias_b.ptr != 0 && !pair) || (any_extra && dots.ptr != 0)) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (pair && (extras.residual.ptr != 0 || extras.activation != AFHIP_ACTIVATION_NONE)) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (extras.activation < AFHIP_ACTIVATION_NONE || extras.activation > AFHIP_ACTIVATION_GELU) return AFHIP_ERR_INVALID_ARGUMENT;
+    for (const afhip_buffer& b : {extras.bias, extras.bias_b}) {
         size_t need;
         if (b.ptr == 0) continue;
         if (b.ptr % 4 != 0 || !checked_mul(out_dim, 4, &need) || b.len < need) return AFHIP_ERR_INVALID_STATE;
     }
-    const float* add = reinterpret_cast<const float*>(bias.ptr);
-    const float* add_b = reinterpret_cast<const float*>(bias_b.ptr);
+    if (extras.residual.ptr != 0) {
+        size_t count, need;
+        if (extras.residual.ptr % 4 != 0 || !checked_mul(rows, out_dim, &count) || !checked_mul(count, 4, &need) ||
+            extras.residual.len < need)
+            return AFHIP_ERR_INVALID_STATE;
+    }
+    Epilogue ep, ep_b;
+    ep.bias = reinterpret_cast<const float*>(extras.bias.ptr);
+    ep.residual = reinterpret_cast<const float*>(extras.residual.ptr);
+    ep.activation = extras.activation;  // AFHIP_ACTIVATION_* and kAct* share their values
+    ep_b.bias = reinterpret_cast<const float*>(extras.bias_b.ptr);
     if (tensor_type == AFHIP_TYPE_Q4_K)
         return linear_q4k_impl(stream, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters, dst_b,
-                               weight_b, bias, bias_b);
+                               weight_b, ep, ep_b);
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -186,11 +200,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     if (!route_a) {
         if (counters) counters->f32_route++;
         hipError_t e = launch_linear_generic(stream, tensor_type, layout, false, y, nullptr, x, nullptr, nullptr, w,
-                                             static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add);
+                                             static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), ep);
         if (e == hipSuccess && pair) {
             if (counters) counters->f32_route++;
             e = launch_linear_generic(stream, tensor_type, layout, false, y_b, nullptr, x, nullptr, nullptr, w_b,
-                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
+                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), ep_b);
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
@@ -212,11 +226,11 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                                                    ws.sx, ws.sums);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
         e = launch_gemm_i8(stream, tensor_type, want_dots ? nullptr : y, dot_out, ws.qx, ws.sx, w, static_cast<int>(rows),
-                           static_cast<int>(in_dim), static_cast<int>(out_dim), add);
+                           static_cast<int>(in_dim), static_cast<int>(out_dim), ep);
         if (e == hipSuccess && pair) {  // the second matrix reuses the quantized activations
             if (counters) counters->mm++;
             e = launch_gemm_i8(stream, tensor_type, y_b, nullptr, ws.qx, ws.sx, w_b, static_cast<int>(rows),
-                               static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
+                               static_cast<int>(in_dim), static_cast<int>(out_dim), ep_b);
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
@@ -253,10 +267,12 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                 pre.sum = ws.sums + r0 * kb;
             }
             // a pair is one launch over the columns of both matrices
+            Epilogue ep_rows = ep;
+            if (ep_rows.residual) ep_rows.residual += r0 * out_dim;
             hipError_t e = launch_gemv_fused(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
                                              want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, pre, w,
                                              nr, static_cast<int>(in_dim), static_cast<int>(out_dim), tune,
-                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr, add, add_b);
+                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr, ep_rows, ep_b);
             if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         return AFHIP_OK;
@@ -275,10 +291,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
                                                ws.sums);
     if (e != hipSuccess) return static_cast<afhip_status>(e);
     e = launch_linear_generic(stream, tensor_type, layout, true, want_dots ? nullptr : y, dot_out, nullptr, ws.qx, ws.sx,
-                              w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add);
+                              w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), ep);
     if (e == hipSuccess && pair)
         e = launch_linear_generic(stream, tensor_type, layout, true, y_b, nullptr, nullptr, ws.qx, ws.sx, w_b,
-                                  static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), add_b);
+                                  static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), ep_b);
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
@@ -495,8 +511,22 @@ afhip_status afhip_launch_linear_bias_f32(void* stream, int tensor_type, int lay
                                           afhip_buffer weight, afhip_buffer bias, size_t rows, size_t in_dim,
                                           size_t out_dim, afhip_buffer workspace, int dispatch) {
     if (bias.ptr == 0 && out_dim != 0) return AFHIP_ERR_INVALID_STATE;
+    LinearExtras extras;
+    extras.bias = bias;
     return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
-                       afhip_buffer{0, 0}, nullptr, afhip_buffer{0, 0}, afhip_buffer{0, 0}, bias);
+                       afhip_buffer{0, 0}, nullptr, afhip_buffer{0, 0}, afhip_buffer{0, 0}, extras);
+}
+
+afhip_status afhip_launch_linear_epilogue_f32(void* stream, int tensor_type, int layout, afhip_buffer dst,
+                                              afhip_buffer input, afhip_buffer weight, afhip_buffer bias,
+                                              afhip_buffer residual, int activation, size_t rows, size_t in_dim,
+                                              size_t out_dim, afhip_buffer workspace, int dispatch) {
+    LinearExtras extras;
+    extras.bias = bias;
+    extras.residual = residual;
+    extras.activation = activation;
+    return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr, afhip_buffer{0, 0}, afhip_buffer{0, 0}, extras);
 }
 
 afhip_status afhip_launch_linear_pair_bias_f32(void* stream, int tensor_type, int layout, afhip_buffer dst_a,
@@ -506,8 +536,11 @@ afhip_status afhip_launch_linear_pair_bias_f32(void* stream, int tensor_type, in
                                                int dispatch) {
     if (weight_b.ptr == 0 || (dst_b.ptr == 0 && rows != 0 && out_dim != 0)) return AFHIP_ERR_INVALID_STATE;
     if ((bias_a.ptr == 0 || bias_b.ptr == 0) && out_dim != 0) return AFHIP_ERR_INVALID_STATE;
+    LinearExtras extras;
+    extras.bias = bias_a;
+    extras.bias_b = bias_b;
     return linear_impl(stream, tensor_type, layout, dst_a, input, weight_a, rows, in_dim, out_dim, workspace, dispatch,
-                       afhip_buffer{0, 0}, nullptr, dst_b, weight_b, bias_a, bias_b);
+                       afhip_buffer{0, 0}, nullptr, dst_b, weight_b, extras);
 }
 
 afhip_status afhip_launch_linear_q8_0_f32(void* stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight_raw,

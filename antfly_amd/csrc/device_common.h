@@ -2,6 +2,8 @@
 // Wavefronts are 64 wide; every helper here assumes that.
 #pragma once
 
+#include "qmatmul_launch.h"
+
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -271,6 +273,20 @@ struct PreparedWeights<8> {
         return r;
     }
 };
+
+// The value stored for output column o (element idx of Y) whose total is v.
+__device__ __forceinline__ float finish_output(const Epilogue& ep, int o, size_t idx, float v) {
+    if (ep.bias != nullptr) v += ep.bias[o];
+    if (ep.activation == kActRelu) {
+        v = v < 0.0f ? 0.0f : v;
+    } else if (ep.activation == kActQuickGelu) {
+        v = v / (1.0f + expf(-1.702f * v));
+    } else if (ep.activation == kActGelu) {
+        v = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+    }
+    if (ep.residual != nullptr) v += ep.residual[idx];
+    return v;
+}
 
 __device__ __forceinline__ int dot32(const int w[8], const int a[8]) {
     int acc = 0;

@@ -128,7 +128,7 @@ template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots>
 __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
-    const float* __restrict__ bias) {
+    Epilogue ep) {
     using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
     constexpr int kWaves = S::kWaves, kSB = S::kStageBlocks, kRPL = S::kRowsPerLoad, kCPR = S::kChunksPerRow;
     constexpr int kTM = S::kTM, kTN = S::kTN, kRing = S::kRing;
@@ -397,8 +397,6 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     // the ring is reused for the reduction (and before the workgroup ends).
     wait_vm_outstanding(0);
     const int n = n0 + col;
-    // linear / linearPair (ops/ops.zig:1728, :915): the column's bias joins every row's total
-    const float column_bias = bias != nullptr && n < out_dim ? bias[n] : 0.0f;
     if (kSplit > 1) {
         // ---- the kSplit partial sums of a tile meet in LDS
         __syncthreads();
@@ -415,14 +413,16 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
 #pragma unroll
             for (int k2 = 1; k2 < kSplit; ++k2) sum += red[((k2 * S::kTiles + tile) * 16 + v) * 64 + lane];
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < rows && n < out_dim) dst[static_cast<size_t>(m) * out_dim + n] = bias != nullptr ? sum + column_bias : sum;
+            if (m < rows && n < out_dim)
+                dst[static_cast<size_t>(m) * out_dim + n] = finish_output(ep, n, static_cast<size_t>(m) * out_dim + n, sum);
         }
     } else {
         if (dst == nullptr) return;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < rows && n < out_dim) dst[static_cast<size_t>(m) * out_dim + n] = bias != nullptr ? acc[v] + column_bias : acc[v];
+            if (m < rows && n < out_dim)
+                dst[static_cast<size_t>(m) * out_dim + n] = finish_output(ep, n, static_cast<size_t>(m) * out_dim + n, acc[v]);
         }
     }
 }
@@ -431,7 +431,7 @@ namespace {
 
 template <int kType, int kWavesM, int kWavesN, int kSplit>
 hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
-                       const uint8_t* weight, int rows, int in_dim, int out_dim, const float* bias) {
+                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep) {
     using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
     const int m_tiles = (rows + S::kTM - 1) / S::kTM;
     const int n_tiles = (out_dim + S::kTN - 1) / S::kTN;
@@ -454,30 +454,30 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     if (attr != hipSuccess) return attr;
     if (dots)
         hipLaunchKernelGGL(kernel_dots, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
-                           m_tiles, n_tiles, bias);
+                           m_tiles, n_tiles, ep);
     else
         hipLaunchKernelGGL(kernel_f32, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
-                           m_tiles, n_tiles, bias);
+                           m_tiles, n_tiles, ep);
     return hipGetLastError();
 }
 
 template <int kType>
 hipError_t launch_type(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
-                       const uint8_t* weight, int rows, int in_dim, int out_dim, const float* bias) {
+                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep) {
     // 64 x 128 tiles while they still give every CU a workgroup, 32 x 64 with a deeper K split otherwise
     const long long big = static_cast<long long>((rows + 63) / 64) * ((out_dim + 127) / 128);
     static const char* force = std::getenv("AFHIP_GEMM_TILE");  // tuning: "L" = 64x128, "S" = 32x64
     const bool use_big = force ? force[0] != 'S' : big >= 256;
-    if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, bias);
-    return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, bias);
+    if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep);
+    return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep);
 }
 
 }  // namespace
 
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
-                          const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, const float* bias) {
-    if (tensor_type == 2) return launch_type<2>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, bias);
-    return launch_type<8>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, bias);
+                          const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, const Epilogue& ep) {
+    if (tensor_type == 2) return launch_type<2>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep);
+    return launch_type<8>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep);
 }
 
 }  // namespace afhip

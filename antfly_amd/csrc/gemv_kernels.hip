@@ -118,14 +118,9 @@ struct GemvTargets {
     const uint8_t* weight_a;
     const uint8_t* weight_b;  // null: one matrix
     int groups_each;
-    const float* bias_a;  // [out_dim] added to every row of the result, or null (linear / linearPair,
-    const float* bias_b;  // ops/ops.zig:1728, :915)
+    Epilogue ep_a;  // bias / activation / residual of each matrix (linear, linearPair ...,
+    Epilogue ep_b;  // ops/ops.zig:1728, :915)
 };
-
-// v + bias[o] when there is a bias.
-__device__ __forceinline__ float with_bias(const float* __restrict__ bias, int o, float v) {
-    return bias != nullptr ? v + bias[o] : v;
-}
 
 constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ? 4 : (n <= 8 ? 8 : 16))); }
 
@@ -348,7 +343,8 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             return;
         }
         if (active && mine && o0 + cc < out_dim && dst)
-            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = with_bias(second ? tg.bias_b : tg.bias_a, o0 + cc, red[0]);
+            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] =
+                finish_output(second ? tg.ep_b : tg.ep_a, o0 + cc, static_cast<size_t>(cr) * out_dim + o0 + cc, red[0]);
         return;
     }
     if (mine) partial[wave * kCells + cell] = red[0];
@@ -372,7 +368,8 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
                 if (k > key) key = k;
             }
         } else if (g < tg.groups_each && o < out_dim && d) {
-            d[static_cast<size_t>(r) * out_dim + o] = with_bias(sec ? tg.bias_b : tg.bias_a, o, total);
+            d[static_cast<size_t>(r) * out_dim + o] =
+                finish_output(sec ? tg.ep_b : tg.ep_a, o, static_cast<size_t>(r) * out_dim + o, total);
         }
     }
     if (kArgmax) {
@@ -567,7 +564,8 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
         const int r = rr == 0 ? r0 : r1;
         if (slices == 1) {
             if (active && mine && o0 + cc < out_dim && dst)
-                dst[static_cast<size_t>(r) * out_dim + o0 + cc] = with_bias(second ? tg.bias_b : tg.bias_a, o0 + cc, red[0]);
+                dst[static_cast<size_t>(r) * out_dim + o0 + cc] =
+                    finish_output(second ? tg.ep_b : tg.ep_a, o0 + cc, static_cast<size_t>(r) * out_dim + o0 + cc, red[0]);
         } else if (mine) {
             partial[wave * cells + r * kCols + cc] = red[0];
         }
@@ -585,7 +583,8 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * cells + rc];
         if (g < tg.groups_each && o < out_dim && d)
-            d[static_cast<size_t>(r) * out_dim + o] = with_bias(sec ? tg.bias_b : tg.bias_a, o, total);
+            d[static_cast<size_t>(r) * out_dim + o] =
+                finish_output(sec ? tg.ep_b : tg.ep_a, o, static_cast<size_t>(r) * out_dim + o, total);
     }
 }
 
@@ -726,10 +725,10 @@ int gemv_fused_max_in_dim() { return 16 * kSliceBlocks * 32; }
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
                              const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
                              int out_dim, const GemvTuning& tune, float* dst_b, const uint8_t* weight_b_prepared,
-                             const float* bias, const float* bias_b) {
+                             const Epilogue& ep, const Epilogue& ep_b) {
     if (in_dim > gemv_fused_max_in_dim()) return hipErrorInvalidValue;
     if (weight_b_prepared != nullptr && dots != nullptr) return hipErrorInvalidValue;  // block dots: one matrix at a time
-    const GemvTargets tg{dst, dst_b, weight_prepared, weight_b_prepared, 0, bias, bias_b};
+    const GemvTargets tg{dst, dst_b, weight_prepared, weight_b_prepared, 0, ep, ep_b};
     if (tensor_type == 2) return launch_gemv_type<2>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
     return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
@@ -738,7 +737,7 @@ hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned
                                    const float* input, const uint8_t* weight_prepared, int in_dim, int out_dim,
                                    const GemvTuning& tune) {
     if (in_dim > gemv_fused_max_in_dim() || keys == nullptr || key_count == nullptr) return hipErrorInvalidValue;
-    const GemvTargets tg{nullptr, nullptr, weight_prepared, nullptr, 0, nullptr, nullptr};
+    const GemvTargets tg{nullptr, nullptr, weight_prepared, nullptr, 0, Epilogue{}, Epilogue{}};
     if (tensor_type == 2)
         return launch_fused<2, 1, false, true>(stream, tg, nullptr, input, in_dim, out_dim, tune, keys, key_count);
     return launch_fused<8, 1, false, true>(stream, tg, nullptr, input, in_dim, out_dim, tune, keys, key_count);

@@ -160,7 +160,8 @@ afhip_status make_f32_result(afhip_compute* self, afhip_buffer device, size_t ro
 afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
                                  size_t rows, size_t in_dim, size_t out_dim, int dispatch, afhip_tensor** out,
                                  const afhip_tensor* weight_b = nullptr, afhip_tensor** out_b = nullptr,
-                                 const afhip_tensor* bias = nullptr, const afhip_tensor* bias_b = nullptr) {
+                                 const afhip_tensor* bias = nullptr, const afhip_tensor* bias_b = nullptr,
+                                 const afhip_tensor* residual = nullptr, int activation = AFHIP_ACTIVATION_NONE) {
     // cuda_compute.zig:689-717; with biases (f32 [out_dim], added to every row): linear :544-575, linearPair :799-815
     const bool pair = weight_b != nullptr || out_b != nullptr;
     if (!self || !input || !weight || !out || (pair && (!weight_b || !out_b)) || (bias_b && !pair))
@@ -173,12 +174,15 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         if (!is_f32(b)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
         if (b->elem_count != out_dim) return AFHIP_ERR_INVALID_SHAPE;
     }
+    if (pair && (residual || activation != AFHIP_ACTIVATION_NONE)) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (residual && !is_f32(residual)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     const afhip_tensor* ws[2] = {weight, weight_b};
     size_t in_count, w_count, out_count, out_bytes;
     if (!checked_mul(rows, in_dim, &in_count) || !checked_mul(out_dim, in_dim, &w_count) ||
         !checked_mul(rows, out_dim, &out_count) || !checked_mul(out_count, 4, &out_bytes))
         return AFHIP_ERR_INVALID_SHAPE;
     if (input->elem_count != in_count) return AFHIP_ERR_INVALID_SHAPE;
+    if (residual && residual->elem_count != out_count) return AFHIP_ERR_INVALID_SHAPE;
     for (int i = 0; i < (pair ? 2 : 1); ++i) {
         const afhip_tensor* w = ws[i];
         if (w->quant_type < 0 && !is_f32(w)) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
@@ -217,10 +221,14 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);
     }
     if (s == AFHIP_OK) {
+        LinearExtras extras;
+        if (bias) extras.bias = bias->buffer;
+        if (bias_b) extras.bias_b = bias_b->buffer;
+        if (residual) extras.residual = residual->buffer;
+        extras.activation = activation;
         s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows,
                         in_dim, out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
-                        pair ? weight_b->buffer : afhip_buffer{0, 0}, bias ? bias->buffer : afhip_buffer{0, 0},
-                        bias_b ? bias_b->buffer : afhip_buffer{0, 0});
+                        pair ? weight_b->buffer : afhip_buffer{0, 0}, extras);
     }
     if (s != AFHIP_OK) {
         release_device_buffer(self, &device);
@@ -549,6 +557,21 @@ afhip_status afhip_compute_linear(afhip_compute* self, const afhip_tensor* input
                                   afhip_tensor** out) {
     if (!bias) return AFHIP_ERR_INVALID_ARGUMENT;
     return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out, nullptr, nullptr, bias);
+}
+
+afhip_status afhip_compute_linear_activation(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
+                                             const afhip_tensor* bias, int activation, size_t rows, size_t in_dim,
+                                             size_t out_dim, afhip_tensor** out) {
+    if (!bias || activation < AFHIP_ACTIVATION_NONE || activation > AFHIP_ACTIVATION_GELU) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out, nullptr, nullptr, bias, nullptr, nullptr,
+                               activation);
+}
+
+afhip_status afhip_compute_linear_add(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight,
+                                      const afhip_tensor* bias, const afhip_tensor* residual, size_t rows, size_t in_dim,
+                                      size_t out_dim, afhip_tensor** out) {
+    if (!bias || !residual) return AFHIP_ERR_INVALID_ARGUMENT;
+    return linear_no_bias_impl(self, input, weight, rows, in_dim, out_dim, -1, out, nullptr, nullptr, bias, nullptr, residual);
 }
 
 afhip_status afhip_compute_linear_pair(afhip_compute* self, const afhip_tensor* input, const afhip_tensor* weight_a,

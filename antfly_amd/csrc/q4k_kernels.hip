@@ -105,8 +105,7 @@ __device__ __forceinline__ int q4k_x_unit(int u) { return (u & ~15) | ((u + ((u 
 template <int kRows, int kCols>
 __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void gemv_q4k_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                                           const uint8_t* __restrict__ weight, int in_dim,
-                                                                          int out_dim, int slices,
-                                                                          const float* __restrict__ bias) {
+                                                                          int out_dim, int slices, Epilogue ep) {
     constexpr int kCells = kRows * kCols;
     constexpr int kXPre = 2;  // 16-byte units of a row of X a thread has in flight at once
     extern __shared__ __align__(16) unsigned char lds[];
@@ -258,7 +257,8 @@ __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void ge
     const bool mine = lane < kPadded && cell < kCells;
     if (slices == 1) {
         if (active && mine && o0 + cc < out_dim)
-            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] = bias != nullptr ? red[0] + bias[o0 + cc] : red[0];
+            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] =
+                finish_output(ep, o0 + cc, static_cast<size_t>(cr) * out_dim + o0 + cc, red[0]);
         return;
     }
     if (mine) partial[wave * kCells + cell] = red[0];
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(512, kRows == 1 ? 3 : (kRows == 2 ? 2 : 1)) void ge
         const int o = (blockIdx.x * groups_per_wg + gi) * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
-        if (o < out_dim) dst[static_cast<size_t>(r) * out_dim + o] = bias != nullptr ? total + bias[o] : total;
+        if (o < out_dim) dst[static_cast<size_t>(r) * out_dim + o] = finish_output(ep, o, static_cast<size_t>(r) * out_dim + o, total);
     }
 }
 
@@ -292,7 +292,7 @@ size_t q4k_lds_bytes(int rows, int in_dim) { return static_cast<size_t>(rows) * 
 
 template <int kRows>
 hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int in_dim, int out_dim,
-                           const float* bias) {
+                           const Epilogue& ep) {
     constexpr int kCols = 2;
     const int kb = in_dim / kQ4kBlockValues;
     const int groups = (out_dim + kCols - 1) / kCols;
@@ -327,7 +327,7 @@ hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const
             return e;
         large_lds = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, in_dim, out_dim, slices, bias);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, in_dim, out_dim, slices, ep);
     return hipGetLastError();
 }
 
@@ -337,7 +337,7 @@ hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const
 int gemv_q4k_max_in_dim() { return 8 * 8 * kQ4kBlockValues; }
 
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                           int out_dim, const float* bias) {
+                           int out_dim, const Epilogue& ep0) {
     if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
     // up to four rows per launch while X fits LDS; more rows walk the weights again (from the
     // Infinity Cache when the matrix fits)
@@ -347,12 +347,14 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
         const int nr = rows - r0 < per_launch ? rows - r0 : per_launch;
         float* d = dst + static_cast<size_t>(r0) * out_dim;
         const float* xr = x + static_cast<size_t>(r0) * in_dim;
+        Epilogue ep = ep0;
+        if (ep.residual) ep.residual += static_cast<size_t>(r0) * out_dim;
         hipError_t e;
         switch (nr) {
-            case 1: e = launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim, bias); break;
-            case 2: e = launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim, bias); break;
-            case 3: e = launch_q4k_rows<3>(stream, d, xr, weight, in_dim, out_dim, bias); break;
-            default: e = launch_q4k_rows<4>(stream, d, xr, weight, in_dim, out_dim, bias); break;
+            case 1: e = launch_q4k_rows<1>(stream, d, xr, weight, in_dim, out_dim, ep); break;
+            case 2: e = launch_q4k_rows<2>(stream, d, xr, weight, in_dim, out_dim, ep); break;
+            case 3: e = launch_q4k_rows<3>(stream, d, xr, weight, in_dim, out_dim, ep); break;
+            default: e = launch_q4k_rows<4>(stream, d, xr, weight, in_dim, out_dim, ep); break;
         }
         if (e != hipSuccess) return e;
     }

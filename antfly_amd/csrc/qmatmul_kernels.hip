@@ -28,7 +28,7 @@ template <typename Weights>
 __global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict__ dst,
                                                               const float* __restrict__ input, Weights w,
                                                               int rows, int in_dim, int out_dim,
-                                                              const float* __restrict__ bias) {
+                                                              Epilogue ep) {
     const int o = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
     const int kb = in_dim >> 5;
     const float* x = input + static_cast<size_t>(r) * in_dim;
@@ -49,7 +49,7 @@ __global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict_
         acc += blk.d * part;
     }
     acc = wave_sum(acc);
-    if (lane == 0) dst[static_cast<size_t>(r) * out_dim + o] = bias != nullptr ? acc + bias[o] : acc;
+    if (lane == 0) dst[static_cast<size_t>(r) * out_dim + o] = finish_output(ep, o, static_cast<size_t>(r) * out_dim + o, acc);
 }
 
 // Route A from pre-quantized activations.  grid = (out_dim, rows), block = 64.
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(64) void linear_act_generic_kernel(float* __restric
                                                                 const int8_t* __restrict__ qx,
                                                                 const float* __restrict__ sx, Weights w,
                                                                 int rows, int in_dim, int out_dim,
-                                                                const float* __restrict__ bias) {
+                                                                Epilogue ep) {
     const int o = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
     const int kb = in_dim >> 5;
     float acc = 0.0f;
@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64) void linear_act_generic_kernel(float* __restric
         acc += t * static_cast<float>(dot);
     }
     acc = wave_sum(acc);
-    if (lane == 0 && dst) dst[static_cast<size_t>(r) * out_dim + o] = bias != nullptr ? acc + bias[o] : acc;
+    if (lane == 0 && dst) dst[static_cast<size_t>(r) * out_dim + o] = finish_output(ep, o, static_cast<size_t>(r) * out_dim + o, acc);
 }
 
 // Stand-alone activation quantizer (ops/native_compute.zig:11998-12028,
@@ -350,21 +350,21 @@ hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int r
 template <typename Weights>
 static hipError_t launch_generic(hipStream_t stream, bool route_a, float* dst, int* dots, const float* input,
                                  const int8_t* qx, const float* sx, Weights w, int rows, int in_dim, int out_dim,
-                                 const float* bias) {
+                                 const Epilogue& ep) {
     dim3 grid(out_dim, rows);
     if (route_a) {
         hipLaunchKernelGGL(linear_act_generic_kernel<Weights>, grid, dim3(64), 0, stream, dst, dots, qx, sx, w, rows,
-                           in_dim, out_dim, bias);
+                           in_dim, out_dim, ep);
     } else {
         hipLaunchKernelGGL(linear_f32_route_kernel<Weights>, grid, dim3(64), 0, stream, dst, input, w, rows, in_dim,
-                           out_dim, bias);
+                           out_dim, ep);
     }
     return launch_status();
 }
 
 hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout, bool route_a, float* dst, int* dots,
                                  const float* input, const int8_t* qx, const float* sx, const uint8_t* weight,
-                                 int rows, int in_dim, int out_dim, const float* bias) {
+                                 int rows, int in_dim, int out_dim, const Epilogue& ep0) {
     const size_t blocks = static_cast<size_t>(out_dim) * (in_dim / 32);
     // grid.y is limited to 65535 rows per launch
     for (int r0 = 0; r0 < rows; r0 += 32768) {
@@ -374,18 +374,20 @@ hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout
         const float* in = input ? input + static_cast<size_t>(r0) * in_dim : nullptr;
         const int8_t* q = qx ? qx + static_cast<size_t>(r0) * in_dim : nullptr;
         const float* s = sx ? sx + static_cast<size_t>(r0) * (in_dim / 32) : nullptr;
+        Epilogue ep = ep0;
+        if (ep.residual) ep.residual += static_cast<size_t>(r0) * out_dim;
         hipError_t e;
         if (layout == 0) {
-            if (tensor_type == 2) e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<2>{weight}, nr, in_dim, out_dim, bias);
-            else e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<8>{weight}, nr, in_dim, out_dim, bias);
+            if (tensor_type == 2) e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<2>{weight}, nr, in_dim, out_dim, ep);
+            else e = launch_generic(stream, route_a, d, dd, in, q, s, RawWeights<8>{weight}, nr, in_dim, out_dim, ep);
         } else {
             const uint4* qs = reinterpret_cast<const uint4*>(weight);
             if (tensor_type == 2) {
                 PreparedWeights<2> w{qs, reinterpret_cast<const uint16_t*>(weight + blocks * 16)};
-                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim, bias);
+                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim, ep);
             } else {
                 PreparedWeights<8> w{qs, reinterpret_cast<const uint16_t*>(weight + blocks * 32)};
-                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim, bias);
+                e = launch_generic(stream, route_a, d, dd, in, q, s, w, nr, in_dim, out_dim, ep);
             }
         }
         if (e != hipSuccess) return e;

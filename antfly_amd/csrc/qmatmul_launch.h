@@ -7,6 +7,17 @@
 
 namespace afhip {
 
+// What the kernel that writes Y does to each total before storing it: + bias[o], then the
+// activation, then + residual[r][o] -- the engine's linear / linearRelu / linearQuickGelu /
+// linearGelu / linearAdd (ops/ops.zig:1728, :2164-2230), in the order of the CUDA backend's
+// kernels (bias, activation or residual).  Nothing set: the total is stored as it is.
+enum : int { kActNone = 0, kActRelu = 1, kActQuickGelu = 2, kActGelu = 3 };
+struct Epilogue {
+    const float* bias = nullptr;      // [out_dim]
+    const float* residual = nullptr;  // [rows][out_dim]
+    int activation = kActNone;
+};
+
 // Launch geometry of the fused GEMV; chosen host-side (ops/cuda/kernels.zig
 // does the same for its launch1d / launchBlocks helpers).
 struct GemvTuning {
@@ -27,13 +38,13 @@ struct GemvActivations {
 
 // rows in 1..16, weight in PREPARED layout, dots optional (int32 [rows][out][in/32]).
 // weight_b_prepared / dst_b (optional): a second matrix of the same shape that shares X,
-// computed by the same launch (not together with dots).  bias / bias_b (optional, f32
-// [out_dim]) are added to every row of dst / dst_b.
+// computed by the same launch (not together with dots).  ep / ep_b: what happens to the
+// totals of dst / dst_b before they are stored (residual rows are relative to this launch's rows).
 hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
                              const GemvActivations& pre, const uint8_t* weight_prepared, int rows, int in_dim,
                              int out_dim, const GemvTuning& tune, float* dst_b = nullptr,
-                             const uint8_t* weight_b_prepared = nullptr, const float* bias = nullptr,
-                             const float* bias_b = nullptr);
+                             const uint8_t* weight_b_prepared = nullptr, const Epilogue& ep = Epilogue{},
+                             const Epilogue& ep_b = Epilogue{});
 
 // One row, no Y: every workgroup leaves the argmax key (see argmax_key) of its output
 // columns in keys[workgroup]; *key_count receives the number of workgroups, which is at
@@ -43,20 +54,18 @@ hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned
                                    const GemvTuning& tune);
 
 // Int8-MFMA GEMM on pre-quantized activations (natural order) and PREPARED
-// weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set;
-// bias optional (f32 [out_dim], added to every row).
+// weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set.
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
                           const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
-                          const float* bias = nullptr);
+                          const Epilogue& ep = Epilogue{});
 
 hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
                                        float* scale, int* sum);
 
 // Any layout / shape.  route_a: uses qx/sx (pre-quantized), else f32 `input`.
-// bias optional (f32 [out_dim], added to every row).
 hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout, bool route_a, float* dst, int* dots,
                                  const float* input, const int8_t* qx, const float* sx, const uint8_t* weight,
-                                 int rows, int in_dim, int out_dim, const float* bias = nullptr);
+                                 int rows, int in_dim, int out_dim, const Epilogue& ep = Epilogue{});
 
 hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
                                  size_t blocks);
@@ -75,7 +84,7 @@ hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* ds
 // cpy_q_to_f32.
 int gemv_q4k_max_in_dim();
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                           int out_dim, const float* bias = nullptr);
+                           int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
                                       size_t rows, int dim);
 

@@ -186,6 +186,38 @@ class HipCompute:
                                               C.byref(h)))
         return HipTensor(h.value)
 
+    def _linear_activation(self, activation, input, weight, bias, rows, in_dim, out_dim):
+        h = C.c_void_p()
+        rc = _lib.lib().afhip_compute_linear_activation(self._h, input.handle, weight.handle, bias.handle, activation, rows,
+                                                        in_dim, out_dim, C.byref(h))
+        if rc == _lib.ERR_OP_UNSUPPORTED:
+            return None  # the engine's optional fast path: the caller composes linear + activation
+        check(rc)
+        return HipTensor(h.value)
+
+    def linearRelu(self, input: HipTensor, weight: HipTensor, bias: HipTensor, rows: int, in_dim: int, out_dim: int):
+        """ops/ops.zig:2177: relu(X @ W^T + bias), or None when this weight has no fused path."""
+        return self._linear_activation(_lib.ACTIVATION_RELU, input, weight, bias, rows, in_dim, out_dim)
+
+    def linearQuickGelu(self, input: HipTensor, weight: HipTensor, bias: HipTensor, rows: int, in_dim: int, out_dim: int):
+        """ops/ops.zig:2164: y / (1 + exp(-1.702 y)) of y = X @ W^T + bias, or None."""
+        return self._linear_activation(_lib.ACTIVATION_QUICK_GELU, input, weight, bias, rows, in_dim, out_dim)
+
+    def linearGelu(self, input: HipTensor, weight: HipTensor, bias: HipTensor, rows: int, in_dim: int, out_dim: int):
+        """ops/ops.zig:2205: tanh-form gelu of X @ W^T + bias, or None."""
+        return self._linear_activation(_lib.ACTIVATION_GELU, input, weight, bias, rows, in_dim, out_dim)
+
+    def linearAdd(self, input: HipTensor, weight: HipTensor, bias: HipTensor, residual: HipTensor, rows: int, in_dim: int,
+                  out_dim: int):
+        """ops/ops.zig:2218: X @ W^T + bias + residual, or None when this weight has no fused path."""
+        h = C.c_void_p()
+        rc = _lib.lib().afhip_compute_linear_add(self._h, input.handle, weight.handle, bias.handle, residual.handle, rows,
+                                                 in_dim, out_dim, C.byref(h))
+        if rc == _lib.ERR_OP_UNSUPPORTED:
+            return None
+        check(rc)
+        return HipTensor(h.value)
+
     def linearPair(self, input: HipTensor, weight_a: HipTensor, bias_a: HipTensor, weight_b: HipTensor,
                    bias_b: HipTensor, rows: int, in_dim: int, out_dim: int):
         """ops/ops.zig:915, :1846-1885: (first, second) = (X @ Wa^T + ba, X @ Wb^T + bb)."""

@@ -34,6 +34,14 @@ def launchLinearBiasF32(stream, tensor_type, layout, dst: Buffer, input: Buffer,
                                                   out_dim, workspace, dispatch))
 
 
+def launchLinearEpilogueF32(stream, tensor_type, layout, dst: Buffer, input: Buffer, weight: Buffer, rows, in_dim, out_dim,
+                            bias: Buffer = NO_BUFFER, residual: Buffer = NO_BUFFER, activation: int = 0,
+                            workspace: Buffer = NO_BUFFER, dispatch: int = -1) -> None:
+    """Y = act(X @ W^T + bias) + residual, all by the kernel that writes Y (bias, residual optional)."""
+    check(_lib.lib().afhip_launch_linear_epilogue_f32(stream, tensor_type, layout, dst, input, weight, bias, residual,
+                                                      activation, rows, in_dim, out_dim, workspace, dispatch))
+
+
 def launchLinearPairBiasF32(stream, tensor_type, layout, dst_a: Buffer, dst_b: Buffer, input: Buffer, weight_a: Buffer,
                             bias_a: Buffer, weight_b: Buffer, bias_b: Buffer, rows, in_dim, out_dim,
                             workspace: Buffer = NO_BUFFER, dispatch: int = -1) -> None:

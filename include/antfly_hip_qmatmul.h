@@ -150,6 +150,26 @@ afhip_status afhip_launch_linear_bias_f32(void *stream, int tensor_type, int lay
                                           afhip_buffer input, afhip_buffer weight, afhip_buffer bias,
                                           size_t rows, size_t in_dim, size_t out_dim,
                                           afhip_buffer workspace, int dispatch);
+/* What follows the bias in the fused linear ops of the backend interface (linearRelu,
+ * linearQuickGelu, linearGelu; ops/ops.zig:2164-2216).  Formulas as in the CUDA backend's
+ * kernels (ops/cuda/artifacts/inference_cuda_kernels.cu:140-146, :1006-1012) and the CPU
+ * activations (backends/activations.zig:43-62, :64-80, :112-127): relu y < 0 ? 0 : y;
+ * quick_gelu y / (1 + exp(-1.702 y)); gelu 0.5 y (1 + tanh(0.7978845608 (y + 0.044715 y^3))). */
+enum afhip_activation {
+    AFHIP_ACTIVATION_NONE = 0,
+    AFHIP_ACTIVATION_RELU = 1,
+    AFHIP_ACTIVATION_QUICK_GELU = 2,
+    AFHIP_ACTIVATION_GELU = 3
+};
+/* Y = act(X * W^T + bias) + residual, all of it by the kernel that writes Y: bias (f32
+ * [out_dim]) and residual (f32 [rows, out_dim]) are optional (.ptr == 0), applied in that
+ * order (linearAdd, ops/ops.zig:2218-2230: bias, then the residual; the CUDA kernels'
+ * MODE 1-4 epilogues).  With nothing set this is afhip_launch_linear_f32. */
+afhip_status afhip_launch_linear_epilogue_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                              afhip_buffer input, afhip_buffer weight, afhip_buffer bias,
+                                              afhip_buffer residual, int activation, size_t rows,
+                                              size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                              int dispatch);
 /* Two biased matmuls that share X (linearPair, ops/ops.zig:915, wrapper :1846-1885; CPU op
  * ops/native_compute.zig:6513ff): afhip_launch_linear_pair_f32 with bias_a / bias_b added. */
 afhip_status afhip_launch_linear_pair_bias_f32(void *stream, int tensor_type, int layout,
@@ -347,6 +367,23 @@ afhip_status afhip_compute_linear_triple(afhip_compute *self, const afhip_tensor
                                          size_t rows, size_t in_dim, size_t out_dim,
                                          afhip_tensor **out_first, afhip_tensor **out_second,
                                          afhip_tensor **out_third);
+
+/* linearRelu / linearQuickGelu / linearGelu, ops/ops.zig:2164-2216 (CUDA backend
+ * cuda_compute.zig:582-656): act(X * W^T + bias) in one op.  The engine treats these as
+ * optional fast paths (a backend answers null and the caller composes linear + activation);
+ * here every quantized format of afhip_compute_linear_no_bias is served, a dense f32 weight
+ * answers AFHIP_ERR_OP_UNSUPPORTED (the binding's null).  `activation` is an afhip_activation. */
+afhip_status afhip_compute_linear_activation(afhip_compute *self, const afhip_tensor *input,
+                                             const afhip_tensor *weight, const afhip_tensor *bias,
+                                             int activation, size_t rows, size_t in_dim, size_t out_dim,
+                                             afhip_tensor **out);
+
+/* linearAdd, ops/ops.zig:2218-2230 (CUDA backend cuda_compute.zig:658-688): X * W^T + bias +
+ * residual with an f32 residual tensor of rows * out_dim elements. */
+afhip_status afhip_compute_linear_add(afhip_compute *self, const afhip_tensor *input,
+                                      const afhip_tensor *weight, const afhip_tensor *bias,
+                                      const afhip_tensor *residual, size_t rows, size_t in_dim,
+                                      size_t out_dim, afhip_tensor **out);
 
 /* linearNoBiasGrouped, ops/ops.zig:901 (wrapper :1786-1800): `weight` is already the
  * concatenation of `num_projections` matrices along the output axis, so this is one

@@ -69,6 +69,8 @@ def lib() -> C.CDLL:
         L.afo_argmax_last_row.argtypes = [vp, sz, sz]
         L.afo_add_linear_bias_rows.restype = None
         L.afo_add_linear_bias_rows.argtypes = [vp, vp, sz, sz]
+        L.afo_apply_activation.restype = None
+        L.afo_apply_activation.argtypes = [i32, vp, sz]
         L.afo_linear_act_f64.argtypes = [i32, vp, vp, vp, sz, sz, sz]
         L.afo_thread_plan.argtypes = [sz, sz, sz, i32, i32, vp]
         L.afo_prepare.restype = vp
@@ -211,6 +213,16 @@ def add_linear_bias_rows(y, bias, rows, out_dim) -> np.ndarray:
 def linear(fmt, x, w_raw, bias, rows, in_dim, out_dim, workers=1) -> np.ndarray:
     """The engine's biased `linear` on a quantized weight: the no-bias op, then the bias rows."""
     return add_linear_bias_rows(linear_no_bias(fmt, x, w_raw, rows, in_dim, out_dim, workers), bias, rows, out_dim)
+
+
+RELU, QUICK_GELU, GELU = 1, 2, 3
+
+
+def apply_activation(kind: int, y) -> np.ndarray:
+    """relu / quick_gelu / tanh-form gelu of every element (a new array)."""
+    out = np.array(_f32(y), dtype=np.float32).copy()
+    lib().afo_apply_activation(kind, _p(out), out.size)
+    return out
 
 
 def linear_act_f64(fmt, x, w_raw, rows, in_dim, out_dim) -> np.ndarray:

@@ -459,6 +459,21 @@ void afo_add_linear_bias_rows(float *y, const float *bias, size_t rows, size_t o
         for (size_t o = 0; o < out_dim; o++) y[r * out_dim + o] += bias[o];
 }
 
+void afo_apply_activation(int kind, float *y, size_t n) {
+    for (size_t i = 0; i < n; i++) {
+        float v = y[i];
+        if (kind == 1) { /* activations.zig:76-79 */
+            if (v < 0.0f) v = 0.0f;
+        } else if (kind == 2) { /* :123-126 */
+            v = v / (1.0f + expf(-1.702f * v));
+        } else if (kind == 3) { /* :57-61 */
+            float inner = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+            v = 0.5f * v * (1.0f + tanhf(inner));
+        }
+        y[i] = v;
+    }
+}
+
 int afo_linear_act_f64(int fmt, const float *x, const uint8_t *w, double *y, size_t rows,
                        size_t in_dim, size_t out_dim) {
     size_t bb = afo_block_bytes(fmt);

@@ -92,6 +92,11 @@ int afo_linear_no_bias(int fmt, const float *x, const uint8_t *w_raw, float *y,
  * (dispatchQuantizedLinear .single_bias, :5065-5077; .pair_bias falls back to it, :5110-5111). */
 void afo_add_linear_bias_rows(float *y, const float *bias, size_t rows, size_t out_dim);
 
+/* Activations applied after the bias by linearRelu / linearQuickGelu / linearGelu
+ * (backends/activations.zig: relu :64-80, quickGelu :112-127, gelu :43-62; scalar forms).
+ * kind: 1 relu, 2 quick_gelu, 3 gelu (tanh form).  In place. */
+void afo_apply_activation(int kind, float *y, size_t n);
+
 int afo_linear_act_f64(int fmt, const float *x, const uint8_t *w_raw, double *y,
                        size_t rows, size_t in_dim, size_t out_dim);
 

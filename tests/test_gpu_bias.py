@@ -96,6 +96,64 @@ def test_q4_k_bias(rows):
     assert G.max_rel_err(y, ref.astype(np.float64)) <= TIGHT
 
 
+def linear_epilogue(fmt, layout, x, w_dev, rows, in_dim, out_dim, bias=None, residual=None, activation=0, dispatch=-1):
+    xd = G.to_dev(x.astype(np.float32))
+    keep = [xd]
+    bb = rb = kernels.NO_BUFFER
+    if bias is not None:
+        keep.append(G.to_dev(bias.astype(np.float32)))
+        bb = G.buf(keep[-1])
+    if residual is not None:
+        keep.append(G.to_dev(residual.astype(np.float32)))
+        rb = G.buf(keep[-1])
+    y = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=G.DEV)
+    ws = torch.empty(max(kernels.workspaceBytes(fmt, rows, in_dim, out_dim), 16), dtype=torch.uint8, device=G.DEV)
+    kernels.launchLinearEpilogueF32(G.stream(), fmt, layout, G.buf(y), G.buf(xd), G.buf(w_dev), rows, in_dim, out_dim, bb, rb,
+                                    activation, G.buf(ws), dispatch)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+EPILOGUE_SHAPES = [(1, 4096, 1024), (1, 8224, 513), (3, 1024, 600), (6, 2048, 640), (40, 512, 640), (300, 512, 1024),
+                   (3, 64, 100)]
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4, Q4K])
+@pytest.mark.parametrize("rows,in_dim,out_dim", EPILOGUE_SHAPES)
+def test_fused_epilogues(fmt, rows, in_dim, out_dim):
+    """linearRelu / linearQuickGelu / linearGelu / linearAdd (ops/ops.zig:2164-2230): the stored value is
+    act(product + bias) + residual.  relu and the residual add are exact functions of the bias op's
+    value; the two gelus are checked against the oracle's formulas applied to that value."""
+    if fmt == Q4K and in_dim % 256 != 0:
+        pytest.skip("Q4_K rows are whole 256-value super-blocks")
+    layout = RAW if fmt == Q4K else PREP
+    print(f"case: fused epilogues fmt={fmt} rows={rows} in={in_dim} out={out_dim}", flush=True)
+    x = synth.activations(650 + rows, rows, in_dim) * 4.0
+    w = synth.weights(fmt, 651, out_dim, in_dim)
+    b = bias_vector(652, out_dim)
+    res = synth.activations(653, rows, out_dim)
+    wd = G.to_dev(w) if fmt == Q4K else G.prepare(fmt, w, out_dim, in_dim)
+    biased = G.linear_bias(fmt, layout, x, wd, b, rows, in_dim, out_dim)
+    plain = G.linear(fmt, layout, x, wd, rows, in_dim, out_dim)
+    assert np.array_equal(linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim), plain)  # nothing set: the plain op
+    assert (biased < 0).any() and (biased > 0).any()
+    relu = linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim, bias=b, activation=_lib.ACTIVATION_RELU)
+    assert np.array_equal(relu, np.maximum(biased, 0))
+    add = linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim, bias=b, residual=res)
+    assert np.array_equal(add, biased + res)
+    assert np.array_equal(linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim, residual=res), plain + res)
+    for act, kind in ((_lib.ACTIVATION_QUICK_GELU, O.QUICK_GELU), (_lib.ACTIVATION_GELU, O.GELU)):
+        got = linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim, bias=b, activation=act)
+        want = O.apply_activation(kind, biased)
+        assert np.allclose(got, want, rtol=3e-6, atol=1e-6 * np.abs(biased).max()), (act, np.abs(got - want).max())
+    both = linear_epilogue(fmt, layout, x, wd, rows, in_dim, out_dim, bias=b, residual=res, activation=_lib.ACTIVATION_RELU)
+    assert np.array_equal(both, np.maximum(biased, 0) + res)
+    # end to end against the engine's CPU definition
+    if fmt != Q4K:
+        ref = O.apply_activation(O.RELU, O.linear(fmt, x, w, b, rows, in_dim, out_dim, workers=8))
+        assert G.max_rel_err(relu, ref.astype(np.float64)) <= TIGHT
+
+
 def test_bias_argument_errors():
     rows, in_dim, out_dim = 2, 512, 512
     x = G.to_dev(synth.activations(1, rows, in_dim))
@@ -109,7 +167,59 @@ def test_bias_argument_errors():
     with pytest.raises(_lib.InvalidHipState):
         kernels.launchLinearBiasF32(G.stream(), Q8, RAW, G.buf(y), G.buf(x), G.buf(w), kernels.NO_BUFFER, rows, in_dim,
                                     out_dim, G.buf(ws))
+    # a residual shorter than Y, an activation that does not exist, activation on a pair
+    res = torch.zeros(rows * out_dim - 1, device=G.DEV)
+    bias = torch.zeros(out_dim, device=G.DEV)
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchLinearEpilogueF32(G.stream(), Q8, RAW, G.buf(y), G.buf(x), G.buf(w), rows, in_dim, out_dim, G.buf(bias),
+                                        G.buf(res), 0, G.buf(ws))
+    with pytest.raises(_lib.HipError):
+        kernels.launchLinearEpilogueF32(G.stream(), Q8, RAW, G.buf(y), G.buf(x), G.buf(w), rows, in_dim, out_dim, G.buf(bias),
+                                        kernels.NO_BUFFER, 7, G.buf(ws))
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4, Q4K])
+def test_backend_fused_linear_ops(fmt):
+    """ComputeBackend linearRelu / linearQuickGelu / linearGelu / linearAdd: a fused op equals the
+    composition of the backend's own `linear` with the activation / the add."""
+    rows, in_dim, out_dim = 3, 1024, 768
+    print(f"case: backend fused linear ops fmt={fmt}", flush=True)
+    cb = HipCompute()
+    try:
+        x = synth.activations(660, rows, in_dim) * 4.0
+        w = synth.weights(fmt, 661, out_dim, in_dim)
+        b, res = bias_vector(662, out_dim), synth.activations(663, rows, out_dim)
+        cb.insertWeightFromLoaded("blk.0.ffn_up.weight", fmt, w, [out_dim, in_dim])
+        wt = cb.getWeight("blk.0.ffn_up.weight")
+        xt, bt, rt = cb.fromFloat32(x, [rows, in_dim]), cb.fromFloat32(b, [out_dim]), cb.fromFloat32(res, [rows, out_dim])
+        lin = cb.linear(xt, wt, bt, rows, in_dim, out_dim)
+        base = cb.toFloat32(lin).reshape(rows, out_dim)
+
+        def values(t):
+            assert t is not None and t.shape == [rows, out_dim]
+            out = cb.toFloat32(t).reshape(rows, out_dim)
+            cb.freeTensor(t)
+            return out
+
+        assert np.array_equal(values(cb.linearRelu(xt, wt, bt, rows, in_dim, out_dim)), np.maximum(base, 0))
+        assert np.array_equal(values(cb.linearAdd(xt, wt, bt, rt, rows, in_dim, out_dim)), base + res)
+        scale = 1e-6 * np.abs(base).max()
+        assert np.allclose(values(cb.linearQuickGelu(xt, wt, bt, rows, in_dim, out_dim)),
+                           O.apply_activation(O.QUICK_GELU, base), rtol=3e-6, atol=scale)
+        assert np.allclose(values(cb.linearGelu(xt, wt, bt, rows, in_dim, out_dim)), O.apply_activation(O.GELU, base),
+                           rtol=3e-6, atol=scale)
+        # a dense f32 weight has no fused path here: the optional op answers None
+        cb.insertWeightFromTensor("dense.weight", np.zeros((4, in_dim), np.float32), [4, in_dim])
+        dense = cb.getWeight("dense.weight")
+        b4 = cb.fromFloat32(np.zeros(4, np.float32), [4])
+        assert cb.linearRelu(xt, dense, b4, rows, in_dim, 4) is None
+        with pytest.raises(_lib.InvalidShape):
+            cb.linearAdd(xt, wt, bt, bt, rows, in_dim, out_dim)  # residual of the wrong size
+        for t in (lin, xt, bt, rt, b4):
+            cb.freeTensor(t)
+    finally:
+        cb.deinit()
 
 
 @pytest.mark.parametrize("fmt", [Q8, Q4])

@@ -429,6 +429,26 @@ def test_biased_linear_is_the_no_bias_op_plus_bias_rows():
         assert np.array_equal(O.linear(fmt, x, w, bias, rows, in_dim, out_dim), plain + bias[None, :])
 
 
+def test_activations_against_float64_closed_forms():
+    """relu / quick_gelu / tanh-form gelu (backends/activations.zig:43-127) against the formulas in
+    float64, plus the values the mathematics fixes: f(0) = 0, f(x) -> x for large x, -> 0 for
+    very negative x, gelu(x) - gelu(-x) = x, quick_gelu(x) - quick_gelu(-x) = x."""
+    x = np.concatenate([np.linspace(-12, 12, 4801), [0.0, 1e-6, -1e-6, 30.0, -30.0, 88.0, -88.0]]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    assert np.array_equal(O.apply_activation(O.RELU, x), np.maximum(x, 0))
+    qg = O.apply_activation(O.QUICK_GELU, x)
+    assert np.allclose(qg, x64 / (1 + np.exp(-1.702 * x64)), rtol=2e-6, atol=1e-30)
+    g = O.apply_activation(O.GELU, x)
+    assert np.allclose(g, 0.5 * x64 * (1 + np.tanh(0.7978845608028654 * (x64 + 0.044715 * x64 ** 3))), rtol=2e-6, atol=1e-7)
+    for kind in (O.RELU, O.QUICK_GELU, O.GELU):
+        y = O.apply_activation(kind, np.float32([0.0, 30.0, -30.0]))
+        assert y[0] == 0 and y[1] == 30.0 and abs(y[2]) < 1e-20
+    for got in (qg, g):  # f(x) - f(-x) = x: pairs of the symmetric grid
+        sym = got[:4801]
+        assert np.allclose(sym - sym[::-1], x[:4801], rtol=1e-5, atol=1e-6)
+    assert np.array_equal(O.apply_activation(0, x), x)
+
+
 def test_synth_is_chunk_invariant_and_in_range():
     a = synth.splitmix64(42, 0, 1000)
     b = np.concatenate([synth.splitmix64(42, 0, 333), synth.splitmix64(42, 333, 667)])
