@@ -82,18 +82,21 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
 }
 
 // Q4_K: f32 activations against the dequantized weights, one kernel family for any row count.
-static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
+static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                     size_t rows, size_t in_dim, size_t out_dim, int dispatch, bool want_dots,
                                     LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b,
                                     const Epilogue& ep, const Epilogue& ep_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // this format has no integer route
     if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
     if (in_dim == 0 || in_dim % 256 != 0) return AFHIP_ERR_INVALID_STATE;
+    const bool tiled = layout == AFHIP_LAYOUT_PREPARED;
     size_t out_count, in_count, w_blocks, w_bytes, bytes;
     if (!checked_mul(rows, out_dim, &out_count) || !checked_mul(rows, in_dim, &in_count) ||
-        !checked_mul(out_dim, in_dim / 256, &w_blocks) || !checked_mul(w_blocks, 144, &w_bytes))
+        !checked_mul(out_dim + (tiled ? 31 : 0), in_dim / 256, &w_blocks) || !checked_mul(w_blocks, 144, &w_bytes))
         return AFHIP_ERR_INVALID_STATE;
+    if (tiled) w_bytes = q4k_tiled_bytes(out_dim, in_dim);
     if (!checked_mul(out_count, 4, &bytes) || bytes > dst.len || (pair && bytes > dst_b.len)) return AFHIP_ERR_INVALID_STATE;
     if (!checked_mul(in_count, 4, &bytes) || bytes > input.len) return AFHIP_ERR_INVALID_STATE;
     if (w_bytes > weight.len || (pair && w_bytes > weight_b.len)) return AFHIP_ERR_INVALID_STATE;
@@ -111,11 +114,10 @@ static afhip_status linear_q4k_impl(hipStream_t stream, afhip_buffer dst, afhip_
             else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
             else counters->mm++;
         }
-        hipError_t e = launch_gemv_q4k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
-                                       reinterpret_cast<const float*>(input.ptr),
-                                       reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
-                                       static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
-                                       i ? ep_b : ep);
+        hipError_t e = (tiled ? launch_gemv_q4k_tiled : launch_gemv_q4k)(
+            stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const float*>(input.ptr),
+            reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), static_cast<int>(rows), static_cast<int>(in_dim),
+            static_cast<int>(out_dim), i ? ep_b : ep);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
     }
     return AFHIP_OK;
@@ -151,8 +153,8 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     ep.activation = extras.activation;  // AFHIP_ACTIVATION_* and kAct* share their values
     ep_b.bias = reinterpret_cast<const float*>(extras.bias_b.ptr);
     if (tensor_type == AFHIP_TYPE_Q4_K)
-        return linear_q4k_impl(stream, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters, dst_b,
-                               weight_b, ep, ep_b);
+        return linear_q4k_impl(stream, layout, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters,
+                               dst_b, weight_b, ep, ep_b);
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -341,8 +343,13 @@ afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip
     size_t count, bytes, w_blocks, w_bytes;
     if (!checked_mul(rows, in_dim, &count) || !checked_mul(count, 4, &bytes) || bytes > input.len)
         return AFHIP_ERR_INVALID_STATE;
-    if (!checked_mul(out_dim, in_dim / block_values, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes) || w_bytes > weight.len)
-        return AFHIP_ERR_INVALID_STATE;
+    if (!checked_mul(out_dim, in_dim / block_values, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes)) return AFHIP_ERR_INVALID_STATE;
+    if (q4k && layout == AFHIP_LAYOUT_PREPARED) {
+        if (!checked_mul(out_dim + 31, in_dim / block_values, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes))
+            return AFHIP_ERR_INVALID_STATE;
+        w_bytes = q4k_tiled_bytes(out_dim, in_dim);
+    }
+    if (w_bytes > weight.len) return AFHIP_ERR_INVALID_STATE;
     if (in_dim > 0x7fffffff || out_dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || weight.ptr == 0)
         return AFHIP_ERR_INVALID_STATE;
     if ((token_u32.ptr == 0 && token_f32.ptr == 0) ||
@@ -563,8 +570,36 @@ afhip_status afhip_launch_block_dots(void* stream, int tensor_type, int layout, 
                        dispatch, dots, nullptr);
 }
 
+size_t afhip_prepared_weight_bytes(int tensor_type, size_t out_dim, size_t in_dim) {
+    size_t blocks, bytes;
+    if (tensor_type == AFHIP_TYPE_Q4_K) {
+        if (in_dim % 256 != 0 || !checked_mul(out_dim + 31, in_dim / 256, &blocks) || !checked_mul(blocks, 144, &bytes)) return 0;
+        return q4k_tiled_bytes(out_dim, in_dim);
+    }
+    const size_t bb = block_bytes(tensor_type);
+    if (bb == 0 || in_dim % 32 != 0 || !checked_mul(out_dim, in_dim / 32, &blocks) || !checked_mul(blocks, bb, &bytes)) return 0;
+    return bytes;
+}
+
 afhip_status afhip_launch_prepare_weight(void* stream, int tensor_type, afhip_buffer dst, afhip_buffer src,
                                          size_t out_dim, size_t in_dim) {
+    if (tensor_type == AFHIP_TYPE_Q4_K) {  // tile-major layout for the MFMA kernel
+        if (in_dim == 0 || in_dim % 256 != 0) return AFHIP_ERR_INVALID_STATE;
+        size_t raw_blocks, raw_bytes;
+        if (!checked_mul(out_dim, in_dim / 256, &raw_blocks) || !checked_mul(raw_blocks, 144, &raw_bytes))
+            return AFHIP_ERR_INVALID_STATE;
+        const size_t tiled_bytes = afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim);
+        if (out_dim != 0 && tiled_bytes == 0) return AFHIP_ERR_INVALID_STATE;
+        if (raw_bytes > src.len || tiled_bytes > dst.len) return AFHIP_ERR_INVALID_STATE;
+        if (raw_blocks == 0) return AFHIP_OK;
+        if (out_dim > 0x7fffffff || in_dim > 0x7fffffff || dst.ptr == 0 || src.ptr == 0 || dst.ptr % 16 != 0 ||
+            src.ptr % 16 != 0)
+            return AFHIP_ERR_INVALID_STATE;
+        hipError_t e = launch_q4k_tile_repack(static_cast<hipStream_t>(stream), reinterpret_cast<uint8_t*>(dst.ptr),
+                                              reinterpret_cast<const uint8_t*>(src.ptr), static_cast<int>(out_dim),
+                                              static_cast<int>(in_dim));
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
@@ -660,6 +695,13 @@ static afhip_status dequantize_rows(void* stream, int tensor_type, int layout, a
     } else if (!checked_mul(w_count / block_values, bb, &w_bytes)) {
         return AFHIP_ERR_INVALID_STATE;
     }
+    const bool q4k_tiled = q4k && layout == AFHIP_LAYOUT_PREPARED;
+    if (q4k_tiled) {
+        size_t padded;
+        if (!checked_mul(weight_rows + 31, dim / block_values, &padded) || !checked_mul(padded, bb, &padded))
+            return AFHIP_ERR_INVALID_STATE;
+        w_bytes = q4k_tiled_bytes(weight_rows, dim);
+    }
     if (out_bytes > dst.len || w_bytes > weight.len || (gather && id_bytes > ids.len)) return AFHIP_ERR_INVALID_STATE;
     if (out_count == 0) return AFHIP_OK;
     if (dim > 0x7fffffff || dst.ptr == 0 || weight.ptr == 0 || dst.ptr % 16 != 0 ||
@@ -667,10 +709,9 @@ static afhip_status dequantize_rows(void* stream, int tensor_type, int layout, a
         (gather && (ids.ptr == 0 || ids.ptr % 8 != 0)))
         return AFHIP_ERR_INVALID_STATE;
     if (q4k) {
-        hipError_t e = launch_dequantize_q4k_rows(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr),
-                                                  reinterpret_cast<const uint8_t*>(weight.ptr),
-                                                  gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows,
-                                                  static_cast<int>(dim));
+        hipError_t e = (q4k_tiled ? launch_dequantize_q4k_tiled_rows : launch_dequantize_q4k_rows)(
+            static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
+            gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows, static_cast<int>(dim));
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     hipError_t e = launch_dequantize_rows(static_cast<hipStream_t>(stream), tensor_type, layout,

@@ -338,11 +338,15 @@ afhip_status afhip_compute_insert_weight_from_loaded(afhip_compute* self, const 
     // Device-side repack for the formats this backend has kernels for; any other
     // quantized type stays resident as raw bytes and is rejected at the op, like
     // the reference backend does (cuda_compute.zig:703-712).
-    const size_t bb = block_bytes(tensor_type);
-    if (!keep_raw_layout && bb != 0 && shape_len == 2 && shape[1] > 0 && shape[1] % 32 == 0 &&
-        raw_len == static_cast<size_t>(shape[0]) * static_cast<size_t>(shape[1] / 32) * bb && raw_len > 0) {
+    const bool q4k = tensor_type == AFHIP_TYPE_Q4_K;
+    const size_t bb = q4k ? 144 : block_bytes(tensor_type);
+    const int64_t block_values = q4k ? 256 : 32;
+    if (!keep_raw_layout && bb != 0 && shape_len == 2 && shape[1] > 0 && shape[1] % block_values == 0 &&
+        raw_len == static_cast<size_t>(shape[0]) * static_cast<size_t>(shape[1] / block_values) * bb && raw_len > 0) {
         afhip_buffer prepared;
-        s = alloc_device_buffer(self, raw_len, &prepared);
+        s = alloc_device_buffer(self, afhip_prepared_weight_bytes(tensor_type, static_cast<size_t>(shape[0]),
+                                                                  static_cast<size_t>(shape[1])),
+                                &prepared);
         if (s == AFHIP_OK) {
             s = afhip_launch_prepare_weight(self->stream, tensor_type, prepared, t.buffer, static_cast<size_t>(shape[0]),
                                             static_cast<size_t>(shape[1]));

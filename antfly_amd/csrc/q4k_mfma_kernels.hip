@@ -1,0 +1,430 @@
+// GGUF Q4_K on the matrix cores: a tile-major device layout and the GEMV / small-batch
+// kernel that reads it.
+//
+// The engine computes Q4_K on f32 activations against the dequantized weights
+// w = (d * sc) * q - (dmin * m) (ops/native_compute.zig:31075-31144, CUDA backend
+// ops/cuda/cuda_compute.zig:708); there is no integer route at these shapes.  Done on the
+// vector ALU that is a convert and a multiply-add per weight, which bounds the kernel by
+// instruction issue at a third of the HBM rate.  Here the per-weight work moves to
+// v_mfma_f32_32x32x16_bf16 without giving up f32 accuracy:
+//
+//   * a byte 0x0n read as an fp8 (e4m3) number is n * 2^-9 (the subnormals and the first
+//     binade of that format are one linear ramp), so v_cvt_scalef32_pk_bf16_fp8 with scale
+//     2^9 turns two masked nibbles into the bf16 numbers n exactly, two weights per instruction;
+//   * an activation x is split once per workgroup into three bf16 numbers hi + mid + lo
+//     (each the bf16 rounding of what the previous ones left over), which together carry
+//     24 mantissa bits; products of bf16 numbers are exact in the f32 accumulator;
+//   * one MFMA pair per 32 output columns and 32-value sub-block leaves, for every
+//     activation row, S = sum(n * x); with X = sum(x) of the sub-block (computed in f32 by the
+//     prologue) the sub-block's contribution is
+//         (d sc) * S - (dmin m) * X  =  sum(x * ((d sc) n - dmin m)).
+//
+// Operand mapping (D = A * B, 32 x 32 x 16): A rows are "x columns" -- row r of X occupies
+// x columns 8 (r / 2) + 4 (r % 2) + {0, 1, 2} for its three parts, so that the results of
+// up to eight rows land in D registers 4 (r / 2) + part of lane half r % 2 -- and B columns
+// are 32 consecutive output columns.  Lane (column c, half g) supplies the K values
+// 16 g + 8 m + 0..7 of the sub-block to MFMA m = 0, 1.  x columns that carry nothing read an
+// all-zero column of LDS.
+//
+// Tile-major layout ("prepared" Q4_K): for every tile of 32 output columns and every
+// super-block of 256 values, 4608 bytes: the 32 headers of 16 bytes (d, dmin, 12 scale
+// bytes) and then, for each of the four 32-byte chunks of nibbles, lane c + 32 g holds bytes
+// 16 g .. 16 g + 15 of column c's chunk.  A wavefront's loads are 1 KiB contiguous each.
+// Columns past out_dim are zero (d = dmin = 0).  Same size as the raw layout when out_dim
+// is a multiple of 32.
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+
+#include <cstdlib>
+
+#include "device_common.h"
+#include "qmatmul_launch.h"
+
+namespace afhip {
+
+namespace {
+
+constexpr int kQ4kBlockBytes = 144;
+constexpr int kQ4kBlockValues = 256;
+constexpr int kTileCols = 32;
+constexpr int kTileBytes = 4608;        // 32 * 16 + 4 * 64 * 16
+constexpr int kTileUnits = kTileBytes / 16;
+constexpr int kRowPadBytes = 48;        // LDS stride of an x column: 2 K + 48 spreads the columns over the banks
+constexpr int kMaxRowsPerLaunch = 8;
+constexpr size_t kLdsBudget = 150 * 1024;
+
+typedef uint32_t t_u32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 t_bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 t_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float t_f32x2 __attribute__((ext_vector_type(2)));
+typedef float t_f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float ubyte_to_f32(uint32_t word, int index) {
+    return static_cast<float>((word >> (8 * index)) & 0xFFu);  // index is a compile-time constant at every use
+}
+
+// ------------------------------------------------------------------ layout
+__global__ __launch_bounds__(256) void q4k_tile_repack_kernel(t_u32x4* __restrict__ dst, const uint8_t* __restrict__ src,
+                                                              int out_dim, int kb, size_t units) {
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t region = u / kTileUnits;
+        const int w = static_cast<int>(u - region * kTileUnits);
+        const size_t tile = region / kb;
+        const int sb = static_cast<int>(region - tile * kb);
+        int c, offset;
+        if (w < kTileCols) {
+            c = w;
+            offset = 0;
+        } else {
+            const int q = w - kTileCols, chunk = q >> 6, lane = q & 63;
+            c = lane & 31;
+            offset = 16 + 32 * chunk + 16 * (lane >> 5);
+        }
+        const size_t o = tile * kTileCols + c;
+        t_u32x4 v = {0u, 0u, 0u, 0u};
+        if (o < static_cast<size_t>(out_dim))
+            v = *reinterpret_cast<const t_u32x4*>(src + (o * kb + sb) * kQ4kBlockBytes + offset);
+        dst[u] = v;
+    }
+}
+
+// get_rows / cpy_q_to_f32 from the tile-major layout; arithmetic as dequantizeQ4K,
+// gguf/quant_codec.zig:2624-2663 (see dequantize_q4k_rows_kernel for the raw layout).
+__global__ __launch_bounds__(256) void dequantize_q4k_tiled_rows_kernel(float* __restrict__ dst,
+                                                                        const uint8_t* __restrict__ weight,
+                                                                        const long long* __restrict__ ids, size_t rows,
+                                                                        int dim) {
+    const size_t per_row = static_cast<size_t>(dim >> 2);
+    const size_t units = rows * per_row;
+    const size_t kb = static_cast<size_t>(dim / kQ4kBlockValues);
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const size_t t = u / per_row;
+        const int g = static_cast<int>(u - t * per_row);  // group of four values in the row
+        const size_t o = static_cast<size_t>(ids ? ids[t] : static_cast<long long>(t));
+        const int v0 = (g & 63) * 4;                      // first value inside the super-block
+        const int chunk = v0 >> 6, pos = v0 & 63, byte = pos & 31;
+        const int sub = chunk * 2 + (pos >> 5);
+        const int c = static_cast<int>(o & 31);
+        const uint8_t* base = weight + ((o >> 5) * kb + (g >> 6)) * kTileBytes;
+        const t_u32x4 header = *reinterpret_cast<const t_u32x4*>(base + 16 * c);
+        const uint32_t packed =
+            *reinterpret_cast<const uint32_t*>(base + 512 + chunk * 1024 + (c + 32 * (byte >> 4)) * 16 + (byte & 15));
+        const uint32_t nib = (pos < 32 ? packed : packed >> 4) & 0x0F0F0F0Fu;
+        const int shift = (sub & 3) * 8;
+        const uint32_t a = (header.y >> shift) & 0xFFu, b = (header.z >> shift) & 0xFFu, cc = (header.w >> shift) & 0xFFu;
+        const uint32_t s = sub < 4 ? (a & 63u) : ((cc & 0x0Fu) | ((a >> 6) << 4));
+        const uint32_t m = sub < 4 ? (b & 63u) : ((cc >> 4) | ((b >> 6) << 4));
+        const float dsc = half_bits_to_f32(static_cast<uint16_t>(header.x & 0xFFFFu)) * static_cast<float>(s);
+        const float dmn = half_bits_to_f32(static_cast<uint16_t>(header.x >> 16)) * static_cast<float>(m);
+        float4 out;
+        out.x = dsc * ubyte_to_f32(nib, 0) - dmn;
+        out.y = dsc * ubyte_to_f32(nib, 1) - dmn;
+        out.z = dsc * ubyte_to_f32(nib, 2) - dmn;
+        out.w = dsc * ubyte_to_f32(nib, 3) - dmn;
+        reinterpret_cast<float4*>(dst)[u] = out;
+    }
+}
+
+// ------------------------------------------------------------------ GEMV
+// Two floats as a packed pair of bf16 numbers (round to nearest even): v_cvt_pk_bf16_f32.
+__device__ __forceinline__ uint32_t bf16_pair(float a, float b) {
+    const t_f32x2 v = {a, b};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, t_bf16x2));
+}
+
+// What a finite v leaves over after its bf16 rounding (bits in the upper half of `rounded`);
+// infinities and NaNs leave nothing (they stay in the first part alone).
+__device__ __forceinline__ float bf16_rest(float v, uint32_t rounded_high) {
+    return __builtin_fabsf(v) < __builtin_inff() ? v - __uint_as_float(rounded_high) : 0.0f;
+}
+
+// hi + mid + lo = (a, b) to 2^-25 of their size: three packed bf16 pairs.
+__device__ __forceinline__ void split3_pair(float a, float b, uint32_t* hi, uint32_t* mid, uint32_t* lo) {
+    const uint32_t h = bf16_pair(a, b);
+    const float ra = bf16_rest(a, h << 16), rb = bf16_rest(b, h & 0xFFFF0000u);
+    const uint32_t m = bf16_pair(ra, rb);
+    *hi = h;
+    *mid = m;
+    *lo = bf16_pair(ra - __uint_as_float(m << 16), rb - __uint_as_float(m & 0xFFFF0000u));
+}
+
+extern __shared__ __align__(16) unsigned char q4k_mfma_lds[];
+
+// kGroups = ceil(rows / 2) row groups (D registers 0 .. 4 kGroups - 1 are read);
+// kFlight super-blocks of weights are requested before any of them is used.
+template <int kGroups, int kFlight>
+__global__ __launch_bounds__(512) void gemv_q4k_mfma_kernel(float* __restrict__ dst, const float* __restrict__ x,
+                                                            const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                            int out_dim, int slices, int sb_per_slice, Epilogue ep) {
+    const int kb = in_dim >> 8;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int threads = static_cast<int>(blockDim.x), waves = threads >> 6;
+    const int row_stride = in_dim * 2 + kRowPadBytes;  // bytes per x column
+    unsigned char* xparts = q4k_mfma_lds;  // [rows * 3 + 1][row_stride]: the parts of every row, then a column of zeros
+    float* xsum = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows * 3 + 1) * row_stride);  // [rows][kb * 8]
+    float* partial = xsum + rows * kb * 8;                                                       // [waves][kGroups][64]
+
+    const int tiles_per_wg = waves / slices;
+    const int n_tiles = (out_dim + kTileCols - 1) >> 5;
+    const int tile_raw = blockIdx.x * tiles_per_wg + wave / slices;
+    const bool tile_ok = tile_raw < n_tiles;
+    const int tile = tile_ok ? tile_raw : n_tiles - 1;  // spare wavefronts load nothing and store nothing
+    const int slice = wave % slices;
+    const int sb_begin = slice * sb_per_slice;
+    const int sb_end = min(kb, sb_begin + sb_per_slice);
+    const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
+
+    t_u32x4 hdr[kFlight], qv[kFlight][4];
+    auto request = [&](int sb_first) {
+#pragma unroll
+        for (int f = 0; f < kFlight; ++f) {
+            const int sb = sb_first + f;
+            if (!(tile_ok && sb < sb_end)) continue;  // wave-uniform; the same test guards the use below
+            const uint8_t* base = tile_base + static_cast<size_t>(sb) * kTileBytes;
+            hdr[f] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 16 * (lane & 31)));
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                qv[f][t] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 512 + t * 1024 + 16 * lane));
+        }
+    };
+
+    // ---- 1. X: requested first, split into bf16 parts while the weights are on their way
+    const int groups_per_row = in_dim >> 3;
+    const int n_groups = rows * groups_per_row;
+    int grp = tid;
+    float4 xa = make_float4(0.f, 0.f, 0.f, 0.f), xb = xa;
+    if (grp < n_groups) {
+        xa = reinterpret_cast<const float4*>(x)[grp * 2];
+        xb = reinterpret_cast<const float4*>(x)[grp * 2 + 1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    request(sb_begin);
+    __builtin_amdgcn_sched_barrier(0);
+    for (int u = tid; u < (row_stride >> 4); u += threads)  // the all-zero x column
+        reinterpret_cast<uint4*>(xparts + static_cast<size_t>(rows) * 3 * row_stride)[u] = make_uint4(0u, 0u, 0u, 0u);
+    // every lane of a quad takes part in the sums below, so the loop runs for whole quads
+    for (int base_grp = tid & ~3; base_grp < n_groups; base_grp += threads) {
+        const bool mine = grp < n_groups;
+        const float v[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+        uint32_t p[3][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) split3_pair(v[2 * i], v[2 * i + 1], &p[0][i], &p[1][i], &p[2][i]);
+        float s = mine ? ((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7])) : 0.0f;
+        s += dpp_move<kDppXor1>(s);
+        s += __shfl_xor(s, 2);
+        if (mine) {
+            const int r = grp / groups_per_row, kg = grp - r * groups_per_row;
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+                *reinterpret_cast<uint4*>(xparts + static_cast<size_t>(r * 3 + part) * row_stride + kg * 16) =
+                    make_uint4(p[part][0], p[part][1], p[part][2], p[part][3]);
+            if ((tid & 3) == 0) xsum[r * (kb * 8) + (kg >> 2)] = s;
+        }
+        grp += threads;
+        if (grp < n_groups) {
+            xa = reinterpret_cast<const float4*>(x)[grp * 2];
+            xb = reinterpret_cast<const float4*>(x)[grp * 2 + 1];
+        }
+    }
+    __syncthreads();
+
+    // ---- 2. this lane's roles
+    const int c = lane & 31, g = lane >> 5;
+    // A operand: x column c of the MFMA = part (c & 3) of row 2 (c >> 3) + ((c >> 2) & 1)
+    const int a_row = 2 * (c >> 3) + ((c >> 2) & 1), a_part = c & 3;
+    const bool a_live = a_part < 3 && (c >> 3) < kGroups && a_row < rows;
+    const unsigned char* a_base = xparts + static_cast<size_t>(a_live ? a_row * 3 + a_part : rows * 3) * row_stride + 32 * g;
+    // results: D register 4 G + part of this lane belongs to row 2 G + g, output column c of the tile
+    float acc[kGroups];
+    const float* xsum_row[kGroups];
+#pragma unroll
+    for (int G = 0; G < kGroups; ++G) {
+        acc[G] = 0.0f;
+        xsum_row[G] = xsum + min(2 * G + g, rows - 1) * (kb * 8);
+    }
+
+    for (int sb_first = sb_begin; sb_first < sb_end; sb_first += kFlight) {
+        if (sb_first != sb_begin) request(sb_first);
+#pragma unroll
+        for (int f = 0; f < kFlight; ++f) {
+            const int sb = sb_first + f;
+            if (!(tile_ok && sb < sb_end)) continue;  // wave-uniform: nothing was requested for it
+            const t_u32x4 h = hdr[f];
+            const float d = half_bits_to_f32(static_cast<uint16_t>(h.x & 0xFFFFu));
+            const float dmin = half_bits_to_f32(static_cast<uint16_t>(h.x >> 16));
+            // the eight 6-bit scales and mins as bytes of four words (unpackQ4KScaleMinsU8,
+            // ops/native_compute.zig:33745-33754)
+            const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
+            const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+            const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+            const unsigned char* a_sb = a_base + sb * 512;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                // bytes 0x0n: the low and the high nibbles of this lane's 16 bytes of chunk t
+                const uint32_t w[4] = {qv[f][t].x, qv[f][t].y, qv[f][t].z, qv[f][t].w};
+                uint32_t nib[2][4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    nib[0][k] = w[k] & 0x0F0F0F0Fu;
+                    nib[1][k] = (w[k] >> 4) & 0x0F0F0F0Fu;
+                }
+#pragma unroll
+                for (int hi = 0; hi < 2; ++hi) {  // low nibbles: sub-block 2 t, high nibbles: 2 t + 1
+                    const int sub = 2 * t + hi;
+                    // (one accumulator set: a second one for the other sub-block costs a wavefront of occupancy)
+                    t_f32x16 D = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int m = 0; m < 2; ++m) {
+                        union {
+                            t_bf16x8 v;
+                            t_bf16x2 pair[4];
+                            uint4 u;
+                        } a, b;
+                        // fp8 0x0n = n * 2^-9; times 2^9: the bf16 numbers n, two per instruction
+                        b.pair[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib[hi][2 * m]), 512.0f, false);
+                        b.pair[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib[hi][2 * m]), 512.0f, true);
+                        b.pair[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib[hi][2 * m + 1]), 512.0f, false);
+                        b.pair[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib[hi][2 * m + 1]), 512.0f, true);
+                        a.u = *reinterpret_cast<const uint4*>(a_sb + (32 * sub + 8 * m) * 2);
+                        D = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, D, 0, 0, 0);
+                    }
+                    const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
+                    const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
+                    const float dsc = d * sc, dmn = dmin * mn;
+#pragma unroll
+                    for (int G = 0; G < kGroups; ++G) {
+                        const float X = xsum_row[G][sb * 8 + sub];
+                        const float S = (D[4 * G] + D[4 * G + 1]) + D[4 * G + 2];
+                        acc[G] = __builtin_fmaf(dsc, S, acc[G]);
+                        acc[G] = __builtin_fmaf(-dmn, X, acc[G]);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- 3. K-slices meet in LDS, in slice order
+#pragma unroll
+    for (int G = 0; G < kGroups; ++G) partial[(wave * kGroups + G) * 64 + lane] = acc[G];
+    __syncthreads();
+    const int cells = tiles_per_wg * kGroups * 64;
+    for (int i = tid; i < cells; i += threads) {
+        const int ti = i / (kGroups * 64), rem = i - ti * (kGroups * 64);
+        const int G = rem >> 6, ln = rem & 63;
+        float total = 0.0f;
+        for (int sl = 0; sl < slices; ++sl) total += partial[((ti * slices + sl) * kGroups + G) * 64 + ln];
+        const int row = 2 * G + (ln >> 5);
+        const int o = (blockIdx.x * tiles_per_wg + ti) * kTileCols + (ln & 31);
+        if (row < rows && o < out_dim) {
+            const size_t idx = static_cast<size_t>(row) * out_dim + o;
+            dst[idx] = finish_output(ep, o, idx, total);
+        }
+    }
+}
+
+// Tuning runs only (the CPU engine exposes TERMITE_QUANT_* knobs the same way,
+// ops/native_compute.zig:2902-2945).
+int tuning_int(const char* name) {
+    const char* v = std::getenv(name);
+    return v && *v ? std::atoi(v) : 0;
+}
+
+size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
+    return static_cast<size_t>(rows * 3 + 1) * (static_cast<size_t>(in_dim) * 2 + kRowPadBytes) +
+           static_cast<size_t>(rows) * (in_dim / 32) * 4 + static_cast<size_t>(waves) * groups * 64 * 4;
+}
+
+template <int kGroups>
+hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                                int out_dim, const Epilogue& ep) {
+    constexpr int kMaxWaves = 8;
+    const int kb = in_dim / kQ4kBlockValues;
+    const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
+    // One or two rows: eight K slices per tile (one tile, eight wavefronts a workgroup) -- the
+    // most wavefronts, the shortest dependent chain each.  More rows: four slices and two tiles
+    // a workgroup, so that twice as many threads share the splitting of X.  (Measured on
+    // 14336 x 4096, 4096 x 14336 and 128256 x 4096.)
+    int slices = rows <= 2 ? 8 : 4;
+    while (slices > kb) slices /= 2;
+    static const int env_slices = tuning_int("AFHIP_Q4K_SLICES"), env_tiles = tuning_int("AFHIP_Q4K_TILES_PER_WG");
+    if (env_slices >= 1 && env_slices <= kMaxWaves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
+    const int sb_per_slice = (kb + slices - 1) / slices;
+    int tiles_per_wg = kMaxWaves / slices;
+    if (env_tiles >= 1 && env_tiles * slices <= kMaxWaves) tiles_per_wg = env_tiles;
+    const int waves = slices * tiles_per_wg;
+    const int grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+    const size_t lds = q4k_mfma_lds_bytes(rows, in_dim, waves, kGroups);
+    // super-blocks requested ahead: all of a short slice (fewer registers, more wavefronts
+    // resident), four at a time of a long one
+    const bool short_slice = sb_per_slice <= 2;
+    auto kernel = short_slice ? gemv_q4k_mfma_kernel<kGroups, 2> : gemv_q4k_mfma_kernel<kGroups, 4>;
+    static bool large_lds[2] = {false, false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    if (lds > 64 * 1024 && !large_lds[short_slice]) {
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               160 * 1024);
+            e != hipSuccess)
+            return e;
+        large_lds[short_slice] = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, rows, in_dim, out_dim, slices,
+                       sb_per_slice, ep);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+size_t q4k_tiled_bytes(size_t out_dim, size_t in_dim) {
+    return (out_dim + kTileCols - 1) / kTileCols * (in_dim / kQ4kBlockValues) * kTileBytes;
+}
+
+hipError_t launch_q4k_tile_repack(hipStream_t stream, uint8_t* dst, const uint8_t* src_raw, int out_dim, int in_dim) {
+    const int kb = in_dim / kQ4kBlockValues;
+    const size_t units = q4k_tiled_bytes(static_cast<size_t>(out_dim), static_cast<size_t>(in_dim)) / 16;
+    if (units == 0) return hipSuccess;
+    size_t grid = (units + 255) / 256;
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(q4k_tile_repack_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream,
+                       reinterpret_cast<t_u32x4*>(dst), src_raw, out_dim, kb, units);
+    return hipGetLastError();
+}
+
+hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
+                                            size_t rows, int dim) {
+    if (rows == 0 || dim == 0) return hipSuccess;
+    size_t grid = (rows * static_cast<size_t>(dim >> 2) + 255) / 256;
+    if (grid > 65536) grid = 65536;
+    hipLaunchKernelGGL(dequantize_q4k_tiled_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst, weight,
+                       ids, rows, dim);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                                 int out_dim, const Epilogue& ep0) {
+    if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
+    // as many rows per launch as LDS holds (three bf16 copies of each), at most eight
+    int per_launch = kMaxRowsPerLaunch;
+    while (per_launch > 1 && q4k_mfma_lds_bytes(per_launch, in_dim, 8, (per_launch + 1) / 2) > kLdsBudget) --per_launch;
+    if (q4k_mfma_lds_bytes(per_launch, in_dim, 8, 1) > kLdsBudget) return hipErrorInvalidValue;
+    for (int r0 = 0; r0 < rows; r0 += per_launch) {
+        const int nr = rows - r0 < per_launch ? rows - r0 : per_launch;
+        float* d = dst + static_cast<size_t>(r0) * out_dim;
+        const float* xr = x + static_cast<size_t>(r0) * in_dim;
+        Epilogue ep = ep0;
+        if (ep.residual) ep.residual += static_cast<size_t>(r0) * out_dim;
+        hipError_t e;
+        switch ((nr + 1) / 2) {
+            case 1: e = launch_q4k_mfma_rows<1>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
+            case 2: e = launch_q4k_mfma_rows<2>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
+            case 3: e = launch_q4k_mfma_rows<3>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
+            default: e = launch_q4k_mfma_rows<4>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
+        }
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace afhip

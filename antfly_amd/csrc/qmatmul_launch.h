@@ -88,6 +88,16 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
                                       size_t rows, int dim);
 
+// Q4_K in the tile-major layout (32 output columns x one super-block per 4608-byte tile; columns
+// past out_dim zero): size, repack from the raw GGUF bytes, the MFMA GEMV for any number of
+// rows, and get_rows / cpy_q_to_f32.
+size_t q4k_tiled_bytes(size_t out_dim, size_t in_dim);
+hipError_t launch_q4k_tile_repack(hipStream_t stream, uint8_t* dst, const uint8_t* src_raw, int out_dim, int in_dim);
+hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                                 int out_dim, const Epilogue& ep = Epilogue{});
+hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
+                                            size_t rows, int dim);
+
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);

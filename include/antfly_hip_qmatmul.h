@@ -233,7 +233,14 @@ afhip_status afhip_launch_dequantize_f32(void *stream, int tensor_type, int layo
 afhip_status afhip_launch_quantize_rows(void *stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
                                         afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows);
 
-/* One-time device-side repack RAW -> PREPARED (dst.len >= src bytes). */
+/* Bytes of the PREPARED layout of a [out_dim, in_dim] weight: the raw size for Q4_0 / Q8_0;
+ * for Q4_K the tile-major layout (32 output columns x one 256-value super-block per
+ * 4608-byte tile, columns past out_dim zero-filled), i.e. the raw size of out_dim rounded up
+ * to a multiple of 32.  0 for an unknown type or an in_dim that is not whole blocks. */
+size_t afhip_prepared_weight_bytes(int tensor_type, size_t out_dim, size_t in_dim);
+/* One-time device-side repack RAW -> PREPARED (dst.len >= afhip_prepared_weight_bytes).  What
+ * the engine's prepareNativeQuantizedStorage does on the CPU for its own kernels
+ * (ops/native_compute.zig:8130-8204): derived from the raw bytes, invisible to callers. */
 afhip_status afhip_launch_prepare_weight(void *stream, int tensor_type, afhip_buffer dst_prepared,
                                          afhip_buffer src_raw, size_t out_dim, size_t in_dim);
 

@@ -22,7 +22,7 @@ def to_dev(a: np.ndarray) -> torch.Tensor:
 
 def prepare(fmt: int, w_raw: np.ndarray, out_dim: int, in_dim: int) -> torch.Tensor:
     raw = to_dev(w_raw)
-    prepared = torch.empty_like(raw)
+    prepared = torch.empty(kernels.preparedWeightBytes(fmt, out_dim, in_dim), dtype=torch.uint8, device=DEV)
     kernels.launchPrepareWeight(stream(), fmt, buf(prepared), buf(raw), out_dim, in_dim)
     torch.cuda.synchronize()
     return prepared
@@ -32,6 +32,20 @@ def numpy_prepare(fmt: int, w_raw: np.ndarray) -> np.ndarray:
     bb = 18 if fmt == _lib.TYPE_Q4_0 else 34
     blocks = np.asarray(w_raw, np.uint8).reshape(-1, bb)
     return np.concatenate([blocks[:, 2:].reshape(-1), blocks[:, :2].reshape(-1)])
+
+
+def numpy_prepare_q4k(w_raw: np.ndarray, out_dim: int, in_dim: int) -> np.ndarray:
+    """The tile-major Q4_K layout: per tile of 32 columns and super-block, 32 headers of 16 bytes, then for
+    each 32-byte chunk of nibbles lane c + 32 g holds bytes 16 g .. 16 g + 15 of column c; columns past
+    out_dim are zero."""
+    kb = in_dim // 256
+    tiles = (out_dim + 31) // 32
+    blocks = np.zeros((tiles * 32, kb, 144), np.uint8)
+    blocks[:out_dim] = np.asarray(w_raw, np.uint8).reshape(out_dim, kb, 144)
+    blocks = blocks.reshape(tiles, 32, kb, 144).transpose(0, 2, 1, 3)          # [tile][sb][c][144]
+    headers = blocks[..., :16].reshape(tiles, kb, 512)
+    quants = blocks[..., 16:].reshape(tiles, kb, 32, 4, 2, 16).transpose(0, 1, 3, 4, 2, 5)  # [tile][sb][chunk][g][c][16]
+    return np.concatenate([headers, quants.reshape(tiles, kb, 4096)], axis=2).reshape(-1)
 
 
 def linear(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, out_dim, dispatch=-1) -> np.ndarray:

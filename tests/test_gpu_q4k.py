@@ -16,8 +16,12 @@ from oracle import oracle as O  # noqa: E402
 from tests import gpu_util as G  # noqa: E402
 
 Q4K = _lib.TYPE_Q4_K
-RAW = _lib.LAYOUT_RAW
+RAW, PREP = _lib.LAYOUT_RAW, _lib.LAYOUT_PREPARED
 TOL, TIGHT = 1e-3, 2e-5
+
+
+def device_weight(layout, w, out_dim, in_dim):
+    return G.prepare(Q4K, w, out_dim, in_dim) if layout == PREP else G.to_dev(w)
 
 
 def q4k_block(d_bits, dmin_bits, scales12, qs128):
@@ -33,34 +37,50 @@ def test_reference_vectors(kats):
     print("case: q4_k direct matmul kat", flush=True)
     w = np.concatenate([q4k_block(15360, 0, scales, [f] * 128) for f in m["row_qs_fill"]])
     x = np.full((1, m["in_dim"]), m["input_fill"], np.float32)
-    y = G.linear(Q4K, RAW, x, G.to_dev(w), 1, m["in_dim"], m["out_dim"])
-    assert np.abs(y[0] - np.array(m["expected"])).max() <= m["tolerance_abs"]
+    for layout in (RAW, PREP):
+        y = G.linear(Q4K, layout, x, device_weight(layout, w, m["out_dim"], m["in_dim"]), 1, m["in_dim"], m["out_dim"])
+        assert np.abs(y[0] - np.array(m["expected"])).max() <= m["tolerance_abs"]
     h = k["header_packing"]
     print("case: q4_k header packing kat", flush=True)
     raw = np.array(h["header"] + h["qs_32"] * 4, np.uint8)
-    out = torch.empty(256, dtype=torch.float32, device=G.DEV)
-    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(out), G.buf(G.to_dev(raw)), 1, 256)
-    torch.cuda.synchronize()
     want = np.array([h["scs"][sub] * (i % 16) - h["mins"][sub] for sub in range(8) for i in range(32)], np.float32)
-    assert np.array_equal(out.cpu().numpy(), want)
+    for layout in (RAW, PREP):
+        out = torch.empty(256, dtype=torch.float32, device=G.DEV)
+        wd = device_weight(layout, raw, 1, 256)
+        kernels.launchDequantizeF32(G.stream(), Q4K, layout, G.buf(out), G.buf(wd), 1, 256)
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(), want)
 
 
-@pytest.mark.parametrize("rows,dim", [(1, 256), (5, 1024), (3, 4096)])
-def test_dequantize_and_get_rows_bit_exact(rows, dim):
-    print(f"case: q4_k cpy_q_to_f32 / get_rows rows={rows} dim={dim}", flush=True)
+@pytest.mark.parametrize("out_dim,in_dim", [(1, 256), (32, 512), (45, 1024), (100, 4096)])
+def test_tile_major_repack_is_a_pure_permutation(out_dim, in_dim):
+    print(f"case: q4_k tile-major repack out={out_dim} in={in_dim}", flush=True)
+    w = synth.weights(Q4K, 3, out_dim, in_dim)
+    want = G.numpy_prepare_q4k(w, out_dim, in_dim)
+    assert kernels.preparedWeightBytes(Q4K, out_dim, in_dim) == want.size == (out_dim + 31) // 32 * (in_dim // 256) * 4608
+    got = G.prepare(Q4K, w, out_dim, in_dim).cpu().numpy()
+    assert np.array_equal(got, want)
+    if out_dim % 32 == 0:
+        assert np.array_equal(np.sort(got), np.sort(w))  # same bytes, other places
+
+
+@pytest.mark.parametrize("layout", [RAW, PREP])
+@pytest.mark.parametrize("rows,dim", [(1, 256), (5, 1024), (3, 4096), (40, 512)])
+def test_dequantize_and_get_rows_bit_exact(rows, dim, layout):
+    print(f"case: q4_k cpy_q_to_f32 / get_rows rows={rows} dim={dim} layout={layout}", flush=True)
     vocab = rows + 7
     w = synth.weights(Q4K, 2, vocab, dim).copy()
     w[0:4] = np.array([0x0001, 0x7BFF], np.uint16).view(np.uint8)  # subnormal d, largest finite dmin
-    wd = G.to_dev(w)
+    wd = device_weight(layout, w, vocab, dim)
     table = O.dequantize_q4_k(w).reshape(vocab, dim)
     out = torch.empty((vocab, dim), dtype=torch.float32, device=G.DEV)
-    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(out), G.buf(wd), vocab, dim)
+    kernels.launchDequantizeF32(G.stream(), Q4K, layout, G.buf(out), G.buf(wd), vocab, dim)
     torch.cuda.synchronize()
     assert np.array_equal(out.cpu().numpy().view(np.uint32), table.view(np.uint32))
     ids = np.array([vocab - 1, 0, 3, 3][:rows + 1], dtype=np.int64)
     idd = G.to_dev(ids)
     emb = torch.empty((len(ids), dim), dtype=torch.float32, device=G.DEV)
-    kernels.launchEmbeddingLookupF32(G.stream(), Q4K, RAW, G.buf(emb), G.buf(wd), G.buf(idd), len(ids), dim, vocab)
+    kernels.launchEmbeddingLookupF32(G.stream(), Q4K, layout, G.buf(emb), G.buf(wd), G.buf(idd), len(ids), dim, vocab)
     torch.cuda.synchronize()
     assert np.array_equal(emb.cpu().numpy().view(np.uint32), table[ids].view(np.uint32))
 
@@ -69,12 +89,16 @@ SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130),
           (1, 14336, 48), (2, 14336, 20), (9, 2048, 24), (1, 16384, 8), (3, 16384, 12), (4, 14336, 8)]
 
 
-@pytest.mark.parametrize("rows,in_dim,out_dim", SHAPES)
-def test_linear_matches_oracle(rows, in_dim, out_dim):
-    print(f"case: q4_k linear rows={rows} in={in_dim} out={out_dim}", flush=True)
+TILED_SHAPES = SHAPES + [(1, 1024, 300), (6, 4096, 70), (7, 1024, 257), (8, 2048, 96), (9, 1024, 64), (17, 512, 40),
+                        (2, 4096, 1000)]
+
+
+@pytest.mark.parametrize("layout,rows,in_dim,out_dim", [(RAW, *s) for s in SHAPES] + [(PREP, *s) for s in TILED_SHAPES])
+def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
+    print(f"case: q4_k linear layout={layout} rows={rows} in={in_dim} out={out_dim}", flush=True)
     w = synth.weights(Q4K, 11, out_dim, in_dim)
     x = synth.activations(12, rows, in_dim)
-    y = G.linear(Q4K, RAW, x, G.to_dev(w), rows, in_dim, out_dim)
+    y = G.linear(Q4K, layout, x, device_weight(layout, w, out_dim, in_dim), rows, in_dim, out_dim)
     ref64 = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
     ref32 = O.linear_q4_k(x, w, rows, in_dim, out_dim)
     err64, err32 = G.max_rel_err(y, ref64), G.max_rel_err(y, ref32.astype(np.float64))
@@ -101,13 +125,15 @@ def test_linear_argument_checks():
         kernels.launchLinearF32(G.stream(), Q4K, RAW, G.buf(y), G.buf(big_x), G.buf(big_w), 1, 32768, 4, ws)
 
 
-def test_full_size_ffn_matrix_and_pair():
+@pytest.mark.parametrize("layout", [RAW, PREP])
+def test_full_size_ffn_matrix_and_pair(layout):
     """Llama-3-8B FFN shapes in Q4_K (33 MB per matrix, as Q4_0): decode rows, a pair, scaling property."""
+    RAW = layout  # the body below runs on the layout under test
     in_dim, out_dim = 4096, 14336
     wa, wb = synth.weights(Q4K, 21, out_dim, in_dim), synth.weights(Q4K, 22, out_dim, in_dim)
-    da, db = G.to_dev(wa), G.to_dev(wb)
-    for rows in (1, 2, 4):
-        print(f"case: q4_k full size rows={rows}", flush=True)
+    da, db = device_weight(layout, wa, out_dim, in_dim), device_weight(layout, wb, out_dim, in_dim)
+    for rows in (1, 2, 4) if layout == _lib.LAYOUT_RAW else (1, 2, 4, 8):
+        print(f"case: q4_k full size layout={layout} rows={rows}", flush=True)
         x = synth.activations(30 + rows, rows, in_dim)
         y = G.linear(Q4K, RAW, x, da, rows, in_dim, out_dim)
         ref = O.linear_q4_k(x, wa, rows, in_dim, out_dim, f64=True)
@@ -121,7 +147,7 @@ def test_full_size_ffn_matrix_and_pair():
     # down projection: K = 14336
     wd_ = synth.weights(Q4K, 23, 4096, 14336)
     x = synth.activations(40, 1, 14336)
-    y = G.linear(Q4K, RAW, x, G.to_dev(wd_), 1, 14336, 4096)
+    y = G.linear(Q4K, RAW, x, device_weight(layout, wd_, 4096, 14336), 1, 14336, 4096)
     assert G.max_rel_err(y, O.linear_q4_k(x, wd_, 1, 14336, 4096, f64=True)) <= TIGHT
 
 
@@ -131,15 +157,18 @@ def test_backend_ops_on_q4_k():
     x = synth.activations(52, rows, in_dim)
     with HipCompute() as cb:
         print("case: backend q4_k ops", flush=True)
+        cb.insertWeightFromLoaded("raw.weight", Q4K, w, [out_dim, in_dim], keep_raw_layout=True)
+        assert cb.getWeight("raw.weight").layout == _lib.LAYOUT_RAW
         cb.insertWeightFromLoaded("output.weight", Q4K, w, [out_dim, in_dim])
         wt = cb.getWeight("output.weight")
-        assert wt.quant_type == Q4K and wt.layout == _lib.LAYOUT_RAW and wt.shape == [out_dim, in_dim]
+        assert wt.quant_type == Q4K and wt.layout == _lib.LAYOUT_PREPARED and wt.shape == [out_dim, in_dim]
+        assert wt.byte_len == (out_dim + 31) // 32 * (in_dim // 256) * 4608
         xt = cb.fromFloat32(x, [rows, in_dim])
         y = cb.toFloat32(cb.linearNoBias(xt, wt, rows, in_dim, out_dim)).reshape(rows, out_dim)
         ref = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
         assert G.max_rel_err(y, ref) <= TIGHT
         stats = cb.debugStats()
-        assert stats["launches_small_batch"] == 1 and stats["launches_activation_quant"] == 0 and stats["launches_prepare"] == 0
+        assert stats["launches_small_batch"] == 1 and stats["launches_activation_quant"] == 0 and stats["launches_prepare"] == 1
         token = cb.linearNoBiasArgmaxLastRow(xt, wt, rows, in_dim, out_dim)
         assert token == int(np.argmax(y[-1]))
         assert token == O.argmax(ref[-1].astype(np.float32)) or ref[-1].max() - ref[-1][token] <= TIGHT * np.abs(ref[-1]).max()
