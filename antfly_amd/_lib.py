@@ -116,6 +116,7 @@ SIGNATURES = {
     "afhip_launch_linear_pair_bias_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_linear_q8_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
     "afhip_launch_linear_q4_0_f32": (_st, [_vp, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer]),
+    "afhip_weight_layout_bytes": (_sz, [_i, _i, _sz, _sz]),
     "afhip_prepared_weight_bytes": (_sz, [_i, _sz, _sz]),
     "afhip_launch_prepare_weight": (_st, [_vp, _i, Buffer, Buffer, _sz, _sz]),
     "afhip_launch_quantize_activations": (_st, [_vp, Buffer, _sz, _sz, Buffer, Buffer, Buffer]),

@@ -581,6 +581,17 @@ size_t afhip_prepared_weight_bytes(int tensor_type, size_t out_dim, size_t in_di
     return bytes;
 }
 
+size_t afhip_weight_layout_bytes(int tensor_type, int layout, size_t out_dim, size_t in_dim) {
+    size_t blocks, bytes;
+    if (layout == AFHIP_LAYOUT_PREPARED) return afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim);
+    if (layout != AFHIP_LAYOUT_RAW) return 0;
+    const size_t bb = tensor_type == AFHIP_TYPE_Q4_K ? 144 : block_bytes(tensor_type);
+    const size_t values = tensor_type == AFHIP_TYPE_Q4_K ? 256 : 32;
+    if (bb == 0 || in_dim % values != 0 || !checked_mul(out_dim, in_dim / values, &blocks) || !checked_mul(blocks, bb, &bytes))
+        return 0;
+    return bytes;
+}
+
 afhip_status afhip_launch_prepare_weight(void* stream, int tensor_type, afhip_buffer dst, afhip_buffer src,
                                          size_t out_dim, size_t in_dim) {
     if (tensor_type == AFHIP_TYPE_Q4_K) {  // tile-major layout for the MFMA kernel

@@ -60,6 +60,11 @@ def launchLinearQ4_0F32(stream, dst: Buffer, input: Buffer, weight_raw: Buffer, 
     check(_lib.lib().afhip_launch_linear_q4_0_f32(stream, dst, input, weight_raw, rows, in_dim, out_dim, workspace))
 
 
+def weightLayoutBytes(tensor_type, layout, out_dim, in_dim) -> int:
+    """Size of a [out_dim, in_dim] weight in a device layout (raw or prepared)."""
+    return int(_lib.lib().afhip_weight_layout_bytes(tensor_type, layout, out_dim, in_dim))
+
+
 def preparedWeightBytes(tensor_type, out_dim, in_dim) -> int:
     """Size of the PREPARED layout (Q4_K pads out_dim to whole 32-column tiles)."""
     return int(_lib.lib().afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim))

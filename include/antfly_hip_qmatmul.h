@@ -233,6 +233,9 @@ afhip_status afhip_launch_dequantize_f32(void *stream, int tensor_type, int layo
 afhip_status afhip_launch_quantize_rows(void *stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
                                         afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows);
 
+/* Bytes of a [out_dim, in_dim] weight in a device layout (0: unknown type / layout, or in_dim
+ * not whole blocks). */
+size_t afhip_weight_layout_bytes(int tensor_type, int layout, size_t out_dim, size_t in_dim);
 /* Bytes of the PREPARED layout of a [out_dim, in_dim] weight: the raw size for Q4_0 / Q8_0;
  * for Q4_K the tile-major layout (32 output columns x one 256-value super-block per
  * 4608-byte tile, columns past out_dim zero-filled), i.e. the raw size of out_dim rounded up
