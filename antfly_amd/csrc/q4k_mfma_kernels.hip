@@ -155,8 +155,8 @@ extern __shared__ __align__(16) unsigned char q4k_mfma_lds[];
 
 // kGroups = ceil(rows / 2) row groups (D registers 0 .. 4 kGroups - 1 are read);
 // kFlight super-blocks of weights are requested before any of them is used.
-template <int kGroups, int kFlight>
-__global__ __launch_bounds__(512) void gemv_q4k_mfma_kernel(float* __restrict__ dst, const float* __restrict__ x,
+template <int kGroups, int kFlight, int kMaxThreads = 512>
+__global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                             const uint8_t* __restrict__ weight, int rows, int in_dim,
                                                             int out_dim, int slices, int sb_per_slice, Epilogue ep) {
     const int kb = in_dim >> 8;
@@ -341,34 +341,50 @@ size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
 template <int kGroups>
 hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                                 int out_dim, const Epilogue& ep) {
-    constexpr int kMaxWaves = 8;
     const int kb = in_dim / kQ4kBlockValues;
     const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
-    // One or two rows: eight K slices per tile (one tile, eight wavefronts a workgroup) -- the
+    // One or two rows: sixteen K slices per tile (one tile, sixteen wavefronts a workgroup) -- the
     // most wavefronts, the shortest dependent chain each.  More rows: four slices and two tiles
-    // a workgroup, so that twice as many threads share the splitting of X.  (Measured on
-    // 14336 x 4096, 4096 x 14336 and 128256 x 4096.)
-    int slices = rows <= 2 ? 8 : 4;
+    // a workgroup of eight wavefronts (their register need rules out sixteen), so that many
+    // threads share the splitting of X.  (Measured on 14336 x 4096, 4096 x 14336, 4096 x 4096
+    // and 128256 x 4096.)
+    const int max_waves = kGroups == 1 ? 16 : 8;
+    int slices = kGroups == 1 ? 16 : 4;
+    // long rows (three or more super-blocks a slice) and vocabulary-sized matrices did better with eight
+    if (slices == 16 && (kb > 32 || n_tiles > 2048)) slices = 8;
     while (slices > kb) slices /= 2;
     static const int env_slices = tuning_int("AFHIP_Q4K_SLICES"), env_tiles = tuning_int("AFHIP_Q4K_TILES_PER_WG");
-    if (env_slices >= 1 && env_slices <= kMaxWaves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
+    if (env_slices >= 1 && env_slices <= max_waves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
     const int sb_per_slice = (kb + slices - 1) / slices;
-    int tiles_per_wg = kMaxWaves / slices;
-    if (env_tiles >= 1 && env_tiles * slices <= kMaxWaves) tiles_per_wg = env_tiles;
+    int tiles_per_wg = (slices > 8 ? 16 : 8) / slices;
+    if (env_tiles >= 1 && env_tiles * slices <= max_waves) tiles_per_wg = env_tiles;
     const int waves = slices * tiles_per_wg;
     const int grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     const size_t lds = q4k_mfma_lds_bytes(rows, in_dim, waves, kGroups);
     // super-blocks requested ahead: all of a short slice (fewer registers, more wavefronts
     // resident), four at a time of a long one
-    const bool short_slice = sb_per_slice <= 2;
-    auto kernel = short_slice ? gemv_q4k_mfma_kernel<kGroups, 2> : gemv_q4k_mfma_kernel<kGroups, 4>;
-    static bool large_lds[2] = {false, false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
-    if (lds > 64 * 1024 && !large_lds[short_slice]) {
+    const int flight = sb_per_slice <= 1 ? 0 : (sb_per_slice <= 2 ? 1 : 2);
+    const int variant = (waves > 8 ? 3 : 0) + flight;
+    void (*kernel)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
+    switch (variant) {
+        case 0:
+        case 1: kernel = gemv_q4k_mfma_kernel<kGroups, 2>; break;
+        case 2: kernel = gemv_q4k_mfma_kernel<kGroups, 4>; break;
+        default:
+            if constexpr (kGroups == 1) {  // sixteen wavefronts: at most 128 registers each
+                kernel = variant == 3 ? gemv_q4k_mfma_kernel<1, 1, 1024>
+                                      : (variant == 4 ? gemv_q4k_mfma_kernel<1, 2, 1024> : gemv_q4k_mfma_kernel<1, 4, 1024>);
+            }
+            break;
+    }
+    if (kernel == nullptr) return hipErrorInvalidValue;
+    static bool large_lds[6] = {false, false, false, false, false, false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    if (lds > 64 * 1024 && !large_lds[variant]) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                160 * 1024);
             e != hipSuccess)
             return e;
-        large_lds[short_slice] = true;
+        large_lds[variant] = true;
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, rows, in_dim, out_dim, slices,
                        sb_per_slice, ep);
