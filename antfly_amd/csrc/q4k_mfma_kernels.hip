@@ -23,8 +23,8 @@
 // x columns 8 (r / 2) + 4 (r % 2) + {0, 1, 2} for its three parts, so that the results of
 // up to eight rows land in D registers 4 (r / 2) + part of lane half r % 2 -- and B columns
 // are 32 consecutive output columns.  Lane (column c, half g) supplies the K values
-// 16 g + 8 m + 0..7 of the sub-block to MFMA m = 0, 1.  x columns that carry nothing read an
-// all-zero column of LDS.
+// 16 g + 8 m + 0..7 of the sub-block to MFMA m = 0, 1.  x columns that carry nothing read
+// some valid column: every D row depends on its own A row only, and their D rows are not read.
 //
 // Tile-major layout ("prepared" Q4_K): for every tile of 32 output columns and every
 // super-block of 256 values, 4608 bytes: the 32 headers of 16 bytes (d, dmin, 12 scale
@@ -52,7 +52,7 @@ constexpr int kTileBytes = 4608;        // 32 * 16 + 4 * 64 * 16
 constexpr int kTileUnits = kTileBytes / 16;
 constexpr int kRowPadBytes = 48;        // LDS stride of an x column: 2 K + 48 spreads the columns over the banks
 constexpr int kMaxRowsPerLaunch = 8;
-constexpr size_t kLdsBudget = 150 * 1024;
+constexpr size_t kLdsBudget = 160 * 1024 - 512;  // of the 160 KiB a workgroup can have
 
 typedef uint32_t t_u32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 t_bf16x8 __attribute__((ext_vector_type(8)));
@@ -164,8 +164,8 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int threads = static_cast<int>(blockDim.x), waves = threads >> 6;
     const int row_stride = in_dim * 2 + kRowPadBytes;  // bytes per x column
-    unsigned char* xparts = q4k_mfma_lds;  // [rows * 3 + 1][row_stride]: the parts of every row, then a column of zeros
-    float* xsum = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows * 3 + 1) * row_stride);  // [rows][kb * 8]
+    unsigned char* xparts = q4k_mfma_lds;  // [rows * 3][row_stride]: the three parts of every row
+    float* xsum = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows) * 3 * row_stride);  // [rows][kb * 8]
     float* partial = xsum + rows * kb * 8;                                                       // [waves][kGroups][64]
 
     const int tiles_per_wg = waves / slices;
@@ -204,8 +204,6 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
     __builtin_amdgcn_sched_barrier(0);
     request(sb_begin);
     __builtin_amdgcn_sched_barrier(0);
-    for (int u = tid; u < (row_stride >> 4); u += threads)  // the all-zero x column
-        reinterpret_cast<uint4*>(xparts + static_cast<size_t>(rows) * 3 * row_stride)[u] = make_uint4(0u, 0u, 0u, 0u);
     // every lane of a quad takes part in the sums below, so the loop runs for whole quads
     for (int base_grp = tid & ~3; base_grp < n_groups; base_grp += threads) {
         const bool mine = grp < n_groups;
@@ -237,7 +235,8 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
     // A operand: x column c of the MFMA = part (c & 3) of row 2 (c >> 3) + ((c >> 2) & 1)
     const int a_row = 2 * (c >> 3) + ((c >> 2) & 1), a_part = c & 3;
     const bool a_live = a_part < 3 && (c >> 3) < kGroups && a_row < rows;
-    const unsigned char* a_base = xparts + static_cast<size_t>(a_live ? a_row * 3 + a_part : rows * 3) * row_stride + 32 * g;
+    // (a lane without a part reads the first column: its D row is never looked at)
+    const unsigned char* a_base = xparts + static_cast<size_t>(a_live ? a_row * 3 + a_part : 0) * row_stride + 32 * g;
     // results: D register 4 G + part of this lane belongs to row 2 G + g, output column c of the tile
     float acc[kGroups];
     const float* xsum_row[kGroups];
@@ -334,7 +333,7 @@ int tuning_int(const char* name) {
 }
 
 size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
-    return static_cast<size_t>(rows * 3 + 1) * (static_cast<size_t>(in_dim) * 2 + kRowPadBytes) +
+    return static_cast<size_t>(rows) * 3 * (static_cast<size_t>(in_dim) * 2 + kRowPadBytes) +
            static_cast<size_t>(rows) * (in_dim / 32) * 4 + static_cast<size_t>(waves) * groups * 64 * 4;
 }
 
