@@ -2,6 +2,7 @@
 // stream-ordered launchers (ops/cuda/kernels.zig:1221-1289).
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cstdlib>
 #include <limits>
 
@@ -83,7 +84,8 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
 
 // Q4_K: f32 activations against the dequantized weights, one kernel family for any row count.
 static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
-                                    size_t rows, size_t in_dim, size_t out_dim, int dispatch, bool want_dots,
+                                    size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace, int dispatch,
+                                    bool want_dots,
                                     LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b,
                                     const Epilogue& ep, const Epilogue& ep_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
@@ -108,11 +110,25 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     if (pair && (dst_b.ptr == 0 || weight_b.ptr == 0 || dst_b.ptr % 4 != 0 || weight_b.ptr % 16 != 0))
         return AFHIP_ERR_INVALID_STATE;
     const int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim, AFHIP_FORMAT_Q4_K);
+    // more rows than one GEMV launch holds: X split once into the caller's scratch, then the
+    // GEMM (without scratch the GEMV serves them a launch at a time)
+    const size_t gemm_rows = std::max(static_cast<size_t>(gemm_q4k_min_rows()),
+                                      static_cast<size_t>(gemv_q4k_tiled_rows_per_launch(static_cast<int>(in_dim))) + 1);
+    const bool gemm = tiled && rows >= gemm_rows && workspace.ptr != 0 && workspace.ptr % 16 == 0 && workspace.len >= gemm_q4k_workspace_bytes(rows, in_dim);
     for (int i = 0; i < (pair ? 2 : 1); ++i) {
         if (counters) {
             if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
             else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
             else counters->mm++;
+        }
+        if (gemm) {
+            hipError_t e = launch_gemm_q4k_tiled(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
+                                                 reinterpret_cast<const float*>(input.ptr),
+                                                 reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
+                                                 reinterpret_cast<void*>(workspace.ptr), static_cast<int>(rows),
+                                                 static_cast<int>(in_dim), static_cast<int>(out_dim), i ? ep_b : ep, i == 0);
+            if (e != hipSuccess) return static_cast<afhip_status>(e);
+            continue;
         }
         hipError_t e = (tiled ? launch_gemv_q4k_tiled : launch_gemv_q4k)(
             stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const float*>(input.ptr),
@@ -153,8 +169,8 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     ep.activation = extras.activation;  // AFHIP_ACTIVATION_* and kAct* share their values
     ep_b.bias = reinterpret_cast<const float*>(extras.bias_b.ptr);
     if (tensor_type == AFHIP_TYPE_Q4_K)
-        return linear_q4k_impl(stream, layout, dst, input, weight, rows, in_dim, out_dim, dispatch, dots.ptr != 0, counters,
-                               dst_b, weight_b, ep, ep_b);
+        return linear_q4k_impl(stream, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch, dots.ptr != 0,
+                               counters, dst_b, weight_b, ep, ep_b);
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -494,6 +510,15 @@ int afhip_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim) {
 // ---- launchers
 
 size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (tensor_type == AFHIP_TYPE_Q4_K) {  // the split of X for the prefill GEMM; decode rows need none
+        size_t count, bytes;
+        if (in_dim == 0 || in_dim % 256 != 0 || in_dim > 0x7fffffff || out_dim == 0 || !checked_mul(rows, in_dim, &count) ||
+            !checked_mul(count, 8, &bytes))
+            return 0;
+        const size_t gemm_rows = std::max(static_cast<size_t>(gemm_q4k_min_rows()),
+                                          static_cast<size_t>(gemv_q4k_tiled_rows_per_launch(static_cast<int>(in_dim))) + 1);
+        return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim) : 0;
+    }
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;
     return workspace_view(0, rows, in_dim).bytes;
 }

@@ -106,6 +106,49 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
     assert err32 <= TOL and err32 <= TIGHT, err32
 
 
+PREFILL_SHAPES = [(7, 4096, 64), (10, 1024, 300), (11, 512, 33), (40, 2048, 256), (41, 1024, 257), (100, 512, 1000),
+                  (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (47, 512, 40), (48, 512, 40), (50, 14336, 64),
+                  (81, 768, 500)]
+
+
+@pytest.mark.parametrize("rows,in_dim,out_dim", PREFILL_SHAPES)
+def test_prefill_gemm_matches_oracle(rows, in_dim, out_dim):
+    """More rows than one GEMV launch holds: the split kernel + MFMA GEMM (with the caller's scratch), and
+    the same rows served by the GEMV a launch at a time (no scratch) -- both against the oracle."""
+    print(f"case: q4_k prefill rows={rows} in={in_dim} out={out_dim}", flush=True)
+    w = synth.weights(Q4K, 61, out_dim, in_dim)
+    x = synth.activations(62, rows, in_dim)
+    wd = device_weight(PREP, w, out_dim, in_dim)
+    ref64 = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+    y = G.linear(Q4K, PREP, x, wd, rows, in_dim, out_dim)  # G.linear lends afhip_linear_workspace_bytes of scratch
+    err = G.max_rel_err(y, ref64)
+    assert err <= TOL and err <= TIGHT, err
+    xd = G.to_dev(x)
+    y2 = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=G.DEV)
+    kernels.launchLinearF32(G.stream(), Q4K, PREP, G.buf(y2), G.buf(xd), G.buf(wd), rows, in_dim, out_dim, kernels.NO_BUFFER)
+    torch.cuda.synchronize()
+    err2 = G.max_rel_err(y2.cpu().numpy(), ref64)
+    assert err2 <= TIGHT, err2
+
+
+def test_prefill_full_size_with_epilogue():
+    rows, in_dim, out_dim = 512, 4096, 14336
+    print("case: q4_k prefill full size", flush=True)
+    w = synth.weights(Q4K, 63, out_dim, in_dim)
+    x = synth.activations(64, rows, in_dim)
+    wd = device_weight(PREP, w, out_dim, in_dim)
+    y = G.linear(Q4K, PREP, x, wd, rows, in_dim, out_dim)
+    sample = np.r_[0:3, 37:43, 255, 509:512]
+    ref = O.linear_q4_k(x[sample], w, len(sample), in_dim, out_dim, f64=True)
+    assert G.max_rel_err(y[sample], ref) <= TIGHT
+    # linearity in X: rows scaled by powers of two scale exactly
+    y4 = G.linear(Q4K, PREP, x * 4.0, wd, rows, in_dim, out_dim)
+    assert np.array_equal(y4, y * 4.0)
+    b = synth.activations(65, 1, out_dim)[0]
+    yb = G.linear_bias(Q4K, PREP, x, wd, b, rows, in_dim, out_dim)
+    assert np.array_equal(yb, y + b[None, :])
+
+
 def test_linear_argument_checks():
     w = G.to_dev(synth.weights(Q4K, 1, 4, 256))
     x = G.to_dev(synth.activations(2, 1, 256))
@@ -118,7 +161,8 @@ def test_linear_argument_checks():
     d = torch.empty(4, dtype=torch.int32, device=G.DEV)
     with pytest.raises(_lib.HipError):  # no integer route, so no block dots
         kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
-    assert kernels.workspaceBytes(Q4K, 8, 4096, 4096) == 0
+    assert kernels.workspaceBytes(Q4K, 4, 4096, 4096) == 0  # decode rows need no scratch
+    assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) == 64 * 4096 * 6 + 64 * 128 * 4  # the split of X for the prefill GEMM
     big_w = torch.zeros(4 * 128 * 144, dtype=torch.uint8, device=G.DEV)
     big_x = torch.zeros(32768, dtype=torch.float32, device=G.DEV)
     with pytest.raises(_lib.HipOpUnsupported):  # K beyond what one workgroup's slices cover
