@@ -390,6 +390,14 @@ def main() -> int:
                            "us_per_call": round(e_s / small_steps * 1e6, 3),
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
+        for m in (128, 512):
+            w_s, e_s = time_config(Q4K, m, 4096, 14336, 40, 5, 2, 78)
+            flops = 2.0 * m * 4096 * 14336
+            extra[f"q4k_gemm_m{m}_k4096_n14336"] = {
+                "what": "Q4_K prefill: X split once into three bf16 parts, bf16-MFMA GEMM, f32-accurate; per call incl. the split",
+                "us_per_call": round(e_s / 40 * 1e6, 1),
+                "TFLOPs_f32_equivalent": round(flops * 40 / e_s / 1e12, 1),
+                "frac_f32_mfma_peak": round(flops * 40 / e_s / 157.3e12, 3)}
         for m in (128, 512, 2048):
             gsteps = 200
             w_s, e_s = time_config(Q8, m, 4096, 4096, gsteps, 20, 4, 7)
