@@ -335,7 +335,7 @@ int tuning_int(const char* name) {
 // ------------------------------------------------------------------ prefill
 // Many rows (more than one GEMV launch holds): X is split once by its own kernel --
 // parts bf16 [rows][3][in_dim], sub-block sums f32 [rows][in_dim / 32] -- and the GEMM below
-// converts every weight once per 40 rows instead of once per launch of six.
+// converts every weight once per 32 rows instead of once per launch of six.
 __global__ __launch_bounds__(256) void q4k_split_rows_kernel(const float* __restrict__ x, uint32_t* __restrict__ parts,
                                                              float* __restrict__ xsum, size_t groups, int groups_per_row) {
     // one thread per eight consecutive values; whole quads run together (groups is a multiple of four)
@@ -359,88 +359,67 @@ __global__ __launch_bounds__(256) void q4k_split_rows_kernel(const float* __rest
     }
 }
 
-constexpr int kGemmRowBlocks = 4;                    // MFMA passes per sub-block: 10 rows each
-constexpr int kGemmRows = 10 * kGemmRowBlocks;       // rows of X a workgroup covers
-constexpr int kGemmPartStride = 512 + 16;            // bytes of one part of one row and super-block in LDS (padded)
-constexpr int kGemmSumStride = kGemmRows;            // floats per sub-block in the sums area
-constexpr int kGemmChunkBytes = kGemmRows * 3 * kGemmPartStride + kGemmSumStride * 8 * 4;  // parts, then sums [sub][row]
-constexpr int kGemmUnits = kGemmRows * 3 * 32;       // 16-byte units of parts per super-block chunk
+// Y[32 rows][256 columns] per workgroup, K walked one super-block at a time: the X chunk of the
+// next super-block travels global -> registers while the current one is computed from LDS,
+// then registers -> the other LDS buffer, one barrier per super-block.  A wavefront owns a
+// 32-column tile for all of K (no K split: nothing to combine).  Here the three parts of X lie
+// along K instead of along the MFMA rows: a sub-block is six chained MFMAs (part x half) into
+// one D of 32 real rows -- lane (row c, half g) supplies the same K values as in the GEMV
+// kernel, from part 0, 1, 2 in turn against the same B -- so a row costs two multiply-adds per
+// sub-block and the weights are converted once per 32 rows.  (A first version with the parts
+// along the rows, ten rows per MFMA pass and four passes, measured 12-28 % slower.)
+constexpr int kG32Rows = 32;
+constexpr int kG32PartStride = 512 + 16;
+constexpr int kG32PartsBytes = kG32Rows * 3 * kG32PartStride;
+constexpr int kG32ChunkBytes = kG32PartsBytes + 8 * kG32Rows * 4;  // parts, then sums [sub][row]
+constexpr int kG32Units = kG32Rows * 3 * 32;
 
-// Y[40 rows][256 columns] per workgroup, K walked one super-block at a time: the X chunk of
-// the next super-block travels global -> registers while the current one is computed from
-// LDS, then registers -> the other LDS buffer, one barrier per super-block.  A wavefront owns
-// a 32-column tile for all of K (no K split: nothing to combine).  Operand mapping as in
-// gemv_q4k_mfma_kernel, packed tighter: lane half h's sixteen x columns hold the three
-// parts of rows 5 h .. 5 h + 4 of the 10-row block (x column 8 q + 4 h + r = slot 4 q + r =
-// 3 * row + part), so D registers 3 i, 3 i + 1, 3 i + 2 are row 5 h + i.
-template <int kGemmTiles>  // column tiles (wavefronts) per workgroup
-__global__ __launch_bounds__(64 * kGemmTiles) void gemm_q4k_mfma_kernel(float* __restrict__ dst, const uint32_t* __restrict__ parts,
-                                                            const float* __restrict__ xsum, const uint8_t* __restrict__ weight,
-                                                            int rows, int in_dim, int out_dim, Epilogue ep) {
+__global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict__ dst, const uint32_t* __restrict__ parts,
+                                                              const float* __restrict__ xsum, const uint8_t* __restrict__ weight,
+                                                              int rows, int in_dim, int out_dim, Epilogue ep) {
     const int kb = in_dim >> 8;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_tiles = (out_dim + kTileCols - 1) >> 5;
-    const int tile_raw = blockIdx.x * kGemmTiles + wave;
+    const int tile_raw = blockIdx.x * 8 + wave;
     const bool tile_ok = tile_raw < n_tiles;
     const int tile = tile_ok ? tile_raw : n_tiles - 1;  // a spare wavefront repeats the last tile and stores nothing
-    const int row0 = blockIdx.y * kGemmRows;
-    const int rows_here = min(kGemmRows, rows - row0);
-    const int row_blocks = (rows_here + 9) / 10;  // workgroup-uniform
+    const int row0 = blockIdx.y * kG32Rows;
+    const int rows_here = min(kG32Rows, rows - row0);
     const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
-    const int groups_per_row = in_dim >> 3;  // 16-byte units of one part of one row
+    const int groups_per_row = in_dim >> 3;
 
-    // ---- the X chunk of one super-block: this thread's share, global -> registers -> LDS
-    constexpr int kThreads = 64 * kGemmTiles;
-    constexpr int kUnitsPerThread = (kGemmUnits + kThreads - 1) / kThreads;
-    constexpr int kSumsPerThread = (kGemmRows * 8 + kThreads - 1) / kThreads;
+    constexpr int kUnitsPerThread = kG32Units / 512;  // 6
     uint4 stage[kUnitsPerThread];
-    float stage_sum[kSumsPerThread];
+    float stage_sum = 0.0f;
     auto fetch = [&](int sb) {
 #pragma unroll
         for (int i = 0; i < kUnitsPerThread; ++i) {
-            const int u = tid + i * kThreads;
-            if (u < kGemmUnits) {
-                const int rp = u >> 5, k16 = u & 31;  // (row, part), 16-byte unit inside the super-block
-                const int r = min(rp / 3, rows_here - 1), part = rp - (rp / 3) * 3;  // rows past the end repeat the last one
-                stage[i] = reinterpret_cast<const uint4*>(parts)[(static_cast<size_t>(row0 + r) * 3 + part) * groups_per_row + sb * 32 + k16];
-            }
+            const int u = tid + i * 512;
+            const int rp = u >> 5, k16 = u & 31;
+            const int r = min(rp / 3, rows_here - 1), part = rp - (rp / 3) * 3;  // rows past the end repeat the last one
+            stage[i] = reinterpret_cast<const uint4*>(parts)[(static_cast<size_t>(row0 + r) * 3 + part) * groups_per_row + sb * 32 + k16];
         }
-#pragma unroll
-        for (int i = 0; i < kSumsPerThread; ++i) {
-            const int u = tid + i * kThreads;
-            if (u < kGemmRows * 8) {
-                const int r = min(u >> 3, rows_here - 1), sub = u & 7;
-                stage_sum[i] = xsum[static_cast<size_t>(row0 + r) * (kb * 8) + sb * 8 + sub];
-            }
+        if (tid < kG32Rows * 8) {
+            const int r = min(tid >> 3, rows_here - 1), sub = tid & 7;
+            stage_sum = xsum[static_cast<size_t>(row0 + r) * (kb * 8) + sb * 8 + sub];
         }
     };
     auto deposit = [&](int buffer) {
-        unsigned char* chunk = q4k_mfma_lds + buffer * kGemmChunkBytes;
+        unsigned char* chunk = q4k_mfma_lds + buffer * kG32ChunkBytes;
 #pragma unroll
         for (int i = 0; i < kUnitsPerThread; ++i) {
-            const int u = tid + i * kThreads;
-            if (u < kGemmUnits) *reinterpret_cast<uint4*>(chunk + (u >> 5) * kGemmPartStride + (u & 31) * 16) = stage[i];
+            const int u = tid + i * 512;
+            *reinterpret_cast<uint4*>(chunk + (u >> 5) * kG32PartStride + (u & 31) * 16) = stage[i];
         }
-#pragma unroll
-        for (int i = 0; i < kSumsPerThread; ++i) {
-            const int u = tid + i * kThreads;
-            if (u < kGemmRows * 8)
-                reinterpret_cast<float*>(chunk + kGemmRows * 3 * kGemmPartStride)[(u & 7) * kGemmSumStride + (u >> 3)] = stage_sum[i];
-        }
+        if (tid < kG32Rows * 8) reinterpret_cast<float*>(chunk + kG32PartsBytes)[(tid & 7) * kG32Rows + (tid >> 3)] = stage_sum;
     };
 
-    // ---- this lane's roles
     const int c = lane & 31, g = lane >> 5;
-    // A operand: x column c = 8 q + 4 h + r is slot 4 q + r of half h: row 5 h + slot / 3, part slot % 3
-    const int a_slot = 4 * (c >> 3) + (c & 3), a_half = (c >> 2) & 1;
-    const int a_row = 5 * a_half + min(a_slot / 3, 4), a_part = a_slot == 15 ? 0 : a_slot % 3;  // slot 15 carries nothing
-    const int a_offset = (a_row * 3 + a_part) * kGemmPartStride + 32 * g;
-    float acc[kGemmRowBlocks][5];
+    const int a_offset = c * 3 * kG32PartStride + 32 * g;  // A operand: row c of the block, K half g
+    float acc[16];
 #pragma unroll
-    for (int rb = 0; rb < kGemmRowBlocks; ++rb)
-#pragma unroll
-        for (int i = 0; i < 5; ++i) acc[rb][i] = 0.0f;
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
 
     t_u32x4 hdr, qv[4], hdr_next, qv_next[4];
     auto request = [&](int sb, t_u32x4& h, t_u32x4 (&q)[4]) {
@@ -461,8 +440,8 @@ __global__ __launch_bounds__(64 * kGemmTiles) void gemm_q4k_mfma_kernel(float* _
             fetch(sb + 1);
             request(sb + 1, hdr_next, qv_next);
         }
-        const unsigned char* chunk = q4k_mfma_lds + (sb & 1) * kGemmChunkBytes;
-        const float* sums = reinterpret_cast<const float*>(chunk + kGemmRows * 3 * kGemmPartStride);
+        const unsigned char* chunk = q4k_mfma_lds + (sb & 1) * kG32ChunkBytes;
+        const float* sums = reinterpret_cast<const float*>(chunk + kG32PartsBytes);
         const float d = half_bits_to_f32(static_cast<uint16_t>(hdr.x & 0xFFFFu));
         const float dmin = half_bits_to_f32(static_cast<uint16_t>(hdr.x >> 16));
         const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, mn_lo = hdr.z & 0x3F3F3F3Fu;
@@ -474,44 +453,47 @@ __global__ __launch_bounds__(64 * kGemmTiles) void gemm_q4k_mfma_kernel(float* _
 #pragma unroll
             for (int hi = 0; hi < 2; ++hi) {
                 const int sub = 2 * t + hi;
-                // the sub-block's 32 x 32 weights as bf16, once for all row blocks
-                union {
-                    t_bf16x8 v;
-                    t_bf16x2 pair[4];
-                } b[2];
+                t_f32x16 D = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int m = 0; m < 2; ++m) {
+                    union {
+                        t_bf16x8 v;
+                        t_bf16x2 pair[4];
+                    } b;
 #pragma unroll
                     for (int k = 0; k < 2; ++k) {
                         const uint32_t nib = hi ? (w[2 * m + k] >> 4) & 0x0F0F0F0Fu : w[2 * m + k] & 0x0F0F0F0Fu;
-                        b[m].pair[2 * k] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, false);
-                        b[m].pair[2 * k + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, true);
+                        b.pair[2 * k] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, false);
+                        b.pair[2 * k + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, true);
                     }
-                }
-                const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
-                const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
-                const float dsc = d * sc, dmn = dmin * mn;
 #pragma unroll
-                for (int rb = 0; rb < kGemmRowBlocks; ++rb) {
-                    if (rb >= row_blocks) continue;  // uniform
-                    t_f32x16 D = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int m = 0; m < 2; ++m) {
+                    for (int part = 0; part < 3; ++part) {
                         union {
                             t_bf16x8 v;
                             uint4 u;
                         } a;
-                        a.u = *reinterpret_cast<const uint4*>(chunk + rb * 30 * kGemmPartStride + a_offset + (32 * sub + 8 * m) * 2);
-                        D = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b[m].v, D, 0, 0, 0);
-                    }
-#pragma unroll
-                    for (int i = 0; i < 5; ++i) {
-                        const float X = sums[sub * kGemmSumStride + rb * 10 + 5 * g + i];
-                        const float S = (D[3 * i] + D[3 * i + 1]) + D[3 * i + 2];
-                        acc[rb][i] = __builtin_fmaf(dsc, S, acc[rb][i]);
-                        acc[rb][i] = __builtin_fmaf(-dmn, X, acc[rb][i]);
+                        a.u = *reinterpret_cast<const uint4*>(chunk + a_offset + part * kG32PartStride + (32 * sub + 8 * m) * 2);
+                        D = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, D, 0, 0, 0);
                     }
                 }
+                const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
+                const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
+                const float dsc = d * sc, ndmn = -(dmin * mn);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    // D registers 4 q .. 4 q + 3 are rows 8 q + 4 g + 0..3
+                    const float4 X = *reinterpret_cast<const float4*>(sums + sub * kG32Rows + 8 * q + 4 * g);
+                    const float xs[4] = {X.x, X.y, X.z, X.w};
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        acc[4 * q + i] = __builtin_fmaf(dsc, D[4 * q + i], acc[4 * q + i]);
+                        acc[4 * q + i] = __builtin_fmaf(ndmn, xs[i], acc[4 * q + i]);
+                    }
+                }
+                // pin the sub-block's accumulation here: left to itself the compiler keeps eight D sets
+                // and all their operands alive and does the accumulation at the end (spills)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(acc[i]));
             }
         }
         if (more) {
@@ -527,15 +509,13 @@ __global__ __launch_bounds__(64 * kGemmTiles) void gemm_q4k_mfma_kernel(float* _
     const int o = tile * kTileCols + c;
     if (o >= out_dim) return;
 #pragma unroll
-    for (int rb = 0; rb < kGemmRowBlocks; ++rb)
-#pragma unroll
-        for (int i = 0; i < 5; ++i) {
-            const int r = rb * 10 + 5 * g + i;
-            if (r < rows_here) {
-                const size_t at = static_cast<size_t>(row0 + r) * out_dim + o;
-                dst[at] = finish_output(ep, o, at, acc[rb][i]);
-            }
+    for (int i = 0; i < 16; ++i) {
+        const int r = 8 * (i >> 2) + 4 * g + (i & 3);
+        if (r < rows_here) {
+            const size_t at = static_cast<size_t>(row0 + r) * out_dim + o;
+            dst[at] = finish_output(ep, o, at, acc[i]);
         }
+    }
 }
 
 size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
@@ -630,8 +610,9 @@ int gemv_q4k_tiled_rows_per_launch(int in_dim) {
 }
 
 // From this many rows on the GEMM beats the GEMV served six rows at a time (measured on
-// 14336 x 4096: 64 rows 143 us against 149 us, 40 rows 138 us against 95 us).
-int gemm_q4k_min_rows() { return 48; }
+// 14336 x 4096: a workgroup's K walk takes about 100 us whatever its rows, 64 rows 100 us
+// against 150 us, 32 rows about 90 us either way).
+int gemm_q4k_min_rows() { return 40; }
 
 size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim) { return rows * in_dim * 6 + rows * (in_dim / 32) * 4; }
 
@@ -649,24 +630,19 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     }
     const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
-    const unsigned grid_y = static_cast<unsigned>((rows + kGemmRows - 1) / kGemmRows);
+    const unsigned grid_y = static_cast<unsigned>((rows + kG32Rows - 1) / kG32Rows);
     if (grid_y > 65535) return hipErrorInvalidValue;
-    // eight column tiles a workgroup, one per wavefront (two-tile workgroups for small problems
-    // measured slower: every thread then stages four times as much of X)
-    constexpr int tiles = 8;
-    auto kernel = gemm_q4k_mfma_kernel<tiles>;
-    const unsigned grid_x = static_cast<unsigned>((n_tiles + tiles - 1) / tiles);
-    constexpr size_t lds = 2 * kGemmChunkBytes;
+    const unsigned grid_x = static_cast<unsigned>((n_tiles + 7) / 8);
     static bool large_lds = false;  // raising the limit is sticky per kernel: once, outside any stream capture opened later
     if (!large_lds) {
-        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               160 * 1024);
+        if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4k_rows32_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             e != hipSuccess)
             return e;
         large_lds = true;
     }
-    hipLaunchKernelGGL(kernel, dim3(grid_x, grid_y), dim3(64 * tiles), lds, stream, dst, parts, xsum, weight, rows, in_dim, out_dim,
-                       ep);
+    hipLaunchKernelGGL(gemm_q4k_rows32_kernel, dim3(grid_x, grid_y), dim3(512), 2 * kG32ChunkBytes, stream, dst, parts, xsum,
+                       weight, rows, in_dim, out_dim, ep);
     return hipGetLastError();
 }
 

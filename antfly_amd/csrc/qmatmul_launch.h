@@ -96,7 +96,7 @@ hipError_t launch_q4k_tile_repack(hipStream_t stream, uint8_t* dst, const uint8_
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                                  int out_dim, const Epilogue& ep = Epilogue{});
 // More rows than one launch of the kernel above holds (gemv_q4k_tiled_rows_per_launch): X is split
-// once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned) and a GEMM walks K for 40 rows
+// once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned) and a GEMM walks K for 32 rows
 // x 256 columns per workgroup.  Any in_dim that is a multiple of 256.  split = false: `workspace`
 // already holds the split of this X (a second matrix on the same input).
 int gemv_q4k_tiled_rows_per_launch(int in_dim);
