@@ -490,11 +490,12 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
                         acc[4 * q + i] = __builtin_fmaf(ndmn, xs[i], acc[4 * q + i]);
                     }
                 }
-                // pin the sub-block's accumulation here: left to itself the compiler keeps eight D sets
-                // and all their operands alive and does the accumulation at the end (spills)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(acc[i]));
             }
+            // pin the accumulation of these two sub-blocks here: left to itself the compiler keeps
+            // eight D sets and all their operands alive and does the accumulation at the end
+            // (spills); two sets let one sub-block's MFMAs run under the other's accumulation
+#pragma unroll
+            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(acc[i]));
         }
         if (more) {
             deposit((sb + 1) & 1);
