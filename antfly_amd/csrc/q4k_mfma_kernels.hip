@@ -376,8 +376,13 @@ constexpr int kG32Units = kG32Rows * 3 * 32;
 
 __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict__ dst, const uint32_t* __restrict__ parts,
                                                               const float* __restrict__ xsum, const uint8_t* __restrict__ weight,
-                                                              int rows, int in_dim, int out_dim, Epilogue ep) {
+                                                              int rows, int in_dim, int out_dim, int sb_per_split,
+                                                              float* __restrict__ partial, Epilogue ep) {
     const int kb = in_dim >> 8;
+    // K range of this workgroup: all of it, or (a small problem spread over more compute units)
+    // share blockIdx.z, whose sums go to partial[z][rows][out_dim] for q4k_splitk_reduce_kernel
+    const int sb_begin = blockIdx.z * sb_per_split;
+    const int sb_end = min(kb, sb_begin + sb_per_split);
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n_tiles = (out_dim + kTileCols - 1) >> 5;
@@ -430,12 +435,13 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
             q[t] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 512 + t * 1024 + 16 * lane));
     };
 
-    fetch(0);
-    request(0, hdr, qv);
-    deposit(0);
+    if (sb_begin >= sb_end) return;  // workgroup-uniform (the host sends no empty shares)
+    fetch(sb_begin);
+    request(sb_begin, hdr, qv);
+    deposit(sb_begin & 1);
     __syncthreads();
-    for (int sb = 0; sb < kb; ++sb) {
-        const bool more = sb + 1 < kb;  // uniform
+    for (int sb = sb_begin; sb < sb_end; ++sb) {
+        const bool more = sb + 1 < sb_end;  // uniform
         if (more) {
             fetch(sb + 1);
             request(sb + 1, hdr_next, qv_next);
@@ -514,8 +520,20 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
         const int r = 8 * (i >> 2) + 4 * g + (i & 3);
         if (r < rows_here) {
             const size_t at = static_cast<size_t>(row0 + r) * out_dim + o;
-            dst[at] = finish_output(ep, o, at, acc[i]);
+            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.z) * rows * out_dim + at] = acc[i];
+            else dst[at] = finish_output(ep, o, at, acc[i]);
         }
+    }
+}
+
+// dst = epilogue(sum over the K shares, in order) for the split-K launches of the GEMM.
+__global__ __launch_bounds__(256) void q4k_splitk_reduce_kernel(float* __restrict__ dst, const float* __restrict__ partial,
+                                                                size_t count, int out_dim, int splits, Epilogue ep) {
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        float total = 0.0f;
+        for (int z = 0; z < splits; ++z) total += partial[static_cast<size_t>(z) * count + i];
+        dst[i] = finish_output(ep, static_cast<int>(i % out_dim), i, total);
     }
 }
 
@@ -610,18 +628,50 @@ int gemv_q4k_tiled_rows_per_launch(int in_dim) {
     return per_launch;
 }
 
-// From this many rows on the GEMM beats the GEMV served six rows at a time (measured on
-// 14336 x 4096: a workgroup's K walk takes about 100 us whatever its rows, 64 rows 100 us
-// against 150 us, 32 rows about 90 us either way).
-int gemm_q4k_min_rows() { return 40; }
+// From this many rows on (three GEMV launches of six rows) the GEMM is the faster way: a
+// workgroup's walk over all of K = 4096 takes about 100 us whatever its rows, and small problems
+// split K over up to eight workgroups whose sums a second kernel adds up.
+int gemm_q4k_min_rows() { return 13; }
 
-size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim) { return rows * in_dim * 6 + rows * (in_dim / 32) * 4; }
+namespace {
+int device_units() {
+    static const int cus = []() {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return cus;
+}
+
+// K shares of the GEMM: one when its workgroups fill the compute units anyway, else as many
+// (a power of two, at most eight, at least two super-blocks each) as spread it over them.
+int gemm_q4k_splits(size_t rows, size_t in_dim, size_t out_dim) {
+    const long workgroups = static_cast<long>((out_dim + 255) / 256) * static_cast<long>((rows + kG32Rows - 1) / kG32Rows);
+    const int kb = static_cast<int>(in_dim / kQ4kBlockValues);
+    int splits = 1;
+    while (splits < 8 && workgroups * splits * 2 <= device_units() && kb / (splits * 2) >= 2) splits *= 2;
+    return splits;
+}
+
+size_t gemm_q4k_split_bytes(size_t rows, size_t in_dim) { return (rows * in_dim * 6 + rows * (in_dim / 32) * 4 + 255) / 256 * 256; }
+}  // namespace
+
+size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim, size_t out_dim) {
+    const int splits = gemm_q4k_splits(rows, in_dim, out_dim);
+    return gemm_q4k_split_bytes(rows, in_dim) + (splits > 1 ? static_cast<size_t>(splits) * rows * out_dim * 4 : 0);
+}
 
 hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, void* workspace,
                                  int rows, int in_dim, int out_dim, const Epilogue& ep, bool split) {
     if (in_dim % kQ4kBlockValues != 0 || rows < 1 || workspace == nullptr) return hipErrorInvalidValue;
     uint32_t* parts = static_cast<uint32_t*>(workspace);
     float* xsum = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + static_cast<size_t>(rows) * in_dim * 6);
+    const int splits = gemm_q4k_splits(rows, in_dim, out_dim);
+    const int kb = in_dim / kQ4kBlockValues;
+    const int sb_per_split = (kb + splits - 1) / splits;
+    const int shares = (kb + sb_per_split - 1) / sb_per_split;  // no empty share
+    float* partial = shares > 1 ? reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + gemm_q4k_split_bytes(rows, in_dim)) : nullptr;
     if (split) {
         const size_t groups = static_cast<size_t>(rows) * (in_dim >> 3);
         size_t split_grid = (groups + 255) / 256;
@@ -642,8 +692,14 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
             return e;
         large_lds = true;
     }
-    hipLaunchKernelGGL(gemm_q4k_rows32_kernel, dim3(grid_x, grid_y), dim3(512), 2 * kG32ChunkBytes, stream, dst, parts, xsum,
-                       weight, rows, in_dim, out_dim, ep);
+    hipLaunchKernelGGL(gemm_q4k_rows32_kernel, dim3(grid_x, grid_y, shares), dim3(512), 2 * kG32ChunkBytes, stream, dst, parts,
+                       xsum, weight, rows, in_dim, out_dim, sb_per_split, partial, ep);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess || shares == 1) return e;
+    const size_t count = static_cast<size_t>(rows) * out_dim;
+    size_t reduce_grid = (count + 255) / 256;
+    if (reduce_grid > 4096) reduce_grid = 4096;
+    hipLaunchKernelGGL(q4k_splitk_reduce_kernel, dim3(static_cast<unsigned>(reduce_grid)), dim3(256), 0, stream, dst, partial, count,
+                       out_dim, shares, ep);
     return hipGetLastError();
 }
 

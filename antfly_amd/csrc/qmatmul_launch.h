@@ -96,12 +96,13 @@ hipError_t launch_q4k_tile_repack(hipStream_t stream, uint8_t* dst, const uint8_
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                                  int out_dim, const Epilogue& ep = Epilogue{});
 // More rows than one launch of the kernel above holds (gemv_q4k_tiled_rows_per_launch): X is split
-// once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned) and a GEMM walks K for 32 rows
+// once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned; it also holds the partial sums when a
+// small problem splits K over several workgroups) and a GEMM walks K for 32 rows
 // x 256 columns per workgroup.  Any in_dim that is a multiple of 256.  split = false: `workspace`
 // already holds the split of this X (a second matrix on the same input).
 int gemv_q4k_tiled_rows_per_launch(int in_dim);
 int gemm_q4k_min_rows();  // fewer rows are faster on the GEMV, a launch at a time
-size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim);
+size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim, size_t out_dim);
 hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, void* workspace,
                                  int rows, int in_dim, int out_dim, const Epilogue& ep = Epilogue{}, bool split = true);
 hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,

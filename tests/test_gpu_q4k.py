@@ -107,7 +107,7 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
 
 
 PREFILL_SHAPES = [(7, 4096, 64), (10, 1024, 300), (11, 512, 33), (40, 2048, 256), (41, 1024, 257), (100, 512, 1000),
-                  (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (39, 512, 40), (40, 512, 40), (33, 1024, 64), (64, 1024, 96), (50, 14336, 64),
+                  (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (12, 512, 40), (13, 512, 40), (13, 4096, 300), (33, 1024, 64), (64, 1024, 96), (20, 2560, 700), (50, 14336, 64),
                   (81, 768, 500)]
 
 
@@ -162,7 +162,8 @@ def test_linear_argument_checks():
     with pytest.raises(_lib.HipError):  # no integer route, so no block dots
         kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
     assert kernels.workspaceBytes(Q4K, 4, 4096, 4096) == 0  # decode rows need no scratch
-    assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) == 64 * 4096 * 6 + 64 * 128 * 4  # the split of X for the prefill GEMM
+    assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 128 * 4  # the split of X for the prefill GEMM
+    assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) > 64 * 4096 * 6 + 64 * 128 * 4  # ... plus partial sums when K is shared out
     big_w = torch.zeros(4 * 128 * 144, dtype=torch.uint8, device=G.DEV)
     big_x = torch.zeros(32768, dtype=torch.float32, device=G.DEV)
     with pytest.raises(_lib.HipOpUnsupported):  # K beyond what one workgroup's slices cover
