@@ -23,6 +23,8 @@
 //   * a launch may serve two matrices of the same shape that share X (GemvTargets).
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "device_common.h"
 #include "qmatmul_launch.h"
 
@@ -634,11 +636,11 @@ int workgroup_waves(int requested_threads, int max_threads, int slices, int grou
 // Raising the dynamic-LDS limit is sticky per kernel: done once per kernel, outside
 // any stream capture a caller may open later.
 template <typename Kernel>
-hipError_t allow_large_lds(Kernel kernel, size_t lds, size_t* limit) {
-    if (lds <= *limit) return hipSuccess;
+hipError_t allow_large_lds(Kernel kernel, size_t lds, std::atomic<size_t>* limit) {
+    if (lds <= limit->load(std::memory_order_acquire)) return hipSuccess;
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                        160 * 1024);
-    if (e == hipSuccess) *limit = 160 * 1024;
+    if (e == hipSuccess) limit->store(160 * 1024, std::memory_order_release);  // (two host threads may both get here: the call is idempotent)
     return e;
 }
 
@@ -661,7 +663,7 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
     auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax>;
-    static size_t lds_limit = 64 * 1024;
+    static std::atomic<size_t> lds_limit{64 * 1024};
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     if (key_count) *key_count = grid;
@@ -682,7 +684,7 @@ hipError_t launch_rows(hipStream_t stream, const GemvTargets& tg0, int* dots, co
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(rows, in_dim);
     auto kernel = gemv_rows_kernel<kType, kCols, kDots>;
-    static size_t lds_limit = 64 * 1024;
+    static std::atomic<size_t> lds_limit{64 * 1024};
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots,

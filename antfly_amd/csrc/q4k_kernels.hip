@@ -8,6 +8,8 @@
 // so a lane reads the 16-byte header and a 16-byte run of nibbles with one load each.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <stdint.h>
 
 #include "device_common.h"
@@ -320,7 +322,7 @@ hipError_t launch_q4k_rows(hipStream_t stream, float* dst, const float* x, const
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     const size_t lds = q4k_lds_bytes(kRows, in_dim);
     auto kernel = gemv_q4k_kernel<kRows, kCols>;
-    static bool large_lds = false;  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    static std::atomic<bool> large_lds{false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
     if (lds > 64 * 1024 && !large_lds) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             e != hipSuccess)

@@ -34,6 +34,8 @@
 // is a multiple of 32.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <stdint.h>
 
 #include <cstdlib>
@@ -394,29 +396,41 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
     const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
     const int groups_per_row = in_dim >> 3;
 
-    constexpr int kUnitsPerThread = kG32Units / 512;  // 6
-    uint4 stage[kUnitsPerThread];
+    static_assert(kG32Units == 6 * 512, "six 16-byte units of the X chunk per thread");
+    // (six named registers, not an array: the array stayed in scratch memory across the two
+    // branches that fill and drain it)
+    uint4 stage0, stage1, stage2, stage3, stage4, stage5;
     float stage_sum = 0.0f;
+    auto fetch_unit = [&](int i, int sb) {
+        const int u = tid + i * 512;
+        const int rp = u >> 5, k16 = u & 31;
+        const int r = min(rp / 3, rows_here - 1), part = rp - (rp / 3) * 3;  // rows past the end repeat the last one
+        return reinterpret_cast<const uint4*>(parts)[(static_cast<size_t>(row0 + r) * 3 + part) * groups_per_row + sb * 32 + k16];
+    };
     auto fetch = [&](int sb) {
-#pragma unroll
-        for (int i = 0; i < kUnitsPerThread; ++i) {
-            const int u = tid + i * 512;
-            const int rp = u >> 5, k16 = u & 31;
-            const int r = min(rp / 3, rows_here - 1), part = rp - (rp / 3) * 3;  // rows past the end repeat the last one
-            stage[i] = reinterpret_cast<const uint4*>(parts)[(static_cast<size_t>(row0 + r) * 3 + part) * groups_per_row + sb * 32 + k16];
-        }
+        stage0 = fetch_unit(0, sb);
+        stage1 = fetch_unit(1, sb);
+        stage2 = fetch_unit(2, sb);
+        stage3 = fetch_unit(3, sb);
+        stage4 = fetch_unit(4, sb);
+        stage5 = fetch_unit(5, sb);
         if (tid < kG32Rows * 8) {
             const int r = min(tid >> 3, rows_here - 1), sub = tid & 7;
             stage_sum = xsum[static_cast<size_t>(row0 + r) * (kb * 8) + sb * 8 + sub];
         }
     };
+    auto deposit_unit = [&](unsigned char* chunk, int i, const uint4& v) {
+        const int u = tid + i * 512;
+        *reinterpret_cast<uint4*>(chunk + (u >> 5) * kG32PartStride + (u & 31) * 16) = v;
+    };
     auto deposit = [&](int buffer) {
         unsigned char* chunk = q4k_mfma_lds + buffer * kG32ChunkBytes;
-#pragma unroll
-        for (int i = 0; i < kUnitsPerThread; ++i) {
-            const int u = tid + i * 512;
-            *reinterpret_cast<uint4*>(chunk + (u >> 5) * kG32PartStride + (u & 31) * 16) = stage[i];
-        }
+        deposit_unit(chunk, 0, stage0);
+        deposit_unit(chunk, 1, stage1);
+        deposit_unit(chunk, 2, stage2);
+        deposit_unit(chunk, 3, stage3);
+        deposit_unit(chunk, 4, stage4);
+        deposit_unit(chunk, 5, stage5);
         if (tid < kG32Rows * 8) reinterpret_cast<float*>(chunk + kG32PartsBytes)[(tid & 7) * kG32Rows + (tid >> 3)] = stage_sum;
     };
 
@@ -453,56 +467,85 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
         const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, mn_lo = hdr.z & 0x3F3F3F3Fu;
         const uint32_t sc_hi = (hdr.w & 0x0F0F0F0Fu) | ((hdr.y >> 2) & 0x30303030u);
         const uint32_t mn_hi = ((hdr.w >> 4) & 0x0F0F0F0Fu) | ((hdr.z >> 2) & 0x30303030u);
+        // Software pipeline over the eight sub-blocks, written out because the compiler on its own
+        // waits for every LDS read right in front of the MFMA that uses it: the A fragments of
+        // sub-block s + 1 are requested before the MFMAs of s are issued, and the accumulation
+        // of s - 1 (vector ALU) runs while those MFMAs are in the matrix core.  Two D sets.
+        uint4 afrag[2][3];  // the three parts of one K half of a sub-block, current and next
+        float4 xs4[4];
+        t_f32x16 D[2];
+        auto load_a = [&](int half, uint4 (&a)[3]) {  // half = 2 * sub-block + m
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const uint32_t w[4] = {qv[t].x, qv[t].y, qv[t].z, qv[t].w};
+            for (int part = 0; part < 3; ++part)
+                a[part] = *reinterpret_cast<const uint4*>(chunk + a_offset + part * kG32PartStride + (32 * (half >> 1) + 8 * (half & 1)) * 2);
+        };
+        auto load_x = [&](int sub) {
 #pragma unroll
-            for (int hi = 0; hi < 2; ++hi) {
-                const int sub = 2 * t + hi;
-                t_f32x16 D = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int q = 0; q < 4; ++q)  // D registers 4 q .. 4 q + 3 are rows 8 q + 4 g + 0..3
+                xs4[q] = *reinterpret_cast<const float4*>(sums + sub * kG32Rows + 8 * q + 4 * g);
+        };
+        auto accumulate = [&](int sub, const t_f32x16& Dv) {
+            const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
+            const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
+            const float dsc = d * sc, ndmn = -(dmin * mn);
 #pragma unroll
-                for (int m = 0; m < 2; ++m) {
-                    union {
-                        t_bf16x8 v;
-                        t_bf16x2 pair[4];
-                    } b;
+            for (int q = 0; q < 4; ++q) {
+                const float xs[4] = {xs4[q].x, xs4[q].y, xs4[q].z, xs4[q].w};
 #pragma unroll
-                    for (int k = 0; k < 2; ++k) {
-                        const uint32_t nib = hi ? (w[2 * m + k] >> 4) & 0x0F0F0F0Fu : w[2 * m + k] & 0x0F0F0F0Fu;
-                        b.pair[2 * k] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, false);
-                        b.pair[2 * k + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, true);
-                    }
-#pragma unroll
-                    for (int part = 0; part < 3; ++part) {
-                        union {
-                            t_bf16x8 v;
-                            uint4 u;
-                        } a;
-                        a.u = *reinterpret_cast<const uint4*>(chunk + a_offset + part * kG32PartStride + (32 * sub + 8 * m) * 2);
-                        D = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, D, 0, 0, 0);
-                    }
-                }
-                const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
-                const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
-                const float dsc = d * sc, ndmn = -(dmin * mn);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    // D registers 4 q .. 4 q + 3 are rows 8 q + 4 g + 0..3
-                    const float4 X = *reinterpret_cast<const float4*>(sums + sub * kG32Rows + 8 * q + 4 * g);
-                    const float xs[4] = {X.x, X.y, X.z, X.w};
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        acc[4 * q + i] = __builtin_fmaf(dsc, D[4 * q + i], acc[4 * q + i]);
-                        acc[4 * q + i] = __builtin_fmaf(ndmn, xs[i], acc[4 * q + i]);
-                    }
+                for (int i = 0; i < 4; ++i) {
+                    acc[4 * q + i] = __builtin_fmaf(dsc, Dv[4 * q + i], acc[4 * q + i]);
+                    acc[4 * q + i] = __builtin_fmaf(ndmn, xs[i], acc[4 * q + i]);
                 }
             }
-            // pin the accumulation of these two sub-blocks here: left to itself the compiler keeps
-            // eight D sets and all their operands alive and does the accumulation at the end
-            // (spills); two sets let one sub-block's MFMAs run under the other's accumulation
+        };
+        union {
+            t_bf16x8 v;
+            t_bf16x2 pair[4];
+        } b[2];
+        load_a(0, afrag[0]);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(acc[i]));
+        for (int half = 0; half < 16; ++half) {
+            const int sub = half >> 1, m = half & 1;
+            const int t = sub >> 1, hi = sub & 1;  // low nibbles of chunk t: sub-block 2 t, high nibbles: 2 t + 1
+            if (half + 1 < 16) load_a(half + 1, afrag[(half + 1) & 1]);
+            if (m == 0) {
+                if (sub > 0) load_x(sub - 1);
+                const uint32_t w[4] = {qv[t].x, qv[t].y, qv[t].z, qv[t].w};
+#pragma unroll
+                for (int mm = 0; mm < 2; ++mm)
+#pragma unroll
+                    for (int k = 0; k < 2; ++k) {
+                        const uint32_t nib = hi ? (w[2 * mm + k] >> 4) & 0x0F0F0F0Fu : w[2 * mm + k] & 0x0F0F0F0Fu;
+                        b[mm].pair[2 * k] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, false);
+                        b[mm].pair[2 * k + 1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(static_cast<int>(nib), 512.0f, true);
+                    }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            t_f32x16 Dv;
+            if (m == 0) Dv = t_f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            else Dv = D[sub & 1];
+#pragma unroll
+            for (int part = 0; part < 3; ++part) {
+                union {
+                    t_bf16x8 v;
+                    uint4 u;
+                } a;
+                a.u = afrag[half & 1][part];
+                Dv = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b[m].v, Dv, 0, 0, 0);
+            }
+            D[sub & 1] = Dv;
+            __builtin_amdgcn_sched_barrier(0);
+            if (m == 0 && sub > 0) {
+                accumulate(sub - 1, D[(sub - 1) & 1]);
+                // pin the accumulation here: left to itself the compiler keeps every D set and its
+                // operands alive and accumulates at the end (spills)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) asm volatile("" : "+v"(acc[i]));
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
+        load_x(7);
+        accumulate(7, D[1]);
         if (more) {
             deposit((sb + 1) & 1);
             hdr = hdr_next;
@@ -582,7 +625,7 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
             break;
     }
     if (kernel == nullptr) return hipErrorInvalidValue;
-    static bool large_lds[6] = {false, false, false, false, false, false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    static std::atomic<bool> large_lds[6] = {};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
     if (lds > 64 * 1024 && !large_lds[variant]) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                160 * 1024);
@@ -684,7 +727,7 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
     const unsigned grid_y = static_cast<unsigned>((rows + kG32Rows - 1) / kG32Rows);
     if (grid_y > 65535) return hipErrorInvalidValue;
     const unsigned grid_x = static_cast<unsigned>((n_tiles + 7) / 8);
-    static bool large_lds = false;  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    static std::atomic<bool> large_lds{false};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
     if (!large_lds) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_q4k_rows32_kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);

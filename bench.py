@@ -63,7 +63,8 @@ def main() -> int:
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--counter-probe", action="store_true",
                     help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
-                         "read kernel over the same number of bytes and of the Q8_0 M=512 GEMM, then exit")
+                         "read kernel over the same number of bytes, of the Q8_0 M=512 GEMM and of the Q4_K kernels "
+                         "(M=1 and M=512), then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -299,6 +300,15 @@ def main() -> int:
         for i in range(n_launch):
             launch(stream, Q8, _lib.LAYOUT_PREPARED, buf(yg), buf(xg), buf(wg[i % 2]), 512, 4096, 4096, buf(sg), -1)
         torch.cuda.synchronize()
+        # Q4_K on the same matrix: the decode kernel (one row) and the prefill GEMM (512 rows)
+        wk = prepared_copies(Q4K, 14336, 4096, copies, 31)
+        for m in (1, 512):
+            xk = torch.from_numpy(synth.activations(32 + m, m, 4096)).to(dev)
+            yk = torch.empty((m, 14336), dtype=torch.float32, device=dev)
+            sk = torch.empty(max(kernels.workspaceBytes(Q4K, m, 4096, 14336), 16), dtype=torch.uint8, device=dev)
+            for i in range(n_launch):
+                launch(stream, Q4K, _lib.LAYOUT_PREPARED, buf(yk), buf(xk), buf(wk[i % copies]), m, 4096, 14336, buf(sk), -1)
+            torch.cuda.synchronize()
         print(json.dumps({"counter_probe": {"launches_each": n_launch, "gemv_bytes": gemv_bytes(Q4, 1, 4096, 14336),
                                             "stream_read_bytes": w_bytes}}))
         return 0
@@ -375,6 +385,8 @@ def main() -> int:
             ("q4_gemv_m8_k4096_n14336", Q4, 8, 4096, 14336),
             ("q4_gemv_m1_k14336_n4096", Q4, 1, 14336, 4096),
             ("q4_gemv_m5_k14336_n4096", Q4, 5, 14336, 4096),
+            ("q4_batch_m16_k4096_n14336", Q4, 16, 4096, 14336),  # batched decode: quantizer + MFMA GEMM, 32-row tiles
+            ("q4_batch_m64_k4096_n14336", Q4, 64, 4096, 14336),
         ]:
             copies = args.copies if fmt == Q4 else 2 * args.copies
             w_s, e_s = time_config(fmt, r, k, n, small_steps, 20, copies, 99)
@@ -390,7 +402,7 @@ def main() -> int:
                            "us_per_call": round(e_s / small_steps * 1e6, 3),
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
-        for m in (128, 512):
+        for m in (32, 128, 512):
             w_s, e_s = time_config(Q4K, m, 4096, 14336, 40, 5, 2, 78)
             flops = 2.0 * m * 4096 * 14336
             extra[f"q4k_gemm_m{m}_k4096_n14336"] = {
