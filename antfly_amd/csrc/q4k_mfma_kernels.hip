@@ -336,10 +336,10 @@ int tuning_int(const char* name) {
 
 // ------------------------------------------------------------------ prefill
 // Many rows (more than one GEMV launch holds): X is split once by its own kernel --
-// parts bf16 [rows][3][in_dim], sub-block sums f32 [rows][in_dim / 32] -- and the GEMM below
+// parts bf16 [rows][3][in_dim], sub-block sums as bf16 parts [rows][in_dim / 256][4][8] -- and the GEMM below
 // converts every weight once per 32 rows instead of once per launch of six.
 __global__ __launch_bounds__(256) void q4k_split_rows_kernel(const float* __restrict__ x, uint32_t* __restrict__ parts,
-                                                             float* __restrict__ xsum, size_t groups, int groups_per_row) {
+                                                             uint16_t* __restrict__ sum_parts, size_t groups, int groups_per_row) {
     // one thread per eight consecutive values; whole quads run together (groups is a multiple of four)
     for (size_t grp = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; grp < groups;
          grp += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -357,7 +357,19 @@ __global__ __launch_bounds__(256) void q4k_split_rows_kernel(const float* __rest
         for (int part = 0; part < 3; ++part)
             reinterpret_cast<uint4*>(parts)[(r * 3 + part) * groups_per_row + kg] =
                 make_uint4(p[part][0], p[part][1], p[part][2], p[part][3]);
-        if ((threadIdx.x & 3) == 0) xsum[r * (groups_per_row >> 2) + (kg >> 2)] = s;
+        // the sub-block sum, split the same way: 64 bytes per row and super-block,
+        // [part 0..2][sub-block 0..7] bf16 and a fourth group of zeros (the K padding of the MFMA)
+        uint16_t* cell = sum_parts + (r * (groups_per_row >> 5) + (kg >> 5)) * 32;
+        const int sub = (kg >> 2) & 7;
+        if ((threadIdx.x & 3) == 0) {
+            uint32_t hi, mid, lo;
+            split3_pair(s, 0.0f, &hi, &mid, &lo);
+            cell[sub] = static_cast<uint16_t>(hi);
+            cell[8 + sub] = static_cast<uint16_t>(mid);
+            cell[16 + sub] = static_cast<uint16_t>(lo);
+        } else if ((kg & 31) == 1) {
+            *reinterpret_cast<uint4*>(cell + 24) = make_uint4(0u, 0u, 0u, 0u);
+        }
     }
 }
 
@@ -373,11 +385,11 @@ __global__ __launch_bounds__(256) void q4k_split_rows_kernel(const float* __rest
 constexpr int kG32Rows = 32;
 constexpr int kG32PartStride = 512 + 16;
 constexpr int kG32PartsBytes = kG32Rows * 3 * kG32PartStride;
-constexpr int kG32ChunkBytes = kG32PartsBytes + 8 * kG32Rows * 4;  // parts, then sums [sub][row]
+constexpr int kG32ChunkBytes = kG32PartsBytes + kG32Rows * 64;  // parts, then the parts of the sums: [row][part 0..3][sub-block] bf16
 constexpr int kG32Units = kG32Rows * 3 * 32;
 
 __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict__ dst, const uint32_t* __restrict__ parts,
-                                                              const float* __restrict__ xsum, const uint8_t* __restrict__ weight,
+                                                              const uint16_t* __restrict__ sum_parts, const uint8_t* __restrict__ weight,
                                                               int rows, int in_dim, int out_dim, int sb_per_split,
                                                               float* __restrict__ partial, Epilogue ep) {
     const int kb = in_dim >> 8;
@@ -400,7 +412,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
     // (six named registers, not an array: the array stayed in scratch memory across the two
     // branches that fill and drain it)
     uint4 stage0, stage1, stage2, stage3, stage4, stage5;
-    float stage_sum = 0.0f;
+    uint4 stage_sum = make_uint4(0u, 0u, 0u, 0u);
     auto fetch_unit = [&](int i, int sb) {
         const int u = tid + i * 512;
         const int rp = u >> 5, k16 = u & 31;
@@ -414,9 +426,9 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
         stage3 = fetch_unit(3, sb);
         stage4 = fetch_unit(4, sb);
         stage5 = fetch_unit(5, sb);
-        if (tid < kG32Rows * 8) {
-            const int r = min(tid >> 3, rows_here - 1), sub = tid & 7;
-            stage_sum = xsum[static_cast<size_t>(row0 + r) * (kb * 8) + sb * 8 + sub];
+        if (tid < kG32Rows * 4) {  // 64 bytes of sum parts per row
+            const int r = min(tid >> 2, rows_here - 1);
+            stage_sum = reinterpret_cast<const uint4*>(sum_parts)[(static_cast<size_t>(row0 + r) * kb + sb) * 4 + (tid & 3)];
         }
     };
     auto deposit_unit = [&](unsigned char* chunk, int i, const uint4& v) {
@@ -431,7 +443,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
         deposit_unit(chunk, 3, stage3);
         deposit_unit(chunk, 4, stage4);
         deposit_unit(chunk, 5, stage5);
-        if (tid < kG32Rows * 8) reinterpret_cast<float*>(chunk + kG32PartsBytes)[(tid & 7) * kG32Rows + (tid >> 3)] = stage_sum;
+        if (tid < kG32Rows * 4) reinterpret_cast<uint4*>(chunk + kG32PartsBytes)[tid] = stage_sum;
     };
 
     const int c = lane & 31, g = lane >> 5;
@@ -461,7 +473,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
             request(sb + 1, hdr_next, qv_next);
         }
         const unsigned char* chunk = q4k_mfma_lds + (sb & 1) * kG32ChunkBytes;
-        const float* sums = reinterpret_cast<const float*>(chunk + kG32PartsBytes);
+        const unsigned char* sums = chunk + kG32PartsBytes + c * 64 + 16 * g;
         const float d = half_bits_to_f32(static_cast<uint16_t>(hdr.x & 0xFFFFu));
         const float dmin = half_bits_to_f32(static_cast<uint16_t>(hdr.x >> 16));
         const uint32_t sc_lo = hdr.y & 0x3F3F3F3Fu, mn_lo = hdr.z & 0x3F3F3F3Fu;
@@ -472,31 +484,17 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
         // sub-block s + 1 are requested before the MFMAs of s are issued, and the accumulation
         // of s - 1 (vector ALU) runs while those MFMAs are in the matrix core.  Two D sets.
         uint4 afrag[2][3];  // the three parts of one K half of a sub-block, current and next
-        float4 xs4[4];
         t_f32x16 D[2];
         auto load_a = [&](int half, uint4 (&a)[3]) {  // half = 2 * sub-block + m
 #pragma unroll
             for (int part = 0; part < 3; ++part)
                 a[part] = *reinterpret_cast<const uint4*>(chunk + a_offset + part * kG32PartStride + (32 * (half >> 1) + 8 * (half & 1)) * 2);
         };
-        auto load_x = [&](int sub) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q)  // D registers 4 q .. 4 q + 3 are rows 8 q + 4 g + 0..3
-                xs4[q] = *reinterpret_cast<const float4*>(sums + sub * kG32Rows + 8 * q + 4 * g);
-        };
         auto accumulate = [&](int sub, const t_f32x16& Dv) {
             const float sc = ubyte_to_f32(sub < 4 ? sc_lo : sc_hi, sub & 3);
-            const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
-            const float dsc = d * sc, ndmn = -(dmin * mn);
+            const float dsc = d * sc;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const float xs[4] = {xs4[q].x, xs4[q].y, xs4[q].z, xs4[q].w};
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc[4 * q + i] = __builtin_fmaf(dsc, Dv[4 * q + i], acc[4 * q + i]);
-                    acc[4 * q + i] = __builtin_fmaf(ndmn, xs[i], acc[4 * q + i]);
-                }
-            }
+            for (int i = 0; i < 16; ++i) acc[i] = __builtin_fmaf(dsc, Dv[i], acc[i]);
         };
         union {
             t_bf16x8 v;
@@ -509,7 +507,6 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
             const int t = sub >> 1, hi = sub & 1;  // low nibbles of chunk t: sub-block 2 t, high nibbles: 2 t + 1
             if (half + 1 < 16) load_a(half + 1, afrag[(half + 1) & 1]);
             if (m == 0) {
-                if (sub > 0) load_x(sub - 1);
                 const uint32_t w[4] = {qv[t].x, qv[t].y, qv[t].z, qv[t].w};
 #pragma unroll
                 for (int mm = 0; mm < 2; ++mm)
@@ -544,8 +541,25 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        load_x(7);
+        // The min term of the whole super-block, sum over sub-blocks of m[column][sub] * X[row][sub],
+        // is one more small product: A = the three bf16 parts of the eight sub-block sums of each
+        // row (K = part * 8 + sub, padded with zeros to 32), B = the eight 6-bit mins of each column.
+        union {
+            t_bf16x8 v;
+            uint4 u;
+        } sa0, sa1, mb;
+        sa0.u = *reinterpret_cast<const uint4*>(sums);       // parts 0 (g = 0) and 1 (g = 1)
+        sa1.u = *reinterpret_cast<const uint4*>(sums + 32);  // part 2 (g = 0) and the zeros (g = 1)
+        mb.u = make_uint4(bf16_pair(ubyte_to_f32(mn_lo, 0), ubyte_to_f32(mn_lo, 1)),
+                          bf16_pair(ubyte_to_f32(mn_lo, 2), ubyte_to_f32(mn_lo, 3)),
+                          bf16_pair(ubyte_to_f32(mn_hi, 0), ubyte_to_f32(mn_hi, 1)),
+                          bf16_pair(ubyte_to_f32(mn_hi, 2), ubyte_to_f32(mn_hi, 3)));
+        t_f32x16 T = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        T = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa0.v, mb.v, T, 0, 0, 0);
+        T = __builtin_amdgcn_mfma_f32_32x32x16_bf16(sa1.v, mb.v, T, 0, 0, 0);
         accumulate(7, D[1]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = __builtin_fmaf(-dmin, T[i], acc[i]);
         if (more) {
             deposit((sb + 1) & 1);
             hdr = hdr_next;
@@ -697,7 +711,7 @@ int gemm_q4k_splits(size_t rows, size_t in_dim, size_t out_dim) {
     return splits;
 }
 
-size_t gemm_q4k_split_bytes(size_t rows, size_t in_dim) { return (rows * in_dim * 6 + rows * (in_dim / 32) * 4 + 255) / 256 * 256; }
+size_t gemm_q4k_split_bytes(size_t rows, size_t in_dim) { return (rows * in_dim * 6 + rows * (in_dim / 32) * 8 + 255) / 256 * 256; }
 }  // namespace
 
 size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim, size_t out_dim) {
@@ -709,7 +723,7 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
                                  int rows, int in_dim, int out_dim, const Epilogue& ep, bool split) {
     if (in_dim % kQ4kBlockValues != 0 || rows < 1 || workspace == nullptr) return hipErrorInvalidValue;
     uint32_t* parts = static_cast<uint32_t*>(workspace);
-    float* xsum = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + static_cast<size_t>(rows) * in_dim * 6);
+    uint16_t* xsum = reinterpret_cast<uint16_t*>(static_cast<uint8_t*>(workspace) + static_cast<size_t>(rows) * in_dim * 6);
     const int splits = gemm_q4k_splits(rows, in_dim, out_dim);
     const int kb = in_dim / kQ4kBlockValues;
     const int sb_per_split = (kb + splits - 1) / splits;

@@ -162,8 +162,8 @@ def test_linear_argument_checks():
     with pytest.raises(_lib.HipError):  # no integer route, so no block dots
         kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
     assert kernels.workspaceBytes(Q4K, 4, 4096, 4096) == 0  # decode rows need no scratch
-    assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 128 * 4  # the split of X for the prefill GEMM
-    assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) > 64 * 4096 * 6 + 64 * 128 * 4  # ... plus partial sums when K is shared out
+    assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 128 * 8  # the split of X for the prefill GEMM
+    assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) > 64 * 4096 * 6 + 64 * 128 * 8  # ... plus partial sums when K is shared out
     big_w = torch.zeros(4 * 128 * 144, dtype=torch.uint8, device=G.DEV)
     big_x = torch.zeros(32768, dtype=torch.float32, device=G.DEV)
     with pytest.raises(_lib.HipOpUnsupported):  # K beyond what one workgroup's slices cover
