@@ -101,3 +101,24 @@ def test_launcher_argument_checks_before_any_launch():
         kernels.launchPrepareWeight(None, 2, Buffer(0x1000, 17), Buffer(0x2000, 18), 1, 32)
     with pytest.raises(_lib.InvalidHipState):
         kernels.launchQuantizeActivations(None, big, 1, 48, big, big)
+
+
+def test_q4_k_prefill_workspace_sizes():
+    """Scratch of the Q4_K prefill GEMM: none for decode rows, from 13 rows on the split of X
+    (three bf16 parts = 6 bytes per value, plus 64 bytes of sum parts per row and super-block) and,
+    while the row x column grid is small, room for the partial sums of the K shares (a power of
+    two, at most eight, at least two super-blocks each)."""
+    Q4K = _lib.TYPE_Q4_K
+    for rows in (1, 6, 12):
+        assert kernels.workspaceBytes(Q4K, rows, 4096, 4096) == 0
+    for rows, k, n in [(13, 4096, 14336), (64, 4096, 4096), (512, 4096, 14336), (40, 512, 40), (33, 14336, 4096)]:
+        split = (rows * k * 6 + rows * (k // 256) * 64 + 255) // 256 * 256
+        got = kernels.workspaceBytes(Q4K, rows, k, n)
+        extra = got - split
+        assert extra >= 0 and extra % (rows * n * 4) == 0, (rows, k, n, got)
+        shares = extra // (rows * n * 4)
+        assert shares in (0, 2, 4, 8) and (shares == 0 or (k // 256) // shares >= 2), (rows, k, n, shares)
+    # a grid that fills the chip anyway shares nothing out
+    assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 16 * 64
+    # the smallest prefill on a small matrix spreads K over workgroups
+    assert kernels.workspaceBytes(Q4K, 13, 4096, 4096) > 13 * 4096 * 6 + 13 * 16 * 64
