@@ -380,6 +380,7 @@ def main() -> int:
         small_steps = max(50, args.steps // 4)
         for name, fmt, r, k, n in [
             ("q8_gemv_m1_k4096_n4096", Q8, 1, 4096, 4096),
+            ("q8_gemv_m1_k4096_n14336", Q8, 1, 4096, 14336),
             ("q4_gemv_m2_k4096_n14336", Q4, 2, 4096, 14336),
             ("q4_gemv_m4_k4096_n14336", Q4, 4, 4096, 14336),
             ("q4_gemv_m8_k4096_n14336", Q4, 8, 4096, 14336),
@@ -388,7 +389,7 @@ def main() -> int:
             ("q4_batch_m16_k4096_n14336", Q4, 16, 4096, 14336),  # batched decode: quantizer + MFMA GEMM, 32-row tiles
             ("q4_batch_m64_k4096_n14336", Q4, 64, 4096, 14336),
         ]:
-            copies = args.copies if fmt == Q4 else 2 * args.copies
+            copies = args.copies if fmt == Q4 or n > 4096 else 2 * args.copies
             w_s, e_s = time_config(fmt, r, k, n, small_steps, 20, copies, 99)
             b = gemv_bytes(fmt, r, k, n)
             extra[name] = {"us_per_call": round(e_s / small_steps * 1e6, 3),
