@@ -12,7 +12,13 @@
  * aborts.  Device pointers are plain 64-bit addresses.  `stream` is a
  * hipStream_t (NULL = the null stream); all launches are asynchronous on it.
  * A backend instance is not thread-safe: one caller thread per instance
- * (ops/cuda/context.zig:44-105 has the same rule).
+ * (ops/cuda/context.zig:44-105 has the same rule).  The stateless layers (the
+ * dispatch vocabulary and the afhip_launch_* launchers) may be called from several
+ * host threads at once; calls that share a workspace buffer must be ordered on one
+ * stream, since the kernels of a call use it until the call's last kernel ends.
+ * The first launch of a kernel that needs more than 64 KiB of LDS raises that
+ * kernel's limit (hipFuncSetAttribute): make the first call of a shape class
+ * outside any stream capture.
  */
 #ifndef ANTFLY_HIP_QMATMUL_H
 #define ANTFLY_HIP_QMATMUL_H
