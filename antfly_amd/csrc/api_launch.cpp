@@ -112,8 +112,7 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     const int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim, AFHIP_FORMAT_Q4_K);
     // more rows than one GEMV launch holds: X split once into the caller's scratch, then the
     // GEMM (without scratch the GEMV serves them a launch at a time)
-    const size_t gemm_rows = std::max(static_cast<size_t>(gemm_q4k_min_rows()),
-                                      static_cast<size_t>(gemv_q4k_tiled_rows_per_launch(static_cast<int>(in_dim))) + 1);
+    const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
     const bool gemm = tiled && rows >= gemm_rows && workspace.ptr != 0 && workspace.ptr % 16 == 0 && workspace.len >= gemm_q4k_workspace_bytes(rows, in_dim, out_dim);
     for (int i = 0; i < (pair ? 2 : 1); ++i) {
         if (counters) {
@@ -515,8 +514,7 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
         if (in_dim == 0 || in_dim % 256 != 0 || in_dim > 0x7fffffff || out_dim == 0 || !checked_mul(rows, in_dim, &count) ||
             !checked_mul(count, 8, &bytes))
             return 0;
-        const size_t gemm_rows = std::max(static_cast<size_t>(gemm_q4k_min_rows()),
-                                          static_cast<size_t>(gemv_q4k_tiled_rows_per_launch(static_cast<int>(in_dim))) + 1);
+        const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
         return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
     }
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;

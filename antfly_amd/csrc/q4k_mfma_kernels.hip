@@ -685,10 +685,15 @@ int gemv_q4k_tiled_rows_per_launch(int in_dim) {
     return per_launch;
 }
 
-// From this many rows on (three GEMV launches of six rows) the GEMM is the faster way: a
-// workgroup's walk over all of K = 4096 takes about 100 us whatever its rows, and small problems
-// split K over up to eight workgroups whose sums a second kernel adds up.
-int gemm_q4k_min_rows() { return 13; }
+// From this many rows on -- more than one launch of the GEMV kernel holds (LDS bounds its rows:
+// six at K = 4096, one at K = 14336), and at least three -- the GEMM is the faster way (measured
+// against two GEMV launches: 23 us against 26-29 at K = 4096, N = 14336; 34 us against 61-180 for
+// 4-12 rows at K = 14336): small problems split K over up to eight workgroups whose sums a
+// second kernel adds up.
+int gemm_q4k_min_rows(int in_dim) {
+    const int one_launch = gemv_q4k_tiled_rows_per_launch(in_dim);
+    return one_launch + 1 > 3 ? one_launch + 1 : 3;
+}
 
 namespace {
 int device_units() {

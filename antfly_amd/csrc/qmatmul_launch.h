@@ -101,7 +101,7 @@ hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x,
 // x 256 columns per workgroup.  Any in_dim that is a multiple of 256.  split = false: `workspace`
 // already holds the split of this X (a second matrix on the same input).
 int gemv_q4k_tiled_rows_per_launch(int in_dim);
-int gemm_q4k_min_rows();  // fewer rows are faster on the GEMV, a launch at a time
+int gemm_q4k_min_rows(int in_dim);  // fewer rows fit one GEMV launch (or are two rows)
 size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim, size_t out_dim);
 hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, void* workspace,
                                  int rows, int in_dim, int out_dim, const Epilogue& ep = Epilogue{}, bool split = true);

@@ -107,7 +107,7 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
 
 
 PREFILL_SHAPES = [(7, 4096, 64), (10, 1024, 300), (11, 512, 33), (40, 2048, 256), (41, 1024, 257), (100, 512, 1000),
-                  (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (12, 512, 40), (13, 512, 40), (13, 4096, 300), (33, 1024, 64), (64, 1024, 96), (20, 2560, 700), (50, 14336, 64),
+                  (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (8, 512, 40), (9, 512, 40), (12, 512, 40), (13, 4096, 300), (7, 4096, 300), (3, 14336, 64), (5, 14336, 200), (33, 1024, 64), (64, 1024, 96), (20, 2560, 700), (50, 14336, 64),
                   (81, 768, 500)]
 
 

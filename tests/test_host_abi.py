@@ -104,13 +104,17 @@ def test_launcher_argument_checks_before_any_launch():
 
 
 def test_q4_k_prefill_workspace_sizes():
-    """Scratch of the Q4_K prefill GEMM: none for decode rows, from 13 rows on the split of X
+    """Scratch of the Q4_K prefill GEMM: none for rows that fit one GEMV launch (six at K = 4096,
+    one at K = 14336; two rows never), beyond that the split of X
     (three bf16 parts = 6 bytes per value, plus 64 bytes of sum parts per row and super-block) and,
     while the row x column grid is small, room for the partial sums of the K shares (a power of
     two, at most eight, at least two super-blocks each)."""
     Q4K = _lib.TYPE_Q4_K
-    for rows in (1, 6, 12):
+    for rows in (1, 6):
         assert kernels.workspaceBytes(Q4K, rows, 4096, 4096) == 0
+    assert kernels.workspaceBytes(Q4K, 7, 4096, 4096) > 0
+    assert kernels.workspaceBytes(Q4K, 2, 14336, 4096) == 0
+    assert kernels.workspaceBytes(Q4K, 3, 14336, 4096) > 0
     for rows, k, n in [(13, 4096, 14336), (64, 4096, 4096), (512, 4096, 14336), (40, 512, 40), (33, 14336, 4096)]:
         split = (rows * k * 6 + rows * (k // 256) * 64 + 255) // 256 * 256
         got = kernels.workspaceBytes(Q4K, rows, k, n)
