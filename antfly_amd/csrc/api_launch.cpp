@@ -242,12 +242,17 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx,
                                                    ws.sx, ws.sums);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
+        // room behind the quantized activations for the partial sums of K shares (small grids): optional
+        const size_t partial_at = (ws.bytes + 255) / 256 * 256;
+        const size_t partial_bytes = gemm_i8_partial_bytes(rows, in_dim, out_dim);
+        float* partial = partial_bytes != 0 && workspace.len >= partial_at + partial_bytes
+                             ? reinterpret_cast<float*>(workspace.ptr + partial_at) : nullptr;
         e = launch_gemm_i8(stream, tensor_type, want_dots ? nullptr : y, dot_out, ws.qx, ws.sx, w, static_cast<int>(rows),
-                           static_cast<int>(in_dim), static_cast<int>(out_dim), ep);
-        if (e == hipSuccess && pair) {  // the second matrix reuses the quantized activations
+                           static_cast<int>(in_dim), static_cast<int>(out_dim), ep, partial);
+        if (e == hipSuccess && pair) {  // the second matrix reuses the quantized activations (and the partial sums' room)
             if (counters) counters->mm++;
             e = launch_gemm_i8(stream, tensor_type, y_b, nullptr, ws.qx, ws.sx, w_b, static_cast<int>(rows),
-                               static_cast<int>(in_dim), static_cast<int>(out_dim), ep_b);
+                               static_cast<int>(in_dim), static_cast<int>(out_dim), ep_b, partial);
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
@@ -518,7 +523,10 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
         return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
     }
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;
-    return workspace_view(0, rows, in_dim).bytes;
+    const size_t base = workspace_view(0, rows, in_dim).bytes;
+    // nine rows and more (the MFMA GEMM): room for the partial sums of K shares when the grid is small
+    const size_t partial = rows >= 9 ? gemm_i8_partial_bytes(rows, in_dim, out_dim) : 0;
+    return partial != 0 ? (base + 255) / 256 * 256 + partial : base;
 }
 
 afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,

@@ -128,7 +128,7 @@ template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots>
 __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
-    Epilogue ep) {
+    int share_blocks, float* __restrict__ partial, Epilogue ep) {
     using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
     constexpr int kWaves = S::kWaves, kSB = S::kStageBlocks, kRPL = S::kRowsPerLoad, kCPR = S::kChunksPerRow;
     constexpr int kTM = S::kTM, kTN = S::kTN, kRing = S::kRing;
@@ -143,7 +143,12 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     // each kind starts its round-robin over the wavefronts where the previous one stopped
     constexpr int kStartB = kUnitsA % kWaves, kStartSx = (kStartB + kUnitsB) % kWaves, kStartSw = (kStartSx + kUnitsSx) % kWaves;
 
-    const int kb = in_dim >> 5;
+    // K range of this workgroup: all of it, or (a small grid spread over more compute units)
+    // share blockIdx.y of share_blocks blocks, whose sums go to partial[share][rows][out_dim]
+    // for splitk_reduce_kernel.  kb_full is the row pitch, kb the blocks walked here.
+    const int kb_full = in_dim >> 5;
+    const int blk_begin = static_cast<int>(blockIdx.y) * share_blocks;
+    const int kb = min(share_blocks, kb_full - blk_begin);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -161,11 +166,11 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     if (n_tile >= n_tiles) return;
     const int m0 = m_tile * kTM, n0 = n_tile * kTN;
 
-    const size_t blocks = static_cast<size_t>(out_dim) * kb;
-    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(qx) + static_cast<size_t>(m0) * in_dim;
-    const uint8_t* b_base = weight + static_cast<size_t>(n0) * kb * kQuantBytes;
-    const uint8_t* sx_base = reinterpret_cast<const uint8_t*>(sx + static_cast<size_t>(m0) * kb);
-    const uint8_t* sw_base = weight + blocks * kQuantBytes + static_cast<size_t>(n0) * kb * 2;
+    const size_t blocks = static_cast<size_t>(out_dim) * kb_full;
+    const uint8_t* a_base = reinterpret_cast<const uint8_t*>(qx) + static_cast<size_t>(m0) * in_dim + static_cast<size_t>(blk_begin) * 32;
+    const uint8_t* b_base = weight + (static_cast<size_t>(n0) * kb_full + blk_begin) * kQuantBytes;
+    const uint8_t* sx_base = reinterpret_cast<const uint8_t*>(sx + static_cast<size_t>(m0) * kb_full + blk_begin);
+    const uint8_t* sw_base = weight + blocks * kQuantBytes + (static_cast<size_t>(n0) * kb_full + blk_begin) * 2;
 
     const int stages = (kb + kSB - 1) / kSB;
     const int last_blocks = kb - (stages - 1) * kSB;  // blocks in the last stage, 1..kSB
@@ -207,7 +212,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
         if (kQ4) {
             const int q = min((ub0 + i * kWaves) * 64 + lane, kTN * kSB - 1);
             const int r = q / kSB, blk = q % kSB;
-            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb) * 16u;
+            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb_full) * 16u;
             off_b[i][0] = rowoff + blk * 16;
             off_b[i][1] = rowoff + min(blk, last_blocks - 1) * 16;
             lds_b4[i][0] = S::chunk_pos(r, 2 * blk);
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
         } else {
             const int r = min((ub0 + i * kWaves) * kRPL + dma_r, kTN - 1);
             const int c = dma_slot ^ ((r / S::kRowsPerWrap) % kCPR);
-            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb) * 32u;
+            const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb_full) * 32u;
             off_b[i][0] = rowoff + c * 16;
             off_b[i][1] = rowoff + dma_chunk_last(c) * 16;
             lds_b4[i][0] = lds_b4[i][1] = 0;
@@ -225,7 +230,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     for (int i = 0; i < kPerSx; ++i) {
         const int q = min((usx0 + i * kWaves) * 64 + lane, kTM * kSB - 1);
         const int r = q / kSB, blk = q % kSB;
-        const uint32_t rowoff = static_cast<uint32_t>(min(m0 + r, rows - 1) - m0) * static_cast<uint32_t>(kb);
+        const uint32_t rowoff = static_cast<uint32_t>(min(m0 + r, rows - 1) - m0) * static_cast<uint32_t>(kb_full);
         off_sx[i][0] = (rowoff + blk) * 4;
         off_sx[i][1] = (rowoff + min(blk, last_blocks - 1)) * 4;
     }
@@ -233,7 +238,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     for (int i = 0; i < kPerSw; ++i) {
         const int q = min((usw0 + i * kWaves) * 64 + lane, kTN * kSB - 1);
         const int r = q / kSB, blk = q % kSB;
-        const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb);
+        const uint32_t rowoff = static_cast<uint32_t>(min(n0 + r, out_dim - 1) - n0) * static_cast<uint32_t>(kb_full);
         off_sw[i][0] = (rowoff + blk) * 2;
         off_sw[i][1] = (rowoff + min(blk, last_blocks - 1)) * 2;
     }
@@ -343,7 +348,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-                    if (m < rows && n < out_dim) dots[(static_cast<size_t>(m) * out_dim + n) * kb + blk + h] = c[v];
+                    if (m < rows && n < out_dim) dots[(static_cast<size_t>(m) * out_dim + n) * kb_full + blk_begin + blk + h] = c[v];
                 }
             }
 #pragma unroll
@@ -413,16 +418,22 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
 #pragma unroll
             for (int k2 = 1; k2 < kSplit; ++k2) sum += red[((k2 * S::kTiles + tile) * 16 + v) * 64 + lane];
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < rows && n < out_dim)
-                dst[static_cast<size_t>(m) * out_dim + n] = finish_output(ep, n, static_cast<size_t>(m) * out_dim + n, sum);
+            if (m < rows && n < out_dim) {
+                const size_t at = static_cast<size_t>(m) * out_dim + n;
+                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                else dst[at] = finish_output(ep, n, at, sum);
+            }
         }
     } else {
         if (dst == nullptr) return;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < rows && n < out_dim)
-                dst[static_cast<size_t>(m) * out_dim + n] = finish_output(ep, n, static_cast<size_t>(m) * out_dim + n, acc[v]);
+            if (m < rows && n < out_dim) {
+                const size_t at = static_cast<size_t>(m) * out_dim + n;
+                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = acc[v];
+                else dst[at] = finish_output(ep, n, at, acc[v]);
+            }
         }
     }
 }
@@ -431,7 +442,7 @@ namespace {
 
 template <int kType, int kWavesM, int kWavesN, int kSplit>
 hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
-                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep) {
+                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep, float* partial) {
     using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
     const int m_tiles = (rows + S::kTM - 1) / S::kTM;
     const int n_tiles = (out_dim + S::kTN - 1) / S::kTN;
@@ -440,7 +451,13 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
     // per-lane load offsets are 32-bit, relative to the workgroup's first row
     if (static_cast<long long>(S::kTM > S::kTN ? S::kTM : S::kTN) * in_dim > 0x7fffffffLL) return hipErrorInvalidValue;
-    dim3 g(static_cast<unsigned>(grid)), b(S::kThreads);
+    // K shares: only with room for their partial sums, never for the block-dot output
+    const int kb = in_dim / 32;
+    const int splits = partial != nullptr && dots == nullptr ? gemm_i8_splits(rows, in_dim, out_dim) : 1;
+    const int share_blocks = (kb + splits - 1) / splits;
+    const int shares = (kb + share_blocks - 1) / share_blocks;  // no empty share
+    float* sums = shares > 1 ? partial : nullptr;
+    dim3 g(static_cast<unsigned>(grid), static_cast<unsigned>(shares)), b(S::kThreads);
     auto kernel_f32 = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, false>;
     auto kernel_dots = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, true>;
     // more than 64 KB of LDS has to be asked for once per kernel
@@ -454,30 +471,70 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     if (attr != hipSuccess) return attr;
     if (dots)
         hipLaunchKernelGGL(kernel_dots, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
-                           m_tiles, n_tiles, ep);
+                           m_tiles, n_tiles, share_blocks, sums, ep);
     else
         hipLaunchKernelGGL(kernel_f32, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
-                           m_tiles, n_tiles, ep);
-    return hipGetLastError();
+                           m_tiles, n_tiles, share_blocks, sums, ep);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess || shares == 1) return e;
+    return launch_splitk_reduce(stream, dst, sums, static_cast<size_t>(rows) * out_dim, out_dim, shares, ep);
 }
 
 template <int kType>
 hipError_t launch_type(hipStream_t stream, float* dst, int* dots, const int8_t* qx, const float* sx,
-                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep) {
+                       const uint8_t* weight, int rows, int in_dim, int out_dim, const Epilogue& ep, float* partial) {
     // 64 x 128 tiles while they still give every CU a workgroup, 32 x 64 with a deeper K split otherwise
     const long long big = static_cast<long long>((rows + 63) / 64) * ((out_dim + 127) / 128);
     static const char* force = std::getenv("AFHIP_GEMM_TILE");  // tuning: "L" = 64x128, "S" = 32x64
     const bool use_big = force ? force[0] != 'S' : big >= 256;
-    if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep);
-    return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep);
+    if (use_big) return launch_tile<kType, 2, 4, 2>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep, partial);
+    return launch_tile<kType, 1, 2, 4>(stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim, ep, partial);
 }
 
 }  // namespace
 
+// K shares of a GEMM launch: one when its 32 x 64 tiles fill the compute units anyway, else as
+// many (a power of two, at most eight, at least 16 blocks = two stages each) as spread it over them.
+int gemm_i8_splits(int rows, int in_dim, int out_dim) {
+    const long workgroups = static_cast<long>((rows + 31) / 32) * ((out_dim + 63) / 64);
+    const int kb = in_dim / 32;
+    int units = 0, dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
+        units = 256;
+    int splits = 1;
+    while (splits < 8 && workgroups * splits * 2 <= units && kb / (splits * 2) >= 16) splits *= 2;
+    return splits;
+}
+
+size_t gemm_i8_partial_bytes(size_t rows, size_t in_dim, size_t out_dim) {
+    if (rows == 0 || rows > 0x7fffffff || in_dim > 0x7fffffff || out_dim > 0x7fffffff) return 0;
+    const int splits = gemm_i8_splits(static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim));
+    return splits > 1 ? static_cast<size_t>(splits) * rows * out_dim * 4 : 0;
+}
+
+// dst = epilogue(sum over the K shares, in order): second kernel of a split-K launch.
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(float* __restrict__ dst, const float* __restrict__ partial,
+                                                            size_t count, int out_dim, int splits, Epilogue ep) {
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count;
+         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        float total = 0.0f;
+        for (int z = 0; z < splits; ++z) total += partial[static_cast<size_t>(z) * count + i];
+        dst[i] = finish_output(ep, static_cast<int>(i % out_dim), i, total);
+    }
+}
+
+hipError_t launch_splitk_reduce(hipStream_t stream, float* dst, const float* partial, size_t count, int out_dim, int shares,
+                                const Epilogue& ep) {
+    size_t grid = (count + 255) / 256;
+    if (grid > 4096) grid = 4096;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst, partial, count, out_dim,
+                       shares, ep);
+    return hipGetLastError();
+}
+
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
-                          const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, const Epilogue& ep) {
-    if (tensor_type == 2) return launch_type<2>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep);
-    return launch_type<8>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep);
+                          const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, const Epilogue& ep, float* partial) {
+    if (tensor_type == 2) return launch_type<2>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep, partial);
+    return launch_type<8>(stream, dst, dots, qx, sx, weight_prepared, rows, in_dim, out_dim, ep, partial);
 }
 
 }  // namespace afhip

@@ -394,7 +394,7 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
                                                               float* __restrict__ partial, Epilogue ep) {
     const int kb = in_dim >> 8;
     // K range of this workgroup: all of it, or (a small problem spread over more compute units)
-    // share blockIdx.z, whose sums go to partial[z][rows][out_dim] for q4k_splitk_reduce_kernel
+    // share blockIdx.z, whose sums go to partial[z][rows][out_dim] for splitk_reduce_kernel
     const int sb_begin = blockIdx.z * sb_per_split;
     const int sb_end = min(kb, sb_begin + sb_per_split);
     const int tid = threadIdx.x, lane = tid & 63;
@@ -583,17 +583,6 @@ __global__ __launch_bounds__(512) void gemm_q4k_rows32_kernel(float* __restrict_
     }
 }
 
-// dst = epilogue(sum over the K shares, in order) for the split-K launches of the GEMM.
-__global__ __launch_bounds__(256) void q4k_splitk_reduce_kernel(float* __restrict__ dst, const float* __restrict__ partial,
-                                                                size_t count, int out_dim, int splits, Epilogue ep) {
-    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < count;
-         i += static_cast<size_t>(gridDim.x) * blockDim.x) {
-        float total = 0.0f;
-        for (int z = 0; z < splits; ++z) total += partial[static_cast<size_t>(z) * count + i];
-        dst[i] = finish_output(ep, static_cast<int>(i % out_dim), i, total);
-    }
-}
-
 size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
     return static_cast<size_t>(rows) * 3 * (static_cast<size_t>(in_dim) * 2 + kRowPadBytes) +
            static_cast<size_t>(rows) * (in_dim / 32) * 4 + static_cast<size_t>(waves) * groups * 64 * 4;
@@ -757,12 +746,7 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
     hipLaunchKernelGGL(gemm_q4k_rows32_kernel, dim3(grid_x, grid_y, shares), dim3(512), 2 * kG32ChunkBytes, stream, dst, parts,
                        xsum, weight, rows, in_dim, out_dim, sb_per_split, partial, ep);
     if (hipError_t e = hipGetLastError(); e != hipSuccess || shares == 1) return e;
-    const size_t count = static_cast<size_t>(rows) * out_dim;
-    size_t reduce_grid = (count + 255) / 256;
-    if (reduce_grid > 4096) reduce_grid = 4096;
-    hipLaunchKernelGGL(q4k_splitk_reduce_kernel, dim3(static_cast<unsigned>(reduce_grid)), dim3(256), 0, stream, dst, partial, count,
-                       out_dim, shares, ep);
-    return hipGetLastError();
+    return launch_splitk_reduce(stream, dst, partial, static_cast<size_t>(rows) * out_dim, out_dim, shares, ep);
 }
 
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,

@@ -55,9 +55,17 @@ hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned
 
 // Int8-MFMA GEMM on pre-quantized activations (natural order) and PREPARED
 // weights; dots optional (int32 [rows][out][in/32]), dst may be null when dots is set.
+// `partial` (optional, gemm_i8_partial_bytes() bytes): lets a launch whose tiles would leave
+// compute units idle share K out over more workgroups (gemm_i8_splits() shares, partial sums
+// added in share order by a second kernel).
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
                           const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
-                          const Epilogue& ep = Epilogue{});
+                          const Epilogue& ep = Epilogue{}, float* partial = nullptr);
+int gemm_i8_splits(int rows, int in_dim, int out_dim);
+size_t gemm_i8_partial_bytes(size_t rows, size_t in_dim, size_t out_dim);
+// dst[i] = epilogue(sum over s < shares of partial[s * count + i]), i < count = rows * out_dim
+hipError_t launch_splitk_reduce(hipStream_t stream, float* dst, const float* partial, size_t count, int out_dim, int shares,
+                                const Epilogue& ep);
 
 hipError_t launch_quantize_activations(hipStream_t stream, const float* x, int rows, int in_dim, int8_t* q,
                                        float* scale, int* sum);

@@ -182,7 +182,7 @@ def test_forced_dispatch_kinds_agree(fmt, rows):
 
 PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K slices, ragged columns, MFMA GEMM, f32 route
     (1, 4096, 1024), (2, 512, 514), (4, 2048, 640), (5, 8224, 513), (8, 4096, 512), (12, 256, 530), (40, 512, 640),
-    (3, 64, 100),
+    (3, 64, 100), (20, 2048, 300),  # the last: MFMA GEMM with K shared out over workgroups, both matrices through one scratch
 ]
 
 

@@ -126,3 +126,19 @@ def test_q4_k_prefill_workspace_sizes():
     assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 16 * 64
     # the smallest prefill on a small matrix spreads K over workgroups
     assert kernels.workspaceBytes(Q4K, 13, 4096, 4096) > 13 * 4096 * 6 + 13 * 16 * 64
+
+
+def test_int8_gemm_workspace_has_room_for_k_shares():
+    """Nine rows and more on a grid too small for the chip: behind the quantized activations the
+    scratch holds the partial sums of 2, 4 or 8 K shares (at least 16 blocks each); a grid that
+    fills the chip, or eight rows and fewer, asks for the quantized activations only."""
+    for fmt in (_lib.TYPE_Q4_0, _lib.TYPE_Q8_0):
+        base = lambda rows, k: kernels.workspaceBytes(fmt, rows, k, 1 << 20)  # a huge matrix never shares K out
+        for rows, k, n in [(16, 4096, 4096), (64, 14336, 4096), (9, 1024, 64)]:
+            extra = kernels.workspaceBytes(fmt, rows, k, n) - (base(rows, k) + 255) // 256 * 256
+            assert extra > 0 and extra % (rows * n * 4) == 0
+            shares = extra // (rows * n * 4)
+            assert shares in (2, 4, 8) and (k // 32) // shares >= 16
+        assert kernels.workspaceBytes(fmt, 8, 4096, 4096) == base(8, 4096)
+        assert kernels.workspaceBytes(fmt, 512, 4096, 4096) == base(512, 4096)
+        assert kernels.workspaceBytes(fmt, 16, 512, 4096) == base(16, 512)  # too short a K to share out
