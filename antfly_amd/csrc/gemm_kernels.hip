@@ -124,7 +124,9 @@ __device__ __forceinline__ void lds_load2(const void* base, uint32_t voff, uint3
 
 extern __shared__ __align__(16) unsigned char gemm_lds[];
 
-template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots>
+// kShareK: this launch walks only a share of K per workgroup (see below); a template parameter
+// so that the ordinary kernel carries none of it.
+template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots, bool kShareK = false>
 __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
@@ -147,8 +149,8 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     // share blockIdx.y of share_blocks blocks, whose sums go to partial[share][rows][out_dim]
     // for splitk_reduce_kernel.  kb_full is the row pitch, kb the blocks walked here.
     const int kb_full = in_dim >> 5;
-    const int blk_begin = static_cast<int>(blockIdx.y) * share_blocks;
-    const int kb = min(share_blocks, kb_full - blk_begin);
+    const int blk_begin = kShareK ? static_cast<int>(blockIdx.y) * share_blocks : 0;
+    const int kb = kShareK ? min(share_blocks, kb_full - blk_begin) : kb_full;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -420,7 +422,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
             if (m < rows && n < out_dim) {
                 const size_t at = static_cast<size_t>(m) * out_dim + n;
-                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                if (kShareK) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
                 else dst[at] = finish_output(ep, n, at, sum);
             }
         }
@@ -431,7 +433,7 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
             if (m < rows && n < out_dim) {
                 const size_t at = static_cast<size_t>(m) * out_dim + n;
-                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = acc[v];
+                if (kShareK) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = acc[v];
                 else dst[at] = finish_output(ep, n, at, acc[v]);
             }
         }
@@ -459,11 +461,15 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     float* sums = shares > 1 ? partial : nullptr;
     dim3 g(static_cast<unsigned>(grid), static_cast<unsigned>(shares)), b(S::kThreads);
     auto kernel_f32 = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, false>;
+    auto kernel_shares = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, false, true>;
     auto kernel_dots = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, true>;
     // more than 64 KB of LDS has to be asked for once per kernel
     static const hipError_t attr = [&]() {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_f32),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes);
+        if (e != hipSuccess) return e;
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_shares), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                S::kLdsBytes);
         if (e != hipSuccess) return e;
         return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_dots), hipFuncAttributeMaxDynamicSharedMemorySize,
                                    S::kLdsBytes);
@@ -471,6 +477,9 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     if (attr != hipSuccess) return attr;
     if (dots)
         hipLaunchKernelGGL(kernel_dots, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
+                           m_tiles, n_tiles, share_blocks, sums, ep);
+    else if (shares > 1)
+        hipLaunchKernelGGL(kernel_shares, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
                            m_tiles, n_tiles, share_blocks, sums, ep);
     else
         hipLaunchKernelGGL(kernel_f32, g, b, S::kLdsBytes, stream, dst, dots, qx, sx, weight, rows, in_dim, out_dim,
