@@ -1,6 +1,6 @@
 // C ABI, part 1: dispatch vocabulary (graph/quant_matmul.zig) and the
 // stream-ordered launchers (ops/cuda/kernels.zig:1221-1289).
-#include <hip/hip_runtime_api.h>
+#include <hip/hip_runtime.h>
 
 #include <algorithm>
 #include <cstdlib>
@@ -188,6 +188,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         if (!checked_mul(out_count, kb, &n) || !checked_mul(n, 4, &bytes) || bytes > dots.len) return AFHIP_ERR_INVALID_STATE;
     }
     if (!checked_mul(in_count, 4, &bytes) || bytes > input.len) return AFHIP_ERR_INVALID_STATE;
+    if (layout == AFHIP_LAYOUT_PREPARED) {  // quant bytes, scales, and the scales in tile order
+        w_bytes = afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim);
+        if (w_bytes == 0 && w_blocks != 0) return AFHIP_ERR_INVALID_STATE;
+    }
     if (w_bytes > weight.len) return AFHIP_ERR_INVALID_STATE;
     if (pair) {
         if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;
@@ -368,6 +372,9 @@ afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip
         if (!checked_mul(out_dim + 31, in_dim / block_values, &w_blocks) || !checked_mul(w_blocks, bb, &w_bytes))
             return AFHIP_ERR_INVALID_STATE;
         w_bytes = q4k_tiled_bytes(out_dim, in_dim);
+    } else if (!q4k && layout == AFHIP_LAYOUT_PREPARED) {
+        w_bytes = afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim);
+        if (w_bytes == 0) return AFHIP_ERR_INVALID_STATE;
     }
     if (w_bytes > weight.len) return AFHIP_ERR_INVALID_STATE;
     if (in_dim > 0x7fffffff || out_dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || weight.ptr == 0)
@@ -609,7 +616,10 @@ size_t afhip_prepared_weight_bytes(int tensor_type, size_t out_dim, size_t in_di
     }
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0 || in_dim % 32 != 0 || !checked_mul(out_dim, in_dim / 32, &blocks) || !checked_mul(blocks, bb, &bytes)) return 0;
-    return bytes;
+    // the scales once more in wavefront-tile order (padded to whole tiles): at most the raw size again
+    size_t padded;
+    if (!checked_mul(out_dim + 3, in_dim / 32 + kTileSliceBlocks, &padded) || !checked_mul(padded, 8, &padded)) return 0;
+    return prepared_bytes_q(tensor_type, out_dim, in_dim / 32);
 }
 
 size_t afhip_weight_layout_bytes(int tensor_type, int layout, size_t out_dim, size_t in_dim) {
@@ -647,12 +657,13 @@ afhip_status afhip_launch_prepare_weight(void* stream, int tensor_type, afhip_bu
     if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
     size_t blocks, bytes;
     if (!checked_mul(out_dim, in_dim / 32, &blocks) || !checked_mul(blocks, bb, &bytes)) return AFHIP_ERR_INVALID_STATE;
-    if (bytes > src.len || bytes > dst.len) return AFHIP_ERR_INVALID_STATE;
+    const size_t prepared = afhip_prepared_weight_bytes(tensor_type, out_dim, in_dim);
+    if (bytes > src.len || (blocks != 0 && prepared == 0) || prepared > dst.len) return AFHIP_ERR_INVALID_STATE;
     if (blocks == 0) return AFHIP_OK;
     if (dst.ptr == 0 || src.ptr == 0 || dst.ptr % 16 != 0 || src.ptr % 2 != 0) return AFHIP_ERR_INVALID_STATE;
     hipError_t e = launch_prepare_weight(static_cast<hipStream_t>(stream), tensor_type,
                                          reinterpret_cast<uint8_t*>(dst.ptr), reinterpret_cast<const uint8_t*>(src.ptr),
-                                         blocks);
+                                         out_dim, in_dim / 32);
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 

@@ -14,6 +14,20 @@ constexpr int kBlockValues = 32;  // weights per quant block (gguf/tensor_types.
 constexpr int kQ4BlockBytes = 18;
 constexpr int kQ8BlockBytes = 34;
 
+// ---- position (in halves) of the scale of block k of output column o in the wavefront-tile
+// copy of the scales (layout: qmatmul_launch.h); `slices` = ceil(blocks per row / 128).
+template <int kType>
+__host__ __device__ __forceinline__ size_t tile_scale_index(size_t o, size_t k, size_t slices) {
+    const size_t in_slice = k % kTileSliceBlocks;
+    if (kType == 2) {
+        const size_t tile = (o / 4) * slices + k / kTileSliceBlocks;
+        return (tile * 64 + in_slice % 64) * 8 + (in_slice / 64) * 4 + o % 4;
+    }
+    const size_t tile = (o / 2) * slices + k / kTileSliceBlocks;
+    const size_t step = in_slice / 32, lane = (in_slice % 32) * 2 + (step >> 1);
+    return (tile * 64 + lane) * 4 + (step & 1) * 2 + o % 2;
+}
+
 // ---- fp16 scale decode (gguf/quant_codec.zig:35-39).  v_cvt_f32_f16 is exact
 // for every half, subnormals included.
 __device__ __forceinline__ float half_bits_to_f32(uint16_t bits) {

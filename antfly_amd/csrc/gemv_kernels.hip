@@ -20,6 +20,11 @@
 //     weights in the order they were requested; the wavefront reduces with DPP;
 //     K-slices are combined through LDS in slice order.  The summation order is
 //     fixed, so results are run-to-run identical.
+//   * the fp16 scales of a lane's blocks are one more load of the same width: the PREPARED
+//     layout keeps a copy of the scales in wavefront-tile order (qmatmul_launch.h), so a
+//     wavefront issues nine 1 KiB loads instead of eight plus eight 128-byte ones.  The
+//     texture addresser takes a 64-lane load of any width in turn, and the requests of a
+//     compute unit's wavefronts all queue there at the start of the kernel.
 //   * a launch may serve two matrices of the same shape that share X (GemvTargets).
 #include <hip/hip_runtime.h>
 
@@ -31,6 +36,7 @@
 namespace afhip {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 template <int kType>
 struct GemvFormat;
@@ -39,14 +45,47 @@ struct GemvFormat<2> {  // Q4_0: lane = block, 16 B of nibbles
     static constexpr int kLanesPerBlock = 1;
     static constexpr int kQuantBytes = 16;
     static constexpr int kSteps = 2;
+    static constexpr int kCols = 4;
+    typedef u32x4 TileScales;  // steps 0..1 x columns 0..3
 };
 template <>
 struct GemvFormat<8> {  // Q8_0: lane = half block, 16 B of int8
     static constexpr int kLanesPerBlock = 2;
     static constexpr int kQuantBytes = 32;
     static constexpr int kSteps = 4;
+    static constexpr int kCols = 2;
+    typedef u32x2 TileScales;  // steps 2 * (lane & 1) + {0, 1} x columns 0..1; the other two steps are the neighbour lane's
 };
-constexpr int kSliceBlocks = 128;  // 4096 values
+constexpr int kSliceBlocks = kTileSliceBlocks;  // 4096 values
+static_assert(kSliceBlocks == 128, "a wavefront's K slice is one tile of the scale layout");
+
+// A lane's entry of the wavefront-tile copy of the scales, and the scale of (step j, column c)
+// out of it.  Q8_0: the two lanes of a block hold two steps each and exchange them.
+template <int kType>
+struct LaneScales;
+template <>
+struct LaneScales<2> {
+    u32x4 w;
+    __device__ __forceinline__ void exchange() {}
+    __device__ __forceinline__ float get(int j, int c, int) const {
+        const int i = j * 4 + c;
+        const uint32_t word = i / 2 == 0 ? w.x : (i / 2 == 1 ? w.y : (i / 2 == 2 ? w.z : w.w));
+        return half_bits_to_f32(static_cast<uint16_t>((i & 1) ? word >> 16 : word & 0xFFFFu));
+    }
+};
+template <>
+struct LaneScales<8> {
+    u32x2 w, other;
+    __device__ __forceinline__ void exchange() {
+        other.x = static_cast<uint32_t>(dpp_move<kDppXor1>(static_cast<int>(w.x)));
+        other.y = static_cast<uint32_t>(dpp_move<kDppXor1>(static_cast<int>(w.y)));
+    }
+    __device__ __forceinline__ float get(int j, int c, int half) const {
+        const u32x2 src = (j >> 1) == half ? w : other;
+        const uint32_t word = (j & 1) ? src.y : src.x;
+        return half_bits_to_f32(static_cast<uint16_t>(c ? word >> 16 : word & 0xFFFFu));
+    }
+};
 
 // LDS image of the quantized activations.
 //   Q4_0: two planes per row so that a lane's two 16-byte reads are unit-stride
@@ -132,8 +171,9 @@ constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ?
 template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices,
-    unsigned long long* __restrict__ keys = nullptr) {
+    int stagger, unsigned long long* __restrict__ keys = nullptr) {
     static_assert(!kArgmax || (kRows == 1 && !kWriteDots), "argmax keys: one row, no block dots");
+    static_assert(kCols == GemvFormat<kType>::kCols, "the scale tiles are laid out for this many columns per wavefront");
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
     constexpr int kBlocksPerStep = kWave / kLpb;
@@ -166,9 +206,13 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const uint8_t* weight = second ? tg.weight_b : tg.weight_a;
     float* dst = second ? tg.dst_b : tg.dst_a;
     const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
-    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
     const int o0 = group * kCols;
     const bool active = group < tg.groups_each && o0 < out_dim;
+    // this wavefront's tile of the scales (an idle wavefront re-reads the last group's)
+    typedef typename F::TileScales TileScales;
+    const TileScales* tile_scales =
+        reinterpret_cast<const TileScales*>(weight + ((blocks * (F::kQuantBytes + 2) + 15) & ~static_cast<size_t>(15))) +
+        (static_cast<size_t>(min(group, tg.groups_each - 1)) * slices + slice) * kWave;
 
     // ---- 1. requests: first the activations (wavefronts that quantize a block per
     // thread), then every weight byte this wavefront needs.  Loads complete in order, so
@@ -176,7 +220,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     // workgroup waits for at the barrier -- must not wait for the weights.
     const int x_blocks = kRows * kb;
     u32x4 wq[kSteps][kCols];
-    uint16_t wd[kSteps][kCols];
+    LaneScales<kType> wd;
     int blk[kSteps];
     bool ok[kSteps];
 #pragma unroll
@@ -185,19 +229,19 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         ok[j] = active && b < kb;
         blk[j] = b < kb ? b : kb - 1;  // lanes past the row end re-read its last block and contribute nothing
     }
-    // Request order = consumption order: column by column for one or two rows, K step by
-    // K step for more (the activations of a step are then in registers for all columns).
+    // Request order = consumption order: the scales, then column by column for one or two
+    // rows, K step by K step for more (the activations of a step are then in registers for
+    // all columns).
     constexpr bool kStepMajor = kRows > 2;
     auto request_weights = [&]() {
+        wd.w = __builtin_nontemporal_load(tile_scales + lane);
 #pragma unroll
         for (int u = 0; u < kCols * kSteps; ++u) {
             const int c = kStepMajor ? u % kCols : u / kSteps;
             const int j = kStepMajor ? u / kCols : u % kSteps;
             const int o = min(o0 + c, out_dim - 1);  // columns past the end re-read the last one
             const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
-            const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
             wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
-            wd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
         }
     };
     if (wave * kWave < x_blocks) {  // wave-uniform
@@ -230,9 +274,15 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             quantize_block_to_lds<kType, true>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
         }
     } else {
+        // The requests of a unit's wavefronts queue at its one texture addresser.  Left alone
+        // they interleave, every wavefront's last bytes arrive at the very end and all of them
+        // finish their arithmetic at once; entering the queue one after the other, a wavefront
+        // gets its bytes in a burst and only the last one still computes when the stream ends.
+        for (int q = 0; q < wave * stagger; ++q) __builtin_amdgcn_s_sleep(1);
         request_weights();
     }
     __syncthreads();
+    wd.exchange();
 
     // ---- 3. block dots and scaled accumulation (the weights stay packed in registers)
     static_assert(kRows <= 4, "the accumulators of all rows and columns live in registers");
@@ -288,7 +338,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         const int dot = block_dot(wq[j][c], a, sm);
         if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim)
             dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + blk[j]] = dot;
-        const float tscale = s * half_bits_to_f32(wd[j][c]);
+        const float tscale = s * wd.get(j, c, half);
         const float term = tscale * static_cast<float>(dot);
         acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
     };
@@ -425,9 +475,13 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
     const uint8_t* weight = second ? tg.weight_b : tg.weight_a;
     float* dst = second ? tg.dst_b : tg.dst_a;
     const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
-    const uint16_t* ds = reinterpret_cast<const uint16_t*>(weight + blocks * F::kQuantBytes);
     const int o0 = group * kCols;
     const bool active = group < tg.groups_each && o0 < out_dim;
+    static_assert(kCols == F::kCols, "the scale tiles are laid out for this many columns per wavefront");
+    typedef typename F::TileScales TileScales;
+    const TileScales* tile_scales =
+        reinterpret_cast<const TileScales*>(weight + ((blocks * (F::kQuantBytes + 2) + 15) & ~static_cast<size_t>(15))) +
+        (static_cast<size_t>(min(group, tg.groups_each - 1)) * slices + slice) * kWave;
 
     int wv[kSteps][kCols][kWords];
     float wd[kSteps][kCols];
@@ -441,18 +495,15 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
     }
     {
         u32x4 raw[kSteps][kCols];
-        uint16_t rawd[kSteps][kCols];
+        LaneScales<kType> rawd;
         auto request_weights = [&]() {
+            rawd.w = __builtin_nontemporal_load(tile_scales + lane);
 #pragma unroll
             for (int c = 0; c < kCols; ++c) {
                 const int o = min(o0 + c, out_dim - 1);
                 const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
-                const uint16_t* dcol = ds + static_cast<size_t>(o) * kb;
 #pragma unroll
-                for (int j = 0; j < kSteps; ++j) {
-                    raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
-                    rawd[j][c] = __builtin_nontemporal_load(dcol + blk[j]);
-                }
+                for (int j = 0; j < kSteps; ++j) raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
             }
         };
 
@@ -499,6 +550,7 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
         __syncthreads();
 
         // unpack once; lanes that own no block get a zero scale
+        rawd.exchange();
 #pragma unroll
         for (int j = 0; j < kSteps; ++j)
 #pragma unroll
@@ -512,7 +564,7 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
                 } else {
                     wv[j][c][0] = w.x; wv[j][c][1] = w.y; wv[j][c][2] = w.z; wv[j][c][3] = w.w;
                 }
-                wd[j][c] = (ok[j] && (kLpb == 1 || half == 0)) ? half_bits_to_f32(rawd[j][c]) : 0.0f;
+                wd[j][c] = (ok[j] && (kLpb == 1 || half == 0)) ? rawd.get(j, c, half) : 0.0f;
             }
     }
 
@@ -667,7 +719,9 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     if (key_count) *key_count = grid;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices, keys);
+    // one round of workgroups: the wavefronts of a unit enter its load queue one after the other
+    const int stagger = grid <= compute_units() ? 1 : 0;
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices, stagger, keys);
     return hipGetLastError();
 }
 

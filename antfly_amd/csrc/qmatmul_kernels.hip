@@ -101,10 +101,11 @@ __global__ __launch_bounds__(256) void quantize_activations_kernel(const float* 
     }
 }
 
-// RAW -> PREPARED repack, one thread per block.
+// RAW -> PREPARED repack, one thread per block: quant bytes, the scale in block order, and
+// the scale once more at its place in the wavefront-tile order (see qmatmul_launch.h).
 template <int kType>
 __global__ __launch_bounds__(256) void prepare_weight_kernel(uint8_t* __restrict__ dst, const uint8_t* __restrict__ src,
-                                                             size_t blocks) {
+                                                             size_t blocks, size_t kb) {
     constexpr int kQuantBytes = kType == 2 ? 16 : 32;
     constexpr int kRawBytes = kQuantBytes + 2;
     const size_t b = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
@@ -112,9 +113,17 @@ __global__ __launch_bounds__(256) void prepare_weight_kernel(uint8_t* __restrict
     const uint16_t* s = reinterpret_cast<const uint16_t*>(src + b * kRawBytes);
     uint16_t* dq = reinterpret_cast<uint16_t*>(dst + b * kQuantBytes);
     uint16_t* dd = reinterpret_cast<uint16_t*>(dst + blocks * kQuantBytes) + b;
+    uint16_t* dt = reinterpret_cast<uint16_t*>(dst + ((blocks * kRawBytes + 15) & ~static_cast<size_t>(15)));
     *dd = s[0];
+    const size_t o = b / kb, k = b - o * kb;
+    dt[tile_scale_index<kType>(o, k, (kb + kTileSliceBlocks - 1) / kTileSliceBlocks)] = s[0];
 #pragma unroll
     for (int j = 0; j < kQuantBytes / 2; ++j) dq[j] = s[1 + j];
+}
+
+__global__ __launch_bounds__(256) void zero_fill_kernel(uint4* __restrict__ dst, size_t n16) {
+    for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < n16; i += static_cast<size_t>(gridDim.x) * blockDim.x)
+        dst[i] = make_uint4(0, 0, 0, 0);
 }
 
 // get_rows / cpy_q_to_f32: dst[t][:] = dequantized row ids[t] of a [*, dim] weight
@@ -396,11 +405,23 @@ hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout
 }
 
 hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
-                                 size_t blocks) {
+                                 size_t out_dim, size_t kb) {
+    const size_t blocks = out_dim * kb;
     if (blocks == 0) return hipSuccess;
+    // tile entries of blocks / columns past the matrix stay zero (a fill kernel, not a memset:
+    // the call may sit in a captured graph)
+    // (from the 16-byte unit that holds the end of the block-order scales, so that the padding
+    // between the two copies is zero as well; the repack kernel, next on the stream, rewrites
+    // the scales in that unit)
+    const size_t fill_from = (blocks * ((tensor_type == 2 ? 16 : 32) + 2)) & ~static_cast<size_t>(15);
+    const size_t tile_n16 = (tile_scales_offset(tensor_type, blocks) + tile_scales_bytes(tensor_type, out_dim, kb) - fill_from) / 16;
+    size_t fill_grid = (tile_n16 + 255) / 256;
+    if (fill_grid > 4096) fill_grid = 4096;
+    hipLaunchKernelGGL(zero_fill_kernel, dim3(static_cast<unsigned>(fill_grid)), dim3(256), 0, stream,
+                       reinterpret_cast<uint4*>(dst + fill_from), tile_n16);
     const unsigned grid = static_cast<unsigned>((blocks + 255) / 256);
-    if (tensor_type == 2) hipLaunchKernelGGL(prepare_weight_kernel<2>, dim3(grid), dim3(256), 0, stream, dst, src, blocks);
-    else hipLaunchKernelGGL(prepare_weight_kernel<8>, dim3(grid), dim3(256), 0, stream, dst, src, blocks);
+    if (tensor_type == 2) hipLaunchKernelGGL(prepare_weight_kernel<2>, dim3(grid), dim3(256), 0, stream, dst, src, blocks, kb);
+    else hipLaunchKernelGGL(prepare_weight_kernel<8>, dim3(grid), dim3(256), 0, stream, dst, src, blocks, kb);
     return launch_status();
 }
 

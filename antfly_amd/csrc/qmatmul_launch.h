@@ -25,6 +25,30 @@ struct GemvTuning {
     bool exact = false;  // use `threads` as it is instead of balancing the grid over the compute units
 };
 
+// PREPARED layout of a Q4_0 / Q8_0 weight [out_dim][in_dim / 32 blocks]:
+//   [quant bytes of every block, block order: 16 B (Q4_0) / 32 B (Q8_0) each]
+//   [fp16 scales, block order]                      <- GEMM, row operators, generic kernels
+//   [pad to 16 bytes]
+//   [the same scales in wavefront-tile order]        <- GEMV: a lane's scales are one load
+// A tile belongs to one GEMV wavefront: kCols output columns (4 / 2) x one K slice of 128
+// blocks; lane l's entry holds the scales of exactly the blocks whose quant bytes lane l
+// fetches (Q4_0: 8 halves = steps 0..1 x columns 0..3 of block 64 * step + l; Q8_0: 4 halves =
+// steps 2 * (l & 1) + {0, 1} x columns 0..1 of block 32 * step + l / 2).  Entries of blocks or
+// columns past the matrix are zero.
+constexpr int kTileSliceBlocks = 128;
+inline int tile_cols(int tensor_type) { return tensor_type == 2 ? 4 : 2; }
+inline size_t tile_lane_bytes(int tensor_type) { return tensor_type == 2 ? 16 : 8; }
+inline size_t tile_scales_offset(int tensor_type, size_t blocks) {
+    return (blocks * ((tensor_type == 2 ? 16 : 32) + 2) + 15) & ~static_cast<size_t>(15);
+}
+inline size_t tile_scales_bytes(int tensor_type, size_t out_dim, size_t kb) {
+    const size_t cols = static_cast<size_t>(tile_cols(tensor_type));
+    return (out_dim + cols - 1) / cols * ((kb + kTileSliceBlocks - 1) / kTileSliceBlocks) * 64 * tile_lane_bytes(tensor_type);
+}
+inline size_t prepared_bytes_q(int tensor_type, size_t out_dim, size_t kb) {
+    return tile_scales_offset(tensor_type, out_dim * kb) + tile_scales_bytes(tensor_type, out_dim, kb);
+}
+
 size_t gemv_fused_lds_bytes(int rows, int in_dim);
 int gemv_fused_max_in_dim();
 
@@ -76,7 +100,7 @@ hipError_t launch_linear_generic(hipStream_t stream, int tensor_type, int layout
                                  int rows, int in_dim, int out_dim, const Epilogue& ep = Epilogue{});
 
 hipError_t launch_prepare_weight(hipStream_t stream, int tensor_type, uint8_t* dst, const uint8_t* src,
-                                 size_t blocks);
+                                 size_t out_dim, size_t kb);
 
 // get_rows / cpy_q_to_f32: dst f32 [rows][dim] = rows ids[t] (ids == nullptr: rows in order) of a
 // weight with weight_rows rows; tensor_type 0 = dense f32 table (ids required).

@@ -61,18 +61,26 @@ const char *afhip_status_string(afhip_status status);
 enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_0 = 8, AFHIP_TYPE_Q4_K = 12 };
 /* Q4_K (144-byte super-blocks of 256 weights) is computed on f32 activations against the
  * dequantized weights, as the engine does on the CPU (ops/native_compute.zig:31075-31144)
- * and in its CUDA backend (ops/cuda/cuda_compute.zig:708): no activation quantizer, no
- * block dots, no repack (the raw layout is used, 16-byte aligned; `layout` is ignored),
- * no workspace; in_dim must be a multiple of 256.  Served by the linear launchers and
- * ops, the pair op, the argmax ops, embedding lookup and cpy_q_to_f32. */
+ * and in its CUDA backend (ops/cuda/cuda_compute.zig:708): no activation quantizer and no
+ * block dots.  Both layouts are served: RAW (GGUF bytes, 16-byte aligned) by a vector-ALU
+ * kernel, PREPARED (tile-major, see afhip_prepared_weight_bytes) by the MFMA kernels; more
+ * rows than one decode launch holds use the caller's workspace
+ * (afhip_linear_workspace_bytes) for the prefill GEMM.  in_dim must be a multiple of 256.
+ * Served by the linear launchers and ops, the pair op, the bias / activation / residual
+ * epilogues, the argmax ops, embedding lookup, cpy_q_to_f32 and GGUF loading. */
 
 /* How a quantized weight sits in device memory.
  * RAW       GGUF bytes as uploaded: [out][in/32] blocks of 18 / 34 bytes.
- * PREPARED  device-side repack of the same bytes (same size): all quant bytes
- *           first, 16 / 32 bytes per block in block order, then all fp16 scales.
- *           16-byte aligned so one lane loads a block (Q4_0) or half a block
- *           (Q8_0) with a single 128-bit load.  The CPU backend prepares its
- *           layouts at load time in the same way (ops/native_compute.zig:8130-8204). */
+ * PREPARED  device-side repack of the same bytes: all quant bytes first, 16 / 32
+ *           bytes per block in block order, then all fp16 scales in block order,
+ *           then (16-byte aligned) the scales once more in the order the decode
+ *           GEMV's wavefronts consume them: one tile per (4 / 2 output columns, 128
+ *           blocks of K), 64 lane entries of 8 / 4 scales, zero where the matrix
+ *           ends.  One lane then loads a block (Q4_0) or half a block (Q8_0), and all
+ *           the scales it needs, with one 128-bit (64-bit) load each.
+ *           afhip_prepared_weight_bytes gives the size (raw size + the second copy
+ *           of the scales).  The CPU backend prepares its layouts at load time in
+ *           the same way (ops/native_compute.zig:8130-8204). */
 enum afhip_weight_layout { AFHIP_LAYOUT_RAW = 0, AFHIP_LAYOUT_PREPARED = 1 };
 
 /* A device allocation, ops/cuda/buffer.zig DeviceBuffer{ptr,len}. */
@@ -242,7 +250,9 @@ afhip_status afhip_launch_quantize_rows(void *stream, int tensor_type, afhip_buf
 /* Bytes of a [out_dim, in_dim] weight in a device layout (0: unknown type / layout, or in_dim
  * not whole blocks). */
 size_t afhip_weight_layout_bytes(int tensor_type, int layout, size_t out_dim, size_t in_dim);
-/* Bytes of the PREPARED layout of a [out_dim, in_dim] weight: the raw size for Q4_0 / Q8_0;
+/* Bytes of the PREPARED layout of a [out_dim, in_dim] weight: for Q4_0 / Q8_0 the raw size
+ * rounded up to 16 plus ceil(out_dim / c) * ceil(in_dim / 4096) * 64 * e bytes for the scales in
+ * wavefront-tile order (c = 4, e = 16 for Q4_0; c = 2, e = 8 for Q8_0);
  * for Q4_K the tile-major layout (32 output columns x one 256-value super-block per
  * 4608-byte tile, columns past out_dim zero-filled), i.e. the raw size of out_dim rounded up
  * to a multiple of 32.  0 for an unknown type or an in_dim that is not whole blocks. */
@@ -506,13 +516,13 @@ afhip_status afhip_gguf_metadata_at(const afhip_gguf *file, size_t index, afhip_
 afhip_status afhip_gguf_find_metadata(const afhip_gguf *file, const char *key, afhip_gguf_metadata *out);
 
 /* One tensor of the file becomes a resident weight under `key` (null: its own name):
- * Q4_0 / Q8_0 through insertWeightFromLoaded with shape = reversed GGUF dimensions
+ * Q4_0 / Q8_0 / Q4_K through insertWeightFromLoaded with shape = reversed GGUF dimensions
  * (normalizedShapeFromDims, models/tensor_store.zig:654-658), F32 through
  * insertWeightFromTensor; other types -> AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE. */
 afhip_status afhip_compute_insert_weight_from_gguf(afhip_compute *self, const afhip_gguf *file,
                                                    const char *tensor_name, const char *key,
                                                    int keep_raw_layout);
-/* Every F32 / Q4_0 / Q8_0 tensor of the file under its own name; tensors of other
+/* Every F32 / Q4_0 / Q8_0 / Q4_K tensor of the file under its own name; tensors of other
  * types are counted in *skipped (either counter may be null). */
 afhip_status afhip_compute_load_gguf(afhip_compute *self, const afhip_gguf *file, int keep_raw_layout,
                                      size_t *loaded, size_t *skipped);

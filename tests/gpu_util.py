@@ -28,10 +28,30 @@ def prepare(fmt: int, w_raw: np.ndarray, out_dim: int, in_dim: int) -> torch.Ten
     return prepared
 
 
-def numpy_prepare(fmt: int, w_raw: np.ndarray) -> np.ndarray:
-    bb = 18 if fmt == _lib.TYPE_Q4_0 else 34
-    blocks = np.asarray(w_raw, np.uint8).reshape(-1, bb)
-    return np.concatenate([blocks[:, 2:].reshape(-1), blocks[:, :2].reshape(-1)])
+def numpy_prepare(fmt: int, w_raw: np.ndarray, out_dim: int, in_dim: int) -> np.ndarray:
+    """The PREPARED layout of a Q4_0 / Q8_0 weight: quant bytes of every block, the fp16 scales in
+    block order, zero padding to 16 bytes, then the scales once more in wavefront-tile order (one
+    tile = the columns of one GEMV wavefront x 128 blocks; 64 lane entries of 8 / 4 halves; entries
+    of blocks or columns past the matrix are zero)."""
+    q4 = fmt == _lib.TYPE_Q4_0
+    bb = 18 if q4 else 34
+    kb = in_dim // 32
+    blocks = np.asarray(w_raw, np.uint8).reshape(out_dim * kb, bb)
+    scales = blocks[:, :2].copy().view(np.uint16).reshape(out_dim, kb)
+    cols, per_lane = (4, 8) if q4 else (2, 4)
+    groups, slices = (out_dim + cols - 1) // cols, (kb + 127) // 128
+    tiles = np.zeros((groups, slices, 64, per_lane), np.uint16)
+    o, k = np.meshgrid(np.arange(out_dim), np.arange(kb), indexing="ij")
+    ks = k % 128
+    if q4:
+        lane, inner = ks % 64, (ks // 64) * 4 + o % 4
+    else:
+        step = ks // 32
+        lane, inner = (ks % 32) * 2 + (step >> 1), (step & 1) * 2 + o % 2
+    tiles[o // cols, k // 128, lane, inner] = scales
+    head = np.concatenate([blocks[:, 2:].reshape(-1), blocks[:, :2].reshape(-1)])
+    pad = np.zeros((-head.size) % 16, np.uint8)
+    return np.concatenate([head, pad, tiles.reshape(-1).view(np.uint8)])
 
 
 def numpy_prepare_q4k(w_raw: np.ndarray, out_dim: int, in_dim: int) -> np.ndarray:
@@ -104,7 +124,23 @@ def block_dots(fmt, layout, x: np.ndarray, w_dev: torch.Tensor, rows, in_dim, ou
 
 
 def max_rel_err(got: np.ndarray, want: np.ndarray) -> float:
-    """Largest |got - want| relative to the largest |want| of the same output row."""
+    """Largest |got - want| relative to the largest |want| of the same output row.
+
+    The gate is normalised by the row maximum, not element by element: an output is a sum of
+    in_dim/32 signed terms, so an element near zero is the difference of large partial sums and
+    its own magnitude says nothing about the rounding error it carries."""
     scale = np.abs(want).max(axis=-1, keepdims=True)
     scale = np.where(scale == 0, 1.0, scale)
     return float((np.abs(got.astype(np.float64) - want) / scale).max())
+
+
+def elementwise_rel_err(got: np.ndarray, want: np.ndarray, floor: float = 1e-3) -> float:
+    """Largest |got - want| / |want| over the outputs whose |want| is above `floor` times the
+    largest |want| of their row (reported next to the row-normalised figure, for information)."""
+    want = np.asarray(want, np.float64)
+    scale = np.abs(want).max(axis=-1, keepdims=True)
+    keep = np.abs(want) > floor * np.where(scale == 0, 1.0, scale)
+    if not keep.any():
+        return 0.0
+    err = np.abs(got.astype(np.float64) - want)
+    return float((err[keep] / np.abs(want[keep])).max())

@@ -105,11 +105,13 @@ def test_activation_quantizer_bit_exact(rows, in_dim):
 
 
 @pytest.mark.parametrize("fmt", [Q8, Q4])
-def test_prepare_weight_is_a_pure_repack(fmt):
-    out_dim, in_dim = 37, 160
+@pytest.mark.parametrize("out_dim,in_dim", [(37, 160), (8, 4096), (5, 8224), (130, 32)])
+def test_prepare_weight_is_a_pure_repack(fmt, out_dim, in_dim):
     w = synth.weights(fmt, 7, out_dim, in_dim)
     got = G.prepare(fmt, w, out_dim, in_dim).cpu().numpy()
-    assert np.array_equal(got, G.numpy_prepare(fmt, w))
+    want = G.numpy_prepare(fmt, w, out_dim, in_dim)
+    assert got.size == want.size == kernels.preparedWeightBytes(fmt, out_dim, in_dim)
+    assert np.array_equal(got, want)
 
 
 SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
@@ -209,11 +211,16 @@ def test_pair_equals_two_single_ops(fmt, layout, rows, in_dim, out_dim):
 
 FULL = [
     ("C1", Q8, [1], 4096, 4096),
-    ("C4", Q8, [128, 512], 4096, 4096),
+    ("C4", Q8, [128, 512, 2048], 4096, 4096),
     ("C4-q4", Q4, [128], 4096, 4096),
     ("C2", Q4, [1, 2, 4, 8], 4096, 14336),
     ("C3", Q4, [1, 5], 14336, 4096),
+    ("C5-qkv", Q4, [1, 5], 4096, 6144),   # the decode-step sweep: attention projections at one and five rows
+    ("C5-o", Q4, [1, 5], 4096, 4096),
 ]
+# element-wise relative error over outputs above 1e-3 of their row maximum (information; the gate
+# is the row-normalised figure): collected here and printed by the last full-size case
+ELEMENTWISE = {}
 
 
 @pytest.mark.parametrize("name,fmt,row_list,in_dim,out_dim", FULL)
@@ -228,6 +235,9 @@ def test_full_size_decode_configs(name, fmt, row_list, in_dim, out_dim):
         ref = prepared.linear(x, rows, workers=8)
         err = G.max_rel_err(y, ref.astype(np.float64))
         assert err <= TOL and err <= TIGHT, err
+        ELEMENTWISE[(name, rows)] = G.elementwise_rel_err(y, ref.astype(np.float64))
+        print(f"  row-normalised max-rel {err:.2e}, element-wise (|want| > 1e-3 row max) {ELEMENTWISE[(name, rows)]:.2e}", flush=True)
+        assert ELEMENTWISE[(name, rows)] <= 100 * TOL  # cancellation near zero amplifies by at most 1/floor
         # block dots on a slice of output columns and rows (the full tensor is rows x out x in/32 ints)
         sub, rsub = 64, min(rows, 40)
         wsub = w[: sub * (in_dim // 32) * O.BLOCK_BYTES[fmt]]
@@ -240,3 +250,24 @@ def test_full_size_decode_configs(name, fmt, row_list, in_dim, out_dim):
         y2 = G.linear(fmt, PREP, x * 2.0, wd, rows, in_dim, out_dim)
         assert np.array_equal(y2, y * 2.0)
     prepared.close()
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+def test_full_size_gate_up_pair(rows):
+    """The decode step's gate + up projections as the one pair call the engine makes
+    (architectures/gpt.zig:5398-5440): each half bit-identical to the single op on that
+    matrix, one half against the oracle."""
+    in_dim, out_dim = 4096, 14336
+    print(f"case: C5 pair rows={rows} in={in_dim} out={out_dim}", flush=True)
+    x = synth.activations(8800 + rows, rows, in_dim)
+    wa = synth.weights(Q4, 8801, out_dim, in_dim)
+    wb = synth.weights(Q4, 8802, out_dim, in_dim)
+    da, db = G.prepare(Q4, wa, out_dim, in_dim), G.prepare(Q4, wb, out_dim, in_dim)
+    ya, yb = G.linear_pair(Q4, PREP, x, da, db, rows, in_dim, out_dim)
+    assert np.array_equal(ya, G.linear(Q4, PREP, x, da, rows, in_dim, out_dim))
+    assert np.array_equal(yb, G.linear(Q4, PREP, x, db, rows, in_dim, out_dim))
+    prepared = O.Prepared(Q4, wb, out_dim, in_dim)
+    ref = prepared.linear(x, rows, workers=8)
+    prepared.close()
+    err = G.max_rel_err(yb, ref.astype(np.float64))
+    assert err <= TOL and err <= TIGHT, err
