@@ -166,10 +166,11 @@ __device__ __forceinline__ unsigned long long row_max_key(unsigned long long key
 // Largest key of the workgroup (at most 16 wavefronts), valid on thread 0.  `slots` = one
 // LDS word per wavefront.  kLiveLanes: only lanes [0, kLiveLanes) of a wavefront hold
 // candidates (at most 16: one row).
+// `tid` / `wavefronts`: the thread's flat index in the workgroup and the workgroup's size.
 template <int kLiveLanes = 64>
-__device__ __forceinline__ unsigned long long workgroup_max_key(unsigned long long key, unsigned long long* slots) {
+__device__ __forceinline__ unsigned long long workgroup_max_key(unsigned long long key, unsigned long long* slots, int tid,
+                                                                int wavefronts) {
     key = row_max_key(key);
-    const int tid = threadIdx.x;
     const int lane = tid & 63;
     if (kLiveLanes > 16) {  // the four rows of the wavefront
         const unsigned long long r1 = __shfl(key, 16), r2 = __shfl(key, 32), r3 = __shfl(key, 48);
@@ -180,10 +181,15 @@ __device__ __forceinline__ unsigned long long workgroup_max_key(unsigned long lo
     if (lane == 0) slots[tid >> 6] = key;
     __syncthreads();
     if (tid < 16) {  // one row of the first wavefront: a slot per lane
-        key = tid < static_cast<int>(blockDim.x >> 6) ? slots[tid] : 0ull;
+        key = tid < wavefronts ? slots[tid] : 0ull;
         key = row_max_key(key);
     }
     return key;
+}
+// one-dimensional workgroups
+template <int kLiveLanes = 64>
+__device__ __forceinline__ unsigned long long workgroup_max_key(unsigned long long key, unsigned long long* slots) {
+    return workgroup_max_key<kLiveLanes>(key, slots, static_cast<int>(threadIdx.x), static_cast<int>(blockDim.x >> 6));
 }
 
 // ---- activation quantizer for one value, given its block's max |x|

@@ -168,10 +168,39 @@ constexpr int pow2_at_least(int n) { return n <= 1 ? 1 : (n <= 2 ? 2 : (n <= 4 ?
 // One to four rows of f32 activations, quantized in the prologue of every workgroup.
 // kArgmax (one row, one matrix): no Y is written; the workgroup leaves the argmax key of
 // its output columns in keys[blockIdx.x] instead.
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false>
+// Arguments of the fused GEMV that only some calls use; they follow the sixteen preloaded
+// dwords in the kernel-argument segment and are loaded from memory on the paths that need
+// them (block dots, argmax keys, a bias / activation / residual epilogue), never on the plain
+// Y = X * W^T path.
+struct GemvExtras {
+    int* dots;
+    unsigned long long* keys;
+    Epilogue ep_a;  // bias / activation / residual of each matrix (linear, linearPair ...,
+    Epilogue ep_b;  // ops/ops.zig:1728, :915)
+};
+constexpr uint32_t kGemvHasEpilogueA = 1u << 24, kGemvHasEpilogueB = 1u << 25;
+
+// Launch shape: blockDim = (64 * slices, groups_per_wg): threadIdx.x / 64 is the K slice,
+// threadIdx.y the column group inside the workgroup (no division in the kernel).  The
+// leading arguments are everything the plain product needs, and fit the sixteen dwords
+// that reach a wavefront in registers at launch (kernel-argument preload): no wavefront
+// waits for a kernel-argument load from memory before its first request, or at all.  A
+// kernel of this size is as long as its longest wavefront, and each of those starts with
+// these instructions.
+//   tile_off16: where the scales in tile order start inside a weight, in 16-byte units
+//   shape:      slices | groups_per_wg << 8 | stagger << 16 | kGemvHasEpilogue*
+//   kCompact:   one K slice (in_dim <= 4096), one matrix, at most one block of X per thread:
+//               the instantiation carries none of the code of the other cases (the
+//               instruction stream a wavefront walks is half as long)
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
-    GemvTargets tg, int* __restrict__ dots, const float* __restrict__ input, int in_dim, int out_dim, int slices,
-    int stagger, unsigned long long* __restrict__ keys = nullptr) {
+    const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
+    float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
+    GemvExtras extras) {
+    const int slices = kCompact ? 1 : static_cast<int>(shape & 0xFF);
+    const int groups_per_wg = (shape >> 8) & 0xFF, stagger = (shape >> 16) & 0xFF;
+    const int groups_each = (out_dim + kCols - 1) / kCols;
+    const size_t tile_off = static_cast<size_t>(tile_off16) << 4;
     static_assert(!kArgmax || (kRows == 1 && !kWriteDots), "argmax keys: one row, no block dots");
     static_assert(kCols == GemvFormat<kType>::kCols, "the scale tiles are laid out for this many columns per wavefront");
     using F = GemvFormat<kType>;
@@ -180,39 +209,36 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     constexpr int kSteps = F::kSteps;
 
     extern __shared__ __align__(16) unsigned char lds[];
-    const int kb = in_dim >> 5;
-    const int row_dwords = in_dim >> 2;
+    const int in_dim = kb << 5;
+    const int row_dwords = kb << 3;
     int* qx = reinterpret_cast<int*>(lds);                                           // [kRows][in_dim] bytes
     float* sx = reinterpret_cast<float*>(lds + static_cast<size_t>(kRows) * in_dim);  // [kRows][kb]
     int* sumx = reinterpret_cast<int*>(sx + kRows * kb);                              // [kRows][kb]
     float* partial = reinterpret_cast<float*>(sumx + kRows * kb);                     // [waves][kRows*kCols]
 
-    const size_t blocks = static_cast<size_t>(out_dim) * kb;
-
-    const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
+    const int lane = threadIdx.x & (kWave - 1);
     // wavefront-uniform values live in scalar registers, so column base addresses
     // are scalar and each load is "scalar base + one 32-bit lane offset"
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int waves = blockDim.x >> 6;
+    const int slice = kCompact ? 0 : __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int group_in_wg = __builtin_amdgcn_readfirstlane(threadIdx.y);
+    const int wave = group_in_wg * slices + slice;  // flat wavefront index
+    const int tid = wave * kWave + lane;
+    const int waves = slices * groups_per_wg;
+    const int threads = waves * kWave;
     const int half = lane & (kLpb - 1);
     const int lane_block = lane / kLpb;
-    const int slice = wave % slices;
-    const int groups_per_wg = waves / slices;
     // column group -> matrix (wave-uniform), columns o0 .. o0 + kCols - 1 of it
-    const int group_all = blockIdx.x * groups_per_wg + wave / slices;
-    const bool second = tg.weight_b != nullptr && group_all >= tg.groups_each;
-    const int group = second ? group_all - tg.groups_each : group_all;
-    const uint8_t* weight = second ? tg.weight_b : tg.weight_a;
-    float* dst = second ? tg.dst_b : tg.dst_a;
+    const int group_all = blockIdx.x * groups_per_wg + group_in_wg;
+    const bool second = !kCompact && weight_b != nullptr && group_all >= groups_each;
+    const int group = second ? group_all - groups_each : group_all;
+    const uint8_t* weight = second ? weight_b : weight_a;
     const u32x4* qs = reinterpret_cast<const u32x4*>(weight);
     const int o0 = group * kCols;
-    const bool active = group < tg.groups_each && o0 < out_dim;
+    const bool active = group < groups_each && o0 < out_dim;
     // this wavefront's tile of the scales (an idle wavefront re-reads the last group's)
     typedef typename F::TileScales TileScales;
-    const TileScales* tile_scales =
-        reinterpret_cast<const TileScales*>(weight + ((blocks * (F::kQuantBytes + 2) + 15) & ~static_cast<size_t>(15))) +
-        (static_cast<size_t>(min(group, tg.groups_each - 1)) * slices + slice) * kWave;
+    const TileScales* tile_scales = reinterpret_cast<const TileScales*>(weight + tile_off) +
+                                    (static_cast<size_t>(min(group, groups_each - 1)) * slices + slice) * kWave;
 
     // ---- 1. requests: first the activations (wavefronts that quantize a block per
     // thread), then every weight byte this wavefront needs.  Loads complete in order, so
@@ -223,11 +249,13 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     LaneScales<kType> wd;
     int blk[kSteps];
     bool ok[kSteps];
+    uint32_t lane_off[kSteps];  // byte offset of this lane's 16 bytes inside a column's quant bytes
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
         const int b = slice * kSliceBlocks + j * kBlocksPerStep + lane_block;
         ok[j] = active && b < kb;
         blk[j] = b < kb ? b : kb - 1;  // lanes past the row end re-read its last block and contribute nothing
+        lane_off[j] = static_cast<uint32_t>(blk[j] * kLpb + half) * 16u;
     }
     // Request order = consumption order: the scales, then column by column for one or two
     // rows, K step by K step for more (the activations of a step are then in registers for
@@ -240,14 +268,15 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             const int c = kStepMajor ? u % kCols : u / kSteps;
             const int j = kStepMajor ? u / kCols : u % kSteps;
             const int o = min(o0 + c, out_dim - 1);  // columns past the end re-read the last one
-            const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
-            wq[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+            // scalar column base + unsigned 32-bit lane offset: the load takes its address as
+            // "SGPR pair + VGPR offset", no 64-bit vector arithmetic between the requests
+            const uint8_t* qcol = reinterpret_cast<const uint8_t*>(qs + static_cast<size_t>(o) * kb * kLpb);
+            wq[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qcol + lane_off[j]));
         }
     };
     if (wave * kWave < x_blocks) {  // wave-uniform
-        const int threads = static_cast<int>(blockDim.x);
         const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
-        const bool two = x_blocks > threads;                 // uniform: a second block per thread
+        const bool two = !kCompact && x_blocks > threads;    // uniform: a second block per thread
         const int xb1 = min(tid + threads, x_blocks - 1);
         float4 v[8], v1[8];
 #pragma unroll
@@ -267,7 +296,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         }
         // more than two blocks per thread (not a shape the host sends here): these requests
         // queue behind the weights
-        for (int xb2 = tid + 2 * threads; xb2 < x_blocks; xb2 += threads) {
+        for (int xb2 = tid + 2 * threads; !kCompact && xb2 < x_blocks; xb2 += threads) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb2 * 8 + i];
             const int r2 = xb2 / kb, b2 = xb2 - r2 * kb;
@@ -337,7 +366,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     auto accumulate = [&](int j, int c, int r, const int (&a)[kWords], float s, int sm) {
         const int dot = block_dot(wq[j][c], a, sm);
         if (kWriteDots && ok[j] && half == 0 && o0 + c < out_dim)
-            dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + blk[j]] = dot;
+            extras.dots[(static_cast<size_t>(r) * out_dim + o0 + c) * kb + blk[j]] = dot;
         const float tscale = s * wd.get(j, c, half);
         const float term = tscale * static_cast<float>(dot);
         acc[r][c] += (kLpb == 1 || half == 0) ? term : 0.0f;
@@ -390,13 +419,18 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             // (`partial` is free here: one word per wavefront)
             const bool live = active && mine && o0 + cc < out_dim;
             const unsigned long long key = workgroup_max_key<kPadded>(
-                live ? argmax_key(red[0], static_cast<uint32_t>(o0 + cc)) : 0ull, reinterpret_cast<unsigned long long*>(partial));
-            if (tid == 0) keys[blockIdx.x] = key;
+                live ? argmax_key(red[0], static_cast<uint32_t>(o0 + cc)) : 0ull, reinterpret_cast<unsigned long long*>(partial), tid,
+                waves);
+            if (tid == 0) extras.keys[blockIdx.x] = key;
             return;
         }
-        if (active && mine && o0 + cc < out_dim && dst)
-            dst[static_cast<size_t>(cr) * out_dim + o0 + cc] =
-                finish_output(second ? tg.ep_b : tg.ep_a, o0 + cc, static_cast<size_t>(cr) * out_dim + o0 + cc, red[0]);
+        float* dst = second ? dst_b : dst_a;
+        if (active && mine && o0 + cc < out_dim && dst) {
+            const size_t at = static_cast<size_t>(cr) * out_dim + o0 + cc;
+            float v = red[0];
+            if (shape & (second ? kGemvHasEpilogueB : kGemvHasEpilogueA)) v = finish_output(second ? extras.ep_b : extras.ep_a, o0 + cc, at, v);
+            dst[at] = v;
+        }
         return;
     }
     if (mine) partial[wave * kCells + cell] = red[0];
@@ -404,30 +438,31 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     __syncthreads();
     const int cells = groups_per_wg * kCells;
     unsigned long long key = 0;
-    for (int i = tid; i < cells; i += blockDim.x) {
+    for (int i = tid; i < cells; i += threads) {
         const int gi = i / kCells, rc = i - gi * kCells;
         const int r = rc / kCols, c = rc - r * kCols;
         const int ga = blockIdx.x * groups_per_wg + gi;
-        const bool sec = tg.weight_b != nullptr && ga >= tg.groups_each;
-        const int g = sec ? ga - tg.groups_each : ga;
-        float* d = sec ? tg.dst_b : tg.dst_a;
+        const bool sec = !kCompact && weight_b != nullptr && ga >= groups_each;
+        const int g = sec ? ga - groups_each : ga;
+        float* d = sec ? dst_b : dst_a;
         const int o = g * kCols + c;
         float total = 0.0f;
         for (int sl = 0; sl < slices; ++sl) total += partial[(gi * slices + sl) * kCells + rc];
         if (kArgmax) {
-            if (g < tg.groups_each && o < out_dim) {
+            if (g < groups_each && o < out_dim) {
                 const unsigned long long k = argmax_key(total, static_cast<uint32_t>(o));
                 if (k > key) key = k;
             }
-        } else if (g < tg.groups_each && o < out_dim && d) {
-            d[static_cast<size_t>(r) * out_dim + o] =
-                finish_output(sec ? tg.ep_b : tg.ep_a, o, static_cast<size_t>(r) * out_dim + o, total);
+        } else if (g < groups_each && o < out_dim && d) {
+            if (shape & (sec ? kGemvHasEpilogueB : kGemvHasEpilogueA))
+                total = finish_output(sec ? extras.ep_b : extras.ep_a, o, static_cast<size_t>(r) * out_dim + o, total);
+            d[static_cast<size_t>(r) * out_dim + o] = total;
         }
     }
     if (kArgmax) {
         __syncthreads();  // every total has been read: the partial sums' memory becomes the key slots
-        key = workgroup_max_key(key, reinterpret_cast<unsigned long long*>(partial));
-        if (tid == 0) keys[blockIdx.x] = key;
+        key = workgroup_max_key(key, reinterpret_cast<unsigned long long*>(partial), tid, waves);
+        if (tid == 0) extras.keys[blockIdx.x] = key;
     }
 }
 
@@ -487,11 +522,13 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
     float wd[kSteps][kCols];
     int blk[kSteps];
     bool ok[kSteps];
+    uint32_t lane_off[kSteps];
 #pragma unroll
     for (int j = 0; j < kSteps; ++j) {
         const int b = slice * kSliceBlocks + j * kBlocksPerStep + lane_block;
         ok[j] = active && b < kb;
         blk[j] = b < kb ? b : kb - 1;
+        lane_off[j] = static_cast<uint32_t>(blk[j] * kLpb + half) * 16u;
     }
     {
         u32x4 raw[kSteps][kCols];
@@ -501,9 +538,10 @@ __global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* 
 #pragma unroll
             for (int c = 0; c < kCols; ++c) {
                 const int o = min(o0 + c, out_dim - 1);
-                const u32x4* qcol = qs + static_cast<size_t>(o) * kb * kLpb;
+                const uint8_t* qcol = reinterpret_cast<const uint8_t*>(qs + static_cast<size_t>(o) * kb * kLpb);
 #pragma unroll
-                for (int j = 0; j < kSteps; ++j) raw[j][c] = __builtin_nontemporal_load(qcol + blk[j] * kLpb + half);
+                for (int j = 0; j < kSteps; ++j)
+                    raw[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qcol + lane_off[j]));
             }
         };
 
@@ -714,14 +752,24 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
         waves = workgroup_waves(512, 512, slices, groups, true);  // many rounds: nothing to balance
     const int groups_per_wg = waves / slices;
     const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
-    auto kernel = gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax>;
-    static std::atomic<size_t> lds_limit{64 * 1024};
-    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
+    const bool compact = slices == 1 && tg.weight_b == nullptr && x_blocks <= waves * 64;
+    auto kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true>
+                          : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false>;
+    static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
+    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[compact ? 1 : 0]); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     if (key_count) *key_count = grid;
     // one round of workgroups: the wavefronts of a unit enter its load queue one after the other
     const int stagger = grid <= compute_units() ? 1 : 0;
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, tg, dots, input, in_dim, out_dim, slices, stagger, keys);
+    const GemvExtras extras{dots, keys, tg.ep_a, tg.ep_b};
+    auto has_epilogue = [](const Epilogue& e) { return e.bias != nullptr || e.residual != nullptr || e.activation != kActNone; };
+    const size_t tile_off = tile_scales_offset(kType, static_cast<size_t>(out_dim) * (in_dim / 32));
+    if ((tile_off >> 4) > 0xFFFFFFFFull || slices > 255 || groups_per_wg > 255) return hipErrorInvalidValue;
+    const uint32_t shape = static_cast<uint32_t>(slices) | static_cast<uint32_t>(groups_per_wg) << 8 |
+                           static_cast<uint32_t>(stagger) << 16 | (has_epilogue(tg.ep_a) ? kGemvHasEpilogueA : 0u) |
+                           (has_epilogue(tg.ep_b) ? kGemvHasEpilogueB : 0u);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * slices, groups_per_wg), lds, stream, tg.weight_a, tg.weight_b, input, tg.dst_a,
+                       tg.dst_b, static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);
     return hipGetLastError();
 }
 
