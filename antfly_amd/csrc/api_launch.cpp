@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <atomic>
 #include <cstdlib>
 #include <limits>
 
@@ -10,7 +11,34 @@
 #include "api_internal.h"
 #include "qmatmul_launch.h"
 
+// Scratch of afhip_launch_linear_f32_static: one copy per GPU, at its own address on each.
+// In host code the name below is only a handle for hipGetSymbolAddress; kernels and copies
+// get the address that call returned.
+static __device__ __align__(256) unsigned char scratch[AFHIP_STATIC_SCRATCH_BYTES];
+
 namespace afhip {
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<unsigned char*> g_static_scratch[kMaxDevices];
+
+// The array's address on the current device, resolved once per device.
+afhip_status static_scratch_address(unsigned char** out) {
+    int dev = -1;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return static_cast<afhip_status>(e);
+    if (dev < 0 || dev >= kMaxDevices) return AFHIP_ERR_INVALID_STATE;
+    unsigned char* p = g_static_scratch[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        void* addr = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)); e != hipSuccess) return static_cast<afhip_status>(e);
+        if (addr == nullptr) return AFHIP_ERR_INVALID_STATE;
+        p = static_cast<unsigned char*>(addr);
+        g_static_scratch[dev].store(p, std::memory_order_release);  // (two threads may both resolve it: same value)
+    }
+    *out = p;
+    return AFHIP_OK;
+}
+}  // namespace
 
 bool checked_mul(size_t a, size_t b, size_t* out) { return !__builtin_mul_overflow(a, b, out); }
 
@@ -539,6 +567,23 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
 afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim,
                                      afhip_buffer workspace, int dispatch) {
+    return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
+                       afhip_buffer{0, 0}, nullptr);
+}
+
+afhip_status afhip_static_scratch_init(void) {
+    unsigned char* p = nullptr;
+    return static_scratch_address(&p);
+}
+
+afhip_status afhip_launch_linear_f32_static(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                                            afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, int dispatch) {
+    // what the call would ask a caller to lend: beyond the array is refused, not truncated
+    if (afhip_linear_workspace_bytes(tensor_type, rows, in_dim, out_dim) > AFHIP_STATIC_SCRATCH_BYTES)
+        return AFHIP_ERR_OP_UNSUPPORTED;
+    unsigned char* p = nullptr;
+    if (afhip_status s = static_scratch_address(&p); s != AFHIP_OK) return s;
+    const afhip_buffer workspace{reinterpret_cast<uint64_t>(p), AFHIP_STATIC_SCRATCH_BYTES};
     return linear_impl(stream, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace, dispatch,
                        afhip_buffer{0, 0}, nullptr);
 }

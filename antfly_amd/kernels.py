@@ -19,6 +19,21 @@ def launchLinearF32(stream, tensor_type, layout, dst: Buffer, input: Buffer, wei
                                              workspace, dispatch))
 
 
+STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def staticScratchInit() -> None:
+    check(_lib.lib().afhip_static_scratch_init())
+
+
+def launchLinearF32Static(stream, tensor_type, layout, dst: Buffer, input: Buffer, weight: Buffer, rows, in_dim, out_dim,
+                          dispatch: int = -1) -> None:
+    """launchLinearF32 without a workspace argument and without any allocation: the scratch is
+    a device array inside the library (one per GPU, shared by all calls on it)."""
+    check(_lib.lib().afhip_launch_linear_f32_static(stream, tensor_type, layout, dst, input, weight, rows, in_dim,
+                                                    out_dim, dispatch))
+
+
 def launchLinearPairF32(stream, tensor_type, layout, dst_a: Buffer, dst_b: Buffer, input: Buffer, weight_a: Buffer,
                         weight_b: Buffer, rows, in_dim, out_dim, workspace: Buffer = NO_BUFFER,
                         dispatch: int = -1) -> None:

@@ -146,6 +146,22 @@ afhip_status afhip_launch_linear_f32(void *stream, int tensor_type, int layout, 
                                      afhip_buffer input, afhip_buffer weight, size_t rows,
                                      size_t in_dim, size_t out_dim, afhip_buffer workspace,
                                      int dispatch);
+/* afhip_launch_linear_f32 for callers that cannot allocate device memory and have no
+ * workspace to lend (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments minus `workspace`, same
+ * results bit for bit: the scratch (quantized activations, partial sums of K shares) is a
+ * file-scope device array of AFHIP_STATIC_SCRATCH_BYTES that every GPU the library runs on
+ * holds until the process ends.  The call allocates and frees nothing.  A shape whose
+ * afhip_linear_workspace_bytes() exceeds the array is refused with
+ * AFHIP_ERR_OP_UNSUPPORTED.  All calls on one GPU share the array: calls that may overlap
+ * (different streams, different host threads) race; order them on one stream.
+ * afhip_static_scratch_init() resolves the array's address on the current device (done by
+ * the first call on a device otherwise); call it once per device before any stream capture. */
+#define AFHIP_STATIC_SCRATCH_BYTES (16u << 20)
+afhip_status afhip_static_scratch_init(void);
+afhip_status afhip_launch_linear_f32_static(void *stream, int tensor_type, int layout, afhip_buffer dst,
+                                            afhip_buffer input, afhip_buffer weight, size_t rows,
+                                            size_t in_dim, size_t out_dim, int dispatch);
 /* Two matmuls of the same shape, format and layout that share X (what the engine's
  * linearNoBiasPair computes for gate + up, ops/ops.zig:909, CPU op
  * ops/native_compute.zig:6262-6307): Ya = X * Wa^T, Yb = X * Wb^T.  Each result is
