@@ -740,6 +740,20 @@ afhip_status afhip_launch_stream_read(void* stream, afhip_buffer src, afhip_buff
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
+                                     size_t in_dim, size_t out_dim) {
+    if (probe < 0 || probe > 7) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || in_dim % 32 != 0 || in_dim > 4096 || out_dim == 0 || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
+    const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q4_0, out_dim, in_dim);
+    if (need == 0 || weight.len < need || input.len < in_dim * 4 || dst.len < out_dim * 4) return AFHIP_ERR_INVALID_STATE;
+    if (dst.ptr == 0 || input.ptr == 0 || weight.ptr == 0 || dst.ptr % 4 != 0 || input.ptr % 16 != 0 || weight.ptr % 16 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_gemv_probe(static_cast<hipStream_t>(stream), probe, reinterpret_cast<float*>(dst.ptr),
+                                     reinterpret_cast<const float*>(input.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
+                                     static_cast<int>(in_dim), static_cast<int>(out_dim));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {
     if (n * 4 > dst.len || n * 2 > src.len) return AFHIP_ERR_INVALID_STATE;
     if (n == 0) return AFHIP_OK;

@@ -192,7 +192,11 @@ constexpr uint32_t kGemvHasEpilogueA = 1u << 24, kGemvHasEpilogueB = 1u << 25;
 //   kCompact:   one K slice (in_dim <= 4096), one matrix, at most one block of X per thread:
 //               the instantiation carries none of the code of the other cases (the
 //               instruction stream a wavefront walks is half as long)
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false>
+//   kProbe:     timing diagnostics (afhip_launch_gemv_probe), results meaningless: bit 0 leaves
+//               out the block dots (one xor per weight register keeps the loads alive), bit 1
+//               the store of Y, bit 2 the activation prologue (no X is read, LDS is used as found)
+constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4;
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
@@ -274,7 +278,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             wq[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qcol + lane_off[j]));
         }
     };
-    if (wave * kWave < x_blocks) {  // wave-uniform
+    if (!(kProbe & kProbeNoPrologue) && wave * kWave < x_blocks) {  // wave-uniform
         const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
         const bool two = !kCompact && x_blocks > threads;    // uniform: a second block per thread
         const int xb1 = min(tid + threads, x_blocks - 1);
@@ -320,6 +324,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     // one block of one column against one row's activations
     auto block_dot = [&](const u32x4& w, const int (&a)[kWords], int sm) {
         int dot;
+        if (kProbe & kProbeNoDots) return static_cast<int>(w.x ^ w.y ^ w.z ^ w.w) + a[0];
         if (kType == 2) {
             // 4-bit dots on the packed nibbles, nothing is unpacked: a[0..3] = high
             // nibbles of the activations (signed), a[4..7] = low nibbles (unsigned),
@@ -425,6 +430,7 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
             return;
         }
         float* dst = second ? dst_b : dst_a;
+        if ((kProbe & kProbeNoStore) && red[0] != 1234.5f) return;  // (keeps the arithmetic alive)
         if (active && mine && o0 + cc < out_dim && dst) {
             const size_t at = static_cast<size_t>(cr) * out_dim + o0 + cc;
             float v = red[0];
@@ -835,6 +841,31 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
     const GemvTargets tg{dst, dst_b, weight_prepared, weight_b_prepared, 0, ep, ep_b};
     if (tensor_type == 2) return launch_gemv_type<2>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
     return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
+}
+
+// Timing diagnostics on the one-row Q4_0 kernel (compact instantiation: in_dim <= 4096).
+hipError_t launch_gemv_probe(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
+                             int in_dim, int out_dim) {
+    constexpr int kCols = 4;
+    if (in_dim > kSliceBlocks * 32 || probe < 0 || probe > 7) return hipErrorInvalidValue;
+    const int groups = (out_dim + kCols - 1) / kCols;
+    const int waves = workgroup_waves(1024, 1024, 1, groups, false, 2);
+    const int grid = (groups + waves - 1) / waves;
+    const size_t tile_off = tile_scales_offset(2, static_cast<size_t>(out_dim) * (in_dim / 32));
+    const uint32_t shape = 1u | static_cast<uint32_t>(waves) << 8 | (grid <= compute_units() ? 1u << 16 : 0u);
+    const GemvExtras extras{nullptr, nullptr, Epilogue{}, Epilogue{}};
+    const size_t lds = gemv_fused_lds_bytes(1, in_dim);
+#define AFHIP_PROBE(P)                                                                                                  \
+    case P:                                                                                                             \
+        hipLaunchKernelGGL((gemv_fused_kernel<2, 1, kCols, false, false, true, P>), dim3(grid), dim3(64, waves), lds, stream, \
+                           weight_prepared, static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),     \
+                           static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);                   \
+        break;
+    switch (probe) {
+        AFHIP_PROBE(0) AFHIP_PROBE(1) AFHIP_PROBE(2) AFHIP_PROBE(3) AFHIP_PROBE(4) AFHIP_PROBE(5) AFHIP_PROBE(6) AFHIP_PROBE(7)
+    }
+#undef AFHIP_PROBE
+    return hipGetLastError();
 }
 
 hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned long long* keys, int* key_count,

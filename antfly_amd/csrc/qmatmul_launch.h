@@ -140,6 +140,11 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
 hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
                                             size_t rows, int dim);
 
+// The one-row Q4_0 decode kernel with parts left out (bit 0: the block dots, bit 1: the store of Y,
+// bit 2: the activation prologue): timing diagnostics, results meaningless.  in_dim <= 4096.
+hipError_t launch_gemv_probe(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
+                             int in_dim, int out_dim);
+
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 
 hipError_t launch_decode_fp16(hipStream_t stream, float* dst, const uint16_t* src, size_t n);

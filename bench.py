@@ -1,10 +1,10 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X quantized matmul (Q4_0 / Q8_0 `linearNoBias`).
 
-One "step" = one Q4_0 decode GEMV at the Llama-3-8B FFN-up shape
-(x f32 [1 x 4096], W [14336 x 4096] in 18-byte blocks), the configuration the
-headline metric is quoted on.  Weights rotate over more distinct copies than the
-256 MB Infinity Cache holds, so every step streams its 33 MB from HBM.
+One "step" = the Q4_0 decode GEMV at the Llama-3-8B FFN-up shape (x f32 [1 x 4096],
+W [14336 x 4096] in 18-byte blocks), the configuration the headline metric is quoted on,
+once on each of `--copies` (16) distinct copies of the weight: 16 launches, 528 MB --
+more than the 256 MB Infinity Cache holds, so every launch streams its 33 MB from HBM.
 
 Prints ONE JSON line: metric/value/unit as the benchmark definition names them,
 `roofline` for the dominant kernel (algorithmic bytes / HIP-event time against
@@ -27,19 +27,23 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_BPS = 8.0e12           # MI355X HBM3E
 INT8_MFMA_PEAK_OPS = 5.0e15     # MI355X dense int8 MFMA
+BF16_MFMA_PEAK_FLOPS = 2.5e15   # MI355X dense bf16 MFMA
 Q4, Q8, Q4K = 2, 8, 12
 BLOCK_BYTES = {Q4: 18, Q8: 34}
 
 
-def measured_traffic():
-    """HBM bytes per launch of the headline kernel from the committed counter summary
-    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-probe`, each scaled
-    by a kernel of known traffic in the same run), or None when that file is not there."""
-    path = os.path.join(ROOT, "profiles", "gemv_q4_0_m1_and_gemm_q8_0_m512_counters.md")
+TRAFFIC_FILE = os.path.join("profiles", "gemv_q4_0_m1_and_gemm_q8_0_m512_counters.md")
+
+
+def measured_traffic(key="traffic_bytes_per_launch_gemv_q4_0_m1"):
+    """HBM bytes per launch of a kernel from the committed counter summary (rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE runs of `bench.py --counter-probe`, each scaled by a kernel of
+    known traffic in the same run), or None when that file or line is not there.  The figure
+    is not measured by this run: `traffic_source` in the output names the file."""
     try:
-        with open(path) as f:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
             for line in f:
-                if line.startswith("traffic_bytes_per_launch_gemv_q4_0_m1:"):
+                if line.startswith(key + ":"):
                     return int(float(line.split(":", 1)[1]))
     except OSError:
         pass
@@ -61,10 +65,17 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--eager", action="store_true", help="launch every step from the host instead of replaying a HIP graph")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="the timed region (exactly --steps steps) is run this many times; the median run is reported")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
                          "read kernel over the same number of bytes, of the Q8_0 M=512 GEMM and of the Q4_K kernels "
                          "(M=1 and M=512), then exit")
+    ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048"], default=None,
+                    help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
+    ap.add_argument("--probe", choices=["gemv"], default=None,
+                    help="gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+                         "a kernel that only reads the same bytes, print a table, exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -95,8 +106,9 @@ def main() -> int:
         torch.cuda.synchronize()
         return out
 
-    def time_config(fmt, rows, in_dim, out_dim, steps, warmup, copies, seed):
-        """Returns (wall seconds, event seconds) for `steps` back-to-back calls."""
+    def time_config(fmt, rows, in_dim, out_dim, steps, warmup, copies, seed, repeats=1):
+        """Returns (wall seconds, event seconds) for `steps` back-to-back calls: the median of
+        `repeats` runs of the same timed region."""
         ws = prepared_copies(fmt, out_dim, in_dim, copies, seed)
         x = torch.from_numpy(synth.activations(seed + 1, rows, in_dim)).to(dev)
         y = torch.empty((rows, out_dim), dtype=torch.float32, device=dev)
@@ -126,19 +138,24 @@ def main() -> int:
                     step(i, cs)
             graph.replay()
             torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        if args.eager:
-            for i in range(steps):
-                step(i, stream)
-        else:
-            for _ in range(steps // chunk):
-                graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        return wall, e0.elapsed_time(e1) * 1e-3
+        walls, events = [], []
+        for _ in range(max(1, repeats)):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            e0.record()
+            if args.eager:
+                for i in range(steps):
+                    step(i, stream)
+            else:
+                for _ in range(steps // chunk):
+                    graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            walls.append(time.perf_counter() - t0)
+            events.append(e0.elapsed_time(e1) * 1e-3)
+        mid = sorted(range(len(events)), key=lambda i: events[i])[len(events) // 2]  # the median run, by device time
+        return walls[mid], events[mid]
 
     def time_lm_head(out_dim=128256, in_dim=4096, steps=40, copies=2):
         """argmax(x @ W^T) over a Llama-3 vocabulary, Q4_0: GEMV into scratch + argmax kernel per call."""
@@ -277,6 +294,109 @@ def main() -> int:
                             "frac_hbm_peak": round(weight_bytes / t / HBM_PEAK_BPS, 4)}
         return out
 
+    def time_quantizer(rows, in_dim, steps=200):
+        """The stand-alone activation quantizer (the first kernel of a prefill call), per launch."""
+        x = torch.from_numpy(synth.activations(5, rows, in_dim)).to(dev)
+        q = torch.empty(rows * in_dim, dtype=torch.int8, device=dev)
+        sc = torch.empty(rows * in_dim // 32, dtype=torch.float32, device=dev)
+        sm = torch.empty(rows * in_dim // 32, dtype=torch.int32, device=dev)
+        call = lambda st: kernels.launchQuantizeActivations(st, buf(x), rows, in_dim, buf(q), buf(sc), buf(sm))
+        for _ in range(5):
+            call(stream)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            cs = torch.cuda.current_stream().cuda_stream
+            for _ in range(steps):
+                call(cs)
+        graph.replay()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(5):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) * 1e-3 / steps)
+        return sorted(times)[2]
+
+    def gemm_roofline(m=512, k=4096, n=4096, steps=200):
+        """Second half of the metric: the Q8_0 prefill GEMM (activation quantizer + int8-MFMA kernel)."""
+        w_s, e_s = time_config(Q8, m, k, n, steps, 20, 4, 7, repeats=args.repeats)
+        t_op = e_s / steps
+        t_quant = time_quantizer(m, k)
+        t_kernel = max(t_op - t_quant, 1e-9)
+        ops = 2.0 * m * k * n
+        return {"bound": "int8_mfma", "achieved": round(ops / t_kernel / 1e12, 2), "peak": INT8_MFMA_PEAK_OPS / 1e12,
+                "unit": "TOP/s", "frac": round(ops / t_kernel / INT8_MFMA_PEAK_OPS, 4),
+                "kernel": "gemm_i8_kernel<Q8_0> (64 x 128 tiles)",
+                "workload": f"Q8_0 prefill GEMM, x f32 [{m}x{k}] quantized on the GPU, W [{n}x{k}] 34-byte blocks",
+                "ops_per_launch": ops, "us_per_op": round(t_op * 1e6, 3), "us_quantizer": round(t_quant * 1e6, 3),
+                "us_per_launch": round(t_kernel * 1e6, 3),
+                "achieved_whole_op": round(ops / t_op / 1e12, 2), "frac_whole_op": round(ops / t_op / INT8_MFMA_PEAK_OPS, 4),
+                "traffic": measured_traffic("traffic_bytes_per_launch_gemm_q8_0_m512"), "traffic_source": TRAFFIC_FILE,
+                "note": "us_per_launch = op time minus the quantizer's own launch time, both from HIP events in this run; "
+                        "every (row, column, block) term also costs one convert and one f32 multiply-add on the vector ALU"}
+
+    if args.only:
+        m = int(args.only.rsplit("m", 1)[1])
+        w_s, e_s = time_config(Q8, m, 4096, 4096, 200, 20, 4, 7, repeats=1)
+        print(json.dumps({"only": args.only, "us_per_op": round(e_s / 200 * 1e6, 3),
+                          "TOPS": round(2.0 * m * 4096 * 4096 * 200 / e_s / 1e12, 2)}))
+        return 0
+
+    if args.probe == "gemv":
+        in_dim, out_dim, copies, per_graph, replays = 4096, 14336, args.copies, 100, 10
+        ws = prepared_copies(Q4, out_dim, in_dim, copies, 2024)
+        x = torch.from_numpy(synth.activations(2025, 1, in_dim)).to(dev)
+        y = torch.empty((1, out_dim), dtype=torch.float32, device=dev)
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        w_bytes = out_dim * (in_dim // 32) * 18
+        lib = _lib.lib()
+
+        def timed(call):
+            for i in range(10):
+                call(i, stream)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for i in range(per_graph):
+                    call(i, cs)
+            graph.replay()
+            torch.cuda.synchronize()
+            out = []
+            for _ in range(7):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(replays):
+                    graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                out.append(e0.elapsed_time(e1) * 1e3 / (per_graph * replays))
+            return sorted(out)[3]
+
+        rows_out = []
+        t = timed(lambda i, st: lib.afhip_launch_stream_read(st, Buffer(ws[i % copies].data_ptr(), w_bytes), buf(sink)))
+        rows_out.append(("read only: the same 33,030,144 bytes, 16 B per lane, nothing else", t))
+        names = {0: "the decode kernel as launched by afhip_launch_linear_f32", 1: "without the block dots",
+                 2: "without the store of Y", 3: "without dots and store", 4: "without the activation prologue",
+                 5: "without prologue and dots", 6: "without prologue and store", 7: "loads and the wavefront reduction only"}
+        for probe in range(8):
+            def call(i, st, probe=probe):
+                rc = lib.afhip_launch_gemv_probe(st, probe, buf(y), buf(x), buf(ws[i % copies]), in_dim, out_dim)
+                if rc != 0:
+                    raise RuntimeError(f"probe failed: {rc}")
+            rows_out.append((f"probe {probe}: {names[probe]}", timed(call)))
+        nbytes = gemv_bytes(Q4, 1, in_dim, out_dim)
+        print("| variant | us per launch | GB/s | % of 8 TB/s |")
+        print("|---|---|---|---|")
+        for name, us in rows_out:
+            print(f"| {name} | {us:.3f} | {nbytes / us / 1e3:.0f} | {nbytes / us / 1e3 / 80:.1f} |")
+        print(json.dumps({"probe": "gemv", "us_per_launch": {n: round(u, 3) for n, u in rows_out}}))
+        return 0
+
     if args.counter_probe:
         n_launch, copies = 40, 8
         launch = _lib.lib().afhip_launch_linear_f32
@@ -315,10 +435,12 @@ def main() -> int:
 
     # ---- headline: Q4_0 decode GEMV, M=1, K=4096, N=14336 --------------------------
     rows, in_dim, out_dim = 1, 4096, 14336
-    wall, ev = time_config(Q4, rows, in_dim, out_dim, args.steps, args.warmup, args.copies, 2024)
+    launches = args.steps * args.copies  # a step visits every weight copy once
+    wall, ev = time_config(Q4, rows, in_dim, out_dim, launches, args.warmup * args.copies, args.copies, 2024,
+                           repeats=args.repeats)
     nbytes = gemv_bytes(Q4, rows, in_dim, out_dim)
-    value = nbytes * args.steps / wall / 1e9
-    achieved = nbytes * args.steps / ev / 1e9
+    value = nbytes * launches / wall / 1e9
+    achieved = nbytes * launches / ev / 1e9
     result = {
         "metric": "Q4 GEMV HBM GB/s (% of 8TB/s) K=4096,N=14336; Q8 GEMM M=512 TOPS",
         "value": round(value, 2),
@@ -326,6 +448,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "repeats": args.repeats,
         "ms_per_step": round(wall / args.steps * 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -334,11 +457,16 @@ def main() -> int:
         "data": "synthetic (seeded SplitMix64: x~N(0,1), Q4_0 nibbles uniform, fp16 scales |N(0,0.02)|/7)",
         "config": {"workload": "Q4_0 decode GEMV, x f32 [1x4096], W [14336x4096] 18-byte blocks (Llama-3-8B FFN-up)",
                    "rows": rows, "in_dim": in_dim, "out_dim": out_dim, "weight_copies": args.copies,
-                   "bytes_per_step": nbytes},
+                   "launches_per_step": args.copies, "bytes_per_launch": nbytes, "bytes_per_step": nbytes * args.copies,
+                   "step": "one GEMV launch on each of the weight copies (every launch reads its weights from HBM, not from "
+                           "the 256 MB Infinity Cache)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK_BPS, 4), "traffic": measured_traffic(),
-                     "kernel": "gemv_fused_kernel<Q4_0, rows=1>", "us_per_launch": round(ev / args.steps * 1e6, 3)},
+                     "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --counter-probe`; not measured by this run)",
+                     "kernel": "gemv_fused_kernel<Q4_0, rows=1>", "us_per_launch": round(ev / launches * 1e6, 3)},
     }
+
+    result["roofline_gemm"] = gemm_roofline()
 
     # ---- other configurations ---------------------------------------------------------
     if not args.no_extra:
@@ -407,11 +535,14 @@ def main() -> int:
         for m in (32, 128, 512):
             w_s, e_s = time_config(Q4K, m, 4096, 14336, 40, 5, 2, 78)
             flops = 2.0 * m * 4096 * 14336
+            # the kernel issues three bf16 MFMA products per f32 product (X as hi + mid + lo parts), so the
+            # matrix-core work is 3 x 2MNK flop, priced against the dense bf16 peak
             extra[f"q4k_gemm_m{m}_k4096_n14336"] = {
                 "what": "Q4_K prefill: X split once into three bf16 parts, bf16-MFMA GEMM, f32-accurate; per call incl. the split",
                 "us_per_call": round(e_s / 40 * 1e6, 1),
                 "TFLOPs_f32_equivalent": round(flops * 40 / e_s / 1e12, 1),
-                "frac_f32_mfma_peak": round(flops * 40 / e_s / 157.3e12, 3)}
+                "bf16_mfma_TFLOPs_issued": round(3 * flops * 40 / e_s / 1e12, 1),
+                "frac_bf16_mfma_peak": round(3 * flops * 40 / e_s / BF16_MFMA_PEAK_FLOPS, 4)}
         for m in (128, 512, 2048):
             gsteps = 200
             w_s, e_s = time_config(Q8, m, 4096, 4096, gsteps, 20, 4, 7)
@@ -444,6 +575,28 @@ def main() -> int:
             if (dt >= args.cpu_seconds and calls >= 20) or dt >= 3 * args.cpu_seconds:
                 break
         prepared.close()
+        # the GEMM half on the same cores: row-split over min(8, rows) workers as the engine plans it
+        # (ops/native_compute.zig:9756-9776), a bounded number of calls
+        gm, gk, gn = 512, 4096, 4096
+        gw = synth.weights(Q8, 7, gn, gk)
+        gx = synth.activations(8, gm, gk)
+        gprep = O.Prepared(Q8, gw, gn, gk)
+        gy = np.zeros((gm, gn), dtype=np.float32)
+        gprep.linear(gx, gm, workers=workers, y=gy)
+        gcalls, g0 = 0, time.perf_counter()
+        while True:
+            gprep.linear(gx, gm, workers=workers, y=gy)
+            gcalls += 1
+            gdt = time.perf_counter() - g0
+            if (gdt >= args.cpu_seconds and gcalls >= 3) or gdt >= 3 * args.cpu_seconds:
+                break
+        gprep.close()
+        result["cpu_baseline_gemm"] = {
+            "value": round(2.0 * gm * gk * gn * gcalls / gdt / 1e12, 4), "unit": "TOP/s", "cores": workers, "kind": "port",
+            "sample": f"{gcalls} calls of the same Q8_0 [{gm}x{gk}]x[{gn}x{gk}] prefill matmul (activation quantizer + int8 block "
+                      f"dots + f32 scaled accumulate) in {gdt:.1f} s ({gdt / gcalls * 1e3:.1f} ms/call), rows split over {workers} threads",
+            "host_cpus": os.cpu_count(),
+        }
         result["cpu_baseline"] = {
             "value": round(nbytes * calls / dt / 1e9, 3), "unit": "GB/s", "cores": workers, "kind": "port",
             "sample": f"{calls} calls of the same Q4_0 [1x4096]x[14336x4096] GEMV in {dt:.1f} s "

@@ -304,6 +304,13 @@ afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_
  * beside the GEMV as "what one launch of this size can draw from HBM", and it is
  * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
 afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
+/* Diagnostic with no counterpart in the reference: the one-row Q4_0 decode GEMV (PREPARED
+ * weight, in_dim <= 4096) with parts left out -- `probe` bit 0: the block dots, bit 1: the
+ * store of Y, bit 2: the activation prologue (no X read, no quantization).  probe 0 is the
+ * kernel afhip_launch_linear_f32 launches; any other value leaves dst meaningless.  bench.py
+ * --probe gemv times the eight variants to show where a launch's time goes. */
+afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
+                                     afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
 
 /* ------------------------------------------------------------------------
  * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
