@@ -288,6 +288,33 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
+    if (fused_ok && rows >= 2 && in_dim > 4096) {
+        // small batches on a K longer than 4096 (also when a plan forces them on more rows: slices
+        // of eight rows): K is shared out over workgroups, each of which stages and quantizes only
+        // its 4096-value slice of X; the slices' sums meet in the caller's scratch.
+        if (counters) {
+            if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+            else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+            else counters->mm++;
+        }
+        constexpr size_t kBatchRows = 8;
+        const size_t partial_bytes = want_dots ? 0 : gemv_batch_partial_bytes(rows < kBatchRows ? rows : kBatchRows, in_dim, out_dim, pair);
+        if (partial_bytes != 0 && (workspace.ptr == 0 || workspace.len < partial_bytes || workspace.ptr % 16 != 0))
+            return AFHIP_ERR_INVALID_STATE;
+        for (size_t r0 = 0; r0 < rows; r0 += kBatchRows) {
+            const int nr = static_cast<int>(rows - r0 < kBatchRows ? rows - r0 : kBatchRows);
+            Epilogue ep_rows = ep;
+            if (ep_rows.residual) ep_rows.residual += r0 * out_dim;
+            hipError_t e = launch_gemv_batch(stream, tensor_type, want_dots ? nullptr : y + r0 * out_dim,
+                                             want_dots ? dot_out + r0 * out_dim * kb : nullptr, x + r0 * in_dim, w, nr,
+                                             static_cast<int>(in_dim), static_cast<int>(out_dim),
+                                             partial_bytes ? reinterpret_cast<float*>(workspace.ptr) : nullptr,
+                                             pair ? y_b + r0 * out_dim : nullptr, pair ? w_b : nullptr, ep_rows, ep_b);
+            if (e != hipSuccess) return static_cast<afhip_status>(e);
+        }
+        return AFHIP_OK;
+    }
+
     if (fused_ok) {
         // mmv / small_batch (also when a plan forces them on more rows: 16-row slices).
         // Few rows: the GEMV quantizes X in its own prologue, one launch.  More: every
@@ -561,7 +588,10 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
     const size_t base = workspace_view(0, rows, in_dim).bytes;
     // nine rows and more (the MFMA GEMM): room for the partial sums of K shares when the grid is small
     const size_t partial = rows >= 9 ? gemm_i8_partial_bytes(rows, in_dim, out_dim) : 0;
-    return partial != 0 ? (base + 255) / 256 * 256 + partial : base;
+    const size_t gemm_bytes = partial != 0 ? (base + 255) / 256 * 256 + partial : base;
+    // small batches on a long K (also slices of eight rows of a forced plan): the K slices' sums, for a pair of matrices
+    const size_t batch_bytes = gemv_batch_partial_bytes(rows < 8 ? rows : 8, in_dim, out_dim, true);
+    return gemm_bytes > batch_bytes ? gemm_bytes : batch_bytes;
 }
 
 afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,

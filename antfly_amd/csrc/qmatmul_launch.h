@@ -70,6 +70,18 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
                              const uint8_t* weight_b_prepared = nullptr, const Epilogue& ep = Epilogue{},
                              const Epilogue& ep_b = Epilogue{});
 
+// Two to eight rows (one works too) of f32 activations, quantized inside the launch; PREPARED
+// weights.  in_dim > 4096: K is shared out over workgroups and `partial`
+// (gemv_batch_partial_bytes; 16-byte aligned) receives the slices' sums, which a second kernel
+// adds in slice order.  dots optional (int32 [rows][out][in/32], one matrix); dst_b /
+// weight_b_prepared: a second matrix of the same shape that shares X.
+hipError_t launch_gemv_batch(hipStream_t stream, int tensor_type, float* dst, int* dots, const float* input,
+                             const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, float* partial,
+                             float* dst_b = nullptr, const uint8_t* weight_b_prepared = nullptr,
+                             const Epilogue& ep = Epilogue{}, const Epilogue& ep_b = Epilogue{});
+int gemv_batch_waves(int rows, int in_dim, int groups);
+size_t gemv_batch_partial_bytes(size_t rows, size_t in_dim, size_t out_dim, bool pair);
+
 // One row, no Y: every workgroup leaves the argmax key (see argmax_key) of its output
 // columns in keys[workgroup]; *key_count receives the number of workgroups, which is at
 // most (out_dim + 1) / 2.  launch_argmax_keys turns the keys into the token.

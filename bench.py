@@ -73,6 +73,8 @@ def main() -> int:
                          "(M=1 and M=512), then exit")
     ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048"], default=None,
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
+    ap.add_argument("--shapes", default=None,
+                    help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k): time only these calls, print one line each, exit")
     ap.add_argument("--probe", choices=["gemv"], default=None,
                     help="gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
@@ -338,6 +340,19 @@ def main() -> int:
                 "traffic": measured_traffic("traffic_bytes_per_launch_gemm_q8_0_m512"), "traffic_source": TRAFFIC_FILE,
                 "note": "us_per_launch = op time minus the quantizer's own launch time, both from HIP events in this run; "
                         "every (row, column, block) term also costs one convert and one f32 multiply-add on the vector ALU"}
+
+    if args.shapes:
+        for spec in args.shapes.split(","):
+            f, r, k, n = spec.split(":")
+            fmt = {"q4": Q4, "q8": Q8, "q4k": Q4K}[f]
+            r, k, n = int(r), int(k), int(n)
+            wbytes = n * (k // 32) * BLOCK_BYTES[fmt] if fmt != Q4K else n * (k // 256) * 144
+            copies = max(2, min(16, (600 << 20) // wbytes))
+            w_s, e_s = time_config(fmt, r, k, n, 400, 20, copies, 99, repeats=3)
+            b = wbytes + 4 * r * (k + n)
+            print(json.dumps({"shape": spec, "us_per_call": round(e_s / 400 * 1e6, 3), "GBps": round(b * 400 / e_s / 1e9, 1),
+                              "frac_hbm_peak": round(b * 400 / e_s / HBM_PEAK_BPS, 4)}), flush=True)
+        return 0
 
     if args.only:
         m = int(args.only.rsplit("m", 1)[1])

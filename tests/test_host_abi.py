@@ -131,14 +131,25 @@ def test_q4_k_prefill_workspace_sizes():
 def test_int8_gemm_workspace_has_room_for_k_shares():
     """Nine rows and more on a grid too small for the chip: behind the quantized activations the
     scratch holds the partial sums of 2, 4 or 8 K shares (at least 16 blocks each); a grid that
-    fills the chip, or eight rows and fewer, asks for the quantized activations only."""
+    fills the chip asks for the quantized activations only.  Up to eight rows (and eight-row
+    slices of a forced plan) on a K longer than 4096 need the sums of the K slices of the
+    small-batch kernel, for a pair of matrices."""
+    def quantized(rows, k):  # int8 values padded to 256 bytes, f32 scales, i32 sums
+        return (rows * k + 255) // 256 * 256 + rows * (k // 32) * 8
+
+    def batch(rows, k, n):
+        slices = (k // 32 + 127) // 128
+        return slices * min(rows, 8) * n * 4 * 2 if slices > 1 else 0
+
     for fmt in (_lib.TYPE_Q4_0, _lib.TYPE_Q8_0):
-        base = lambda rows, k: kernels.workspaceBytes(fmt, rows, k, 1 << 20)  # a huge matrix never shares K out
         for rows, k, n in [(16, 4096, 4096), (64, 14336, 4096), (9, 1024, 64)]:
-            extra = kernels.workspaceBytes(fmt, rows, k, n) - (base(rows, k) + 255) // 256 * 256
-            assert extra > 0 and extra % (rows * n * 4) == 0
+            got = kernels.workspaceBytes(fmt, rows, k, n)
+            extra = got - (quantized(rows, k) + 255) // 256 * 256
+            assert extra > 0 and extra % (rows * n * 4) == 0 and got >= batch(rows, k, n)
             shares = extra // (rows * n * 4)
             assert shares in (2, 4, 8) and (k // 32) // shares >= 16
-        assert kernels.workspaceBytes(fmt, 8, 4096, 4096) == base(8, 4096)
-        assert kernels.workspaceBytes(fmt, 512, 4096, 4096) == base(512, 4096)
-        assert kernels.workspaceBytes(fmt, 16, 512, 4096) == base(16, 512)  # too short a K to share out
+        assert kernels.workspaceBytes(fmt, 8, 4096, 4096) == quantized(8, 4096)
+        assert kernels.workspaceBytes(fmt, 512, 4096, 4096) == quantized(512, 4096)
+        assert kernels.workspaceBytes(fmt, 16, 512, 4096) == quantized(16, 512)  # too short a K to share out
+        assert kernels.workspaceBytes(fmt, 5, 14336, 4096) == max(quantized(5, 14336), batch(5, 14336, 4096))
+        assert batch(5, 14336, 4096) == 4 * 5 * 4096 * 4 * 2
