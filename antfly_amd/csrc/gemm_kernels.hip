@@ -39,9 +39,11 @@
 // lane % 32, so stores are 128 bytes contiguous along n.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstdlib>
 
 #include "device_common.h"
+#include "gemv_common.h"
 #include "qmatmul_launch.h"
 
 namespace afhip {
@@ -110,16 +112,15 @@ __device__ __forceinline__ void wait_vm_outstanding(int n) {
 // to 4).  Issued as inline assembly on purpose: the compiler would otherwise make
 // every later LDS read wait for all such loads in flight, which defeats the ring.
 // Completion is tracked with wait_vm_outstanding(); base and lds_addr are wave-uniform.
-// M0 is written without being declared (it is reserved to the compiler, which has no
-// use for it in this kernel: no LDS-direct builtins, no relative register moves).
+// M0 is declared as clobbered, so the compiler keeps nothing of its own in it across these statements.
 __device__ __forceinline__ void lds_load16(const void* base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_load4(const void* base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void lds_load2(const void* base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 extern __shared__ __align__(16) unsigned char gemm_lds[];
@@ -464,15 +465,18 @@ hipError_t launch_tile(hipStream_t stream, float* dst, int* dots, const int8_t* 
     auto kernel_shares = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, false, true>;
     auto kernel_dots = gemm_i8_kernel<kType, kWavesM, kWavesN, kSplit, true>;
     // more than 64 KB of LDS has to be asked for once per kernel
-    static const hipError_t attr = [&]() {
+    static std::atomic<bool> attr_done{false};
+    const hipError_t attr = attr_done.load(std::memory_order_acquire) ? hipSuccess : [&]() {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_f32),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, S::kLdsBytes);
         if (e != hipSuccess) return e;
         e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_shares), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 S::kLdsBytes);
         if (e != hipSuccess) return e;
-        return hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_dots), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                   S::kLdsBytes);
+        e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_dots), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                S::kLdsBytes);
+        if (e == hipSuccess) attr_done.store(true, std::memory_order_release);  // a failure is not remembered: the next call tries again
+        return e;
     }();
     if (attr != hipSuccess) return attr;
     if (dots)
@@ -506,9 +510,7 @@ hipError_t launch_type(hipStream_t stream, float* dst, int* dots, const int8_t* 
 int gemm_i8_splits(int rows, int in_dim, int out_dim) {
     const long workgroups = static_cast<long>((rows + 31) / 32) * ((out_dim + 63) / 64);
     const int kb = in_dim / 32;
-    int units = 0, dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || units <= 0)
-        units = 256;
+    const int units = gemv_compute_units();
     int splits = 1;
     while (splits < 8 && workgroups * splits * 2 <= units && kb / (splits * 2) >= 16) splits *= 2;
     return splits;

@@ -71,10 +71,10 @@ struct GemvTargets {
 //               the store of Y, bit 2 the activation prologue (no X is read, LDS is used as found)
 constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4;
 template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
-__global__ __launch_bounds__(1024) void gemv_fused_kernel(
+__device__ __forceinline__ void gemv_fused_body(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
-    GemvExtras extras) {
+    const GemvExtras& extras) {
     const int slices = kCompact ? 1 : static_cast<int>(shape & 0xFF);
     const int groups_per_wg = (shape >> 8) & 0xFF, stagger = (shape >> 16) & 0xFF;
     const int groups_each = (out_dim + kCols - 1) / kCols;
@@ -344,6 +344,15 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
         key = workgroup_max_key(key, reinterpret_cast<unsigned long long*>(partial), tid, waves);
         if (tid == 0) extras.keys[blockIdx.x] = key;
     }
+}
+
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
+__global__ __launch_bounds__(1024) void gemv_fused_kernel(
+    const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
+    float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
+    GemvExtras extras) {
+    gemv_fused_body<kType, kRows, kCols, kWriteDots, kArgmax, kCompact, kProbe>(weight_a, weight_b, input, dst_a, dst_b, tile_off16,
+                                                                                 kb, out_dim, shape, extras);
 }
 
 // =====================================================================
