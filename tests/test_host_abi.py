@@ -153,3 +153,37 @@ def test_int8_gemm_workspace_has_room_for_k_shares():
         assert kernels.workspaceBytes(fmt, 16, 512, 4096) == quantized(16, 512)  # too short a K to share out
         assert kernels.workspaceBytes(fmt, 5, 14336, 4096) == max(quantized(5, 14336), batch(5, 14336, 4096))
         assert batch(5, 14336, 4096) == 4 * 5 * 4096 * 4 * 2
+
+
+def test_zig_backend_sources_bind_what_exists():
+    """The Zig `hip` backend sources (zig/pkg/inference/src/ops/hip) cannot be compiled in this
+    image; this keeps them honest against what can be checked here: every C-ABI function they
+    declare is in the header with the same argument count, and every kernel they look up by
+    name is an extern "C" entry of the code object's source."""
+    zig_dir = os.path.join(ROOT, "zig", "pkg", "inference", "src", "ops", "hip")
+    names = sorted(os.listdir(zig_dir))
+    assert names == ["buffer.zig", "context.zig", "driver.zig", "hip_compute.zig", "kernels.zig", "scratch.zig"]
+    kernels_zig = open(os.path.join(zig_dir, "kernels.zig")).read()
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "antfly_hip_qmatmul.h")).read(), flags=re.S)
+    externs = re.findall(r'extern "c" fn (afhip_[a-z0-9_]+)\((.*?)\)\s*[a-z_]+;', kernels_zig, flags=re.S)
+    assert len(externs) >= 3
+    for name, params in externs:
+        m = re.search(r"\b" + name + r"\s*\((.*?)\);", header, flags=re.S)
+        assert m, name
+        zig_args = [p for p in params.split(",") if p.strip()]
+        c_args = [p for p in m.group(1).split(",") if p.strip() and p.strip() != "void"]
+        assert len(zig_args) == len(c_args), (name, zig_args, c_args)
+    entries = set(re.findall(r'"(termite_hip_[a-z0-9_]+)"', kernels_zig))
+    source = open(os.path.join(ROOT, "antfly_amd", "csrc", "code_object_kernels.hip")).read()
+    exported = set(re.findall(r'extern "C" __global__[^\n]*void (termite_hip_[a-z0-9_]+)\(', source))
+    assert entries and entries <= exported, entries - exported
+    # the driver table binds only symbols libamdhip64 exports under these names
+    driver_zig = open(os.path.join(zig_dir, "driver.zig")).read()
+    table = re.findall(r"^\s+(hip[A-Za-z]+): \*const fn", driver_zig, flags=re.M)
+    assert len(table) >= 20 and len(set(table)) == len(table)
+    try:
+        hip = C.CDLL("libamdhip64.so")
+    except OSError:
+        pytest.skip("libamdhip64.so not loadable here")
+    missing = [n for n in table if not hasattr(hip, n)]
+    assert not missing, missing
