@@ -271,3 +271,30 @@ def test_full_size_gate_up_pair(rows):
     prepared.close()
     err = G.max_rel_err(yb, ref.astype(np.float64))
     assert err <= TOL and err <= TIGHT, err
+
+
+@pytest.mark.parametrize("fmt_name,fmt", [("q4_0", Q4), ("q8_0", Q8)])
+@pytest.mark.parametrize("case,rows,in_dim,out_dim", [("k256_n64", 5, 256, 64), ("k96_n512", 5, 96, 512)])
+def test_committed_tiny_vectors(fmt_name, fmt, case, rows, in_dim, out_dim):
+    """The HIP path against tests/golden/tiny_vectors.npz (no oracle call): quantized activations,
+    scales, sums and int32 block dots bit-exact, outputs within tolerance."""
+    import os
+
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "tiny_vectors.npz"), allow_pickle=False)
+    key = f"{fmt_name}_{case}_"
+    x, w = g[key + "x"], g[key + "w_raw"]
+    print(f"case: tiny vectors {key}", flush=True)
+    xd = G.to_dev(x)
+    q = torch.empty(rows * in_dim, dtype=torch.int8, device=G.DEV)
+    s = torch.empty(rows * in_dim // 32, dtype=torch.float32, device=G.DEV)
+    sums = torch.empty(rows * in_dim // 32, dtype=torch.int32, device=G.DEV)
+    kernels.launchQuantizeActivations(G.stream(), G.buf(xd), rows, in_dim, G.buf(q), G.buf(s), G.buf(sums))
+    torch.cuda.synchronize()
+    assert np.array_equal(q.cpu().numpy().reshape(rows, in_dim), g[key + "qx"])
+    assert np.array_equal(s.cpu().numpy().view(np.uint32).reshape(rows, -1), g[key + "sx"].view(np.uint32))
+    assert np.array_equal(sums.cpu().numpy().reshape(rows, -1), g[key + "sumx"])
+    for layout in (RAW, PREP):
+        wd = G.prepare(fmt, w, out_dim, in_dim) if layout == PREP else G.to_dev(w)
+        assert np.array_equal(G.block_dots(fmt, layout, x, wd, rows, in_dim, out_dim), g[key + "block_dots"])
+        y = G.linear(fmt, layout, x, wd, rows, in_dim, out_dim)
+        assert G.max_rel_err(y, g[key + "y_op"].astype(np.float64)) <= TIGHT

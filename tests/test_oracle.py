@@ -1,5 +1,7 @@
 """Pins the CPU oracle against the reference's known-answer vectors and against
 what the mathematics fixes (closed forms, brute force, invariants).  No GPU."""
+import os
+
 import numpy as np
 import pytest
 
@@ -7,6 +9,7 @@ from antfly_amd import synth
 from oracle import oracle as O
 
 Q4, Q8 = O.FMT_Q4_0, O.FMT_Q8_0
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def smoke_row(fmt, scale, value):
@@ -462,3 +465,40 @@ def test_synth_is_chunk_invariant_and_in_range():
     assert w4.size == synth.weight_bytes(Q4, 8, 64) == 8 * 2 * 18
     x = synth.activations(3, 64, 512)
     assert abs(float(x.mean())) < 0.02 and abs(float(x.std()) - 1.0) < 0.02
+
+
+def test_oracle_reproduces_committed_tiny_vectors():
+    """tests/golden/tiny_vectors.npz (written by tests/golden/make_tiny_vectors.py) holds the
+    oracle's intermediates for two tiny shapes per format; the oracle as built now must give the
+    same bits, and the fixture must be self-consistent with what the mathematics fixes."""
+    import importlib.util
+
+    spec = importlib.util.spec_from_file_location("make_tiny_vectors", os.path.join(ROOT, "tests", "golden", "make_tiny_vectors.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    want = np.load(os.path.join(ROOT, "tests", "golden", "tiny_vectors.npz"), allow_pickle=False)
+    got = mod.build()
+    assert sorted(want.files) == sorted(got)
+    for name in want.files:
+        assert np.array_equal(want[name], got[name]), name
+    # independent of the oracle: the block dots are the integer sums of products of the stored
+    # quantized activations and the weights as numpy unpacks them
+    for fmt_name, fmt in mod.FORMATS:
+        for case, rows, in_dim, out_dim in mod.CASES:
+            key = f"{fmt_name}_{case}_"
+            raw = want[key + "w_raw"].reshape(out_dim, in_dim // 32, -1)
+            if fmt == Q8:
+                wq = raw[:, :, 2:].view(np.int8).astype(np.int64)
+            else:
+                b = raw[:, :, 2:].astype(np.int64)
+                wq = np.concatenate([(b & 15) - 8, (b >> 4) - 8], axis=2)
+            qx = want[key + "qx"].reshape(rows, in_dim // 32, 32).astype(np.int64)
+            dots = np.einsum("rbi,obi->rob", qx, wq)
+            assert np.array_equal(dots, want[key + "block_dots"].astype(np.int64)), key
+            d = raw[:, :, :2].copy().view(np.float16).astype(np.float64)[:, :, 0]
+            y64 = np.einsum("rb,ob,rob->ro", want[key + "sx"].astype(np.float64), d, dots.astype(np.float64))
+            for assoc in ("y_pair_assoc", "y_single_assoc"):
+                assert np.abs(want[key + assoc] - y64).max() <= 2e-6 * np.abs(y64).max(), (key, assoc)
+            gate = bool(want[key + "uses_activation_quant"][0])
+            assert gate == (out_dim >= 512 and in_dim // 32 >= 3)
+            assert np.array_equal(want[key + "y_op"], want[key + ("y_single_assoc" if gate else "y_f32_route")]) or gate
