@@ -75,7 +75,8 @@ class DebugStats(C.Structure):
     _fields_ = [(n, C.c_uint64) for n in (
         "h2d_bytes", "d2h_bytes", "resident_weight_bytes", "pooled_buffers", "device_allocs",
         "launches_mmv", "launches_small_batch", "launches_mm", "launches_f32_route",
-        "launches_activation_quant", "launches_prepare", "scratch_bytes")]
+        "launches_activation_quant", "launches_prepare", "scratch_bytes",
+        "activation_quant_ns", "compute_ns", "timed_ops")]
 
 
 GGUF_MAX_DIMS = 8
@@ -181,6 +182,7 @@ SIGNATURES = {
     "afhip_compute_insert_weight_from_gguf": (_st, [_vp, _vp, C.c_char_p, C.c_char_p, _i]),
     "afhip_compute_load_gguf": (_st, [_vp, _vp, _i, C.POINTER(_sz), C.POINTER(_sz)]),
     "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
+    "afhip_compute_set_phase_timing": (_st, [_vp, _i]),
     "afhip_smoke_q8_0": (_st, []),
     "afhip_smoke_q4_0": (_st, []),
 }

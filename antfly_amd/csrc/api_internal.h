@@ -10,6 +10,11 @@ namespace afhip {
 
 struct LaunchCounters {
     uint64_t mmv = 0, small_batch = 0, mm = 0, f32_route = 0, activation_quant = 0, prepare = 0;
+    // Opt-in phase timing (the engine's QuantExecutionTimingStats, ops/ops.zig:649-713): when
+    // `phase_events` is set, the op records phase_events[0] before its first kernel, [1] behind the
+    // stand-alone activation quantizer (or at once, when the kernel quantizes in its own prologue)
+    // and [2] behind its last kernel, all on the op's stream.  They are hipEvent_t.
+    void** phase_events = nullptr;
 };
 
 bool checked_mul(size_t a, size_t b, size_t* out);

@@ -42,6 +42,11 @@ afhip_status static_scratch_address(unsigned char** out) {
 
 bool checked_mul(size_t a, size_t b, size_t* out) { return !__builtin_mul_overflow(a, b, out); }
 
+// Records phase event `i` of an op that is being timed (see LaunchCounters).
+static void mark_phase(LaunchCounters* counters, int i, hipStream_t stream) {
+    if (counters && counters->phase_events) (void)hipEventRecord(static_cast<hipEvent_t>(counters->phase_events[i]), stream);
+}
+
 size_t block_bytes(int tensor_type) {
     if (tensor_type == AFHIP_TYPE_Q4_0) return 18;
     if (tensor_type == AFHIP_TYPE_Q8_0) return 34;
@@ -166,10 +171,29 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     return AFHIP_OK;
 }
 
+static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                                     afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                     int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
+                                     afhip_buffer weight_b, const LinearExtras& extras, bool* quantizer_marked);
+
 afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
                          afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
                          int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
                          afhip_buffer weight_b, const LinearExtras& extras) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    bool quantizer_marked = false;
+    mark_phase(counters, 0, stream);
+    const afhip_status s = linear_impl_body(stream_v, tensor_type, layout, dst, input, weight, rows, in_dim, out_dim, workspace,
+                                            dispatch, dots, counters, dst_b, weight_b, extras, &quantizer_marked);
+    if (!quantizer_marked) mark_phase(counters, 1, stream);  // no stand-alone quantizer ran (or nothing ran): an empty phase
+    mark_phase(counters, 2, stream);
+    return s;
+}
+
+static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,
+                                     afhip_buffer weight, size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                     int dispatch, afhip_buffer dots, LaunchCounters* counters, afhip_buffer dst_b,
+                                     afhip_buffer weight_b, const LinearExtras& extras, bool* quantizer_marked) {
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     // biases: f32 [out_dim], the second one only with a second matrix; activation and residual
@@ -273,6 +297,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         }
         hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx,
                                                    ws.sx, ws.sums);
+        if (e == hipSuccess) {
+            mark_phase(counters, 1, stream);
+            *quantizer_marked = true;
+        }
         if (e != hipSuccess) return static_cast<afhip_status>(e);
         // room behind the quantized activations for the partial sums of K shares (small grids): optional
         const size_t partial_at = (ws.bytes + 255) / 256 * 256;
@@ -336,6 +364,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
         if (prequantize) {
             hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx,
                                                        ws.sx, ws.sums);
+            if (e == hipSuccess) {
+                mark_phase(counters, 1, stream);
+                *quantizer_marked = true;
+            }
             if (e != hipSuccess) return static_cast<afhip_status>(e);
         }
         for (size_t r0 = 0; r0 < rows; r0 += static_cast<size_t>(chunk)) {
@@ -370,6 +402,10 @@ afhip_status linear_impl(void* stream_v, int tensor_type, int layout, afhip_buff
     }
     hipError_t e = launch_quantize_activations(stream, x, static_cast<int>(rows), static_cast<int>(in_dim), ws.qx, ws.sx,
                                                ws.sums);
+    if (e == hipSuccess) {
+        mark_phase(counters, 1, stream);
+        *quantizer_marked = true;
+    }
     if (e != hipSuccess) return static_cast<afhip_status>(e);
     e = launch_linear_generic(stream, tensor_type, layout, true, want_dots ? nullptr : y, dot_out, nullptr, ws.qx, ws.sx,
                               w, static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), ep);
@@ -585,6 +621,10 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
         return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
     }
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;
+    size_t guard;  // the sizes below are sums of a few such products: refuse shapes whose products wrap
+    if (!checked_mul(rows, in_dim, &guard) || !checked_mul(guard, 16, &guard) || !checked_mul(rows, out_dim, &guard) ||
+        !checked_mul(guard, 256, &guard))
+        return 0;
     const size_t base = workspace_view(0, rows, in_dim).bytes;
     // nine rows and more (the MFMA GEMM): room for the partial sums of K shares when the grid is small
     const size_t partial = rows >= 9 ? gemm_i8_partial_bytes(rows, in_dim, out_dim) : 0;
@@ -747,7 +787,7 @@ afhip_status afhip_launch_quantize_activations(void* stream, afhip_buffer input,
     if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
     size_t count, bytes;
     if (!checked_mul(rows, in_dim, &count) || !checked_mul(count, 4, &bytes)) return AFHIP_ERR_INVALID_STATE;
-    const size_t nb = count / 32;
+    const size_t nb = count / 32;  // (count * 4 did not overflow: nb * 4 cannot)
     if (bytes > input.len || count > q.len || nb * 4 > scales.len) return AFHIP_ERR_INVALID_STATE;
     if (sums.ptr != 0 && nb * 4 > sums.len) return AFHIP_ERR_INVALID_STATE;
     if (count == 0) return AFHIP_OK;
@@ -785,7 +825,9 @@ afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, 
 }
 
 afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {
-    if (n * 4 > dst.len || n * 2 > src.len) return AFHIP_ERR_INVALID_STATE;
+    size_t dst_bytes, src_bytes;
+    if (!checked_mul(n, 4, &dst_bytes) || !checked_mul(n, 2, &src_bytes) || dst_bytes > dst.len || src_bytes > src.len)
+        return AFHIP_ERR_INVALID_STATE;
     if (n == 0) return AFHIP_OK;
     if (dst.ptr == 0 || src.ptr == 0) return AFHIP_ERR_INVALID_STATE;
     hipError_t e = launch_decode_fp16(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr),
@@ -853,7 +895,7 @@ static afhip_status dequantize_rows(void* stream, int tensor_type, int layout, a
     if (q4k) {
         hipError_t e = (q4k_tiled ? launch_dequantize_q4k_tiled_rows : launch_dequantize_q4k_rows)(
             static_cast<hipStream_t>(stream), reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
-            gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows, static_cast<int>(dim));
+            gather ? reinterpret_cast<const long long*>(ids.ptr) : nullptr, rows, static_cast<int>(dim), weight_rows);
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     hipError_t e = launch_dequantize_rows(static_cast<hipStream_t>(stream), tensor_type, layout,
@@ -894,7 +936,7 @@ afhip_status afhip_launch_quantize_rows(void* stream, int tensor_type, afhip_buf
     hipError_t e = launch_quantize_rows(static_cast<hipStream_t>(stream), tensor_type,
                                         reinterpret_cast<uint8_t*>(dst_raw.ptr), reinterpret_cast<const float*>(input.ptr),
                                         scatter ? reinterpret_cast<const long long*>(row_ids_i64.ptr) : nullptr, rows,
-                                        static_cast<int>(dim));
+                                        static_cast<int>(dim), dst_rows);
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 

@@ -35,6 +35,8 @@ struct afhip_compute {
     afhip_buffer scratch{0, 0};              // DeviceScratch, scratch.zig
     afhip_debug_stats stats{};
     LaunchCounters counters;
+    hipEvent_t phase_events[3] = {nullptr, nullptr, nullptr};  // created by afhip_compute_set_phase_timing
+    bool phase_timing = false;
 };
 
 namespace {
@@ -229,9 +231,20 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         if (bias_b) extras.bias_b = bias_b->buffer;
         if (residual) extras.residual = residual->buffer;
         extras.activation = activation;
+        self->counters.phase_events = self->phase_timing ? reinterpret_cast<void**>(self->phase_events) : nullptr;
         s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows,
                         in_dim, out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
                         pair ? weight_b->buffer : afhip_buffer{0, 0}, extras);
+        self->counters.phase_events = nullptr;
+        if (s == AFHIP_OK && self->phase_timing && hipEventSynchronize(self->phase_events[2]) == hipSuccess) {
+            float quant_ms = 0.0f, compute_ms = 0.0f;
+            if (hipEventElapsedTime(&quant_ms, self->phase_events[0], self->phase_events[1]) == hipSuccess &&
+                hipEventElapsedTime(&compute_ms, self->phase_events[1], self->phase_events[2]) == hipSuccess) {
+                self->stats.activation_quant_ns += static_cast<uint64_t>(quant_ms * 1e6f);
+                self->stats.compute_ns += static_cast<uint64_t>(compute_ms * 1e6f);
+                self->stats.timed_ops++;
+            }
+        }
     }
     if (s != AFHIP_OK) {
         release_device_buffer(self, &device);
@@ -286,6 +299,8 @@ void afhip_compute_destroy(afhip_compute* self) {
     for (auto& kv : self->resident_weights) free_device_buffer(&kv.second.buffer);
     for (auto& b : self->temp_buffers) free_device_buffer(&b);
     free_device_buffer(&self->scratch);
+    for (hipEvent_t e : self->phase_events)
+        if (e) (void)hipEventDestroy(e);
     if (self->stream) (void)hipStreamDestroy(self->stream);
     delete self;
 }
@@ -347,10 +362,10 @@ afhip_status afhip_compute_insert_weight_from_loaded(afhip_compute* self, const 
     if (!keep_raw_layout && bb != 0 && shape_len == 2 && shape[1] > 0 && shape[1] % block_values == 0 &&
         raw_len == static_cast<size_t>(shape[0]) * static_cast<size_t>(shape[1] / block_values) * bb && raw_len > 0) {
         afhip_buffer prepared;
-        s = alloc_device_buffer(self, afhip_prepared_weight_bytes(tensor_type, static_cast<size_t>(shape[0]),
-                                                                  static_cast<size_t>(shape[1])),
-                                &prepared);
+        const size_t prepared_len = afhip_prepared_weight_bytes(tensor_type, static_cast<size_t>(shape[0]), static_cast<size_t>(shape[1]));
+        s = alloc_device_buffer(self, prepared_len, &prepared);
         if (s == AFHIP_OK) {
+            prepared.len = prepared_len;  // (a pooled buffer may be longer: the weight's own size is what the counters report)
             s = afhip_launch_prepare_weight(self->stream, tensor_type, prepared, t.buffer, static_cast<size_t>(shape[0]),
                                             static_cast<size_t>(shape[1]));
             if (s == AFHIP_OK) s = from_hip(hipStreamSynchronize(self->stream));
@@ -360,7 +375,7 @@ afhip_status afhip_compute_insert_weight_from_loaded(afhip_compute* self, const 
                 return s;
             }
             self->counters.prepare++;
-            release_device_buffer(self, &t.buffer);
+            free_device_buffer(&t.buffer);  // weight-sized staging copy of the raw bytes: freed, not pooled
             t.buffer = prepared;
             t.layout = AFHIP_LAYOUT_PREPARED;
         } else {
@@ -371,7 +386,10 @@ afhip_status afhip_compute_insert_weight_from_loaded(afhip_compute* self, const 
     auto it = self->resident_weights.find(key);
     if (it != self->resident_weights.end()) {
         self->stats.resident_weight_bytes -= it->second.buffer.len;
-        release_device_buffer(self, &it->second.buffer);
+        // a replaced weight goes back to the driver, not into the pool of temporaries (queued
+        // kernels may still read it: wait for them first)
+        (void)hipStreamSynchronize(self->stream);
+        free_device_buffer(&it->second.buffer);
         self->resident_weights.erase(it);
     }
     self->stats.resident_weight_bytes += t.buffer.len;
@@ -405,7 +423,10 @@ afhip_status afhip_compute_insert_weight_f32(afhip_compute* self, const char* ke
     auto it = self->resident_weights.find(key);
     if (it != self->resident_weights.end()) {
         self->stats.resident_weight_bytes -= it->second.buffer.len;
-        release_device_buffer(self, &it->second.buffer);
+        // a replaced weight goes back to the driver, not into the pool of temporaries (queued
+        // kernels may still read it: wait for them first)
+        (void)hipStreamSynchronize(self->stream);
+        free_device_buffer(&it->second.buffer);
         self->resident_weights.erase(it);
     }
     self->stats.resident_weight_bytes += t.buffer.len;
@@ -736,6 +757,20 @@ afhip_status afhip_compute_linear_no_bias_planned(afhip_compute* self,
     if (q.dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_PARTITION_PLAN;
     return linear_no_bias_impl(self, request->input, request->weight, request->rows, request->in_dim, request->out_dim,
                                q.dispatch, out);
+}
+
+afhip_status afhip_compute_set_phase_timing(afhip_compute* self, int enabled) {
+    if (!self) return AFHIP_ERR_INVALID_ARGUMENT;
+    afhip_status s = make_current(self);
+    if (s != AFHIP_OK) return s;
+    if (enabled && self->phase_events[0] == nullptr) {
+        for (hipEvent_t& e : self->phase_events) {
+            s = from_hip(hipEventCreate(&e));
+            if (s != AFHIP_OK) return s;
+        }
+    }
+    self->phase_timing = enabled != 0;
+    return AFHIP_OK;
 }
 
 afhip_status afhip_compute_debug_stats(const afhip_compute* self, afhip_debug_stats* out) {

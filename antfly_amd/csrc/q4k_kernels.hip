@@ -60,7 +60,8 @@ __device__ __forceinline__ float byte_to_f32(uint32_t word, int pass = 0) {
 // products are rounded on their own, then one multiply and one subtraction per value.
 // A lane produces four consecutive values (one 16-byte store).
 __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restrict__ dst, const uint8_t* __restrict__ weight,
-                                                                  const long long* __restrict__ ids, size_t rows, int dim) {
+                                                                  const long long* __restrict__ ids, size_t rows, int dim,
+                                                                  size_t weight_rows) {
     const size_t per_row = static_cast<size_t>(dim >> 2);
     const size_t units = rows * per_row;
     const size_t kb = static_cast<size_t>(dim / kQ4kBlockValues);
@@ -68,7 +69,12 @@ __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restr
          u += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const size_t t = u / per_row;
         const int g = static_cast<int>(u - t * per_row);  // group of four values in the row
-        const size_t block = static_cast<size_t>(ids ? ids[t] : static_cast<long long>(t)) * kb + (g >> 6);
+        const long long row = ids ? ids[t] : static_cast<long long>(t);
+        if (row < 0 || static_cast<size_t>(row) >= weight_rows) {  // an id outside the weight reads nothing: zeros
+            reinterpret_cast<float4*>(dst)[u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+            continue;
+        }
+        const size_t block = static_cast<size_t>(row) * kb + (g >> 6);
         const int v0 = (g & 63) * 4;                      // first value inside the super-block
         const int chunk = v0 >> 6, pos = v0 & 63;
         const int sub = chunk * 2 + (pos >> 5);
@@ -364,12 +370,12 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
 }
 
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
-                                      size_t rows, int dim) {
+                                      size_t rows, int dim, size_t weight_rows) {
     if (rows == 0 || dim == 0) return hipSuccess;
     size_t grid = (rows * static_cast<size_t>(dim >> 2) + 255) / 256;
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(dequantize_q4k_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst, weight, ids,
-                       rows, dim);
+                       rows, dim, weight_rows);
     return hipGetLastError();
 }
 

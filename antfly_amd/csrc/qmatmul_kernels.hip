@@ -143,7 +143,12 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict_
         const int j = static_cast<int>(u & 7);  // values 4j .. 4j+3 of the block
         const size_t tb = u >> 3;
         const size_t t = tb / kb, b = tb - t * kb;
-        const size_t block = static_cast<size_t>(ids ? ids[t] : static_cast<long long>(t)) * kb + b;
+        const long long row = ids ? ids[t] : static_cast<long long>(t);
+        if (row < 0 || static_cast<size_t>(row) >= blocks_total / kb) {  // an id outside the weight reads nothing: zeros
+            reinterpret_cast<float4*>(dst)[u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
+            continue;
+        }
+        const size_t block = static_cast<size_t>(row) * kb + b;
         const uint8_t* quants = kPrepared ? weight + block * kQuantBytes : weight + block * (kQuantBytes + 2) + 2;
         const uint16_t scale_bits = kPrepared ? reinterpret_cast<const uint16_t*>(weight + blocks_total * kQuantBytes)[block]
                                               : *reinterpret_cast<const uint16_t*>(weight + block * (kQuantBytes + 2));
@@ -176,12 +181,14 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict_
 
 // Dense f32 table: dst[t][:] = weight[ids[t]][:] (embedding lookup on an unquantized table).
 __global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict__ dst, const float* __restrict__ weight,
-                                                              const long long* __restrict__ ids, size_t rows, int dim) {
+                                                              const long long* __restrict__ ids, size_t rows, int dim,
+                                                              size_t weight_rows) {
     const size_t total = rows * static_cast<size_t>(dim);
     for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < total;
          i += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const size_t t = i / dim, c = i - t * dim;
-        dst[i] = weight[static_cast<size_t>(ids[t]) * dim + c];
+        const long long row = ids[t];
+        dst[i] = row < 0 || static_cast<size_t>(row) >= weight_rows ? 0.0f : weight[static_cast<size_t>(row) * dim + c];
     }
 }
 
@@ -193,7 +200,8 @@ __global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict_
 // block has scale 1.  Eight lanes per block.
 template <int kType>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
-                                                            const long long* __restrict__ ids, size_t rows, int dim) {
+                                                            const long long* __restrict__ ids, size_t rows, int dim,
+                                                            size_t dst_rows) {
     constexpr int kRawBytes = kType == 2 ? 18 : 34;
     const size_t kb = static_cast<size_t>(dim >> 5);
     const size_t units = rows * kb * 8;
@@ -208,7 +216,9 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict_
         const int j = static_cast<int>(u & 7);
         const size_t tb = u >> 3;
         const size_t t = live ? tb / kb : 0, b = live ? tb - t * kb : 0;
-        const size_t block = static_cast<size_t>(ids && live ? ids[t] : static_cast<long long>(t)) * kb + b;
+        const long long row = ids && live ? ids[t] : static_cast<long long>(t);
+        const bool in_range = row >= 0 && static_cast<size_t>(row) < dst_rows;  // a row id outside the destination writes nothing
+        const size_t block = (in_range ? static_cast<size_t>(row) : 0) * kb + b;
         uint8_t* out = dst + block * kRawBytes;
         uint32_t packed;
         if (kType == 2) {
@@ -226,7 +236,7 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict_
             const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv), q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
             packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
         }
-        if (!live) continue;
+        if (!live || !in_range) continue;
         // blocks are 2-byte aligned: 16-bit stores
         if (j == 0) *reinterpret_cast<uint16_t*>(out) = __builtin_bit_cast(uint16_t, static_cast<_Float16>(scale));
         if (kType != 2 || j < 4) {
@@ -444,7 +454,7 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
     if (tensor_type == 0) {
         if (ids == nullptr) return hipErrorInvalidValue;  // a plain copy is not this kernel's job
         hipLaunchKernelGGL(gather_rows_f32_kernel, dim3(grid_for(rows * dim)), dim3(256), 0, stream, dst,
-                           reinterpret_cast<const float*>(weight), ids, rows, dim);
+                           reinterpret_cast<const float*>(weight), ids, rows, dim, weight_rows);
         return launch_status();
     }
     const size_t blocks_total = weight_rows * static_cast<size_t>(dim >> 5);
@@ -460,11 +470,11 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
 }
 
 hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
-                                size_t rows, int dim) {
+                                size_t rows, int dim, size_t dst_rows) {
     if (rows == 0 || dim == 0) return hipSuccess;
     const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
-    if (tensor_type == 2) hipLaunchKernelGGL(quantize_rows_kernel<2>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim);
-    else hipLaunchKernelGGL(quantize_rows_kernel<8>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim);
+    if (tensor_type == 2) hipLaunchKernelGGL(quantize_rows_kernel<2>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+    else hipLaunchKernelGGL(quantize_rows_kernel<8>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
     return launch_status();
 }
 

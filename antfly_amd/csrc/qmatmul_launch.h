@@ -121,7 +121,7 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
 
 // set_rows / cpy_f32_to_q: f32 [rows][dim] -> raw GGUF blocks at rows ids[t] of dst_raw (ids == nullptr: in order).
 hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
-                                size_t rows, int dim);
+                                size_t rows, int dim, size_t dst_rows);
 
 // Q4_K (raw GGUF layout, 16-byte aligned): Y = X * W^T on f32 activations, any number of rows
 // (two per launch), in_dim a multiple of 256 up to gemv_q4k_max_in_dim(); and its get_rows /
@@ -130,7 +130,7 @@ int gemv_q4k_max_in_dim();
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                            int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
-                                      size_t rows, int dim);
+                                      size_t rows, int dim, size_t weight_rows);
 
 // Q4_K in the tile-major layout (32 output columns x one super-block per 4608-byte tile; columns
 // past out_dim zero): size, repack from the raw GGUF bytes, the MFMA GEMV for any number of
@@ -150,7 +150,7 @@ size_t gemm_q4k_workspace_bytes(size_t rows, size_t in_dim, size_t out_dim);
 hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, void* workspace,
                                  int rows, int in_dim, int out_dim, const Epilogue& ep = Epilogue{}, bool split = true);
 hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
-                                            size_t rows, int dim);
+                                            size_t rows, int dim, size_t weight_rows);
 
 // The one-row Q4_0 decode kernel with parts left out (bit 0: the block dots, bit 1: the store of Y,
 // bit 2: the activation prologue): timing diagnostics, results meaningless.  in_dim <= 4096.

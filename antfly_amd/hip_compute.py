@@ -281,6 +281,11 @@ class HipCompute:
         return self.linearNoBias(input, weight, rows, in_dim, out_dim)
 
     # -- counters ------------------------------------------------------------
+    def setPhaseTiming(self, enabled: bool) -> None:
+        """Opt-in device time per phase (activation quantizer / compute) in debugStats(); every
+        linear op then waits for its own events, so this is for debugging runs only."""
+        check(_lib.lib().afhip_compute_set_phase_timing(self._h, 1 if enabled else 0))
+
     def debugStats(self) -> dict:
         s = _lib.DebugStats()
         check(_lib.lib().afhip_compute_debug_stats(self._h, C.byref(s)))

@@ -248,8 +248,10 @@ afhip_status afhip_launch_linear_argmax_last_row_f32(void *stream, int tensor_ty
  * dequantized rows ids[t] of a [vocab, dim] table, w = d * f32(q)
  * (gguf/quant_codec.zig:1877-1895, :1918-1942).  tensor_type AFHIP_TYPE_F32 gathers
  * from a dense table.  ids_i64: `total` little-endian int64 on the device, every one
- * in [0, vocab) -- the backend op checks them on the host as the reference does; the
- * launcher cannot.  dim % 32 != 0 for a quantized table -> AFHIP_ERR_INVALID_STATE. */
+ * in [0, vocab) -- the backend op checks them on the host as the reference does
+ * (AFHIP_ERR_INVALID_TOKEN_ID); the launcher cannot, so its kernels check: a row whose id is
+ * outside [0, vocab) reads nothing and comes out as zeros.  dim % 32 != 0 for a quantized
+ * table -> AFHIP_ERR_INVALID_STATE. */
 afhip_status afhip_launch_embedding_lookup_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
                                                afhip_buffer weight, afhip_buffer ids_i64, size_t total,
                                                size_t dim, size_t vocab);
@@ -259,7 +261,10 @@ afhip_status afhip_launch_dequantize_f32(void *stream, int tensor_type, int layo
 /* cpy_f32_to_q (row_ids_i64.ptr == 0: rows in order, dst_rows == rows) and set_rows
  * (row t of `input` becomes row row_ids[t] of the [dst_rows, dim] destination): f32 ->
  * raw GGUF blocks with the engine's weight quantizers (gguf/quant_codec.zig:601-623
- * Q8_0, :895-910 and :1261-1265 Q4_0).  dst_raw must be 2-byte aligned. */
+ * Q8_0, :895-910 and :1261-1265 Q4_0).  dst_raw must be 2-byte aligned.  set_rows
+ * preconditions: a row id outside [0, dst_rows) writes nothing (the row is skipped); two
+ * rows with the same id race and either may win -- give every destination row at most
+ * once. */
 afhip_status afhip_launch_quantize_rows(void *stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
                                         afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows);
 
@@ -556,8 +561,17 @@ typedef struct afhip_debug_stats {
     uint64_t h2d_bytes, d2h_bytes, resident_weight_bytes, pooled_buffers, device_allocs;
     uint64_t launches_mmv, launches_small_batch, launches_mm, launches_f32_route;
     uint64_t launches_activation_quant, launches_prepare, scratch_bytes;
+    /* Device time per phase of the linear ops, in nanoseconds, summed over `timed_ops` ops
+     * (QuantExecutionTimingStats' activation-quantization and compute phases, ops/ops.zig:649-713):
+     * zero unless afhip_compute_set_phase_timing switched it on. */
+    uint64_t activation_quant_ns, compute_ns, timed_ops;
 } afhip_debug_stats;
 afhip_status afhip_compute_debug_stats(const afhip_compute *self, afhip_debug_stats *out);
+/* Opt-in phase timing for debugging: while enabled every linear op records HIP events around its
+ * stand-alone activation quantizer and around its compute kernels on the backend's stream and
+ * waits for them before it returns (so it serializes host and device: not for production runs).
+ * A kernel that quantizes activations in its own prologue counts entirely as compute. */
+afhip_status afhip_compute_set_phase_timing(afhip_compute *self, int enabled);
 
 /* Known-answer smokes run entirely inside the library on device 0
  * (ops/cuda/kernels.zig:2309-2399, driven by `cuda-info --smoke`,

@@ -277,3 +277,30 @@ def test_gguf_file_to_device_weights(cb, tmp_path):
     nt = cb.getWeight("blk.0.ffn_norm.weight")
     assert nt.dtype == _lib.DTYPE_F32 and nt.shape == [in_dim]
     assert np.array_equal(cb.toFloat32(nt), norm)
+
+
+def test_phase_timing_is_opt_in(cb):
+    """afhip_compute_set_phase_timing: device time of the stand-alone activation quantizer and of
+    the compute kernels per linear op (the engine's timing snapshot, ops/ops.zig:649-713)."""
+    in_dim, out_dim = 1024, 768
+    w = synth.weights(_lib.TYPE_Q8_0, 70, out_dim, in_dim)
+    cb.insertWeightFromLoaded("timed.weight", _lib.TYPE_Q8_0, w, [out_dim, in_dim])
+    wt = cb.getWeight("timed.weight")
+    x = synth.activations(71, 24, in_dim)
+    xt = cb.fromFloat32(x, [24, in_dim])
+    cb.freeTensor(cb.linearNoBias(xt, wt, 24, in_dim, out_dim))
+    s0 = cb.debugStats()
+    assert s0["timed_ops"] == 0 and s0["activation_quant_ns"] == 0 and s0["compute_ns"] == 0
+    cb.setPhaseTiming(True)
+    y = cb.toFloat32(cb.linearNoBias(xt, wt, 24, in_dim, out_dim)).reshape(24, out_dim)  # quantizer + MFMA GEMM
+    s1 = cb.debugStats()
+    assert s1["timed_ops"] == 1 and s1["activation_quant_ns"] > 0 and s1["compute_ns"] > 0
+    x1 = cb.fromFloat32(x[:1], [1, in_dim])
+    cb.freeTensor(cb.linearNoBias(x1, wt, 1, in_dim, out_dim))  # one row: quantized in the kernel's prologue
+    s2 = cb.debugStats()
+    assert s2["timed_ops"] == 2 and s2["compute_ns"] > s1["compute_ns"]
+    cb.setPhaseTiming(False)
+    cb.freeTensor(cb.linearNoBias(xt, wt, 24, in_dim, out_dim))
+    assert cb.debugStats()["timed_ops"] == 2
+    ref = O.linear_no_bias(_lib.TYPE_Q8_0, x, w, 24, in_dim, out_dim, workers=8)
+    assert G.max_rel_err(y, ref.astype(np.float64)) <= 2e-5

@@ -183,3 +183,38 @@ def test_backend_embedding_lookup(kats):
         cb.insertWeightFromTensor("pos_embd", dense, [20, 48])
         out = cb.embeddingLookup(cb.getWeight("pos_embd"), [19, 0], 2, 48)
         assert np.array_equal(cb.toFloat32(out).reshape(2, 48), dense[[19, 0]])
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_row_ids_outside_the_tensor_touch_nothing(fmt):
+    """get_rows: an id outside [0, vocab) comes out as a row of zeros; set_rows: a row id outside
+    [0, dst_rows) is skipped.  Neither reads nor writes outside the tensors (the kernels check:
+    the launcher has no way to)."""
+    vocab, dim = 12, 256
+    w = synth.weights(fmt, 61, vocab, dim)
+    ids = np.array([3, -1, vocab, 11, 1 << 40], dtype=np.int64)
+    for layout in (RAW, PREP):
+        wd = G.prepare(fmt, w, vocab, dim) if layout == PREP else G.to_dev(w)
+        out = torch.full((ids.size, dim), float("nan"), dtype=torch.float32, device=G.DEV)
+        ids_d = G.to_dev(ids)
+        kernels.launchEmbeddingLookupF32(G.stream(), fmt, layout, G.buf(out), G.buf(wd), G.buf(ids_d), ids.size, dim, vocab)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        dense = O.dequantize(fmt, w).reshape(vocab, dim)
+        assert np.array_equal(got[0], dense[3]) and np.array_equal(got[3], dense[11])
+        assert not got[[1, 2, 4]].any()
+    # set_rows into a 6-row destination guarded by canaries on both sides
+    dst_rows, bb = 6, (18 if fmt == Q4 else 34)
+    row_bytes = dim // 32 * bb
+    x = synth.activations(62, 4, dim)
+    canvas = torch.full(((dst_rows + 2) * row_bytes,), 0xAB, dtype=torch.uint8, device=G.DEV)
+    dst = canvas[row_bytes : (dst_rows + 1) * row_bytes]
+    rid = np.array([5, -2, dst_rows, 0], dtype=np.int64)
+    x_d, rid_d = G.to_dev(x), G.to_dev(rid)  # (kept alive until the launch has run)
+    kernels.launchQuantizeRows(G.stream(), fmt, G.buf(dst), G.buf(x_d), 4, dim, row_ids_i64=G.buf(rid_d), dst_rows=dst_rows)
+    torch.cuda.synchronize()
+    got = canvas.cpu().numpy().reshape(dst_rows + 2, row_bytes)
+    want = O.quantize_weights(fmt, x).reshape(4, row_bytes)
+    assert np.array_equal(got[1 + 5], want[0]) and np.array_equal(got[1 + 0], want[3])
+    untouched = [0, 2, 3, 4, 5, dst_rows + 1]  # canaries and the rows nobody addressed
+    assert (got[untouched] == 0xAB).all()

@@ -17,14 +17,23 @@ PREP = _lib.LAYOUT_PREPARED
 
 
 def static_linear(fmt, x, w_dev, rows, in_dim, out_dim):
+    """One eager call, then the same call recorded into a HIP graph and replayed: a library that
+    allocated device memory inside the call could not be captured (hipMalloc is refused while a
+    stream is capturing)."""
     xd = G.to_dev(x.astype(np.float32))
     y = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=G.DEV)
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
     kernels.launchLinearF32Static(G.stream(), fmt, PREP, G.buf(y), G.buf(xd), G.buf(w_dev), rows, in_dim, out_dim)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
-    return y.cpu().numpy()
+    eager = y.cpu().numpy()
+    y.fill_(float("nan"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        kernels.launchLinearF32Static(torch.cuda.current_stream().cuda_stream, fmt, PREP, G.buf(y), G.buf(xd), G.buf(w_dev), rows,
+                                      in_dim, out_dim)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert np.array_equal(y.cpu().numpy(), eager)
+    return eager
 
 
 @pytest.mark.parametrize("fmt", [Q4, Q8])
