@@ -236,8 +236,13 @@ afhip_status parse_into(afhip_gguf* g) {  // format.parse, :113-161
         if (afhip_status s = c.read_int(&t.offset); s != AFHIP_OK) return s;
         g->tensors.push_back(std::move(t));
     }
-    g->data_region_offset = align_forward(c.pos, g->alignment);
-    for (TensorInfo& t : g->tensors) t.data_offset = g->data_region_offset + t.offset;
+    // file-supplied alignment and offsets: sums that wrap 64 bits would pass the bounds check in
+    // afhip_gguf_tensor_data with the wrong bytes, so they are refused here
+    const uint64_t aligned = align_forward(c.pos, g->alignment);
+    if (aligned < c.pos) return AFHIP_ERR_GGUF_UNEXPECTED_EOF;
+    g->data_region_offset = aligned;
+    for (TensorInfo& t : g->tensors)
+        if (__builtin_add_overflow(g->data_region_offset, t.offset, &t.data_offset)) return AFHIP_ERR_GGUF_UNEXPECTED_EOF;
     return AFHIP_OK;
 }
 

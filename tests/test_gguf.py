@@ -121,6 +121,13 @@ def test_parser_errors():
             f.tensorData("w")
         with pytest.raises(_lib.TensorNotFound):
             f.tensorData("nope")
+    # a tensor offset that wraps 64 bits when the data region's start is added would land back inside the image
+    with gguf.File.parse(img) as f:
+        region = f.data_region_offset
+    at = img.index(W.le("I", 8) + W.le("Q", 0)) + 4       # the offset field of "w" (type 8, offset 0)
+    for offset in (2 ** 64 - region, 2 ** 64 - region + 32, 2 ** 64 - 1):
+        with pytest.raises(_lib.UnexpectedEndOfFile):
+            gguf.File.parse(img[:at] + W.le("Q", offset) + img[at + 8:])
 
 
 def test_truncated_and_corrupted_images_fail_cleanly():
