@@ -134,6 +134,7 @@ SIGNATURES = {
     "afhip_launch_quantize_rows": (_st, [_vp, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
+    "afhip_launch_stream_copy": (_st, [_vp, Buffer, Buffer]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),
     "afhip_compute_destroy": (None, [_vp]),
     "afhip_compute_backend_kind": (_i, [_vp]),

@@ -810,6 +810,15 @@ afhip_status afhip_launch_stream_read(void* stream, afhip_buffer src, afhip_buff
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_stream_copy(void* stream, afhip_buffer src, afhip_buffer dst) {
+    if (src.len / 16 > 0xffffffffull * 256 || dst.len < src.len / 16 * 16) return AFHIP_ERR_INVALID_STATE;
+    if (src.len < 16) return AFHIP_OK;
+    if (src.ptr == 0 || src.ptr % 16 != 0 || dst.ptr == 0 || dst.ptr % 16 != 0) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_stream_copy(static_cast<hipStream_t>(stream), reinterpret_cast<uint8_t*>(dst.ptr),
+                                      reinterpret_cast<const uint8_t*>(src.ptr), src.len);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                      size_t in_dim, size_t out_dim) {
     if (probe < 0 || probe > 7) return AFHIP_ERR_INVALID_ARGUMENT;

@@ -265,6 +265,14 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4* __
     if (x == 0x9E3779B9u && i == n16 + 1) sink[0] = x;  // never true for i < n16; keeps the loads alive
 }
 
+// The plain copy: dst[i] = src[i], 16 bytes per lane, each byte read once and written
+// once.  The kernel of known traffic that the hardware write counter is scaled against.
+__global__ __launch_bounds__(256) void stream_copy_kernel(stream_u32x4* __restrict__ dst, const stream_u32x4* __restrict__ src,
+                                                          size_t n16) {
+    const size_t i = blockIdx.x * static_cast<size_t>(256) + threadIdx.x;
+    if (i < n16) dst[i] = __builtin_nontemporal_load(src + i);
+}
+
 // =====================================================================
 // Launchers
 // =====================================================================
@@ -440,6 +448,14 @@ hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* 
     if (n16 == 0) return hipSuccess;
     hipLaunchKernelGGL(stream_read_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0, stream,
                        reinterpret_cast<const stream_u32x4*>(src), sink, n16);
+    return launch_status();
+}
+
+hipError_t launch_stream_copy(hipStream_t stream, uint8_t* dst, const uint8_t* src, size_t bytes) {
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return hipSuccess;
+    hipLaunchKernelGGL(stream_copy_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0, stream,
+                       reinterpret_cast<stream_u32x4*>(dst), reinterpret_cast<const stream_u32x4*>(src), n16);
     return launch_status();
 }
 

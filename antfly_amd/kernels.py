@@ -149,6 +149,10 @@ def launchStreamRead(stream, src: Buffer, sink: Buffer) -> None:
     check(_lib.lib().afhip_launch_stream_read(stream, src, sink))
 
 
+def launchStreamCopy(stream, src: Buffer, dst: Buffer) -> None:
+    check(_lib.lib().afhip_launch_stream_copy(stream, src, dst))
+
+
 def smokeQ8_0() -> None:
     check(_lib.lib().afhip_smoke_q8_0())
 

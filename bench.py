@@ -69,7 +69,7 @@ def main() -> int:
                     help="the timed region (exactly --steps steps) is run this many times; the median run is reported")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
-                         "read kernel over the same number of bytes, of the Q8_0 M=512 GEMM and of the Q4_K kernels "
+                         "read kernel and of the plain copy kernel over the same number of bytes, of the Q8_0 M=512 GEMM and of the Q4_K kernels "
                          "(M=1 and M=512), then exit")
     ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048"], default=None,
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
@@ -428,6 +428,9 @@ def main() -> int:
         for i in range(n_launch):
             _lib.lib().afhip_launch_stream_read(stream, buf(srcs[i % copies]), buf(sink))
         torch.cuda.synchronize()
+        for i in range(n_launch):  # the plain copy: the same bytes read once and written once
+            _lib.lib().afhip_launch_stream_copy(stream, buf(srcs[i % copies]), buf(srcs[(i + copies // 2) % copies]))
+        torch.cuda.synchronize()
         wg = prepared_copies(Q8, 4096, 4096, 2, 7)
         xg = torch.from_numpy(synth.activations(8, 512, 4096)).to(dev)
         yg = torch.empty((512, 4096), dtype=torch.float32, device=dev)
@@ -445,7 +448,8 @@ def main() -> int:
                 launch(stream, Q4K, _lib.LAYOUT_PREPARED, buf(yk), buf(xk), buf(wk[i % copies]), m, 4096, 14336, buf(sk), -1)
             torch.cuda.synchronize()
         print(json.dumps({"counter_probe": {"launches_each": n_launch, "gemv_bytes": gemv_bytes(Q4, 1, 4096, 14336),
-                                            "stream_read_bytes": w_bytes}}))
+                                            "stream_read_bytes": w_bytes,
+                                            "stream_copy_bytes": w_bytes}}))
         return 0
 
     # ---- headline: Q4_0 decode GEMV, M=1, K=4096, N=14336 --------------------------

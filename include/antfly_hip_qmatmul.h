@@ -309,6 +309,11 @@ afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_
  * beside the GEMV as "what one launch of this size can draw from HBM", and it is
  * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
 afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
+/* Diagnostic with no counterpart in the reference: the plain copy, dst[0 .. src.len) =
+ * src (16 bytes per lane; src.len is rounded down to a multiple of 16, both pointers
+ * 16-byte aligned, dst.len >= the copied length).  The kernel of known traffic that
+ * WRITE_SIZE readings are scaled against. */
+afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buffer dst);
 /* Diagnostic with no counterpart in the reference: the one-row Q4_0 decode GEMV (PREPARED
  * weight, in_dim <= 4096) with parts left out -- `probe` bit 0: the block dots, bit 1: the
  * store of Y, bit 2: the activation prologue (no X read, no quantization).  probe 0 is the

@@ -218,3 +218,20 @@ def test_row_ids_outside_the_tensor_touch_nothing(fmt):
     assert np.array_equal(got[1 + 5], want[0]) and np.array_equal(got[1 + 0], want[3])
     untouched = [0, 2, 3, 4, 5, dst_rows + 1]  # canaries and the rows nobody addressed
     assert (got[untouched] == 0xAB).all()
+
+
+@pytest.mark.parametrize("nbytes", [16, 4096 + 16, 1 << 20, (1 << 20) + 7])
+def test_stream_copy_copies_whole_16_byte_units(nbytes):
+    """The diagnostic copy kernel (the calibrator of the write counter): dst = src over the
+    whole 16-byte units of src.len, nothing past them, and a too-short dst is refused."""
+    print(f"case: stream_copy nbytes={nbytes}", flush=True)
+    rng = np.random.default_rng(nbytes)
+    src = G.to_dev(rng.integers(0, 256, nbytes + 16, dtype=np.uint8))
+    dst = torch.full((nbytes + 64,), 0xAB, dtype=torch.uint8, device="cuda")
+    kernels.launchStreamCopy(G.stream(), _lib.Buffer(src.data_ptr(), nbytes), G.buf(dst))
+    torch.cuda.synchronize()
+    n = nbytes // 16 * 16
+    assert torch.equal(dst[:n], src[:n])
+    assert bool((dst[n:] == 0xAB).all())
+    with pytest.raises(_lib.HipError):
+        kernels.launchStreamCopy(G.stream(), _lib.Buffer(src.data_ptr(), nbytes), _lib.Buffer(dst.data_ptr(), n - 16))
