@@ -833,6 +833,15 @@ afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, 
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_rate_probe(void* stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink) {
+    if (pattern < 0 || pattern > 11 || wavefronts_per_simd < 1 || wavefronts_per_simd > 8 || iterations < 1 || iterations > (1 << 20))
+        return AFHIP_ERR_INVALID_ARGUMENT;
+    if (sink.ptr == 0 || sink.ptr % 4 != 0 || sink.len < 65536 * 4) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_rate_probe(static_cast<hipStream_t>(stream), pattern, wavefronts_per_simd, iterations,
+                                     reinterpret_cast<int*>(sink.ptr));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {
     size_t dst_bytes, src_bytes;
     if (!checked_mul(n, 4, &dst_bytes) || !checked_mul(n, 2, &src_bytes) || dst_bytes > dst.len || src_bytes > src.len)

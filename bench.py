@@ -75,8 +75,8 @@ def main() -> int:
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k): time only these calls, print one line each, exit")
-    ap.add_argument("--probe", choices=["gemv"], default=None,
-                    help="gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+    ap.add_argument("--probe", choices=["gemv", "rates"], default=None,
+                    help="rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -359,6 +359,54 @@ def main() -> int:
         w_s, e_s = time_config(Q8, m, 4096, 4096, 200, 20, 4, 7, repeats=1)
         print(json.dumps({"only": args.only, "us_per_op": round(e_s / 200 * 1e6, 3),
                           "TOPS": round(2.0 * m * 4096 * 4096 * 200 / e_s / 1e12, 2)}))
+        return 0
+
+    if args.probe == "rates":
+        lib = _lib.lib()
+        sink = torch.zeros(65536, dtype=torch.int32, device=dev)
+        iterations = 4000
+        clock_ghz = 2.4  # MI355X peak engine clock; the clock a run really holds is not read here
+        patterns = [(0, "v_fma_f32 x 16", 16), (1, "v_mul_f32 x 16", 16), (2, "v_add_u32 x 16", 16), (3, "v_cvt_f32_i32 x 16", 16),
+                    (4, "v_dot8_u32_u4 x 16", 16), (5, "v_dot8_i32_i4 x 16", 16), (6, "v_dot4_i32_i8 x 16", 16),
+                    (7, "v_mfma_i32_32x32x32_i8 x 4", 4), (8, "4 x (MFMA + 4 v_fma_f32), one wavefront", 4),
+                    (9, "4 x (MFMA + 8 v_fma_f32), one wavefront", 4)]
+        mixed = [(7, 1, "MFMA x 4 alone, 1 wavefront per SIMD"), (0, 1, "v_fma_f32 x 16 alone, 1 wavefront per SIMD"),
+                 (3, 1, "v_cvt_f32_i32 x 16 alone, 1 wavefront per SIMD"),
+                 (10, 2, "a wavefront of MFMA x 4 beside a wavefront of v_fma_f32 x 16 on each SIMD"),
+                 (11, 2, "a wavefront of MFMA x 4 beside a wavefront of v_cvt_f32_i32 x 16 on each SIMD"),
+                 (7, 2, "MFMA x 4, 2 wavefronts per SIMD")]
+
+        def run(pattern, waves):
+            times = []
+            for _ in range(4):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                rc = lib.afhip_launch_rate_probe(stream, pattern, waves, iterations, buf(sink))
+                e1.record()
+                torch.cuda.synchronize()
+                if rc != 0:
+                    raise RuntimeError(f"rate probe failed: {rc}")
+                times.append(e0.elapsed_time(e1))
+            return sorted(times[1:])[1]  # ms; the first launch is warm-up
+
+        print(f"shader clock taken as {clock_ghz:.2f} GHz (the published peak engine clock); {iterations} rounds per wavefront")
+        print("| pattern (one round) | wavefronts per SIMD | ms | cycles per round and wavefront | cycles per instruction and SIMD |")
+        print("|---|---|---|---|---|")
+        out = {}
+        for pattern, name, per_round in patterns:
+            for waves in (1, 2, 4):
+                ms = run(pattern, waves)
+                per_wave_round = ms * 1e6 * clock_ghz / iterations
+                print(f"| {name} | {waves} | {ms:.3f} | {per_wave_round:.1f} | {per_wave_round / waves / per_round:.2f} |")
+                out[f"{name} @{waves}"] = round(ms, 4)
+        print()
+        print("| two kinds of wavefront on a SIMD | ms |")
+        print("|---|---|")
+        for pattern, waves, name in mixed:
+            ms = run(pattern, waves)
+            print(f"| {name} | {ms:.3f} |")
+            out[name] = round(ms, 4)
+        print(json.dumps({"probe": "rates", "ms": out}))
         return 0
 
     if args.probe == "gemv":

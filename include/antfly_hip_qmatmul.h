@@ -321,6 +321,15 @@ afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buff
  * --probe gemv times the eight variants to show where a launch's time goes. */
 afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* Diagnostic with no counterpart in the reference: instruction issue rates.  Puts
+ * `wavefronts_per_simd` (1..8) wavefronts on every SIMD, each running `iterations` rounds of
+ * pattern 0..6 (16 independent v_fma_f32 / v_mul_f32 / v_add_u32 / v_cvt_f32_i32 /
+ * v_dot8_u32_u4 / v_dot8_i32_i4 / v_dot4_i32_i8), 7 (four v_mfma_i32_32x32x32_i8), 8 / 9 (four
+ * times one MFMA followed by 4 / 8 independent v_fma_f32 in the same wavefront) or 10 / 11
+ * (alternate workgroups run pattern 7 and pattern 0 / 3: with two wavefronts per SIMD, one that
+ * only issues MFMAs beside one that only issues vector-ALU work).  `sink` takes 256 KiB of
+ * meaningless results.  `bench.py --probe rates` times it. */
+afhip_status afhip_launch_rate_probe(void *stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink);
 
 /* ------------------------------------------------------------------------
  * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
