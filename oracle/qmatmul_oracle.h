@@ -7,7 +7,13 @@
  * Reference files are cited as INF = zig/pkg/inference/src in the reference
  * tree.  Every function here is pinned by the reference's own known-answer
  * tests (re-encoded under tests/golden/) plus closed forms / brute force in
- * tests/test_oracle_*.py; no function is "parity unpinned".
+ * tests/test_oracle_*.py; no function here is "parity unpinned".
+ *
+ * Not restated here, hence parity unpinned for it: the engine's Q8_K
+ * activation-quantized route for Q4_K (INF/ops/native_compute.zig:3468-3479,
+ * :32031-32049), taken only for in_dim in {512, 768, 1536, 2048, 3072} with
+ * out_dim >= 512 and a fixed list of row counts.  The Q4_K functions below follow
+ * the engine's f32 route, which is what it computes at every other shape.
  */
 #ifndef ANTFLY_QMATMUL_ORACLE_H
 #define ANTFLY_QMATMUL_ORACLE_H
