@@ -77,6 +77,8 @@ static WorkspaceView workspace_view(uint64_t base, size_t rows, size_t in_dim) {
 // two rows of any length, and for three or four rows of Q4_0 up to this many 32-value
 // blocks of X; beyond, a separate kernel quantizes X once.
 constexpr size_t kGemvFusedQuantBlocks = 512;
+// fewest rows served by the single-shot MFMA kernel (batch_mfma_kernels.hip)
+constexpr size_t kBatchMfmaMinRows = 5;
 
 // LDS the GEMV may use per workgroup; gfx950 has 160 KiB per CU.  The larger figure is
 // for up to eight rows of a long K (8 x 14336): one workgroup per CU then, but the
@@ -99,6 +101,23 @@ static int gemv_row_chunk(size_t rows, size_t in_dim) {
 static int env_int(const char* name) {
     const char* v = std::getenv(name);
     return v && *v ? std::atoi(v) : 0;
+}
+
+// Whether the single-shot MFMA kernel serves this shape (measured against the kernels it replaces;
+// AFHIP_BATCH_MFMA_MIN_ROWS overrides the lower row bound for tuning runs, 0 switches the kernel off):
+// from five rows on (six on a K longer than 4096, where the split-K GEMV still wins at five), and for
+// Q8_0, whose K shares are half as long, only while all workgroups of the launch are resident at once.
+static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    static const char* v = std::getenv("AFHIP_BATCH_MFMA_MIN_ROWS");
+    static const long forced = v && *v ? std::atol(v) : -1;
+    if (forced == 0 || rows > 64 || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
+    if (forced > 0) return rows >= static_cast<size_t>(forced);
+    if (rows < (in_dim > 4096 ? kBatchMfmaMinRows + 1 : kBatchMfmaMinRows)) return false;
+    if (tensor_type == AFHIP_TYPE_Q8_0) {
+        const size_t shares = (in_dim / 32 + 63) / 64, tiles = (out_dim + 31) / 32;
+        return shares == 1 || tiles * shares <= 2 * static_cast<size_t>(gemv_compute_units());
+    }
+    return true;
 }
 
 static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t out_dim) {
@@ -287,6 +306,26 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
     const int chunk = gemv_row_chunk(rows, in_dim);
     const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR &&
                           in_dim <= static_cast<size_t>(gemv_fused_max_in_dim());
+    // Five to 64 rows: the weights are read once, so the single-shot MFMA kernel (X quantized into
+    // MFMA operand order first) beats both the row-by-row GEMV and the tiled GEMM.
+    if (layout == AFHIP_LAYOUT_PREPARED && !want_dots && kind != AFHIP_DISPATCH_SCALAR &&
+        batch_mfma_preferred(tensor_type, rows, in_dim, out_dim)) {
+        const size_t need = batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim);
+        if (workspace.ptr == 0 || workspace.len < need || workspace.ptr % 16 != 0) return AFHIP_ERR_INVALID_STATE;
+        if (counters) {
+            if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+            else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+            else counters->mm++;
+            if (pair) {
+                if (kind == AFHIP_DISPATCH_MM) counters->mm++;
+            }
+            counters->activation_quant++;
+        }
+        hipError_t e = launch_batch_mfma(stream, tensor_type, y, x, w, static_cast<int>(rows), static_cast<int>(in_dim),
+                                         static_cast<int>(out_dim), reinterpret_cast<uint8_t*>(workspace.ptr), pair ? y_b : nullptr,
+                                         pair ? w_b : nullptr, ep, ep_b);
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     if (layout == AFHIP_LAYOUT_PREPARED && kind == AFHIP_DISPATCH_MM) {
         // rows >= 9 (or a plan that asks for mul_mm): quantize X once, then the int8-MFMA GEMM
         const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
@@ -631,7 +670,10 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
     const size_t gemm_bytes = partial != 0 ? (base + 255) / 256 * 256 + partial : base;
     // small batches on a long K (also slices of eight rows of a forced plan): the K slices' sums, for a pair of matrices
     const size_t batch_bytes = gemv_batch_partial_bytes(rows < 8 ? rows : 8, in_dim, out_dim, true);
-    return gemm_bytes > batch_bytes ? gemm_bytes : batch_bytes;
+    // up to 64 rows: X in MFMA operand order and the partial sums of K shares of the single-shot MFMA kernel
+    const size_t mfma_bytes = rows <= 64 ? batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim) : 0;
+    size_t need = gemm_bytes > batch_bytes ? gemm_bytes : batch_bytes;
+    return need > mfma_bytes ? need : mfma_bytes;
 }
 
 afhip_status afhip_launch_linear_f32(void* stream, int tensor_type, int layout, afhip_buffer dst, afhip_buffer input,

@@ -1,0 +1,408 @@
+// Batched decode (a few to 64 rows) on CDNA4 int8 MFMA, activation-quantized route
+// (ops/native_compute.zig:13304-13478 for Q8_0, :23427-23775 for Q4_0):
+//   dot[m][n][b] = sum_i qx[m][32b+i] * qw[n][32b+i]            (int32, exact)
+//   y[m][n]      = sum_b (sx[m][b] * sw[n][b]) * f32(dot[m][n][b])
+//
+// With so few rows the weights are read once and nothing is reused across workgroups, so the
+// kernel is built like the decode GEMV, not like the prefill GEMM: single shot, no ring, no
+// barrier inside the K loop.
+//   * A workgroup of eight wavefronts owns 32 output columns and one share of K of at most
+//     8 * kWaveBlocks blocks; wavefront w owns kWaveBlocks consecutive blocks of it (16 Q4_0 /
+//     8 Q8_0: 8 KB of quant bytes).  It requests ALL its weight bytes at once with eight
+//     global_load_lds_dwordx4 into its own 8 KB of LDS -- whole 128-byte lines, eight lanes per
+//     line, chunk slots XOR-swizzled by the column so that the later fragment reads of 16
+//     consecutive columns hit 16 different bank groups.  The LDS region is private to the
+//     wavefront: no barrier before it is read.
+//   * The activations were quantized beforehand into MFMA operand order
+//     (quantize_fragments_kernel): the A fragment of 32 rows and one block is 1 KB contiguous,
+//     lane l holding bytes [16 * (l / 32), +16) of row l % 32, so a wavefront takes it with one
+//     coalesced 16-byte load per lane, straight into registers.  Rows past `rows` are zeros.
+//   * Per block: v_mfma_i32_32x32x32_i8 gives the 32 x 32 int32 dots.  Q4_0 nibbles never become
+//     separate bytes: with bit 3 flipped and placed in the high half of a byte a nibble n reads as
+//     the int8 16 * (n - 8) (three operations per dword), so the MFMA yields 16 * dot exactly and
+//     the weight scale is taken times 1/16 (a power of two: exact).  The scale products
+//     sx[m][b] * sw[n][b] of two blocks come from one v_mfma_f32_32x32x1_2b_f32 (two rank-1
+//     products, each entry the correctly rounded f32 product), then one convert and one fused
+//     multiply-add per live result register and block.  Only the registers of rows that exist
+//     are touched (kLive of 16: 4 for up to 8 rows, 8 for up to 16, ...).
+//   * The eight wavefronts' sums meet in LDS in wavefront order (y is a fixed-order sum of eight
+//     block-ascending partial sums); K shares of a long K go to partial[share][rows][out_dim]
+//     and splitk_reduce_kernel adds them in share order.
+#include <hip/hip_runtime.h>
+
+#include "device_common.h"
+#include "gemv_common.h"
+#include "qmatmul_launch.h"
+
+namespace afhip {
+
+namespace {
+
+typedef int bm_v4i __attribute__((ext_vector_type(4)));
+typedef int bm_v16i __attribute__((ext_vector_type(16)));
+typedef float bm_v32f __attribute__((ext_vector_type(32)));
+
+constexpr int kBmWaves = 8;
+constexpr int kBmThreads = 64 * kBmWaves;
+constexpr int kBmWaveBytes = 8192;  // quant bytes one wavefront owns: 32 columns x kWaveBlocks blocks
+constexpr int kBmLdsBytes = kBmWaves * kBmWaveBytes;
+
+template <int kType>
+struct BmFormat {
+    static constexpr int kQuantBytes = kType == 2 ? 16 : 32;
+    static constexpr int kWaveBlocks = kBmWaveBytes / (32 * kQuantBytes);  // 16 (Q4_0) / 8 (Q8_0)
+    static constexpr int kShareBlocks = kBmWaves * kWaveBlocks;            // 128 / 64
+};
+
+// One 64-lane load from global memory straight into LDS: lane l's 16 bytes at base + voff land
+// at lds_addr + 16 * l.  Inline assembly: the compiler does not track these loads, which is why
+// the kernel waits for them by hand before anything reads the LDS region.
+__device__ __forceinline__ void bm_lds_load16(const void* base, uint32_t voff, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+}
+
+extern __shared__ __align__(16) unsigned char bm_lds[];
+
+// Program-order fence for the compiler (no instruction): what was computed into `a` so far is
+// finished before anything behind the fence starts.  Keeps the scheduler from running the MFMAs of
+// several blocks ahead and holding all their results in registers.
+__device__ __forceinline__ void fence_registers(float (&a)[4]) {
+    asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]));
+}
+__device__ __forceinline__ void fence_registers(float (&a)[8]) {
+    asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]));
+}
+__device__ __forceinline__ void fence_registers(float (&a)[12]) {
+    asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]), "+v"(a[8]),
+                 "+v"(a[9]), "+v"(a[10]), "+v"(a[11]));
+}
+__device__ __forceinline__ void fence_registers(float (&a)[16]) {
+    asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]), "+v"(a[8]),
+                 "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]), "+v"(a[15]));
+}
+
+}  // namespace
+
+// X f32 [rows][in_dim] -> qa: [row tile][block][64 lanes][16 bytes] (lane = 32 * half + row % 32:
+// bytes [16 * half, +16) of the block's 32 int8), sa: f32 [block][32 * row_tiles].  Rows past
+// `rows` get zeros and scale 0.  Eight lanes per block as in quantize_activations_kernel
+// (ops/native_compute.zig:11998-12028): same scale, reciprocal and rounding, bit for bit.
+__global__ __launch_bounds__(256) void quantize_fragments_kernel(const float* __restrict__ x, int rows, int in_dim, int row_tiles,
+                                                                  uint32_t* __restrict__ qa, float* __restrict__ sa) {
+    const int units_per_row = in_dim >> 2, kb = in_dim >> 5, padded = row_tiles * 32;
+    const size_t units = static_cast<size_t>(padded) * units_per_row;
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const int r = static_cast<int>(u / units_per_row), c4 = static_cast<int>(u % units_per_row);
+        const int b = c4 >> 3, j = c4 & 7;
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (r < rows) v = reinterpret_cast<const float4*>(x)[static_cast<size_t>(r) * units_per_row + c4];
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        const float s = act_scale(m);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
+        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+        const size_t lane_entry = (static_cast<size_t>(r >> 5) * kb + b) * 64 + (j >> 2) * 32 + (r & 31);
+        qa[lane_entry * 4 + (j & 3)] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        if (j == 0) sa[static_cast<size_t>(b) * padded + r] = r < rows ? s : 0.0f;
+    }
+}
+
+template <int kType, int kRowTiles, int kLive>
+__global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma_kernel(float* __restrict__ dst, float* __restrict__ partial,
+                                                                  const uint32_t* __restrict__ qa, const float* __restrict__ sa,
+                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                                  int out_dim, int share_blocks, Epilogue ep) {
+    using F = BmFormat<kType>;
+    constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kPairs = kWB / 2;
+    constexpr int kAhead = kRowTiles == 1 ? 8 : 4;  // A fragments in registers per row tile
+    static_assert(kWB % kAhead == 0 && kAhead % 2 == 0, "fragment ring");
+    const int kb_full = in_dim >> 5;
+    const int padded = kRowTiles * 32;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lj = lane & 31, lh = lane >> 5;
+    const int n0 = blockIdx.x * 32;
+    // blocks of this wavefront: [blk0, blk0 + nb), nb in 0..kWB; indices past the end are clamped
+    // to the last valid block for every load and their scale products are forced to zero
+    const int share_begin = static_cast<int>(blockIdx.y) * share_blocks;
+    const int share_end = min(share_begin + share_blocks, kb_full);
+    const int blk0 = share_begin + wave * kWB;
+    const int nb = max(0, min(kWB, share_end - blk0));
+    const int last = blk0 + max(nb, 1) - 1 < kb_full ? blk0 + max(nb, 1) - 1 : kb_full - 1;  // a valid block whatever nb is
+    auto clamp_blk = [&](int j) { return min(blk0 + j, last); };
+
+    const size_t blocks_total = static_cast<size_t>(out_dim) * kb_full;
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(bm_lds))) + wave * kBmWaveBytes;
+
+    // ---- 1. loads.  Order matters: a wavefront's loads complete in the order they were issued,
+    // and every wavefront of the grid issues at once, so memory serves all first halves before all
+    // second halves.  First half of the weights (LDS-direct, four 1 KB loads), then what the first
+    // half of the K loop needs (A fragments, scales), then values only the second half needs, then
+    // the second half of the weights.  The compiler counts only its own loads when it waits for
+    // one: with at least four of its loads issued behind everything the first half needs, its
+    // wait lets exactly the four youngest loads -- the second half of the weights -- stay in flight
+    // while the first half is computed.  (Its count can only be too strict, never too lax: loads
+    // it does not know of only add to the number outstanding.)
+    auto issue_weights = [&](int hb) {
+        const uint8_t* wbase = weight + static_cast<size_t>(n0) * kb_full * kQB;
+        const int c8 = lane >> 3, slot = lane & 7;
+#pragma unroll
+        for (int cg = 0; cg < 4; ++cg) {
+            const int c = 8 * cg + c8;
+            const int chunk = slot ^ ((c >> 1) & 7);
+            const int cc = min(n0 + c, out_dim - 1) - n0;
+            uint32_t off;
+            if (kType == 2) {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(8 * hb + chunk)) * 16u;
+            } else {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(4 * hb + (chunk >> 1))) * 32u + (chunk & 1) * 16u;
+            }
+            bm_lds_load16(wbase, off, lds_wave + (hb * 4 + cg) * 1024);
+        }
+    };
+    issue_weights(0);
+
+    // Rows that exist live in the first 2 * kLive lanes of each half of a fragment.  The other
+    // lanes' values only reach result rows nobody reads, so they repeat a live lane's address
+    // instead of fetching their own zeros: a fragment load then touches 2 * kLive * 32 bytes.
+    const int lr = lj % (2 * kLive);
+    const int alane = lh * 32 + lr;
+    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa);
+    auto load_a = [&](int rt, int j) { return qa4[(static_cast<size_t>(rt) * kb_full + clamp_blk(j)) * 64 + alane]; };
+    auto load_ta = [&](int rt, int p) { return sa[static_cast<size_t>(clamp_blk(2 * p + lh)) * padded + rt * 32 + lr]; };
+    bm_v4i afrag[kRowTiles][kAhead];
+    float ta[kRowTiles][kPairs];  // activation scale of row lj, block 2p + lh
+    constexpr int kHalfBlocks = kWB / 2, kHalfPairs = kPairs / 2;
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j)
+            if (j < kHalfBlocks) afrag[rt][j] = load_a(rt, j);
+    // Weight scales, fp16 in block order: pair p needs block 2p + lh = half lh of dword p of the
+    // wavefront's run of scales.  With rows of whole 16-byte runs (in_dim a multiple of 256) that is
+    // one or two 16-byte loads per lane; otherwise one 2-byte load per pair.
+    uint32_t tb_word[kPairs];
+    {
+        const int cc = min(n0 + lj, out_dim - 1);
+        const uint16_t* sw = reinterpret_cast<const uint16_t*>(weight + blocks_total * kQB) + static_cast<size_t>(cc) * kb_full;
+        if ((kb_full & 7) == 0) {
+            // (reads past the wavefront's last valid block stay inside the scale regions; those pairs count for nothing)
+            const uint4* run = reinterpret_cast<const uint4*>(sw + min(blk0, kb_full - 8));
+#pragma unroll
+            for (int q = 0; q < kPairs / 4; ++q) {
+                const uint4 v = run[q];
+                tb_word[4 * q] = v.x;
+                tb_word[4 * q + 1] = v.y;
+                tb_word[4 * q + 2] = v.z;
+                tb_word[4 * q + 3] = v.w;
+            }
+        } else {
+#pragma unroll
+            for (int p = 0; p < kPairs; ++p) tb_word[p] = static_cast<uint32_t>(sw[clamp_blk(2 * p + lh)]) * 0x10001u;
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int p = 0; p < kHalfPairs; ++p) ta[rt][p] = load_ta(rt, p);
+    // ... and what only the second half needs (at least four loads)
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int j = kHalfBlocks; j < kAhead; ++j) afrag[rt][j] = load_a(rt, j);
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int p = kHalfPairs; p < kPairs; ++p) ta[rt][p] = load_ta(rt, p);
+    static_assert(kRowTiles * ((kAhead > kHalfBlocks ? kAhead - kHalfBlocks : 0) + kPairs - kHalfPairs) >= 4 || kType == 8,
+                  "cover loads");
+    issue_weights(1);
+
+    // The first A fragment was requested behind the first half of the weights: once it is here, so
+    // are they.  (The statement makes the compiler wait for that fragment and keeps the LDS reads
+    // below it.)
+    asm volatile("" : "+v"(afrag[0][0]) : : "memory");
+
+    // this lane's fragment position inside a 1 KB load unit: column lj, chunk slot swizzled by the column
+    const int frag_unit = lj >> 3;  // cg
+    const int frag_row = (lj & 7) * 8, frag_swz = (lj >> 1) & 7;
+    const uint4* wlds = reinterpret_cast<const uint4*>(bm_lds + wave * kBmWaveBytes);
+    auto read_b = [&](int j) {
+        int li, chunk;
+        if (kType == 2) {
+            li = (j >> 3) * 4 + frag_unit;
+            chunk = j & 7;
+        } else {
+            li = (j >> 2) * 4 + frag_unit;
+            chunk = (j & 3) * 2 + lh;
+        }
+        const uint4 w = wlds[li * 64 + frag_row + (chunk ^ frag_swz)];
+        bm_v4i b;
+        if (kType == 2) {
+            // A nibble n stands for n - 8.  As the HIGH nibble of a byte, n ^ 8 reads as the int8
+            // 16 * (n - 8): flip bit 3 of every nibble, move the wanted nibbles (low = values 0..15
+            // = k half 0, high = values 16..31) to the high positions and clear the others.  The
+            // dots come out multiplied by 16, which the weight scale takes back (exactly).
+            const uint32_t sh = 4u * (1 - lh);
+            b = bm_v4i{static_cast<int>(((w.x ^ 0x88888888u) << sh) & 0xF0F0F0F0u), static_cast<int>(((w.y ^ 0x88888888u) << sh) & 0xF0F0F0F0u),
+                       static_cast<int>(((w.z ^ 0x88888888u) << sh) & 0xF0F0F0F0u), static_cast<int>(((w.w ^ 0x88888888u) << sh) & 0xF0F0F0F0u)};
+        } else {
+            b = bm_v4i{static_cast<int>(w.x), static_cast<int>(w.y), static_cast<int>(w.z), static_cast<int>(w.w)};
+        }
+        return b;
+    };
+
+    float acc[kRowTiles][kLive];
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int v = 0; v < kLive; ++v) acc[rt][v] = 0.0f;
+
+    // ---- 3. the K loop of this wavefront: pairs of blocks, no barrier
+    if (nb > 0) {
+        const bm_v16i zi = {};
+        const bm_v32f zf = {};
+#pragma unroll
+        for (int p = 0; p < kPairs; ++p) {
+            // the second half of the weights (and every fragment requested so far) has to be here
+            if (p == kHalfPairs) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+            const bool live_blk = 2 * p + lh < nb;  // a clamped re-read of the last block counts for nothing
+            const float tb = live_blk ? half_bits_to_f32(static_cast<uint16_t>(tb_word[p] >> (16 * lh))) * (kType == 2 ? 0.0625f : 1.0f) : 0.0f;
+#pragma unroll
+            for (int rt = 0; rt < kRowTiles; ++rt) {
+                const bm_v4i a0 = afrag[rt][(2 * p) % kAhead], a1 = afrag[rt][(2 * p + 1) % kAhead];
+                const bm_v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(live_blk ? ta[rt][p] : 0.0f, tb, zf, 0, 0, 0);
+                // one block after the other: the second block's dots take the registers the first one's have left
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const bm_v4i a = h == 0 ? a0 : a1, b = read_b(2 * p + h);
+                    bm_v16i c = zi;
+                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+#pragma unroll
+                    for (int v = 0; v < kLive; ++v) acc[rt][v] = __builtin_fmaf(t[16 * h + v], static_cast<float>(c[v]), acc[rt][v]);
+                    fence_registers(acc[rt]);
+                }
+                // the fragments of blocks 2p, 2p + 1 are consumed: fetch the ones kAhead blocks on
+                if (2 * p + kAhead < kWB) {
+                    afrag[rt][(2 * p) % kAhead] = load_a(rt, 2 * p + kAhead);
+                    afrag[rt][(2 * p + 1) % kAhead] = load_a(rt, 2 * p + 1 + kAhead);
+                }
+            }
+        }
+    }
+
+    // ---- 4. the wavefronts' sums meet in LDS (the weight regions are dead after the barrier)
+    __syncthreads();
+    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][rt][v][lane]
+#pragma unroll
+    for (int rt = 0; rt < kRowTiles; ++rt)
+#pragma unroll
+        for (int v = 0; v < kLive; ++v) red[((wave * kRowTiles + rt) * kLive + v) * 64 + lane] = acc[rt][v];
+    __syncthreads();
+    constexpr int kItems = kRowTiles * kLive * 64;
+    for (int i = tid; i < kItems; i += kBmThreads) {
+        float sum = red[i];
+#pragma unroll
+        for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
+        const int l = i & 63, v = (i >> 6) % kLive, rt = (i >> 6) / kLive;
+        const int m = rt * 32 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+        const int n = n0 + (l & 31);
+        if (m < rows && n < out_dim) {
+            const size_t at = static_cast<size_t>(m) * out_dim + n;
+            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+            else dst[at] = finish_output(ep, n, at, sum);
+        }
+    }
+}
+
+namespace {
+
+template <int kType, int kRowTiles, int kLive>
+hipError_t bm_launch(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
+                     int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep) {
+    const dim3 grid(static_cast<unsigned>((out_dim + 31) / 32), static_cast<unsigned>(shares)), block(kBmThreads);
+    hipLaunchKernelGGL((batch_mfma_kernel<kType, kRowTiles, kLive>), grid, block, kBmLdsBytes, stream, dst,
+                       shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep);
+    return hipGetLastError();
+}
+
+template <int kType>
+hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
+                          int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep) {
+#define AFHIP_BM(TILES, LIVE) \
+    return bm_launch<kType, TILES, LIVE>(stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, shares, share_blocks, ep)
+    if (rows <= 8) AFHIP_BM(1, 4);
+    if (rows <= 16) AFHIP_BM(1, 8);
+    if (rows <= 24) AFHIP_BM(1, 12);
+    if (rows <= 32) AFHIP_BM(1, 16);
+    AFHIP_BM(2, 16);
+#undef AFHIP_BM
+}
+
+int bm_shares(int tensor_type, int in_dim) {
+    const int share_max = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
+    return (in_dim / 32 + share_max - 1) / share_max;
+}
+
+}  // namespace
+
+bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (tensor_type != 2 && tensor_type != 8) return false;
+    if (rows < 1 || rows > 64 || in_dim == 0 || in_dim % 32 != 0 || out_dim == 0) return false;
+    // 32-bit lane offsets relative to a column tile, grid.y
+    if (in_dim > (1u << 22) || out_dim > 0x7fffffff) return false;
+    return true;
+}
+
+// Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares]
+size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return 0;
+    const size_t padded = (rows + 31) / 32 * 32;
+    const size_t shares = static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim)));
+    const size_t front = padded * in_dim + (in_dim / 32) * padded * 4;
+    return (front + 255) / 256 * 256 + (shares > 1 ? shares * rows * out_dim * 4 : 0);
+}
+
+hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
+                             int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b,
+                             const uint8_t* weight_b_prepared, const Epilogue& ep, const Epilogue& ep_b) {
+    if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim) || workspace == nullptr) return hipErrorInvalidValue;
+    const int row_tiles = (rows + 31) / 32, padded = row_tiles * 32, kb = in_dim / 32;
+    uint32_t* qa = reinterpret_cast<uint32_t*>(workspace);
+    float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(padded) * in_dim);
+    const size_t front = static_cast<size_t>(padded) * in_dim + static_cast<size_t>(kb) * padded * 4;
+    float* partial = reinterpret_cast<float*>(workspace + (front + 255) / 256 * 256);
+    {
+        const size_t units = static_cast<size_t>(padded) * (in_dim / 4);
+        size_t grid = (units + 255) / 256;
+        if (grid > 4096) grid = 4096;
+        hipLaunchKernelGGL(quantize_fragments_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
+                           row_tiles, qa, sa);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    }
+    const int shares = bm_shares(tensor_type, in_dim);
+    // equal shares, whole wavefront slices: a multiple of the blocks one wavefront owns
+    const int wave_blocks = tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks;
+    int share_blocks = (kb + shares - 1) / shares;
+    share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
+    const int real_shares = (kb + share_blocks - 1) / share_blocks;
+    const size_t count = static_cast<size_t>(rows) * out_dim;
+    for (int which = 0; which < (weight_b_prepared ? 2 : 1); ++which) {
+        float* d = which ? dst_b : dst;
+        const uint8_t* w = which ? weight_b_prepared : weight_prepared;
+        const Epilogue& e_out = which ? ep_b : ep;
+        hipError_t e = tensor_type == 2
+                           ? bm_launch_rows<2>(stream, d, partial, qa, sa, w, rows, in_dim, out_dim, real_shares, share_blocks, e_out)
+                           : bm_launch_rows<8>(stream, d, partial, qa, sa, w, rows, in_dim, out_dim, real_shares, share_blocks, e_out);
+        if (e != hipSuccess) return e;
+        if (real_shares > 1) {
+            e = launch_splitk_reduce(stream, d, partial, count, out_dim, real_shares, e_out);
+            if (e != hipSuccess) return e;
+        }
+    }
+    return hipSuccess;
+}
+
+}  // namespace afhip

@@ -82,6 +82,18 @@ hipError_t launch_gemv_batch(hipStream_t stream, int tensor_type, float* dst, in
 int gemv_batch_waves(int rows, int in_dim, int groups);
 size_t gemv_batch_partial_bytes(size_t rows, size_t in_dim, size_t out_dim, bool pair);
 
+// Batched decode on int8 MFMA, 1..64 rows, PREPARED weights (batch_mfma_kernels.hip): quantizes X
+// into MFMA operand order in `workspace` (batch_mfma_workspace_bytes() bytes, 16-byte aligned), then one
+// single-shot launch per matrix (+ splitk_reduce_kernel when K exceeds one share).
+// compute units of the current device (cached)
+int gemv_compute_units();
+bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
+size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
+hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
+                             int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b = nullptr,
+                             const uint8_t* weight_b_prepared = nullptr, const Epilogue& ep = Epilogue{},
+                             const Epilogue& ep_b = Epilogue{});
+
 // One row, no Y: every workgroup leaves the argmax key (see argmax_key) of its output
 // columns in keys[workgroup]; *key_count receives the number of workgroups, which is at
 // most (out_dim + 1) / 2.  launch_argmax_keys turns the keys into the token.

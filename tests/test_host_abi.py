@@ -128,31 +128,49 @@ def test_q4_k_prefill_workspace_sizes():
     assert kernels.workspaceBytes(Q4K, 13, 4096, 4096) > 13 * 4096 * 6 + 13 * 16 * 64
 
 
-def test_int8_gemm_workspace_has_room_for_k_shares():
-    """Nine rows and more on a grid too small for the chip: behind the quantized activations the
-    scratch holds the partial sums of 2, 4 or 8 K shares (at least 16 blocks each); a grid that
-    fills the chip asks for the quantized activations only.  Up to eight rows (and eight-row
-    slices of a forced plan) on a K longer than 4096 need the sums of the K slices of the
-    small-batch kernel, for a pair of matrices."""
+def test_linear_workspace_covers_every_kernel_family():
+    """The scratch size is the largest of what the kernels a shape may run on need.  Nine rows and
+    more on a grid too small for the chip: behind the quantized activations, the partial sums of
+    2, 4 or 8 K shares (at least 16 blocks each) of the tiled GEMM.  Up to eight rows (and
+    eight-row slices of a forced plan) on a K longer than 4096: the sums of the K slices of the
+    small-batch kernel, for a pair of matrices.  Up to 64 rows: X in MFMA operand order (rows
+    padded to 32), its scales, and the partial sums of the K shares (128 blocks of Q4_0, 64 of
+    Q8_0 each) of the single-shot MFMA kernel."""
+    def up256(v):
+        return (v + 255) // 256 * 256
+
     def quantized(rows, k):  # int8 values padded to 256 bytes, f32 scales, i32 sums
-        return (rows * k + 255) // 256 * 256 + rows * (k // 32) * 8
+        return up256(rows * k) + rows * (k // 32) * 8
 
     def batch(rows, k, n):
         slices = (k // 32 + 127) // 128
         return slices * min(rows, 8) * n * 4 * 2 if slices > 1 else 0
 
+    def mfma(fmt, rows, k, n):
+        if rows > 64:
+            return 0
+        padded = (rows + 31) // 32 * 32
+        share = 128 if fmt == _lib.TYPE_Q4_0 else 64
+        shares = (k // 32 + share - 1) // share
+        return up256(padded * k + (k // 32) * padded * 4) + (shares * rows * n * 4 if shares > 1 else 0)
+
     for fmt in (_lib.TYPE_Q4_0, _lib.TYPE_Q8_0):
-        for rows, k, n in [(16, 4096, 4096), (64, 14336, 4096), (9, 1024, 64)]:
+        for rows, k, n in [(16, 4096, 4096), (64, 14336, 4096), (9, 1024, 64), (128, 4096, 1024)]:
             got = kernels.workspaceBytes(fmt, rows, k, n)
-            extra = got - (quantized(rows, k) + 255) // 256 * 256
-            assert extra > 0 and extra % (rows * n * 4) == 0 and got >= batch(rows, k, n)
-            shares = extra // (rows * n * 4)
-            assert shares in (2, 4, 8) and (k // 32) // shares >= 16
-        assert kernels.workspaceBytes(fmt, 8, 4096, 4096) == quantized(8, 4096)
+            assert got >= max(quantized(rows, k), batch(rows, k, n), mfma(fmt, rows, k, n))
+            if got > max(batch(rows, k, n), mfma(fmt, rows, k, n)):  # the tiled GEMM's K shares decide
+                extra = got - up256(quantized(rows, k))
+                assert extra > 0 and extra % (rows * n * 4) == 0
+                shares = extra // (rows * n * 4)
+                assert shares in (2, 4, 8) and (k // 32) // shares >= 16
+        assert kernels.workspaceBytes(fmt, 128, 4096, 1024) > quantized(128, 4096)   # 128 workgroups: K is shared out
+        assert kernels.workspaceBytes(fmt, 8, 4096, 4096) == max(quantized(8, 4096), mfma(fmt, 8, 4096, 4096))
         assert kernels.workspaceBytes(fmt, 512, 4096, 4096) == quantized(512, 4096)
-        assert kernels.workspaceBytes(fmt, 16, 512, 4096) == quantized(16, 512)  # too short a K to share out
-        assert kernels.workspaceBytes(fmt, 5, 14336, 4096) == max(quantized(5, 14336), batch(5, 14336, 4096))
+        assert kernels.workspaceBytes(fmt, 16, 512, 4096) == max(quantized(16, 512), mfma(fmt, 16, 512, 4096))
+        assert kernels.workspaceBytes(fmt, 5, 14336, 4096) == max(quantized(5, 14336), batch(5, 14336, 4096), mfma(fmt, 5, 14336, 4096))
         assert batch(5, 14336, 4096) == 4 * 5 * 4096 * 4 * 2
+    assert mfma(_lib.TYPE_Q4_0, 33, 4096, 512) == 64 * 4096 + 128 * 64 * 4
+    assert mfma(_lib.TYPE_Q8_0, 4, 4096, 512) == 32 * 4096 + 128 * 32 * 4 + 2 * 4 * 512 * 4
 
 
 def test_zig_backend_sources_bind_what_exists():
