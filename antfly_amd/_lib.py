@@ -109,6 +109,7 @@ SIGNATURES = {
     "afhip_quant_row_bucket": (_i, [_sz]),
     "afhip_quant_format_from_tensor_type": (_i, [_i]),
     "afhip_uses_activation_quant": (_i, [_sz, _sz, _sz]),
+    "afhip_uses_q8k_activation_quant": (_i, [_i, _sz, _sz, _sz]),
     "afhip_linear_workspace_bytes": (_sz, [_i, _sz, _sz, _sz]),
     "afhip_launch_linear_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),
     "afhip_launch_gemv_probe": (_st, [_vp, _i, Buffer, Buffer, Buffer, _sz, _sz]),

@@ -134,14 +134,15 @@ static GemvTuning gemv_tuning(int tensor_type, int rows, size_t in_dim, size_t o
     return t;
 }
 
-// Q4_K: f32 activations against the dequantized weights, one kernel family for any row count.
+// Q4_K: f32 activations against the dequantized weights, one kernel family for any row count;
+// on the CPU engine's gated short-K shapes, Q8_K-quantized activations and integer sub-block dots.
 static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                     size_t rows, size_t in_dim, size_t out_dim, afhip_buffer workspace, int dispatch,
                                     bool want_dots,
                                     LaunchCounters* counters, afhip_buffer dst_b, afhip_buffer weight_b,
                                     const Epilogue& ep, const Epilogue& ep_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
-    if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // this format has no integer route
+    if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // the block-dot output exists for the 32-value formats only
     if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
     if (in_dim == 0 || in_dim % 256 != 0) return AFHIP_ERR_INVALID_STATE;
@@ -162,6 +163,26 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     if (pair && (dst_b.ptr == 0 || weight_b.ptr == 0 || dst_b.ptr % 4 != 0 || weight_b.ptr % 16 != 0))
         return AFHIP_ERR_INVALID_STATE;
     const int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim, AFHIP_FORMAT_Q4_K);
+    if (afhip_uses_q8k_activation_quant(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim)) {
+        // the CPU engine's gated shapes: activations quantized to Q8_K, integer sub-block dots
+        if (workspace.ptr == 0 || workspace.ptr % 16 != 0 || workspace.len < q4k_q8k_workspace_bytes(rows, in_dim))
+            return AFHIP_ERR_INVALID_STATE;
+        if (counters) counters->activation_quant++;
+        hipError_t e = launch_quantize_q8k(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
+                                           static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
+        for (int i = 0; e == hipSuccess && i < (pair ? 2 : 1); ++i) {
+            if (counters) {
+                if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+                else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+                else counters->mm++;
+            }
+            e = launch_linear_q4k_q8k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
+                                      reinterpret_cast<const void*>(workspace.ptr),
+                                      reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), tiled,
+                                      static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim), i ? ep_b : ep);
+        }
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     // more rows than one GEMV launch holds: X split once into the caller's scratch, then the
     // GEMM (without scratch the GEMV serves them a launch at a time)
     const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
@@ -455,6 +476,12 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
 }
 
 static size_t argmax_logits_bytes(size_t out_dim) { return (out_dim * 4 + 255) / 256 * 256; }
+// scratch of the one-row linear inside the fused lm_head (Q4_K: none, or the Q8_K activations on its gated shapes)
+static size_t argmax_linear_bytes(int tensor_type, size_t in_dim, size_t out_dim) {
+    if (tensor_type != AFHIP_TYPE_Q4_K) return workspace_view(0, 1, in_dim).bytes;
+    const size_t q8k = afhip_uses_q8k_activation_quant(tensor_type, 1, in_dim, out_dim) ? q4k_q8k_workspace_bytes(1, in_dim) : 0;
+    return q8k > 256 ? q8k : 256;
+}
 static size_t argmax_keys_bytes(size_t dim) {
     if (dim > 0x7fffffff) return 0;
     const int groups = argmax_row_workgroups(static_cast<int>(dim));
@@ -537,7 +564,7 @@ afhip_status linear_argmax_impl(void* stream, int tensor_type, int layout, afhip
     }
 
     const afhip_buffer logits{workspace.ptr, out_dim * 4};
-    const size_t linear_bytes = q4k ? 256 : workspace_view(0, 1, in_dim).bytes;
+    const size_t linear_bytes = argmax_linear_bytes(tensor_type, in_dim, out_dim);
     const afhip_buffer linear_ws{workspace.ptr + logits_bytes, linear_bytes};
     const size_t keys_offset = logits_bytes + (linear_bytes + 255) / 256 * 256;
     const afhip_buffer keys_ws{workspace.ptr + keys_offset, workspace.len - keys_offset};
@@ -648,6 +675,15 @@ int afhip_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim) {
     return out_dim >= 512 && in_dim / 32 >= 3;
 }
 
+int afhip_uses_q8k_activation_quant(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (tensor_type != AFHIP_TYPE_Q4_K || in_dim % 256 != 0 || out_dim < 512) return 0;
+    const size_t row_blocks = in_dim / 256;
+    if (!(row_blocks == 2 || row_blocks == 3 || row_blocks == 6 || row_blocks == 8 || row_blocks == 12)) return 0;
+    if (rows == 1 || rows == 2 || rows == 4 || rows == 9) return 1;
+    if (rows == 50 || rows == 64 || rows == 77 || rows == 197 || rows == 257 || rows == 308 || rows == 514) return 1;
+    return rows > 0 && rows <= 308 && rows % 77 == 0;
+}
+
 // ---- launchers
 
 size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
@@ -656,6 +692,7 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
         if (in_dim == 0 || in_dim % 256 != 0 || in_dim > 0x7fffffff || out_dim == 0 || !checked_mul(rows, in_dim, &count) ||
             !checked_mul(count, 8, &bytes))
             return 0;
+        if (afhip_uses_q8k_activation_quant(tensor_type, rows, in_dim, out_dim)) return q4k_q8k_workspace_bytes(rows, in_dim);
         const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
         return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
     }
@@ -906,7 +943,10 @@ afhip_status afhip_launch_argmax_last_row_f32(void* stream, afhip_buffer token_u
 
 size_t afhip_linear_argmax_workspace_bytes(int tensor_type, size_t in_dim, size_t out_dim) {
     if (tensor_type == AFHIP_TYPE_Q4_K)
-        return in_dim == 0 || in_dim % 256 != 0 || out_dim == 0 ? 0 : argmax_logits_bytes(out_dim) + 256 + argmax_keys_bytes(out_dim);
+        return in_dim == 0 || in_dim % 256 != 0 || out_dim == 0
+                   ? 0
+                   : argmax_logits_bytes(out_dim) + (argmax_linear_bytes(tensor_type, in_dim, out_dim) + 255) / 256 * 256 +
+                         argmax_keys_bytes(out_dim);
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || in_dim == 0 || out_dim == 0) return 0;
     return argmax_logits_bytes(out_dim) + (workspace_view(0, 1, in_dim).bytes + 255) / 256 * 256 + argmax_keys_bytes(out_dim);
 }

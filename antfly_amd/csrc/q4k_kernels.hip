@@ -3,7 +3,8 @@
 //
 // The engine computes this format on f32 activations against the dequantized weights
 // w = (d * sc) * q - (dmin * m) (CPU: ops/native_compute.zig:31075-31144; CUDA:
-// ops/cuda/cuda_compute.zig:708 -> launchLinearQ4KTile4F32): there is no integer route.
+// ops/cuda/cuda_compute.zig:708 -> launchLinearQ4KTile4F32); the CPU engine's integer route
+// (Q8_K activations, gated to short K and listed row counts) is at the end of this file.
 // The raw GGUF layout is used as it is: super-blocks are 16-byte aligned (144 = 9 * 16),
 // so a lane reads the 16-byte header and a 16-byte run of nibbles with one load each.
 #include <hip/hip_runtime.h>
@@ -367,6 +368,126 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
+}
+
+// ---- Q4_K with Q8_K-quantized activations: the route the CPU engine takes on a gated set of
+// shapes (shouldUseQ4Q5KQ8KActivationShape, ops/native_compute.zig:3468-3479: short K, listed
+// row counts).  Correctness path for those shapes (CLIP / CLAP projections, 1B / 3B-class
+// decode), not tuned.
+
+// quantizeQ8_KBlock, gguf/quant_codec.zig:710-751: one wavefront per 256-value block, four
+// values per lane.  d = max|x| / 127 (1 for a zero block), q = clamp(round_half_away(x * (1 / d))),
+// sums[block][s] = sum of the 32 quantized values of sub-block s (the engine adds its two
+// 16-value sums whenever it uses them, :32018-32022).
+__global__ __launch_bounds__(256) void quantize_q8k_kernel(const float* __restrict__ x, size_t blocks, int8_t* __restrict__ q,
+                                                           float* __restrict__ d, int* __restrict__ sums) {
+    const int lane = threadIdx.x & 63;
+    for (size_t b = blockIdx.x * 4 + (threadIdx.x >> 6); b < blocks; b += static_cast<size_t>(gridDim.x) * 4) {
+        const float4 v = reinterpret_cast<const float4*>(x)[b * 64 + lane];
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
+        const int bits = __builtin_bit_cast(int, m);
+        m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)),
+                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))),
+                  fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)),
+                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48))));
+        const float s = act_scale(m);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
+        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+        reinterpret_cast<int*>(q)[b * 64 + lane] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        const int total = sum_over_8(q0 + q1 + q2 + q3);
+        if ((lane & 7) == 0) sums[b * 8 + (lane >> 3)] = total;
+        if (lane == 0) d[b] = s;
+    }
+}
+
+// y[r][o] = sum over super-blocks and their sub-blocks of
+//   xd[r][sb] * ((d * sc) * f32(sum q_x * nibble) - (dmin * m) * f32(sum q_x))
+// (dotQ4Q5KPreparedQ8KBlock, ops/native_compute.zig:32031-32049).  One wavefront per output
+// column; a lane takes (super-block, sub-block) pairs lane, lane + 64, ...; rows in turn.  The
+// integer dots are exact; the f32 sum over the pairs is a wavefront tree instead of the
+// engine's running sum.  kTiled: the tile-major layout of the repacked tensor.
+template <bool kTiled>
+__global__ __launch_bounds__(64) void linear_q4k_q8k_kernel(float* __restrict__ dst, const int8_t* __restrict__ q,
+                                                            const float* __restrict__ xd, const int* __restrict__ sums,
+                                                            const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim,
+                                                            Epilogue ep) {
+    const int o = blockIdx.x, lane = threadIdx.x;
+    const int kb = in_dim / kQ4kBlockValues, pairs = kb * 8;
+    for (int r = 0; r < rows; ++r) {
+        float acc = 0.0f;
+        for (int p = lane; p < pairs; p += 64) {
+            const int sb = p >> 3, sub = p & 7, chunk = sub >> 1;
+            q4k_u32x4 header, lo, hi;
+            if (kTiled) {
+                const uint8_t* tile = weight + (static_cast<size_t>(o >> 5) * kb + sb) * (32 * kQ4kBlockBytes);
+                header = *reinterpret_cast<const q4k_u32x4*>(tile + (o & 31) * 16);
+                lo = *reinterpret_cast<const q4k_u32x4*>(tile + 512 + chunk * 1024 + (o & 31) * 16);
+                hi = *reinterpret_cast<const q4k_u32x4*>(tile + 512 + chunk * 1024 + ((o & 31) + 32) * 16);
+            } else {
+                const uint8_t* base = weight + (static_cast<size_t>(o) * kb + sb) * kQ4kBlockBytes;
+                header = *reinterpret_cast<const q4k_u32x4*>(base);
+                lo = *reinterpret_cast<const q4k_u32x4*>(base + 16 + chunk * 32);
+                hi = *reinterpret_cast<const q4k_u32x4*>(base + 32 + chunk * 32);
+            }
+            const uint32_t sh = (sub & 1) * 4;  // low nibbles = sub-block 2c, high nibbles = 2c + 1
+            const uint32_t w[8] = {(lo.x >> sh) & 0x0F0F0F0Fu, (lo.y >> sh) & 0x0F0F0F0Fu, (lo.z >> sh) & 0x0F0F0F0Fu,
+                                   (lo.w >> sh) & 0x0F0F0F0Fu, (hi.x >> sh) & 0x0F0F0F0Fu, (hi.y >> sh) & 0x0F0F0F0Fu,
+                                   (hi.z >> sh) & 0x0F0F0F0Fu, (hi.w >> sh) & 0x0F0F0F0Fu};
+            const int4* xq = reinterpret_cast<const int4*>(q + static_cast<size_t>(r) * in_dim + p * 32);
+            const int4 a0 = xq[0], a1 = xq[1];
+            const int a[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+            int dot = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dot = dot4(a[j], static_cast<int>(w[j]), dot);
+            float sc, mn;
+            q4k_scale_min(header, sub, &sc, &mn);
+            const float dsc = half_bits_to_f32(static_cast<uint16_t>(header.x & 0xFFFFu)) * sc;
+            const float dmn = half_bits_to_f32(static_cast<uint16_t>(header.x >> 16)) * mn;
+            const size_t xb = static_cast<size_t>(r) * kb + sb;
+            acc += xd[xb] * (dsc * static_cast<float>(dot) - dmn * static_cast<float>(sums[xb * 8 + sub]));
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            const size_t at = static_cast<size_t>(r) * out_dim + o;
+            dst[at] = finish_output(ep, o, at, acc);
+        }
+    }
+}
+
+// int8 [rows][in_dim] (padded to 256 bytes), f32 d [rows][in_dim / 256], int32 sums [rows][in_dim / 32]
+size_t q4k_q8k_workspace_bytes(size_t rows, size_t in_dim) {
+    return (rows * in_dim + 255) / 256 * 256 + rows * (in_dim / 256) * 4 + rows * (in_dim / 32) * 4;
+}
+
+hipError_t launch_quantize_q8k(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace) {
+    const size_t blocks = static_cast<size_t>(rows) * (in_dim / kQ4kBlockValues);
+    if (blocks == 0) return hipSuccess;
+    uint8_t* ws = static_cast<uint8_t*>(workspace);
+    int8_t* q = reinterpret_cast<int8_t*>(ws);
+    float* d = reinterpret_cast<float*>(ws + (static_cast<size_t>(rows) * in_dim + 255) / 256 * 256);
+    int* sums = reinterpret_cast<int*>(d + blocks);
+    size_t grid = (blocks + 3) / 4;
+    if (grid > 4096) grid = 4096;
+    hipLaunchKernelGGL(quantize_q8k_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, x, blocks, q, d, sums);
+    return hipGetLastError();
+}
+
+hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, bool tiled, int rows,
+                                 int in_dim, int out_dim, const Epilogue& ep) {
+    if (rows == 0 || out_dim == 0) return hipSuccess;
+    const size_t blocks = static_cast<size_t>(rows) * (in_dim / kQ4kBlockValues);
+    const uint8_t* ws = static_cast<const uint8_t*>(workspace);
+    const int8_t* q = reinterpret_cast<const int8_t*>(ws);
+    const float* d = reinterpret_cast<const float*>(ws + (static_cast<size_t>(rows) * in_dim + 255) / 256 * 256);
+    const int* sums = reinterpret_cast<const int*>(d + blocks);
+    if (tiled)
+        hipLaunchKernelGGL(linear_q4k_q8k_kernel<true>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
+    else
+        hipLaunchKernelGGL(linear_q4k_q8k_kernel<false>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
+    return hipGetLastError();
 }
 
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,

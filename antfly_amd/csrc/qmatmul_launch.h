@@ -139,6 +139,13 @@ hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* ds
 // (two per launch), in_dim a multiple of 256 up to gemv_q4k_max_in_dim(); and its get_rows /
 // cpy_q_to_f32.
 int gemv_q4k_max_in_dim();
+// Q4_K with Q8_K-quantized activations (the CPU engine's route on its gated short-K shapes):
+// launch_quantize_q8k fills `workspace` (q4k_q8k_workspace_bytes() bytes, 16-byte aligned) from X,
+// launch_linear_q4k_q8k multiplies one matrix (raw or tile-major layout) by it.
+size_t q4k_q8k_workspace_bytes(size_t rows, size_t in_dim);
+hipError_t launch_quantize_q8k(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace);
+hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, bool tiled, int rows,
+                                 int in_dim, int out_dim, const Epilogue& ep);
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                            int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,

@@ -581,9 +581,11 @@ def main() -> int:
             ("q4_gemv_m8_k4096_n14336", Q4, 8, 4096, 14336),
             ("q4_gemv_m1_k14336_n4096", Q4, 1, 14336, 4096),
             ("q4_gemv_m5_k14336_n4096", Q4, 5, 14336, 4096),
-            ("q4_batch_m16_k4096_n14336", Q4, 16, 4096, 14336),  # batched decode: quantizer + MFMA GEMM, 32-row tiles
+            ("q4_batch_m16_k4096_n14336", Q4, 16, 4096, 14336),  # batched decode: fragment quantizer + single-shot MFMA kernel
+            ("q4_batch_m32_k4096_n14336", Q4, 32, 4096, 14336),
             ("q4_batch_m64_k4096_n14336", Q4, 64, 4096, 14336),
-            ("q4_batch_m16_k14336_n4096", Q4, 16, 14336, 4096),  # few column tiles: K shared out over workgroups
+            ("q4_batch_m16_k14336_n4096", Q4, 16, 14336, 4096),  # K longer than one share: partial sums + reduce kernel
+            ("q4_batch_m16_k4096_n4096", Q4, 16, 4096, 4096),
         ]:
             copies = args.copies if fmt == Q4 or n > 4096 else 2 * args.copies
             w_s, e_s = time_config(fmt, r, k, n, small_steps, 20, copies, 99)

@@ -61,8 +61,9 @@ const char *afhip_status_string(afhip_status status);
 enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_0 = 8, AFHIP_TYPE_Q4_K = 12 };
 /* Q4_K (144-byte super-blocks of 256 weights) is computed on f32 activations against the
  * dequantized weights, as the engine does on the CPU (ops/native_compute.zig:31075-31144)
- * and in its CUDA backend (ops/cuda/cuda_compute.zig:708): no activation quantizer and no
- * block dots.  Both layouts are served: RAW (GGUF bytes, 16-byte aligned) by a vector-ALU
+ * and in its CUDA backend (ops/cuda/cuda_compute.zig:708) -- except on the CPU engine's gated
+ * short-K shapes (afhip_uses_q8k_activation_quant), where the activations are quantized to
+ * Q8_K as it does there.  No block-dot output for this format.  Both layouts are served: RAW (GGUF bytes, 16-byte aligned) by a vector-ALU
  * kernel, PREPARED (tile-major, see afhip_prepared_weight_bytes) by the MFMA kernels; more
  * rows than one decode launch holds use the caller's workspace
  * (afhip_linear_workspace_bytes) for the prefill GEMM.  in_dim must be a multiple of 256.
@@ -127,6 +128,13 @@ int afhip_quant_format_from_tensor_type(int tensor_type); /* graph/backend_contr
  * quantizes activations to int8 per 32-block, 0 when it multiplies f32
  * activations by dequantized weights. */
 int afhip_uses_activation_quant(size_t rows, size_t in_dim, size_t out_dim);
+/* Q4_K only: whether the op quantizes the activations to Q8_K (256-value blocks) and takes
+ * integer sub-block dots, as the CPU engine does on a gated set of shapes
+ * (shouldUseQ4Q5KQ8KActivationShape, ops/native_compute.zig:3468-3479, used at :6684-6700):
+ * out_dim >= 512, in_dim / 256 in {2, 3, 6, 8, 12}, rows in {1, 2, 4, 9, 50, 64, 77, 154, 197, 231,
+ * 257, 308, 514}.  Everywhere else Q4_K is computed on f32 activations.  On these shapes the
+ * launchers need afhip_linear_workspace_bytes() of scratch. */
+int afhip_uses_q8k_activation_quant(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 
 /* ------------------------------------------------------------------------
  * Kernel launchers: ops/cuda/kernels.zig:1221-1289 (launchLinearQ8_0F32 /

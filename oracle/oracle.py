@@ -63,6 +63,10 @@ def lib() -> C.CDLL:
         L.afo_dequantize_q4_k.argtypes = [vp, sz, vp]
         L.afo_linear_q4_k.argtypes = [vp, vp, vp, sz, sz, sz]
         L.afo_linear_q4_k_f64.argtypes = [vp, vp, vp, sz, sz, sz]
+        L.afo_uses_q4k_q8k_activation.argtypes = [sz, sz, sz]
+        L.afo_quantize_q8_k.argtypes = [vp, sz, vp, vp, vp]
+        L.afo_quantize_q8_k.restype = None
+        L.afo_linear_q4_k_q8k.argtypes = [vp, vp, vp, sz, sz, sz]
         L.afo_argmax.restype = sz
         L.afo_argmax.argtypes = [vp, sz]
         L.afo_argmax_last_row.restype = C.c_long
@@ -248,6 +252,29 @@ def dequantize_q4_k(raw) -> np.ndarray:
     out = np.zeros(r.size // 144 * 256, np.float32)
     lib().afo_dequantize_q4_k(_p(r), r.size // 144, _p(out))
     return out
+
+
+def uses_q4k_q8k_activation(rows, in_dim, out_dim) -> bool:
+    return bool(lib().afo_uses_q4k_q8k_activation(rows, in_dim, out_dim))
+
+
+def quantize_q8_k(x):
+    """(q int8 [n], d f32 [n / 256], bsums int16 [n / 16]) of a flat f32 array of whole 256-blocks."""
+    xx = _f32(x)
+    assert xx.size % 256 == 0
+    nb = xx.size // 256
+    q, d, bs = np.zeros(nb * 256, np.int8), np.zeros(nb, np.float32), np.zeros(nb * 16, np.int16)
+    lib().afo_quantize_q8_k(_p(xx), nb, _p(q), _p(d), _p(bs))
+    return q, d, bs
+
+
+def linear_q4_k_q8k(x, w_raw, rows, in_dim, out_dim) -> np.ndarray:
+    xx, w = _f32(x), _u8(w_raw)
+    assert xx.size == rows * in_dim and w.size == out_dim * (in_dim // 256) * 144
+    y = np.zeros((rows, out_dim), np.float32)
+    if lib().afo_linear_q4_k_q8k(_p(xx), _p(w), _p(y), rows, in_dim, out_dim) != 0:
+        raise ValueError("InvalidQuantizedLinearShape")
+    return y
 
 
 def linear_q4_k(x, w_raw, rows, in_dim, out_dim, f64=False) -> np.ndarray:

@@ -736,3 +736,80 @@ int afo_linear_q4_k_f64(const float *x, const uint8_t *w, double *y, size_t rows
     }
     return 0;
 }
+
+int afo_uses_q4k_q8k_activation(size_t rows, size_t in_dim, size_t out_dim) {
+    if (in_dim % AFO_Q4_K_BLOCK_VALUES != 0) return 0;
+    size_t row_blocks = in_dim / AFO_Q4_K_BLOCK_VALUES;
+    if (out_dim < 512 || row_blocks < 1) return 0;
+    if (!(row_blocks == 2 || row_blocks == 3 || row_blocks == 6 || row_blocks == 8 || row_blocks == 12)) return 0;
+    if (rows == 1 || rows == 2 || rows == 4 || rows == 9) return 1;
+    if (rows == 50 || rows == 64 || rows == 77 || rows == 197 || rows == 257 || rows == 308 || rows == 514) return 1;
+    if (rows > 0 && rows <= 308 && rows % 77 == 0) return 1;
+    return 0;
+}
+
+void afo_quantize_q8_k(const float *x, size_t n_blocks, int8_t *q, float *d, int16_t *bsums) {
+    for (size_t b = 0; b < n_blocks; b++) {
+        const float *xb = x + b * 256;
+        float max_abs = 0.0f;
+        for (int i = 0; i < 256; i++) {
+            float a = fabsf(xb[i]);
+            if (a > max_abs) max_abs = a;
+        }
+        float scale = max_abs == 0.0f ? 1.0f : max_abs / 127.0f;
+        d[b] = scale;
+        float inv = 1.0f / scale;
+        for (int g = 0; g < 16; g++) {
+            int sum = 0;
+            for (int i = 0; i < 16; i++) {
+                float r = max_abs == 0.0f ? 0.0f : roundf(xb[g * 16 + i] * inv);
+                if (r < -127.0f) r = -127.0f;
+                if (r > 127.0f) r = 127.0f;
+                q[b * 256 + g * 16 + i] = (int8_t)r;
+                sum += (int)r;
+            }
+            bsums[b * 16 + g] = (int16_t)sum;
+        }
+    }
+}
+
+int afo_linear_q4_k_q8k(const float *x, const uint8_t *w, float *y, size_t rows, size_t in_dim, size_t out_dim) {
+    if (in_dim % AFO_Q4_K_BLOCK_VALUES != 0) return -1;
+    size_t kb = in_dim / AFO_Q4_K_BLOCK_VALUES;
+    size_t n_blocks = rows * kb, n_alloc = n_blocks > 0 ? n_blocks : 1;
+    int8_t *q = (int8_t *)malloc(n_alloc * 256);
+    float *xd = (float *)malloc(n_alloc * sizeof(float));
+    int16_t *bs = (int16_t *)malloc(n_alloc * 16 * sizeof(int16_t));
+    if (!q || !xd || !bs) { free(q); free(xd); free(bs); return -2; }
+    afo_quantize_q8_k(x, n_blocks, q, xd, bs);
+    for (size_t o = 0; o < out_dim; o++) {
+        for (size_t r = 0; r < rows; r++) {
+            float total = 0.0f;
+            for (size_t b = 0; b < kb; b++) {
+                const uint8_t *blk = w + (o * kb + b) * AFO_Q4_K_BLOCK_BYTES;
+                float dd = afo_fp16_to_f32((uint16_t)(blk[0] | (blk[1] << 8))), dmin = afo_fp16_to_f32((uint16_t)(blk[2] | (blk[3] << 8)));
+                uint8_t scs[8], mins[8];
+                afo_q4k_unpack_scale_mins(blk + 4, scs, mins);
+                const uint8_t *qs = blk + 16;
+                const int8_t *qx = q + (r * kb + b) * 256;
+                const int16_t *sums = bs + (r * kb + b) * 16;
+                float x_d = xd[r * kb + b];
+                float acc = 0.0f;
+                for (int sub = 0; sub < 8; sub++) {
+                    int chunk = sub / 2, dot = 0;
+                    for (int i = 0; i < 32; i++) {
+                        int nib = (sub & 1) ? (qs[chunk * 32 + i] >> 4) : (qs[chunk * 32 + i] & 15);
+                        dot += (int)qx[sub * 32 + i] * nib;
+                    }
+                    int asum = (int)sums[sub * 2] + (int)sums[sub * 2 + 1];
+                    float dsc = dd * (float)scs[sub], dmn = dmin * (float)mins[sub];
+                    acc += x_d * (dsc * (float)dot - dmn * (float)asum);
+                }
+                total += acc;
+            }
+            y[r * out_dim + o] = total;
+        }
+    }
+    free(q); free(xd); free(bs);
+    return 0;
+}

@@ -7,13 +7,11 @@
  * Reference files are cited as INF = zig/pkg/inference/src in the reference
  * tree.  Every function here is pinned by the reference's own known-answer
  * tests (re-encoded under tests/golden/) plus closed forms / brute force in
- * tests/test_oracle_*.py; no function here is "parity unpinned".
- *
- * Not restated here, hence parity unpinned for it: the engine's Q8_K
- * activation-quantized route for Q4_K (INF/ops/native_compute.zig:3468-3479,
- * :32031-32049), taken only for in_dim in {512, 768, 1536, 2048, 3072} with
- * out_dim >= 512 and a fixed list of row counts.  The Q4_K functions below follow
- * the engine's f32 route, which is what it computes at every other shape.
+ * tests/test_oracle_*.py; no function here is "parity unpinned".  (The Q8_K
+ * activation route of Q4_K has no known-answer vectors in the reference -- its own
+ * tests hold it to invariants and to a 1e-2 tolerance against the f32 route -- so it
+ * is pinned by those invariants, by exact rational arithmetic on inputs whose
+ * quantized values are known in closed form, and by brute-force integer sums.)
  */
 #ifndef ANTFLY_QMATMUL_ORACLE_H
 #define ANTFLY_QMATMUL_ORACLE_H
@@ -125,7 +123,7 @@ int afo_linear_prepared(const afo_prepared *p, const float *x, float *y, size_t 
 /* ---- Q4_K: 144-byte super-blocks of 256 weights (INF/gguf/tensor_types.zig:160-219):
  * fp16 d, fp16 dmin, 12 bytes of packed 6-bit (scale, min) pairs for 8 sub-blocks of
  * 32, 128 bytes of nibbles.  The CPU engine multiplies f32 activations by the
- * dequantized weights; there is no integer route for this format. */
+ * dequantized weights, except on the gated shapes of the Q8_K route further down. */
 enum { AFO_FMT_Q4_K = 12, AFO_Q4_K_BLOCK_VALUES = 256, AFO_Q4_K_BLOCK_BYTES = 144 };
 /* unpackQ4KScaleMinsU8, INF/ops/native_compute.zig:33745-33754 (= quant_codec.zig:2742-2751). */
 void afo_q4k_unpack_scale_mins(const uint8_t *scales12, uint8_t *scs8, uint8_t *mins8);
@@ -142,6 +140,22 @@ int afo_linear_q4_k(const float *x, const uint8_t *w_raw, float *y, size_t rows,
 /* The same sum in double precision over the f32 dequantized weights. */
 int afo_linear_q4_k_f64(const float *x, const uint8_t *w_raw, double *y, size_t rows, size_t in_dim,
                         size_t out_dim);
+
+/* ---- Q4_K with Q8_K-quantized activations: the route the CPU engine takes for Q4_K on a
+ * gated set of shapes (shouldUseQ4Q5KQ8KActivationShape, INF/ops/native_compute.zig:3468-3479,
+ * used at :6684-6700): out_dim >= 512, in_dim / 256 in {2, 3, 6, 8, 12} and rows in
+ * {1, 2, 4, 9, 50, 64, 77, 197, 257, 308, 514} or a multiple of 77 up to 308. */
+int afo_uses_q4k_q8k_activation(size_t rows, size_t in_dim, size_t out_dim);
+/* quantizeQ8_KBlock, INF/gguf/quant_codec.zig:710-751, per 256 values: d = max|x| / 127 (1 for
+ * an all-zero block), q = clamp(round_half_away(x * (1 / d)), -127, 127), and the sum of every
+ * 16 consecutive q as int16.  q: n_blocks * 256, d: n_blocks, bsums: n_blocks * 16. */
+void afo_quantize_q8_k(const float *x, size_t n_blocks, int8_t *q, float *d, int16_t *bsums);
+/* linearNoBiasQ4Q5KPreparedQ8KActivation (INF/ops/native_compute.zig:22477-22534) with the block
+ * dot of dotQ4Q5KPreparedQ8KBlock (:32031-32049): per super-block, over its 8 sub-blocks in
+ * order, acc += xd * ((d*sc) * f32(sum q_x * nibble) - (dmin*m) * f32(sum q_x)); the
+ * super-blocks' values are added in order.  (The engine's panel kernels vectorise this sum
+ * over columns, not over K: the order per output is the same.)  -1 when in_dim % 256 != 0. */
+int afo_linear_q4_k_q8k(const float *x, const uint8_t *w_raw, float *y, size_t rows, size_t in_dim, size_t out_dim);
 
 /* Greedy token pick, INF/backends/activations.zig:331-357 (vectorMax + argmax) as used
  * by argmaxLastRow (INF/ops/native_compute.zig:37901-37907): the largest value's

@@ -106,6 +106,57 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
     assert err32 <= TOL and err32 <= TIGHT, err32
 
 
+Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
+
+
+@pytest.mark.parametrize("layout", [RAW, PREP])
+@pytest.mark.parametrize("rows,in_dim,out_dim", Q8K_SHAPES)
+def test_q8k_activation_route_on_the_gated_shapes(layout, rows, in_dim, out_dim):
+    """The CPU engine's gated short-K shapes (native_compute.zig:3468-3479): activations quantized
+    to Q8_K, integer sub-block dots.  Against the oracle's restatement of that route; the f32 route
+    is a different number there (about 1e-3 .. 1e-2 away), so this also shows which route ran."""
+    print(f"case: q4_k q8k route layout={layout} rows={rows} in={in_dim} out={out_dim}", flush=True)
+    assert O.uses_q4k_q8k_activation(rows, in_dim, out_dim)
+    assert _lib.lib().afhip_uses_q8k_activation_quant(Q4K, rows, in_dim, out_dim) == 1
+    w = synth.weights(Q4K, 71, out_dim, in_dim)
+    x = synth.activations(72, rows, in_dim)
+    wd = device_weight(layout, w, out_dim, in_dim)
+    y = G.linear(Q4K, layout, x, wd, rows, in_dim, out_dim)
+    ref = O.linear_q4_k_q8k(x, w, rows, in_dim, out_dim)
+    err = G.max_rel_err(y, ref.astype(np.float64))
+    assert err <= TOL and err <= TIGHT, err
+    f32_route = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+    assert G.max_rel_err(y, f32_route) > 10 * TIGHT
+    # the launcher needs the scratch on these shapes
+    with pytest.raises(_lib.InvalidHipState):
+        kernels.launchLinearF32(G.stream(), Q4K, layout, G.buf(torch.empty((rows, out_dim), dtype=torch.float32, device=G.DEV)),
+                                G.buf(G.to_dev(x)), G.buf(wd), rows, in_dim, out_dim, kernels.NO_BUFFER)
+
+
+def test_q8k_gate_neighbours_stay_on_the_f32_route():
+    for rows, in_dim, out_dim in [(3, 2048, 512), (1, 1024, 512), (1, 2048, 511), (5, 3072, 640), (16, 512, 512)]:
+        assert not O.uses_q4k_q8k_activation(rows, in_dim, out_dim)
+        assert _lib.lib().afhip_uses_q8k_activation_quant(Q4K, rows, in_dim, out_dim) == 0
+        w = synth.weights(Q4K, 73, out_dim, in_dim)
+        x = synth.activations(74, rows, in_dim)
+        y = G.linear(Q4K, PREP, x, device_weight(PREP, w, out_dim, in_dim), rows, in_dim, out_dim)
+        assert G.max_rel_err(y, O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)) <= TIGHT
+    assert _lib.lib().afhip_uses_q8k_activation_quant(_lib.TYPE_Q4_0, 1, 2048, 512) == 0
+
+
+def test_q8k_route_pair_and_bias():
+    rows, in_dim, out_dim = 2, 2048, 640
+    wa, wb = synth.weights(Q4K, 75, out_dim, in_dim), synth.weights(Q4K, 76, out_dim, in_dim)
+    x = synth.activations(77, rows, in_dim)
+    da, db = device_weight(PREP, wa, out_dim, in_dim), device_weight(PREP, wb, out_dim, in_dim)
+    ya, yb = G.linear_pair(Q4K, PREP, x, da, db, rows, in_dim, out_dim)
+    assert np.array_equal(ya, G.linear(Q4K, PREP, x, da, rows, in_dim, out_dim))
+    assert np.array_equal(yb, G.linear(Q4K, PREP, x, db, rows, in_dim, out_dim))
+    bias = synth.activations(78, 1, out_dim).reshape(-1)
+    yb2 = G.linear_bias(Q4K, PREP, x, da, bias, rows, in_dim, out_dim)
+    assert np.array_equal(yb2, ya + bias[None, :])
+
+
 PREFILL_SHAPES = [(7, 4096, 64), (10, 1024, 300), (11, 512, 33), (40, 2048, 256), (41, 1024, 257), (100, 512, 1000),
                   (128, 4096, 512), (3, 14336, 40), (45, 14336, 96), (300, 256, 64), (8, 512, 40), (9, 512, 40), (12, 512, 40), (13, 4096, 300), (7, 4096, 300), (3, 14336, 64), (5, 14336, 200), (33, 1024, 64), (64, 1024, 96), (20, 2560, 700), (50, 14336, 64),
                   (81, 768, 500)]
@@ -214,9 +265,16 @@ def test_backend_ops_on_q4_k():
         assert G.max_rel_err(y, ref) <= TIGHT
         stats = cb.debugStats()
         assert stats["launches_small_batch"] == 1 and stats["launches_activation_quant"] == 0 and stats["launches_prepare"] == 1
+        # the fused lm_head is one matmul on the last row alone: at this K (512) and width that is one of
+        # the shapes on which the engine quantizes the activations to Q8_K
         token = cb.linearNoBiasArgmaxLastRow(xt, wt, rows, in_dim, out_dim)
-        assert token == int(np.argmax(y[-1]))
-        assert token == O.argmax(ref[-1].astype(np.float32)) or ref[-1].max() - ref[-1][token] <= TIGHT * np.abs(ref[-1]).max()
+        assert O.uses_q4k_q8k_activation(1, in_dim, out_dim) and not O.uses_q4k_q8k_activation(rows, in_dim, out_dim)
+        last = cb.toFloat32(cb.linearNoBias(cb.fromFloat32(x[-1:].copy(), [1, in_dim]), wt, 1, in_dim, out_dim)).reshape(out_dim)
+        assert cb.debugStats()["launches_activation_quant"] == 2
+        assert token == int(np.argmax(last))
+        ref_last = O.linear_q4_k_q8k(x[-1:], w, 1, in_dim, out_dim)[0]
+        assert G.max_rel_err(last[None, :], ref_last[None, :].astype(np.float64)) <= TIGHT
+        assert token == O.argmax(ref_last) or ref_last.max() - ref_last[token] <= TIGHT * np.abs(ref_last).max()
         emb = cb.toFloat32(cb.embeddingLookup(wt, [999, 0], 2, in_dim)).reshape(2, in_dim)
         assert np.array_equal(emb.view(np.uint32), O.dequantize_q4_k(w).reshape(out_dim, in_dim)[[999, 0]].view(np.uint32))
         with pytest.raises(_lib.InvalidHipState):

@@ -387,6 +387,96 @@ def test_q4_k_against_independent_numpy_form():
     del wf
 
 
+# ---------------------------------------------------------------- Q4_K with Q8_K activations
+
+def test_q8k_route_gate_is_the_reference_list():
+    """shouldUseQ4Q5KQ8KActivationShape, native_compute.zig:3468-3479, case by case."""
+    yes_rows = [1, 2, 4, 9, 50, 64, 77, 154, 197, 231, 257, 308, 514]
+    for blocks in (2, 3, 6, 8, 12):
+        for rows in yes_rows:
+            assert O.uses_q4k_q8k_activation(rows, blocks * 256, 512), (rows, blocks)
+        for rows in (0, 3, 5, 8, 16, 32, 63, 65, 100, 385, 462, 513, 1024):
+            assert not O.uses_q4k_q8k_activation(rows, blocks * 256, 4096), (rows, blocks)
+        assert not O.uses_q4k_q8k_activation(1, blocks * 256, 511)
+    for blocks in (1, 4, 5, 7, 9, 10, 11, 13, 16, 56):
+        assert not O.uses_q4k_q8k_activation(1, blocks * 256, 4096), blocks
+    assert not O.uses_q4k_q8k_activation(1, 2048 + 32, 4096)
+
+
+def test_q8_k_quantizer_invariants_and_closed_forms():
+    """quantizeQ8_KBlock: the reference's own checks (block sums = sums of the stored bytes,
+    quant_codec.zig:3342-3360; ramp round trip within 1.5, :3329-3340) and the quantized values
+    themselves from exact rational arithmetic wherever the exact quotient is not within 1e-4 of a tie."""
+    from fractions import Fraction
+    i = np.arange(256)
+    cases = [((i % 31 - 15) * 0.25).astype(np.float32), (-48.0 + 0.375 * i).astype(np.float32),
+             synth.activations(5, 1, 256).reshape(-1), np.zeros(256, np.float32),
+             np.where(i % 2 == 0, 3.0, -3.0).astype(np.float32)]
+    for x in cases:
+        q, d, bs = O.quantize_q8_k(x)
+        assert np.array_equal(bs, q.astype(np.int32).reshape(16, 16).sum(axis=1).astype(np.int16))
+        m = float(np.abs(x).max())
+        if m == 0.0:
+            assert d[0] == 1.0 and not q.any()
+            continue
+        assert d[0] == np.float32(m) / np.float32(127.0)
+        assert np.abs(q.astype(np.float64) * float(d[0]) - x).max() <= 1.5
+        assert np.abs(q).max() == 127 and np.abs(q.astype(np.int32)).max() <= 127
+        checked = 0
+        for v, got in zip(x.tolist(), q.tolist()):
+            t = Fraction(v) * 127 / Fraction(m)
+            frac = abs(t) - int(abs(t))
+            if abs(frac - Fraction(1, 2)) < Fraction(1, 10000):
+                continue
+            want = int(abs(t) + Fraction(1, 2)) * (1 if t >= 0 else -1)
+            assert got == want, (v, got, want)
+            checked += 1
+        assert checked > 200
+    q, d, bs = O.quantize_q8_k(np.concatenate([cases[0], cases[2]]))  # blocks are independent
+    assert np.array_equal(q[:256], O.quantize_q8_k(cases[0])[0]) and np.array_equal(q[256:], O.quantize_q8_k(cases[2])[0])
+
+
+def test_q4_k_q8k_route_against_brute_force_and_the_dequantized_dot():
+    """The route's sum restated independently: integer sub-block dots by numpy on the unpacked
+    nibbles, combined in float64 -- and the property the reference tests its Q8_K routes with
+    (native_compute.zig:42279-42346): the result is the f32-route product of the DEQUANTIZED
+    activations q * d.  A dropped min term, a swapped nibble order or a wrong sub-block index fails both."""
+    rows, in_dim, out_dim = 4, 768, 9
+    kb = in_dim // 256
+    x = synth.activations(21, rows, in_dim)
+    x[1, 256:512] = 0.0  # an all-zero activation block
+    w = synth.weights(synth.Q4_K, 22, out_dim, in_dim)
+    y = O.linear_q4_k_q8k(x, w, rows, in_dim, out_dim)
+    q, d, bs = O.quantize_q8_k(x)
+    q = q.reshape(rows, kb, 8, 32).astype(np.int64)
+    d = d.reshape(rows, kb).astype(np.float64)
+    b = w.reshape(out_dim, kb, 144)
+    dw = b[:, :, 0:2].copy().view(np.float16).astype(np.float64)[..., 0]
+    dmin = b[:, :, 2:4].copy().view(np.float16).astype(np.float64)[..., 0]
+    want = np.zeros((rows, out_dim))
+    for o in range(out_dim):
+        for k in range(kb):
+            scs, mins = O.q4k_unpack_scale_mins(b[o, k, 4:16])
+            qs = b[o, k, 16:].reshape(4, 32)
+            nib = np.stack([qs & 15, qs >> 4], axis=1).reshape(8, 32).astype(np.int64)
+            for r in range(rows):
+                dots = (q[r, k] * nib).sum(axis=1)
+                sums = q[r, k].sum(axis=1)
+                want[r, o] += d[r, k] * float(((dw[o, k] * scs) * dots - (dmin[o, k] * mins) * sums).sum())
+    scale = np.abs(want).max(axis=1, keepdims=True)
+    assert (np.abs(y - want) / scale).max() <= 2e-6
+    xq = (q.reshape(rows, kb, 256) * d[:, :, None]).reshape(rows, in_dim).astype(np.float32)
+    via_dequant = O.linear_q4_k(xq, w, rows, in_dim, out_dim, f64=True)
+    assert (np.abs(y - via_dequant) / scale).max() <= 2e-6
+    # and it stays close to the f32 route on the unquantized activations (the reference's own
+    # bound is 1e-2 of the value or 5e-2, native_compute.zig:42392-42437)
+    f32_route = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+    assert (np.abs(y - f32_route) / scale).max() <= 2e-2
+    assert (np.abs(y - f32_route) / scale).max() > 1e-5  # it IS another route
+    with pytest.raises(ValueError):
+        O.linear_q4_k_q8k(np.zeros((1, 128), np.float32), np.zeros(0, np.uint8), 1, 128, 0)
+
+
 # ---------------------------------------------------------------- greedy token pick
 
 def test_argmax_reference_vectors_and_properties(kats):
