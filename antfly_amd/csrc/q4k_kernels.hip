@@ -457,6 +457,113 @@ __global__ __launch_bounds__(64) void linear_q4k_q8k_kernel(float* __restrict__ 
     }
 }
 
+// The same op on the tile-major layout, for the shapes that matter (decode and a few rows at
+// K = 2048 / 3072; CLIP-sized batches): the weights of a tile are read once whatever the row count.
+// A workgroup owns a tile of 32 columns and a group of rows; wavefront w owns super-block w of the
+// tile (blockDim.x = 64 * in_dim / 256, at most 12 wavefronts): lane (column c, half g) keeps the
+// header of its column decoded (eight d*sc, eight dmin*m) and, for each of the four 32-byte
+// chunks, its 16 bytes -- values 16g .. 16g+15 of sub-blocks 2c (low nibbles) and 2c+1 (high) --
+// in registers.  Rows pass through LDS eight at a time (quantized values, scales, sums as
+// floats); per row a lane reads the 16 bytes of each of the 8 sub-blocks that face its nibbles
+// (all lanes of a half read the same address: a broadcast), takes 32 v_dot4 and adds
+// xd * (sum_s (d*sc)_s * f32(dot_s) - its four sub-blocks' share of sum_s (dmin*m)_s * f32(sum_s)).
+// Each half's dots cover half a sub-block, so the products of the two halves are rounded
+// separately before they meet in the final sum (the engine rounds the product of the whole
+// sub-block dot): a difference in the last bit of a term.  Halves and wavefronts meet in LDS
+// in a fixed order.
+constexpr int kQ8kPassRows = 8;
+__global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __restrict__ dst, const int8_t* __restrict__ q,
+                                                                  const float* __restrict__ xd, const int* __restrict__ sums,
+                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                                  int out_dim, int rows_per_group, Epilogue ep) {
+    extern __shared__ __align__(16) unsigned char q8k_lds[];
+    const int kb = in_dim / kQ4kBlockValues;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = blockDim.x;
+    const int col = lane & 31, g = lane >> 5;
+    const int tile = blockIdx.x;
+    int8_t* xq_s = reinterpret_cast<int8_t*>(q8k_lds);                                             // [8][in_dim]
+    float* xd_s = reinterpret_cast<float*>(q8k_lds + kQ8kPassRows * in_dim);                       // [8][kb]
+    float* fs_s = xd_s + kQ8kPassRows * kb;                                                        // [8][kb][8]
+    float* red = fs_s + kQ8kPassRows * kb * 8;                                                     // [kb][2][8][32]
+
+    const uint8_t* tbase = weight + (static_cast<size_t>(tile) * kb + wave) * (32 * kQ4kBlockBytes);
+    const q4k_u32x4 header = *reinterpret_cast<const q4k_u32x4*>(tbase + col * 16);
+    q4k_u32x4 nib[4];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) nib[c] = *reinterpret_cast<const q4k_u32x4*>(tbase + 512 + c * 1024 + (col + 32 * g) * 16);
+    float dsc[8], dmn[8];
+    {
+        const float d = half_bits_to_f32(static_cast<uint16_t>(header.x & 0xFFFFu));
+        const float dmin = half_bits_to_f32(static_cast<uint16_t>(header.x >> 16));
+#pragma unroll
+        for (int sub = 0; sub < 8; ++sub) {
+            float sc, mn;
+            q4k_scale_min(header, sub, &sc, &mn);
+            dsc[sub] = d * sc;
+            dmn[sub] = dmin * mn;
+        }
+    }
+    // unsigned nibbles as bytes: w[c][0..3] = sub-block 2c, w[c][4..7] = sub-block 2c + 1
+    uint32_t w[4][8];
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const uint32_t p[4] = {nib[c].x, nib[c].y, nib[c].z, nib[c].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            w[c][j] = p[j] & 0x0F0F0F0Fu;
+            w[c][4 + j] = (p[j] >> 4) & 0x0F0F0F0Fu;
+        }
+    }
+
+    const int row_begin = blockIdx.y * rows_per_group;
+    const int row_end = min(rows, row_begin + rows_per_group);
+    for (int r0 = row_begin; r0 < row_end; r0 += kQ8kPassRows) {
+        const int nr = min(kQ8kPassRows, row_end - r0);
+        __syncthreads();  // the previous pass has been read
+        {
+            const uint4* src = reinterpret_cast<const uint4*>(q + static_cast<size_t>(r0) * in_dim);
+            uint4* dst4 = reinterpret_cast<uint4*>(xq_s);
+            for (int u = tid; u < nr * (in_dim >> 4); u += threads) dst4[u] = src[u];
+            for (int u = tid; u < nr * kb; u += threads) xd_s[u] = xd[static_cast<size_t>(r0) * kb + u];
+            for (int u = tid; u < nr * kb * 8; u += threads) fs_s[u] = static_cast<float>(sums[static_cast<size_t>(r0) * kb * 8 + u]);
+        }
+        __syncthreads();
+        for (int r = 0; r < nr; ++r) {
+            const int8_t* xrow = xq_s + r * in_dim + wave * kQ4kBlockValues + 16 * g;
+            float part = 0.0f;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int sub = 2 * c + h;
+                    const int4 a = *reinterpret_cast<const int4*>(xrow + sub * 32);
+                    int dot = dot4(a.x, static_cast<int>(w[c][4 * h]), 0);
+                    dot = dot4(a.y, static_cast<int>(w[c][4 * h + 1]), dot);
+                    dot = dot4(a.z, static_cast<int>(w[c][4 * h + 2]), dot);
+                    dot = dot4(a.w, static_cast<int>(w[c][4 * h + 3]), dot);
+                    part = __builtin_fmaf(dsc[sub], static_cast<float>(dot), part);
+                }
+            }
+            // the min terms: each half takes four of the eight sub-blocks
+            const float4 fsum = *reinterpret_cast<const float4*>(fs_s + (r * kb + wave) * 8 + 4 * g);
+            const float m0 = g ? dmn[4] : dmn[0], m1 = g ? dmn[5] : dmn[1], m2 = g ? dmn[6] : dmn[2], m3 = g ? dmn[7] : dmn[3];
+            part -= (m0 * fsum.x + m1 * fsum.y) + (m2 * fsum.z + m3 * fsum.w);
+            red[((wave * 2 + g) * kQ8kPassRows + r) * 32 + col] = xd_s[r * kb + wave] * part;
+        }
+        __syncthreads();
+        for (int i = tid; i < nr * 32; i += threads) {
+            const int r = i >> 5, c = i & 31;
+            float total = 0.0f;
+            for (int ww = 0; ww < kb; ++ww) total += red[((ww * 2) * kQ8kPassRows + r) * 32 + c] + red[((ww * 2 + 1) * kQ8kPassRows + r) * 32 + c];
+            const int n = tile * 32 + c;
+            if (n < out_dim) {
+                const size_t at = static_cast<size_t>(r0 + r) * out_dim + n;
+                dst[at] = finish_output(ep, n, at, total);
+            }
+        }
+    }
+}
+
 // int8 [rows][in_dim] (padded to 256 bytes), f32 d [rows][in_dim / 256], int32 sums [rows][in_dim / 32]
 size_t q4k_q8k_workspace_bytes(size_t rows, size_t in_dim) {
     return (rows * in_dim + 255) / 256 * 256 + rows * (in_dim / 256) * 4 + rows * (in_dim / 32) * 4;
@@ -483,7 +590,20 @@ hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* wor
     const int8_t* q = reinterpret_cast<const int8_t*>(ws);
     const float* d = reinterpret_cast<const float*>(ws + (static_cast<size_t>(rows) * in_dim + 255) / 256 * 256);
     const int* sums = reinterpret_cast<const int*>(d + blocks);
-    if (tiled)
+    const int kb = in_dim / kQ4kBlockValues;
+    if (tiled && kb <= 12) {
+        // row groups: enough workgroups for the chip on narrow matrices, whole passes of eight rows each
+        const int tiles = (out_dim + 31) / 32;
+        int groups = (2 * gemv_compute_units() + tiles - 1) / tiles;
+        const int passes = (rows + kQ8kPassRows - 1) / kQ8kPassRows;
+        if (groups > passes) groups = passes;
+        const int rows_per_group = (passes + groups - 1) / groups * kQ8kPassRows;
+        groups = (rows + rows_per_group - 1) / rows_per_group;
+        const size_t lds = static_cast<size_t>(kQ8kPassRows) * in_dim + kQ8kPassRows * kb * 4 + kQ8kPassRows * kb * 32 +
+                           static_cast<size_t>(kb) * 2 * kQ8kPassRows * 32 * 4;
+        hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel, dim3(tiles, groups), dim3(64 * kb), lds, stream, dst, q, d, sums, weight, rows,
+                           in_dim, out_dim, rows_per_group, ep);
+    } else if (tiled)
         hipLaunchKernelGGL(linear_q4k_q8k_kernel<true>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
     else
         hipLaunchKernelGGL(linear_q4k_q8k_kernel<false>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
