@@ -105,12 +105,16 @@ static int env_int(const char* name) {
 
 // Whether the single-shot MFMA kernel serves this shape (measured against the kernels it replaces;
 // AFHIP_BATCH_MFMA_MIN_ROWS overrides the lower row bound for tuning runs, 0 switches the kernel off):
-// from five rows on (six on a K longer than 4096, where the split-K GEMV still wins at five), and for
-// Q8_0, whose K shares are half as long, only while all workgroups of the launch are resident at once.
+// from five rows on (six on a K longer than 4096, where the split-K GEMV still wins at five) up to 64
+// (128 on wide Q4_0 matrices), and for Q8_0, whose K shares are half as long, only while all workgroups
+// of the launch are resident at once.
 static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     static const char* v = std::getenv("AFHIP_BATCH_MFMA_MIN_ROWS");
     static const long forced = v && *v ? std::atol(v) : -1;
-    if (forced == 0 || rows > 64 || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
+    // up to 64 rows everywhere; up to 128 on a Q4_0 matrix wide enough to give every compute unit a
+    // column tile (there the tiled GEMM, whose 64 x 128 workgroup tiles re-read X per tile, is slower)
+    const size_t max_rows = tensor_type == AFHIP_TYPE_Q4_0 && (out_dim + 31) / 32 >= static_cast<size_t>(gemv_compute_units()) ? 128 : 64;
+    if (forced == 0 || rows > max_rows || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
     if (forced > 0) return rows >= static_cast<size_t>(forced);
     if (rows < (in_dim > 4096 ? kBatchMfmaMinRows + 1 : kBatchMfmaMinRows)) return false;
     if (tensor_type == AFHIP_TYPE_Q8_0) {
@@ -327,7 +331,7 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
     const int chunk = gemv_row_chunk(rows, in_dim);
     const bool fused_ok = layout == AFHIP_LAYOUT_PREPARED && chunk > 0 && kind != AFHIP_DISPATCH_SCALAR &&
                           in_dim <= static_cast<size_t>(gemv_fused_max_in_dim());
-    // Five to 64 rows: the weights are read once, so the single-shot MFMA kernel (X quantized into
+    // Five to 64 (128) rows: the weights are read once, so the single-shot MFMA kernel (X quantized into
     // MFMA operand order first) beats both the row-by-row GEMV and the tiled GEMM.
     if (layout == AFHIP_LAYOUT_PREPARED && !want_dots && kind != AFHIP_DISPATCH_SCALAR &&
         batch_mfma_preferred(tensor_type, rows, in_dim, out_dim)) {
@@ -707,8 +711,8 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
     const size_t gemm_bytes = partial != 0 ? (base + 255) / 256 * 256 + partial : base;
     // small batches on a long K (also slices of eight rows of a forced plan): the K slices' sums, for a pair of matrices
     const size_t batch_bytes = gemv_batch_partial_bytes(rows < 8 ? rows : 8, in_dim, out_dim, true);
-    // up to 64 rows: X in MFMA operand order and the partial sums of K shares of the single-shot MFMA kernel
-    const size_t mfma_bytes = rows <= 64 ? batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim) : 0;
+    // up to 128 rows: X in MFMA operand order and the partial sums of K shares of the single-shot MFMA kernel
+    const size_t mfma_bytes = rows <= 128 ? batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim) : 0;
     size_t need = gemm_bytes > batch_bytes ? gemm_bytes : batch_bytes;
     return need > mfma_bytes ? need : mfma_bytes;
 }

@@ -1,4 +1,4 @@
-// Batched decode (a few to 64 rows) on CDNA4 int8 MFMA, activation-quantized route
+// Batched decode (a few to 128 rows) on CDNA4 int8 MFMA, activation-quantized route
 // (ops/native_compute.zig:13304-13478 for Q8_0, :23427-23775 for Q4_0):
 //   dot[m][n][b] = sum_i qx[m][32b+i] * qw[n][32b+i]            (int32, exact)
 //   y[m][n]      = sum_b (sx[m][b] * sw[n][b]) * f32(dot[m][n][b])
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
                                                                   int out_dim, int share_blocks, Epilogue ep) {
     using F = BmFormat<kType>;
     constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kPairs = kWB / 2;
-    constexpr int kAhead = kRowTiles == 1 ? 8 : 4;  // A fragments in registers per row tile
+    constexpr int kAhead = kRowTiles == 1 ? 8 : (kRowTiles == 2 ? 4 : 2);  // A fragments in registers per row tile
     static_assert(kWB % kAhead == 0 && kAhead % 2 == 0, "fragment ring");
     const int kb_full = in_dim >> 5;
     const int padded = kRowTiles * 32;
@@ -293,26 +293,28 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
         }
     }
 
-    // ---- 4. the wavefronts' sums meet in LDS (the weight regions are dead after the barrier)
-    __syncthreads();
-    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][rt][v][lane]
+    // ---- 4. the wavefronts' sums meet in LDS, one row tile at a time (the weight regions are dead
+    // after the first barrier; 8 wavefronts x 16 registers x 64 lanes of floats are half the LDS)
+    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][v][lane]
+    constexpr int kItems = kLive * 64;
 #pragma unroll
-    for (int rt = 0; rt < kRowTiles; ++rt)
+    for (int rt = 0; rt < kRowTiles; ++rt) {
+        __syncthreads();
 #pragma unroll
-        for (int v = 0; v < kLive; ++v) red[((wave * kRowTiles + rt) * kLive + v) * 64 + lane] = acc[rt][v];
-    __syncthreads();
-    constexpr int kItems = kRowTiles * kLive * 64;
-    for (int i = tid; i < kItems; i += kBmThreads) {
-        float sum = red[i];
+        for (int v = 0; v < kLive; ++v) red[(wave * kLive + v) * 64 + lane] = acc[rt][v];
+        __syncthreads();
+        for (int i = tid; i < kItems; i += kBmThreads) {
+            float sum = red[i];
 #pragma unroll
-        for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
-        const int l = i & 63, v = (i >> 6) % kLive, rt = (i >> 6) / kLive;
-        const int m = rt * 32 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-        const int n = n0 + (l & 31);
-        if (m < rows && n < out_dim) {
-            const size_t at = static_cast<size_t>(m) * out_dim + n;
-            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
-            else dst[at] = finish_output(ep, n, at, sum);
+            for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
+            const int l = i & 63, v = i >> 6;
+            const int m = rt * 32 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+            const int n = n0 + (l & 31);
+            if (m < rows && n < out_dim) {
+                const size_t at = static_cast<size_t>(m) * out_dim + n;
+                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                else dst[at] = finish_output(ep, n, at, sum);
+            }
         }
     }
 }
@@ -337,7 +339,9 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
     if (rows <= 16) AFHIP_BM(1, 8);
     if (rows <= 24) AFHIP_BM(1, 12);
     if (rows <= 32) AFHIP_BM(1, 16);
-    AFHIP_BM(2, 16);
+    if (rows <= 64) AFHIP_BM(2, 16);
+    if (rows <= 96) AFHIP_BM(3, 16);
+    AFHIP_BM(4, 16);
 #undef AFHIP_BM
 }
 
@@ -350,7 +354,7 @@ int bm_shares(int tensor_type, int in_dim) {
 
 bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     if (tensor_type != 2 && tensor_type != 8) return false;
-    if (rows < 1 || rows > 64 || in_dim == 0 || in_dim % 32 != 0 || out_dim == 0) return false;
+    if (rows < 1 || rows > 128 || in_dim == 0 || in_dim % 32 != 0 || out_dim == 0) return false;
     // 32-bit lane offsets relative to a column tile, grid.y
     if (in_dim > (1u << 22) || out_dim > 0x7fffffff) return false;
     return true;

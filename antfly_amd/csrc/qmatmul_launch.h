@@ -82,7 +82,7 @@ hipError_t launch_gemv_batch(hipStream_t stream, int tensor_type, float* dst, in
 int gemv_batch_waves(int rows, int in_dim, int groups);
 size_t gemv_batch_partial_bytes(size_t rows, size_t in_dim, size_t out_dim, bool pair);
 
-// Batched decode on int8 MFMA, 1..64 rows, PREPARED weights (batch_mfma_kernels.hip): quantizes X
+// Batched decode on int8 MFMA, 1..128 rows, PREPARED weights (batch_mfma_kernels.hip): quantizes X
 // into MFMA operand order in `workspace` (batch_mfma_workspace_bytes() bytes, 16-byte aligned), then one
 // single-shot launch per matrix (+ splitk_reduce_kernel when K exceeds one share).
 // compute units of the current device (cached)

@@ -123,6 +123,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # the single-shot MFMA kernel (5..64 rows): every count of live result registers, two row tiles, a K
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
+    (70, 512, 8200), (128, 1056, 8192), (97, 256, 8224),  # three and four row tiles (Q4_0 on a wide matrix)
 ]
 
 

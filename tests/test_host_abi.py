@@ -133,7 +133,7 @@ def test_linear_workspace_covers_every_kernel_family():
     more on a grid too small for the chip: behind the quantized activations, the partial sums of
     2, 4 or 8 K shares (at least 16 blocks each) of the tiled GEMM.  Up to eight rows (and
     eight-row slices of a forced plan) on a K longer than 4096: the sums of the K slices of the
-    small-batch kernel, for a pair of matrices.  Up to 64 rows: X in MFMA operand order (rows
+    small-batch kernel, for a pair of matrices.  Up to 128 rows: X in MFMA operand order (rows
     padded to 32), its scales, and the partial sums of the K shares (128 blocks of Q4_0, 64 of
     Q8_0 each) of the single-shot MFMA kernel."""
     def up256(v):
@@ -147,7 +147,7 @@ def test_linear_workspace_covers_every_kernel_family():
         return slices * min(rows, 8) * n * 4 * 2 if slices > 1 else 0
 
     def mfma(fmt, rows, k, n):
-        if rows > 64:
+        if rows > 128:
             return 0
         padded = (rows + 31) // 32 * 32
         share = 128 if fmt == _lib.TYPE_Q4_0 else 64
@@ -170,6 +170,7 @@ def test_linear_workspace_covers_every_kernel_family():
         assert kernels.workspaceBytes(fmt, 5, 14336, 4096) == max(quantized(5, 14336), batch(5, 14336, 4096), mfma(fmt, 5, 14336, 4096))
         assert batch(5, 14336, 4096) == 4 * 5 * 4096 * 4 * 2
     assert mfma(_lib.TYPE_Q4_0, 33, 4096, 512) == 64 * 4096 + 128 * 64 * 4
+    assert kernels.workspaceBytes(_lib.TYPE_Q4_0, 100, 4096, 8192) >= mfma(_lib.TYPE_Q4_0, 100, 4096, 8192) == 128 * 4096 + 128 * 128 * 4
     assert mfma(_lib.TYPE_Q8_0, 4, 4096, 512) == 32 * 4096 + 128 * 32 * 4 + 2 * 4 * 512 * 4
 
 
