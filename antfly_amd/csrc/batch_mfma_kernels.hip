@@ -63,6 +63,13 @@ __device__ __forceinline__ void bm_lds_load16(const void* base, uint32_t voff, u
 
 extern __shared__ __align__(16) unsigned char bm_lds[];
 
+// the second matrix of a pair launch (grid.z == 2)
+struct BmSecond {
+    float* dst;
+    const uint8_t* weight;
+    Epilogue ep;
+};
+
 // Program-order fence for the compiler (no instruction): what was computed into `a` so far is
 // finished before anything behind the fence starts.  Keeps the scheduler from running the MFMAs of
 // several blocks ahead and holding all their results in registers.
@@ -110,11 +117,17 @@ __global__ __launch_bounds__(256) void quantize_fragments_kernel(const float* __
 }
 
 template <int kType, int kRowTiles, int kLive>
-__global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma_kernel(float* __restrict__ dst, float* __restrict__ partial,
+__global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                   const uint32_t* __restrict__ qa, const float* __restrict__ sa,
-                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
-                                                                  int out_dim, int share_blocks, Epilogue ep) {
+                                                                  const uint8_t* __restrict__ weight_a, int rows, int in_dim,
+                                                                  int out_dim, int share_blocks, Epilogue ep_a, BmSecond second) {
     using F = BmFormat<kType>;
+    // blockIdx.z == 1: the second matrix of a pair (same X, same shape)
+    const bool is_b = blockIdx.z != 0;
+    float* dst = is_b ? second.dst : dst_a;
+    const uint8_t* weight = is_b ? second.weight : weight_a;
+    const Epilogue ep = is_b ? second.ep : ep_a;
+    float* partial = partial_a == nullptr ? nullptr : partial_a + (is_b ? static_cast<size_t>(gridDim.y) * rows * out_dim : 0);
     constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kPairs = kWB / 2;
     constexpr int kAhead = kRowTiles == 1 ? 8 : (kRowTiles == 2 ? 4 : 2);  // A fragments in registers per row tile
     static_assert(kWB % kAhead == 0 && kAhead % 2 == 0, "fragment ring");
@@ -323,18 +336,18 @@ namespace {
 
 template <int kType, int kRowTiles, int kLive>
 hipError_t bm_launch(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
-                     int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep) {
-    const dim3 grid(static_cast<unsigned>((out_dim + 31) / 32), static_cast<unsigned>(shares)), block(kBmThreads);
+                     int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+    const dim3 grid(static_cast<unsigned>((out_dim + 31) / 32), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
     hipLaunchKernelGGL((batch_mfma_kernel<kType, kRowTiles, kLive>), grid, block, kBmLdsBytes, stream, dst,
-                       shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep);
+                       shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep, second);
     return hipGetLastError();
 }
 
 template <int kType>
 hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
-                          int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep) {
+                          int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
 #define AFHIP_BM(TILES, LIVE) \
-    return bm_launch<kType, TILES, LIVE>(stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, shares, share_blocks, ep)
+    return bm_launch<kType, TILES, LIVE>(stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, shares, share_blocks, ep, second)
     if (rows <= 8) AFHIP_BM(1, 4);
     if (rows <= 16) AFHIP_BM(1, 8);
     if (rows <= 24) AFHIP_BM(1, 12);
@@ -360,13 +373,13 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
     return true;
 }
 
-// Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares]
+// Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares, for two matrices]
 size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return 0;
     const size_t padded = (rows + 31) / 32 * 32;
     const size_t shares = static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim)));
     const size_t front = padded * in_dim + (in_dim / 32) * padded * 4;
-    return (front + 255) / 256 * 256 + (shares > 1 ? shares * rows * out_dim * 4 : 0);
+    return (front + 255) / 256 * 256 + (shares > 1 ? 2 * shares * rows * out_dim * 4 : 0);  // (twice: a pair of matrices)
 }
 
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
@@ -393,16 +406,17 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
     const int real_shares = (kb + share_blocks - 1) / share_blocks;
     const size_t count = static_cast<size_t>(rows) * out_dim;
-    for (int which = 0; which < (weight_b_prepared ? 2 : 1); ++which) {
-        float* d = which ? dst_b : dst;
-        const uint8_t* w = which ? weight_b_prepared : weight_prepared;
-        const Epilogue& e_out = which ? ep_b : ep;
-        hipError_t e = tensor_type == 2
-                           ? bm_launch_rows<2>(stream, d, partial, qa, sa, w, rows, in_dim, out_dim, real_shares, share_blocks, e_out)
-                           : bm_launch_rows<8>(stream, d, partial, qa, sa, w, rows, in_dim, out_dim, real_shares, share_blocks, e_out);
+    // a pair is one launch over both matrices (grid.z)
+    const BmSecond second{dst_b, weight_b_prepared, ep_b};
+    hipError_t e = tensor_type == 2
+                       ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
+                       : bm_launch_rows<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
+    if (e != hipSuccess) return e;
+    if (real_shares > 1) {
+        e = launch_splitk_reduce(stream, dst, partial, count, out_dim, real_shares, ep);
         if (e != hipSuccess) return e;
-        if (real_shares > 1) {
-            e = launch_splitk_reduce(stream, d, partial, count, out_dim, real_shares, e_out);
+        if (weight_b_prepared) {
+            e = launch_splitk_reduce(stream, dst_b, partial + static_cast<size_t>(real_shares) * count, count, out_dim, real_shares, ep_b);
             if (e != hipSuccess) return e;
         }
     }

@@ -135,7 +135,7 @@ def test_linear_workspace_covers_every_kernel_family():
     eight-row slices of a forced plan) on a K longer than 4096: the sums of the K slices of the
     small-batch kernel, for a pair of matrices.  Up to 128 rows: X in MFMA operand order (rows
     padded to 32), its scales, and the partial sums of the K shares (128 blocks of Q4_0, 64 of
-    Q8_0 each) of the single-shot MFMA kernel."""
+    Q8_0 each) of the single-shot MFMA kernel, for a pair of matrices."""
     def up256(v):
         return (v + 255) // 256 * 256
 
@@ -152,7 +152,7 @@ def test_linear_workspace_covers_every_kernel_family():
         padded = (rows + 31) // 32 * 32
         share = 128 if fmt == _lib.TYPE_Q4_0 else 64
         shares = (k // 32 + share - 1) // share
-        return up256(padded * k + (k // 32) * padded * 4) + (shares * rows * n * 4 if shares > 1 else 0)
+        return up256(padded * k + (k // 32) * padded * 4) + (2 * shares * rows * n * 4 if shares > 1 else 0)
 
     for fmt in (_lib.TYPE_Q4_0, _lib.TYPE_Q8_0):
         for rows, k, n in [(16, 4096, 4096), (64, 14336, 4096), (9, 1024, 64), (128, 4096, 1024)]:
@@ -171,7 +171,7 @@ def test_linear_workspace_covers_every_kernel_family():
         assert batch(5, 14336, 4096) == 4 * 5 * 4096 * 4 * 2
     assert mfma(_lib.TYPE_Q4_0, 33, 4096, 512) == 64 * 4096 + 128 * 64 * 4
     assert kernels.workspaceBytes(_lib.TYPE_Q4_0, 100, 4096, 8192) >= mfma(_lib.TYPE_Q4_0, 100, 4096, 8192) == 128 * 4096 + 128 * 128 * 4
-    assert mfma(_lib.TYPE_Q8_0, 4, 4096, 512) == 32 * 4096 + 128 * 32 * 4 + 2 * 4 * 512 * 4
+    assert mfma(_lib.TYPE_Q8_0, 4, 4096, 512) == 32 * 4096 + 128 * 32 * 4 + 2 * 2 * 4 * 512 * 4
 
 
 def test_zig_backend_sources_bind_what_exists():
