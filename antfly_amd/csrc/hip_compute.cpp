@@ -219,8 +219,11 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         }
     }
     afhip_buffer scratch{0, 0};
-    if (weight->quant_type == AFHIP_TYPE_Q4_K) {  // scratch for the split of X when the prefill GEMM serves the rows
-        const size_t need = weight->layout == AFHIP_LAYOUT_PREPARED ? afhip_linear_workspace_bytes(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim) : 0;
+    if (weight->quant_type == AFHIP_TYPE_Q4_K) {
+        // scratch for the split of X when the prefill GEMM serves the rows (repacked tensors), or for the Q8_K
+        // activations on the gated short-K shapes (either layout)
+        const bool needs = weight->layout == AFHIP_LAYOUT_PREPARED || afhip_uses_q8k_activation_quant(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim);
+        const size_t need = needs ? afhip_linear_workspace_bytes(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim) : 0;
         if (need) s = acquire_scratch(self, need, &scratch);
     } else if (afhip_uses_activation_quant(rows, in_dim, out_dim)) {  // scratch for separately quantized activations
         s = acquire_scratch(self, afhip_linear_workspace_bytes(weight->quant_type, rows, in_dim, out_dim), &scratch);

@@ -275,6 +275,9 @@ def test_backend_ops_on_q4_k():
         ref_last = O.linear_q4_k_q8k(x[-1:], w, 1, in_dim, out_dim)[0]
         assert G.max_rel_err(last[None, :], ref_last[None, :].astype(np.float64)) <= TIGHT
         assert token == O.argmax(ref_last) or ref_last.max() - ref_last[token] <= TIGHT * np.abs(ref_last).max()
+        # the same gated shape on the tensor kept in the GGUF layout (the backend lends the Q8_K scratch there too)
+        raw_last = cb.toFloat32(cb.linearNoBias(cb.fromFloat32(x[-1:].copy(), [1, in_dim]), cb.getWeight("raw.weight"), 1, in_dim, out_dim))
+        assert G.max_rel_err(raw_last.reshape(1, out_dim), ref_last[None, :].astype(np.float64)) <= TIGHT
         emb = cb.toFloat32(cb.embeddingLookup(wt, [999, 0], 2, in_dim)).reshape(2, in_dim)
         assert np.array_equal(emb.view(np.uint32), O.dequantize_q4_k(w).reshape(out_dim, in_dim)[[999, 0]].view(np.uint32))
         with pytest.raises(_lib.InvalidHipState):
