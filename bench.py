@@ -69,7 +69,7 @@ def main() -> int:
                     help="the timed region (exactly --steps steps) is run this many times; the median run is reported")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
-                         "read kernel and of the plain copy kernel over the same number of bytes, of the Q8_0 M=512 GEMM and of the Q4_K kernels "
+                         "read kernel and of the plain copy kernel over the same number of bytes, of the Q8_0 M=512 GEMM, of the 16-row batch kernel and of the Q4_K kernels "
                          "(M=1 and M=512), then exit")
     ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048"], default=None,
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
@@ -485,6 +485,13 @@ def main() -> int:
         sg = torch.empty(kernels.workspaceBytes(Q8, 512, 4096, 4096), dtype=torch.uint8, device=dev)
         for i in range(n_launch):
             launch(stream, Q8, _lib.LAYOUT_PREPARED, buf(yg), buf(xg), buf(wg[i % 2]), 512, 4096, 4096, buf(sg), -1)
+        torch.cuda.synchronize()
+        # batched decode, 16 rows on the FFN matrix: fragment quantizer + single-shot MFMA kernel
+        xb = torch.from_numpy(synth.activations(9, 16, 4096)).to(dev)
+        yb = torch.empty((16, 14336), dtype=torch.float32, device=dev)
+        sb = torch.empty(kernels.workspaceBytes(Q4, 16, 4096, 14336), dtype=torch.uint8, device=dev)
+        for i in range(n_launch):
+            launch(stream, Q4, _lib.LAYOUT_PREPARED, buf(yb), buf(xb), buf(ws[i % copies]), 16, 4096, 14336, buf(sb), -1)
         torch.cuda.synchronize()
         # Q4_K on the same matrix: the decode kernel (one row) and the prefill GEMM (512 rows)
         wk = prepared_copies(Q4K, 14336, 4096, copies, 31)
