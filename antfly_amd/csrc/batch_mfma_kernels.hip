@@ -28,7 +28,11 @@
 //   * The eight wavefronts' sums meet in LDS in wavefront order (y is a fixed-order sum of eight
 //     block-ascending partial sums); K shares of a long K go to partial[share][rows][out_dim]
 //     and splitk_reduce_kernel adds them in share order.
+//   * Up to eight rows on a grid that fills the chip take batch8_mfma_kernel (further down): the
+//     16x16x64 MFMA on two blocks at once, 32- or 64-column tiles, weights requested two stages
+//     ahead instead of all at once.
 #include <hip/hip_runtime.h>
+#include <type_traits>
 
 #include "device_common.h"
 #include "gemv_common.h"
@@ -304,6 +308,8 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
                 }
             }
         }
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // its weight loads still write LDS, which the sums are about to reuse
     }
 
     // ---- 4. the wavefronts' sums meet in LDS, one row tile at a time (the weight regions are dead
@@ -328,6 +334,314 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
                 if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
                 else dst[at] = finish_output(ep, n, at, sum);
             }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Up to eight rows: v_mfma_i32_16x16x64_i8 on two blocks at once.
+//
+// The instruction multiplies 16 rows x 64 k by 64 k x 16 columns, twice the k of one block, and two
+// blocks cannot share an int32 sum (their scales differ).  With at most eight rows the A operand has
+// room to keep them apart: A row 8 * s + r (s = 0, 1) is row r of X with the bytes of block 2P + s
+// in its k half s and ZEROS in the other half, the B operand is the weights of block 2P in k half 0
+// and of block 2P + 1 in k half 1.  Result row 8 * s + r is then exactly the dot of row r with block
+// 2P + s: one instruction of a quarter of the 32x32x32 one's work gives the dots of two blocks for
+// 16 columns, and all four of its result registers are live (lane l: column l % 16, lane group
+// g = l / 16: block 2P + g / 2, rows 4 * (g % 2) + v).
+//
+// The scale products sx[row][block] * sw[column][block] come in the same register layout from one
+// v_mfma_f32_16x16x4_f32: A row 8 * s + r carries sx of (r, block 2P + s) at k = s and zeros
+// elsewhere, B row k carries sw of block 2P + k (k < 2): every entry is one product plus zeros,
+// the correctly rounded f32 product.  What is left for the vector unit per MFMA is the nibble
+// unpacking, four conversions and four fused multiply-adds; the LDS sees one read.  (Fetching the
+// row scales per result register through the lane-exchange crossbar instead made the LDS pipe, one
+// per compute unit, the bottleneck.)
+//
+// The smaller column granule also makes four load stages of a wavefront's eight 1 KB units instead
+// of two: (blocks first half, columns 0..15), (first half, 16..31), (second half, 0..15), (second
+// half, 16..31), each waited for by itself, so that a quarter of the arithmetic, not half, is left
+// when the last byte arrives.
+
+// X f32 [rows <= 8][in_dim] -> qa8: [pair P][32 entries][16 bytes], sa8: f32 [pair][16].
+// Entry 16 * s + 8 * h + r holds sixteen int8 of row r, block 2P + s, k half h, in the k order of the
+// weight operand (below): what lane 16 * (2 s + h) + 8 * s + r of the A operand needs; the other lanes
+// of the operand are zeros and are not stored.  Slot 8 * s + r of sa8 is the block's scale.  Rows
+// past `rows` and a block past the last one are zeros with scale 0.  Same scale, reciprocal and
+// rounding as quantize_fragments_kernel.
+// k order, lane half h = g % 2:  Q8_0: values [16 h, 16 h + 16).  Q4_0: dwords x[8h..8h+3],
+// x[16+8h..+3], x[8h+4..8h+7], x[16+8h+4..+7] -- the low and the high nibbles of bytes [8 h, 8 h + 8) of
+// the block, dword by dword, so that one lane unpacks whole bytes.
+template <int kType>
+__global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* __restrict__ x, int rows, int in_dim,
+                                                                   uint32_t* __restrict__ qa8, float* __restrict__ sa8) {
+    const int kb = in_dim >> 5, slots = ((kb + 1) >> 1) * 2;  // block slots: whole pairs
+    const int units = 8 * slots * 8;                           // (row, block slot, eight lanes)
+    for (int u = blockIdx.x * blockDim.x + threadIdx.x; u < units; u += gridDim.x * blockDim.x) {
+        const int j = u & 7, bs = (u >> 3) % slots, r = (u >> 3) / slots;
+        const bool real = r < rows && bs < kb;
+        float4 v = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (real) v = reinterpret_cast<const float4*>(x)[(static_cast<size_t>(r) * in_dim >> 2) + bs * 8 + j];
+        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        m = max_over_8(m);
+        const float s = act_scale(m);
+        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
+        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+        const int pair = bs >> 1, hs = bs & 1, i = hs * 8 + r;
+        // values [4 j, 4 j + 4) of the block: which 16-byte half, which dword of it
+        const int h2 = kType == 2 ? (j >> 1) & 1 : j >> 2;
+        const int dw = kType == 2 ? 2 * (j & 1) + (j >> 2) : j & 3;
+        // entry 16 * s + 8 * h2 + r of the pair: sixteen bytes
+        qa8[static_cast<size_t>(pair) * 128 + (16 * hs + 8 * h2 + r) * 4 + dw] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        if (j == 0) sa8[pair * 16 + i] = real ? s : 0.0f;
+    }
+}
+
+template <int kType, int kCG>
+__global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
+                                                                     const uint32_t* __restrict__ qa8, const float* __restrict__ sa8,
+                                                                     const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
+                                                                     int share_blocks, Epilogue ep_a, BmSecond second) {
+    using F = BmFormat<kType>;
+    const bool is_b = blockIdx.z != 0;
+    float* dst = is_b ? second.dst : dst_a;
+    const uint8_t* weight = is_b ? second.weight : weight_a;
+    const Epilogue ep = is_b ? second.ep : ep_a;
+    float* partial = partial_a == nullptr ? nullptr : partial_a + (is_b ? static_cast<size_t>(gridDim.y) * rows * out_dim : 0);
+    constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kPairs = kWB / 2, kHalfPairs = kPairs / 2;
+    constexpr int kCols = 16 * kCG, kStages = 2 * kCG, kSteps = kStages * kHalfPairs;
+    const int kb_full = in_dim >> 5, pairs_total = (kb_full + 1) >> 1;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l16 = lane & 15, g = lane >> 4, par = g >> 1, kh = g & 1;  // column, lane group, block parity, k half
+    const int n0 = blockIdx.x * kCols;
+    const int share_begin = static_cast<int>(blockIdx.y) * share_blocks;  // a multiple of kWB: even
+    const int share_end = min(share_begin + share_blocks, kb_full);
+    const int blk0 = share_begin + wave * kWB;
+    const int nb = max(0, min(kWB, share_end - blk0));
+    const int last = blk0 + max(nb, 1) - 1 < kb_full ? blk0 + max(nb, 1) - 1 : kb_full - 1;
+    auto clamp_blk = [&](int j) { return min(blk0 + j, last); };
+    const size_t blocks_total = static_cast<size_t>(out_dim) * kb_full;
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(bm_lds))) + wave * kBmWaveBytes;
+
+    // ---- 1. loads.  Stage s = (half hb = s / kCG of the wavefront's blocks, column group cg =
+    // s % kCG) is two 1 KB units of weights (8 columns x 8 chunks each), written to slot s % 4 of
+    // the wavefront's 8 KB of LDS.  What a compute unit can keep in flight is a small part of what
+    // its wavefronts want, and a wavefront that cannot issue a load cannot compute either, so a
+    // wavefront requests two stages ahead of the one it works on, not everything at once.
+    // The first stage goes out first (a compute unit has one address unit and all its wavefronts
+    // queue there), then what goes to registers, kept small: one or two 4-byte loads for the row
+    // scales of the wavefront's pairs, an 8-byte load per column group for the weight scales, the
+    // operand fragments in their compact form (two pairs a load), two spares; then the second stage.
+    // A wavefront's loads complete in the order issued, so "all but the youngest n have completed"
+    // says that a stage is there.  The compiler counts only its own loads when it waits for one of
+    // them, which can only be too strict: it retires as many more of the oldest younger loads as
+    // there are loads it does not know of (two at that point: the second stage).  The two spare
+    // loads are those (they are looked at once, after the loop).
+    auto issue_stage = [&](int st) {
+        const int hb = st / kCG, cg = st % kCG;
+        const uint8_t* wbase = weight + static_cast<size_t>(n0) * kb_full * kQB;
+        const int c8 = lane >> 3, slot = lane & 7;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int c = 16 * cg + 8 * u + c8;
+            const int chunk = slot ^ ((c >> 1) & 7);
+            const int cc = min(n0 + c, out_dim - 1) - n0;
+            uint32_t off;
+            if (kType == 2) {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(8 * hb + chunk)) * 16u;
+            } else {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(4 * hb + (chunk >> 1))) * 32u + (chunk & 1) * 16u;
+            }
+            bm_lds_load16(wbase, off, lds_wave + ((st & 3) * 2 + u) * 1024);
+        }
+    };
+    issue_stage(0);
+    const int pair0 = blk0 >> 1;
+    // row scales: 64 bytes a pair; lane L of load q takes slot L % 16 of pair 4 q + L / 16
+    constexpr int kScaleLoads = (kPairs + 3) / 4;
+    float sx_part[kScaleLoads];
+#pragma unroll
+    for (int q = 0; q < kScaleLoads; ++q)
+        sx_part[q] = sa8[min(pair0 + 4 * q + g, pairs_total - 1) * 16 + l16];
+    // weight scales, fp16 in block order (rows of whole 16-byte runs: the host sends no other shape
+    // here): word p of a column's run holds blocks 2p and 2p + 1; lane group g takes words
+    // [g * kWpl, +kWpl) and the lane exchange hands word p out when its stage comes
+    constexpr int kWpl = kPairs / 4;
+    uint32_t tb_part[kCG][kWpl];
+#pragma unroll
+    for (int cg = 0; cg < kCG; ++cg) {
+        const int cc = min(n0 + 16 * cg + l16, out_dim - 1);
+        const uint16_t* sw = reinterpret_cast<const uint16_t*>(weight + blocks_total * kQB) + static_cast<size_t>(cc) * kb_full;
+        const uint32_t* run = reinterpret_cast<const uint32_t*>(sw + min(blk0, kb_full - 8)) + g * kWpl;
+        if constexpr (kWpl == 2) {
+            const uint2 v = *reinterpret_cast<const uint2*>(run);
+            tb_part[cg][0] = v.x;
+            tb_part[cg][1] = v.y;
+        } else {
+            tb_part[cg][0] = run[0];
+        }
+    }
+    // operand fragments, compact: 512 bytes a pair, two pairs a load; lane L of load q holds entry
+    // L % 32 of pair 2 q + L / 32
+    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa8);
+    bm_v4i packed[kPairs / 2];
+#pragma unroll
+    for (int q = 0; q < kPairs / 2; ++q) {
+        packed[q] = qa4[static_cast<size_t>(min(pair0 + 2 * q + (lane >> 5), pairs_total - 1)) * 32 + (lane & 31)];
+    }
+    constexpr int kSpares = 2;
+    uint32_t spare[kSpares];
+#pragma unroll
+    for (int k = 0; k < kSpares; ++k) spare[k] = __builtin_nontemporal_load(qa8 + k * 32 + (lane & 31));  // inside the first pair's entries
+    constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
+#pragma unroll
+    for (int st = 1; st < kAheadStages; ++st) issue_stage(st);
+
+    // this lane's B operand: column 16 * cg + l16, block 2p + par, k half kh.  Q8_0: bytes
+    // [16 kh, +16) of the block.  Q4_0: bytes [8 kh, +8), low nibbles and high nibbles dword by
+    // dword; a nibble n stands for n - 8: with bit 3 flipped and in the high half of a byte it reads as
+    // the int8 16 * (n - 8).  Its address inside a stage's slot (the column group does not enter:
+    // 16 columns are two whole units and the swizzle repeats every 16 columns).
+    uint32_t baddr[kHalfPairs];
+#pragma unroll
+    for (int q = 0; q < kHalfPairs; ++q) {
+        const int j = 2 * q + par;
+        const int unit = l16 >> 3, row = (l16 & 7) * 8, swz = (l16 >> 1) & 7;
+        const int chunk = kType == 2 ? j : j * 2 + kh;
+        baddr[q] = lds_wave + (unit * 64 + row + (chunk ^ swz)) * 16 + (kType == 2 ? 8 * kh : 0);
+    }
+
+    float acc[kCG][4];
+#pragma unroll
+    for (int cg = 0; cg < kCG; ++cg)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[cg][v] = 0.0f;
+
+    // ---- 2. the stages, software-pipelined by hand over the steps (one step = a pair of blocks,
+    // sixteen columns: one int8 MFMA and one scale-product MFMA).  A step's weight bytes are
+    // requested from LDS one step ahead and its results are scaled one step behind, after the next
+    // MFMAs have been issued: no step waits for the LDS or for the matrix unit's latency.  (The
+    // weight bytes of a stage's first step cannot be requested before the stage is there.)  The
+    // scheduling barriers keep the compiler from undoing that order.
+    if (nb > 0) {
+        typedef unsigned bm_v2u __attribute__((ext_vector_type(2)));
+        typedef unsigned bm_v4u __attribute__((ext_vector_type(4)));
+        typedef typename std::conditional<kType == 2, bm_v2u, bm_v4u>::type Raw;
+        typedef float bm_v4f __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) const Raw LdsRaw;
+        Raw raw[2];
+        bm_v4i afrag[kHalfPairs];
+        float sxm[kHalfPairs], tbm[kHalfPairs];
+        bm_v4i cres[2];
+        bm_v4f tres[2];
+        auto stage_of = [&](int it) { return it / kHalfPairs; };
+        auto fetch_weights = [&](int it) { raw[it & 1] = *reinterpret_cast<LdsRaw*>(baddr[it % kHalfPairs] + (stage_of(it) & 3) * 2048); };
+        auto scale = [&](int it) {
+            const int cg = stage_of(it) % kCG;
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[cg][v] = __builtin_fmaf(tres[it & 1][v], static_cast<float>(cres[it & 1][v]), acc[cg][v]);
+        };
+#pragma unroll
+        for (int it = 0; it < kSteps; ++it) {
+            if (it % kHalfPairs == 0) {
+                const int st = stage_of(it), hb = st / kCG, cg = st % kCG;
+                if (st == 0) {
+                    // everything older than the second stage: the first stage and all the register loads
+                    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * (kAheadStages - 1)) : "memory");
+#pragma unroll
+                    for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(packed[q]));
+#pragma unroll
+                    for (int c = 0; c < kCG; ++c) asm volatile("" : "+v"(tb_part[c][0]), "+v"(tb_part[c][kWpl - 1]));
+                    asm volatile("" : "+v"(sx_part[0]), "+v"(sx_part[kScaleLoads - 1]));
+                }
+                if (st + kAheadStages < kStages) issue_stage(st + kAheadStages);
+                // operands of this stage's scale products (in the shadow of the wait below).
+                // A: lane (slot i = l16, k = g) carries sx of slot i if k is the slot's block (i / 8), else 0
+                // B: lane (column l16, k = g) carries sw of block 2p + k for k < 2 (zero if that block is not
+                //    this wavefront's: a clamped re-read of the last block counts for nothing), else 0;
+                //    Q4_0: times 1/16, the nibbles enter the dots as 16 * (n - 8)
+#pragma unroll
+                for (int q = 0; q < kHalfPairs; ++q) {
+                    const int p = hb * kHalfPairs + q;
+                    const uint32_t word = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(4 * (16 * (p / kWpl) + l16), static_cast<int>(tb_part[cg][p % kWpl])));
+                    const float sw = half_bits_to_f32(static_cast<uint16_t>(word >> (16 * kh))) * (kType == 2 ? 0.0625f : 1.0f);
+                    tbm[q] = (g < 2 && 2 * p + g < nb) ? sw : 0.0f;
+                }
+                if (cg == 0) {
+                    // first stage of a half: the half's row scales and A operands.  Lane (g, slot i) takes
+                    // entry 8 g + i % 8 of its pair through the lane exchange if the slot's block is the lane
+                    // group's, else zeros
+#pragma unroll
+                    for (int q = 0; q < kHalfPairs; ++q) {
+                        const int p = hb * kHalfPairs + q;
+                        const float sx = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (16 * (p & 3) + l16), __float_as_int(sx_part[p >> 2])));
+                        sxm[q] = g == (l16 >> 3) ? sx : 0.0f;
+                        const int from = 4 * (32 * (p & 1) + 8 * g + (l16 & 7));
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const int got = __builtin_amdgcn_ds_bpermute(from, packed[p >> 1][d]);
+                            afrag[q][d] = (l16 >> 3) == par ? got : 0;
+                        }
+                    }
+                }
+                // this stage is there when at most the stages requested behind it are in flight
+                {
+                    const int younger = 2 * ((kStages - 1 - st) < kAheadStages ? (kStages - 1 - st) : kAheadStages);
+                    if (younger == 6) asm volatile("s_waitcnt vmcnt(6)" : : : "memory");
+                    else if (younger == 4) asm volatile("s_waitcnt vmcnt(4)" : : : "memory");
+                    else if (younger == 2) asm volatile("s_waitcnt vmcnt(2)" : : : "memory");
+                    else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+                }
+                fetch_weights(it);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (it + 1 < kSteps && (it + 1) % kHalfPairs != 0) fetch_weights(it + 1);
+            bm_v4i b;
+            {
+                const Raw w = raw[it & 1];
+                if constexpr (kType == 2) {
+                    const uint32_t x = w[0] ^ 0x88888888u, y = w[1] ^ 0x88888888u;
+                    b = bm_v4i{static_cast<int>((x << 4) & 0xF0F0F0F0u), static_cast<int>(x & 0xF0F0F0F0u), static_cast<int>((y << 4) & 0xF0F0F0F0u),
+                               static_cast<int>(y & 0xF0F0F0F0u)};
+                } else {
+                    b = bm_v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[kType == 2 ? 0 : 2]), static_cast<int>(w[kType == 2 ? 1 : 3])};
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            const int q = it % kHalfPairs;
+            cres[it & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[q], b, bm_v4i{0, 0, 0, 0}, 0, 0, 0);
+            tres[it & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(sxm[q], tbm[q], bm_v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (it > 0) scale(it - 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        scale(kSteps - 1);
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may still be writing LDS when the region is reused
+    }
+    asm volatile("" : : "v"(spare[0]), "v"(spare[1]));
+
+    // ---- 3. the wavefronts' sums (and the two block parities) meet in LDS
+    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][cg * 4 + v][lane]
+    __syncthreads();
+#pragma unroll
+    for (int cg = 0; cg < kCG; ++cg)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[(wave * kCG * 4 + cg * 4 + v) * 64 + lane] = acc[cg][v];
+    __syncthreads();
+    if (tid < 8 * kCols) {
+        const int m = tid / kCols, c = tid % kCols;
+        const int item = ((c >> 4) * 4 + (m & 3)) * 64 + 16 * (m >> 2) + (c & 15);
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kBmWaves; ++w) sum += red[w * kCG * 256 + item] + red[w * kCG * 256 + item + 32];
+        const int n = n0 + c;
+        if (m < rows && n < out_dim) {
+            const size_t at = static_cast<size_t>(m) * out_dim + n;
+            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+            else dst[at] = finish_output(ep, n, at, sum);
         }
     }
 }
@@ -358,9 +672,32 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
 #undef AFHIP_BM
 }
 
+template <int kType, int kCG>
+hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
+                      int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+    const dim3 grid(static_cast<unsigned>((out_dim + 16 * kCG - 1) / (16 * kCG)), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
+    hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows,
+                       in_dim, out_dim, share_blocks, ep, second);
+    return hipGetLastError();
+}
+
+// Column groups of sixteen a workgroup takes: four (64 columns: the activations' share of a
+// workgroup's traffic and a wavefront's set-up halve) where that still gives most compute units a
+// workgroup, else two.
+int bm8_column_groups(int out_dim) { return (out_dim + 63) / 64 >= gemv_compute_units() * 3 / 4 ? 4 : 2; }
+
 int bm_shares(int tensor_type, int in_dim) {
     const int share_max = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
     return (in_dim / 32 + share_max - 1) / share_max;
+}
+
+// The eight-row kernel: at most eight rows, rows of whole 16-byte runs of weight scales, and at
+// least a workgroup per compute unit (32-column tiles times K shares) -- on a smaller grid the
+// memory system is not the limit and the shorter dependency chain of batch_mfma_kernel wins.
+bool bm8_preferred(int tensor_type, int rows, int in_dim, int out_dim) {
+    const int kb = in_dim / 32;
+    if (rows > 8 || kb % 8 != 0) return false;
+    return static_cast<long>((out_dim + 31) / 32) * bm_shares(tensor_type, in_dim) >= gemv_compute_units();
 }
 
 }  // namespace
@@ -391,7 +728,18 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(padded) * in_dim);
     const size_t front = static_cast<size_t>(padded) * in_dim + static_cast<size_t>(kb) * padded * 4;
     float* partial = reinterpret_cast<float*>(workspace + (front + 255) / 256 * 256);
-    {
+    const bool eight = bm8_preferred(tensor_type, rows, in_dim, out_dim);  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
+    if (eight) {
+        const int pairs = (kb + 1) / 2;
+        sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
+        const int units = 8 * (2 * pairs) * 8;
+        const dim3 qgrid(static_cast<unsigned>((units + 255) / 256));
+        if (tensor_type == 2)
+            hipLaunchKernelGGL(quantize_fragments8_kernel<2>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+        else
+            hipLaunchKernelGGL(quantize_fragments8_kernel<8>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+        if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    } else {
         const size_t units = static_cast<size_t>(padded) * (in_dim / 4);
         size_t grid = (units + 255) / 256;
         if (grid > 4096) grid = 4096;
@@ -408,7 +756,15 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const size_t count = static_cast<size_t>(rows) * out_dim;
     // a pair is one launch over both matrices (grid.z)
     const BmSecond second{dst_b, weight_b_prepared, ep_b};
-    hipError_t e = tensor_type == 2
+    hipError_t e;
+    if (eight) {
+        const bool wide = bm8_column_groups(out_dim) == 4;
+#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
+        e = tensor_type == 2 ? (wide ? AFHIP_BM8(2, 4) : AFHIP_BM8(2, 2)) : (wide ? AFHIP_BM8(8, 4) : AFHIP_BM8(8, 2));
+#undef AFHIP_BM8
+    }
+    else
+        e = tensor_type == 2
                        ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
                        : bm_launch_rows<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
     if (e != hipSuccess) return e;

@@ -23,7 +23,8 @@ TIGHT = 2e-5
 # kernel, both MFMA tiles, ragged columns, the f32 route
 SHAPES = [(1, 4096, 1024), (1, 512, 514), (2, 2048, 640), (4, 1024, 600), (5, 8224, 513), (8, 4096, 512),
           (12, 256, 530), (40, 512, 640), (300, 512, 1024), (3, 64, 100),
-          (20, 2048, 300), (33, 8224, 200)]  # MFMA GEMM with K shared out over workgroups: the reduce kernel adds the bias
+          (20, 2048, 300), (33, 8224, 200),  # MFMA GEMM with K shared out over workgroups: the reduce kernel adds the bias
+          (7, 512, 8200), (5, 9216, 4112)]  # the eight-row MFMA kernel; with K shares (the reduce kernel adds the bias)
 
 
 def bias_vector(seed, out_dim):
@@ -116,7 +117,7 @@ def linear_epilogue(fmt, layout, x, w_dev, rows, in_dim, out_dim, bias=None, res
 
 
 EPILOGUE_SHAPES = [(1, 4096, 1024), (1, 8224, 513), (3, 1024, 600), (6, 2048, 640), (40, 512, 640), (300, 512, 1024), (20, 2048, 300),
-                   (3, 64, 100)]
+                   (3, 64, 100), (6, 512, 8200)]
 
 
 @pytest.mark.parametrize("fmt", [Q8, Q4, Q4K])

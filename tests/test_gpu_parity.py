@@ -124,6 +124,10 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
     (70, 512, 8200), (128, 1056, 8192), (97, 256, 8224),  # three and four row tiles (Q4_0 on a wide matrix)
+    # the eight-row MFMA kernel (5..8 rows on a grid of at least a workgroup per compute unit): one live
+    # wavefront and a ragged last tile; 64-column tiles, ragged; K shares with a short last share; a
+    # wavefront with half its blocks
+    (8, 512, 8200), (5, 4096, 12290), (7, 9216, 4112), (6, 256, 16416),
 ]
 
 
@@ -189,6 +193,7 @@ def test_forced_dispatch_kinds_agree(fmt, rows):
 PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K slices, ragged columns, MFMA GEMM, f32 route
     (1, 4096, 1024), (2, 512, 514), (4, 2048, 640), (5, 8224, 513), (8, 4096, 512), (12, 256, 530), (40, 512, 640),
     (3, 64, 100), (20, 2048, 300),  # the last: MFMA GEMM with K shared out over workgroups, both matrices through one scratch
+    (6, 512, 8200), (7, 9216, 4112),  # the eight-row MFMA kernel, one launch over both matrices; with K shares
 ]
 
 
