@@ -107,7 +107,8 @@ static int env_int(const char* name) {
 // AFHIP_BATCH_MFMA_MIN_ROWS overrides the lower row bound for tuning runs, 0 switches the kernel off):
 // from five rows on (six on a K longer than 4096, where the split-K GEMV still wins at five) up to 64
 // (128 on wide Q4_0 matrices), and for Q8_0, whose K shares are half as long, only while all workgroups
-// of the launch are resident at once.
+// of the launch are resident at once.  Five to eight rows on a grid that fills the chip always:
+// its eight-row kernel requests weights as it goes and needs neither condition.
 static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     static const char* v = std::getenv("AFHIP_BATCH_MFMA_MIN_ROWS");
     static const long forced = v && *v ? std::atol(v) : -1;
@@ -116,6 +117,7 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
     const size_t max_rows = tensor_type == AFHIP_TYPE_Q4_0 && (out_dim + 31) / 32 >= static_cast<size_t>(gemv_compute_units()) ? 128 : 64;
     if (forced == 0 || rows > max_rows || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
     if (forced > 0) return rows >= static_cast<size_t>(forced);
+    if (rows >= kBatchMfmaMinRows && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
     if (rows < (in_dim > 4096 ? kBatchMfmaMinRows + 1 : kBatchMfmaMinRows)) return false;
     if (tensor_type == AFHIP_TYPE_Q8_0) {
         const size_t shares = (in_dim / 32 + 63) / 64, tiles = (out_dim + 31) / 32;

@@ -691,15 +691,6 @@ int bm_shares(int tensor_type, int in_dim) {
     return (in_dim / 32 + share_max - 1) / share_max;
 }
 
-// The eight-row kernel: at most eight rows, rows of whole 16-byte runs of weight scales, and at
-// least a workgroup per compute unit (32-column tiles times K shares) -- on a smaller grid the
-// memory system is not the limit and the shorter dependency chain of batch_mfma_kernel wins.
-bool bm8_preferred(int tensor_type, int rows, int in_dim, int out_dim) {
-    const int kb = in_dim / 32;
-    if (rows > 8 || kb % 8 != 0) return false;
-    return static_cast<long>((out_dim + 31) / 32) * bm_shares(tensor_type, in_dim) >= gemv_compute_units();
-}
-
 }  // namespace
 
 bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
@@ -708,6 +699,16 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
     // 32-bit lane offsets relative to a column tile, grid.y
     if (in_dim > (1u << 22) || out_dim > 0x7fffffff) return false;
     return true;
+}
+
+// The eight-row kernel: at most eight rows, rows of whole 16-byte runs of weight scales, and at
+// least a workgroup per compute unit (32-column tiles times K shares) -- on a smaller grid the
+// memory system is not the limit and the shorter dependency chain of batch_mfma_kernel wins.
+bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+    if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
+    const size_t kb = in_dim / 32;
+    if (rows > 8 || kb % 8 != 0) return false;
+    return (out_dim + 31) / 32 * static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim))) >= static_cast<size_t>(gemv_compute_units());
 }
 
 // Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares, for two matrices]
@@ -728,7 +729,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(padded) * in_dim);
     const size_t front = static_cast<size_t>(padded) * in_dim + static_cast<size_t>(kb) * padded * 4;
     float* partial = reinterpret_cast<float*>(workspace + (front + 255) / 256 * 256);
-    const bool eight = bm8_preferred(tensor_type, rows, in_dim, out_dim);  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
+    const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
     if (eight) {
         const int pairs = (kb + 1) / 2;
         sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);

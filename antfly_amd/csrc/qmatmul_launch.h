@@ -88,6 +88,8 @@ size_t gemv_batch_partial_bytes(size_t rows, size_t in_dim, size_t out_dim, bool
 // compute units of the current device (cached)
 int gemv_compute_units();
 bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
+// whether launch_batch_mfma takes its eight-row kernel for this shape (the faster one where it applies)
+bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
                              int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b = nullptr,
