@@ -233,9 +233,16 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
     for (int rt = 0; rt < kRowTiles; ++rt)
 #pragma unroll
         for (int p = kHalfPairs; p < kPairs; ++p) ta[rt][p] = load_ta(rt, p);
-    static_assert(kRowTiles * ((kAhead > kHalfBlocks ? kAhead - kHalfBlocks : 0) + kPairs - kHalfPairs) >= 4 || kType == 8,
+    // With a fragment ring shorter than half the blocks, fragments of the first half are still
+    // requested inside the loop.  Loads complete in order: requested behind the second half of the
+    // weights they would arrive behind it and the first half would be computed only after the
+    // whole stream.  There the second half of the weights is requested from inside the loop, right
+    // after the loads that complete the first half's fragments and the first ones of the second half's
+    // (which are the loads the compiler's wait may retire early instead of the weights).
+    constexpr int kIssuePair = kAhead >= kHalfBlocks ? -1 : (kHalfBlocks - kAhead) / 2;
+    static_assert(kIssuePair >= 0 || kRowTiles * ((kAhead > kHalfBlocks ? kAhead - kHalfBlocks : 0) + kPairs - kHalfPairs) >= 4 || kType == 8,
                   "cover loads");
-    issue_weights(1);
+    if (kIssuePair < 0) issue_weights(1);
 
     // The first A fragment was requested behind the first half of the weights: once it is here, so
     // are they.  (The statement makes the compiler wait for that fragment and keeps the LDS reads
@@ -307,6 +314,7 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
                     afrag[rt][(2 * p + 1) % kAhead] = load_a(rt, 2 * p + 1 + kAhead);
                 }
             }
+            if (p == kIssuePair) issue_weights(1);
         }
     } else {
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // its weight loads still write LDS, which the sums are about to reuse
