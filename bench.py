@@ -493,6 +493,13 @@ def main() -> int:
         for i in range(n_launch):
             launch(stream, Q4, _lib.LAYOUT_PREPARED, buf(yb), buf(xb), buf(ws[i % copies]), 16, 4096, 14336, buf(sb), -1)
         torch.cuda.synchronize()
+        # speculative verify, 8 rows on the FFN matrix: compact-fragment quantizer + eight-row MFMA kernel
+        x8 = torch.from_numpy(synth.activations(10, 8, 4096)).to(dev)
+        y8 = torch.empty((8, 14336), dtype=torch.float32, device=dev)
+        s8 = torch.empty(kernels.workspaceBytes(Q4, 8, 4096, 14336), dtype=torch.uint8, device=dev)
+        for i in range(n_launch):
+            launch(stream, Q4, _lib.LAYOUT_PREPARED, buf(y8), buf(x8), buf(ws[i % copies]), 8, 4096, 14336, buf(s8), -1)
+        torch.cuda.synchronize()
         # Q4_K on the same matrix: the decode kernel (one row) and the prefill GEMM (512 rows)
         wk = prepared_copies(Q4K, 14336, 4096, copies, 31)
         for m in (1, 512):
@@ -585,9 +592,10 @@ def main() -> int:
             ("q8_gemv_m1_k4096_n14336", Q8, 1, 4096, 14336),
             ("q4_gemv_m2_k4096_n14336", Q4, 2, 4096, 14336),
             ("q4_gemv_m4_k4096_n14336", Q4, 4, 4096, 14336),
-            ("q4_gemv_m8_k4096_n14336", Q4, 8, 4096, 14336),
+            ("q4_batch_m8_k4096_n14336", Q4, 8, 4096, 14336),   # speculative verify: compact-fragment quantizer + eight-row MFMA kernel
             ("q4_gemv_m1_k14336_n4096", Q4, 1, 14336, 4096),
-            ("q4_gemv_m5_k14336_n4096", Q4, 5, 14336, 4096),
+            ("q4_batch_m5_k14336_n4096", Q4, 5, 14336, 4096),
+            ("q8_batch_m8_k4096_n14336", Q8, 8, 4096, 14336),
             ("q4_batch_m16_k4096_n14336", Q4, 16, 4096, 14336),  # batched decode: fragment quantizer + single-shot MFMA kernel
             ("q4_batch_m32_k4096_n14336", Q4, 32, 4096, 14336),
             ("q4_batch_m64_k4096_n14336", Q4, 64, 4096, 14336),

@@ -28,6 +28,7 @@ CALLS = [
     (Q4K, 5, 1024, 200),    # Q4_K decode kernel, several rows
     (Q4K, 20, 4096, 300),   # Q4_K prefill GEMM, K shared out over workgroups
     (Q4K, 70, 1024, 200),   # Q4_K prefill GEMM, three row groups
+    (Q4, 7, 512, 8200),     # compact-fragment quantizer + eight-row MFMA kernel
 ]
 
 
