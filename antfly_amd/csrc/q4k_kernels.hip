@@ -92,7 +92,8 @@ __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restr
         out.y = dsc * byte_to_f32<1>(nib) - dmn;
         out.z = dsc * byte_to_f32<2>(nib) - dmn;
         out.w = dsc * byte_to_f32<3>(nib) - dmn;
-        reinterpret_cast<float4*>(dst)[u] = out;
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));  // written once, read by someone else: streamed past the caches
+        __builtin_nontemporal_store(f32x4_t{out.x, out.y, out.z, out.w}, reinterpret_cast<f32x4_t*>(dst) + u);
     }
 }
 

@@ -131,7 +131,9 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(uint4* __restrict__ dst,
 // 0 .. rows-1 in order.  Eight lanes per block, four values (one 16-byte store) per lane,
 // so a wavefront writes 1 KB of contiguous output.  `blocks_total` = blocks of the whole
 // weight (where the scales of the repacked layout start).
-template <int kType, bool kPrepared>
+// (kNarrow: rows * blocks per row fits 32 bits, so the row of a block is a 32-bit division -- a 64-bit
+// one is several dozen instructions per 16 bytes of output and made these copies ALU-bound.)
+template <int kType, bool kPrepared, bool kNarrow>
 __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict__ dst, const uint8_t* __restrict__ weight,
                                                               const long long* __restrict__ ids, size_t rows, int dim,
                                                               size_t blocks_total) {
@@ -142,7 +144,7 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict_
          u += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const int j = static_cast<int>(u & 7);  // values 4j .. 4j+3 of the block
         const size_t tb = u >> 3;
-        const size_t t = tb / kb, b = tb - t * kb;
+        const size_t t = kNarrow ? static_cast<uint32_t>(tb) / static_cast<uint32_t>(kb) : tb / kb, b = tb - t * kb;
         const long long row = ids ? ids[t] : static_cast<long long>(t);
         if (row < 0 || static_cast<size_t>(row) >= blocks_total / kb) {  // an id outside the weight reads nothing: zeros
             reinterpret_cast<float4*>(dst)[u] = float4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -175,7 +177,10 @@ __global__ __launch_bounds__(256) void dequantize_rows_kernel(float* __restrict_
             out.z = d * static_cast<float>(static_cast<int8_t>((packed >> 16) & 0xFF));
             out.w = d * static_cast<float>(static_cast<int8_t>(packed >> 24));
         }
-        reinterpret_cast<float4*>(dst)[u] = out;
+        // written once, read by someone else: one 16-byte store streamed past the caches (a cached store
+        // cost a third more time on a 235 MB output; four 4-byte streamed stores cost twice as much)
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));
+        __builtin_nontemporal_store(f32x4_t{out.x, out.y, out.z, out.w}, reinterpret_cast<f32x4_t*>(dst) + u);
     }
 }
 
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict_
 // Q4_0 :895-910, :1261-1265 (scale = max|x| / 8, nibble = clamp(round_half_away(x / scale) + 8, 0, 15),
 // byte i = value i | value i+16 << 4); the stored scale is f16(scale), an all-zero
 // block has scale 1.  Eight lanes per block.
-template <int kType>
+template <int kType, bool kNarrow>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
                                                             const long long* __restrict__ ids, size_t rows, int dim,
                                                             size_t dst_rows) {
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict_
         const float inv = m == 0.0f ? 0.0f : 1.0f / scale;
         const int j = static_cast<int>(u & 7);
         const size_t tb = u >> 3;
-        const size_t t = live ? tb / kb : 0, b = live ? tb - t * kb : 0;
+        const size_t t = live ? (kNarrow ? static_cast<uint32_t>(tb) / static_cast<uint32_t>(kb) : tb / kb) : 0, b = live ? tb - t * kb : 0;
         const long long row = ids && live ? ids[t] : static_cast<long long>(t);
         const bool in_range = row >= 0 && static_cast<size_t>(row) < dst_rows;  // a row id outside the destination writes nothing
         const size_t block = (in_range ? static_cast<size_t>(row) : 0) * kb + b;
@@ -475,13 +480,20 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
     }
     const size_t blocks_total = weight_rows * static_cast<size_t>(dim >> 5);
     const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
+    const bool narrow = rows * static_cast<size_t>(dim >> 5) <= 0xFFFFFFFFull;
+#define AFHIP_DEQ(T, P)                                                                                                          \
+    do {                                                                                                                         \
+        if (narrow) hipLaunchKernelGGL((dequantize_rows_kernel<T, P, true>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total); \
+        else hipLaunchKernelGGL((dequantize_rows_kernel<T, P, false>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);      \
+    } while (0)
     if (tensor_type == 2) {
-        if (layout == 0) hipLaunchKernelGGL((dequantize_rows_kernel<2, false>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
-        else hipLaunchKernelGGL((dequantize_rows_kernel<2, true>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+        if (layout == 0) AFHIP_DEQ(2, false);
+        else AFHIP_DEQ(2, true);
     } else {
-        if (layout == 0) hipLaunchKernelGGL((dequantize_rows_kernel<8, false>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
-        else hipLaunchKernelGGL((dequantize_rows_kernel<8, true>), grid, dim3(256), 0, stream, dst, weight, ids, rows, dim, blocks_total);
+        if (layout == 0) AFHIP_DEQ(8, false);
+        else AFHIP_DEQ(8, true);
     }
+#undef AFHIP_DEQ
     return launch_status();
 }
 
@@ -489,8 +501,14 @@ hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* ds
                                 size_t rows, int dim, size_t dst_rows) {
     if (rows == 0 || dim == 0) return hipSuccess;
     const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
-    if (tensor_type == 2) hipLaunchKernelGGL(quantize_rows_kernel<2>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
-    else hipLaunchKernelGGL(quantize_rows_kernel<8>, grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+    const bool narrow = rows * static_cast<size_t>(dim >> 5) <= 0xFFFFFFFFull;
+    if (tensor_type == 2) {
+        if (narrow) hipLaunchKernelGGL((quantize_rows_kernel<2, true>), grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+        else hipLaunchKernelGGL((quantize_rows_kernel<2, false>), grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+    } else {
+        if (narrow) hipLaunchKernelGGL((quantize_rows_kernel<8, true>), grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+        else hipLaunchKernelGGL((quantize_rows_kernel<8, false>), grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+    }
     return launch_status();
 }
 

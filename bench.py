@@ -71,7 +71,7 @@ def main() -> int:
                     help="for hardware-counter runs: 40 eager launches each of the headline GEMV, of the plain "
                          "read kernel and of the plain copy kernel over the same number of bytes, of the Q8_0 M=512 GEMM, of the 16-row batch kernel and of the Q4_K kernels "
                          "(M=1 and M=512), then exit")
-    ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048"], default=None,
+    ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048", "row_ops"], default=None,
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k): time only these calls, print one line each, exit")
@@ -354,6 +354,9 @@ def main() -> int:
                               "frac_hbm_peak": round(b * 400 / e_s / HBM_PEAK_BPS, 4)}), flush=True)
         return 0
 
+    if args.only == "row_ops":
+        print(json.dumps({"only": "row_ops", "row_ops_14336x4096": time_row_ops()}))
+        return 0
     if args.only:
         m = int(args.only.rsplit("m", 1)[1])
         w_s, e_s = time_config(Q8, m, 4096, 4096, 200, 20, 4, 7, repeats=1)
