@@ -62,7 +62,7 @@ struct BmFormat {
 // at lds_addr + 16 * l.  Inline assembly: the compiler does not track these loads, which is why
 // the kernel waits for them by hand before anything reads the LDS region.
 __device__ __forceinline__ void bm_lds_load16(const void* base, uint32_t voff, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" : : "s"(lds_addr), "v"(voff), "s"(base) : "memory", "m0");
 }
 
 extern __shared__ __align__(16) unsigned char bm_lds[];
