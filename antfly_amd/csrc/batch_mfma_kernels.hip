@@ -32,6 +32,8 @@
 //     16x16x64 MFMA on two blocks at once, 32- or 64-column tiles, weights requested two stages
 //     ahead instead of all at once.
 #include <hip/hip_runtime.h>
+
+#include <cstdlib>
 #include <type_traits>
 
 #include "device_common.h"
@@ -98,6 +100,10 @@ __device__ __forceinline__ void fence_registers(float (&a)[16]) {
 // bytes [16 * half, +16) of the block's 32 int8), sa: f32 [block][32 * row_tiles].  Rows past
 // `rows` get zeros and scale 0.  Eight lanes per block as in quantize_activations_kernel
 // (ops/native_compute.zig:11998-12028): same scale, reciprocal and rounding, bit for bit.
+// kByteOrder (Q4_0 operands of batch32_mfma_kernel): within a block the lane half h holds the dwords
+// x[8h..8h+3], x[16+8h..+3], x[8h+4..8h+7], x[16+8h+4..+7] instead of x[16h..16h+15] -- the values whose
+// nibbles share the bytes [8 h, 8 h + 8) of the weight block, so that a lane unpacks whole bytes.
+template <bool kByteOrder>
 __global__ __launch_bounds__(256) void quantize_fragments_kernel(const float* __restrict__ x, int rows, int in_dim, int row_tiles,
                                                                   uint32_t* __restrict__ qa, float* __restrict__ sa) {
     const int units_per_row = in_dim >> 2, kb = in_dim >> 5, padded = row_tiles * 32;
@@ -114,8 +120,9 @@ __global__ __launch_bounds__(256) void quantize_fragments_kernel(const float* __
         const float inv = m == 0.0f ? 0.0f : 1.0f / s;
         const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
         const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
-        const size_t lane_entry = (static_cast<size_t>(r >> 5) * kb + b) * 64 + (j >> 2) * 32 + (r & 31);
-        qa[lane_entry * 4 + (j & 3)] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+        const int half = kByteOrder ? (j >> 1) & 1 : j >> 2, dw = kByteOrder ? 2 * (j & 1) + (j >> 2) : j & 3;
+        const size_t lane_entry = (static_cast<size_t>(r >> 5) * kb + b) * 64 + half * 32 + (r & 31);
+        qa[lane_entry * 4 + dw] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
         if (j == 0) sa[static_cast<size_t>(b) * padded + r] = r < rows ? s : 0.0f;
     }
 }
@@ -654,6 +661,205 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Nine to 32 rows on a matrix wide enough for 64-column tiles: batch_mfma_kernel's arithmetic
+// (v_mfma_i32_32x32x32_i8 per block, scale products of a pair of blocks from one
+// v_mfma_f32_32x32x1_2b_f32, one convert and one multiply-add per live result register) with what
+// the eight-row kernel showed to matter:
+//   * 64 columns per workgroup (two groups of 32): the A fragments -- 16 KB per wavefront, as much
+//     as the weights per 32 columns -- are read once for both groups, and there is one workgroup
+//     per compute unit with the whole register file (no second workgroup to leave room for);
+//   * weights staged: stage (half hb of the wavefront's blocks, column group cg) is four 1 KB
+//     units in one of two 4 KB slots; a stage is requested when the stage two before it has been
+//     computed, so one stage travels while one is worked on (requesting all at once leaves a
+//     wavefront stuck issuing loads while the data it could work on is already there);
+//   * the A fragments of the second half of the blocks are requested block by block during the
+//     last stage that uses the first half's (behind the weight requests already out, in front of
+//     the last one);
+//   * a lane unpacks whole bytes of Q4_0 nibbles (low and high: 8 operations per block instead of
+//     12; the fragments' k order follows, quantize_fragments_kernel<true>);
+//   * the arithmetic of a pair of blocks is ordered by hand: both int8 MFMAs and the scale MFMA
+//     first, then the conversions and multiply-adds of both blocks, with the next pair's LDS reads
+//     in flight meanwhile.
+template <int kType, int kLive>
+__global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
+                                                                      const uint32_t* __restrict__ qa, const float* __restrict__ sa,
+                                                                      const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
+                                                                      int share_blocks, Epilogue ep_a, BmSecond second) {
+    using F = BmFormat<kType>;
+    const bool is_b = blockIdx.z != 0;
+    float* dst = is_b ? second.dst : dst_a;
+    const uint8_t* weight = is_b ? second.weight : weight_a;
+    const Epilogue ep = is_b ? second.ep : ep_a;
+    float* partial = partial_a == nullptr ? nullptr : partial_a + (is_b ? static_cast<size_t>(gridDim.y) * rows * out_dim : 0);
+    constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kHB = kWB / 2, kPairs = kWB / 2, kHalfPairs = kPairs / 2;
+    const int kb_full = in_dim >> 5;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lj = lane & 31, lh = lane >> 5;
+    const int n0 = blockIdx.x * 64;
+    const int share_begin = static_cast<int>(blockIdx.y) * share_blocks;
+    const int share_end = min(share_begin + share_blocks, kb_full);
+    const int blk0 = share_begin + wave * kWB;
+    const int nb = max(0, min(kWB, share_end - blk0));
+    const int last = blk0 + max(nb, 1) - 1 < kb_full ? blk0 + max(nb, 1) - 1 : kb_full - 1;
+    auto clamp_blk = [&](int j) { return min(blk0 + j, last); };
+    const size_t blocks_total = static_cast<size_t>(out_dim) * kb_full;
+    const uint32_t lds_wave = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(bm_lds))) + wave * kBmWaveBytes;
+
+    // stage st = 2 * hb + cg -> slot st % 2
+    auto issue_stage = [&](int st) {
+        const int hb = st >> 1, cg = st & 1;
+        const uint8_t* wbase = weight + static_cast<size_t>(n0) * kb_full * kQB;
+        const int c8 = lane >> 3, slot = lane & 7;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = 32 * cg + 8 * u + c8;
+            const int chunk = slot ^ ((c >> 1) & 7);
+            const int cc = min(n0 + c, out_dim - 1) - n0;
+            uint32_t off;
+            if (kType == 2) {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(8 * hb + chunk)) * 16u;
+            } else {
+                off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(4 * hb + (chunk >> 1))) * 32u + (chunk & 1) * 16u;
+            }
+            bm_lds_load16(wbase, off, lds_wave + ((st & 1) * 4 + u) * 1024);
+        }
+    };
+    issue_stage(0);
+    // weight scales of both column groups (fp16, block order; rows of whole 16-byte runs): word p of a
+    // column's run holds blocks 2p and 2p + 1
+    uint32_t tb_word[2][kPairs];
+#pragma unroll
+    for (int cg = 0; cg < 2; ++cg) {
+        const int cc = min(n0 + 32 * cg + lj, out_dim - 1);
+        const uint16_t* sw = reinterpret_cast<const uint16_t*>(weight + blocks_total * kQB) + static_cast<size_t>(cc) * kb_full;
+        const uint4* run = reinterpret_cast<const uint4*>(sw + min(blk0, kb_full - 8));
+#pragma unroll
+        for (int q = 0; q < kPairs / 4; ++q) {
+            const uint4 v = run[q];
+            tb_word[cg][4 * q] = v.x;
+            tb_word[cg][4 * q + 1] = v.y;
+            tb_word[cg][4 * q + 2] = v.z;
+            tb_word[cg][4 * q + 3] = v.w;
+        }
+    }
+    // A fragments and row scales of the first half of the blocks.  Rows that exist live in the first
+    // 2 * kLive lanes of each half of a fragment; the other lanes repeat a live lane's address.
+    const int lr = lj % (2 * kLive);
+    const int alane = lh * 32 + lr;
+    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa);
+    auto load_a = [&](int j) { return qa4[static_cast<size_t>(clamp_blk(j)) * 64 + alane]; };
+    auto load_ta = [&](int p) { return sa[static_cast<size_t>(clamp_blk(2 * p + lh)) * 32 + lr]; };
+    bm_v4i afrag[kHB];
+    float ta[kHalfPairs];
+#pragma unroll
+    for (int j = 0; j < kHB; ++j) afrag[j] = load_a(j);
+#pragma unroll
+    for (int p = 0; p < kHalfPairs; ++p) ta[p] = load_ta(p);
+    issue_stage(1);
+
+    // this lane's B operand inside a slot: column lj of the group, block j of the half, k half lh
+    uint32_t baddr[kHB];
+#pragma unroll
+    for (int j = 0; j < kHB; ++j) {
+        const int unit = lj >> 3, row = (lj & 7) * 8, swz = (lj >> 1) & 7;
+        const int chunk = kType == 2 ? j : 2 * j + lh;
+        baddr[j] = lds_wave + (unit * 64 + row + (chunk ^ swz)) * 16 + (kType == 2 ? 8 * lh : 0);
+    }
+#pragma unroll
+    for (int j = 0; j < kHB; ++j) asm volatile("" : "+v"(baddr[j]));
+
+    float acc[2][kLive];
+#pragma unroll
+    for (int cg = 0; cg < 2; ++cg)
+#pragma unroll
+        for (int v = 0; v < kLive; ++v) acc[cg][v] = 0.0f;
+
+    if (nb > 0) {
+        typedef unsigned bm_v2u __attribute__((ext_vector_type(2)));
+        typedef unsigned bm_v4u __attribute__((ext_vector_type(4)));
+        typedef typename std::conditional<kType == 2, bm_v2u, bm_v4u>::type Raw;
+        typedef __attribute__((address_space(3))) const Raw LdsRaw;
+        auto unpack = [&](const Raw& w) {
+            bm_v4i b;
+            if constexpr (kType == 2) {
+                const uint32_t x = w[0] ^ 0x88888888u, y = w[1] ^ 0x88888888u;
+                b = bm_v4i{static_cast<int>((x << 4) & 0xF0F0F0F0u), static_cast<int>(x & 0xF0F0F0F0u), static_cast<int>((y << 4) & 0xF0F0F0F0u),
+                           static_cast<int>(y & 0xF0F0F0F0u)};
+            } else {
+                b = bm_v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[kType == 2 ? 0 : 2]), static_cast<int>(w[kType == 2 ? 1 : 3])};
+            }
+            return b;
+        };
+        const bm_v16i zi = {};
+        const bm_v32f zf = {};
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+            const int hb = st >> 1, cg = st & 1;
+            // this stage is there when at most the stage requested behind it is in flight
+            if (st < 3) asm volatile("s_waitcnt vmcnt(4)" : : : "memory");
+            else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+            Raw raw0 = *reinterpret_cast<LdsRaw*>(baddr[0] + (st & 1) * 4096);
+            Raw raw1 = *reinterpret_cast<LdsRaw*>(baddr[1] + (st & 1) * 4096);
+#pragma unroll
+            for (int q = 0; q < kHalfPairs; ++q) {
+                const int p = hb * kHalfPairs + q;
+                const bool live_blk = 2 * p + lh < nb;  // a clamped re-read of the last block counts for nothing
+                const float tb = live_blk ? half_bits_to_f32(static_cast<uint16_t>(tb_word[cg][p] >> (16 * lh))) * (kType == 2 ? 0.0625f : 1.0f) : 0.0f;
+                const bm_v4i b0 = unpack(raw0), b1 = unpack(raw1);
+                __builtin_amdgcn_sched_barrier(0);
+                if (q + 1 < kHalfPairs) {
+                    raw0 = *reinterpret_cast<LdsRaw*>(baddr[2 * q + 2] + (st & 1) * 4096);
+                    raw1 = *reinterpret_cast<LdsRaw*>(baddr[2 * q + 3] + (st & 1) * 4096);
+                }
+                const bm_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q], b0, zi, 0, 0, 0);
+                const bm_v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(live_blk ? ta[q] : 0.0f, tb, zf, 0, 0, 0);
+                const bm_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q + 1], b1, zi, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (cg == 1 && hb == 0) {
+                    // last use of the first half's fragments of this pair: the second half's take their place
+                    afrag[2 * q] = load_a(kHB + 2 * q);
+                    afrag[2 * q + 1] = load_a(kHB + 2 * q + 1);
+                    ta[q] = load_ta(kHalfPairs + q);
+                }
+#pragma unroll
+                for (int v = 0; v < kLive; ++v) acc[cg][v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[cg][v]);
+#pragma unroll
+                for (int v = 0; v < kLive; ++v) acc[cg][v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[cg][v]);
+                fence_registers(acc[cg]);
+            }
+            // the slot is free: the stage two on takes it
+            if (st + 2 < 4) issue_stage(st + 2);
+        }
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may still be writing LDS when the region is reused
+    }
+
+    // ---- the wavefronts' sums meet in LDS: [wave][cg][v][lane] (8 x 2 x 16 x 64 floats = the whole 64 KB)
+    float* red = reinterpret_cast<float*>(bm_lds);
+    __syncthreads();
+#pragma unroll
+    for (int cg = 0; cg < 2; ++cg)
+#pragma unroll
+        for (int v = 0; v < kLive; ++v) red[((wave * 2 + cg) * kLive + v) * 64 + lane] = acc[cg][v];
+    __syncthreads();
+    constexpr int kItems = 2 * kLive * 64;
+    for (int i = tid; i < kItems; i += kBmThreads) {
+        float sum = red[i];
+#pragma unroll
+        for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
+        const int l = i & 63, v = (i >> 6) % kLive, cg = (i >> 6) / kLive;
+        const int m = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+        const int n = n0 + 32 * cg + (l & 31);
+        if (m < rows && n < out_dim) {
+            const size_t at = static_cast<size_t>(m) * out_dim + n;
+            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+            else dst[at] = finish_output(ep, n, at, sum);
+        }
+    }
+}
+
 namespace {
 
 template <int kType, int kRowTiles, int kLive>
@@ -693,6 +899,20 @@ hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint
 // workgroup's traffic and a wavefront's set-up halve) where that still gives most compute units a
 // workgroup, else two.
 int bm8_column_groups(int out_dim) { return (out_dim + 63) / 64 >= gemv_compute_units() * 3 / 4 ? 4 : 2; }
+
+template <int kType>
+hipError_t bm_launch32(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
+                       int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+    const dim3 grid(static_cast<unsigned>((out_dim + 63) / 64), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
+#define AFHIP_BM32(LIVE)                                                                                                                 \
+    hipLaunchKernelGGL((batch32_mfma_kernel<kType, LIVE>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, \
+                       weight, rows, in_dim, out_dim, share_blocks, ep, second)
+    if (rows <= 16) AFHIP_BM32(8);
+    else if (rows <= 24) AFHIP_BM32(12);
+    else AFHIP_BM32(16);
+#undef AFHIP_BM32
+    return hipGetLastError();
+}
 
 int bm_shares(int tensor_type, int in_dim) {
     const int share_max = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
@@ -737,8 +957,23 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(padded) * in_dim);
     const size_t front = static_cast<size_t>(padded) * in_dim + static_cast<size_t>(kb) * padded * 4;
     float* partial = reinterpret_cast<float*>(workspace + (front + 255) / 256 * 256);
-    const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
-    if (eight) {
+    const int shares = bm_shares(tensor_type, in_dim);
+    // equal shares, whole wavefront slices: a multiple of the blocks one wavefront owns
+    const int wave_blocks = tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks;
+    int share_blocks = (kb + shares - 1) / shares;
+    share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
+    const int real_shares = (kb + share_blocks - 1) / share_blocks;
+    const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);
+    // Nine to 32 rows on a matrix wide enough for 64-column tiles (and rows of whole 16-byte runs of
+    // scales), with no more workgroups than compute units: batch32_mfma_kernel holds one workgroup per
+    // unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
+    // unit (N = 20480: 21.1 against 18.5 us).  AFHIP_BATCH32_MAX_WORKGROUPS overrides the bound (tests
+    // reach the kernel's K shares and pair launches that way; 0 switches the kernel off).
+    const char* bound_env = std::getenv("AFHIP_BATCH32_MAX_WORKGROUPS");
+    const long bound = bound_env ? std::atol(bound_env) : gemv_compute_units();
+    const bool thirty_two = !eight && rows <= 32 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
+                            static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
+    if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
         const int pairs = (kb + 1) / 2;
         sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
         const int units = 8 * (2 * pairs) * 8;
@@ -752,16 +987,14 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
         const size_t units = static_cast<size_t>(padded) * (in_dim / 4);
         size_t grid = (units + 255) / 256;
         if (grid > 4096) grid = 4096;
-        hipLaunchKernelGGL(quantize_fragments_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
-                           row_tiles, qa, sa);
+        if (thirty_two && tensor_type == 2)
+            hipLaunchKernelGGL(quantize_fragments_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
+                               row_tiles, qa, sa);
+        else
+            hipLaunchKernelGGL(quantize_fragments_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
+                               row_tiles, qa, sa);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     }
-    const int shares = bm_shares(tensor_type, in_dim);
-    // equal shares, whole wavefront slices: a multiple of the blocks one wavefront owns
-    const int wave_blocks = tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks;
-    int share_blocks = (kb + shares - 1) / shares;
-    share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
-    const int real_shares = (kb + share_blocks - 1) / share_blocks;
     const size_t count = static_cast<size_t>(rows) * out_dim;
     // a pair is one launch over both matrices (grid.z)
     const BmSecond second{dst_b, weight_b_prepared, ep_b};
@@ -772,6 +1005,9 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
         e = tensor_type == 2 ? (wide ? AFHIP_BM8(2, 4) : AFHIP_BM8(2, 2)) : (wide ? AFHIP_BM8(8, 4) : AFHIP_BM8(8, 2));
 #undef AFHIP_BM8
     }
+    else if (thirty_two)
+        e = tensor_type == 2 ? bm_launch32<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
+                             : bm_launch32<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
     else
         e = tensor_type == 2
                        ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)

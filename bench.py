@@ -74,7 +74,7 @@ def main() -> int:
     ap.add_argument("--only", choices=["gemm_q8_m512", "gemm_q8_m128", "gemm_q8_m2048", "row_ops"], default=None,
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
-                    help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k): time only these calls, print one line each, exit")
+                    help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k; q4p / q8p: pair calls): time only these calls, print one line each, exit")
     ap.add_argument("--probe", choices=["gemv", "rates"], default=None,
                     help="rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
@@ -108,20 +108,27 @@ def main() -> int:
         torch.cuda.synchronize()
         return out
 
-    def time_config(fmt, rows, in_dim, out_dim, steps, warmup, copies, seed, repeats=1):
+    def time_config(fmt, rows, in_dim, out_dim, steps, warmup, copies, seed, repeats=1, pair=False):
         """Returns (wall seconds, event seconds) for `steps` back-to-back calls: the median of
-        `repeats` runs of the same timed region."""
+        `repeats` runs of the same timed region.  pair: every call is one pair call (two matrices of
+        this shape that share X, as gate and up do)."""
         ws = prepared_copies(fmt, out_dim, in_dim, copies, seed)
         x = torch.from_numpy(synth.activations(seed + 1, rows, in_dim)).to(dev)
         y = torch.empty((rows, out_dim), dtype=torch.float32, device=dev)
+        y2 = torch.empty((rows, out_dim), dtype=torch.float32, device=dev) if pair else None
         wsb = kernels.workspaceBytes(fmt, rows, in_dim, out_dim)
         scratch = torch.empty(max(wsb, 16), dtype=torch.uint8, device=dev)
         bx, by, bs = buf(x), buf(y), buf(scratch)
         bws = [buf(w) for w in ws]
         launch = _lib.lib().afhip_launch_linear_f32
+        launch_pair = _lib.lib().afhip_launch_linear_pair_f32
 
         def step(i, st):
-            rc = launch(st, fmt, _lib.LAYOUT_PREPARED, by, bx, bws[i % copies], rows, in_dim, out_dim, bs, -1)
+            if pair:
+                rc = launch_pair(st, fmt, _lib.LAYOUT_PREPARED, by, buf(y2), bx, bws[(2 * i) % copies], bws[(2 * i + 1) % copies],
+                                 rows, in_dim, out_dim, bs, -1)
+            else:
+                rc = launch(st, fmt, _lib.LAYOUT_PREPARED, by, bx, bws[i % copies], rows, in_dim, out_dim, bs, -1)
             if rc != 0:
                 raise RuntimeError(f"launch failed: {rc}")
 
@@ -344,12 +351,15 @@ def main() -> int:
     if args.shapes:
         for spec in args.shapes.split(","):
             f, r, k, n = spec.split(":")
-            fmt = {"q4": Q4, "q8": Q8, "q4k": Q4K}[f]
+            pair = f.endswith("p")  # q4p / q8p: pair calls (two matrices, one X)
+            fmt = {"q4": Q4, "q8": Q8, "q4k": Q4K}[f[:-1] if pair else f]
             r, k, n = int(r), int(k), int(n)
             wbytes = n * (k // 32) * BLOCK_BYTES[fmt] if fmt != Q4K else n * (k // 256) * 144
             copies = max(2, min(16, (600 << 20) // wbytes))
-            w_s, e_s = time_config(fmt, r, k, n, 400, 20, copies, 99, repeats=3)
-            b = wbytes + 4 * r * (k + n)
+            w_s, e_s = time_config(fmt, r, k, n, 400, 20, copies, 99, repeats=3, pair=pair)
+            if pair:
+                wbytes *= 2
+            b = wbytes + 4 * r * (k + n * (2 if pair else 1))
             print(json.dumps({"shape": spec, "us_per_call": round(e_s / 400 * 1e6, 3), "GBps": round(b * 400 / e_s / 1e9, 1),
                               "frac_hbm_peak": round(b * 400 / e_s / HBM_PEAK_BPS, 4)}), flush=True)
         return 0

@@ -128,6 +128,9 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # wavefront and a ragged last tile; 64-column tiles, ragged; K shares with a short last share; a
     # wavefront with half its blocks
     (8, 512, 8200), (5, 4096, 12290), (7, 9216, 4112), (6, 256, 16416),
+    # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
+    # wavefront with half its blocks, K shares with a short last share
+    (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
 ]
 
 
@@ -194,6 +197,7 @@ PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K sl
     (1, 4096, 1024), (2, 512, 514), (4, 2048, 640), (5, 8224, 513), (8, 4096, 512), (12, 256, 530), (40, 512, 640),
     (3, 64, 100), (20, 2048, 300),  # the last: MFMA GEMM with K shared out over workgroups, both matrices through one scratch
     (6, 512, 8200), (7, 9216, 4112),  # the eight-row MFMA kernel, one launch over both matrices; with K shares
+    (20, 512, 12290),                 # the 32-row MFMA kernel on 64-column tiles, both matrices
 ]
 
 
@@ -307,3 +311,41 @@ def test_committed_tiny_vectors(fmt_name, fmt, case, rows, in_dim, out_dim):
         assert np.array_equal(G.block_dots(fmt, layout, x, wd, rows, in_dim, out_dim), g[key + "block_dots"])
         y = G.linear(fmt, layout, x, wd, rows, in_dim, out_dim)
         assert G.max_rel_err(y, g[key + "y_op"].astype(np.float64)) <= TIGHT
+
+
+@pytest.mark.parametrize("fmt,rows,in_dim,out_dim,pair", [(Q4, 29, 9216, 12288, False), (Q8, 20, 2048, 12290, True),
+                                                          (Q4, 20, 512, 12290, True), (Q4, 12, 8192, 12352, True)])
+def test_thirty_two_row_kernel_with_k_shares_and_pairs(fmt, rows, in_dim, out_dim, pair):
+    """On this chip the 32-row kernel's grid bound (one workgroup per compute unit) keeps launches with
+    K shares or two matrices on the older kernel; with the bound lifted they take the 32-row kernel and
+    must give what the older kernel gives to f32 summation order, and the oracle's result within its bound."""
+    import os
+    print(f"case: 32-row kernel, bound lifted fmt={fmt} rows={rows} in={in_dim} out={out_dim} pair={pair}", flush=True)
+    x = synth.activations(5100 + rows, rows, in_dim)
+    wa = synth.weights(fmt, 5101, out_dim, in_dim)
+    da = G.prepare(fmt, wa, out_dim, in_dim)
+    db = G.prepare(fmt, synth.weights(fmt, 5102, out_dim, in_dim), out_dim, in_dim) if pair else None
+
+    def run():
+        if pair:
+            return G.linear_pair(fmt, PREP, x, da, db, rows, in_dim, out_dim)
+        return (G.linear(fmt, PREP, x, da, rows, in_dim, out_dim),)
+
+    older = run()
+    os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"] = "1000000"
+    try:
+        got = run()
+    finally:
+        del os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"]
+    ref = O.linear_no_bias(fmt, x, wa, rows, in_dim, out_dim, workers=8)
+    err = G.max_rel_err(got[0], ref.astype(np.float64))
+    assert err <= TOL and err <= TIGHT, err
+    for a, b in zip(got, older):
+        assert G.max_rel_err(a, b.astype(np.float64)) <= TIGHT
+    if pair:  # each half of the pair equals the single op on that matrix, bit for bit
+        os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"] = "1000000"
+        try:
+            assert np.array_equal(got[0], G.linear(fmt, PREP, x, da, rows, in_dim, out_dim))
+            assert np.array_equal(got[1], G.linear(fmt, PREP, x, db, rows, in_dim, out_dim))
+        finally:
+            del os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"]
