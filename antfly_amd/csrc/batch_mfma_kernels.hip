@@ -802,20 +802,30 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
             else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
             Raw raw0 = *reinterpret_cast<LdsRaw*>(baddr[0] + (st & 1) * 4096);
             Raw raw1 = *reinterpret_cast<LdsRaw*>(baddr[1] + (st & 1) * 4096);
+            bm_v4i b0 = unpack(raw0), b1 = unpack(raw1);
+            if (kHalfPairs > 1) {
+                raw0 = *reinterpret_cast<LdsRaw*>(baddr[2] + (st & 1) * 4096);
+                raw1 = *reinterpret_cast<LdsRaw*>(baddr[3] + (st & 1) * 4096);
+            }
 #pragma unroll
             for (int q = 0; q < kHalfPairs; ++q) {
                 const int p = hb * kHalfPairs + q;
                 const bool live_blk = 2 * p + lh < nb;  // a clamped re-read of the last block counts for nothing
                 const float tb = live_blk ? half_bits_to_f32(static_cast<uint16_t>(tb_word[cg][p] >> (16 * lh))) * (kType == 2 ? 0.0625f : 1.0f) : 0.0f;
-                const bm_v4i b0 = unpack(raw0), b1 = unpack(raw1);
                 __builtin_amdgcn_sched_barrier(0);
-                if (q + 1 < kHalfPairs) {
-                    raw0 = *reinterpret_cast<LdsRaw*>(baddr[2 * q + 2] + (st & 1) * 4096);
-                    raw1 = *reinterpret_cast<LdsRaw*>(baddr[2 * q + 3] + (st & 1) * 4096);
-                }
-                const bm_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q], b0, zi, 0, 0, 0);
                 const bm_v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(live_blk ? ta[q] : 0.0f, tb, zf, 0, 0, 0);
+                const bm_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q], b0, zi, 0, 0, 0);
                 const bm_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q + 1], b1, zi, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                // while the matrix unit works: the next pair's weights out of their nibbles, the pair after that out of LDS
+                if (q + 1 < kHalfPairs) {
+                    b0 = unpack(raw0);
+                    b1 = unpack(raw1);
+                    if (q + 2 < kHalfPairs) {
+                        raw0 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 4) % kHB] + (st & 1) * 4096);
+                        raw1 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 5) % kHB] + (st & 1) * 4096);
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
                 if (cg == 1 && hb == 0) {
                     // last use of the first half's fragments of this pair: the second half's take their place
