@@ -681,7 +681,7 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
 //   * the arithmetic of a pair of blocks is ordered by hand: both int8 MFMAs and the scale MFMA
 //     first, then the conversions and multiply-adds of both blocks, with the next pair's LDS reads
 //     in flight meanwhile.
-template <int kType, int kLive>
+template <int kType, int kRT, int kLive>
 __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                       const uint32_t* __restrict__ qa, const float* __restrict__ sa,
                                                                       const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
@@ -749,14 +749,17 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
     const int lr = lj % (2 * kLive);
     const int alane = lh * 32 + lr;
     const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa);
-    auto load_a = [&](int j) { return qa4[static_cast<size_t>(clamp_blk(j)) * 64 + alane]; };
-    auto load_ta = [&](int p) { return sa[static_cast<size_t>(clamp_blk(2 * p + lh)) * 32 + lr]; };
-    bm_v4i afrag[kHB];
-    float ta[kHalfPairs];
+    auto load_a = [&](int rt, int j) { return qa4[(static_cast<size_t>(rt) * kb_full + clamp_blk(j)) * 64 + (rt + 1 < kRT ? lane : alane)]; };
+    auto load_ta = [&](int rt, int p) { return sa[static_cast<size_t>(clamp_blk(2 * p + lh)) * (32 * kRT) + rt * 32 + (rt + 1 < kRT ? lj : lr)]; };
+    bm_v4i afrag[kRT][kHB];
+    float ta[kRT][kHalfPairs];
 #pragma unroll
-    for (int j = 0; j < kHB; ++j) afrag[j] = load_a(j);
+    for (int rt = 0; rt < kRT; ++rt) {
 #pragma unroll
-    for (int p = 0; p < kHalfPairs; ++p) ta[p] = load_ta(p);
+        for (int j = 0; j < kHB; ++j) afrag[rt][j] = load_a(rt, j);
+#pragma unroll
+        for (int p = 0; p < kHalfPairs; ++p) ta[rt][p] = load_ta(rt, p);
+    }
     issue_stage(1);
 
     // this lane's B operand inside a slot: column lj of the group, block j of the half, k half lh
@@ -770,11 +773,14 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
 #pragma unroll
     for (int j = 0; j < kHB; ++j) asm volatile("" : "+v"(baddr[j]));
 
-    float acc[2][kLive];
+    // (a full row tile has all 16 result registers live; kLive counts those of the last one)
+    float acc[2][kRT][16];
 #pragma unroll
     for (int cg = 0; cg < 2; ++cg)
 #pragma unroll
-        for (int v = 0; v < kLive; ++v) acc[cg][v] = 0.0f;
+        for (int rt = 0; rt < kRT; ++rt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[cg][rt][v] = 0.0f;
 
     if (nb > 0) {
         typedef unsigned bm_v2u __attribute__((ext_vector_type(2)));
@@ -812,32 +818,40 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
                 const int p = hb * kHalfPairs + q;
                 const bool live_blk = 2 * p + lh < nb;  // a clamped re-read of the last block counts for nothing
                 const float tb = live_blk ? half_bits_to_f32(static_cast<uint16_t>(tb_word[cg][p] >> (16 * lh))) * (kType == 2 ? 0.0625f : 1.0f) : 0.0f;
-                __builtin_amdgcn_sched_barrier(0);
-                const bm_v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(live_blk ? ta[q] : 0.0f, tb, zf, 0, 0, 0);
-                const bm_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q], b0, zi, 0, 0, 0);
-                const bm_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[2 * q + 1], b1, zi, 0, 0, 0);
-                __builtin_amdgcn_sched_barrier(0);
-                // while the matrix unit works: the next pair's weights out of their nibbles, the pair after that out of LDS
-                if (q + 1 < kHalfPairs) {
-                    b0 = unpack(raw0);
-                    b1 = unpack(raw1);
-                    if (q + 2 < kHalfPairs) {
-                        raw0 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 4) % kHB] + (st & 1) * 4096);
-                        raw1 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 5) % kHB] + (st & 1) * 4096);
+#pragma unroll
+                for (int rt = 0; rt < kRT; ++rt) {
+                    constexpr int kFull = 16;
+                    const int live_regs = rt + 1 < kRT ? kFull : kLive;
+                    __builtin_amdgcn_sched_barrier(0);
+                    const bm_v32f t = __builtin_amdgcn_mfma_f32_32x32x1f32(live_blk ? ta[rt][q] : 0.0f, tb, zf, 0, 0, 0);
+                    const bm_v16i c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[rt][2 * q], b0, zi, 0, 0, 0);
+                    const bm_v16i c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(afrag[rt][2 * q + 1], b1, zi, 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (cg == 1 && hb == 0) {
+                        // last use of the first half's fragments of this pair: the second half's take their place
+                        afrag[rt][2 * q] = load_a(rt, kHB + 2 * q);
+                        afrag[rt][2 * q + 1] = load_a(rt, kHB + 2 * q + 1);
+                        ta[rt][q] = load_ta(rt, kHalfPairs + q);
                     }
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                if (cg == 1 && hb == 0) {
-                    // last use of the first half's fragments of this pair: the second half's take their place
-                    afrag[2 * q] = load_a(kHB + 2 * q);
-                    afrag[2 * q + 1] = load_a(kHB + 2 * q + 1);
-                    ta[q] = load_ta(kHalfPairs + q);
-                }
+                    // while the matrix unit works (last row tile: its operands are no longer needed): the next
+                    // pair's weights out of their nibbles, the pair after that out of LDS
+                    if (rt == kRT - 1 && q + 1 < kHalfPairs) {
+                        b0 = unpack(raw0);
+                        b1 = unpack(raw1);
+                        if (q + 2 < kHalfPairs) {
+                            raw0 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 4) % kHB] + (st & 1) * 4096);
+                            raw1 = *reinterpret_cast<LdsRaw*>(baddr[(2 * q + 5) % kHB] + (st & 1) * 4096);
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int v = 0; v < kLive; ++v) acc[cg][v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[cg][v]);
+                    for (int v = 0; v < kFull; ++v)
+                        if (v < live_regs) acc[cg][rt][v] = __builtin_fmaf(t[v], static_cast<float>(c0[v]), acc[cg][rt][v]);
 #pragma unroll
-                for (int v = 0; v < kLive; ++v) acc[cg][v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[cg][v]);
-                fence_registers(acc[cg]);
+                    for (int v = 0; v < kFull; ++v)
+                        if (v < live_regs) acc[cg][rt][v] = __builtin_fmaf(t[16 + v], static_cast<float>(c1[v]), acc[cg][rt][v]);
+                    fence_registers(acc[cg][rt]);
+                }
             }
             // the slot is free: the stage two on takes it
             if (st + 2 < 4) issue_stage(st + 2);
@@ -846,26 +860,29 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may still be writing LDS when the region is reused
     }
 
-    // ---- the wavefronts' sums meet in LDS: [wave][cg][v][lane] (8 x 2 x 16 x 64 floats = the whole 64 KB)
+    // ---- the wavefronts' sums meet in LDS, one row tile at a time: [wave][cg][v][lane] (8 x 2 x 16 x 64 floats = the whole 64 KB)
     float* red = reinterpret_cast<float*>(bm_lds);
-    __syncthreads();
+    constexpr int kItems = 2 * 16 * 64;
 #pragma unroll
-    for (int cg = 0; cg < 2; ++cg)
+    for (int rt = 0; rt < kRT; ++rt) {
+        __syncthreads();
 #pragma unroll
-        for (int v = 0; v < kLive; ++v) red[((wave * 2 + cg) * kLive + v) * 64 + lane] = acc[cg][v];
-    __syncthreads();
-    constexpr int kItems = 2 * kLive * 64;
-    for (int i = tid; i < kItems; i += kBmThreads) {
-        float sum = red[i];
+        for (int cg = 0; cg < 2; ++cg)
 #pragma unroll
-        for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
-        const int l = i & 63, v = (i >> 6) % kLive, cg = (i >> 6) / kLive;
-        const int m = 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
-        const int n = n0 + 32 * cg + (l & 31);
-        if (m < rows && n < out_dim) {
-            const size_t at = static_cast<size_t>(m) * out_dim + n;
-            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
-            else dst[at] = finish_output(ep, n, at, sum);
+            for (int v = 0; v < 16; ++v) red[((wave * 2 + cg) * 16 + v) * 64 + lane] = acc[cg][rt][v];
+        __syncthreads();
+        for (int i = tid; i < kItems; i += kBmThreads) {
+            const int l = i & 63, v = (i >> 6) & 15, cg = i >> 10;
+            const int m = rt * 32 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
+            const int n = n0 + 32 * cg + (l & 31);
+            if (m < rows && n < out_dim) {
+                float sum = red[i];
+#pragma unroll
+                for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
+                const size_t at = static_cast<size_t>(m) * out_dim + n;
+                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                else dst[at] = finish_output(ep, n, at, sum);
+            }
         }
     }
 }
@@ -914,12 +931,13 @@ template <int kType>
 hipError_t bm_launch32(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
                        int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
     const dim3 grid(static_cast<unsigned>((out_dim + 63) / 64), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
-#define AFHIP_BM32(LIVE)                                                                                                                 \
-    hipLaunchKernelGGL((batch32_mfma_kernel<kType, LIVE>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, \
+#define AFHIP_BM32(RT, LIVE)                                                                                                                 \
+    hipLaunchKernelGGL((batch32_mfma_kernel<kType, RT, LIVE>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, \
                        weight, rows, in_dim, out_dim, share_blocks, ep, second)
-    if (rows <= 16) AFHIP_BM32(8);
-    else if (rows <= 24) AFHIP_BM32(12);
-    else AFHIP_BM32(16);
+    if (rows <= 16) AFHIP_BM32(1, 8);
+    else if (rows <= 24) AFHIP_BM32(1, 12);
+    else if (rows <= 32) AFHIP_BM32(1, 16);
+    else AFHIP_BM32(2, 16);
 #undef AFHIP_BM32
     return hipGetLastError();
 }
@@ -981,7 +999,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     // reach the kernel's K shares and pair launches that way; 0 switches the kernel off).
     const char* bound_env = std::getenv("AFHIP_BATCH32_MAX_WORKGROUPS");
     const long bound = bound_env ? std::atol(bound_env) : gemv_compute_units();
-    const bool thirty_two = !eight && rows <= 32 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
+    const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
                             static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
     if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
         const int pairs = (kb + 1) / 2;

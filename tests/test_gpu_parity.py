@@ -131,6 +131,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
+    (33, 1024, 12352), (48, 512, 12290), (64, 4096, 12288),  # ... and two row tiles
 ]
 
 
@@ -314,7 +315,7 @@ def test_committed_tiny_vectors(fmt_name, fmt, case, rows, in_dim, out_dim):
 
 
 @pytest.mark.parametrize("fmt,rows,in_dim,out_dim,pair", [(Q4, 29, 9216, 12288, False), (Q8, 20, 2048, 12290, True),
-                                                          (Q4, 20, 512, 12290, True), (Q4, 12, 8192, 12352, True)])
+                                                          (Q4, 20, 512, 12290, True), (Q4, 12, 8192, 12352, True), (Q4, 40, 8192, 12288, True)])
 def test_thirty_two_row_kernel_with_k_shares_and_pairs(fmt, rows, in_dim, out_dim, pair):
     """On this chip the 32-row kernel's grid bound (one workgroup per compute unit) keeps launches with
     K shares or two matrices on the older kernel; with the bound lifted they take the 32-row kernel and
