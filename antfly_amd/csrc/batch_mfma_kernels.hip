@@ -31,6 +31,9 @@
 //   * Up to eight rows on a grid that fills the chip take batch8_mfma_kernel (further down): the
 //     16x16x64 MFMA on two blocks at once, 32- or 64-column tiles, weights requested two stages
 //     ahead instead of all at once.
+//   * Nine to 64 rows on a wide matrix whose grid is one round of 64-column tiles take
+//     batch32_mfma_kernel (further down): this kernel's arithmetic, staged weight requests, one
+//     workgroup per compute unit.
 #include <hip/hip_runtime.h>
 
 #include <cstdlib>
@@ -662,7 +665,7 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
 }
 
 // ---------------------------------------------------------------------------------------------
-// Nine to 32 rows on a matrix wide enough for 64-column tiles: batch_mfma_kernel's arithmetic
+// Nine to 64 rows (one or two row tiles) on a matrix wide enough for 64-column tiles: batch_mfma_kernel's arithmetic
 // (v_mfma_i32_32x32x32_i8 per block, scale products of a pair of blocks from one
 // v_mfma_f32_32x32x1_2b_f32, one convert and one multiply-add per live result register) with what
 // the eight-row kernel showed to matter:
@@ -992,7 +995,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
     const int real_shares = (kb + share_blocks - 1) / share_blocks;
     const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);
-    // Nine to 32 rows on a matrix wide enough for 64-column tiles (and rows of whole 16-byte runs of
+    // Nine to 64 rows on a matrix wide enough for 64-column tiles (and rows of whole 16-byte runs of
     // scales), with no more workgroups than compute units: batch32_mfma_kernel holds one workgroup per
     // unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
     // unit (N = 20480: 21.1 against 18.5 us).  AFHIP_BATCH32_MAX_WORKGROUPS overrides the bound (tests
