@@ -1024,21 +1024,30 @@ afhip_status afhip_launch_dequantize_f32(void* stream, int tensor_type, int layo
 
 afhip_status afhip_launch_quantize_rows(void* stream, int tensor_type, afhip_buffer dst_raw, afhip_buffer input,
                                         afhip_buffer row_ids_i64, size_t rows, size_t dim, size_t dst_rows) {
-    const size_t bb = block_bytes(tensor_type);
+    const bool q4k = tensor_type == AFHIP_TYPE_Q4_K;
+    const size_t bb = q4k ? 144 : block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
-    if (dim == 0 || dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
+    const size_t block_values = q4k ? 256 : 32;
+    if (dim == 0 || dim % block_values != 0) return AFHIP_ERR_INVALID_STATE;
     const bool scatter = row_ids_i64.ptr != 0;
     if (!scatter && dst_rows != rows) return AFHIP_ERR_INVALID_STATE;
     size_t in_count, in_bytes, d_count, d_bytes, id_bytes;
     if (!checked_mul(rows, dim, &in_count) || !checked_mul(in_count, 4, &in_bytes) ||
-        !checked_mul(dst_rows, dim, &d_count) || !checked_mul(d_count / 32, bb, &d_bytes) ||
+        !checked_mul(dst_rows, dim, &d_count) || !checked_mul(d_count / block_values, bb, &d_bytes) ||
         !checked_mul(rows, 8, &id_bytes))
         return AFHIP_ERR_INVALID_STATE;
     if (in_bytes > input.len || d_bytes > dst_raw.len || (scatter && id_bytes > row_ids_i64.len)) return AFHIP_ERR_INVALID_STATE;
     if (in_count == 0) return AFHIP_OK;
-    if (dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || dst_raw.ptr == 0 || dst_raw.ptr % 2 != 0 ||
+    if (dim > 0x7fffffff || input.ptr == 0 || input.ptr % 16 != 0 || dst_raw.ptr == 0 || dst_raw.ptr % (q4k ? 16 : 2) != 0 ||
         (scatter && row_ids_i64.ptr % 8 != 0))
         return AFHIP_ERR_INVALID_STATE;
+    if (q4k) {
+        hipError_t e = launch_quantize_q4k_rows(static_cast<hipStream_t>(stream), reinterpret_cast<uint8_t*>(dst_raw.ptr),
+                                                reinterpret_cast<const float*>(input.ptr),
+                                                scatter ? reinterpret_cast<const long long*>(row_ids_i64.ptr) : nullptr, rows,
+                                                static_cast<int>(dim), dst_rows);
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     hipError_t e = launch_quantize_rows(static_cast<hipStream_t>(stream), tensor_type,
                                         reinterpret_cast<uint8_t*>(dst_raw.ptr), reinterpret_cast<const float*>(input.ptr),
                                         scatter ? reinterpret_cast<const long long*>(row_ids_i64.ptr) : nullptr, rows,

@@ -97,6 +97,89 @@ __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restr
     }
 }
 
+// set_rows / cpy_f32_to_q for Q4_K: rows of f32 -> 144-byte super-blocks (raw layout) at row
+// ids[t] of the destination (ids == nullptr: rows in order), quantizeQ4_KBlock,
+// gguf/quant_codec.zig:1183-1238, byte for byte.  Per sub-block of 32:
+//   min_mag = max(-min, 0), scale = (max + min_mag) / 15 (1 when that sum is 0);
+// per super-block d = max scale / 63, dmin = max min_mag / 63 (1 when 0), stored as fp16;
+//   sc = clamp(round(scale / d), 0, 63), m = clamp(round(min_mag / dmin), 0, 63)  (f32 d, dmin),
+//   nibble = clamp(round((x + min_mag) * (1 / scale)), 0, 15)                      (the unrounded scale),
+// round = half away from zero; every quotient is a correctly rounded f32 division.
+// A wavefront is one super-block: lane l holds values 4l .. 4l+3 (one coalesced 16-byte load),
+// the eight lanes of (l >> 3) are a sub-block.  The lanes of sub-block 2c take the nibbles of
+// sub-block 2c+1 from eight lanes up and store four bytes each; lane 0 stores the header.
+__device__ __forceinline__ float min_over_8(float v) {
+    v = fminf(v, dpp_move<kDppXor1>(v));
+    v = fminf(v, dpp_move<kDppXor2>(v));
+    v = fminf(v, dpp_move<kDppHalfMirror>(v));
+    return v;
+}
+// max over the eight sub-blocks of a value that is uniform inside each of them; result uniform
+__device__ __forceinline__ float max_over_sub_blocks(float v) {
+    const int bits = __builtin_bit_cast(int, v);
+    float m = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+#pragma unroll
+    for (int s = 1; s < 8; ++s) m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 8 * s)));
+    return m;
+}
+// round half away from zero of t >= 0, clamped to [0, hi]
+__device__ __forceinline__ uint32_t round_clamp(float t, int hi) {
+    return static_cast<uint32_t>(min(max(static_cast<int>(t + 0x1.fffffep-2f), 0), hi));
+}
+
+template <bool kNarrow>
+__global__ __launch_bounds__(256) void quantize_q4k_rows_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
+                                                                const long long* __restrict__ ids, size_t rows, int dim,
+                                                                size_t dst_rows) {
+    const size_t kb = static_cast<size_t>(dim / kQ4kBlockValues);
+    const size_t units = rows * kb * 64;  // a multiple of 64: a wavefront is live or idle as a whole
+    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
+         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
+        const float4 v = reinterpret_cast<const float4*>(x)[u];
+        const float lo = min_over_8(fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
+        const float hi = max_over_8(fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
+        const float min_mag = fmaxf(-lo, 0.0f);
+        const float range = hi + min_mag;
+        const float scale = range == 0.0f ? 1.0f : range / 15.0f;
+        const float max_scale = max_over_sub_blocks(scale), max_min = max_over_sub_blocks(min_mag);
+        const float d = max_scale == 0.0f ? 1.0f : max_scale / 63.0f;
+        const float dmin = max_min == 0.0f ? 1.0f : max_min / 63.0f;
+        const uint32_t sc = max_scale == 0.0f ? 0u : round_clamp(scale / d, 63);
+        const uint32_t mn = max_min == 0.0f ? 0u : round_clamp(min_mag / dmin, 63);
+        const float inv = scale == 0.0f ? 0.0f : 1.0f / scale;
+        const uint32_t mine = round_clamp((v.x + min_mag) * inv, 15) | (round_clamp((v.y + min_mag) * inv, 15) << 8) |
+                              (round_clamp((v.z + min_mag) * inv, 15) << 16) | (round_clamp((v.w + min_mag) * inv, 15) << 24);
+        const uint32_t other = static_cast<uint32_t>(__shfl_down(static_cast<int>(mine), 8));
+        // the 6-bit pairs of all eight sub-blocks, as uniform values
+        uint32_t scs[8], mns[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            scs[s] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(sc), 8 * s));
+            mns[s] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mn), 8 * s));
+        }
+        const size_t tb = u >> 6;
+        const size_t t = kNarrow ? static_cast<uint32_t>(tb) / static_cast<uint32_t>(kb) : tb / kb, b = tb - t * kb;
+        const long long row = ids ? ids[t] : static_cast<long long>(t);
+        if (row < 0 || static_cast<size_t>(row) >= dst_rows) continue;  // a row id outside the destination writes nothing
+        uint8_t* out = dst + (static_cast<size_t>(row) * kb + b) * kQ4kBlockBytes;
+        const int lane = static_cast<int>(u & 63), sub = lane >> 3, j = lane & 7;
+        if ((sub & 1) == 0) *reinterpret_cast<uint32_t*>(out + 16 + 32 * (sub >> 1) + 4 * j) = mine | (other << 4);
+        if (lane == 0) {
+            q4k_u32x4 header;
+            header.x = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d)) |
+                       (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(dmin))) << 16);
+            header.y = header.z = header.w = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {  // packQ4KScaleMins, gguf/quant_codec.zig:1273-1287
+                header.y |= ((scs[i] & 63) | ((scs[i + 4] >> 4) << 6)) << (8 * i);
+                header.z |= ((mns[i] & 63) | ((mns[i + 4] >> 4) << 6)) << (8 * i);
+                header.w |= ((scs[i + 4] & 15) | ((mns[i + 4] & 15) << 4)) << (8 * i);
+            }
+            *reinterpret_cast<q4k_u32x4*>(out) = header;
+        }
+    }
+}
+
 // Y[r][o] = sum over K of x[r][k] * w[o][k] for kRows rows of f32 activations.
 // A wavefront owns kCols consecutive output columns and one K-slice of 8 super-blocks
 // (2048 values); eight lanes share a super-block, each with one 16-byte run of nibbles:
@@ -618,6 +701,17 @@ hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint
     if (grid > 65536) grid = 65536;
     hipLaunchKernelGGL(dequantize_q4k_rows_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst, weight, ids,
                        rows, dim, weight_rows);
+    return hipGetLastError();
+}
+
+hipError_t launch_quantize_q4k_rows(hipStream_t stream, uint8_t* dst_raw, const float* x, const long long* ids, size_t rows,
+                                    int dim, size_t dst_rows) {
+    if (rows == 0 || dim == 0) return hipSuccess;
+    size_t grid = (rows * static_cast<size_t>(dim >> 2) + 255) / 256;
+    if (grid > 65536) grid = 65536;
+    const bool narrow = rows * static_cast<size_t>(dim / kQ4kBlockValues) <= 0xFFFFFFFFull;
+    if (narrow) hipLaunchKernelGGL(quantize_q4k_rows_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+    else hipLaunchKernelGGL(quantize_q4k_rows_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
     return hipGetLastError();
 }
 

@@ -152,6 +152,9 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
                            int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
                                       size_t rows, int dim, size_t weight_rows);
+// set_rows / cpy_f32_to_q for Q4_K (raw layout; dst_raw 16-byte aligned, dim a multiple of 256).
+hipError_t launch_quantize_q4k_rows(hipStream_t stream, uint8_t* dst_raw, const float* x, const long long* ids, size_t rows,
+                                    int dim, size_t dst_rows);
 
 // Q4_K in the tile-major layout (32 output columns x one super-block per 4608-byte tile; columns
 // past out_dim zero): size, repack from the raw GGUF bytes, the MFMA GEMV for any number of

@@ -223,9 +223,9 @@ def main() -> int:
         out = {}
         f32_bytes = rows * dim * 4
         dense = torch.empty((rows, dim), dtype=torch.float32, device=dev)
-        for name, fmt, bb in (("q4_0", Q4, 18), ("q8_0", Q8, 34)):
+        for name, fmt, bb, bv in (("q4_0", Q4, 18, 32), ("q8_0", Q8, 34, 32), ("q4_k", Q4K, 144, 256)):
             w = prepared_copies(fmt, rows, dim, 1, 41)[0]
-            q_bytes = rows * dim // 32 * bb
+            q_bytes = rows * dim // bv * bb
             sec = timed(lambda st: kernels.launchDequantizeF32(st, fmt, _lib.LAYOUT_PREPARED, buf(dense), buf(w), rows, dim))
             out[f"cpy_{name}_to_f32"] = {"us_per_call": round(sec * 1e6, 2),
                                         "GBps": round((q_bytes + f32_bytes) / sec / 1e9, 1),
@@ -240,7 +240,7 @@ def main() -> int:
             emb = torch.empty((tokens, dim), dtype=torch.float32, device=dev)
             sec = timed(lambda st: kernels.launchEmbeddingLookupF32(st, fmt, _lib.LAYOUT_PREPARED, buf(emb), buf(w), buf(ids),
                                                                    tokens, dim, rows))
-            moved = tokens * dim // 32 * bb + tokens * dim * 4
+            moved = tokens * dim // bv * bb + tokens * dim * 4
             out[f"get_rows_{name}_512_tokens"] = {"us_per_call": round(sec * 1e6, 2), "GBps": round(moved / sec / 1e9, 1)}
         out["what"] = (f"row operators on a {rows} x {dim} tensor: dequantize all of it, quantize all of it "
                        "(bytes = quantized + f32 side), embedding lookup of 512 rows")

@@ -269,7 +269,8 @@ afhip_status afhip_launch_dequantize_f32(void *stream, int tensor_type, int layo
 /* cpy_f32_to_q (row_ids_i64.ptr == 0: rows in order, dst_rows == rows) and set_rows
  * (row t of `input` becomes row row_ids[t] of the [dst_rows, dim] destination): f32 ->
  * raw GGUF blocks with the engine's weight quantizers (gguf/quant_codec.zig:601-623
- * Q8_0, :895-910 and :1261-1265 Q4_0).  dst_raw must be 2-byte aligned.  set_rows
+ * Q8_0, :895-910 and :1261-1265 Q4_0, :1183-1238 Q4_K).  dst_raw must be 2-byte aligned
+ * (Q4_K: 16-byte aligned, dim a multiple of 256).  set_rows
  * preconditions: a row id outside [0, dst_rows) writes nothing (the row is skipped); two
  * rows with the same id race and either may win -- give every destination row at most
  * once. */

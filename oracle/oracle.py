@@ -61,6 +61,8 @@ def lib() -> C.CDLL:
         L.afo_linear_no_bias.argtypes = [i32, vp, vp, vp, sz, sz, sz, i32]
         L.afo_q4k_unpack_scale_mins.argtypes = [vp, vp, vp]
         L.afo_dequantize_q4_k.argtypes = [vp, sz, vp]
+        L.afo_quantize_q4_k_block.argtypes = [vp, vp]
+        L.afo_quantize_q4_k_block.restype = None
         L.afo_linear_q4_k.argtypes = [vp, vp, vp, sz, sz, sz]
         L.afo_linear_q4_k_f64.argtypes = [vp, vp, vp, sz, sz, sz]
         L.afo_uses_q4k_q8k_activation.argtypes = [sz, sz, sz]
@@ -252,6 +254,15 @@ def dequantize_q4_k(raw) -> np.ndarray:
     out = np.zeros(r.size // 144 * 256, np.float32)
     lib().afo_dequantize_q4_k(_p(r), r.size // 144, _p(out))
     return out
+
+
+def quantize_q4_k(w) -> np.ndarray:
+    """f32 [.., 256 n] -> raw Q4_K super-blocks (the reference's weight quantizer)."""
+    w = _f32(w).reshape(-1, 256)
+    out = np.zeros((w.shape[0], 144), dtype=np.uint8)
+    for i in range(w.shape[0]):
+        lib().afo_quantize_q4_k_block(_p(w[i]), _p(out[i]))
+    return out.reshape(-1)
 
 
 def uses_q4k_q8k_activation(rows, in_dim, out_dim) -> bool:

@@ -699,6 +699,61 @@ void afo_dequantize_q4_k(const uint8_t *raw, size_t n_blocks, float *out) {
     }
 }
 
+static uint8_t quantize_unsigned(float v, float inv, float max_q) {
+    /* quant_codec.zig:1267-1271 */
+    if (inv == 0.0f) return 0;
+    return (uint8_t)clampf(roundf(v * inv), 0.0f, max_q);
+}
+
+void afo_quantize_q4_k_block(const float *x, uint8_t *out) {
+    /* quantizeQ4_KBlock, quant_codec.zig:1183-1238; header packing :1273-1287 */
+    float sub_scale[8], sub_min[8];
+    float max_scale = 0.0f, max_min = 0.0f;
+    memset(out, 0, AFO_Q4_K_BLOCK_BYTES);
+    for (int s = 0; s < 8; s++) {
+        const float *v = x + 32 * s;
+        float lo = v[0], hi = v[0];
+        for (int i = 1; i < 32; i++) {
+            lo = v[i] < lo ? v[i] : lo;
+            hi = v[i] > hi ? v[i] : hi;
+        }
+        float min_mag = -lo > 0.0f ? -lo : 0.0f;
+        float scale = hi + min_mag == 0.0f ? 1.0f : (hi + min_mag) / 15.0f;
+        sub_scale[s] = scale;
+        sub_min[s] = min_mag;
+        max_scale = scale > max_scale ? scale : max_scale;
+        max_min = min_mag > max_min ? min_mag : max_min;
+    }
+    float d = max_scale == 0.0f ? 1.0f : max_scale / 63.0f;
+    float dmin = max_min == 0.0f ? 1.0f : max_min / 63.0f;
+    uint16_t hd = afo_f32_to_fp16(d), hm = afo_f32_to_fp16(dmin);
+    out[0] = (uint8_t)(hd & 0xff);
+    out[1] = (uint8_t)(hd >> 8);
+    out[2] = (uint8_t)(hm & 0xff);
+    out[3] = (uint8_t)(hm >> 8);
+    uint8_t sc[8], mn[8];
+    for (int s = 0; s < 8; s++) {
+        sc[s] = max_scale == 0.0f ? 0 : (uint8_t)clampf(roundf(sub_scale[s] / d), 0.0f, 63.0f);
+        mn[s] = max_min == 0.0f ? 0 : (uint8_t)clampf(roundf(sub_min[s] / dmin), 0.0f, 63.0f);
+    }
+    uint8_t *h = out + 4;
+    for (int j = 0; j < 4; j++) {
+        h[j] = (uint8_t)((sc[j] & 63) | ((sc[j + 4] >> 4) << 6));
+        h[4 + j] = (uint8_t)((mn[j] & 63) | ((mn[j + 4] >> 4) << 6));
+        h[8 + j] = (uint8_t)((sc[j + 4] & 0x0F) | ((mn[j + 4] & 0x0F) << 4));
+    }
+    for (int c = 0; c < 4; c++) {
+        int s0 = 2 * c, s1 = s0 + 1;
+        float inv0 = sub_scale[s0] == 0.0f ? 0.0f : 1.0f / sub_scale[s0];
+        float inv1 = sub_scale[s1] == 0.0f ? 0.0f : 1.0f / sub_scale[s1];
+        for (int i = 0; i < 32; i++) {
+            uint8_t q0 = quantize_unsigned(x[32 * s0 + i] + sub_min[s0], inv0, 15.0f);
+            uint8_t q1 = quantize_unsigned(x[32 * s1 + i] + sub_min[s1], inv1, 15.0f);
+            out[16 + 32 * c + i] = (uint8_t)(q0 | (q1 << 4));
+        }
+    }
+}
+
 int afo_linear_q4_k(const float *x, const uint8_t *w, float *y, size_t rows, size_t in_dim, size_t out_dim) {
     if (in_dim % AFO_Q4_K_BLOCK_VALUES != 0) return -1;
     size_t kb = in_dim / AFO_Q4_K_BLOCK_VALUES;

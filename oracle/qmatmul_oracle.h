@@ -130,6 +130,13 @@ void afo_q4k_unpack_scale_mins(const uint8_t *scales12, uint8_t *scs8, uint8_t *
 /* dequantizeQ4K, INF/gguf/quant_codec.zig:2624-2663: w = (d*sc)*f32(q) - (dmin*m), low
  * nibbles of a 32-byte chunk = sub-block 2c, high nibbles = sub-block 2c+1. */
 void afo_dequantize_q4_k(const uint8_t *raw, size_t n_blocks, float *out);
+/* quantizeQ4_KBlock, INF/gguf/quant_codec.zig:1183-1238: per sub-block of 32 min_mag =
+ * max(-min, 0), scale = (max + min_mag) / 15 (1 when that sum is 0); d = max scale / 63,
+ * dmin = max min_mag / 63 (stored as fp16; the f32 values divide the sub-block figures);
+ * sc = clamp(round(scale / d), 0, 63), m likewise, packed by packQ4KScaleMins (:1273-1287);
+ * nibble = clamp(round((x + min_mag) * (1 / scale)), 0, 15) with the UNROUNDED sub-block
+ * scale, round = half away from zero. */
+void afo_quantize_q4_k_block(const float *x256, uint8_t *out144);
 /* y[r][o] = sum_b dot(x block, dequantized block) in f32, values in natural order
  * (dotQ4_KBlock, INF/ops/native_compute.zig:31075-31113, with one accumulator lane:
  * the engine's lane count, and with it the order of the f32 sums, is a build

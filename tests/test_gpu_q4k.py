@@ -85,6 +85,86 @@ def test_dequantize_and_get_rows_bit_exact(rows, dim, layout):
     assert np.array_equal(emb.cpu().numpy().view(np.uint32), table[ids].view(np.uint32))
 
 
+def values_for_q4k_quantizer(seed, rows, dim):
+    """Normal data of mixed magnitudes, a zero sub-block, a zero super-block, one-signed sub-blocks, exact ties."""
+    rng = np.random.default_rng(seed)
+    x = (rng.standard_normal((rows * dim // 32, 32)) * np.exp2(rng.integers(-10, 10, (rows * dim // 32, 1)))).astype(np.float32)
+    x[1] = 0.0
+    x[3] = np.abs(x[3])
+    x[4] = -np.abs(x[4])
+    x[5] = np.round(x[5] * 4) / 4
+    x[6, :] = np.float32(-2.5)
+    if x.shape[0] >= 24:
+        x[8:16] = 0.0
+        x[16:24] = np.abs(x[16:24])  # no minimum in the whole super-block: dmin = 1, m = 0
+    return x.reshape(rows, dim)
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 256), (3, 1024), (9, 4096), (130, 512)])
+def test_quantize_rows_matches_weight_quantizer(rows, dim, kats):
+    print(f"case: q4_k cpy_f32_to_q rows={rows} dim={dim}", flush=True)
+    x = values_for_q4k_quantizer(31, rows, dim)
+    if dim == 256:  # the block whose bytes the reference's own test fixes (gguf/quant_codec.zig:2925-2955)
+        h = kats["q4_k"]["header_packing"]
+        x = np.array([h["scs"][sub] * (i % 16) - h["mins"][sub] for sub in range(8) for i in range(32)], np.float32).reshape(1, 256)
+    xd = G.to_dev(x)
+    nbytes = rows * dim // 256 * 144
+    out = torch.full((nbytes + 16,), 0xEE, dtype=torch.uint8, device=G.DEV)
+    kernels.launchQuantizeRows(G.stream(), Q4K, G.buf(out[:nbytes]), G.buf(xd), rows, dim)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    assert (got[nbytes:] == 0xEE).all()
+    assert np.array_equal(got[:nbytes], O.quantize_q4_k(x))
+    if dim == 256:
+        assert got[:nbytes].tolist() == h["header"] + h["qs_32"] * 4
+    # and back: the dequantized bytes are the oracle's dequantization of the same bytes
+    back = torch.empty((rows, dim), dtype=torch.float32, device=G.DEV)
+    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(back), G.buf(out[:nbytes]), rows, dim)
+    torch.cuda.synchronize()
+    assert np.array_equal(back.cpu().numpy().view(np.uint32), O.dequantize_q4_k(got[:nbytes]).reshape(rows, dim).view(np.uint32))
+
+
+def test_set_rows_scatters_and_skips_rows_outside():
+    dst_rows, dim = 6, 512
+    row_bytes = dim // 256 * 144
+    x = values_for_q4k_quantizer(32, 4, dim)
+    canvas = torch.full(((dst_rows + 2) * row_bytes,), 0xAB, dtype=torch.uint8, device=G.DEV)
+    dst = canvas[row_bytes:(dst_rows + 1) * row_bytes]
+    rid = np.array([5, -2, dst_rows, 0], dtype=np.int64)
+    x_d, rid_d = G.to_dev(x), G.to_dev(rid)  # (kept alive until the launch has run)
+    kernels.launchQuantizeRows(G.stream(), Q4K, G.buf(dst), G.buf(x_d), 4, dim, row_ids_i64=G.buf(rid_d), dst_rows=dst_rows)
+    torch.cuda.synchronize()
+    got = canvas.cpu().numpy().reshape(dst_rows + 2, row_bytes)
+    want = O.quantize_q4_k(x).reshape(4, row_bytes)
+    assert np.array_equal(got[1 + 5], want[0]) and np.array_equal(got[1 + 0], want[3])
+    assert (got[[0, 2, 3, 4, 5, dst_rows + 1]] == 0xAB).all()
+    with pytest.raises(_lib.InvalidHipState):  # a row is whole super-blocks
+        kernels.launchQuantizeRows(G.stream(), Q4K, G.buf(dst), G.buf(x_d), 4, 288)
+    with pytest.raises(_lib.InvalidHipState):  # destination too short
+        kernels.launchQuantizeRows(G.stream(), Q4K, G.buf(dst[:row_bytes]), G.buf(x_d), 4, dim)
+
+
+def test_quantize_full_size_round_trip_properties():
+    """A whole FFN matrix (14336 x 4096): every value comes back within half a nibble step of its sub-block plus
+    the 6-bit rounding of the sub-block's scale and minimum; the first rows equal the oracle's bytes."""
+    rows, dim = 14336, 4096
+    x = synth.activations(12, 512, dim)
+    x = np.tile(x, (rows // 512, 1)) * np.linspace(0.5, 2.0, rows, dtype=np.float32)[:, None]
+    xd = G.to_dev(x)
+    q = torch.empty(rows * dim // 256 * 144, dtype=torch.uint8, device=G.DEV)
+    kernels.launchQuantizeRows(G.stream(), Q4K, G.buf(q), G.buf(xd), rows, dim)
+    back = torch.empty((rows, dim), dtype=torch.float32, device=G.DEV)
+    kernels.launchDequantizeF32(G.stream(), Q4K, RAW, G.buf(back), G.buf(q), rows, dim)
+    torch.cuda.synchronize()
+    assert np.array_equal(q[:16 * dim // 256 * 144].cpu().numpy(), O.quantize_q4_k(x[:16]))
+    sub = xd.view(rows, dim // 256, 8, 32)
+    mins = (-sub.amin(dim=3)).clamp_min(0)
+    span = sub.amax(dim=3) + mins
+    bound = span.amax(dim=2) / 30 + 15 * (span.amax(dim=2) / 15 / 63) * 0.51 + mins.amax(dim=2) / 63 * 0.51
+    err = (back - xd).abs().view(rows, dim // 256, 256).amax(dim=2)
+    assert bool((err <= bound * 1.05).all())  # 5 %: the fp16 rounding of d and dmin
+
+
 SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130), (3, 1024, 40), (5, 4096, 96),
           (1, 14336, 48), (2, 14336, 20), (9, 2048, 24), (1, 16384, 8), (3, 16384, 12), (4, 14336, 8)]
 

@@ -387,6 +387,99 @@ def test_q4_k_against_independent_numpy_form():
     del wf
 
 
+def numpy_pack_q4_k(d, dmin, sc, mn, q):
+    """Independent packer of the published ggml Q4_K layout: sc, mn [n, 8] (6 bits), q [n, 8, 32] nibbles."""
+    n = sc.shape[0]
+    b = np.zeros((n, 144), np.uint8)
+    b[:, 0:2] = np.asarray(d, np.float16).reshape(n, 1).view(np.uint8)
+    b[:, 2:4] = np.asarray(dmin, np.float16).reshape(n, 1).view(np.uint8)
+    b[:, 4:8] = (sc[:, :4] & 63) | ((sc[:, 4:] >> 4) << 6)
+    b[:, 8:12] = (mn[:, :4] & 63) | ((mn[:, 4:] >> 4) << 6)
+    b[:, 12:16] = (sc[:, 4:] & 15) | ((mn[:, 4:] & 15) << 4)
+    qq = q.reshape(n, 4, 2, 32)
+    b[:, 16:] = (qq[:, :, 0, :] | (qq[:, :, 1, :] << 4)).reshape(n, 128)
+    return b.reshape(-1)
+
+
+def round_half_away_f32(v):
+    v64 = np.asarray(v, np.float32).astype(np.float64)  # exact; + 0.5 is exact in f64 too
+    return np.sign(v64) * np.floor(np.abs(v64) + 0.5)
+
+
+def numpy_quantize_q4_k(x):
+    """Vectorised f32 restatement of the quantizer from its description (quant_codec.zig:1183-1238)."""
+    f = np.float32
+    v = np.asarray(x, f).reshape(-1, 8, 32)
+    lo, hi = v.min(axis=2), v.max(axis=2)
+    mm = np.maximum(-lo, f(0))
+    rng = (hi + mm).astype(f)
+    scale = np.where(rng == 0, f(1), (rng / f(15)).astype(f)).astype(f)
+    max_scale, max_min = scale.max(axis=1), mm.max(axis=1)
+    d = np.where(max_scale == 0, f(1), (max_scale / f(63)).astype(f)).astype(f)
+    dmin = np.where(max_min == 0, f(1), (max_min / f(63)).astype(f)).astype(f)
+    sc = np.clip(round_half_away_f32((scale / d[:, None]).astype(f)), 0, 63).astype(np.uint8)
+    mn = np.clip(round_half_away_f32((mm / dmin[:, None]).astype(f)), 0, 63).astype(np.uint8)
+    mn[max_min == 0] = 0
+    inv = np.where(scale == 0, f(0), (f(1) / scale).astype(f)).astype(f)
+    t = ((v + mm[:, :, None]).astype(f) * inv[:, :, None]).astype(f)
+    q = np.clip(round_half_away_f32(t), 0, 15).astype(np.uint8)
+    return numpy_pack_q4_k(d, dmin, sc, mn, q)
+
+
+def test_q4_k_quantizer_reference_vectors(kats):
+    k = kats["q4_k"]
+    h = k["header_packing"]
+    x = np.array([h["scs"][sub] * (i % 16) - h["mins"][sub] for sub in range(8) for i in range(32)], np.float32)
+    assert O.quantize_q4_k(x).tolist() == h["header"] + h["qs_32"] * 4
+    r = k["quantizer_round_trip"]
+    ramp = (r["start"] + r["step"] * np.arange(r["count"])).astype(np.float32)
+    assert np.abs(O.dequantize_q4_k(O.quantize_q4_k(ramp)) - ramp).max() <= r["tolerance_abs"]
+
+
+def test_q4_k_quantizer_by_construction_and_against_numpy_form():
+    rng = np.random.default_rng(41)
+    # values on a grid the format represents exactly: x = 2^e * (sc * q - m) with one sub-block at sc = 63, one
+    # at m = 63 (so d = dmin = 2^e), every sub-block spanning q = 0 .. 15 -> the bytes are known in advance
+    n = 24
+    sc = rng.integers(1, 64, (n, 8)).astype(np.uint8)
+    mn = rng.integers(0, 64, (n, 8)).astype(np.uint8)
+    sc[np.arange(n), rng.integers(0, 8, n)] = 63
+    mn[np.arange(n), rng.integers(0, 8, n)] = 63
+    q = rng.integers(0, 16, (n, 8, 32)).astype(np.uint8)
+    q[:, :, 3], q[:, :, 17] = 0, 15
+    e = np.exp2(rng.integers(-9, 6, n)).astype(np.float32)
+    x = (e[:, None, None] * (sc[:, :, None].astype(np.float32) * q - mn[:, :, None].astype(np.float32))).astype(np.float32)
+    want = numpy_pack_q4_k(e, e, sc, mn, q)
+    got = O.quantize_q4_k(x)
+    assert np.array_equal(got, want)
+    assert np.array_equal(O.dequantize_q4_k(got), x.reshape(-1))
+    # an all-zero super-block: every sub-block scale is 1, d = 1/63 -> sc = 63; no minimum -> dmin = 1, m = 0
+    z = O.quantize_q4_k(np.zeros(256, np.float32))
+    assert np.array_equal(z, numpy_pack_q4_k([np.float32(1) / np.float32(63)], [1.0], np.full((1, 8), 63, np.uint8),
+                                             np.zeros((1, 8), np.uint8), np.zeros((1, 8, 32), np.uint8)))
+    # all-positive values: no offset, nibble = round(15 x / max); all-negative: offset -min, the largest value is
+    # not at nibble 15
+    pos = np.tile(np.linspace(1.0, 3.0, 32, dtype=np.float32), 8)
+    bp = O.quantize_q4_k(pos)
+    assert bp[2:4].tolist() == [0x00, 0x3C] and not bp[8:12].any() and (bp[12:16] >> 4).tolist() == [0] * 4
+    assert (bp[16:48] & 15).tolist() == [int(np.floor(15.0 * v / 3.0 + 0.5)) for v in pos[:32].astype(np.float64)]
+    neg = -pos
+    bn = O.quantize_q4_k(neg)
+    assert (bn[16:48] & 15).tolist() == [int(np.floor((float(v) + 3.0) / (np.float32(2.0) / np.float32(15.0)) + 0.5)) for v in neg[:32]]
+    # random data, random magnitudes per sub-block, ties included: byte-identical to the vectorised restatement
+    xr = (rng.standard_normal((64, 8, 32)) * np.exp2(rng.integers(-12, 12, (64, 8, 1)))).astype(np.float32)
+    xr[5, 2] = 0.0
+    xr[6] = np.abs(xr[6])
+    xr[7, :, :] = np.round(xr[7] * 2) / 2
+    assert np.array_equal(O.quantize_q4_k(xr), numpy_quantize_q4_k(xr))
+    # and close to the input: nibble rounding (scale / 2) plus the 6-bit rounding of scale and minimum
+    deq = O.dequantize_q4_k(O.quantize_q4_k(xr)).reshape(64, 8, 32)
+    span = (xr.max(axis=2) + np.maximum(-xr.min(axis=2), 0)).max(axis=1)
+    mins = np.maximum(-xr.min(axis=2), 0).max(axis=1)
+    bound = span / 30 + 15 * (span / 15 / 63) * 0.51 + mins / 63 * 0.51
+    assert (np.abs(deq - xr).max(axis=(1, 2)) <= bound * 1.01 + 1e-30).all()
+
+
 # ---------------------------------------------------------------- Q4_K with Q8_K activations
 
 def test_q8k_route_gate_is_the_reference_list():
