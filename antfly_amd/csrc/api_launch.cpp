@@ -174,13 +174,23 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
         if (workspace.ptr == 0 || workspace.ptr % 16 != 0 || workspace.len < q4k_q8k_workspace_bytes(rows, in_dim))
             return AFHIP_ERR_INVALID_STATE;
         if (counters) counters->activation_quant++;
-        hipError_t e = launch_quantize_q8k(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
-                                           static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
+        const bool fused = linear_q4k_q8k_fuses_quantizer(tiled, rows, in_dim);  // decode: the quantizer inside the matmul launch
+        hipError_t e = fused ? hipSuccess
+                             : launch_quantize_q8k(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
+                                                   static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
         for (int i = 0; e == hipSuccess && i < (pair ? 2 : 1); ++i) {
             if (counters) {
                 if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
                 else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
                 else counters->mm++;
+            }
+            if (fused) {
+                e = launch_linear_q4k_q8k_fused(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
+                                                reinterpret_cast<const float*>(input.ptr),
+                                                reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
+                                                static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
+                                                i ? ep_b : ep);
+                continue;
             }
             e = launch_linear_q4k_q8k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
                                       reinterpret_cast<const void*>(workspace.ptr),

@@ -463,27 +463,38 @@ hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const
 // values per lane.  d = max|x| / 127 (1 for a zero block), q = clamp(round_half_away(x * (1 / d))),
 // sums[block][s] = sum of the 32 quantized values of sub-block s (the engine adds its two
 // 16-value sums whenever it uses them, :32018-32022).
+struct Q8kLane {
+    int packed;  // the lane's four quantized values
+    int total;   // sum of the 32 quantized values of the lane's sub-block (lane >> 3)
+    float d;     // the block's scale
+};
+__device__ __forceinline__ Q8kLane quantize_q8k_block(const float4 v) {
+    float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    m = max_over_8(m);
+    m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
+    const int bits = __builtin_bit_cast(int, m);
+    m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)),
+                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))),
+              fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)),
+                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48))));
+    Q8kLane out;
+    out.d = act_scale(m);
+    const float inv = m == 0.0f ? 0.0f : 1.0f / out.d;
+    const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
+    const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
+    out.packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+    out.total = sum_over_8(q0 + q1 + q2 + q3);
+    return out;
+}
+
 __global__ __launch_bounds__(256) void quantize_q8k_kernel(const float* __restrict__ x, size_t blocks, int8_t* __restrict__ q,
                                                            float* __restrict__ d, int* __restrict__ sums) {
     const int lane = threadIdx.x & 63;
     for (size_t b = blockIdx.x * 4 + (threadIdx.x >> 6); b < blocks; b += static_cast<size_t>(gridDim.x) * 4) {
-        const float4 v = reinterpret_cast<const float4*>(x)[b * 64 + lane];
-        float m = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        m = max_over_8(m);
-        m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
-        const int bits = __builtin_bit_cast(int, m);
-        m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0)),
-                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16))),
-                  fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32)),
-                        __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48))));
-        const float s = act_scale(m);
-        const float inv = m == 0.0f ? 0.0f : 1.0f / s;
-        const int q0 = act_quant(v.x, inv), q1 = act_quant(v.y, inv);
-        const int q2 = act_quant(v.z, inv), q3 = act_quant(v.w, inv);
-        reinterpret_cast<int*>(q)[b * 64 + lane] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-        const int total = sum_over_8(q0 + q1 + q2 + q3);
-        if ((lane & 7) == 0) sums[b * 8 + (lane >> 3)] = total;
-        if (lane == 0) d[b] = s;
+        const Q8kLane ql = quantize_q8k_block(reinterpret_cast<const float4*>(x)[b * 64 + lane]);
+        reinterpret_cast<int*>(q)[b * 64 + lane] = ql.packed;
+        if ((lane & 7) == 0) sums[b * 8 + (lane >> 3)] = ql.total;
+        if (lane == 0) d[b] = ql.d;
     }
 }
 
@@ -555,9 +566,15 @@ __global__ __launch_bounds__(64) void linear_q4k_q8k_kernel(float* __restrict__ 
 // separately before they meet in the final sum (the engine rounds the product of the whole
 // sub-block dot): a difference in the last bit of a term.  Halves and wavefronts meet in LDS
 // in a fixed order.
+// kFusedRows > 0 (exactly that many rows, one row group): no separate quantizer launch -- wavefront w
+// quantizes super-block w of every row from `x` straight into LDS (the same arithmetic, so the same bits),
+// which is all it reads itself.  Its loads of X go out before the weight loads (loads retire in order),
+// and it quantizes while the weights are on their way.
 constexpr int kQ8kPassRows = 8;
+template <int kFusedRows>
 __global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __restrict__ dst, const int8_t* __restrict__ q,
                                                                   const float* __restrict__ xd, const int* __restrict__ sums,
+                                                                  const float* __restrict__ x,
                                                                   const uint8_t* __restrict__ weight, int rows, int in_dim,
                                                                   int out_dim, int rows_per_group, Epilogue ep) {
     extern __shared__ __align__(16) unsigned char q8k_lds[];
@@ -570,11 +587,27 @@ __global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __rest
     float* fs_s = xd_s + kQ8kPassRows * kb;                                                        // [8][kb][8]
     float* red = fs_s + kQ8kPassRows * kb * 8;                                                     // [kb][2][8][32]
 
+    constexpr bool kFused = kFusedRows > 0;
+    float4 xv[kFused ? kFusedRows : 1];
+    if (kFused) {
+#pragma unroll
+        for (int r = 0; r < kFusedRows; ++r)
+            xv[r] = reinterpret_cast<const float4*>(x + static_cast<size_t>(r) * in_dim + wave * kQ4kBlockValues)[lane];
+    }
     const uint8_t* tbase = weight + (static_cast<size_t>(tile) * kb + wave) * (32 * kQ4kBlockBytes);
     const q4k_u32x4 header = *reinterpret_cast<const q4k_u32x4*>(tbase + col * 16);
     q4k_u32x4 nib[4];
 #pragma unroll
     for (int c = 0; c < 4; ++c) nib[c] = *reinterpret_cast<const q4k_u32x4*>(tbase + 512 + c * 1024 + (col + 32 * g) * 16);
+    if (kFused) {
+#pragma unroll
+        for (int r = 0; r < kFusedRows; ++r) {
+            const Q8kLane ql = quantize_q8k_block(xv[r]);
+            reinterpret_cast<int*>(xq_s + r * in_dim + wave * kQ4kBlockValues)[lane] = ql.packed;
+            if ((lane & 7) == 0) fs_s[(r * kb + wave) * 8 + (lane >> 3)] = static_cast<float>(ql.total);
+            if (lane == 0) xd_s[r * kb + wave] = ql.d;
+        }
+    }
     float dsc[8], dmn[8];
     {
         const float d = half_bits_to_f32(static_cast<uint16_t>(header.x & 0xFFFFu));
@@ -603,8 +636,8 @@ __global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __rest
     const int row_end = min(rows, row_begin + rows_per_group);
     for (int r0 = row_begin; r0 < row_end; r0 += kQ8kPassRows) {
         const int nr = min(kQ8kPassRows, row_end - r0);
-        __syncthreads();  // the previous pass has been read
-        {
+        if (!kFused) {
+            __syncthreads();  // the previous pass has been read
             const uint4* src = reinterpret_cast<const uint4*>(q + static_cast<size_t>(r0) * in_dim);
             uint4* dst4 = reinterpret_cast<uint4*>(xq_s);
             for (int u = tid; u < nr * (in_dim >> 4); u += threads) dst4[u] = src[u];
@@ -685,12 +718,35 @@ hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* wor
         groups = (rows + rows_per_group - 1) / rows_per_group;
         const size_t lds = static_cast<size_t>(kQ8kPassRows) * in_dim + kQ8kPassRows * kb * 4 + kQ8kPassRows * kb * 32 +
                            static_cast<size_t>(kb) * 2 * kQ8kPassRows * 32 * 4;
-        hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel, dim3(tiles, groups), dim3(64 * kb), lds, stream, dst, q, d, sums, weight, rows,
-                           in_dim, out_dim, rows_per_group, ep);
+        hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel<0>, dim3(tiles, groups), dim3(64 * kb), lds, stream, dst, q, d, sums,
+                           static_cast<const float*>(nullptr), weight, rows, in_dim, out_dim, rows_per_group, ep);
     } else if (tiled)
         hipLaunchKernelGGL(linear_q4k_q8k_kernel<true>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
     else
         hipLaunchKernelGGL(linear_q4k_q8k_kernel<false>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
+    return hipGetLastError();
+}
+
+bool linear_q4k_q8k_fuses_quantizer(bool tiled, size_t rows, size_t in_dim) {
+    return tiled && (rows == 1 || rows == 2 || rows == 4) && in_dim / kQ4kBlockValues <= 12;  // the gate's decode row counts
+}
+
+hipError_t launch_linear_q4k_q8k_fused(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                                       int out_dim, const Epilogue& ep) {
+    if (rows == 0 || out_dim == 0) return hipSuccess;
+    if (!linear_q4k_q8k_fuses_quantizer(true, static_cast<size_t>(rows), static_cast<size_t>(in_dim))) return hipErrorInvalidValue;
+    const int kb = in_dim / kQ4kBlockValues;
+    const int tiles = (out_dim + 31) / 32;
+    const size_t lds = static_cast<size_t>(kQ8kPassRows) * in_dim + kQ8kPassRows * kb * 4 + kQ8kPassRows * kb * 32 +
+                       static_cast<size_t>(kb) * 2 * kQ8kPassRows * 32 * 4;
+#define AFHIP_Q8K_FUSED(R)                                                                                                   \
+    hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel<R>, dim3(tiles, 1), dim3(64 * kb), lds, stream, dst,                       \
+                       static_cast<const int8_t*>(nullptr), static_cast<const float*>(nullptr), static_cast<const int*>(nullptr), x, \
+                       weight, rows, in_dim, out_dim, kQ8kPassRows, ep)
+    if (rows == 1) AFHIP_Q8K_FUSED(1);
+    else if (rows == 2) AFHIP_Q8K_FUSED(2);
+    else AFHIP_Q8K_FUSED(4);
+#undef AFHIP_Q8K_FUSED
     return hipGetLastError();
 }
 

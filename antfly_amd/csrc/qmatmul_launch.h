@@ -148,6 +148,11 @@ size_t q4k_q8k_workspace_bytes(size_t rows, size_t in_dim);
 hipError_t launch_quantize_q8k(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace);
 hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, bool tiled, int rows,
                                  int in_dim, int out_dim, const Epilogue& ep);
+// One, two or four rows on the tile-major layout at K <= 3072: the quantizer runs inside the matmul launch
+// (same bits as the two launches; `workspace` is not touched).
+bool linear_q4k_q8k_fuses_quantizer(bool tiled, size_t rows, size_t in_dim);
+hipError_t launch_linear_q4k_q8k_fused(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
+                                       int out_dim, const Epilogue& ep);
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                            int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,

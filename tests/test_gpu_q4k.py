@@ -213,6 +213,22 @@ def test_q8k_activation_route_on_the_gated_shapes(layout, rows, in_dim, out_dim)
                                 G.buf(G.to_dev(x)), G.buf(wd), rows, in_dim, out_dim, kernels.NO_BUFFER)
 
 
+@pytest.mark.parametrize("in_dim,out_dim", [(512, 520), (2048, 8192), (3072, 1000)])
+def test_q8k_route_decode_rows_equal_the_rows_of_a_larger_call(in_dim, out_dim):
+    """With one, two or four rows the quantizer runs inside the matmul launch; nine rows take the separate quantizer.  A row's
+    result does not depend on which: rows 0 .. r-1 of the nine-row product are the r-row product, bit for bit."""
+    print(f"case: q4_k q8k fused quantizer in={in_dim} out={out_dim}", flush=True)
+    w = synth.weights(Q4K, 79, out_dim, in_dim)
+    x = synth.activations(80, 9, in_dim)
+    x[1, :256] = 0.0  # a zero block: scale 1
+    wd = device_weight(PREP, w, out_dim, in_dim)
+    y9 = G.linear(Q4K, PREP, x, wd, 9, in_dim, out_dim)
+    for rows in (1, 2, 4):
+        assert O.uses_q4k_q8k_activation(rows, in_dim, out_dim)
+        y = G.linear(Q4K, PREP, x[:rows].copy(), wd, rows, in_dim, out_dim)
+        assert np.array_equal(y.view(np.uint32), y9[:rows].view(np.uint32)), rows
+
+
 def test_q8k_gate_neighbours_stay_on_the_f32_route():
     for rows, in_dim, out_dim in [(3, 2048, 512), (1, 1024, 512), (1, 2048, 511), (5, 3072, 640), (16, 512, 512)]:
         assert not O.uses_q4k_q8k_activation(rows, in_dim, out_dim)
