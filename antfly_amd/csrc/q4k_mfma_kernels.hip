@@ -162,7 +162,11 @@ extern __shared__ __align__(16) unsigned char q4k_mfma_lds[];
 
 // kGroups = ceil(rows / 2) row groups (D registers 0 .. 4 kGroups - 1 are read);
 // kFlight super-blocks of weights are requested before any of them is used.
-template <int kGroups, int kFlight, int kMaxThreads = 512>
+// kOwnSlice (one tile per workgroup: the wavefronts partition K): a wavefront splits the slice of X
+// that it alone multiplies, four values per lane, and goes on without waiting for the others --
+// no workgroup barrier between the split and the matrix work, so wavefronts whose weights have
+// arrived start at once and the vector work spreads over the time the stream takes.
+template <int kGroups, int kFlight, int kMaxThreads = 512, bool kOwnSlice = false>
 __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                             const uint8_t* __restrict__ weight, int rows, int in_dim,
                                                             int out_dim, int slices, int sb_per_slice, Epilogue ep) {
@@ -199,6 +203,41 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
         }
     };
 
+    if (kOwnSlice) {
+        // ---- 1. this wavefront's slice of X: item i = (row i / n_sb, super-block sb_begin + i % n_sb)
+        const int n_sb = max(sb_end - sb_begin, 0), n_items = rows * n_sb;
+        auto item_ptr = [&](int i) {
+            const int r = i / n_sb, sb = sb_begin + (i - r * n_sb);
+            return reinterpret_cast<const float4*>(x + static_cast<size_t>(r) * in_dim + sb * kQ4kBlockValues) + lane;
+        };
+        auto split_item = [&](int i, const float4 v) {
+            const int r = i / n_sb, sb = sb_begin + (i - r * n_sb);
+            uint32_t p[3][2];
+            split3_pair(v.x, v.y, &p[0][0], &p[1][0], &p[2][0]);
+            split3_pair(v.z, v.w, &p[0][1], &p[1][1], &p[2][1]);
+#pragma unroll
+            for (int part = 0; part < 3; ++part)
+                *reinterpret_cast<uint2*>(xparts + static_cast<size_t>(r * 3 + part) * row_stride + (sb * kQ4kBlockValues + 4 * lane) * 2) =
+                    make_uint2(p[part][0], p[part][1]);
+            const float s = sum_over_8((v.x + v.y) + (v.z + v.w));
+            if ((lane & 7) == 0) xsum[r * (kb * 8) + sb * 8 + (lane >> 3)] = s;
+        };
+        constexpr int kAhead = 2;  // items requested before the weights (one row, or two rows, of a one-super-block slice)
+        float4 first[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) first[i] = i < n_items ? *item_ptr(i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        __builtin_amdgcn_sched_barrier(0);
+        request(sb_begin);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i)
+            if (i < n_items) split_item(i, first[i]);
+        for (int i = kAhead; i < n_items; ++i) split_item(i, *item_ptr(i));
+        // the wavefront reads back what its own lanes wrote: LDS operations of a wavefront complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
     // ---- 1. X: requested first, split into bf16 parts while the weights are on their way
     const int groups_per_row = in_dim >> 3;
     const int n_groups = rows * groups_per_row;
@@ -236,6 +275,7 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
         }
     }
     __syncthreads();
+    }
 
     // ---- 2. this lane's roles
     const int c = lane & 31, g = lane >> 5;
@@ -620,26 +660,38 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     // resident), four at a time of a long one
     const int flight = sb_per_slice <= 1 ? 0 : (sb_per_slice <= 2 ? 1 : 2);
     const int variant = (waves > 8 ? 3 : 0) + flight;
+    static const int env_shared = tuning_int("AFHIP_Q4K_SHARED_SPLIT");
+    const bool own_slice = kGroups == 1 && tiles_per_wg == 1 && env_shared == 0;
     void (*kernel)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
     switch (variant) {
         case 0:
-        case 1: kernel = gemv_q4k_mfma_kernel<kGroups, 2>; break;
-        case 2: kernel = gemv_q4k_mfma_kernel<kGroups, 4>; break;
+        case 1:
+            if constexpr (kGroups == 1) kernel = own_slice ? gemv_q4k_mfma_kernel<1, 2, 512, true> : gemv_q4k_mfma_kernel<1, 2>;
+            else kernel = gemv_q4k_mfma_kernel<kGroups, 2>;
+            break;
+        case 2:
+            if constexpr (kGroups == 1) kernel = own_slice ? gemv_q4k_mfma_kernel<1, 4, 512, true> : gemv_q4k_mfma_kernel<1, 4>;
+            else kernel = gemv_q4k_mfma_kernel<kGroups, 4>;
+            break;
         default:
             if constexpr (kGroups == 1) {  // sixteen wavefronts: at most 128 registers each
-                kernel = variant == 3 ? gemv_q4k_mfma_kernel<1, 1, 1024>
-                                      : (variant == 4 ? gemv_q4k_mfma_kernel<1, 2, 1024> : gemv_q4k_mfma_kernel<1, 4, 1024>);
+                if (own_slice)
+                    kernel = variant == 3 ? gemv_q4k_mfma_kernel<1, 1, 1024, true>
+                                          : (variant == 4 ? gemv_q4k_mfma_kernel<1, 2, 1024, true> : gemv_q4k_mfma_kernel<1, 4, 1024, true>);
+                else
+                    kernel = variant == 3 ? gemv_q4k_mfma_kernel<1, 1, 1024>
+                                          : (variant == 4 ? gemv_q4k_mfma_kernel<1, 2, 1024> : gemv_q4k_mfma_kernel<1, 4, 1024>);
             }
             break;
     }
     if (kernel == nullptr) return hipErrorInvalidValue;
-    static std::atomic<bool> large_lds[6] = {};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
-    if (lds > 64 * 1024 && !large_lds[variant]) {
+    static std::atomic<bool> large_lds[12] = {};  // raising the limit is sticky per kernel: once, outside any stream capture opened later
+    if (lds > 64 * 1024 && !large_lds[variant + (own_slice ? 6 : 0)]) {
         if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                160 * 1024);
             e != hipSuccess)
             return e;
-        large_lds[variant] = true;
+        large_lds[variant + (own_slice ? 6 : 0)] = true;
     }
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(waves * 64), lds, stream, dst, x, weight, rows, in_dim, out_dim, slices,
                        sb_per_slice, ep);
