@@ -372,6 +372,203 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
     }
 }
 
+
+// ------------------------------------------------------------------ one or two rows on the int8 matrix core
+// The masked nibble bytes 0x0n are int8 numbers as they stand, so with integer activations a
+// sub-block costs no conversion at all and one v_mfma_i32_32x32x32_i8.  X keeps f32 accuracy as
+// fixed point: per super-block of 256 values a power of two 2^s with |x| * 2^s < 2^27, q =
+// trunc(x * 2^s) (28 bits with sign) cut into four base-128 digits q = d3 * 2^21 + d2 * 2^14 +
+// d1 * 2^7 + d0 (d0..d2 in 0..127, d3 signed) -- four int8 planes that take MFMA rows
+// 4 * row + digit.  The digit dots of a sub-block are exact int32; the eight sub-blocks of a
+// super-block are added as integers, each times its 6-bit scale (at most 63 * 32 * 127 * 15 * 8 <
+// 2^25), and only the super-block's four sums become floats:
+//   y += d * (2^-s * (((D3 * 128 + D2) * 128 + D1) * 128 + D0))  -  dmin * sum_sub m_sub * X_sub.
+// Against the three-part bf16 kernel: no conversions (64 per super-block and wavefront), half the
+// MFMAs, integer multiply-adds instead of float sums per sub-block; the truncation error is
+// 2^-27 of the super-block's largest |x| per value (the bf16 parts: 2^-25 of each value).
+// A super-block that holds an infinity or a NaN gives NaN in every column.
+// Every wavefront prepares the K slice it alone multiplies (no workgroup barrier before the matrix
+// work); one tile per workgroup, its wavefronts partition K.
+typedef int t_i32x4 __attribute__((ext_vector_type(4)));
+typedef int t_i32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int kDigitPadBytes = 48;  // LDS stride of a digit plane: K + 48 spreads the planes over the banks
+
+template <int kFlight, int kMaxThreads>
+__global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst, const float* __restrict__ x,
+                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
+                                                                  int out_dim, int slices, int sb_per_slice, Epilogue ep) {
+    const int kb = in_dim >> 8;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int threads = static_cast<int>(blockDim.x);
+    const int plane_stride = in_dim + kDigitPadBytes;
+    unsigned char* xdig = q4k_mfma_lds;  // [rows * 4][plane_stride]: the digit planes of every row
+    float* xscale = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows) * 4 * plane_stride);  // [rows][kb]: -s
+    float* xsum = xscale + ((rows * kb + 3) & ~3);                                                          // [rows][kb * 8], 16-byte aligned
+    float* partial = xsum + rows * kb * 8;                                                                  // [waves][64]
+
+    const int n_tiles = (out_dim + kTileCols - 1) >> 5;
+    const int tile = blockIdx.x < static_cast<unsigned>(n_tiles) ? blockIdx.x : n_tiles - 1;
+    const int slice = wave;  // one tile per workgroup: blockDim.x = 64 * slices
+    const int sb_begin = slice * sb_per_slice;
+    const int sb_end = min(kb, sb_begin + sb_per_slice);
+    const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
+
+    t_u32x4 hdr[kFlight], qv[kFlight][4];
+    auto request = [&](int sb_first) {
+#pragma unroll
+        for (int f = 0; f < kFlight; ++f) {
+            const int sb = sb_first + f;
+            if (sb >= sb_end) continue;  // wave-uniform; the same test guards the use below
+            const uint8_t* base = tile_base + static_cast<size_t>(sb) * kTileBytes;
+            hdr[f] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 16 * (lane & 31)));
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                qv[f][t] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 512 + t * 1024 + 16 * lane));
+        }
+    };
+
+    // ---- 1. this wavefront's slice of X: item i = (row i / n_sb, super-block sb_begin + i % n_sb), four values a lane
+    {
+        const int n_sb = max(sb_end - sb_begin, 0), n_items = rows * n_sb;
+        auto item_ptr = [&](int i) {
+            const int r = i / n_sb, sb = sb_begin + (i - r * n_sb);
+            return reinterpret_cast<const float4*>(x + static_cast<size_t>(r) * in_dim + sb * kQ4kBlockValues) + lane;
+        };
+        auto digits_of_item = [&](int i, const float4 v) {
+            const int r = i / n_sb, sb = sb_begin + (i - r * n_sb);
+            float m = fmaxf(fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)), fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+            m = max_over_8(m);
+            m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
+            const int mb = __builtin_bit_cast(int, m);
+            m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 0)),
+                            __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 16))),
+                      fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 32)),
+                            __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 48))));
+            // |x| < 2^(e - 126) (subnormals: e = 1): times 2^(153 - e) it stays below 2^27.  The exponent goes by
+            // v_ldexp_f32 both ways (2^(153 - e) itself is past the f32 range for small e).
+            const int e_raw = (__builtin_bit_cast(int, m) >> 23) & 0xFF;
+            const int e = e_raw < 1 ? 1 : e_raw;
+            const float down = e_raw == 255 ? __builtin_nanf("") : static_cast<float>(e - 153);  // -s, as a number
+            const int q[4] = {static_cast<int>(__builtin_ldexpf(v.x, 153 - e)), static_cast<int>(__builtin_ldexpf(v.y, 153 - e)),
+                              static_cast<int>(__builtin_ldexpf(v.z, 153 - e)), static_cast<int>(__builtin_ldexpf(v.w, 153 - e))};
+            uint32_t plane[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const uint32_t u = static_cast<uint32_t>(q[k]);
+                plane[0] |= (u & 127u) << (8 * k);
+                plane[1] |= ((u >> 7) & 127u) << (8 * k);
+                plane[2] |= ((u >> 14) & 127u) << (8 * k);
+                plane[3] |= ((u >> 21) & 255u) << (8 * k);  // bits 21 .. 28: the signed top digit as a byte
+            }
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+                *reinterpret_cast<uint32_t*>(xdig + static_cast<size_t>(r * 4 + d) * plane_stride + sb * kQ4kBlockValues + 4 * lane) = plane[d];
+            const float s = sum_over_8((v.x + v.y) + (v.z + v.w));
+            if ((lane & 7) == 0) xsum[r * (kb * 8) + sb * 8 + (lane >> 3)] = s;
+            if (lane == 0) xscale[r * kb + sb] = down;
+        };
+        constexpr int kAhead = 2;  // items requested before the weights (one row, or two rows, of a one-super-block slice)
+        float4 first[kAhead];
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) first[i] = i < n_items ? *item_ptr(i) : make_float4(0.f, 0.f, 0.f, 0.f);
+        __builtin_amdgcn_sched_barrier(0);
+        request(sb_begin);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i)
+            if (i < n_items) digits_of_item(i, first[i]);
+        for (int i = kAhead; i < n_items; ++i) digits_of_item(i, *item_ptr(i));
+        // the wavefront reads back what its own lanes wrote: LDS operations of a wavefront complete in order
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+
+    // ---- 2. this lane's roles.  A operand: MFMA row c = digit (c & 3) of row (c >> 2); rows past the
+    // last read row 0's first plane (their D rows are never looked at).  Lane half g supplies K = 16 g .. 16 g + 15.
+    const int c = lane & 31, g = lane >> 5;
+    const bool a_live = (c >> 2) < rows;
+    const unsigned char* a_base = xdig + static_cast<size_t>(a_live ? c : 0) * plane_stride + 16 * g;
+    // results: D registers 0 .. 3 (digits) of lane half g belong to row g, output column c of the tile
+    const int my_row = min(g, rows - 1);
+    const float* xsum_row = xsum + my_row * (kb * 8);
+    const float* xscale_row = xscale + my_row * kb;
+    float acc = 0.0f;
+
+    for (int sb_first = sb_begin; sb_first < sb_end; sb_first += kFlight) {
+        if (sb_first != sb_begin) request(sb_first);
+#pragma unroll
+        for (int f = 0; f < kFlight; ++f) {
+            const int sb = sb_first + f;
+            if (sb >= sb_end) continue;  // wave-uniform: nothing was requested for it
+            const t_u32x4 h = hdr[f];
+            const float d = half_bits_to_f32(static_cast<uint16_t>(h.x & 0xFFFFu));
+            const float dmin = half_bits_to_f32(static_cast<uint16_t>(h.x >> 16));
+            // the eight 6-bit scales and mins as bytes of four words (unpackQ4KScaleMinsU8,
+            // ops/native_compute.zig:33745-33754)
+            const uint32_t sc_lo = h.y & 0x3F3F3F3Fu, mn_lo = h.z & 0x3F3F3F3Fu;
+            const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
+            const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
+            const unsigned char* a_sb = a_base + sb * kQ4kBlockValues;
+            const float4 xs_lo = *reinterpret_cast<const float4*>(xsum_row + sb * 8);
+            const float4 xs_hi = *reinterpret_cast<const float4*>(xsum_row + sb * 8 + 4);
+            const float xs[8] = {xs_lo.x, xs_lo.y, xs_lo.z, xs_lo.w, xs_hi.x, xs_hi.y, xs_hi.z, xs_hi.w};
+            int digit_sum[4] = {0, 0, 0, 0};
+            float min_sum = 0.0f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int hi = 0; hi < 2; ++hi) {  // low nibbles: sub-block 2 t, high nibbles: 2 t + 1
+                    const int sub = 2 * t + hi;
+                    const uint32_t w[4] = {qv[f][t].x, qv[f][t].y, qv[f][t].z, qv[f][t].w};
+                    t_i32x4 b;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) b[k] = static_cast<int>((hi ? w[k] >> 4 : w[k]) & 0x0F0F0F0Fu);
+                    const t_i32x4 a = *reinterpret_cast<const t_i32x4*>(a_sb + 32 * sub);
+                    const t_i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+                    const t_i32x16 D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
+                    const int sc = static_cast<int>(((sub < 4 ? sc_lo : sc_hi) >> (8 * (sub & 3))) & 0xFFu);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) digit_sum[k] += __mul24(D[k], sc);
+                    min_sum = __builtin_fmaf(ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3), xs[sub], min_sum);
+                }
+            }
+            float S = static_cast<float>(digit_sum[3]);
+            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[2]));
+            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[1]));
+            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[0]));
+            // times 2^-s (xscale holds -s as a number, NaN for a super-block with an infinity or a NaN in it)
+            const float minus_s = xscale_row[sb];
+            S = __builtin_fmaf(minus_s, 0.0f, __builtin_ldexpf(S, static_cast<int>(minus_s)));
+            acc = __builtin_fmaf(d, S, acc);
+            acc = __builtin_fmaf(-dmin, min_sum, acc);
+        }
+    }
+
+    // ---- 3. K-slices meet in LDS, in slice order
+    partial[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (tid < 64) {
+        float total = 0.0f;
+        for (int sl = 0; sl < slices; ++sl) total += partial[sl * 64 + tid];
+        const int row = tid >> 5;
+        const int o = static_cast<int>(blockIdx.x) * kTileCols + (tid & 31);
+        if (row < rows && o < out_dim) {
+            const size_t idx = static_cast<size_t>(row) * out_dim + o;
+            dst[idx] = finish_output(ep, o, idx, total);
+        }
+    }
+    (void)threads;
+}
+
+size_t q4k_i8_lds_bytes(int rows, int in_dim, int waves) {
+    return static_cast<size_t>(rows) * 4 * (static_cast<size_t>(in_dim) + kDigitPadBytes) +
+           ((static_cast<size_t>(rows) * (in_dim / 256) + 3) & ~static_cast<size_t>(3)) * 4 + static_cast<size_t>(rows) * (in_dim / 32) * 4 +
+           static_cast<size_t>(waves) * 64 * 4;
+}
+
 // Tuning runs only (the CPU engine exposes TERMITE_QUANT_* knobs the same way,
 // ops/native_compute.zig:2902-2945).
 int tuning_int(const char* name) {
@@ -644,15 +841,20 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     // threads share the splitting of X.  (Measured on 14336 x 4096, 4096 x 14336, 4096 x 4096
     // and 128256 x 4096.)
     const int max_waves = kGroups == 1 ? 16 : 8;
+    static const int env_shared = tuning_int("AFHIP_Q4K_SHARED_SPLIT"), env_bf16 = tuning_int("AFHIP_Q4K_BF16_DECODE");
+    // one or two rows: fixed-point activations on the int8 matrix core (the bf16 kernel when a tuning run asks
+    // for it and its three copies of X fit)
+    const bool use_i8 = kGroups == 1 && !((env_bf16 != 0 || env_shared != 0) && q4k_mfma_lds_bytes(rows, in_dim, 16, 1) <= kLdsBudget);
     int slices = kGroups == 1 ? 16 : 4;
-    // long rows (three or more super-blocks a slice) and vocabulary-sized matrices did better with eight
-    if (slices == 16 && (kb > 32 || n_tiles > 2048)) slices = 8;
+    // bf16 kernel: long rows (three or more super-blocks a slice) and vocabulary-sized matrices did better with
+    // eight; the int8 kernel with sixteen everywhere (K = 14336: 12.5 against 13.8 us, K = 11008: 10.3 against 12.0)
+    if (!use_i8 && slices == 16 && (kb > 32 || n_tiles > 2048)) slices = 8;
     while (slices > kb) slices /= 2;
     static const int env_slices = tuning_int("AFHIP_Q4K_SLICES"), env_tiles = tuning_int("AFHIP_Q4K_TILES_PER_WG");
     if (env_slices >= 1 && env_slices <= max_waves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
     const int sb_per_slice = (kb + slices - 1) / slices;
-    int tiles_per_wg = (slices > 8 ? 16 : 8) / slices;
-    if (env_tiles >= 1 && env_tiles * slices <= max_waves) tiles_per_wg = env_tiles;
+    int tiles_per_wg = use_i8 ? 1 : (slices > 8 ? 16 : 8) / slices;  // (the int8 kernel: its wavefronts partition K, nothing else)
+    if (!use_i8 && env_tiles >= 1 && env_tiles * slices <= max_waves) tiles_per_wg = env_tiles;
     const int waves = slices * tiles_per_wg;
     const int grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
     const size_t lds = q4k_mfma_lds_bytes(rows, in_dim, waves, kGroups);
@@ -660,8 +862,31 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     // resident), four at a time of a long one
     const int flight = sb_per_slice <= 1 ? 0 : (sb_per_slice <= 2 ? 1 : 2);
     const int variant = (waves > 8 ? 3 : 0) + flight;
-    static const int env_shared = tuning_int("AFHIP_Q4K_SHARED_SPLIT");
     const bool own_slice = kGroups == 1 && tiles_per_wg == 1 && env_shared == 0;
+    if constexpr (kGroups == 1) {
+        if (use_i8) {
+            if (tiles_per_wg != 1) return hipErrorInvalidValue;  // (a tuning knob asked for a shape this kernel does not have)
+            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
+            switch (variant) {
+                case 0:
+                case 1: k8 = gemv_q4k_i8_kernel<2, 512>; break;
+                case 2: k8 = gemv_q4k_i8_kernel<2, 512>; break;  // (four in flight do not fit 128 registers here)
+                case 3: k8 = gemv_q4k_i8_kernel<1, 1024>; break;
+                case 4: k8 = gemv_q4k_i8_kernel<2, 1024>; break;
+                default: k8 = gemv_q4k_i8_kernel<2, 1024>; break;  // (a longer slice: two super-blocks at a time)
+            }
+            const size_t lds8 = q4k_i8_lds_bytes(rows, in_dim, waves);
+            static std::atomic<bool> large_lds8[6] = {};
+            if (lds8 > 64 * 1024 && !large_lds8[variant]) {
+                if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(k8), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+                    e != hipSuccess)
+                    return e;
+                large_lds8[variant] = true;
+            }
+            hipLaunchKernelGGL(k8, dim3(grid), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices, sb_per_slice, ep);
+            return hipGetLastError();
+        }
+    }
     void (*kernel)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
     switch (variant) {
         case 0:
@@ -728,6 +953,8 @@ hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, cons
 int gemv_q4k_tiled_rows_per_launch(int in_dim) {
     int per_launch = kMaxRowsPerLaunch;
     while (per_launch > 1 && q4k_mfma_lds_bytes(per_launch, in_dim, 8, (per_launch + 1) / 2) > kLdsBudget) --per_launch;
+    // two rows on the int8 kernel: four one-byte digit planes a row instead of three bf16 copies
+    if (per_launch < 2 && q4k_i8_lds_bytes(2, in_dim, 16) <= kLdsBudget) per_launch = 2;
     return per_launch;
 }
 
@@ -811,7 +1038,8 @@ hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x,
     if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
     // as many rows per launch as LDS holds (three bf16 copies of each), at most eight
     const int per_launch = gemv_q4k_tiled_rows_per_launch(in_dim);
-    if (q4k_mfma_lds_bytes(per_launch, in_dim, 8, 1) > kLdsBudget) return hipErrorInvalidValue;
+    if (per_launch > 2 && q4k_mfma_lds_bytes(per_launch, in_dim, 8, 1) > kLdsBudget) return hipErrorInvalidValue;
+    if (per_launch <= 2 && q4k_i8_lds_bytes(per_launch, in_dim, 16) > kLdsBudget) return hipErrorInvalidValue;
     for (int r0 = 0; r0 < rows; r0 += per_launch) {
         const int nr = rows - r0 < per_launch ? rows - r0 : per_launch;
         float* d = dst + static_cast<size_t>(r0) * out_dim;

@@ -186,6 +186,36 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
     assert err32 <= TOL and err32 <= TIGHT, err32
 
 
+def test_decode_rows_on_extreme_activations():
+    """One and two rows run on fixed-point activations (a power-of-two scale per super-block of 256 values): zero
+    super-blocks, outliers 10^6 times their neighbours, magnitudes near the ends of the f32 range; a row that
+    holds an infinity comes out non-finite and leaves the other row alone."""
+    in_dim, out_dim = 2048, 96
+    w = synth.weights(Q4K, 91, out_dim, in_dim)
+    wd = device_weight(PREP, w, out_dim, in_dim)
+    rng = np.random.default_rng(92)
+    base = synth.activations(93, 2, in_dim)
+    cases = {
+        "zero super-blocks": base * np.repeat(np.array([0, 1, 1, 0, 1, 0, 1, 1], np.float32), 256)[None, :],
+        "outliers": base * np.where(rng.random((2, in_dim)) < 0.004, 1.0e6, 1.0).astype(np.float32),
+        "huge": base * np.float32(1.0e30),
+        "tiny": base * np.float32(1.0e-32),
+        "mixed scales per super-block": base * np.repeat(np.exp2(rng.integers(-40, 40, 8)).astype(np.float32), 256)[None, :],
+    }
+    for name, x in cases.items():
+        print(f"case: q4_k decode extremes: {name}", flush=True)
+        for rows in (1, 2):
+            y = G.linear(Q4K, PREP, x[:rows].copy(), wd, rows, in_dim, out_dim)
+            ref = O.linear_q4_k(x[:rows].copy(), w, rows, in_dim, out_dim, f64=True)
+            err = G.max_rel_err(y, ref)
+            assert err <= TIGHT, (name, rows, err)
+    x = base.copy()
+    x[0, 700] = np.inf
+    y = G.linear(Q4K, PREP, x, wd, 2, in_dim, out_dim)
+    assert not np.isfinite(y[0]).any()
+    assert np.array_equal(y[1], G.linear(Q4K, PREP, x[1:].copy(), wd, 1, in_dim, out_dim)[0])
+
+
 Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
 
 
