@@ -373,19 +373,21 @@ __global__ __launch_bounds__(kMaxThreads) void gemv_q4k_mfma_kernel(float* __res
 }
 
 
-// ------------------------------------------------------------------ one or two rows on the int8 matrix core
+// ------------------------------------------------------------------ one to four rows on the int8 matrix core
 // The masked nibble bytes 0x0n are int8 numbers as they stand, so with integer activations a
 // sub-block costs no conversion at all and one v_mfma_i32_32x32x32_i8.  X keeps f32 accuracy as
-// fixed point: per super-block of 256 values a power of two 2^s with |x| * 2^s < 2^27, q =
-// trunc(x * 2^s) (28 bits with sign) cut into four base-128 digits q = d3 * 2^21 + d2 * 2^14 +
-// d1 * 2^7 + d0 (d0..d2 in 0..127, d3 signed) -- four int8 planes that take MFMA rows
-// 4 * row + digit.  The digit dots of a sub-block are exact int32; the eight sub-blocks of a
-// super-block are added as integers, each times its 6-bit scale (at most 63 * 32 * 127 * 15 * 8 <
-// 2^25), and only the super-block's four sums become floats:
-//   y += d * (2^-s * (((D3 * 128 + D2) * 128 + D1) * 128 + D0))  -  dmin * sum_sub m_sub * X_sub.
+// fixed point: per super-block of 256 values a power of two 2^s with |x| * 2^s < 2^30, q =
+// trunc(x * 2^s) (31 bits with sign) written with four signed base-256 digits q = d3 * 2^24 +
+// d2 * 2^16 + d1 * 2^8 + d0, every d in -128..127: they are the bytes of (q + 0x80808080) ^
+// 0x80808080 (adding 128 to every byte position with the carries, then taking 128 off every
+// byte) -- four int8 planes that take MFMA rows 4 * row + digit.  The digit dots of a sub-block
+// are exact int32; the eight sub-blocks of a super-block are added as integers, each times its
+// 6-bit scale (at most 63 * 32 * 128 * 15 * 8 < 2^25), and only the super-block's four sums
+// become floats:
+//   y += d * (2^-s * (((D3 * 256 + D2) * 256 + D1) * 256 + D0))  -  dmin * sum_sub m_sub * X_sub.
 // Against the three-part bf16 kernel: no conversions (64 per super-block and wavefront), half the
 // MFMAs, integer multiply-adds instead of float sums per sub-block; the truncation error is
-// 2^-27 of the super-block's largest |x| per value (the bf16 parts: 2^-25 of each value).
+// 2^-30 of the super-block's largest |x| per value (the bf16 parts: 2^-25 of each value).
 // A super-block that holds an infinity or a NaN gives NaN in every column.
 // Every wavefront prepares the K slice it alone multiplies (no workgroup barrier before the matrix
 // work); one tile per workgroup, its wavefronts partition K.
@@ -394,7 +396,8 @@ typedef int t_i32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kDigitPadBytes = 48;  // LDS stride of a digit plane: K + 48 spreads the planes over the banks
 
-template <int kFlight, int kMaxThreads>
+// kGroups = ceil(rows / 2) row groups: row r sits in lane half r % 2, D registers 4 (r / 2) + digit.
+template <int kGroups, int kFlight, int kMaxThreads>
 __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                                   const uint8_t* __restrict__ weight, int rows, int in_dim,
                                                                   int out_dim, int slices, int sb_per_slice, Epilogue ep) {
@@ -406,7 +409,7 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
     unsigned char* xdig = q4k_mfma_lds;  // [rows * 4][plane_stride]: the digit planes of every row
     float* xscale = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows) * 4 * plane_stride);  // [rows][kb]: -s
     float* xsum = xscale + ((rows * kb + 3) & ~3);                                                          // [rows][kb * 8], 16-byte aligned
-    float* partial = xsum + rows * kb * 8;                                                                  // [waves][64]
+    float* partial = xsum + rows * kb * 8;                                                                  // [waves][kGroups][64]
 
     const int n_tiles = (out_dim + kTileCols - 1) >> 5;
     const int tile = blockIdx.x < static_cast<unsigned>(n_tiles) ? blockIdx.x : n_tiles - 1;
@@ -446,22 +449,22 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
                             __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 16))),
                       fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 32)),
                             __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 48))));
-            // |x| < 2^(e - 126) (subnormals: e = 1): times 2^(153 - e) it stays below 2^27.  The exponent goes by
-            // v_ldexp_f32 both ways (2^(153 - e) itself is past the f32 range for small e).
+            // |x| < 2^(e - 126) (subnormals: e = 1): times 2^(156 - e) it stays below 2^30.  The exponent goes by
+            // v_ldexp_f32 both ways (2^(156 - e) itself is past the f32 range for small e).
             const int e_raw = (__builtin_bit_cast(int, m) >> 23) & 0xFF;
             const int e = e_raw < 1 ? 1 : e_raw;
-            const float down = e_raw == 255 ? __builtin_nanf("") : static_cast<float>(e - 153);  // -s, as a number
-            const int q[4] = {static_cast<int>(__builtin_ldexpf(v.x, 153 - e)), static_cast<int>(__builtin_ldexpf(v.y, 153 - e)),
-                              static_cast<int>(__builtin_ldexpf(v.z, 153 - e)), static_cast<int>(__builtin_ldexpf(v.w, 153 - e))};
-            uint32_t plane[4] = {0u, 0u, 0u, 0u};
+            const float down = e_raw == 255 ? __builtin_nanf("") : static_cast<float>(e - 156);  // -s, as a number
+            const float vv[4] = {v.x, v.y, v.z, v.w};
+            uint32_t t[4];  // the four signed digits of each value, lowest in byte 0
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const uint32_t u = static_cast<uint32_t>(q[k]);
-                plane[0] |= (u & 127u) << (8 * k);
-                plane[1] |= ((u >> 7) & 127u) << (8 * k);
-                plane[2] |= ((u >> 14) & 127u) << (8 * k);
-                plane[3] |= ((u >> 21) & 255u) << (8 * k);  // bits 21 .. 28: the signed top digit as a byte
-            }
+            for (int k = 0; k < 4; ++k)
+                t[k] = (static_cast<uint32_t>(static_cast<int>(__builtin_ldexpf(vv[k], 156 - e))) + 0x80808080u) ^ 0x80808080u;
+            // 4 x 4 byte transpose: plane[d] = digit d of the lane's four values (v_perm_b32: selectors 0..3 take
+            // bytes of the second operand, 4..7 of the first)
+            const uint32_t lo01 = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(t[1], t[0], 0x07030602u);
+            const uint32_t lo23 = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(t[3], t[2], 0x07030602u);
+            const uint32_t plane[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                                       __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
 #pragma unroll
             for (int d = 0; d < 4; ++d)
                 *reinterpret_cast<uint32_t*>(xdig + static_cast<size_t>(r * 4 + d) * plane_stride + sb * kQ4kBlockValues + 4 * lane) = plane[d];
@@ -491,11 +494,17 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
     const int c = lane & 31, g = lane >> 5;
     const bool a_live = (c >> 2) < rows;
     const unsigned char* a_base = xdig + static_cast<size_t>(a_live ? c : 0) * plane_stride + 16 * g;
-    // results: D registers 0 .. 3 (digits) of lane half g belong to row g, output column c of the tile
-    const int my_row = min(g, rows - 1);
-    const float* xsum_row = xsum + my_row * (kb * 8);
-    const float* xscale_row = xscale + my_row * kb;
-    float acc = 0.0f;
+    // results: D registers 4 G .. 4 G + 3 (digits) of lane half g belong to row 2 G + g, output column c of the tile
+    const float* xsum_row[kGroups];
+    const float* xscale_row[kGroups];
+    float acc[kGroups];
+#pragma unroll
+    for (int G = 0; G < kGroups; ++G) {
+        const int my_row = min(2 * G + g, rows - 1);
+        xsum_row[G] = xsum + my_row * (kb * 8);
+        xscale_row[G] = xscale + my_row * kb;
+        acc[G] = 0.0f;
+    }
 
     for (int sb_first = sb_begin; sb_first < sb_end; sb_first += kFlight) {
         if (sb_first != sb_begin) request(sb_first);
@@ -512,11 +521,18 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
             const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
             const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
             const unsigned char* a_sb = a_base + sb * kQ4kBlockValues;
-            const float4 xs_lo = *reinterpret_cast<const float4*>(xsum_row + sb * 8);
-            const float4 xs_hi = *reinterpret_cast<const float4*>(xsum_row + sb * 8 + 4);
-            const float xs[8] = {xs_lo.x, xs_lo.y, xs_lo.z, xs_lo.w, xs_hi.x, xs_hi.y, xs_hi.z, xs_hi.w};
-            int digit_sum[4] = {0, 0, 0, 0};
-            float min_sum = 0.0f;
+            float xs[kGroups][8];
+            int digit_sum[kGroups][4];
+            float min_sum[kGroups];
+#pragma unroll
+            for (int G = 0; G < kGroups; ++G) {
+                const float4 xs_lo = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8);
+                const float4 xs_hi = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8 + 4);
+                xs[G][0] = xs_lo.x, xs[G][1] = xs_lo.y, xs[G][2] = xs_lo.z, xs[G][3] = xs_lo.w;
+                xs[G][4] = xs_hi.x, xs[G][5] = xs_hi.y, xs[G][6] = xs_hi.z, xs[G][7] = xs_hi.w;
+                digit_sum[G][0] = digit_sum[G][1] = digit_sum[G][2] = digit_sum[G][3] = 0;
+                min_sum[G] = 0.0f;
+            }
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
 #pragma unroll
@@ -530,43 +546,51 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
                     const t_i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                     const t_i32x16 D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
                     const int sc = static_cast<int>(((sub < 4 ? sc_lo : sc_hi) >> (8 * (sub & 3))) & 0xFFu);
+                    const float mn = ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3);
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) digit_sum[k] += __mul24(D[k], sc);
-                    min_sum = __builtin_fmaf(ubyte_to_f32(sub < 4 ? mn_lo : mn_hi, sub & 3), xs[sub], min_sum);
+                    for (int G = 0; G < kGroups; ++G) {
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) digit_sum[G][k] += __mul24(D[4 * G + k], sc);
+                        min_sum[G] = __builtin_fmaf(mn, xs[G][sub], min_sum[G]);
+                    }
                 }
             }
-            float S = static_cast<float>(digit_sum[3]);
-            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[2]));
-            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[1]));
-            S = __builtin_fmaf(S, 128.0f, static_cast<float>(digit_sum[0]));
-            // times 2^-s (xscale holds -s as a number, NaN for a super-block with an infinity or a NaN in it)
-            const float minus_s = xscale_row[sb];
-            S = __builtin_fmaf(minus_s, 0.0f, __builtin_ldexpf(S, static_cast<int>(minus_s)));
-            acc = __builtin_fmaf(d, S, acc);
-            acc = __builtin_fmaf(-dmin, min_sum, acc);
+#pragma unroll
+            for (int G = 0; G < kGroups; ++G) {
+                float S = static_cast<float>(digit_sum[G][3]);
+                S = __builtin_fmaf(S, 256.0f, static_cast<float>(digit_sum[G][2]));
+                S = __builtin_fmaf(S, 256.0f, static_cast<float>(digit_sum[G][1]));
+                S = __builtin_fmaf(S, 256.0f, static_cast<float>(digit_sum[G][0]));
+                // times 2^-s (xscale holds -s as a number, NaN for a super-block with an infinity or a NaN in it)
+                const float minus_s = xscale_row[G][sb];
+                S = __builtin_fmaf(minus_s, 0.0f, __builtin_ldexpf(S, static_cast<int>(minus_s)));
+                acc[G] = __builtin_fmaf(d, S, acc[G]);
+                acc[G] = __builtin_fmaf(-dmin, min_sum[G], acc[G]);
+            }
         }
     }
 
     // ---- 3. K-slices meet in LDS, in slice order
-    partial[wave * 64 + lane] = acc;
+#pragma unroll
+    for (int G = 0; G < kGroups; ++G) partial[(wave * kGroups + G) * 64 + lane] = acc[G];
     __syncthreads();
-    if (tid < 64) {
+    for (int i = tid; i < kGroups * 64; i += threads) {
+        const int G = i >> 6, ln = i & 63;
         float total = 0.0f;
-        for (int sl = 0; sl < slices; ++sl) total += partial[sl * 64 + tid];
-        const int row = tid >> 5;
-        const int o = static_cast<int>(blockIdx.x) * kTileCols + (tid & 31);
+        for (int sl = 0; sl < slices; ++sl) total += partial[(sl * kGroups + G) * 64 + ln];
+        const int row = 2 * G + (ln >> 5);
+        const int o = static_cast<int>(blockIdx.x) * kTileCols + (ln & 31);
         if (row < rows && o < out_dim) {
             const size_t idx = static_cast<size_t>(row) * out_dim + o;
             dst[idx] = finish_output(ep, o, idx, total);
         }
     }
-    (void)threads;
 }
 
 size_t q4k_i8_lds_bytes(int rows, int in_dim, int waves) {
     return static_cast<size_t>(rows) * 4 * (static_cast<size_t>(in_dim) + kDigitPadBytes) +
            ((static_cast<size_t>(rows) * (in_dim / 256) + 3) & ~static_cast<size_t>(3)) * 4 + static_cast<size_t>(rows) * (in_dim / 32) * 4 +
-           static_cast<size_t>(waves) * 64 * 4;
+           static_cast<size_t>(waves) * ((rows + 1) / 2) * 64 * 4;
 }
 
 // Tuning runs only (the CPU engine exposes TERMITE_QUANT_* knobs the same way,
@@ -844,8 +868,14 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     static const int env_shared = tuning_int("AFHIP_Q4K_SHARED_SPLIT"), env_bf16 = tuning_int("AFHIP_Q4K_BF16_DECODE");
     // one or two rows: fixed-point activations on the int8 matrix core (the bf16 kernel when a tuning run asks
     // for it and its three copies of X fit)
-    const bool use_i8 = kGroups == 1 && !((env_bf16 != 0 || env_shared != 0) && q4k_mfma_lds_bytes(rows, in_dim, 16, 1) <= kLdsBudget);
-    int slices = kGroups == 1 ? 16 : 4;
+    // ... three or four rows too (eight slices, 512 threads) while their digit planes fit LDS and every workgroup has a
+    // compute unit to itself: each workgroup makes the digits of all rows itself, which two workgroups sharing a unit's
+    // vector ALUs cannot afford (N = 14336: 12.9 / 14.0 us against 12.6 / 13.0 on the bf16 kernel; 8192 x 8192: 15.2
+    // against 18.3; 4096 x 4096: 8.9 against 11.1)
+    const bool use_i8 = kGroups == 1 ? !((env_bf16 != 0 || env_shared != 0) && q4k_mfma_lds_bytes(rows, in_dim, 16, 1) <= kLdsBudget)
+                                     : (kGroups == 2 && env_bf16 == 0 && n_tiles <= gemv_compute_units() &&
+                                        q4k_i8_lds_bytes(rows, in_dim, 8) <= kLdsBudget);
+    int slices = kGroups == 1 ? 16 : (use_i8 ? 8 : 4);
     // bf16 kernel: long rows (three or more super-blocks a slice) and vocabulary-sized matrices did better with
     // eight; the int8 kernel with sixteen everywhere (K = 14336: 12.5 against 13.8 us, K = 11008: 10.3 against 12.0)
     if (!use_i8 && slices == 16 && (kb > 32 || n_tiles > 2048)) slices = 8;
@@ -863,17 +893,21 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     const int flight = sb_per_slice <= 1 ? 0 : (sb_per_slice <= 2 ? 1 : 2);
     const int variant = (waves > 8 ? 3 : 0) + flight;
     const bool own_slice = kGroups == 1 && tiles_per_wg == 1 && env_shared == 0;
-    if constexpr (kGroups == 1) {
+    if constexpr (kGroups <= 2) {
         if (use_i8) {
             if (tiles_per_wg != 1) return hipErrorInvalidValue;  // (a tuning knob asked for a shape this kernel does not have)
             void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
-            switch (variant) {
-                case 0:
-                case 1: k8 = gemv_q4k_i8_kernel<2, 512>; break;
-                case 2: k8 = gemv_q4k_i8_kernel<2, 512>; break;  // (four in flight do not fit 128 registers here)
-                case 3: k8 = gemv_q4k_i8_kernel<1, 1024>; break;
-                case 4: k8 = gemv_q4k_i8_kernel<2, 1024>; break;
-                default: k8 = gemv_q4k_i8_kernel<2, 1024>; break;  // (a longer slice: two super-blocks at a time)
+            if constexpr (kGroups == 1) {
+                switch (variant) {
+                    case 0:
+                    case 1: k8 = gemv_q4k_i8_kernel<1, 2, 512>; break;
+                    case 2: k8 = gemv_q4k_i8_kernel<1, 2, 512>; break;  // (four in flight do not fit 128 registers here)
+                    case 3: k8 = gemv_q4k_i8_kernel<1, 1, 1024>; break;
+                    case 4: k8 = gemv_q4k_i8_kernel<1, 2, 1024>; break;
+                    default: k8 = gemv_q4k_i8_kernel<1, 2, 1024>; break;  // (a longer slice: two super-blocks at a time)
+                }
+            } else {
+                k8 = gemv_q4k_i8_kernel<2, 2, 512>;
             }
             const size_t lds8 = q4k_i8_lds_bytes(rows, in_dim, waves);
             static std::atomic<bool> large_lds8[6] = {};

@@ -170,7 +170,7 @@ SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130),
 
 
 TILED_SHAPES = SHAPES + [(1, 1024, 300), (6, 4096, 70), (7, 1024, 257), (8, 2048, 96), (9, 1024, 64), (17, 512, 40),
-                        (2, 4096, 1000)]
+                        (2, 4096, 1000), (4, 4096, 96), (3, 8192, 200), (4, 1024, 8192), (3, 4096, 8200)]
 
 
 @pytest.mark.parametrize("layout,rows,in_dim,out_dim", [(RAW, *s) for s in SHAPES] + [(PREP, *s) for s in TILED_SHAPES])
@@ -187,33 +187,35 @@ def test_linear_matches_oracle(layout, rows, in_dim, out_dim):
 
 
 def test_decode_rows_on_extreme_activations():
-    """One and two rows run on fixed-point activations (a power-of-two scale per super-block of 256 values): zero
+    """Up to four rows run on fixed-point activations (a power-of-two scale per super-block of 256 values): zero
     super-blocks, outliers 10^6 times their neighbours, magnitudes near the ends of the f32 range; a row that
-    holds an infinity comes out non-finite and leaves the other row alone."""
+    holds an infinity comes out non-finite and leaves the other rows alone."""
     in_dim, out_dim = 2048, 96
     w = synth.weights(Q4K, 91, out_dim, in_dim)
     wd = device_weight(PREP, w, out_dim, in_dim)
     rng = np.random.default_rng(92)
-    base = synth.activations(93, 2, in_dim)
+    base = synth.activations(93, 4, in_dim)
     cases = {
         "zero super-blocks": base * np.repeat(np.array([0, 1, 1, 0, 1, 0, 1, 1], np.float32), 256)[None, :],
-        "outliers": base * np.where(rng.random((2, in_dim)) < 0.004, 1.0e6, 1.0).astype(np.float32),
+        "outliers": base * np.where(rng.random((4, in_dim)) < 0.004, 1.0e6, 1.0).astype(np.float32),
         "huge": base * np.float32(1.0e30),
         "tiny": base * np.float32(1.0e-32),
         "mixed scales per super-block": base * np.repeat(np.exp2(rng.integers(-40, 40, 8)).astype(np.float32), 256)[None, :],
     }
     for name, x in cases.items():
         print(f"case: q4_k decode extremes: {name}", flush=True)
-        for rows in (1, 2):
+        for rows in (1, 2, 3, 4):
             y = G.linear(Q4K, PREP, x[:rows].copy(), wd, rows, in_dim, out_dim)
             ref = O.linear_q4_k(x[:rows].copy(), w, rows, in_dim, out_dim, f64=True)
             err = G.max_rel_err(y, ref)
             assert err <= TIGHT, (name, rows, err)
     x = base.copy()
     x[0, 700] = np.inf
-    y = G.linear(Q4K, PREP, x, wd, 2, in_dim, out_dim)
-    assert not np.isfinite(y[0]).any()
-    assert np.array_equal(y[1], G.linear(Q4K, PREP, x[1:].copy(), wd, 1, in_dim, out_dim)[0])
+    for rows in (2, 4):
+        y = G.linear(Q4K, PREP, x[:rows].copy(), wd, rows, in_dim, out_dim)
+        assert not np.isfinite(y[0]).any()
+        assert np.isfinite(y[1:]).all()
+        assert G.max_rel_err(y[1:], O.linear_q4_k(x[1:rows].copy(), w, rows - 1, in_dim, out_dim, f64=True)) <= TIGHT
 
 
 Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
