@@ -199,6 +199,24 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
+    // three to eight rows with scratch: X as fixed-point digit planes once, then the int8 kernel on each matrix
+    static const int env_no_planes = env_int("AFHIP_Q4K_NO_DIGIT_PLANES");
+    if (tiled && env_no_planes == 0 && q4k_i8_rows_supports(rows, in_dim) && workspace.ptr != 0 && workspace.ptr % 16 == 0 &&
+        workspace.len >= q4k_i8_rows_workspace_bytes(in_dim)) {
+        hipError_t e = launch_q4k_digit_planes(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
+                                               static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
+        for (int i = 0; e == hipSuccess && i < (pair ? 2 : 1); ++i) {
+            if (counters) {
+                if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
+                else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
+                else counters->mm++;
+            }
+            e = launch_gemv_q4k_i8_rows(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const void*>(workspace.ptr),
+                                        reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), static_cast<int>(rows),
+                                        static_cast<int>(in_dim), static_cast<int>(out_dim), i ? ep_b : ep);
+        }
+        return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+    }
     // more rows than one GEMV launch holds: X split once into the caller's scratch, then the
     // GEMM (without scratch the GEMV serves them a launch at a time)
     const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
@@ -710,7 +728,9 @@ size_t afhip_linear_workspace_bytes(int tensor_type, size_t rows, size_t in_dim,
             return 0;
         if (afhip_uses_q8k_activation_quant(tensor_type, rows, in_dim, out_dim)) return q4k_q8k_workspace_bytes(rows, in_dim);
         const size_t gemm_rows = static_cast<size_t>(gemm_q4k_min_rows(static_cast<int>(in_dim)));
-        return rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
+        const size_t gemm_bytes = rows >= gemm_rows ? gemm_q4k_workspace_bytes(rows, in_dim, out_dim) : 0;
+        const size_t planes_bytes = q4k_i8_rows_supports(rows, in_dim) ? q4k_i8_rows_workspace_bytes(in_dim) : 0;  // 3 .. 8 rows
+        return gemm_bytes > planes_bytes ? gemm_bytes : planes_bytes;
     }
     if (block_bytes(tensor_type) == 0 || in_dim % 32 != 0 || rows == 0 || out_dim == 0) return 0;
     size_t guard;  // the sizes below are sums of a few such products: refuse shapes whose products wrap

@@ -396,18 +396,82 @@ typedef int t_i32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kDigitPadBytes = 48;  // LDS stride of a digit plane: K + 48 spreads the planes over the banks
 
+// One super-block of one row, four values a lane: the lane's word of each of the four digit planes, -s as a
+// number (NaN for a block with an infinity or a NaN in it), and the f32 sum of the lane's sub-block (lane >> 3).
+struct Q4kDigits {
+    uint32_t plane[4];
+    float minus_s;
+    float sub_sum;
+};
+__device__ __forceinline__ Q4kDigits q4k_digit_planes(const float4 v) {
+    float m = fmaxf(fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)), fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
+    m = max_over_8(m);
+    m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
+    const int mb = __builtin_bit_cast(int, m);
+    m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 0)),
+                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 16))),
+              fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 32)),
+                    __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 48))));
+    // |x| < 2^(e - 126) (subnormals: e = 1): times 2^(156 - e) it stays below 2^30.  The exponent goes by
+    // v_ldexp_f32 both ways (2^(156 - e) itself is past the f32 range for small e).
+    const int e_raw = (__builtin_bit_cast(int, m) >> 23) & 0xFF;
+    const int e = e_raw < 1 ? 1 : e_raw;
+    Q4kDigits out;
+    out.minus_s = e_raw == 255 ? __builtin_nanf("") : static_cast<float>(e - 156);
+    const float vv[4] = {v.x, v.y, v.z, v.w};
+    uint32_t t[4];  // the four signed digits of each value, lowest in byte 0
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        t[k] = (static_cast<uint32_t>(static_cast<int>(__builtin_ldexpf(vv[k], 156 - e))) + 0x80808080u) ^ 0x80808080u;
+    // 4 x 4 byte transpose: plane[d] = digit d of the lane's four values (v_perm_b32: selectors 0..3 take
+    // bytes of the second operand, 4..7 of the first)
+    const uint32_t lo01 = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(t[1], t[0], 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(t[3], t[2], 0x07030602u);
+    out.plane[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    out.plane[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    out.plane[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    out.plane[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+    out.sub_sum = sum_over_8((v.x + v.y) + (v.z + v.w));
+    return out;
+}
+
+// The digit planes of up to eight rows made once, for the kernel below with kPlanesGiven: in MFMA
+// operand order -- 1 KB per (super-block, sub-block): lane (MFMA row c = 4 * row + digit, half g) holds
+// its 16 bytes (K = 16 g .. 16 g + 15 of the sub-block) at 16 * (32 g + c) -- so a wavefront's operand is
+// one contiguous load; then -s per (row, super-block) and the sub-block sums.  One wavefront per item.
+__global__ __launch_bounds__(256) void q4k_digit_planes_kernel(const float* __restrict__ x, int rows, int in_dim,
+                                                               uint8_t* __restrict__ frag, float* __restrict__ minus_s,
+                                                               float* __restrict__ sub_sums) {
+    const int kb = in_dim >> 8, lane = threadIdx.x & 63;
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= rows * kb) return;
+    const int r = item / kb, sb = item - r * kb;
+    const Q4kDigits dg = q4k_digit_planes(reinterpret_cast<const float4*>(x + static_cast<size_t>(r) * in_dim + sb * kQ4kBlockValues)[lane]);
+    // the lane's values are K = 4 (lane % 8) .. + 3 of sub-block lane / 8: half g = (lane % 8) / 4, bytes 4 (lane % 4) ..
+    uint8_t* base = frag + (static_cast<size_t>(sb) * 8 + (lane >> 3)) * 1024 + (32 * ((lane & 7) >> 2) + 4 * r) * 16 + 4 * (lane & 3);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) *reinterpret_cast<uint32_t*>(base + 16 * d) = dg.plane[d];
+    if ((lane & 7) == 0) sub_sums[(static_cast<size_t>(r) * kb + sb) * 8 + (lane >> 3)] = dg.sub_sum;
+    if (lane == 0) minus_s[r * kb + sb] = dg.minus_s;
+}
+
 // kGroups = ceil(rows / 2) row groups: row r sits in lane half r % 2, D registers 4 (r / 2) + digit.
-template <int kGroups, int kFlight, int kMaxThreads>
-__global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst, const float* __restrict__ x,
+// kPlanesGiven: the digit planes, -s and the sub-block sums come from q4k_digit_planes_kernel (`frag`, `frag_scale`,
+// `frag_sums`) instead of being made here from `x`: the MFMA operand is then a 16-byte load per lane and sub-block,
+// requested with the weights, and nothing of X passes through LDS but the few floats of the wavefront's own slice.
+template <int kGroups, int kFlight, int kMaxThreads, bool kPlanesGiven = false>
+__global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst, const float* __restrict__ x,
                                                                   const uint8_t* __restrict__ weight, int rows, int in_dim,
-                                                                  int out_dim, int slices, int sb_per_slice, Epilogue ep) {
+                                                                  int out_dim, int slices, int sb_per_slice, Epilogue ep,
+                                                                  const uint8_t* __restrict__ frag, const float* __restrict__ frag_scale,
+                                                                  const float* __restrict__ frag_sums) {
     const int kb = in_dim >> 8;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int threads = static_cast<int>(blockDim.x);
     const int plane_stride = in_dim + kDigitPadBytes;
-    unsigned char* xdig = q4k_mfma_lds;  // [rows * 4][plane_stride]: the digit planes of every row
-    float* xscale = reinterpret_cast<float*>(q4k_mfma_lds + static_cast<size_t>(rows) * 4 * plane_stride);  // [rows][kb]: -s
+    unsigned char* xdig = q4k_mfma_lds;  // [rows * 4][plane_stride]: the digit planes of every row (not with kPlanesGiven)
+    float* xscale = reinterpret_cast<float*>(q4k_mfma_lds + (kPlanesGiven ? 0 : static_cast<size_t>(rows) * 4 * plane_stride));  // [rows][kb]: -s
     float* xsum = xscale + ((rows * kb + 3) & ~3);                                                          // [rows][kb * 8], 16-byte aligned
     float* partial = xsum + rows * kb * 8;                                                                  // [waves][kGroups][64]
 
@@ -418,7 +482,12 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
     const int sb_end = min(kb, sb_begin + sb_per_slice);
     const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
 
+    // MFMA row c = digit (c & 3) of row (c >> 2); rows past the last read row 0's first plane (their D rows are
+    // never looked at).  Lane half g supplies K = 16 g .. 16 g + 15.
+    const int c = lane & 31, g = lane >> 5;
+    const int a_lane = 32 * g + ((c >> 2) < rows ? c : 0);
     t_u32x4 hdr[kFlight], qv[kFlight][4];
+    t_i32x4 av[kPlanesGiven ? kFlight : 1][8];
     auto request = [&](int sb_first) {
 #pragma unroll
         for (int f = 0; f < kFlight; ++f) {
@@ -429,9 +498,25 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
 #pragma unroll
             for (int t = 0; t < 4; ++t)
                 qv[f][t] = __builtin_nontemporal_load(reinterpret_cast<const t_u32x4*>(base + 512 + t * 1024 + 16 * lane));
+            if (kPlanesGiven) {
+#pragma unroll
+                for (int sub = 0; sub < 8; ++sub)
+                    av[f][sub] = *reinterpret_cast<const t_i32x4*>(frag + (static_cast<size_t>(sb) * 8 + sub) * 1024 + a_lane * 16);
+            }
         }
     };
 
+    if (kPlanesGiven) {
+        // ---- 1. the weights and operands first, then the few floats of this wavefront's slice: -s and the sub-block sums
+        request(sb_begin);
+        for (int sb = sb_begin; sb < sb_end; ++sb) {
+            if (lane < 8 * rows) xsum[(lane >> 3) * (kb * 8) + sb * 8 + (lane & 7)] = frag_sums[(static_cast<size_t>(lane >> 3) * kb + sb) * 8 + (lane & 7)];
+            if (lane < rows) xscale[lane * kb + sb] = frag_scale[lane * kb + sb];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    } else {
     // ---- 1. this wavefront's slice of X: item i = (row i / n_sb, super-block sb_begin + i % n_sb), four values a lane
     {
         const int n_sb = max(sb_end - sb_begin, 0), n_items = rows * n_sb;
@@ -441,36 +526,12 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
         };
         auto digits_of_item = [&](int i, const float4 v) {
             const int r = i / n_sb, sb = sb_begin + (i - r * n_sb);
-            float m = fmaxf(fmaxf(__builtin_fabsf(v.x), __builtin_fabsf(v.y)), fmaxf(__builtin_fabsf(v.z), __builtin_fabsf(v.w)));
-            m = max_over_8(m);
-            m = fmaxf(m, dpp_move<kDppRowMirror>(m));  // 16-lane row maximum in every lane
-            const int mb = __builtin_bit_cast(int, m);
-            m = fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 0)),
-                            __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 16))),
-                      fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 32)),
-                            __builtin_bit_cast(float, __builtin_amdgcn_readlane(mb, 48))));
-            // |x| < 2^(e - 126) (subnormals: e = 1): times 2^(156 - e) it stays below 2^30.  The exponent goes by
-            // v_ldexp_f32 both ways (2^(156 - e) itself is past the f32 range for small e).
-            const int e_raw = (__builtin_bit_cast(int, m) >> 23) & 0xFF;
-            const int e = e_raw < 1 ? 1 : e_raw;
-            const float down = e_raw == 255 ? __builtin_nanf("") : static_cast<float>(e - 156);  // -s, as a number
-            const float vv[4] = {v.x, v.y, v.z, v.w};
-            uint32_t t[4];  // the four signed digits of each value, lowest in byte 0
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-                t[k] = (static_cast<uint32_t>(static_cast<int>(__builtin_ldexpf(vv[k], 156 - e))) + 0x80808080u) ^ 0x80808080u;
-            // 4 x 4 byte transpose: plane[d] = digit d of the lane's four values (v_perm_b32: selectors 0..3 take
-            // bytes of the second operand, 4..7 of the first)
-            const uint32_t lo01 = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(t[1], t[0], 0x07030602u);
-            const uint32_t lo23 = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(t[3], t[2], 0x07030602u);
-            const uint32_t plane[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
-                                       __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+            const Q4kDigits dg = q4k_digit_planes(v);
 #pragma unroll
             for (int d = 0; d < 4; ++d)
-                *reinterpret_cast<uint32_t*>(xdig + static_cast<size_t>(r * 4 + d) * plane_stride + sb * kQ4kBlockValues + 4 * lane) = plane[d];
-            const float s = sum_over_8((v.x + v.y) + (v.z + v.w));
-            if ((lane & 7) == 0) xsum[r * (kb * 8) + sb * 8 + (lane >> 3)] = s;
-            if (lane == 0) xscale[r * kb + sb] = down;
+                *reinterpret_cast<uint32_t*>(xdig + static_cast<size_t>(r * 4 + d) * plane_stride + sb * kQ4kBlockValues + 4 * lane) = dg.plane[d];
+            if ((lane & 7) == 0) xsum[r * (kb * 8) + sb * 8 + (lane >> 3)] = dg.sub_sum;
+            if (lane == 0) xscale[r * kb + sb] = dg.minus_s;
         };
         constexpr int kAhead = 2;  // items requested before the weights (one row, or two rows, of a one-super-block slice)
         float4 first[kAhead];
@@ -488,10 +549,9 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
+    }
 
-    // ---- 2. this lane's roles.  A operand: MFMA row c = digit (c & 3) of row (c >> 2); rows past the
-    // last read row 0's first plane (their D rows are never looked at).  Lane half g supplies K = 16 g .. 16 g + 15.
-    const int c = lane & 31, g = lane >> 5;
+    // ---- 2. this lane's roles
     const bool a_live = (c >> 2) < rows;
     const unsigned char* a_base = xdig + static_cast<size_t>(a_live ? c : 0) * plane_stride + 16 * g;
     // results: D registers 4 G .. 4 G + 3 (digits) of lane half g belong to row 2 G + g, output column c of the tile
@@ -521,15 +581,19 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
             const uint32_t sc_hi = (h.w & 0x0F0F0F0Fu) | ((h.y >> 2) & 0x30303030u);
             const uint32_t mn_hi = ((h.w >> 4) & 0x0F0F0F0Fu) | ((h.z >> 2) & 0x30303030u);
             const unsigned char* a_sb = a_base + sb * kQ4kBlockValues;
-            float xs[kGroups][8];
+            // the sub-block sums of a row group: all eight at once for one or two groups, one by one for more (registers)
+            constexpr bool kSumsAhead = kGroups <= 2;
+            float xs[kSumsAhead ? kGroups : 1][8];
             int digit_sum[kGroups][4];
             float min_sum[kGroups];
 #pragma unroll
             for (int G = 0; G < kGroups; ++G) {
-                const float4 xs_lo = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8);
-                const float4 xs_hi = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8 + 4);
-                xs[G][0] = xs_lo.x, xs[G][1] = xs_lo.y, xs[G][2] = xs_lo.z, xs[G][3] = xs_lo.w;
-                xs[G][4] = xs_hi.x, xs[G][5] = xs_hi.y, xs[G][6] = xs_hi.z, xs[G][7] = xs_hi.w;
+                if (kSumsAhead) {
+                    const float4 xs_lo = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8);
+                    const float4 xs_hi = *reinterpret_cast<const float4*>(xsum_row[G] + sb * 8 + 4);
+                    xs[G][0] = xs_lo.x, xs[G][1] = xs_lo.y, xs[G][2] = xs_lo.z, xs[G][3] = xs_lo.w;
+                    xs[G][4] = xs_hi.x, xs[G][5] = xs_hi.y, xs[G][6] = xs_hi.z, xs[G][7] = xs_hi.w;
+                }
                 digit_sum[G][0] = digit_sum[G][1] = digit_sum[G][2] = digit_sum[G][3] = 0;
                 min_sum[G] = 0.0f;
             }
@@ -542,7 +606,7 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
                     t_i32x4 b;
 #pragma unroll
                     for (int k = 0; k < 4; ++k) b[k] = static_cast<int>((hi ? w[k] >> 4 : w[k]) & 0x0F0F0F0Fu);
-                    const t_i32x4 a = *reinterpret_cast<const t_i32x4*>(a_sb + 32 * sub);
+                    const t_i32x4 a = kPlanesGiven ? av[f][sub] : *reinterpret_cast<const t_i32x4*>(a_sb + 32 * sub);
                     const t_i32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
                     const t_i32x16 D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, zero, 0, 0, 0);
                     const int sc = static_cast<int>(((sub < 4 ? sc_lo : sc_hi) >> (8 * (sub & 3))) & 0xFFu);
@@ -551,8 +615,11 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
                     for (int G = 0; G < kGroups; ++G) {
 #pragma unroll
                         for (int k = 0; k < 4; ++k) digit_sum[G][k] += __mul24(D[4 * G + k], sc);
-                        min_sum[G] = __builtin_fmaf(mn, xs[G][sub], min_sum[G]);
+                        min_sum[G] = __builtin_fmaf(mn, kSumsAhead ? xs[kSumsAhead ? G : 0][sub] : xsum_row[G][sb * 8 + sub], min_sum[G]);
                     }
+                    // three and four row groups: one set of MFMA results at a time (the scheduler would keep two or
+                    // three sub-blocks' worth live and spill); the other wavefronts of the SIMD fill the matrix core's latency
+                    if (kGroups >= 3) __builtin_amdgcn_sched_barrier(0);
                 }
             }
 #pragma unroll
@@ -585,6 +652,11 @@ __global__ __launch_bounds__(kMaxThreads, kFlight == 1 ? 8 : 4) void gemv_q4k_i8
             dst[idx] = finish_output(ep, o, idx, total);
         }
     }
+}
+
+size_t q4k_i8_rows_lds_bytes(int rows, int in_dim, int waves) {  // kPlanesGiven: -s, sub-block sums, the slices' partial sums
+    return ((static_cast<size_t>(rows) * (in_dim / 256) + 3) & ~static_cast<size_t>(3)) * 4 + static_cast<size_t>(rows) * (in_dim / 32) * 4 +
+           static_cast<size_t>(waves) * ((rows + 1) / 2) * 64 * 4;
 }
 
 size_t q4k_i8_lds_bytes(int rows, int in_dim, int waves) {
@@ -896,7 +968,7 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     if constexpr (kGroups <= 2) {
         if (use_i8) {
             if (tiles_per_wg != 1) return hipErrorInvalidValue;  // (a tuning knob asked for a shape this kernel does not have)
-            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
+            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue, const uint8_t*, const float*, const float*) = nullptr;
             if constexpr (kGroups == 1) {
                 switch (variant) {
                     case 0:
@@ -917,7 +989,8 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
                     return e;
                 large_lds8[variant] = true;
             }
-            hipLaunchKernelGGL(k8, dim3(grid), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices, sb_per_slice, ep);
+            hipLaunchKernelGGL(k8, dim3(grid), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices, sb_per_slice, ep,
+                               static_cast<const uint8_t*>(nullptr), static_cast<const float*>(nullptr), static_cast<const float*>(nullptr));
             return hipGetLastError();
         }
     }
@@ -1065,6 +1138,60 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
                        xsum, weight, rows, in_dim, out_dim, sb_per_split, partial, ep);
     if (hipError_t e = hipGetLastError(); e != hipSuccess || shares == 1) return e;
     return launch_splitk_reduce(stream, dst, partial, static_cast<size_t>(rows) * out_dim, out_dim, shares, ep);
+}
+
+// Three to eight rows with the caller's scratch: the digit planes of X made once by their own kernel
+// (launch_q4k_digit_planes), then one launch per matrix of the int8 kernel with its operands read from them.
+bool q4k_i8_rows_supports(size_t rows, size_t in_dim) {
+    return rows >= 3 && rows <= 8 && in_dim % kQ4kBlockValues == 0 && in_dim <= static_cast<size_t>(gemv_q4k_max_in_dim());
+}
+
+// [operand fragments: 8 KB a super-block][-s: 8 rows x super-blocks][sub-block sums: 8 rows x super-blocks x 8]
+size_t q4k_i8_rows_workspace_bytes(size_t in_dim) {
+    const size_t kb = in_dim / kQ4kBlockValues;
+    return kb * 8192 + kb * 8 * 4 + kb * 8 * 8 * 4;
+}
+
+hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace) {
+    if (!q4k_i8_rows_supports(static_cast<size_t>(rows), static_cast<size_t>(in_dim)) || workspace == nullptr) return hipErrorInvalidValue;
+    const int kb = in_dim / kQ4kBlockValues;
+    uint8_t* frag = static_cast<uint8_t*>(workspace);
+    float* minus_s = reinterpret_cast<float*>(frag + static_cast<size_t>(kb) * 8192);
+    float* sums = minus_s + static_cast<size_t>(kb) * 8;
+    const int items = rows * kb;
+    hipLaunchKernelGGL(q4k_digit_planes_kernel, dim3((items + 3) / 4), dim3(256), 0, stream, x, rows, in_dim, frag, minus_s, sums);
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, int rows, int in_dim,
+                                   int out_dim, const Epilogue& ep) {
+    if (!q4k_i8_rows_supports(static_cast<size_t>(rows), static_cast<size_t>(in_dim)) || workspace == nullptr) return hipErrorInvalidValue;
+    if (out_dim == 0) return hipSuccess;
+    const int kb = in_dim / kQ4kBlockValues;
+    const uint8_t* frag = static_cast<const uint8_t*>(workspace);
+    const float* minus_s = reinterpret_cast<const float*>(frag + static_cast<size_t>(kb) * 8192);
+    const float* sums = minus_s + static_cast<size_t>(kb) * 8;
+    int slices = 8;
+    while (slices > kb) slices /= 2;
+    const int sb_per_slice = (kb + slices - 1) / slices;
+    const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
+    const size_t lds = q4k_i8_rows_lds_bytes(rows, in_dim, slices);
+    const float* no_x = nullptr;
+    switch ((rows + 1) / 2) {
+        case 2:
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<2, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            break;
+        case 3:
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<3, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            break;
+        default:
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<4, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            break;
+    }
+    return hipGetLastError();
 }
 
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,

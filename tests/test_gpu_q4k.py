@@ -219,6 +219,28 @@ def test_decode_rows_on_extreme_activations():
         assert G.max_rel_err(y[1:], O.linear_q4_k(x[1:rows].copy(), w, rows - 1, in_dim, out_dim, f64=True)) <= TIGHT
 
 
+@pytest.mark.parametrize("rows,in_dim,out_dim", [(3, 4096, 200), (5, 1024, 96), (8, 4096, 14336), (6, 14336, 100), (7, 16384, 40)])
+def test_three_to_eight_rows_with_and_without_scratch(rows, in_dim, out_dim):
+    """With the caller's scratch X becomes digit planes once and the int8 kernel runs on them; without it the bf16
+    kernel (or several launches of the two-row kernel) serves the rows.  Both are held to the oracle."""
+    print(f"case: q4_k rows with / without scratch rows={rows} in={in_dim} out={out_dim}", flush=True)
+    w = synth.weights(Q4K, 95, out_dim, in_dim)
+    x = synth.activations(96, rows, in_dim)
+    x[rows - 1, :256] = 0.0
+    wd = device_weight(PREP, w, out_dim, in_dim)
+    ref = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
+    xd = G.to_dev(x)
+    need = kernels.workspaceBytes(Q4K, rows, in_dim, out_dim)
+    assert need >= in_dim // 256 * (8192 + 32 + 256)
+    scratch = torch.empty(need, dtype=torch.uint8, device=G.DEV)
+    for ws in (G.buf(scratch), kernels.NO_BUFFER):
+        y = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=G.DEV)
+        kernels.launchLinearF32(G.stream(), Q4K, PREP, G.buf(y), G.buf(xd), G.buf(wd), rows, in_dim, out_dim, ws)
+        torch.cuda.synchronize()
+        err = G.max_rel_err(y.cpu().numpy(), ref)
+        assert err <= TIGHT, (ws is kernels.NO_BUFFER, err)
+
+
 Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
 
 
@@ -341,7 +363,9 @@ def test_linear_argument_checks():
     d = torch.empty(4, dtype=torch.int32, device=G.DEV)
     with pytest.raises(_lib.HipError):  # no integer route, so no block dots
         kernels.launchBlockDots(G.stream(), Q4K, RAW, G.buf(d), G.buf(x), G.buf(w), 1, 256, 4, ws)
-    assert kernels.workspaceBytes(Q4K, 4, 4096, 4096) == 0  # decode rows need no scratch
+    assert kernels.workspaceBytes(Q4K, 2, 4096, 4096) == 0  # one or two decode rows need no scratch
+    # three to eight rows: room for X as digit planes (8 KB a super-block + scales and sums); optional, see below
+    assert kernels.workspaceBytes(Q4K, 4, 4096, 4096) == 16 * 8192 + 16 * 32 + 16 * 256
     assert kernels.workspaceBytes(Q4K, 2048, 4096, 14336) == 2048 * 4096 * 6 + 2048 * 128 * 8  # the split of X for the prefill GEMM
     assert kernels.workspaceBytes(Q4K, 64, 4096, 4096) > 64 * 4096 * 6 + 64 * 128 * 8  # ... plus partial sums when K is shared out
     big_w = torch.zeros(4 * 128 * 144, dtype=torch.uint8, device=G.DEV)
