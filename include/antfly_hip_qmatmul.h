@@ -64,9 +64,11 @@ enum afhip_tensor_type { AFHIP_TYPE_F32 = 0, AFHIP_TYPE_Q4_0 = 2, AFHIP_TYPE_Q8_
  * and in its CUDA backend (ops/cuda/cuda_compute.zig:708) -- except on the CPU engine's gated
  * short-K shapes (afhip_uses_q8k_activation_quant), where the activations are quantized to
  * Q8_K as it does there.  No block-dot output for this format.  Both layouts are served: RAW (GGUF bytes, 16-byte aligned) by a vector-ALU
- * kernel, PREPARED (tile-major, see afhip_prepared_weight_bytes) by the MFMA kernels; more
- * rows than one decode launch holds use the caller's workspace
- * (afhip_linear_workspace_bytes) for the prefill GEMM.  in_dim must be a multiple of 256.
+ * kernel, PREPARED (tile-major, see afhip_prepared_weight_bytes) by the MFMA kernels: one or
+ * two rows need no scratch; three to eight rows run fastest with the caller's workspace
+ * (afhip_linear_workspace_bytes: X once as fixed-point digit planes, then an int8-MFMA launch
+ * per matrix) and without it on the bf16-MFMA kernel, as many rows a launch as LDS holds; more
+ * rows use the workspace for the prefill GEMM.  in_dim must be a multiple of 256.
  * Served by the linear launchers and ops, the pair op, the bias / activation / residual
  * epilogues, the argmax ops, embedding lookup, cpy_q_to_f32 and GGUF loading. */
 

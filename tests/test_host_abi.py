@@ -104,17 +104,22 @@ def test_launcher_argument_checks_before_any_launch():
 
 
 def test_q4_k_prefill_workspace_sizes():
-    """Scratch of the Q4_K prefill GEMM: none for rows that fit one GEMV launch (six at K = 4096,
-    one at K = 14336; two rows never), beyond that the split of X
-    (three bf16 parts = 6 bytes per value, plus 64 bytes of sum parts per row and super-block) and,
-    while the row x column grid is small, room for the partial sums of the K shares (a power of
-    two, at most eight, at least two super-blocks each)."""
+    """Scratch of Q4_K: none for one or two rows; three to eight rows: X as digit planes in MFMA operand
+    order (8 KB per super-block, plus a scale per row and super-block and a sum per row and sub-block, laid
+    out for eight rows); rows of the prefill GEMM (more than one GEMV launch holds: seven at K = 4096, three at
+    K = 14336): the split of X (three bf16 parts = 6 bytes per value, plus 64 bytes of sum parts per row and
+    super-block) and, while the row x column grid is small, room for the partial sums of the K shares (a power
+    of two, at most eight, at least two super-blocks each) -- the larger of the two where both apply."""
     Q4K = _lib.TYPE_Q4_K
-    for rows in (1, 6):
+    planes = lambda k: k // 256 * (8192 + 32 + 256)
+    for rows in (1, 2):
         assert kernels.workspaceBytes(Q4K, rows, 4096, 4096) == 0
-    assert kernels.workspaceBytes(Q4K, 7, 4096, 4096) > 0
-    assert kernels.workspaceBytes(Q4K, 2, 14336, 4096) == 0
-    assert kernels.workspaceBytes(Q4K, 3, 14336, 4096) > 0
+        assert kernels.workspaceBytes(Q4K, rows, 14336, 4096) == 0
+    for rows in (3, 6):
+        assert kernels.workspaceBytes(Q4K, rows, 4096, 4096) == planes(4096)
+    assert kernels.workspaceBytes(Q4K, 7, 4096, 4096) >= max(planes(4096), 7 * 4096 * 6)
+    assert kernels.workspaceBytes(Q4K, 3, 14336, 4096) >= max(planes(14336), 3 * 14336 * 6)
+    assert kernels.workspaceBytes(Q4K, 9, 4096, 4096) > 9 * 4096 * 6
     for rows, k, n in [(13, 4096, 14336), (64, 4096, 4096), (512, 4096, 14336), (40, 512, 40), (33, 14336, 4096)]:
         split = (rows * k * 6 + rows * (k // 256) * 64 + 255) // 256 * 256
         got = kernels.workspaceBytes(Q4K, rows, k, n)
