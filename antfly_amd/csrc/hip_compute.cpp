@@ -220,8 +220,8 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
     }
     afhip_buffer scratch{0, 0};
     if (weight->quant_type == AFHIP_TYPE_Q4_K) {
-        // scratch for the split of X when the prefill GEMM serves the rows (repacked tensors), or for the Q8_K
-        // activations on the gated short-K shapes (either layout)
+        // scratch for the digit planes of three to eight rows and for the split of X when the prefill GEMM serves the
+        // rows (repacked tensors), or for the Q8_K activations on the gated short-K shapes (either layout)
         const bool needs = weight->layout == AFHIP_LAYOUT_PREPARED || afhip_uses_q8k_activation_quant(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim);
         const size_t need = needs ? afhip_linear_workspace_bytes(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim) : 0;
         if (need) s = acquire_scratch(self, need, &scratch);
