@@ -105,77 +105,118 @@ __global__ __launch_bounds__(256) void dequantize_q4k_rows_kernel(float* __restr
 //   sc = clamp(round(scale / d), 0, 63), m = clamp(round(min_mag / dmin), 0, 63)  (f32 d, dmin),
 //   nibble = clamp(round((x + min_mag) * (1 / scale)), 0, 15)                      (the unrounded scale),
 // round = half away from zero; every quotient is a correctly rounded f32 division.
-// A wavefront is one super-block: lane l holds values 4l .. 4l+3 (one coalesced 16-byte load),
-// the eight lanes of (l >> 3) are a sub-block.  The lanes of sub-block 2c take the nibbles of
-// sub-block 2c+1 from eight lanes up and store four bytes each; lane 0 stores the header.
+// A wavefront takes eight super-blocks at a time: lane l holds values 4l .. 4l+3 of each (one coalesced
+// 16-byte load a super-block), the eight lanes of (l >> 3) are a sub-block.  After the sub-block minima and
+// maxima (DPP within the eight lanes) lane l keeps those of super-block l & 7, so the 64 lanes hold the 64
+// (super-block, sub-block) pairs and every quotient of the format -- / 15, / 63 twice, scale / d, min / dmin,
+// 1 / scale -- is one correctly rounded division for all eight super-blocks instead of one a super-block
+// (they were two thirds of the kernel's instructions).  The super-block maxima and the 12 header bytes meet by
+// exchanges among the lanes eight apart; the lanes of a sub-block fetch its offset and reciprocal back, form their
+// nibbles, the lanes of sub-block 2c take those of 2c+1 from eight lanes up and store four bytes each.
 __device__ __forceinline__ float min_over_8(float v) {
     v = fminf(v, dpp_move<kDppXor1>(v));
     v = fminf(v, dpp_move<kDppXor2>(v));
     v = fminf(v, dpp_move<kDppHalfMirror>(v));
     return v;
 }
-// max over the eight sub-blocks of a value that is uniform inside each of them; result uniform
-__device__ __forceinline__ float max_over_sub_blocks(float v) {
-    const int bits = __builtin_bit_cast(int, v);
-    float m = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
-#pragma unroll
-    for (int s = 1; s < 8; ++s) m = fmaxf(m, __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 8 * s)));
-    return m;
-}
 // round half away from zero of t >= 0, clamped to [0, hi]
 __device__ __forceinline__ uint32_t round_clamp(float t, int hi) {
     return static_cast<uint32_t>(min(max(static_cast<int>(t + 0x1.fffffep-2f), 0), hi));
+}
+// max / or over the eight lanes that are eight apart (same lane & 7); every lane gets the result
+__device__ __forceinline__ float max_over_stride_8(float v) {
+    v = fmaxf(v, __shfl_xor(v, 8));
+    v = fmaxf(v, __shfl_xor(v, 16));
+    v = fmaxf(v, __shfl_xor(v, 32));
+    return v;
+}
+__device__ __forceinline__ uint32_t or_over_stride_8(uint32_t v) {
+    v |= static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 8));
+    v |= static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 16));
+    v |= static_cast<uint32_t>(__shfl_xor(static_cast<int>(v), 32));
+    return v;
 }
 
 template <bool kNarrow>
 __global__ __launch_bounds__(256) void quantize_q4k_rows_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
                                                                 const long long* __restrict__ ids, size_t rows, int dim,
                                                                 size_t dst_rows) {
+    constexpr int kGroup = 8;  // super-blocks a wavefront takes at a time
     const size_t kb = static_cast<size_t>(dim / kQ4kBlockValues);
-    const size_t units = rows * kb * 64;  // a multiple of 64: a wavefront is live or idle as a whole
-    for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
-         u += static_cast<size_t>(gridDim.x) * blockDim.x) {
-        const float4 v = reinterpret_cast<const float4*>(x)[u];
-        const float lo = min_over_8(fminf(fminf(v.x, v.y), fminf(v.z, v.w)));
-        const float hi = max_over_8(fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
-        const float min_mag = fmaxf(-lo, 0.0f);
-        const float range = hi + min_mag;
+    const size_t total = rows * kb;  // super-blocks
+    const int lane = threadIdx.x & 63, sub = lane >> 3, mine_j = lane & 7;
+    const size_t wave = blockIdx.x * static_cast<size_t>(blockDim.x >> 6) + (threadIdx.x >> 6);
+    const size_t waves = static_cast<size_t>(gridDim.x) * (blockDim.x >> 6);
+    for (size_t first = wave * kGroup; first < total; first += waves * kGroup) {
+        float4 v[kGroup];
+        float lo_m = 0.0f, hi_m = 0.0f;  // of the pair (super-block first + (lane & 7), sub-block lane >> 3)
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+            const size_t sb = first + j < total ? first + j : total - 1;  // past the end: the last one again, nothing stored
+            v[j] = reinterpret_cast<const float4*>(x)[sb * 64 + lane];
+        }
+#pragma unroll
+        for (int j = 0; j < kGroup; ++j) {
+            const float lo = min_over_8(fminf(fminf(v[j].x, v[j].y), fminf(v[j].z, v[j].w)));
+            const float hi = max_over_8(fmaxf(fmaxf(v[j].x, v[j].y), fmaxf(v[j].z, v[j].w)));
+            if (j == 0 || mine_j == j) {
+                lo_m = lo;
+                hi_m = hi;
+            }
+        }
+        const float min_mag = fmaxf(-lo_m, 0.0f);
+        const float range = hi_m + min_mag;
         const float scale = range == 0.0f ? 1.0f : range / 15.0f;
-        const float max_scale = max_over_sub_blocks(scale), max_min = max_over_sub_blocks(min_mag);
+        const float max_scale = max_over_stride_8(scale), max_min = max_over_stride_8(min_mag);
         const float d = max_scale == 0.0f ? 1.0f : max_scale / 63.0f;
         const float dmin = max_min == 0.0f ? 1.0f : max_min / 63.0f;
         const uint32_t sc = max_scale == 0.0f ? 0u : round_clamp(scale / d, 63);
         const uint32_t mn = max_min == 0.0f ? 0u : round_clamp(min_mag / dmin, 63);
         const float inv = scale == 0.0f ? 0.0f : 1.0f / scale;
-        const uint32_t mine = round_clamp((v.x + min_mag) * inv, 15) | (round_clamp((v.y + min_mag) * inv, 15) << 8) |
-                              (round_clamp((v.z + min_mag) * inv, 15) << 16) | (round_clamp((v.w + min_mag) * inv, 15) << 24);
-        const uint32_t other = static_cast<uint32_t>(__shfl_down(static_cast<int>(mine), 8));
-        // the 6-bit pairs of all eight sub-blocks, as uniform values
-        uint32_t scs[8], mns[8];
-#pragma unroll
-        for (int s = 0; s < 8; ++s) {
-            scs[s] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(sc), 8 * s));
-            mns[s] = static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(mn), 8 * s));
+        // this pair's bits of the 12 scale bytes (packQ4KScaleMins, gguf/quant_codec.zig:1273-1287), then all eight pairs' together
+        const int at = 8 * (sub & 3);
+        uint32_t hy, hz, hw;
+        if (sub < 4) {
+            hy = (sc & 63u) << at;
+            hz = (mn & 63u) << at;
+            hw = 0u;
+        } else {
+            hy = ((sc >> 4) << 6) << at;
+            hz = ((mn >> 4) << 6) << at;
+            hw = ((sc & 15u) | ((mn & 15u) << 4)) << at;
         }
-        const size_t tb = u >> 6;
-        const size_t t = kNarrow ? static_cast<uint32_t>(tb) / static_cast<uint32_t>(kb) : tb / kb, b = tb - t * kb;
-        const long long row = ids ? ids[t] : static_cast<long long>(t);
-        if (row < 0 || static_cast<size_t>(row) >= dst_rows) continue;  // a row id outside the destination writes nothing
-        uint8_t* out = dst + (static_cast<size_t>(row) * kb + b) * kQ4kBlockBytes;
-        const int lane = static_cast<int>(u & 63), sub = lane >> 3, j = lane & 7;
-        if ((sub & 1) == 0) *reinterpret_cast<uint32_t*>(out + 16 + 32 * (sub >> 1) + 4 * j) = mine | (other << 4);
-        if (lane == 0) {
+        hy = or_over_stride_8(hy);
+        hz = or_over_stride_8(hz);
+        hw = or_over_stride_8(hw);
+        // where super-block first + j goes (lanes 0 .. 7 hold one destination each; every lane fetches them as it needs them)
+        const size_t my_sb = first + mine_j;
+        long long my_out = -1;  // byte offset of the super-block in dst, -1: not stored
+        if (my_sb < total) {
+            const size_t t = kNarrow ? static_cast<uint32_t>(my_sb) / static_cast<uint32_t>(kb) : my_sb / kb, b = my_sb - t * kb;
+            const long long row = ids ? ids[t] : static_cast<long long>(t);
+            if (row >= 0 && static_cast<size_t>(row) < dst_rows)  // a row id outside the destination writes nothing
+                my_out = static_cast<long long>((static_cast<size_t>(row) * kb + b) * kQ4kBlockBytes);
+        }
+        if (sub == 0 && my_out >= 0) {
             q4k_u32x4 header;
             header.x = __builtin_bit_cast(uint16_t, static_cast<_Float16>(d)) |
                        (static_cast<uint32_t>(__builtin_bit_cast(uint16_t, static_cast<_Float16>(dmin))) << 16);
-            header.y = header.z = header.w = 0;
+            header.y = hy;
+            header.z = hz;
+            header.w = hw;
+            *reinterpret_cast<q4k_u32x4*>(dst + my_out) = header;
+        }
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {  // packQ4KScaleMins, gguf/quant_codec.zig:1273-1287
-                header.y |= ((scs[i] & 63) | ((scs[i + 4] >> 4) << 6)) << (8 * i);
-                header.z |= ((mns[i] & 63) | ((mns[i + 4] >> 4) << 6)) << (8 * i);
-                header.w |= ((scs[i + 4] & 15) | ((mns[i + 4] & 15) << 4)) << (8 * i);
-            }
-            *reinterpret_cast<q4k_u32x4*>(out) = header;
+        for (int j = 0; j < kGroup; ++j) {
+            // offset and reciprocal of (super-block j, this lane's sub-block): from lane 8 * sub + j
+            const float off = __shfl(min_mag, 8 * sub + j), rcp = __shfl(inv, 8 * sub + j);
+            const int out_lo = __shfl(static_cast<int>(my_out & 0xFFFFFFFFll), j), out_hi = __shfl(static_cast<int>(my_out >> 32), j);
+            const long long out = (static_cast<long long>(out_hi) << 32) | static_cast<uint32_t>(out_lo);
+            const uint32_t nib = round_clamp((v[j].x + off) * rcp, 15) | (round_clamp((v[j].y + off) * rcp, 15) << 8) |
+                                 (round_clamp((v[j].z + off) * rcp, 15) << 16) | (round_clamp((v[j].w + off) * rcp, 15) << 24);
+            const uint32_t other = static_cast<uint32_t>(__shfl_down(static_cast<int>(nib), 8));
+            if ((sub & 1) == 0 && out >= 0)
+                *reinterpret_cast<uint32_t*>(dst + out + 16 + 32 * (sub >> 1) + 4 * mine_j) = nib | (other << 4);
         }
     }
 }
@@ -763,7 +804,8 @@ hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint
 hipError_t launch_quantize_q4k_rows(hipStream_t stream, uint8_t* dst_raw, const float* x, const long long* ids, size_t rows,
                                     int dim, size_t dst_rows) {
     if (rows == 0 || dim == 0) return hipSuccess;
-    size_t grid = (rows * static_cast<size_t>(dim >> 2) + 255) / 256;
+    const size_t groups = (rows * static_cast<size_t>(dim / kQ4kBlockValues) + 7) / 8;  // a wavefront takes eight super-blocks at a time
+    size_t grid = (groups + 3) / 4;
     if (grid > 65536) grid = 65536;
     const bool narrow = rows * static_cast<size_t>(dim / kQ4kBlockValues) <= 0xFFFFFFFFull;
     if (narrow) hipLaunchKernelGGL(quantize_q4k_rows_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
