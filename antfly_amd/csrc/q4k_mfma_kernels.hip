@@ -131,7 +131,8 @@ __global__ __launch_bounds__(256) void dequantize_q4k_tiled_rows_kernel(float* _
         out.y = dsc * ubyte_to_f32(nib, 1) - dmn;
         out.z = dsc * ubyte_to_f32(nib, 2) - dmn;
         out.w = dsc * ubyte_to_f32(nib, 3) - dmn;
-        reinterpret_cast<float4*>(dst)[u] = out;
+        typedef float f32x4_t __attribute__((ext_vector_type(4)));  // written once, read by someone else: streamed past the caches
+        __builtin_nontemporal_store(f32x4_t{out.x, out.y, out.z, out.w}, reinterpret_cast<f32x4_t*>(dst) + u);
     }
 }
 
