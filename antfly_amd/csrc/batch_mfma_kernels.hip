@@ -930,6 +930,20 @@ hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint
 // workgroup, else two.
 int bm8_column_groups(int out_dim) { return (out_dim + 63) / 64 >= gemv_compute_units() * 3 / 4 ? 4 : 2; }
 
+int bm_shares(int tensor_type, int in_dim) {
+    const int share_max = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
+    return (in_dim / 32 + share_max - 1) / share_max;
+}
+
+// A single group of sixteen columns a workgroup: for a matrix whose 32-column tiles (times K shares) leave compute
+// units idle while its 16-column tiles fill them in one round -- 4096 columns at K = 4096: 7.9 against 9.0 us on
+// batch_mfma_kernel; with a second, partial round (6144 columns: 9.7 against 9.4) it does not pay.
+bool bm8_one_column_group(int tensor_type, size_t in_dim, size_t out_dim) {
+    const size_t shares = static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim))), units = static_cast<size_t>(gemv_compute_units());
+    const size_t narrow = (out_dim + 15) / 16 * shares;
+    return (out_dim + 31) / 32 * shares < units && narrow >= units && narrow <= units + units / 8;
+}
+
 template <int kType>
 hipError_t bm_launch32(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
                        int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
@@ -945,11 +959,6 @@ hipError_t bm_launch32(hipStream_t stream, float* dst, float* partial, const uin
     return hipGetLastError();
 }
 
-int bm_shares(int tensor_type, int in_dim) {
-    const int share_max = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
-    return (in_dim / 32 + share_max - 1) / share_max;
-}
-
 }  // namespace
 
 bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
@@ -961,12 +970,13 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
 }
 
 // The eight-row kernel: at most eight rows, rows of whole 16-byte runs of weight scales, and at
-// least a workgroup per compute unit (32-column tiles times K shares) -- on a smaller grid the
-// memory system is not the limit and the shorter dependency chain of batch_mfma_kernel wins.
+// least a workgroup per compute unit (32-column tiles times K shares, or 16-column tiles in one round) -- on a
+// smaller grid the memory system is not the limit and the shorter dependency chain of batch_mfma_kernel wins.
 bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
     const size_t kb = in_dim / 32;
     if (rows > 8 || kb % 8 != 0) return false;
+    if (bm8_one_column_group(tensor_type, in_dim, out_dim)) return true;
     return (out_dim + 31) / 32 * static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim))) >= static_cast<size_t>(gemv_compute_units());
 }
 
@@ -1033,7 +1043,8 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     if (eight) {
         const bool wide = bm8_column_groups(out_dim) == 4;
 #define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
-        e = tensor_type == 2 ? (wide ? AFHIP_BM8(2, 4) : AFHIP_BM8(2, 2)) : (wide ? AFHIP_BM8(8, 4) : AFHIP_BM8(8, 2));
+        const bool one = bm8_one_column_group(tensor_type, static_cast<size_t>(in_dim), static_cast<size_t>(out_dim));
+        e = tensor_type == 2 ? (wide ? AFHIP_BM8(2, 4) : (one ? AFHIP_BM8(2, 1) : AFHIP_BM8(2, 2))) : (wide ? AFHIP_BM8(8, 4) : (one ? AFHIP_BM8(8, 1) : AFHIP_BM8(8, 2)));
 #undef AFHIP_BM8
     }
     else if (thirty_two)

@@ -128,6 +128,8 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # wavefront and a ragged last tile; 64-column tiles, ragged; K shares with a short last share; a
     # wavefront with half its blocks
     (8, 512, 8200), (5, 4096, 12290), (7, 9216, 4112), (6, 256, 16416),
+    # ... on 16-column tiles (4096 to 4608 columns and one K share): full, ragged last tile, one live wavefront
+    (5, 4096, 4096), (8, 1024, 4600), (6, 256, 4100),
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
