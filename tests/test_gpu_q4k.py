@@ -241,6 +241,21 @@ def test_three_to_eight_rows_with_and_without_scratch(rows, in_dim, out_dim):
         assert err <= TIGHT, (ws is kernels.NO_BUFFER, err)
 
 
+def test_digit_plane_rows_pair_and_bias():
+    """Three to eight rows: a pair call makes the digit planes once and runs both matrices on them; each half equals
+    the single op bit for bit, and a bias is added to that value in f32."""
+    rows, in_dim, out_dim = 5, 1024, 640
+    wa, wb = synth.weights(Q4K, 97, out_dim, in_dim), synth.weights(Q4K, 98, out_dim, in_dim)
+    x = synth.activations(99, rows, in_dim)
+    da, db = device_weight(PREP, wa, out_dim, in_dim), device_weight(PREP, wb, out_dim, in_dim)
+    ya, yb = G.linear_pair(Q4K, PREP, x, da, db, rows, in_dim, out_dim)
+    assert np.array_equal(ya, G.linear(Q4K, PREP, x, da, rows, in_dim, out_dim))
+    assert np.array_equal(yb, G.linear(Q4K, PREP, x, db, rows, in_dim, out_dim))
+    assert G.max_rel_err(yb, O.linear_q4_k(x, wb, rows, in_dim, out_dim, f64=True)) <= TIGHT
+    bias = synth.activations(100, 1, out_dim).reshape(-1)
+    assert np.array_equal(G.linear_bias(Q4K, PREP, x, da, bias, rows, in_dim, out_dim), ya + bias[None, :])
+
+
 Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
 
 
