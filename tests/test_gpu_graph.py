@@ -24,8 +24,8 @@ CALLS = [
     (Q8, 2, 1024, 640),     # fused GEMV, two rows
     (Q4, 6, 1024, 1536),    # quantizer + rows kernel
     (Q8, 40, 1024, 640),    # quantizer + MFMA GEMM
-    (Q4K, 1, 1024, 200),    # Q4_K decode kernel (ragged last tile)
-    (Q4K, 5, 1024, 200),    # Q4_K decode kernel, several rows
+    (Q4K, 1, 1024, 200),    # Q4_K int8 decode kernel (ragged last tile)
+    (Q4K, 5, 1024, 200),    # Q4_K digit-plane kernel + int8 kernel on the planes, several rows
     (Q4K, 20, 4096, 300),   # Q4_K prefill GEMM, K shared out over workgroups
     (Q4K, 70, 1024, 200),   # Q4_K prefill GEMM, three row groups
     (Q4, 7, 512, 8200),     # compact-fragment quantizer + eight-row MFMA kernel
