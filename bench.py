@@ -614,6 +614,7 @@ def main() -> int:
             ("q4_batch_m64_k4096_n14336", Q4, 64, 4096, 14336),
             ("q4_batch_m16_k14336_n4096", Q4, 16, 14336, 4096),  # K longer than one share: partial sums + reduce kernel
             ("q4_batch_m16_k4096_n4096", Q4, 16, 4096, 4096),
+            ("q4_batch_m5_k4096_n4096", Q4, 5, 4096, 4096),
         ]:
             copies = args.copies if fmt == Q4 or n > 4096 else 2 * args.copies
             w_s, e_s = time_config(fmt, r, k, n, small_steps, 20, copies, 99)
@@ -622,10 +623,12 @@ def main() -> int:
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
         for name, r, k, n in [("q4k_gemv_m1_k4096_n14336", 1, 4096, 14336), ("q4k_gemv_m2_k4096_n14336", 2, 4096, 14336),
-                              ("q4k_gemv_m5_k4096_n14336", 5, 4096, 14336), ("q4k_gemv_m1_k14336_n4096", 1, 14336, 4096)]:
+                              ("q4k_gemv_m5_k4096_n14336", 5, 4096, 14336), ("q4k_gemv_m8_k4096_n14336", 8, 4096, 14336),
+                              ("q4k_gemv_m1_k14336_n4096", 1, 14336, 4096), ("q4k_gemv_m5_k14336_n4096", 5, 14336, 4096)]:
             w_s, e_s = time_config(Q4K, r, k, n, small_steps, 20, args.copies, 77)
             b = n * (k // 256) * 144 + 4 * r * (k + n)
-            extra[name] = {"what": "Q4_K (144-byte super-blocks, tile-major device layout), f32-accurate on bf16 MFMA",
+            extra[name] = {"what": "Q4_K (144-byte super-blocks, tile-major device layout), f32-accurate: fixed-point activations on int8 MFMA "
+                                   "(3+ rows: digit planes made once by their own launch, included)",
                            "us_per_call": round(e_s / small_steps * 1e6, 3),
                            "GBps": round(b * small_steps / e_s / 1e9, 1),
                            "frac_hbm_peak": round(b * small_steps / e_s / HBM_PEAK_BPS, 4)}
