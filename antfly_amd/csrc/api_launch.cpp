@@ -205,16 +205,18 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
         workspace.len >= q4k_i8_rows_workspace_bytes(in_dim)) {
         hipError_t e = launch_q4k_digit_planes(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
                                                static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
-        for (int i = 0; e == hipSuccess && i < (pair ? 2 : 1); ++i) {
-            if (counters) {
+        if (counters) {
+            for (int i = 0; i < (pair ? 2 : 1); ++i) {
                 if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
                 else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
                 else counters->mm++;
             }
-            e = launch_gemv_q4k_i8_rows(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const void*>(workspace.ptr),
-                                        reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), static_cast<int>(rows),
-                                        static_cast<int>(in_dim), static_cast<int>(out_dim), i ? ep_b : ep);
         }
+        if (e == hipSuccess)  // a pair: both matrices in one launch
+            e = launch_gemv_q4k_i8_rows(stream, reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const void*>(workspace.ptr),
+                                        reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(rows), static_cast<int>(in_dim),
+                                        static_cast<int>(out_dim), ep, pair ? reinterpret_cast<float*>(dst_b.ptr) : nullptr,
+                                        pair ? reinterpret_cast<const uint8_t*>(weight_b.ptr) : nullptr, ep_b);
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     // more rows than one GEMV launch holds: X split once into the caller's scratch, then the
@@ -236,10 +238,18 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
             if (e != hipSuccess) return static_cast<afhip_status>(e);
             continue;
         }
-        hipError_t e = (tiled ? launch_gemv_q4k_tiled : launch_gemv_q4k)(
-            stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const float*>(input.ptr),
-            reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), static_cast<int>(rows), static_cast<int>(in_dim),
-            static_cast<int>(out_dim), i ? ep_b : ep);
+        if (tiled) {  // a pair goes down together: one launch for both where the int8 kernel serves the rows
+            if (i == 1) continue;
+            hipError_t e = launch_gemv_q4k_tiled(stream, reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const float*>(input.ptr),
+                                                 reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(rows), static_cast<int>(in_dim),
+                                                 static_cast<int>(out_dim), ep, pair ? reinterpret_cast<float*>(dst_b.ptr) : nullptr,
+                                                 pair ? reinterpret_cast<const uint8_t*>(weight_b.ptr) : nullptr, ep_b);
+            if (e != hipSuccess) return static_cast<afhip_status>(e);
+            continue;
+        }
+        hipError_t e = launch_gemv_q4k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr), reinterpret_cast<const float*>(input.ptr),
+                                       reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr), static_cast<int>(rows),
+                                       static_cast<int>(in_dim), static_cast<int>(out_dim), i ? ep_b : ep);
         if (e != hipSuccess) return static_cast<afhip_status>(e);
     }
     return AFHIP_OK;

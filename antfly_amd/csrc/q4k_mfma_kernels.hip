@@ -460,12 +460,23 @@ __global__ __launch_bounds__(256) void q4k_digit_planes_kernel(const float* __re
 // kPlanesGiven: the digit planes, -s and the sub-block sums come from q4k_digit_planes_kernel (`frag`, `frag_scale`,
 // `frag_sums`) instead of being made here from `x`: the MFMA operand is then a 16-byte load per lane and sub-block,
 // requested with the weights, and nothing of X passes through LDS but the few floats of the wavefront's own slice.
+// A second matrix of the same shape on the same X (gate and up: grid.y = 2): one launch for both.
+struct Q4kSecond {
+    float* dst;
+    const uint8_t* weight;
+    Epilogue ep;
+};
+
 template <int kGroups, int kFlight, int kMaxThreads, bool kPlanesGiven = false>
-__global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst, const float* __restrict__ x,
-                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
-                                                                  int out_dim, int slices, int sb_per_slice, Epilogue ep,
+__global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 8 : 4) void gemv_q4k_i8_kernel(float* __restrict__ dst_a, const float* __restrict__ x,
+                                                                  const uint8_t* __restrict__ weight_a, int rows, int in_dim,
+                                                                  int out_dim, int slices, int sb_per_slice, Epilogue ep_a,
                                                                   const uint8_t* __restrict__ frag, const float* __restrict__ frag_scale,
-                                                                  const float* __restrict__ frag_sums) {
+                                                                  const float* __restrict__ frag_sums, Q4kSecond second) {
+    const bool is_b = blockIdx.y != 0;
+    float* dst = is_b ? second.dst : dst_a;
+    const uint8_t* weight = is_b ? second.weight : weight_a;
+    const Epilogue ep = is_b ? second.ep : ep_a;
     const int kb = in_dim >> 8;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -929,7 +940,12 @@ size_t q4k_mfma_lds_bytes(int rows, int in_dim, int waves, int groups) {
 
 template <int kGroups>
 hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                                int out_dim, const Epilogue& ep) {
+                                int out_dim, const Epilogue& ep, const Q4kSecond* second = nullptr) {
+    // a second matrix on the same X: one launch where the int8 kernel serves the rows, else one after the other
+    if (second != nullptr && kGroups > 2) {
+        if (hipError_t e = launch_q4k_mfma_rows<kGroups>(stream, dst, x, weight, rows, in_dim, out_dim, ep); e != hipSuccess) return e;
+        return launch_q4k_mfma_rows<kGroups>(stream, second->dst, x, second->weight, rows, in_dim, out_dim, second->ep);
+    }
     const int kb = in_dim / kQ4kBlockValues;
     const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
     // One or two rows: sixteen K slices per tile (one tile, sixteen wavefronts a workgroup) -- the
@@ -969,7 +985,7 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     if constexpr (kGroups <= 2) {
         if (use_i8) {
             if (tiles_per_wg != 1) return hipErrorInvalidValue;  // (a tuning knob asked for a shape this kernel does not have)
-            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue, const uint8_t*, const float*, const float*) = nullptr;
+            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue, const uint8_t*, const float*, const float*, Q4kSecond) = nullptr;
             if constexpr (kGroups == 1) {
                 switch (variant) {
                     case 0:
@@ -990,10 +1006,15 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
                     return e;
                 large_lds8[variant] = true;
             }
-            hipLaunchKernelGGL(k8, dim3(grid), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices, sb_per_slice, ep,
-                               static_cast<const uint8_t*>(nullptr), static_cast<const float*>(nullptr), static_cast<const float*>(nullptr));
+            hipLaunchKernelGGL(k8, dim3(grid, second ? 2 : 1), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices,
+                               sb_per_slice, ep, static_cast<const uint8_t*>(nullptr), static_cast<const float*>(nullptr),
+                               static_cast<const float*>(nullptr), second ? *second : Q4kSecond{nullptr, nullptr, Epilogue{}});
             return hipGetLastError();
         }
+    }
+    if (second != nullptr) {  // (the bf16 kernel: one matrix a launch)
+        if (hipError_t e = launch_q4k_mfma_rows<kGroups>(stream, dst, x, weight, rows, in_dim, out_dim, ep); e != hipSuccess) return e;
+        return launch_q4k_mfma_rows<kGroups>(stream, second->dst, x, second->weight, rows, in_dim, out_dim, second->ep);
     }
     void (*kernel)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue) = nullptr;
     switch (variant) {
@@ -1165,7 +1186,7 @@ hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows,
 }
 
 hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, int rows, int in_dim,
-                                   int out_dim, const Epilogue& ep) {
+                                   int out_dim, const Epilogue& ep, float* dst_b, const uint8_t* weight_b, const Epilogue& ep_b) {
     if (!q4k_i8_rows_supports(static_cast<size_t>(rows), static_cast<size_t>(in_dim)) || workspace == nullptr) return hipErrorInvalidValue;
     if (out_dim == 0) return hipSuccess;
     const int kb = in_dim / kQ4kBlockValues;
@@ -1178,25 +1199,27 @@ hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* w
     const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
     const size_t lds = q4k_i8_rows_lds_bytes(rows, in_dim, slices);
     const float* no_x = nullptr;
+    const Q4kSecond second{dst_b, weight_b, ep_b};
+    const dim3 grid(n_tiles, weight_b != nullptr ? 2 : 1);
     switch ((rows + 1) / 2) {
         case 2:
-            hipLaunchKernelGGL((gemv_q4k_i8_kernel<2, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<2, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
             break;
         case 3:
-            hipLaunchKernelGGL((gemv_q4k_i8_kernel<3, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<3, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
             break;
         default:
-            hipLaunchKernelGGL((gemv_q4k_i8_kernel<4, 1, 512, true>), dim3(n_tiles), dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums);
+            hipLaunchKernelGGL((gemv_q4k_i8_kernel<4, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
             break;
     }
     return hipGetLastError();
 }
 
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                                 int out_dim, const Epilogue& ep0) {
+                                 int out_dim, const Epilogue& ep0, float* dst_b, const uint8_t* weight_b, const Epilogue& ep_b0) {
     if (in_dim % kQ4kBlockValues != 0 || in_dim > gemv_q4k_max_in_dim()) return hipErrorInvalidValue;
     // as many rows per launch as LDS holds (three bf16 copies of each), at most eight
     const int per_launch = gemv_q4k_tiled_rows_per_launch(in_dim);
@@ -1208,12 +1231,15 @@ hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x,
         const float* xr = x + static_cast<size_t>(r0) * in_dim;
         Epilogue ep = ep0;
         if (ep.residual) ep.residual += static_cast<size_t>(r0) * out_dim;
+        Q4kSecond second{dst_b ? dst_b + static_cast<size_t>(r0) * out_dim : nullptr, weight_b, ep_b0};
+        if (second.ep.residual) second.ep.residual += static_cast<size_t>(r0) * out_dim;
+        const Q4kSecond* sec = weight_b != nullptr ? &second : nullptr;
         hipError_t e;
         switch ((nr + 1) / 2) {
-            case 1: e = launch_q4k_mfma_rows<1>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
-            case 2: e = launch_q4k_mfma_rows<2>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
-            case 3: e = launch_q4k_mfma_rows<3>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
-            default: e = launch_q4k_mfma_rows<4>(stream, d, xr, weight, nr, in_dim, out_dim, ep); break;
+            case 1: e = launch_q4k_mfma_rows<1>(stream, d, xr, weight, nr, in_dim, out_dim, ep, sec); break;
+            case 2: e = launch_q4k_mfma_rows<2>(stream, d, xr, weight, nr, in_dim, out_dim, ep, sec); break;
+            case 3: e = launch_q4k_mfma_rows<3>(stream, d, xr, weight, nr, in_dim, out_dim, ep, sec); break;
+            default: e = launch_q4k_mfma_rows<4>(stream, d, xr, weight, nr, in_dim, out_dim, ep, sec); break;
         }
         if (e != hipSuccess) return e;
     }

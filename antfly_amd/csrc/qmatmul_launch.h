@@ -166,16 +166,19 @@ hipError_t launch_quantize_q4k_rows(hipStream_t stream, uint8_t* dst_raw, const 
 // rows, and get_rows / cpy_q_to_f32.
 size_t q4k_tiled_bytes(size_t out_dim, size_t in_dim);
 hipError_t launch_q4k_tile_repack(hipStream_t stream, uint8_t* dst, const uint8_t* src_raw, int out_dim, int in_dim);
+// (dst_b / weight_b: a second matrix of the same shape on the same X -- one launch for both where the int8 kernel serves the rows)
 hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                                 int out_dim, const Epilogue& ep = Epilogue{});
+                                 int out_dim, const Epilogue& ep = Epilogue{}, float* dst_b = nullptr, const uint8_t* weight_b = nullptr,
+                                 const Epilogue& ep_b = Epilogue{});
 // Three to eight rows of Q4_K (tile-major layout) with scratch: launch_q4k_digit_planes writes X as fixed-point
 // digit planes in MFMA operand order into `workspace` (q4k_i8_rows_workspace_bytes, 16-byte aligned) once,
-// launch_gemv_q4k_i8_rows multiplies one matrix by them (a pair: two launches on the same planes).
+// launch_gemv_q4k_i8_rows multiplies one matrix, or a pair of them in one launch, by them.
 bool q4k_i8_rows_supports(size_t rows, size_t in_dim);
 size_t q4k_i8_rows_workspace_bytes(size_t in_dim);
 hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace);
 hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, int rows, int in_dim,
-                                   int out_dim, const Epilogue& ep);
+                                   int out_dim, const Epilogue& ep, float* dst_b = nullptr, const uint8_t* weight_b = nullptr,
+                                   const Epilogue& ep_b = Epilogue{});
 // More rows than one launch of the kernel above holds (gemv_q4k_tiled_rows_per_launch): X is split
 // once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned; it also holds the partial sums when a
 // small problem splits K over several workgroups) and a GEMM walks K for 32 rows
