@@ -184,12 +184,13 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
                 else if (kind == AFHIP_DISPATCH_SMALL_BATCH) counters->small_batch++;
                 else counters->mm++;
             }
-            if (fused) {
-                e = launch_linear_q4k_q8k_fused(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),
-                                                reinterpret_cast<const float*>(input.ptr),
-                                                reinterpret_cast<const uint8_t*>(i ? weight_b.ptr : weight.ptr),
-                                                static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
-                                                i ? ep_b : ep);
+            if (fused) {  // a pair: both matrices in one launch
+                if (i == 0)
+                    e = launch_linear_q4k_q8k_fused(stream, reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const float*>(input.ptr),
+                                                    reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(rows),
+                                                    static_cast<int>(in_dim), static_cast<int>(out_dim), ep,
+                                                    pair ? reinterpret_cast<float*>(dst_b.ptr) : nullptr,
+                                                    pair ? reinterpret_cast<const uint8_t*>(weight_b.ptr) : nullptr, ep_b);
                 continue;
             }
             e = launch_linear_q4k_q8k(stream, reinterpret_cast<float*>(i ? dst_b.ptr : dst.ptr),

@@ -612,12 +612,23 @@ __global__ __launch_bounds__(64) void linear_q4k_q8k_kernel(float* __restrict__ 
 // which is all it reads itself.  Its loads of X go out before the weight loads (loads retire in order),
 // and it quantizes while the weights are on their way.
 constexpr int kQ8kPassRows = 8;
+// A second matrix of the same shape on the same X (gate and up: grid.z = 2 of the fused launch).
+struct Q8kSecond {
+    float* dst;
+    const uint8_t* weight;
+    Epilogue ep;
+};
+
 template <int kFusedRows>
-__global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __restrict__ dst, const int8_t* __restrict__ q,
+__global__ __launch_bounds__(768) void linear_q4k_q8k_tiled_kernel(float* __restrict__ dst_a, const int8_t* __restrict__ q,
                                                                   const float* __restrict__ xd, const int* __restrict__ sums,
                                                                   const float* __restrict__ x,
-                                                                  const uint8_t* __restrict__ weight, int rows, int in_dim,
-                                                                  int out_dim, int rows_per_group, Epilogue ep) {
+                                                                  const uint8_t* __restrict__ weight_a, int rows, int in_dim,
+                                                                  int out_dim, int rows_per_group, Epilogue ep_a, Q8kSecond second) {
+    const bool is_b = blockIdx.z != 0;
+    float* dst = is_b ? second.dst : dst_a;
+    const uint8_t* weight = is_b ? second.weight : weight_a;
+    const Epilogue ep = is_b ? second.ep : ep_a;
     extern __shared__ __align__(16) unsigned char q8k_lds[];
     const int kb = in_dim / kQ4kBlockValues;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, threads = blockDim.x;
@@ -760,7 +771,8 @@ hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* wor
         const size_t lds = static_cast<size_t>(kQ8kPassRows) * in_dim + kQ8kPassRows * kb * 4 + kQ8kPassRows * kb * 32 +
                            static_cast<size_t>(kb) * 2 * kQ8kPassRows * 32 * 4;
         hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel<0>, dim3(tiles, groups), dim3(64 * kb), lds, stream, dst, q, d, sums,
-                           static_cast<const float*>(nullptr), weight, rows, in_dim, out_dim, rows_per_group, ep);
+                           static_cast<const float*>(nullptr), weight, rows, in_dim, out_dim, rows_per_group, ep,
+                           Q8kSecond{nullptr, nullptr, Epilogue{}});
     } else if (tiled)
         hipLaunchKernelGGL(linear_q4k_q8k_kernel<true>, dim3(out_dim), dim3(64), 0, stream, dst, q, d, sums, weight, rows, in_dim, out_dim, ep);
     else
@@ -773,7 +785,7 @@ bool linear_q4k_q8k_fuses_quantizer(bool tiled, size_t rows, size_t in_dim) {
 }
 
 hipError_t launch_linear_q4k_q8k_fused(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                                       int out_dim, const Epilogue& ep) {
+                                       int out_dim, const Epilogue& ep, float* dst_b, const uint8_t* weight_b, const Epilogue& ep_b) {
     if (rows == 0 || out_dim == 0) return hipSuccess;
     if (!linear_q4k_q8k_fuses_quantizer(true, static_cast<size_t>(rows), static_cast<size_t>(in_dim))) return hipErrorInvalidValue;
     const int kb = in_dim / kQ4kBlockValues;
@@ -781,9 +793,9 @@ hipError_t launch_linear_q4k_q8k_fused(hipStream_t stream, float* dst, const flo
     const size_t lds = static_cast<size_t>(kQ8kPassRows) * in_dim + kQ8kPassRows * kb * 4 + kQ8kPassRows * kb * 32 +
                        static_cast<size_t>(kb) * 2 * kQ8kPassRows * 32 * 4;
 #define AFHIP_Q8K_FUSED(R)                                                                                                   \
-    hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel<R>, dim3(tiles, 1), dim3(64 * kb), lds, stream, dst,                       \
+    hipLaunchKernelGGL(linear_q4k_q8k_tiled_kernel<R>, dim3(tiles, 1, weight_b ? 2 : 1), dim3(64 * kb), lds, stream, dst,     \
                        static_cast<const int8_t*>(nullptr), static_cast<const float*>(nullptr), static_cast<const int*>(nullptr), x, \
-                       weight, rows, in_dim, out_dim, kQ8kPassRows, ep)
+                       weight, rows, in_dim, out_dim, kQ8kPassRows, ep, Q8kSecond{dst_b, weight_b, ep_b})
     if (rows == 1) AFHIP_Q8K_FUSED(1);
     else if (rows == 2) AFHIP_Q8K_FUSED(2);
     else AFHIP_Q8K_FUSED(4);

@@ -152,7 +152,8 @@ hipError_t launch_linear_q4k_q8k(hipStream_t stream, float* dst, const void* wor
 // (same bits as the two launches; `workspace` is not touched).
 bool linear_q4k_q8k_fuses_quantizer(bool tiled, size_t rows, size_t in_dim);
 hipError_t launch_linear_q4k_q8k_fused(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
-                                       int out_dim, const Epilogue& ep);
+                                       int out_dim, const Epilogue& ep, float* dst_b = nullptr, const uint8_t* weight_b = nullptr,
+                                       const Epilogue& ep_b = Epilogue{});  // (dst_b / weight_b: a second matrix in the same launch)
 hipError_t launch_gemv_q4k(hipStream_t stream, float* dst, const float* x, const uint8_t* weight, int rows, int in_dim,
                            int out_dim, const Epilogue& ep = Epilogue{});
 hipError_t launch_dequantize_q4k_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
