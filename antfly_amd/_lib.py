@@ -136,7 +136,8 @@ SIGNATURES = {
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_launch_stream_copy": (_st, [_vp, Buffer, Buffer]),
-    "afhip_launch_rate_probe": (_st, [_vp, _i, _i, _i, Buffer]),
+    "afhip_launch_rate_probe": (_st, [_vp, _i, _i, _i, Buffer, Buffer]),
+    "afhip_rate_probe_wavefronts": (_sz, [_i]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),
     "afhip_compute_destroy": (None, [_vp]),
     "afhip_compute_backend_kind": (_i, [_vp]),

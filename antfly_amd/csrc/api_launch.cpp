@@ -959,13 +959,21 @@ afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, 
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
-afhip_status afhip_launch_rate_probe(void* stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink) {
-    if (pattern < 0 || pattern > 11 || wavefronts_per_simd < 1 || wavefronts_per_simd > 8 || iterations < 1 || iterations > (1 << 20))
+afhip_status afhip_launch_rate_probe(void* stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink,
+                                     afhip_buffer stamps) {
+    if (pattern < 0 || pattern > 20 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2 && wavefronts_per_simd != 4) ||
+        iterations < 1 || iterations > (1 << 20))
         return AFHIP_ERR_INVALID_ARGUMENT;
-    if (sink.ptr == 0 || sink.ptr % 4 != 0 || sink.len < 65536 * 4) return AFHIP_ERR_INVALID_STATE;
+    if (sink.ptr == 0 || sink.ptr % 16 != 0 || sink.len < 65536 * 4 + (2u << 20) + 8192) return AFHIP_ERR_INVALID_STATE;
+    if (stamps.ptr == 0 || stamps.ptr % 4 != 0 || stamps.len < afhip_rate_probe_wavefronts(wavefronts_per_simd) * 16)
+        return AFHIP_ERR_INVALID_STATE;
     hipError_t e = launch_rate_probe(static_cast<hipStream_t>(stream), pattern, wavefronts_per_simd, iterations,
-                                     reinterpret_cast<int*>(sink.ptr));
+                                     reinterpret_cast<int*>(sink.ptr), reinterpret_cast<uint32_t*>(stamps.ptr));
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+size_t afhip_rate_probe_wavefronts(int wavefronts_per_simd) {
+    return wavefronts_per_simd < 1 ? 0 : static_cast<size_t>(rate_probe_wavefronts(wavefronts_per_simd));
 }
 
 afhip_status afhip_launch_decode_fp16(void* stream, afhip_buffer dst, afhip_buffer src, size_t n) {

@@ -375,51 +375,75 @@ def main() -> int:
         return 0
 
     if args.probe == "rates":
+        import numpy as np
         lib = _lib.lib()
-        sink = torch.zeros(65536, dtype=torch.int32, device=dev)
-        iterations = 4000
-        clock_ghz = 2.4  # MI355X peak engine clock; the clock a run really holds is not read here
-        patterns = [(0, "v_fma_f32 x 16", 16), (1, "v_mul_f32 x 16", 16), (2, "v_add_u32 x 16", 16), (3, "v_cvt_f32_i32 x 16", 16),
-                    (4, "v_dot8_u32_u4 x 16", 16), (5, "v_dot8_i32_i4 x 16", 16), (6, "v_dot4_i32_i8 x 16", 16),
-                    (7, "v_mfma_i32_32x32x32_i8 x 4", 4), (8, "4 x (MFMA + 4 v_fma_f32), one wavefront", 4),
-                    (9, "4 x (MFMA + 8 v_fma_f32), one wavefront", 4)]
-        mixed = [(7, 1, "MFMA x 4 alone, 1 wavefront per SIMD"), (0, 1, "v_fma_f32 x 16 alone, 1 wavefront per SIMD"),
-                 (3, 1, "v_cvt_f32_i32 x 16 alone, 1 wavefront per SIMD"),
-                 (10, 2, "a wavefront of MFMA x 4 beside a wavefront of v_fma_f32 x 16 on each SIMD"),
-                 (11, 2, "a wavefront of MFMA x 4 beside a wavefront of v_cvt_f32_i32 x 16 on each SIMD"),
-                 (7, 2, "MFMA x 4, 2 wavefronts per SIMD")]
+        sink = torch.zeros(65536 + (2 << 18) + 2048, dtype=torch.int32, device=dev)
+        iterations = 2000
+        # (pattern, name, instructions the "per instruction" column divides by, wavefronts per SIMD to run)
+        patterns = [
+            (0, "32 v_fma_f32", 32, (1, 2, 4)),
+            (1, "32 v_cvt_f32_i32", 32, (1, 2, 4)),
+            (2, "32 v_sub_f32", 32, (1, 2, 4)),
+            (3, "16 x (v_cvt_f32_i32 -> v_fma_f32 that consumes it)", 32, (1, 2, 4)),
+            (4, "4 v_mfma_i32_32x32x32_i8", 4, (1, 2, 4)),
+            (5, "2 v_mfma_f32_32x32x1_2b_f32", 2, (1, 2, 4)),
+            (6, "4 x (int8 MFMA + 8 v_fma_f32), one wavefront", 4, (1, 2, 4)),
+            (7, "4 x (int8 MFMA + 8 cvt + 8 fma), one wavefront", 4, (1, 2, 4)),
+            (8, "4 x (int8 MFMA + 16 cvt + 16 fma), one wavefront", 4, (1, 2, 4)),
+            (9, "GEMM recipe, 4 tile-blocks: 4 int8 MFMA + 2 f32 rank-1 MFMA + 64 cvt + 64 fma, two register sets", 4, (1, 2)),
+            (10, "the same with v_sub_f32 for the conversion", 4, (1, 2)),
+            (13, "4 tile-blocks: 4 int8 MFMA + 4 f32 rank-1 MFMA + 64 fma (bias term on the matrix pipe)", 4, (1, 2)),
+            (11, "wavefronts 0-3: 4 int8 MFMA; wavefronts 4+: 32 v_fma_f32", 1, (2, 4)),
+            (12, "wavefronts 0-3: 4 int8 MFMA; wavefronts 4+: 32 v_cvt_f32_i32", 1, (2,)),
+            (15, "4 tile-blocks on one register set: 2 x (2 int8 MFMA + 1 f32 rank-1 MFMA, wait, 32 cvt + 32 fma)", 4, (1, 2, 4)),
+            (14, "8 ds_read_b128 (1 KiB each per wavefront, lane l at byte 16 l), waited for together", 8, (1, 2, 4)),
+            (16, "8 ds_read_b128 of MFMA fragments from XOR-swizzled 128-byte rows", 8, (1, 2, 4)),
+            (17, "8 global_load_lds_dwordx4 (1 KiB each per wavefront, from L2), waited for together", 8, (1, 2, 4)),
+            (18, "8 global_load_lds_dword (256 B each per wavefront)", 8, (1, 2, 4)),
+            (19, "8 global_load_lds_ushort (128 B each per wavefront)", 8, (1, 2, 4)),
+            (20, "8 global_load_dwordx4 to registers, wait, 8 ds_write_b128", 8, (1, 2, 4)),
+        ]
 
         def run(pattern, waves):
-            times = []
-            for _ in range(4):
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                rc = lib.afhip_launch_rate_probe(stream, pattern, waves, iterations, buf(sink))
-                e1.record()
-                torch.cuda.synchronize()
+            n = int(lib.afhip_rate_probe_wavefronts(waves))
+            stamps = torch.zeros((n, 4), dtype=torch.int32, device=dev)
+            for _ in range(2):  # the first launch warms the clocks up
+                rc = lib.afhip_launch_rate_probe(stream, pattern, waves, iterations, buf(sink), buf(stamps))
                 if rc != 0:
                     raise RuntimeError(f"rate probe failed: {rc}")
-                times.append(e0.elapsed_time(e1))
-            return sorted(times[1:])[1]  # ms; the first launch is warm-up
+                torch.cuda.synchronize()
+            return stamps.cpu().numpy().view(np.uint32).astype(np.int64)
 
-        print(f"shader clock taken as {clock_ghz:.2f} GHz (the published peak engine clock); {iterations} rounds per wavefront")
-        print("| pattern (one round) | wavefronts per SIMD | ms | cycles per round and wavefront | cycles per instruction and SIMD |")
-        print("|---|---|---|---|---|")
+        def placement(st):
+            hw, xcc = st[:, 2], st[:, 3] & 0xF
+            # HW_ID (gfx9 layout): simd [5:4], cu [11:8], sh [12], se [15:13]
+            key = (xcc << 12) | (((hw >> 13) & 7) << 8) | (((hw >> 12) & 1) << 7) | (((hw >> 8) & 0xF) << 2) | ((hw >> 4) & 3)
+            return key
+
+        print(f"{iterations} rounds per wavefront; cycles = s_memtime differences read by the wavefronts, clock = cycles / (s_memrealtime ticks / 100 MHz)")
+        print("| pattern (one round) | wavefronts per SIMD | cycles per round and wavefront (median; min-max) | SIMD cycles per instruction | clock GHz | SIMDs hosting exactly that many wavefronts |")
+        print("|---|---|---|---|---|---|")
         out = {}
-        for pattern, name, per_round in patterns:
-            for waves in (1, 2, 4):
-                ms = run(pattern, waves)
-                per_wave_round = ms * 1e6 * clock_ghz / iterations
-                print(f"| {name} | {waves} | {ms:.3f} | {per_wave_round:.1f} | {per_wave_round / waves / per_round:.2f} |")
-                out[f"{name} @{waves}"] = round(ms, 4)
-        print()
-        print("| two kinds of wavefront on a SIMD | ms |")
-        print("|---|---|")
-        for pattern, waves, name in mixed:
-            ms = run(pattern, waves)
-            print(f"| {name} | {ms:.3f} |")
-            out[name] = round(ms, 4)
-        print(json.dumps({"probe": "rates", "ms": out}))
+        for pattern, name, per_round, wave_counts in patterns:
+            for waves in wave_counts:
+                st = run(pattern, waves)
+                key = placement(st)
+                simds, counts = np.unique(key, return_counts=True)
+                exact = int((counts == waves).sum())
+                ghz = float(np.median(st[:, 0] / (st[:, 1] / 100e6))) / 1e9
+                if pattern in (11, 12):
+                    # two roles: report each
+                    wave_in_group = np.arange(st.shape[0]) % (4 * waves)
+                    for role, sel in (("MFMA wavefronts", wave_in_group < 4), ("vector wavefronts", wave_in_group >= 4)):
+                        cyc = st[sel, 0] / iterations
+                        print(f"| {name} -- {role} | {waves} | {np.median(cyc):.1f}; {cyc.min():.1f}-{cyc.max():.1f} | | {ghz:.3f} | {exact} of {len(simds)} |")
+                        out[f"{name} -- {role} @{waves}"] = round(float(np.median(cyc)), 2)
+                    continue
+                cyc = st[:, 0] / iterations
+                med = float(np.median(cyc))
+                print(f"| {name} | {waves} | {med:.1f}; {cyc.min():.1f}-{cyc.max():.1f} | {med / waves / per_round:.2f} | {ghz:.3f} | {exact} of {len(simds)} |")
+                out[f"{name} @{waves}"] = round(med, 2)
+        print(json.dumps({"probe": "rates", "cycles_per_round": out}))
         return 0
 
     if args.probe == "gemv":

@@ -332,15 +332,19 @@ afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buff
  * --probe gemv times the eight variants to show where a launch's time goes. */
 afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
-/* Diagnostic with no counterpart in the reference: instruction issue rates.  Puts
- * `wavefronts_per_simd` (1..8) wavefronts on every SIMD, each running `iterations` rounds of
- * pattern 0..6 (16 independent v_fma_f32 / v_mul_f32 / v_add_u32 / v_cvt_f32_i32 /
- * v_dot8_u32_u4 / v_dot8_i32_i4 / v_dot4_i32_i8), 7 (four v_mfma_i32_32x32x32_i8), 8 / 9 (four
- * times one MFMA followed by 4 / 8 independent v_fma_f32 in the same wavefront) or 10 / 11
- * (alternate workgroups run pattern 7 and pattern 0 / 3: with two wavefronts per SIMD, one that
- * only issues MFMAs beside one that only issues vector-ALU work).  `sink` takes 256 KiB of
- * meaningless results.  `bench.py --probe rates` times it. */
-afhip_status afhip_launch_rate_probe(void *stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink);
+/* Diagnostic with no counterpart in the reference: what instruction patterns cost a SIMD, timed
+ * by the wavefronts themselves.  One workgroup of 256 x `wavefronts_per_simd` (1, 2 or 4) threads
+ * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 20, listed in
+ * csrc/rate_probe_kernels.hip: vector-ALU instructions, int8 and f32 MFMAs, their mixes inside one
+ * wavefront and side by side in two) and stores four 32-bit words into `stamps`
+ * [wavefront][4]: shader-clock cycles of its loop, 100 MHz reference ticks of its loop, the
+ * HW_ID register and the XCC_ID register (where it ran).  afhip_rate_probe_wavefronts() says how
+ * many wavefronts a launch has.  `sink` (16-byte aligned, 256 KiB + 2 MiB + 8 KiB) takes meaningless
+ * results and is what the load patterns read.
+ * `bench.py --probe rates` prints the table. */
+afhip_status afhip_launch_rate_probe(void *stream, int pattern, int wavefronts_per_simd, int iterations,
+                                     afhip_buffer sink, afhip_buffer stamps);
+size_t afhip_rate_probe_wavefronts(int wavefronts_per_simd);
 
 /* ------------------------------------------------------------------------
  * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
