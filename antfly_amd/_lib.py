@@ -136,6 +136,7 @@ SIGNATURES = {
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_launch_stream_copy": (_st, [_vp, Buffer, Buffer]),
+    "afhip_launch_gemm_stamps": (_st, [_vp, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
     "afhip_launch_rate_probe": (_st, [_vp, _i, _i, _i, Buffer, Buffer]),
     "afhip_rate_probe_wavefronts": (_sz, [_i]),
     "afhip_compute_create": (_st, [C.POINTER(_vp)]),

@@ -959,6 +959,25 @@ afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, 
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_gemm_stamps(void* stream, afhip_buffer stamps, afhip_buffer q, afhip_buffer scales,
+                                      afhip_buffer weight_prepared, size_t rows, size_t in_dim, size_t out_dim) {
+    if (rows == 0 || rows > 0x7fffffff || in_dim == 0 || in_dim % 32 != 0 || in_dim > 0x7fffffff || out_dim == 0 ||
+        out_dim > 0x7fffffff)
+        return AFHIP_ERR_INVALID_STATE;
+    const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q8_0, out_dim, in_dim);
+    if (need == 0 || weight_prepared.len < need || q.len < rows * in_dim || scales.len < rows * (in_dim / 32) * 4 ||
+        stamps.len < rows * out_dim * 4)
+        return AFHIP_ERR_INVALID_STATE;
+    if (stamps.ptr == 0 || q.ptr == 0 || scales.ptr == 0 || weight_prepared.ptr == 0 || stamps.ptr % 4 != 0 ||
+        q.ptr % 16 != 0 || scales.ptr % 4 != 0 || weight_prepared.ptr % 16 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_gemm_i8_stamps(static_cast<hipStream_t>(stream), reinterpret_cast<float*>(stamps.ptr),
+                                         reinterpret_cast<const int8_t*>(q.ptr), reinterpret_cast<const float*>(scales.ptr),
+                                         reinterpret_cast<const uint8_t*>(weight_prepared.ptr), static_cast<int>(rows),
+                                         static_cast<int>(in_dim), static_cast<int>(out_dim));
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_rate_probe(void* stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink,
                                      afhip_buffer stamps) {
     if (pattern < 0 || pattern > 20 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2 && wavefronts_per_simd != 4) ||

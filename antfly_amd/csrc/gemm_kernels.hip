@@ -127,7 +127,11 @@ extern __shared__ __align__(16) unsigned char gemm_lds[];
 
 // kShareK: this launch walks only a share of K per workgroup (see below); a template parameter
 // so that the ordinary kernel carries none of it.
-template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots, bool kShareK = false>
+// kStamps (diagnostic): the kernel computes as usual but, instead of results, every wavefront stores eight
+// 32-bit counts over the start of dst, [8 * (workgroup * wavefronts + wavefront)]: shader-clock cycles before
+// the K loop, in it, waiting for its own loads, waiting at the workgroup barrier, 100 MHz reference ticks
+// spent in the loop (cycles / ticks = the clock the chip held), cycles after the loop, 0, and the HW_ID register.
+template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots, bool kShareK = false, bool kStamps = false>
 __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
@@ -369,6 +373,8 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
     // in one place and spills their results.
     auto pin_acc = [&]() { asm volatile("" : "+v"(acc) : : "memory"); };
 
+    uint64_t stamp_begin = 0, stamp_loop = 0, stamp_tail = 0, ref_loop = 0, ref_tail = 0, stamp_wait = 0, stamp_barrier = 0;
+    if (kStamps) stamp_begin = __builtin_readcyclecounter();
     // ---- prologue: stages 0 .. kRing-2 in flight, stages 0 and 1 landed, stage 0 in registers
     static_assert(kRing == 4, "the loop reads stage st + 1 while stage st + 2 lands and stage st + 3 is issued");
 #pragma unroll
@@ -383,6 +389,10 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
         // The next stage's operands are read from LDS while this stage's arithmetic runs.
         Frag frag[2];
         read_frag(0, frag[0]);
+        if (kStamps) {
+            stamp_loop = __builtin_readcyclecounter();
+            ref_loop = __builtin_amdgcn_s_memrealtime();
+        }
         for (int st0 = 0; st0 < stages; st0 += kRing) {
 #pragma unroll
             for (int d = 0; d < kRing; ++d) {
@@ -394,11 +404,22 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
                 pin_acc();
                 // stage st + 2 (issued two stages ago) has to be complete before the barrier:
                 // the next stage reads its operands
+                uint64_t s0 = 0, s1 = 0;
+                if (kStamps) s0 = __builtin_readcyclecounter();
                 wait_vm_outstanding(loads_per_stage);
                 expand_q4((d + 2) % kRing);
+                if (kStamps) s1 = __builtin_readcyclecounter();
                 __syncthreads();
+                if (kStamps) {
+                    stamp_wait += s1 - s0;
+                    stamp_barrier += __builtin_readcyclecounter() - s1;
+                }
             }
         }
+    }
+    if (kStamps) {
+        stamp_tail = __builtin_readcyclecounter();
+        ref_tail = __builtin_amdgcn_s_memrealtime();
     }
 
     // Loads still in flight target ring slots nobody reads again; they must land before
@@ -421,11 +442,25 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
 #pragma unroll
             for (int k2 = 1; k2 < kSplit; ++k2) sum += red[((k2 * S::kTiles + tile) * 16 + v) * 64 + lane];
             const int m = m0 + wm * 32 + 8 * (v >> 2) + 4 * lh + (v & 3);
-            if (m < rows && n < out_dim) {
+            if (kStamps) {
+                asm volatile("" : : "v"(sum));  // the sum is formed, not stored
+            } else if (m < rows && n < out_dim) {
                 const size_t at = static_cast<size_t>(m) * out_dim + n;
                 if (kShareK) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
                 else dst[at] = finish_output(ep, n, at, sum);
             }
+        }
+        if (kStamps && lane == 0) {
+            const uint64_t stamp_end = __builtin_readcyclecounter();
+            int* out = reinterpret_cast<int*>(dst) + 8 * (static_cast<size_t>(blockIdx.x) * kWaves + wave);
+            out[0] = static_cast<int>(stamp_loop - stamp_begin);
+            out[1] = static_cast<int>(stamp_tail - stamp_loop);
+            out[2] = static_cast<int>(stamp_wait);
+            out[3] = static_cast<int>(stamp_barrier);
+            out[4] = static_cast<int>(ref_tail - ref_loop);
+            out[5] = static_cast<int>(stamp_end - stamp_tail);
+            out[6] = 0;
+            out[7] = static_cast<int>(__builtin_amdgcn_s_getreg((31 << 11) | 4));
         }
     } else {
         if (dst == nullptr) return;
@@ -539,6 +574,25 @@ hipError_t launch_splitk_reduce(hipStream_t stream, float* dst, const float* par
     if (grid > 4096) grid = 4096;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, dst, partial, count, out_dim,
                        shares, ep);
+    return hipGetLastError();
+}
+
+// Diagnostic: the Q8_0 64 x 128 tile kernel with its clock readings in place of results (see kStamps); dst has to
+// hold 8 ints per wavefront of the grid, which it does whenever it holds the rows x out_dim results.
+hipError_t launch_gemm_i8_stamps(hipStream_t stream, float* dst, const int8_t* qx, const float* sx, const uint8_t* weight,
+                                 int rows, int in_dim, int out_dim) {
+    using S = GemmShape<2, 4, 2, false>;
+    const int m_tiles = (rows + S::kTM - 1) / S::kTM, n_tiles = (out_dim + S::kTN - 1) / S::kTN;
+    const long long grid = static_cast<long long>((n_tiles + 7) / 8) * m_tiles * 8;
+    if (grid > 0x7fffffffLL || static_cast<long long>(S::kTN) * in_dim > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (static_cast<long long>(rows) * out_dim < grid * S::kWaves * 8) return hipErrorInvalidValue;
+    auto kernel = gemm_i8_kernel<8, 2, 4, 2, false, false, true>;
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           S::kLdsBytes);
+        e != hipSuccess)
+        return e;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(S::kThreads), S::kLdsBytes, stream, dst, nullptr, qx, sx,
+                       weight, rows, in_dim, out_dim, m_tiles, n_tiles, in_dim / 32, nullptr, Epilogue{});
     return hipGetLastError();
 }
 

@@ -108,6 +108,8 @@ hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned
 // `partial` (optional, gemm_i8_partial_bytes() bytes): lets a launch whose tiles would leave
 // compute units idle share K out over more workgroups (gemm_i8_splits() shares, partial sums
 // added in share order by a second kernel).
+hipError_t launch_gemm_i8_stamps(hipStream_t stream, float* dst, const int8_t* qx, const float* sx, const uint8_t* weight,
+                                 int rows, int in_dim, int out_dim);
 hipError_t launch_gemm_i8(hipStream_t stream, int tensor_type, float* dst, int* dots, const int8_t* qx, const float* sx,
                           const uint8_t* weight_prepared, int rows, int in_dim, int out_dim,
                           const Epilogue& ep = Epilogue{}, float* partial = nullptr);

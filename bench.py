@@ -75,8 +75,8 @@ def main() -> int:
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k; q4p / q8p: pair calls): time only these calls, print one line each, exit")
-    ap.add_argument("--probe", choices=["gemv", "rates"], default=None,
-                    help="rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+    ap.add_argument("--probe", choices=["gemv", "rates", "gemm"], default=None,
+                    help="gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -444,6 +444,45 @@ def main() -> int:
                 print(f"| {name} | {waves} | {med:.1f}; {cyc.min():.1f}-{cyc.max():.1f} | {med / waves / per_round:.2f} | {ghz:.3f} | {exact} of {len(simds)} |")
                 out[f"{name} @{waves}"] = round(med, 2)
         print(json.dumps({"probe": "rates", "cycles_per_round": out}))
+        return 0
+
+    if args.probe == "gemm":
+        import numpy as np
+        lib = _lib.lib()
+        m, k, n = 512, 4096, 4096
+        ws = prepared_copies(Q8, n, k, 4, 7)
+        x = torch.from_numpy(synth.activations(8, m, k)).to(dev)
+        q = torch.empty(m * k, dtype=torch.int8, device=dev)
+        sc = torch.empty(m * k // 32, dtype=torch.float32, device=dev)
+        sm = torch.empty(m * k // 32, dtype=torch.int32, device=dev)
+        y = torch.zeros((m, n), dtype=torch.float32, device=dev)
+        kernels.launchQuantizeActivations(stream, buf(x), m, k, buf(q), buf(sc), buf(sm))
+        launches = 300  # back to back, so that the clocks are those of a sustained run; the last launch is read
+        for i in range(launches):
+            rc = lib.afhip_launch_gemm_stamps(stream, buf(y), buf(q), buf(sc), buf(ws[i % 4]), m, k, n)
+            if rc != 0:
+                raise RuntimeError(f"gemm stamps failed: {rc}")
+        torch.cuda.synchronize()
+        groups = ((n + 127) // 128 + 7) // 8 * ((m + 63) // 64) * 8
+        st = y.cpu().numpy().reshape(-1).view(np.int32)[: groups * 16 * 8].reshape(groups, 16, 8).astype(np.int64)
+        ghz = float(np.median(st[:, :, 1] / (st[:, :, 4] / 100e6))) / 1e9
+        print(f"Q8_0 prefill kernel, M={m}, K={k}, N={n}: {groups} workgroups x 16 wavefronts, launch {launches} of {launches} back to back")
+        print(f"clock held in the K loop: {ghz:.3f} GHz (loop cycles / 100 MHz reference ticks, median over wavefronts)")
+        print("| per wavefront, shader-clock cycles | median | min | max |")
+        print("|---|---|---|---|")
+        for name, col in (("before the K loop", 0), ("K loop", 1), ("... of which waiting for its own loads", 2),
+                          ("... of which waiting at the workgroup barrier", 3), ("after the K loop", 5)):
+            v = st[:, :, col]
+            print(f"| {name} | {int(np.median(v))} | {v.min()} | {v.max()} |")
+        print("| wavefront of the workgroup (launch order = age on its SIMD) | K loop | waiting at barriers |")
+        print("|---|---|---|")
+        for wv in range(16):
+            print(f"| {wv} | {int(np.median(st[:, wv, 1]))} | {int(np.median(st[:, wv, 3]))} |")
+        tile_blocks = (m // 32) * (n // 32) * (k // 32) / (groups * 4)  # per SIMD
+        print(f"tile-blocks (32 x 32 outputs x one 32-value block) per SIMD: {tile_blocks:.0f}; loop cycles per tile-block and SIMD: "
+              f"{float(np.median(st[:, :, 1])) / tile_blocks:.0f}")
+        print(json.dumps({"probe": "gemm", "clock_ghz": round(ghz, 3), "loop_cycles_median": int(np.median(st[:, :, 1])),
+                          "barrier_cycles_median": int(np.median(st[:, :, 3])), "load_wait_cycles_median": int(np.median(st[:, :, 2]))}))
         return 0
 
     if args.probe == "gemv":

@@ -332,6 +332,14 @@ afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buff
  * --probe gemv times the eight variants to show where a launch's time goes. */
 afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* Diagnostic with no counterpart in the reference: the Q8_0 prefill kernel (64 x 128 tiles) on activations
+ * already quantized by afhip_launch_quantize_activations, computing as usual but storing, instead of results,
+ * eight 32-bit counts per wavefront over the start of `stamps` (which has to hold rows x out_dim floats):
+ * [8 * (workgroup * 16 + wavefront)] = shader-clock cycles before the K loop, in it, waiting for the wavefront's
+ * own loads, waiting at the workgroup barrier, 100 MHz reference ticks in the loop, cycles after the loop, 0, HW_ID.
+ * `bench.py --probe gemm` prints them. */
+afhip_status afhip_launch_gemm_stamps(void *stream, afhip_buffer stamps, afhip_buffer q, afhip_buffer scales,
+                                      afhip_buffer weight_prepared, size_t rows, size_t in_dim, size_t out_dim);
 /* Diagnostic with no counterpart in the reference: what instruction patterns cost a SIMD, timed
  * by the wavefronts themselves.  One workgroup of 256 x `wavefronts_per_simd` (1, 2 or 4) threads
  * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 20, listed in
