@@ -34,6 +34,8 @@ ERR_IO = -18
 TYPE_F32, TYPE_Q4_0, TYPE_Q8_0, TYPE_Q4_K = 0, 2, 8, 12
 ACTIVATION_NONE, ACTIVATION_RELU, ACTIVATION_QUICK_GELU, ACTIVATION_GELU = 0, 1, 2, 3
 LAYOUT_RAW, LAYOUT_PREPARED = 0, 1
+# a launcher's `dispatch` besides a kind (0 .. 3): choose by rows; ... and keep Q4_K on f32 activations everywhere
+DISPATCH_AUTO, DISPATCH_AUTO_F32_ACTIVATIONS = -1, -2
 DTYPE_F32, DTYPE_U8 = 0, 1
 
 
@@ -136,6 +138,7 @@ SIGNATURES = {
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_launch_stream_copy": (_st, [_vp, Buffer, Buffer]),
+    "afhip_tune_batch32_max_workgroups": (_st, [C.c_long]),
     "afhip_launch_gemm_stamps": (_st, [_vp, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
     "afhip_launch_rate_probe": (_st, [_vp, _i, _i, _i, Buffer, Buffer]),
     "afhip_rate_probe_wavefronts": (_sz, [_i]),
@@ -188,6 +191,7 @@ SIGNATURES = {
     "afhip_compute_load_gguf": (_st, [_vp, _vp, _i, C.POINTER(_sz), C.POINTER(_sz)]),
     "afhip_compute_debug_stats": (_st, [_vp, C.POINTER(DebugStats)]),
     "afhip_compute_set_phase_timing": (_st, [_vp, _i]),
+    "afhip_compute_set_q4k_f32_activations": (_st, [_vp, _i]),
     "afhip_smoke_q8_0": (_st, []),
     "afhip_smoke_q4_0": (_st, []),
 }

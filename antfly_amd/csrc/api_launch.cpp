@@ -149,7 +149,10 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
                                     const Epilogue& ep, const Epilogue& ep_b) {
     const bool pair = weight_b.ptr != 0 || dst_b.ptr != 0;
     if (want_dots) return AFHIP_ERR_INVALID_ARGUMENT;  // the block-dot output exists for the 32-value formats only
-    if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (dispatch < AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    // f32 activations everywhere (what the engine's accelerator backends compute), also on the CPU engine's gated shapes
+    const bool f32_everywhere = dispatch == AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS;
+    if (f32_everywhere) dispatch = AFHIP_DISPATCH_AUTO;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
     if (in_dim == 0 || in_dim % 256 != 0) return AFHIP_ERR_INVALID_STATE;
     const bool tiled = layout == AFHIP_LAYOUT_PREPARED;
@@ -169,12 +172,13 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     if (pair && (dst_b.ptr == 0 || weight_b.ptr == 0 || dst_b.ptr % 4 != 0 || weight_b.ptr % 16 != 0))
         return AFHIP_ERR_INVALID_STATE;
     const int kind = dispatch >= 0 ? dispatch : afhip_quant_matmul_select(rows, in_dim, out_dim, AFHIP_FORMAT_Q4_K);
-    if (afhip_uses_q8k_activation_quant(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim)) {
+    if (!f32_everywhere && afhip_uses_q8k_activation_quant(AFHIP_TYPE_Q4_K, rows, in_dim, out_dim)) {
         // the CPU engine's gated shapes: activations quantized to Q8_K, integer sub-block dots
-        if (workspace.ptr == 0 || workspace.ptr % 16 != 0 || workspace.len < q4k_q8k_workspace_bytes(rows, in_dim))
+        const bool fused = linear_q4k_q8k_fuses_quantizer(tiled, rows, in_dim);  // decode: the quantizer inside the matmul launch
+        // (which reads no workspace; the stand-alone quantizer writes the Q8_K rows there)
+        if (!fused && (workspace.ptr == 0 || workspace.ptr % 16 != 0 || workspace.len < q4k_q8k_workspace_bytes(rows, in_dim)))
             return AFHIP_ERR_INVALID_STATE;
         if (counters) counters->activation_quant++;
-        const bool fused = linear_q4k_q8k_fuses_quantizer(tiled, rows, in_dim);  // decode: the quantizer inside the matmul launch
         hipError_t e = fused ? hipSuccess
                              : launch_quantize_q8k(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
                                                    static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
@@ -310,7 +314,8 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
     const size_t bb = block_bytes(tensor_type);
     if (bb == 0) return AFHIP_ERR_UNSUPPORTED_TENSOR_TYPE;
     if (layout != AFHIP_LAYOUT_RAW && layout != AFHIP_LAYOUT_PREPARED) return AFHIP_ERR_INVALID_ARGUMENT;
-    if (dispatch < -1 || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (dispatch < AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS || dispatch > AFHIP_DISPATCH_MM) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (dispatch == AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS) dispatch = AFHIP_DISPATCH_AUTO;  // a Q4_K matter: the same as auto here
     if (in_dim == 0 || in_dim % 32 != 0) return AFHIP_ERR_INVALID_STATE;
     const size_t kb = in_dim / 32;
     size_t out_count, in_count, w_blocks, w_bytes, bytes;
@@ -957,6 +962,11 @@ afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, 
                                      reinterpret_cast<const float*>(input.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
                                      static_cast<int>(in_dim), static_cast<int>(out_dim));
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_tune_batch32_max_workgroups(long bound) {
+    set_batch32_max_workgroups(bound);
+    return AFHIP_OK;
 }
 
 afhip_status afhip_launch_gemm_stamps(void* stream, afhip_buffer stamps, afhip_buffer q, afhip_buffer scales,

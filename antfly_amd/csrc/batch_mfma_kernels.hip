@@ -36,6 +36,8 @@
 //     workgroup per compute unit.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstdlib>
 #include <type_traits>
 
@@ -989,6 +991,10 @@ size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, s
     return (front + 255) / 256 * 256 + (shares > 1 ? 2 * shares * rows * out_dim * 4 : 0);  // (twice: a pair of matrices)
 }
 
+// Largest grid the 32-row kernel is chosen for; negative: one workgroup per compute unit.
+static std::atomic<long> batch32_bound{-1};
+void set_batch32_max_workgroups(long bound) { batch32_bound.store(bound, std::memory_order_relaxed); }
+
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
                              int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b,
                              const uint8_t* weight_b_prepared, const Epilogue& ep, const Epilogue& ep_b) {
@@ -1008,10 +1014,10 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     // Nine to 64 rows on a matrix wide enough for 64-column tiles (and rows of whole 16-byte runs of
     // scales), with no more workgroups than compute units: batch32_mfma_kernel holds one workgroup per
     // unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
-    // unit (N = 20480: 21.1 against 18.5 us).  AFHIP_BATCH32_MAX_WORKGROUPS overrides the bound (tests
+    // unit (N = 20480: 21.1 against 18.5 us).  set_batch32_max_workgroups overrides the bound (tests
     // reach the kernel's K shares and pair launches that way; 0 switches the kernel off).
-    const char* bound_env = std::getenv("AFHIP_BATCH32_MAX_WORKGROUPS");
-    const long bound = bound_env ? std::atol(bound_env) : gemv_compute_units();
+    const long bound_set = batch32_bound.load(std::memory_order_relaxed);
+    const long bound = bound_set >= 0 ? bound_set : gemv_compute_units();
     const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
                             static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
     if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region

@@ -37,6 +37,7 @@ struct afhip_compute {
     LaunchCounters counters;
     hipEvent_t phase_events[3] = {nullptr, nullptr, nullptr};  // created by afhip_compute_set_phase_timing
     bool phase_timing = false;
+    bool q4k_f32_activations = false;  // afhip_compute_set_q4k_f32_activations
 };
 
 namespace {
@@ -235,8 +236,10 @@ afhip_status linear_no_bias_impl(afhip_compute* self, const afhip_tensor* input,
         if (residual) extras.residual = residual->buffer;
         extras.activation = activation;
         self->counters.phase_events = self->phase_timing ? reinterpret_cast<void**>(self->phase_events) : nullptr;
+        const int launch_dispatch =
+            dispatch == AFHIP_DISPATCH_AUTO && self->q4k_f32_activations ? AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS : dispatch;
         s = linear_impl(self->stream, weight->quant_type, weight->layout, device, input->buffer, weight->buffer, rows,
-                        in_dim, out_dim, scratch, dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
+                        in_dim, out_dim, scratch, launch_dispatch, afhip_buffer{0, 0}, &self->counters, device_b,
                         pair ? weight_b->buffer : afhip_buffer{0, 0}, extras);
         self->counters.phase_events = nullptr;
         if (s == AFHIP_OK && self->phase_timing && hipEventSynchronize(self->phase_events[2]) == hipSuccess) {
@@ -762,6 +765,12 @@ afhip_status afhip_compute_linear_no_bias_planned(afhip_compute* self,
                                q.dispatch, out);
 }
 
+afhip_status afhip_compute_set_q4k_f32_activations(afhip_compute* self, int enabled) {
+    if (!self) return AFHIP_ERR_INVALID_ARGUMENT;
+    self->q4k_f32_activations = enabled != 0;
+    return AFHIP_OK;
+}
+
 afhip_status afhip_compute_set_phase_timing(afhip_compute* self, int enabled) {
     if (!self) return AFHIP_ERR_INVALID_ARGUMENT;
     afhip_status s = make_current(self);
@@ -769,7 +778,14 @@ afhip_status afhip_compute_set_phase_timing(afhip_compute* self, int enabled) {
     if (enabled && self->phase_events[0] == nullptr) {
         for (hipEvent_t& e : self->phase_events) {
             s = from_hip(hipEventCreate(&e));
-            if (s != AFHIP_OK) return s;
+            if (s != AFHIP_OK) {
+                // all three or none: a later call starts over
+                for (hipEvent_t& made : self->phase_events) {
+                    if (made != nullptr) (void)hipEventDestroy(made);
+                    made = nullptr;
+                }
+                return s;
+            }
         }
     }
     self->phase_timing = enabled != 0;

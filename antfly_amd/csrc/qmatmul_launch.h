@@ -91,6 +91,7 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
 // whether launch_batch_mfma takes its eight-row kernel for this shape (the faster one where it applies)
 bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
+void set_batch32_max_workgroups(long bound);
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
                              int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b = nullptr,
                              const uint8_t* weight_b_prepared = nullptr, const Epilogue& ep = Epilogue{},

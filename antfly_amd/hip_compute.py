@@ -286,6 +286,11 @@ class HipCompute:
         linear op then waits for its own events, so this is for debugging runs only."""
         check(_lib.lib().afhip_compute_set_phase_timing(self._h, 1 if enabled else 0))
 
+    def setQ4KF32Activations(self, enabled: bool) -> None:
+        """Q4_K linear ops with f32 activations on every shape (the engine's CUDA backend,
+        ops/cuda/cuda_compute.zig:708) instead of following the CPU engine onto its Q8_K route."""
+        check(_lib.lib().afhip_compute_set_q4k_f32_activations(self._h, 1 if enabled else 0))
+
     def debugStats(self) -> dict:
         s = _lib.DebugStats()
         check(_lib.lib().afhip_compute_debug_stats(self._h, C.byref(s)))

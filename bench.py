@@ -50,6 +50,40 @@ def measured_traffic(key="traffic_bytes_per_launch_gemv_q4_0_m1"):
     return None
 
 
+# Sources a kernel's traffic figure depends on: the counter summary records their hash
+# (`kernel_source_sha256_<kernel>: ...`), and a line whose hash no longer matches is reported as stale.
+TRAFFIC_SOURCES = {
+    "gemv_q4_0_m1": ("gemv_kernels.hip", "gemv_common.h", "device_common.h"),
+    "gemm_q8_0_m512": ("gemm_kernels.hip", "device_common.h"),
+}
+
+
+def kernel_source_hash(kernel):
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES[kernel]:
+        with open(os.path.join(ROOT, "antfly_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def traffic_is_stale(kernel):
+    """True when the committed counter summary was made from other kernel sources than the ones in the tree
+    (or does not say which)."""
+    recorded = None
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+            for line in f:
+                if line.startswith(f"kernel_source_sha256_{kernel}:"):
+                    recorded = line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    try:
+        return recorded != kernel_source_hash(kernel)
+    except OSError:
+        return True
+
+
 def gemv_bytes(fmt, rows, in_dim, out_dim):
     """Algorithmic bytes of one call: weights once + f32 activations + f32 outputs."""
     return out_dim * (in_dim // 32) * BLOCK_BYTES[fmt] + 4 * rows * in_dim + 4 * rows * out_dim
@@ -337,15 +371,17 @@ def main() -> int:
         t_quant = time_quantizer(m, k)
         t_kernel = max(t_op - t_quant, 1e-9)
         ops = 2.0 * m * k * n
-        return {"bound": "int8_mfma", "achieved": round(ops / t_kernel / 1e12, 2), "peak": INT8_MFMA_PEAK_OPS / 1e12,
-                "unit": "TOP/s", "frac": round(ops / t_kernel / INT8_MFMA_PEAK_OPS, 4),
-                "kernel": "gemm_i8_kernel<Q8_0> (64 x 128 tiles)",
+        return {"bound": "int8_mfma", "achieved": round(ops / t_op / 1e12, 2), "peak": INT8_MFMA_PEAK_OPS / 1e12,
+                "unit": "TOP/s", "frac": round(ops / t_op / INT8_MFMA_PEAK_OPS, 4),
+                "kernel": "quantize_activations_kernel + gemm_i8_kernel<Q8_0> (64 x 128 tiles)",
                 "workload": f"Q8_0 prefill GEMM, x f32 [{m}x{k}] quantized on the GPU, W [{n}x{k}] 34-byte blocks",
                 "ops_per_launch": ops, "us_per_op": round(t_op * 1e6, 3), "us_quantizer": round(t_quant * 1e6, 3),
-                "us_per_launch": round(t_kernel * 1e6, 3),
-                "achieved_whole_op": round(ops / t_op / 1e12, 2), "frac_whole_op": round(ops / t_op / INT8_MFMA_PEAK_OPS, 4),
+                "us_kernel_by_subtraction": round(t_kernel * 1e6, 3),
+                "frac_kernel_by_subtraction": round(ops / t_kernel / INT8_MFMA_PEAK_OPS, 4),
                 "traffic": measured_traffic("traffic_bytes_per_launch_gemm_q8_0_m512"), "traffic_source": TRAFFIC_FILE,
-                "note": "us_per_launch = op time minus the quantizer's own launch time, both from HIP events in this run; "
+                "traffic_stale": traffic_is_stale("gemm_q8_0_m512"),
+                "note": "achieved and frac are the whole op (activation quantizer + GEMM kernel, HIP events in this run); "
+                        "us_kernel_by_subtraction = op time minus the quantizer launched alone, a side figure; "
                         "every (row, column, block) term also costs one convert and one f32 multiply-add on the vector ALU"}
 
     if args.shapes:
@@ -587,7 +623,8 @@ def main() -> int:
             torch.cuda.synchronize()
         print(json.dumps({"counter_probe": {"launches_each": n_launch, "gemv_bytes": gemv_bytes(Q4, 1, 4096, 14336),
                                             "stream_read_bytes": w_bytes,
-                                            "stream_copy_bytes": w_bytes}}))
+                                            "stream_copy_bytes": w_bytes,
+                                            "kernel_source_sha256": {k: kernel_source_hash(k) for k in TRAFFIC_SOURCES}}}))
         return 0
 
     # ---- headline: Q4_0 decode GEMV, M=1, K=4096, N=14336 --------------------------
@@ -619,6 +656,7 @@ def main() -> int:
                            "the 256 MB Infinity Cache)"},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 2), "peak": HBM_PEAK_BPS / 1e9, "unit": "GB/s",
                      "frac": round(achieved * 1e9 / HBM_PEAK_BPS, 4), "traffic": measured_traffic(),
+                     "traffic_stale": traffic_is_stale("gemv_q4_0_m1"),
                      "traffic_source": TRAFFIC_FILE + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --counter-probe`; not measured by this run)",
                      "kernel": "gemv_fused_kernel<Q4_0, rows=1>", "us_per_launch": round(ev / launches * 1e6, 3)},
     }

@@ -97,6 +97,13 @@ typedef struct afhip_buffer {
  * (plan/select), :558-576 (rowBucket, validShape).
  * ---------------------------------------------------------------------- */
 enum afhip_dispatch_kind { AFHIP_DISPATCH_SCALAR = 0, AFHIP_DISPATCH_MMV = 1, AFHIP_DISPATCH_SMALL_BATCH = 2, AFHIP_DISPATCH_MM = 3 };
+/* Values of a launcher's `dispatch` argument besides a kind: AUTO lets quant_matmul.select choose by rows and, for
+ * Q4_K, follows the CPU engine onto its Q8_K-activation route on that engine's gated shapes
+ * (afhip_uses_q8k_activation_quant; ops/native_compute.zig:3468-3479, :6684-6700).  AUTO_F32_ACTIVATIONS chooses
+ * the same way but keeps Q4_K on f32 activations everywhere, which is what the engine's CUDA backend computes
+ * (ops/cuda/cuda_compute.zig:708); for the 32-value formats it is the same as AUTO. */
+#define AFHIP_DISPATCH_AUTO (-1)
+#define AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS (-2)
 enum afhip_primitive { AFHIP_PRIM_MAT_VEC = 0, AFHIP_PRIM_MAT_VEC_EXT = 1, AFHIP_PRIM_MAT_MAT = 2, AFHIP_PRIM_SCALAR = 3 };
 enum afhip_operator { AFHIP_OP_FALLBACK = 0, AFHIP_OP_MUL_MV = 1, AFHIP_OP_MUL_MV_EXT = 2, AFHIP_OP_MUL_MM = 3, AFHIP_OP_GET_ROWS = 4 };
 enum afhip_row_bucket { AFHIP_ROWS_0 = 0, AFHIP_ROWS_1 = 1, AFHIP_ROWS_2_8 = 2, AFHIP_ROWS_9_64 = 3, AFHIP_ROWS_65_PLUS = 4 };
@@ -332,6 +339,10 @@ afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buff
  * --probe gemv times the eight variants to show where a launch's time goes. */
 afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* Tuning, process-wide, no counterpart in the reference: the largest grid (workgroups) for which 9 .. 64 rows on a
+ * wide matrix take the 32-row MFMA kernel on 64-column tiles; negative restores the default (one workgroup per
+ * compute unit), 0 switches that kernel off.  Tests lift the bound to reach the kernel's K shares and pair launches. */
+afhip_status afhip_tune_batch32_max_workgroups(long bound);
 /* Diagnostic with no counterpart in the reference: the Q8_0 prefill kernel (64 x 128 tiles) on activations
  * already quantized by afhip_launch_quantize_activations, computing as usual but storing, instead of results,
  * eight 32-bit counts per wavefront over the start of `stamps` (which has to hold rows x out_dim floats):
@@ -609,6 +620,10 @@ afhip_status afhip_compute_debug_stats(const afhip_compute *self, afhip_debug_st
  * waits for them before it returns (so it serializes host and device: not for production runs).
  * A kernel that quantizes activations in its own prologue counts entirely as compute. */
 afhip_status afhip_compute_set_phase_timing(afhip_compute *self, int enabled);
+/* Q4_K route of this backend's linear ops: 0 (the default) follows the CPU engine, which quantizes the activations
+ * to Q8_K on its gated shapes (afhip_uses_q8k_activation_quant); non-zero keeps f32 activations everywhere, as
+ * the engine's CUDA backend does (ops/cuda/cuda_compute.zig:708) -- the launchers' AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS. */
+afhip_status afhip_compute_set_q4k_f32_activations(afhip_compute *self, int enabled);
 
 /* Known-answer smokes run entirely inside the library on device 0
  * (ops/cuda/kernels.zig:2309-2399, driven by `cuda-info --smoke`,

@@ -304,3 +304,26 @@ def test_phase_timing_is_opt_in(cb):
     assert cb.debugStats()["timed_ops"] == 2
     ref = O.linear_no_bias(_lib.TYPE_Q8_0, x, w, 24, in_dim, out_dim, workers=8)
     assert G.max_rel_err(y, ref.astype(np.float64)) <= 2e-5
+
+
+def test_q4k_route_switch_of_the_backend(cb):
+    """Q4_K on one of the CPU engine's gated shapes (one row, K = 2048): by default the backend follows that engine
+    onto Q8_K activations; afhip_compute_set_q4k_f32_activations keeps f32 activations, which is what the engine's
+    CUDA backend computes (ops/cuda/cuda_compute.zig:708).  The two numbers differ by the activation quantization."""
+    in_dim, out_dim = 2048, 1024
+    w = synth.weights(_lib.TYPE_Q4_K, 90, out_dim, in_dim)
+    cb.insertWeightFromLoaded("switch.weight", _lib.TYPE_Q4_K, w, [out_dim, in_dim])
+    wt = cb.getWeight("switch.weight")
+    x = synth.activations(91, 1, in_dim)
+    xt = cb.fromFloat32(x, [1, in_dim])
+    assert O.uses_q4k_q8k_activation(1, in_dim, out_dim)
+    q8k = O.linear_q4_k_q8k(x, w, 1, in_dim, out_dim).astype(np.float64)
+    f32 = O.linear_q4_k(x, w, 1, in_dim, out_dim, f64=True)
+    y = cb.toFloat32(cb.linearNoBias(xt, wt, 1, in_dim, out_dim)).reshape(1, out_dim)
+    assert G.max_rel_err(y, q8k) <= 2e-5 and G.max_rel_err(y, f32) > 2e-4
+    cb.setQ4KF32Activations(True)
+    y = cb.toFloat32(cb.linearNoBias(xt, wt, 1, in_dim, out_dim)).reshape(1, out_dim)
+    assert G.max_rel_err(y, f32) <= 2e-5 and G.max_rel_err(y, q8k) > 2e-4
+    cb.setQ4KF32Activations(False)
+    y = cb.toFloat32(cb.linearNoBias(xt, wt, 1, in_dim, out_dim)).reshape(1, out_dim)
+    assert G.max_rel_err(y, q8k) <= 2e-5

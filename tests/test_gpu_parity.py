@@ -322,7 +322,6 @@ def test_thirty_two_row_kernel_with_k_shares_and_pairs(fmt, rows, in_dim, out_di
     """On this chip the 32-row kernel's grid bound (one workgroup per compute unit) keeps launches with
     K shares or two matrices on the older kernel; with the bound lifted they take the 32-row kernel and
     must give what the older kernel gives to f32 summation order, and the oracle's result within its bound."""
-    import os
     print(f"case: 32-row kernel, bound lifted fmt={fmt} rows={rows} in={in_dim} out={out_dim} pair={pair}", flush=True)
     x = synth.activations(5100 + rows, rows, in_dim)
     wa = synth.weights(fmt, 5101, out_dim, in_dim)
@@ -335,20 +334,20 @@ def test_thirty_two_row_kernel_with_k_shares_and_pairs(fmt, rows, in_dim, out_di
         return (G.linear(fmt, PREP, x, da, rows, in_dim, out_dim),)
 
     older = run()
-    os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"] = "1000000"
+    _lib.lib().afhip_tune_batch32_max_workgroups(1000000)
     try:
         got = run()
     finally:
-        del os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"]
+        _lib.lib().afhip_tune_batch32_max_workgroups(-1)
     ref = O.linear_no_bias(fmt, x, wa, rows, in_dim, out_dim, workers=8)
     err = G.max_rel_err(got[0], ref.astype(np.float64))
     assert err <= TOL and err <= TIGHT, err
     for a, b in zip(got, older):
         assert G.max_rel_err(a, b.astype(np.float64)) <= TIGHT
     if pair:  # each half of the pair equals the single op on that matrix, bit for bit
-        os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"] = "1000000"
+        _lib.lib().afhip_tune_batch32_max_workgroups(1000000)
         try:
             assert np.array_equal(got[0], G.linear(fmt, PREP, x, da, rows, in_dim, out_dim))
             assert np.array_equal(got[1], G.linear(fmt, PREP, x, db, rows, in_dim, out_dim))
         finally:
-            del os.environ["AFHIP_BATCH32_MAX_WORKGROUPS"]
+            _lib.lib().afhip_tune_batch32_max_workgroups(-1)

@@ -277,10 +277,23 @@ def test_q8k_activation_route_on_the_gated_shapes(layout, rows, in_dim, out_dim)
     assert err <= TOL and err <= TIGHT, err
     f32_route = O.linear_q4_k(x, w, rows, in_dim, out_dim, f64=True)
     assert G.max_rel_err(y, f32_route) > 10 * TIGHT
-    # the launcher needs the scratch on these shapes
-    with pytest.raises(_lib.InvalidHipState):
-        kernels.launchLinearF32(G.stream(), Q4K, layout, G.buf(torch.empty((rows, out_dim), dtype=torch.float32, device=G.DEV)),
-                                G.buf(G.to_dev(x)), G.buf(wd), rows, in_dim, out_dim, kernels.NO_BUFFER)
+    # The launcher needs the scratch on these shapes -- except where the quantizer runs inside the matmul launch
+    # (one, two or four rows of a repacked tensor), which reads none: there a call without scratch is the same call.
+    yd = torch.full((rows, out_dim), float("nan"), dtype=torch.float32, device=G.DEV)
+    if layout == PREP and rows in (1, 2, 4):
+        kernels.launchLinearF32(G.stream(), Q4K, layout, G.buf(yd), G.buf(G.to_dev(x)), G.buf(wd), rows, in_dim, out_dim,
+                                kernels.NO_BUFFER)
+        torch.cuda.synchronize()
+        assert np.array_equal(yd.cpu().numpy().view(np.uint32), y.view(np.uint32))
+    else:
+        with pytest.raises(_lib.InvalidHipState):
+            kernels.launchLinearF32(G.stream(), Q4K, layout, G.buf(yd), G.buf(G.to_dev(x)), G.buf(wd), rows, in_dim, out_dim,
+                                    kernels.NO_BUFFER)
+    # AFHIP_DISPATCH_AUTO_F32_ACTIVATIONS keeps the same shape on f32 activations (the engine's CUDA backend): the
+    # f32 route's number, with or without scratch
+    yf = G.linear(Q4K, layout, x, wd, rows, in_dim, out_dim, dispatch=_lib.DISPATCH_AUTO_F32_ACTIVATIONS)
+    assert G.max_rel_err(yf, f32_route) <= TIGHT
+    assert G.max_rel_err(yf, O.linear_q4_k(x, w, rows, in_dim, out_dim).astype(np.float64)) <= TIGHT
 
 
 @pytest.mark.parametrize("in_dim,out_dim", [(512, 520), (2048, 8192), (3072, 1000)])
