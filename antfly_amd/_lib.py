@@ -138,6 +138,7 @@ SIGNATURES = {
     "afhip_launch_decode_fp16": (_st, [_vp, Buffer, Buffer, _sz]),
     "afhip_launch_stream_read": (_st, [_vp, Buffer, Buffer]),
     "afhip_launch_stream_copy": (_st, [_vp, Buffer, Buffer]),
+    "afhip_launch_stream_read_shaped": (_st, [_vp, Buffer, Buffer, _i, _i, _i]),
     "afhip_tune_batch32_max_workgroups": (_st, [C.c_long]),
     "afhip_launch_gemm_stamps": (_st, [_vp, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz]),
     "afhip_launch_rate_probe": (_st, [_vp, _i, _i, _i, Buffer, Buffer]),

@@ -941,6 +941,16 @@ afhip_status afhip_launch_stream_read(void* stream, afhip_buffer src, afhip_buff
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_stream_read_shaped(void* stream, afhip_buffer src, afhip_buffer sink, int threads, int loads_per_lane,
+                                            int nontemporal) {
+    if (src.len < 16) return AFHIP_OK;
+    if (src.ptr == 0 || src.ptr % 16 != 0 || sink.ptr == 0 || sink.len < 4) return AFHIP_ERR_INVALID_STATE;
+    hipError_t e = launch_stream_read_shaped(static_cast<hipStream_t>(stream), reinterpret_cast<const uint8_t*>(src.ptr),
+                                             reinterpret_cast<uint32_t*>(sink.ptr), src.len, threads, loads_per_lane, nontemporal);
+    if (e == hipErrorInvalidValue) return AFHIP_ERR_INVALID_ARGUMENT;
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_stream_copy(void* stream, afhip_buffer src, afhip_buffer dst) {
     if (src.len / 16 > 0xffffffffull * 256 || dst.len < src.len / 16 * 16) return AFHIP_ERR_INVALID_STATE;
     if (src.len < 16) return AFHIP_OK;

@@ -270,6 +270,28 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4* __
     if (x == 0x9E3779B9u && i == n16 + 1) sink[0] = x;  // never true for i < n16; keeps the loads alive
 }
 
+// The same read in other launch shapes: a wavefront requests kLoads consecutive KiB (16 bytes per lane and load), every
+// load issued before any is waited for; a workgroup of blockDim.x threads covers blockDim.x / 64 * kLoads KiB in a row.
+// kHint: 0 plain loads, 1 non-temporal.  bench.py --probe read sweeps it to show what a launch of a given size can
+// draw from HBM at best, and in which shape.
+template <int kLoads, int kHint>
+__global__ __launch_bounds__(1024) void stream_read_shaped_kernel(const stream_u32x4* __restrict__ src, uint32_t* __restrict__ sink,
+                                                                  size_t n16) {
+    const size_t wave = blockIdx.x * static_cast<size_t>(blockDim.x >> 6) + (threadIdx.x >> 6);
+    const size_t first = wave * (64 * kLoads) + (threadIdx.x & 63);
+    stream_u32x4 v[kLoads];
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) {
+        const size_t i = first + 64 * j;
+        const stream_u32x4* at = src + (i < n16 ? i : n16 - 1);
+        v[j] = kHint ? __builtin_nontemporal_load(at) : *at;
+    }
+    uint32_t x = 0;
+#pragma unroll
+    for (int j = 0; j < kLoads; ++j) x ^= v[j].x ^ v[j].y ^ v[j].z ^ v[j].w;
+    if (x == 0x9E3779B9u && first == n16 + 1) sink[0] = x;  // never true; keeps the loads alive
+}
+
 // The plain copy: dst[i] = src[i], 16 bytes per lane, each byte read once and written
 // once.  The kernel of known traffic that the hardware write counter is scaled against.
 __global__ __launch_bounds__(256) void stream_copy_kernel(stream_u32x4* __restrict__ dst, const stream_u32x4* __restrict__ src,
@@ -453,6 +475,32 @@ hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* 
     if (n16 == 0) return hipSuccess;
     hipLaunchKernelGGL(stream_read_kernel, dim3(static_cast<unsigned>((n16 + 255) / 256)), dim3(256), 0, stream,
                        reinterpret_cast<const stream_u32x4*>(src), sink, n16);
+    return launch_status();
+}
+
+hipError_t launch_stream_read_shaped(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes, int threads,
+                                     int loads_per_lane, int nontemporal) {
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return hipSuccess;
+    if (threads < 64 || threads > 1024 || threads % 64 != 0) return hipErrorInvalidValue;
+    const size_t per_group = static_cast<size_t>(threads) * loads_per_lane;
+    const size_t grid = (n16 + per_group - 1) / per_group;
+    if (grid > 0x7fffffffull) return hipErrorInvalidValue;
+    const stream_u32x4* s = reinterpret_cast<const stream_u32x4*>(src);
+#define AFHIP_READ_SHAPE(L)                                                                                                        \
+    case L:                                                                                                                        \
+        if (nontemporal)                                                                                                           \
+            hipLaunchKernelGGL((stream_read_shaped_kernel<L, 1>), dim3(static_cast<unsigned>(grid)), dim3(threads), 0, stream, s,   \
+                               sink, n16);                                                                                         \
+        else                                                                                                                       \
+            hipLaunchKernelGGL((stream_read_shaped_kernel<L, 0>), dim3(static_cast<unsigned>(grid)), dim3(threads), 0, stream, s,   \
+                               sink, n16);                                                                                         \
+        break;
+    switch (loads_per_lane) {
+        AFHIP_READ_SHAPE(1) AFHIP_READ_SHAPE(2) AFHIP_READ_SHAPE(4) AFHIP_READ_SHAPE(8) AFHIP_READ_SHAPE(16)
+        default: return hipErrorInvalidValue;
+    }
+#undef AFHIP_READ_SHAPE
     return launch_status();
 }
 

@@ -202,6 +202,8 @@ hipError_t launch_gemv_probe(hipStream_t stream, int probe, float* dst, const fl
                              int in_dim, int out_dim);
 
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
+hipError_t launch_stream_read_shaped(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes, int threads,
+                                     int loads_per_lane, int nontemporal);
 hipError_t launch_rate_probe(hipStream_t stream, int pattern, int wavefronts_per_simd, int iterations, int* sink, uint32_t* stamps);
 int rate_probe_wavefronts(int wavefronts_per_simd);
 hipError_t launch_stream_copy(hipStream_t stream, uint8_t* dst, const uint8_t* src, size_t bytes);

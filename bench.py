@@ -109,8 +109,8 @@ def main() -> int:
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k; q4p / q8p: pair calls): time only these calls, print one line each, exit")
-    ap.add_argument("--probe", choices=["gemv", "rates", "gemm"], default=None,
-                    help="gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+    ap.add_argument("--probe", choices=["gemv", "rates", "gemm", "read"], default=None,
+                    help="read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -480,6 +480,56 @@ def main() -> int:
                 print(f"| {name} | {waves} | {med:.1f}; {cyc.min():.1f}-{cyc.max():.1f} | {med / waves / per_round:.2f} | {ghz:.3f} | {exact} of {len(simds)} |")
                 out[f"{name} @{waves}"] = round(med, 2)
         print(json.dumps({"probe": "rates", "cycles_per_round": out}))
+        return 0
+
+    if args.probe == "read":
+        copies, per_graph, replays = args.copies, 100, 10
+        w_bytes = 14336 * (4096 // 32) * 18
+        srcs = [torch.randint(0, 255, (w_bytes,), dtype=torch.uint8, device=dev) for _ in range(copies)]
+        sink = torch.zeros(4, dtype=torch.int32, device=dev)
+        lib = _lib.lib()
+
+        def timed(call):
+            for i in range(10):
+                call(i, stream)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                cs = torch.cuda.current_stream().cuda_stream
+                for i in range(per_graph):
+                    call(i, cs)
+            graph.replay()
+            torch.cuda.synchronize()
+            out = []
+            for _ in range(5):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(replays):
+                    graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                out.append(e0.elapsed_time(e1) * 1e3 / (per_graph * replays))
+            return sorted(out)[2]
+
+        print(f"read of {w_bytes} bytes per launch, {copies} buffers in turn (more than the 256 MB last-level cache), graph replays")
+        print("| threads per workgroup | 16-byte loads in flight per lane | workgroups | hint | us per launch | GB/s | % of 8 TB/s |")
+        print("|---|---|---|---|---|---|---|")
+        t = timed(lambda i, st: lib.afhip_launch_stream_read(st, Buffer(srcs[i % copies].data_ptr(), w_bytes), buf(sink)))
+        print(f"| 256 | 1 (afhip_launch_stream_read) | {(w_bytes // 16 + 255) // 256} | non-temporal | {t:.3f} | {w_bytes / t / 1e3:.0f} | {w_bytes / t / 1e3 / 80:.1f} |")
+        best = {}
+        for threads in (256, 512, 1024):
+            for loads in (1, 2, 4, 8, 16):
+                for hint in (1, 0):
+                    def call(i, st, threads=threads, loads=loads, hint=hint):
+                        rc = lib.afhip_launch_stream_read_shaped(st, Buffer(srcs[i % copies].data_ptr(), w_bytes), buf(sink), threads, loads, hint)
+                        if rc != 0:
+                            raise RuntimeError(f"read probe failed: {rc}")
+                    t = timed(call)
+                    groups = (w_bytes // 16 + threads * loads - 1) // (threads * loads)
+                    print(f"| {threads} | {loads} | {groups} | {'non-temporal' if hint else 'plain'} | {t:.3f} | {w_bytes / t / 1e3:.0f} | {w_bytes / t / 1e3 / 80:.1f} |", flush=True)
+                    best[(threads, loads, hint)] = t
+        k = min(best, key=best.get)
+        print(json.dumps({"probe": "read", "best_us": round(best[k], 3), "best_shape": {"threads": k[0], "loads_per_lane": k[1], "nontemporal": k[2]}}))
         return 0
 
     if args.probe == "gemm":

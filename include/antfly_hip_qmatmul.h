@@ -327,6 +327,11 @@ afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_
  * beside the GEMV as "what one launch of this size can draw from HBM", and it is
  * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
 afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
+/* The same read in another launch shape: workgroups of `threads` (a multiple of 64, at most 1024), every lane
+ * requesting `loads_per_lane` (1, 2, 4, 8 or 16) x 16 bytes at once, a wavefront's loads covering consecutive KiB;
+ * `nontemporal` picks the load hint.  `bench.py --probe read` sweeps it. */
+afhip_status afhip_launch_stream_read_shaped(void *stream, afhip_buffer src, afhip_buffer sink, int threads,
+                                            int loads_per_lane, int nontemporal);
 /* Diagnostic with no counterpart in the reference: the plain copy, dst[0 .. src.len) =
  * src (16 bytes per lane; src.len is rounded down to a multiple of 16, both pointers
  * 16-byte aligned, dst.len >= the copied length).  The kernel of known traffic that
