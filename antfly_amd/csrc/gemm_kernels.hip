@@ -132,10 +132,10 @@ extern __shared__ __align__(16) unsigned char gemm_lds[];
 // the K loop, in it, waiting for its own loads, waiting at the workgroup barrier, 100 MHz reference ticks
 // spent in the loop (cycles / ticks = the clock the chip held), cycles after the loop, 0, and the HW_ID register.
 template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots, bool kShareK = false, bool kStamps = false>
-__global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
+__device__ __forceinline__ void gemm_i8_body(
     float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
     const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
-    int share_blocks, float* __restrict__ partial, Epilogue ep) {
+    int share_blocks, float* __restrict__ partial, const Epilogue& ep) {
     using S = GemmShape<kWavesM, kWavesN, kSplit, kType == 2>;
     constexpr int kWaves = S::kWaves, kSB = S::kStageBlocks, kRPL = S::kRowsPerLoad, kCPR = S::kChunksPerRow;
     constexpr int kTM = S::kTM, kTN = S::kTN, kRing = S::kRing;
@@ -474,6 +474,15 @@ __global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kerne
             }
         }
     }
+}
+
+template <int kType, int kWavesM, int kWavesN, int kSplit, bool kWriteDots, bool kShareK = false, bool kStamps = false>
+__global__ __launch_bounds__(64 * kWavesM * kWavesN * kSplit) void gemm_i8_kernel(
+    float* __restrict__ dst, int* __restrict__ dots, const int8_t* __restrict__ qx, const float* __restrict__ sx,
+    const uint8_t* __restrict__ weight, int rows, int in_dim, int out_dim, int m_tiles, int n_tiles,
+    int share_blocks, float* __restrict__ partial, Epilogue ep) {
+    gemm_i8_body<kType, kWavesM, kWavesN, kSplit, kWriteDots, kShareK, kStamps>(dst, dots, qx, sx, weight, rows, in_dim, out_dim,
+                                                                                 m_tiles, n_tiles, share_blocks, partial, ep);
 }
 
 namespace {

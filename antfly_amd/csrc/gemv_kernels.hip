@@ -363,11 +363,9 @@ __global__ __launch_bounds__(1024) void gemv_fused_kernel(
 // use does not grow with the row count; `rows` is a run-time value bounded only by LDS.
 // =====================================================================
 template <int kType, int kCols, bool kWriteDots>
-__global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* __restrict__ dots,
-                                                            const int4* __restrict__ pre_q,
-                                                            const float* __restrict__ pre_scale,
-                                                            const int* __restrict__ pre_sum, int rows, int in_dim,
-                                                            int out_dim, int slices) {
+__device__ __forceinline__ void gemv_rows_body(const GemvTargets& tg, int* __restrict__ dots, const int4* __restrict__ pre_q,
+                                               const float* __restrict__ pre_scale, const int* __restrict__ pre_sum, int rows,
+                                               int in_dim, int out_dim, int slices) {
     using F = GemvFormat<kType>;
     constexpr int kLpb = F::kLanesPerBlock;
     constexpr int kBlocksPerStep = kWave / kLpb;
@@ -579,6 +577,15 @@ int gemv_compute_units() {
         return n;
     }();
     return cus;
+}
+
+template <int kType, int kCols, bool kWriteDots>
+__global__ __launch_bounds__(512, 4) void gemv_rows_kernel(GemvTargets tg, int* __restrict__ dots,
+                                                            const int4* __restrict__ pre_q,
+                                                            const float* __restrict__ pre_scale,
+                                                            const int* __restrict__ pre_sum, int rows, int in_dim,
+                                                            int out_dim, int slices) {
+    gemv_rows_body<kType, kCols, kWriteDots>(tg, dots, pre_q, pre_scale, pre_sum, rows, in_dim, out_dim, slices);
 }
 
 namespace {

@@ -25,10 +25,8 @@ namespace afhip {
 
 // Route B.  grid = (out_dim, rows), block = 64.
 template <typename Weights>
-__global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict__ dst,
-                                                              const float* __restrict__ input, Weights w,
-                                                              int rows, int in_dim, int out_dim,
-                                                              Epilogue ep) {
+__device__ __forceinline__ void linear_f32_route_body(float* __restrict__ dst, const float* __restrict__ input, const Weights& w,
+                                                      int rows, int in_dim, int out_dim, const Epilogue& ep) {
     const int o = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
     const int kb = in_dim >> 5;
     const float* x = input + static_cast<size_t>(r) * in_dim;
@@ -50,6 +48,14 @@ __global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict_
     }
     acc = wave_sum(acc);
     if (lane == 0) dst[static_cast<size_t>(r) * out_dim + o] = finish_output(ep, o, static_cast<size_t>(r) * out_dim + o, acc);
+}
+
+template <typename Weights>
+__global__ __launch_bounds__(64) void linear_f32_route_kernel(float* __restrict__ dst,
+                                                              const float* __restrict__ input, Weights w,
+                                                              int rows, int in_dim, int out_dim,
+                                                              Epilogue ep) {
+    linear_f32_route_body(dst, input, w, rows, in_dim, out_dim, ep);
 }
 
 // Route A from pre-quantized activations.  grid = (out_dim, rows), block = 64.
@@ -79,9 +85,9 @@ __global__ __launch_bounds__(64) void linear_act_generic_kernel(float* __restric
 
 // Stand-alone activation quantizer (ops/native_compute.zig:11998-12028,
 // :23799-23832).  8 lanes per block, grid-stride over float4 units.
-__global__ __launch_bounds__(256) void quantize_activations_kernel(const float* __restrict__ x, int rows, int in_dim,
-                                                                    int8_t* __restrict__ q, float* __restrict__ scale,
-                                                                    int* __restrict__ sum) {
+__device__ __forceinline__ void quantize_activations_body(const float* __restrict__ x, int rows, int in_dim,
+                                                          int8_t* __restrict__ q, float* __restrict__ scale,
+                                                          int* __restrict__ sum) {
     const size_t units = static_cast<size_t>(rows) * (in_dim >> 2);
     for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
          u += static_cast<size_t>(gridDim.x) * blockDim.x) {
@@ -99,6 +105,12 @@ __global__ __launch_bounds__(256) void quantize_activations_kernel(const float* 
             if (sum) sum[u >> 3] = total;
         }
     }
+}
+
+__global__ __launch_bounds__(256) void quantize_activations_kernel(const float* __restrict__ x, int rows, int in_dim,
+                                                                    int8_t* __restrict__ q, float* __restrict__ scale,
+                                                                    int* __restrict__ sum) {
+    quantize_activations_body(x, rows, in_dim, q, scale, sum);
 }
 
 // RAW -> PREPARED repack, one thread per block: quant bytes, the scale in block order, and

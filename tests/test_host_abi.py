@@ -211,3 +211,44 @@ def test_zig_backend_sources_bind_what_exists():
         pytest.skip("libamdhip64.so not loadable here")
     missing = [n for n in table if not hasattr(hip, n)]
     assert not missing, missing
+
+
+def test_session_wiring_patches_are_well_formed_and_apply():
+    """zig/patches/*.patch (the `--backend hip` wiring, unified diffs against the antfly tree): headers and hunk line
+    counts are consistent, the added lines name the hip backend, and -- where the reference tree is present (it
+    is not on a GPU box) -- every context and removed line is found at the place the hunk header names."""
+    pdir = os.path.join(ROOT, "zig", "patches")
+    names = sorted(n for n in os.listdir(pdir) if n.endswith(".patch"))
+    assert len(names) >= 9
+    ref_root = "/root/reference"
+    for name in names:
+        lines = open(os.path.join(pdir, name)).read().split("\n")
+        assert lines[0].startswith("--- a/zig/pkg/inference/") and lines[1].startswith("+++ b/zig/pkg/inference/"), name
+        rel = lines[0][len("--- a/"):]
+        assert lines[1][len("+++ b/"):] == rel
+        ref_lines = None
+        if os.path.exists(os.path.join(ref_root, rel)):
+            ref_lines = open(os.path.join(ref_root, rel)).read().split("\n")
+        i, hunks, added = 2, 0, []
+        while i < len(lines) and lines[i]:
+            m = re.match(r"@@ -(\d+),(\d+) \+(\d+),(\d+) @@", lines[i])
+            assert m, (name, lines[i])
+            old_at, old_n, new_n = int(m.group(1)), int(m.group(2)), int(m.group(4))
+            i += 1
+            seen_old = seen_new = 0
+            while i < len(lines) and lines[i] and not lines[i].startswith("@@"):
+                tag, text = lines[i][0], lines[i][1:]
+                assert tag in " +-", (name, lines[i])
+                if tag in " -":
+                    if ref_lines is not None:
+                        assert ref_lines[old_at - 1 + seen_old] == text, (name, old_at + seen_old, text)
+                    seen_old += 1
+                if tag in " +":
+                    seen_new += 1
+                if tag == "+":
+                    added.append(text)
+                i += 1
+            assert (seen_old, seen_new) == (old_n, new_n), (name, m.group(0))
+            hunks += 1
+        assert hunks >= 1, name
+        assert added and any(re.search(r"hip|Hip", t) for t in added), name

@@ -1,11 +1,9 @@
 //! `--backend hip`: a session whose resident quantized weights live on the MI355X and whose
 //! quantized `linearNoBias` runs there (session_factory.zig:1261-1301 builds the CUDA session
-//! the same way).  session_factory.zig imports this file behind `build_options.enable_hip`:
-//!
-//!     const hip_session = if (build_options.enable_hip) @import("hip_session.zig") else struct {};
-//!     pub const createHipSession = hip_session.createHipSession;
-//!
-//! and adds `hip: struct { compute: hip_compute_mod.HipCompute }` to ArchSession.backend_data.
+//! the same way).  session_factory.zig imports this file behind `build_options.enable_hip`, re-exports
+//! `createHipSession*`, adds `hip: HipData` to its `BackendData` and the `hip` arms to its switches:
+//! zig/patches/0009 holds that edit as a diff, 0001 .. 0010 the rest of the wiring from `-Dhip` and
+//! `--backend hip` down to here.
 const std = @import("std");
 const build_options = @import("build_options");
 const factory = @import("session_factory.zig");

@@ -3,12 +3,17 @@
 //! :1980-2007 do the same with their image), its entry points, and the launchers the compute
 //! ops call (ops/cuda/kernels.zig:1221-1289 for the quantized matmul).
 //!
-//! Dispatch by rows (graph/quant_matmul.zig:263-268):
-//!   mmv (1 row)             this module's own decode kernel, launched from a parameter block
-//!   small_batch (2..8 rows) libantfly_hip_qmatmul's launcher (afhip_launch_linear_f32), on this
-//!   mm (9+ rows)            backend's stream and buffers; workspace from this backend's scratch
-//! The library is a thin C ABI over the same kernels: it owns no device state when called
-//! through its afhip_launch_* layer -- stream, buffers and module loading stay here.
+//! Dispatch by rows (graph/quant_matmul.zig:263-268), every bucket from this module's own code object,
+//! launched from a parameter block:
+//!   small shapes (out_dim < 512 or in_dim < 96)  the f32 route entry (the CPU engine's route gate)
+//!   mmv (1 row), small_batch up to 4 rows of Q4_0 / 2 of Q8_0 on K <= 4096
+//!                                       the decode entry, activations quantized inside the kernel
+//!   small_batch otherwise               the quantizer entry, then the rows entry
+//!   mm (9+ rows)                        the quantizer entry, then the int8-MFMA GEMM entry
+//! `batch_kernels = .library` (the default) hands 5 .. 128 rows to libantfly_hip_qmatmul's launcher
+//! (afhip_launch_linear_f32) instead, whose MFMA batch kernels are faster there; the library is a thin C
+//! ABI over the same kernels and owns no device state when called through its afhip_launch_* layer --
+//! stream, buffers and module loading stay here.  `.module` keeps every launch in this file.
 const std = @import("std");
 const buffer_mod = @import("buffer.zig");
 const context_mod = @import("context.zig");
@@ -53,6 +58,8 @@ pub fn linearWorkspaceBytes(tensor_type: TensorType, rows: usize, in_dim: usize,
     return afhip_linear_workspace_bytes(@intFromEnum(tensor_type), rows, in_dim, out_dim);
 }
 
+pub const BatchKernels = enum { module, library };
+
 pub const KernelModule = struct {
     module: driver_mod.hipModule_t = null,
     zero_fill: driver_mod.hipFunction_t = null,
@@ -60,6 +67,17 @@ pub const KernelModule = struct {
     prepare_weight_q8_0: driver_mod.hipFunction_t = null,
     linear_q4_0_f32: driver_mod.hipFunction_t = null,
     linear_q8_0_f32: driver_mod.hipFunction_t = null,
+    linear_q4_0_f32_route: driver_mod.hipFunction_t = null,
+    linear_q8_0_f32_route: driver_mod.hipFunction_t = null,
+    quantize_activations: driver_mod.hipFunction_t = null,
+    linear_q4_0_rows_f32: driver_mod.hipFunction_t = null,
+    linear_q8_0_rows_f32: driver_mod.hipFunction_t = null,
+    gemm_q4_0_f32: driver_mod.hipFunction_t = null,
+    gemm_q8_0_f32: driver_mod.hipFunction_t = null,
+    gemm_q4_0_f32_small: driver_mod.hipFunction_t = null,
+    gemm_q8_0_f32_small: driver_mod.hipFunction_t = null,
+    /// who serves 5 .. 128 rows (see the file comment)
+    batch_kernels: BatchKernels = .library,
 
     pub fn load(ctx: *context_mod.HipContext) driver_mod.Error!KernelModule {
         try ctx.makeCurrent();
@@ -76,6 +94,15 @@ pub const KernelModule = struct {
             .{ &self.prepare_weight_q8_0, "termite_hip_prepare_weight_q8_0" },
             .{ &self.linear_q4_0_f32, "termite_hip_linear_q4_0_f32" },
             .{ &self.linear_q8_0_f32, "termite_hip_linear_q8_0_f32" },
+            .{ &self.linear_q4_0_f32_route, "termite_hip_linear_q4_0_f32_route" },
+            .{ &self.linear_q8_0_f32_route, "termite_hip_linear_q8_0_f32_route" },
+            .{ &self.quantize_activations, "termite_hip_quantize_activations" },
+            .{ &self.linear_q4_0_rows_f32, "termite_hip_linear_q4_0_rows_f32" },
+            .{ &self.linear_q8_0_rows_f32, "termite_hip_linear_q8_0_rows_f32" },
+            .{ &self.gemm_q4_0_f32, "termite_hip_gemm_q4_0_f32" },
+            .{ &self.gemm_q8_0_f32, "termite_hip_gemm_q8_0_f32" },
+            .{ &self.gemm_q4_0_f32_small, "termite_hip_gemm_q4_0_f32_small" },
+            .{ &self.gemm_q8_0_f32_small, "termite_hip_gemm_q8_0_f32_small" },
         };
         inline for (entries) |entry| {
             try ctx.driver.check(ctx.driver.fns.hipModuleGetFunction(entry[0], self.module, entry[1]));
@@ -148,26 +175,177 @@ pub const KernelModule = struct {
 
         const format: quant_matmul.Format = if (tensor_type == .q4_0) .q4_0 else .q8_0;
         const kind = quant_matmul.select(.{ .rows = rows, .in_dim = in_dim, .out_dim = out_dim, .format = format });
+        const kb = in_dim / block_values;
         // the CPU engine's route gate (ops/native_compute.zig:3410-3419): small shapes multiply f32
-        // activations by dequantized weights, which the library's generic kernels do
-        const activation_quant = out_dim >= 512 and in_dim / block_values >= 3;
-        if (kind == .mmv and activation_quant and in_dim <= 16 * 4096) {
-            return self.launchDecodeRow(ctx, tensor_type, dst, input, weight_prepared, in_dim, out_dim);
+        // activations by dequantized weights
+        const activation_quant = out_dim >= 512 and kb >= 3;
+        if (!activation_quant) return self.launchF32Route(ctx, tensor_type, dst, input, weight_prepared, rows, in_dim, out_dim);
+        // activations quantized inside the decode kernel: one row up to K = 16384; up to 4 (Q4_0) / 2 (Q8_0)
+        // rows on one K slice, at most 512 blocks of X from three rows on
+        const fused_rows: usize = if (tensor_type == .q4_0) 4 else 2;
+        const fused = (rows == 1 and kb <= 16 * 128) or
+            (rows >= 2 and rows <= fused_rows and kb <= 128 and (rows <= 2 or rows * kb <= 512));
+        if (kind != .mm and fused) {
+            return self.launchDecodeRows(ctx, tensor_type, dst, input, weight_prepared, rows, in_dim, out_dim);
         }
-        try ctx.makeCurrent();
-        const rc = afhip_launch_linear_f32(ctx.stream, @intFromEnum(tensor_type), layout_prepared, dst, input, weight_prepared, rows, in_dim, out_dim, workspace, -1);
-        if (rc != 0) return error.HipDriverError;
+        if (self.batch_kernels == .library and rows >= 5 and rows <= 128) {
+            try ctx.makeCurrent();
+            const rc = afhip_launch_linear_f32(ctx.stream, @intFromEnum(tensor_type), layout_prepared, dst, input, weight_prepared, rows, in_dim, out_dim, workspace, -1);
+            if (rc != 0) return error.HipDriverError;
+            return;
+        }
+        // quantized activations in the workspace: int8 [rows][in_dim], then f32 scales and i32 sums [rows][kb]
+        const q_bytes = try checkedMul(rows, in_dim);
+        const s_bytes = try checkedMul(try checkedMul(rows, kb), @sizeOf(f32));
+        if (workspace.ptr % 16 != 0 or q_bytes % 16 != 0) return error.InvalidHipState;
+        try checkBytes(workspace, q_bytes + 2 * s_bytes);
+        const q = buffer_mod.DeviceBuffer{ .ptr = workspace.ptr, .len = q_bytes };
+        const scales = buffer_mod.DeviceBuffer{ .ptr = workspace.ptr + q_bytes, .len = s_bytes };
+        const sums = buffer_mod.DeviceBuffer{ .ptr = workspace.ptr + q_bytes + s_bytes, .len = s_bytes };
+        try self.launchQuantizeActivations(ctx, q, scales, sums, input, rows, in_dim);
+        if (kind == .mm) {
+            return self.launchGemm(ctx, tensor_type, dst, input, weight_prepared, rows, in_dim, out_dim, q, scales);
+        }
+        return self.launchRows(ctx, tensor_type, dst, input, weight_prepared, rows, in_dim, out_dim, q, scales, sums);
     }
 
-    /// The mmv bucket: this module's own kernel, launched from a parameter block whose leading
-    /// entries are the reference kernel's (dst, input, weight, rows, in_dim, out_dim).
-    fn launchDecodeRow(
+    /// Route B: grid (out_dim, rows), one wavefront per output element.
+    fn launchF32Route(
         self: *KernelModule,
         ctx: *context_mod.HipContext,
         tensor_type: TensorType,
         dst: buffer_mod.DeviceBuffer,
         input: buffer_mod.DeviceBuffer,
         weight_prepared: buffer_mod.DeviceBuffer,
+        rows: usize,
+        in_dim: usize,
+        out_dim: usize,
+    ) driver_mod.Error!void {
+        var dst_ptr = dst.ptr;
+        var input_ptr = input.ptr;
+        var weight_ptr = weight_prepared.ptr;
+        var rows_u32 = try toU32(rows);
+        var in_dim_u32 = try toU32(in_dim);
+        var out_dim_u32 = try toU32(out_dim);
+        var params = [_]?*anyopaque{ @ptrCast(&dst_ptr), @ptrCast(&input_ptr), @ptrCast(&weight_ptr), @ptrCast(&rows_u32), @ptrCast(&in_dim_u32), @ptrCast(&out_dim_u32) };
+        const f = if (tensor_type == .q4_0) self.linear_q4_0_f32_route else self.linear_q8_0_f32_route;
+        if (rows > 65535) return error.InvalidHipState; // grid.y
+        try launch(ctx, f, .{ try toU32(out_dim), try toU32(rows) }, .{ 64, 1 }, 0, &params);
+    }
+
+    /// int8 values, f32 scales and i32 sums of every 32-value block of X (ops/native_compute.zig:23799-23832).
+    fn launchQuantizeActivations(
+        self: *KernelModule,
+        ctx: *context_mod.HipContext,
+        q: buffer_mod.DeviceBuffer,
+        scales: buffer_mod.DeviceBuffer,
+        sums: buffer_mod.DeviceBuffer,
+        input: buffer_mod.DeviceBuffer,
+        rows: usize,
+        in_dim: usize,
+    ) driver_mod.Error!void {
+        var q_ptr = q.ptr;
+        var scales_ptr = scales.ptr;
+        var sums_ptr = sums.ptr;
+        var input_ptr = input.ptr;
+        var rows_u32 = try toU32(rows);
+        var in_dim_u32 = try toU32(in_dim);
+        var params = [_]?*anyopaque{ @ptrCast(&q_ptr), @ptrCast(&scales_ptr), @ptrCast(&sums_ptr), @ptrCast(&input_ptr), @ptrCast(&rows_u32), @ptrCast(&in_dim_u32) };
+        const units: u64 = @intCast(try checkedMul(rows, in_dim / 4));
+        try launch(ctx, self.quantize_activations, .{ gridFor(units, 256, 4096), 1 }, .{ 256, 1 }, 0, &params);
+    }
+
+    /// small_batch from quantized activations: eight wavefronts a workgroup (a multiple of the K slices).
+    fn launchRows(
+        self: *KernelModule,
+        ctx: *context_mod.HipContext,
+        tensor_type: TensorType,
+        dst: buffer_mod.DeviceBuffer,
+        input: buffer_mod.DeviceBuffer,
+        weight_prepared: buffer_mod.DeviceBuffer,
+        rows: usize,
+        in_dim: usize,
+        out_dim: usize,
+        q: buffer_mod.DeviceBuffer,
+        scales: buffer_mod.DeviceBuffer,
+        sums: buffer_mod.DeviceBuffer,
+    ) driver_mod.Error!void {
+        const kb = in_dim / block_values;
+        const cols: usize = if (tensor_type == .q4_0) 4 else 2;
+        const slices = (kb + 127) / 128;
+        if (slices > 16) return error.InvalidHipState;
+        const waves = @max(8 / slices * slices, slices);
+        const groups = (out_dim + cols - 1) / cols;
+        const groups_per_wg = waves / slices;
+        const grid = (groups + groups_per_wg - 1) / groups_per_wg;
+        const lds = fusedLdsBytes(rows, in_dim);
+        if (lds > 160 * 1024) return error.InvalidHipState; // more rows than LDS holds: the caller slices them
+        var dst_ptr = dst.ptr;
+        var input_ptr = input.ptr;
+        var weight_ptr = weight_prepared.ptr;
+        var rows_u32 = try toU32(rows);
+        var in_dim_u32 = try toU32(in_dim);
+        var out_dim_u32 = try toU32(out_dim);
+        var q_ptr = q.ptr;
+        var scales_ptr = scales.ptr;
+        var sums_ptr = sums.ptr;
+        var params = [_]?*anyopaque{ @ptrCast(&dst_ptr), @ptrCast(&input_ptr), @ptrCast(&weight_ptr), @ptrCast(&rows_u32), @ptrCast(&in_dim_u32), @ptrCast(&out_dim_u32), @ptrCast(&q_ptr), @ptrCast(&scales_ptr), @ptrCast(&sums_ptr) };
+        const f = if (tensor_type == .q4_0) self.linear_q4_0_rows_f32 else self.linear_q8_0_rows_f32;
+        try launch(ctx, f, .{ try toU32(grid), 1 }, .{ try toU32(64 * waves), 1 }, try toU32(lds), &params);
+    }
+
+    /// The mm bucket: 64 x 128 tiles while they give every compute unit a workgroup, 32 x 64 tiles otherwise.
+    fn launchGemm(
+        self: *KernelModule,
+        ctx: *context_mod.HipContext,
+        tensor_type: TensorType,
+        dst: buffer_mod.DeviceBuffer,
+        input: buffer_mod.DeviceBuffer,
+        weight_prepared: buffer_mod.DeviceBuffer,
+        rows: usize,
+        in_dim: usize,
+        out_dim: usize,
+        q: buffer_mod.DeviceBuffer,
+        scales: buffer_mod.DeviceBuffer,
+    ) driver_mod.Error!void {
+        const units: usize = @intCast(@max(ctx.info.compute_units, 1));
+        const big = ((rows + 63) / 64) * ((out_dim + 127) / 128) >= units;
+        const tile_m: usize = if (big) 64 else 32;
+        const tile_n: usize = if (big) 128 else 64;
+        const m_tiles = (rows + tile_m - 1) / tile_m;
+        const n_tiles = (out_dim + tile_n - 1) / tile_n;
+        const grid = try checkedMul(try checkedMul((n_tiles + 7) / 8, m_tiles), 8);
+        // four stages of operands: 27648 bytes each, and 8192 more for Q4_0's nibble chunks
+        const lds: usize = if (tensor_type == .q4_0) 143360 else 110592;
+        var dst_ptr = dst.ptr;
+        var input_ptr = input.ptr;
+        var weight_ptr = weight_prepared.ptr;
+        var rows_u32 = try toU32(rows);
+        var in_dim_u32 = try toU32(in_dim);
+        var out_dim_u32 = try toU32(out_dim);
+        var q_ptr = q.ptr;
+        var scales_ptr = scales.ptr;
+        var m_tiles_u32 = try toU32(m_tiles);
+        var n_tiles_u32 = try toU32(n_tiles);
+        var params = [_]?*anyopaque{ @ptrCast(&dst_ptr), @ptrCast(&input_ptr), @ptrCast(&weight_ptr), @ptrCast(&rows_u32), @ptrCast(&in_dim_u32), @ptrCast(&out_dim_u32), @ptrCast(&q_ptr), @ptrCast(&scales_ptr), @ptrCast(&m_tiles_u32), @ptrCast(&n_tiles_u32) };
+        const f = if (tensor_type == .q4_0)
+            (if (big) self.gemm_q4_0_f32 else self.gemm_q4_0_f32_small)
+        else
+            (if (big) self.gemm_q8_0_f32 else self.gemm_q8_0_f32_small);
+        const threads: u32 = if (big) 1024 else 512;
+        try launch(ctx, f, .{ try toU32(grid), 1 }, .{ threads, 1 }, try toU32(lds), &params);
+    }
+
+    /// The mmv bucket and the first rows of small_batch: launched from a parameter block whose leading
+    /// entries are the reference kernel's (dst, input, weight, rows, in_dim, out_dim).
+    fn launchDecodeRows(
+        self: *KernelModule,
+        ctx: *context_mod.HipContext,
+        tensor_type: TensorType,
+        dst: buffer_mod.DeviceBuffer,
+        input: buffer_mod.DeviceBuffer,
+        weight_prepared: buffer_mod.DeviceBuffer,
+        rows: usize,
         in_dim: usize,
         out_dim: usize,
     ) driver_mod.Error!void {
@@ -176,13 +354,13 @@ pub const KernelModule = struct {
         const slices = (kb + 127) / 128; // wavefronts that share one column group along K
         const groups = (out_dim + cols - 1) / cols;
         const units: usize = @intCast(@max(ctx.info.compute_units, 1));
-        const groups_per_wg = decodeGroupsPerWorkgroup(groups, slices, units, (kb + 127) / 128);
+        const groups_per_wg = decodeGroupsPerWorkgroup(groups, slices, units, (rows * kb + 127) / 128);
         const grid = (groups + groups_per_wg - 1) / groups_per_wg;
 
         var dst_ptr = dst.ptr;
         var input_ptr = input.ptr;
         var weight_ptr = weight_prepared.ptr;
-        var rows_u32: u32 = 1;
+        var rows_u32 = try toU32(rows);
         var in_dim_u32 = try toU32(in_dim);
         var out_dim_u32 = try toU32(out_dim);
         var groups_u32 = try toU32(groups_per_wg);
@@ -197,8 +375,7 @@ pub const KernelModule = struct {
             @ptrCast(&groups_u32),
             @ptrCast(&stagger_u32),
         };
-        // quantized X (int8 + f32 scale + i32 sum per block) + one partial-sum slot per wavefront and column
-        const lds = in_dim + kb * 8 + 1024;
+        const lds = fusedLdsBytes(rows, in_dim);
         const f = if (tensor_type == .q4_0) self.linear_q4_0_f32 else self.linear_q8_0_f32;
         try launch(ctx, f, .{ try toU32(grid), 1 }, .{ try toU32(64 * slices), try toU32(groups_per_wg) }, try toU32(lds), &params);
     }
@@ -223,6 +400,12 @@ fn decodeGroupsPerWorkgroup(groups: usize, slices: usize, units: usize, x_waves_
         if (g == 1) break;
     }
     return best;
+}
+
+/// LDS of the decode and rows entries: quantized X (int8 + f32 scale + i32 sum per block) and one partial-sum
+/// slot per wavefront, row and column.
+fn fusedLdsBytes(rows: usize, in_dim: usize) usize {
+    return rows * (in_dim + in_dim / block_values * 8) + 256 * @max(rows, 4);
 }
 
 fn launch(
