@@ -392,9 +392,12 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
             }
             counters->activation_quant++;
         }
+        // (the launcher records the end of its quantizer launch for an op that is being timed)
+        void* quantizer_done = counters && counters->phase_events ? counters->phase_events[1] : nullptr;
+        if (quantizer_done) *quantizer_marked = true;
         hipError_t e = launch_batch_mfma(stream, tensor_type, y, x, w, static_cast<int>(rows), static_cast<int>(in_dim),
                                          static_cast<int>(out_dim), reinterpret_cast<uint8_t*>(workspace.ptr), pair ? y_b : nullptr,
-                                         pair ? w_b : nullptr, ep, ep_b);
+                                         pair ? w_b : nullptr, ep, ep_b, quantizer_done);
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     if (layout == AFHIP_LAYOUT_PREPARED && kind == AFHIP_DISPATCH_MM) {

@@ -198,9 +198,15 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
     // instead of fetching their own zeros: a fragment load then touches 2 * kLive * 32 bytes.
     const int lr = lj % (2 * kLive);
     const int alane = lh * 32 + lr;
-    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa);
+    // The fragment and scale loads below have to be issued BEHIND the weight requests above (the wait for the first
+    // fragment is what says that the first half of the weights has landed).  Their addresses are taken from pointers
+    // that pass through a statement ordered after those requests, so no scheduling can lift them above.
+    const uint32_t* qa_behind = qa;
+    const float* sa_behind = sa;
+    asm volatile("" : "+s"(qa_behind), "+s"(sa_behind) : : "memory");
+    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa_behind);
     auto load_a = [&](int rt, int j) { return qa4[(static_cast<size_t>(rt) * kb_full + clamp_blk(j)) * 64 + alane]; };
-    auto load_ta = [&](int rt, int p) { return sa[static_cast<size_t>(clamp_blk(2 * p + lh)) * padded + rt * 32 + lr]; };
+    auto load_ta = [&](int rt, int p) { return sa_behind[static_cast<size_t>(clamp_blk(2 * p + lh)) * padded + rt * 32 + lr]; };
     bm_v4i afrag[kRowTiles][kAhead];
     float ta[kRowTiles][kPairs];  // activation scale of row lj, block 2p + lh
     constexpr int kHalfBlocks = kWB / 2, kHalfPairs = kPairs / 2;
@@ -997,7 +1003,7 @@ void set_batch32_max_workgroups(long bound) { batch32_bound.store(bound, std::me
 
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
                              int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b,
-                             const uint8_t* weight_b_prepared, const Epilogue& ep, const Epilogue& ep_b) {
+                             const uint8_t* weight_b_prepared, const Epilogue& ep, const Epilogue& ep_b, void* quantizer_done) {
     if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim) || workspace == nullptr) return hipErrorInvalidValue;
     const int row_tiles = (rows + 31) / 32, padded = row_tiles * 32, kb = in_dim / 32;
     uint32_t* qa = reinterpret_cast<uint32_t*>(workspace);
@@ -1042,6 +1048,8 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
                                row_tiles, qa, sa);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     }
+    // (an op that is being timed: its activation-quantizer phase ends here)
+    if (quantizer_done != nullptr) (void)hipEventRecord(static_cast<hipEvent_t>(quantizer_done), stream);
     const size_t count = static_cast<size_t>(rows) * out_dim;
     // a pair is one launch over both matrices (grid.z)
     const BmSecond second{dst_b, weight_b_prepared, ep_b};

@@ -95,7 +95,7 @@ void set_batch32_max_workgroups(long bound);
 hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, const float* input, const uint8_t* weight_prepared,
                              int rows, int in_dim, int out_dim, uint8_t* workspace, float* dst_b = nullptr,
                              const uint8_t* weight_b_prepared = nullptr, const Epilogue& ep = Epilogue{},
-                             const Epilogue& ep_b = Epilogue{});
+                             const Epilogue& ep_b = Epilogue{}, void* quantizer_done = nullptr);
 
 // One row, no Y: every workgroup leaves the argmax key (see argmax_key) of its output
 // columns in keys[workgroup]; *key_count receives the number of workgroups, which is at

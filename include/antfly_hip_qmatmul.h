@@ -322,54 +322,6 @@ afhip_status afhip_launch_block_dots(void *stream, int tensor_type, int layout, 
  * (gguf/quant_codec.zig:35-39).  Parity probe for subnormal scales. */
 afhip_status afhip_launch_decode_fp16(void *stream, afhip_buffer dst_f32, afhip_buffer src_u16, size_t n);
 
-/* Diagnostic with no counterpart in the reference: reads src.len bytes (16 per
- * lane, every load issued at once) and does nothing else.  bench.py times it
- * beside the GEMV as "what one launch of this size can draw from HBM", and it is
- * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
-afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
-/* The same read in another launch shape: workgroups of `threads` (a multiple of 64, at most 1024), every lane
- * requesting `loads_per_lane` (1, 2, 4, 8 or 16) x 16 bytes at once, a wavefront's loads covering consecutive KiB;
- * `nontemporal` picks the load hint.  `bench.py --probe read` sweeps it. */
-afhip_status afhip_launch_stream_read_shaped(void *stream, afhip_buffer src, afhip_buffer sink, int threads,
-                                            int loads_per_lane, int nontemporal);
-/* Diagnostic with no counterpart in the reference: the plain copy, dst[0 .. src.len) =
- * src (16 bytes per lane; src.len is rounded down to a multiple of 16, both pointers
- * 16-byte aligned, dst.len >= the copied length).  The kernel of known traffic that
- * WRITE_SIZE readings are scaled against. */
-afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buffer dst);
-/* Diagnostic with no counterpart in the reference: the one-row Q4_0 decode GEMV (PREPARED
- * weight, in_dim <= 4096) with parts left out -- `probe` bit 0: the block dots, bit 1: the
- * store of Y, bit 2: the activation prologue (no X read, no quantization).  probe 0 is the
- * kernel afhip_launch_linear_f32 launches; any other value leaves dst meaningless.  bench.py
- * --probe gemv times the eight variants to show where a launch's time goes. */
-afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
-                                     afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
-/* Tuning, process-wide, no counterpart in the reference: the largest grid (workgroups) for which 9 .. 64 rows on a
- * wide matrix take the 32-row MFMA kernel on 64-column tiles; negative restores the default (one workgroup per
- * compute unit), 0 switches that kernel off.  Tests lift the bound to reach the kernel's K shares and pair launches. */
-afhip_status afhip_tune_batch32_max_workgroups(long bound);
-/* Diagnostic with no counterpart in the reference: the Q8_0 prefill kernel (64 x 128 tiles) on activations
- * already quantized by afhip_launch_quantize_activations, computing as usual but storing, instead of results,
- * eight 32-bit counts per wavefront over the start of `stamps` (which has to hold rows x out_dim floats):
- * [8 * (workgroup * 16 + wavefront)] = shader-clock cycles before the K loop, in it, waiting for the wavefront's
- * own loads, waiting at the workgroup barrier, 100 MHz reference ticks in the loop, cycles after the loop, 0, HW_ID.
- * `bench.py --probe gemm` prints them. */
-afhip_status afhip_launch_gemm_stamps(void *stream, afhip_buffer stamps, afhip_buffer q, afhip_buffer scales,
-                                      afhip_buffer weight_prepared, size_t rows, size_t in_dim, size_t out_dim);
-/* Diagnostic with no counterpart in the reference: what instruction patterns cost a SIMD, timed
- * by the wavefronts themselves.  One workgroup of 256 x `wavefronts_per_simd` (1, 2 or 4) threads
- * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 20, listed in
- * csrc/rate_probe_kernels.hip: vector-ALU instructions, int8 and f32 MFMAs, their mixes inside one
- * wavefront and side by side in two) and stores four 32-bit words into `stamps`
- * [wavefront][4]: shader-clock cycles of its loop, 100 MHz reference ticks of its loop, the
- * HW_ID register and the XCC_ID register (where it ran).  afhip_rate_probe_wavefronts() says how
- * many wavefronts a launch has.  `sink` (16-byte aligned, 256 KiB + 2 MiB + 8 KiB) takes meaningless
- * results and is what the load patterns read.
- * `bench.py --probe rates` prints the table. */
-afhip_status afhip_launch_rate_probe(void *stream, int pattern, int wavefronts_per_simd, int iterations,
-                                     afhip_buffer sink, afhip_buffer stamps);
-size_t afhip_rate_probe_wavefronts(int wavefronts_per_simd);
-
 /* ------------------------------------------------------------------------
  * Backend object: ops/cuda/cuda_compute.zig (CudaCompute + the ComputeBackend
  * vtable entries on this path).  Owns one device context, ONE stream, resident
@@ -635,6 +587,59 @@ afhip_status afhip_compute_set_q4k_f32_activations(afhip_compute *self, int enab
  * cuda_info.zig:57-82). */
 afhip_status afhip_smoke_q8_0(void);
 afhip_status afhip_smoke_q4_0(void);
+
+/* ------------------------------------------------------------------------
+ * Measurement and tuning entry points.  None has a counterpart in the reference and no
+ * engine binding needs them: bench.py and the tests are their only callers.  They live in
+ * the same library so that what they time is the shipped device code, not a copy of it.
+ * ---------------------------------------------------------------------- */
+/* Diagnostic with no counterpart in the reference: reads src.len bytes (16 per
+ * lane, every load issued at once) and does nothing else.  bench.py times it
+ * beside the GEMV as "what one launch of this size can draw from HBM", and it is
+ * the kernel of known traffic that FETCH_SIZE readings are scaled against. */
+afhip_status afhip_launch_stream_read(void *stream, afhip_buffer src, afhip_buffer sink);
+/* The same read in another launch shape: workgroups of `threads` (a multiple of 64, at most 1024), every lane
+ * requesting `loads_per_lane` (1, 2, 4, 8 or 16) x 16 bytes at once, a wavefront's loads covering consecutive KiB;
+ * `nontemporal` picks the load hint.  `bench.py --probe read` sweeps it. */
+afhip_status afhip_launch_stream_read_shaped(void *stream, afhip_buffer src, afhip_buffer sink, int threads,
+                                            int loads_per_lane, int nontemporal);
+/* Diagnostic with no counterpart in the reference: the plain copy, dst[0 .. src.len) =
+ * src (16 bytes per lane; src.len is rounded down to a multiple of 16, both pointers
+ * 16-byte aligned, dst.len >= the copied length).  The kernel of known traffic that
+ * WRITE_SIZE readings are scaled against. */
+afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buffer dst);
+/* Diagnostic with no counterpart in the reference: the one-row Q4_0 decode GEMV (PREPARED
+ * weight, in_dim <= 4096) with parts left out -- `probe` bit 0: the block dots, bit 1: the
+ * store of Y, bit 2: the activation prologue (no X read, no quantization).  probe 0 is the
+ * kernel afhip_launch_linear_f32 launches; any other value leaves dst meaningless.  bench.py
+ * --probe gemv times the eight variants to show where a launch's time goes. */
+afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
+                                     afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* Tuning, process-wide, no counterpart in the reference: the largest grid (workgroups) for which 9 .. 64 rows on a
+ * wide matrix take the 32-row MFMA kernel on 64-column tiles; negative restores the default (one workgroup per
+ * compute unit), 0 switches that kernel off.  Tests lift the bound to reach the kernel's K shares and pair launches. */
+afhip_status afhip_tune_batch32_max_workgroups(long bound);
+/* Diagnostic with no counterpart in the reference: the Q8_0 prefill kernel (64 x 128 tiles) on activations
+ * already quantized by afhip_launch_quantize_activations, computing as usual but storing, instead of results,
+ * eight 32-bit counts per wavefront over the start of `stamps` (which has to hold rows x out_dim floats):
+ * [8 * (workgroup * 16 + wavefront)] = shader-clock cycles before the K loop, in it, waiting for the wavefront's
+ * own loads, waiting at the workgroup barrier, 100 MHz reference ticks in the loop, cycles after the loop, 0, HW_ID.
+ * `bench.py --probe gemm` prints them. */
+afhip_status afhip_launch_gemm_stamps(void *stream, afhip_buffer stamps, afhip_buffer q, afhip_buffer scales,
+                                      afhip_buffer weight_prepared, size_t rows, size_t in_dim, size_t out_dim);
+/* Diagnostic with no counterpart in the reference: what instruction patterns cost a SIMD, timed
+ * by the wavefronts themselves.  One workgroup of 256 x `wavefronts_per_simd` (1, 2 or 4) threads
+ * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 20, listed in
+ * csrc/rate_probe_kernels.hip: vector-ALU instructions, int8 and f32 MFMAs, their mixes inside one
+ * wavefront and side by side in two) and stores four 32-bit words into `stamps`
+ * [wavefront][4]: shader-clock cycles of its loop, 100 MHz reference ticks of its loop, the
+ * HW_ID register and the XCC_ID register (where it ran).  afhip_rate_probe_wavefronts() says how
+ * many wavefronts a launch has.  `sink` (16-byte aligned, 256 KiB + 2 MiB + 8 KiB) takes meaningless
+ * results and is what the load patterns read.
+ * `bench.py --probe rates` prints the table. */
+afhip_status afhip_launch_rate_probe(void *stream, int pattern, int wavefronts_per_simd, int iterations,
+                                     afhip_buffer sink, afhip_buffer stamps);
+size_t afhip_rate_probe_wavefronts(int wavefronts_per_simd);
 
 #ifdef __cplusplus
 }
