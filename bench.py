@@ -411,7 +411,6 @@ def main() -> int:
         return 0
 
     if args.probe == "rates":
-        import numpy as np
         lib = _lib.lib()
         sink = torch.zeros(65536 + (2 << 18) + 2048, dtype=torch.int32, device=dev)
         iterations = 2000
@@ -533,7 +532,6 @@ def main() -> int:
         return 0
 
     if args.probe == "gemm":
-        import numpy as np
         lib = _lib.lib()
         m, k, n = 512, 4096, 4096
         ws = prepared_copies(Q8, n, k, 4, 7)
