@@ -456,7 +456,7 @@ def main() -> int:
             return key
 
         print(f"{iterations} rounds per wavefront; cycles = s_memtime differences read by the wavefronts, clock = cycles / (s_memrealtime ticks / 100 MHz)")
-        print("| pattern (one round) | wavefronts per SIMD | cycles per round and wavefront (median; min-max) | SIMD cycles per instruction | clock GHz | SIMDs hosting exactly that many wavefronts |")
+        print("| pattern (one round) | wavefronts per SIMD | cycles per round and wavefront (median; min-max) | SIMD cycles per instruction (from the SIMD's last wavefront to finish) | clock GHz | SIMDs hosting exactly that many wavefronts |")
         print("|---|---|---|---|---|---|")
         out = {}
         for pattern, name, per_round, wave_counts in patterns:
@@ -476,8 +476,14 @@ def main() -> int:
                     continue
                 cyc = st[:, 0] / iterations
                 med = float(np.median(cyc))
-                print(f"| {name} | {waves} | {med:.1f}; {cyc.min():.1f}-{cyc.max():.1f} | {med / waves / per_round:.2f} | {ghz:.3f} | {exact} of {len(simds)} |")
+                # Throughput of a SIMD: its wavefronts start together and the oldest is served first, so the
+                # work of all of them is done when the last one finishes.
+                order = np.argsort(key, kind="stable")
+                last = np.maximum.reduceat(cyc[order], np.flatnonzero(np.r_[True, np.diff(key[order]) != 0]))
+                busy = float(np.median(last))
+                print(f"| {name} | {waves} | {med:.1f}; {cyc.min():.1f}-{cyc.max():.1f} | {busy / waves / per_round:.2f} | {ghz:.3f} | {exact} of {len(simds)} |")
                 out[f"{name} @{waves}"] = round(med, 2)
+                out[f"{name} @{waves} simd_cycles_per_instruction"] = round(busy / waves / per_round, 2)
         print(json.dumps({"probe": "rates", "cycles_per_round": out}))
         return 0
 
