@@ -963,18 +963,42 @@ afhip_status afhip_launch_stream_copy(void* stream, afhip_buffer src, afhip_buff
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
-afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
-                                     size_t in_dim, size_t out_dim) {
-    if (probe < 0 || probe > 7) return AFHIP_ERR_INVALID_ARGUMENT;
+afhip_status afhip_launch_gemv_probe_rows(void* stream, int probe, size_t rows, afhip_buffer dst, afhip_buffer input,
+                                          afhip_buffer weight, size_t in_dim, size_t out_dim) {
+    if (probe < 0 || probe > 7 || (rows != 1 && rows != 2 && rows != 4)) return AFHIP_ERR_INVALID_ARGUMENT;
     if (in_dim == 0 || in_dim % 32 != 0 || in_dim > 4096 || out_dim == 0 || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
     const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q4_0, out_dim, in_dim);
-    if (need == 0 || weight.len < need || input.len < in_dim * 4 || dst.len < out_dim * 4) return AFHIP_ERR_INVALID_STATE;
+    if (need == 0 || weight.len < need || input.len < rows * in_dim * 4 || dst.len < rows * out_dim * 4) return AFHIP_ERR_INVALID_STATE;
     if (dst.ptr == 0 || input.ptr == 0 || weight.ptr == 0 || dst.ptr % 4 != 0 || input.ptr % 16 != 0 || weight.ptr % 16 != 0)
         return AFHIP_ERR_INVALID_STATE;
-    hipError_t e = launch_gemv_probe(static_cast<hipStream_t>(stream), probe, reinterpret_cast<float*>(dst.ptr),
-                                     reinterpret_cast<const float*>(input.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
-                                     static_cast<int>(in_dim), static_cast<int>(out_dim));
+    hipError_t e = launch_gemv_probe(static_cast<hipStream_t>(stream), probe, static_cast<int>(rows),
+                                     reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const float*>(input.ptr),
+                                     reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(in_dim),
+                                     static_cast<int>(out_dim));
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_launch_gemv_timeline(void* stream, size_t rows, afhip_buffer stamps, afhip_buffer input, afhip_buffer weight,
+                                        size_t in_dim, size_t out_dim, size_t* workgroups, size_t* wavefronts_per_workgroup) {
+    if (rows != 1 && rows != 2 && rows != 4) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || in_dim % 32 != 0 || in_dim > 4096 || out_dim == 0 || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
+    const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q4_0, out_dim, in_dim);
+    if (need == 0 || weight.len < need || input.len < rows * in_dim * 4) return AFHIP_ERR_INVALID_STATE;
+    if (stamps.ptr == 0 || stamps.ptr % 4 != 0 || input.ptr == 0 || weight.ptr == 0 || input.ptr % 16 != 0 || weight.ptr % 16 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    int grid = 0, waves = 0;
+    hipError_t e = launch_gemv_probe(static_cast<hipStream_t>(stream), 8, static_cast<int>(rows), nullptr,
+                                     reinterpret_cast<const float*>(input.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
+                                     static_cast<int>(in_dim), static_cast<int>(out_dim), reinterpret_cast<uint32_t*>(stamps.ptr),
+                                     stamps.len, &grid, &waves);
+    if (workgroups) *workgroups = static_cast<size_t>(grid);
+    if (wavefronts_per_workgroup) *wavefronts_per_workgroup = static_cast<size_t>(waves);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
+afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
+                                     size_t in_dim, size_t out_dim) {
+    return afhip_launch_gemv_probe_rows(stream, probe, 1, dst, input, weight, in_dim, out_dim);
 }
 
 afhip_status afhip_tune_batch32_max_workgroups(long bound) {
@@ -1003,7 +1027,7 @@ afhip_status afhip_launch_gemm_stamps(void* stream, afhip_buffer stamps, afhip_b
 
 afhip_status afhip_launch_rate_probe(void* stream, int pattern, int wavefronts_per_simd, int iterations, afhip_buffer sink,
                                      afhip_buffer stamps) {
-    if (pattern < 0 || pattern > 20 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2 && wavefronts_per_simd != 4) ||
+    if (pattern < 0 || pattern > 23 || (wavefronts_per_simd != 1 && wavefronts_per_simd != 2 && wavefronts_per_simd != 4) ||
         iterations < 1 || iterations > (1 << 20))
         return AFHIP_ERR_INVALID_ARGUMENT;
     if (sink.ptr == 0 || sink.ptr % 16 != 0 || sink.len < 65536 * 4 + (2u << 20) + 8192) return AFHIP_ERR_INVALID_STATE;

@@ -69,7 +69,12 @@ struct GemvTargets {
 //   kProbe:     timing diagnostics (afhip_launch_gemv_probe), results meaningless: bit 0 leaves
 //               out the block dots (one xor per weight register keeps the loads alive), bit 1
 //               the store of Y, bit 2 the activation prologue (no X is read, LDS is used as found)
-constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4;
+//               bit 3 (alone): nothing is left out, but instead of Y every wavefront stores eight readings of the 100 MHz
+//               clock at extras.dots[8 * (workgroup * wavefronts + wavefront)]: [0] entry, [1] past the wait for the
+//               quantized activations (barrier or counter), [2] block dots done, [3] reduction done; quantizing
+//               wavefronts of a counter launch also [4] past the barrier behind the requests for X, [5] X there,
+//               [6] blocks quantized
+constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4, kProbeTimeline = 8;
 template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
 __device__ __forceinline__ void gemv_fused_body(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
@@ -87,12 +92,24 @@ __device__ __forceinline__ void gemv_fused_body(
     constexpr int kSteps = F::kSteps;
 
     extern __shared__ __align__(16) unsigned char lds[];
+    uint32_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // kProbeTimeline: 100 MHz clock readings, see below
+    if (kProbe & kProbeTimeline) stamp[0] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     const int in_dim = kb << 5;
     const int row_dwords = kb << 3;
     int* qx = reinterpret_cast<int*>(lds);                                           // [kRows][in_dim] bytes
     float* sx = reinterpret_cast<float*>(lds + static_cast<size_t>(kRows) * in_dim);  // [kRows][kb]
     int* sumx = reinterpret_cast<int*>(sx + kRows * kb);                              // [kRows][kb]
     float* partial = reinterpret_cast<float*>(sumx + kRows * kb);                     // [waves][kRows*kCols]
+
+    // [0] = wavefronts that have finished quantizing their blocks of X; 16 bytes in front of the staging area
+    const uint32_t flag_off = (static_cast<uint32_t>(kRows) * in_dim + static_cast<uint32_t>(kRows) * kb * 8 +
+                               16 * (kRows < 4 ? 4 : kRows) * 16 + 15) & ~15u;
+    uint32_t* ready = reinterpret_cast<uint32_t*>(lds + flag_off);
+    // Several rows, and wavefronts that do not quantize (the host decides): the quantizers' blocks are waited for
+    // through a counter in LDS instead of a barrier (below).
+    // (one row of at most 4096 values never takes the counter: that instantiation does not carry its code)
+    const bool ready_counter = !(kRows == 1 && kCompact) && (shape & kGemvReadyCounter) != 0;  // wave-uniform
+    if (ready_counter && threadIdx.x == 0 && threadIdx.y == 0) *ready = 0;  // (the barrier that publishes it is further down)
 
     const int lane = threadIdx.x & (kWave - 1);
     // wavefront-uniform values live in scalar registers, so column base addresses
@@ -152,43 +169,120 @@ __device__ __forceinline__ void gemv_fused_body(
             wq[j][c] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(qcol + lane_off[j]));
         }
     };
-    if (!(kProbe & kProbeNoPrologue) && wave * kWave < x_blocks) {  // wave-uniform
-        const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
-        const bool two = !kCompact && x_blocks > threads;    // uniform: a second block per thread
-        const int xb1 = min(tid + threads, x_blocks - 1);
-        float4 v[8], v1[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
-        if (two) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) v1[i] = reinterpret_cast<const float4*>(input)[xb1 * 8 + i];
+    // With more than one row several wavefronts quantize, and the memory pipeline serves requests in the order it
+    // accepted them: a quantizer whose requests for X queued behind other wavefronts' weight requests gets X after
+    // those kilobytes.  So nobody asks for weights before every quantizer has asked for X: one barrier, reached within
+    // a few instructions by everybody (it also publishes the cleared counter).
+    auto x_requests_first = [&]() {
+        if (ready_counter) {
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            if (kProbe & kProbeTimeline) stamp[4] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
         }
-        __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
-        request_weights();
-        __builtin_amdgcn_sched_barrier(0);
-        const int r = xb / kb, b = xb - r * kb;
-        quantize_block_to_lds<kType, true>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
-        if (two) {
-            const int r1 = xb1 / kb, b1 = xb1 - r1 * kb;
-            quantize_block_to_lds<kType, true>(v1, b1, kb, qx + r1 * row_dwords, sx + r1 * kb, sumx + r1 * kb);
+    };
+    if (!(kProbe & kProbeNoPrologue) && wave * kWave < x_blocks) {  // wave-uniform
+        if (ready_counter) {
+            // (The host sets the counter bit only when some wavefront does not quantize: one block a thread at most.)
+            // A thread quantizes block `tid` but does not fetch it itself: the wavefront reads its 64 blocks as eight
+            // contiguous kilobytes (lane l takes 16-byte chunk 64 i + l), passes them through 8 KB of LDS of its own
+            // (chunk c of block b in slot c ^ ((b >> 1) & 7) of the block's eight: the per-thread reads that follow are
+            // conflict-free) and each thread picks up its block.  No other wavefront touches that region: no barrier.
+            // The requests are inline assembly so that they leave here, ahead of every weight request, whatever the
+            // compiler would make of loads whose values are first needed much later; it does not count them, hence
+            // the wait by hand: all but the weight requests issued in between.
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            f32x4* stage = reinterpret_cast<f32x4*>(lds + flag_off + 16) + wave * 512;
+            const int last_chunk = x_blocks * 8 - 1;
+            f32x4 t[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const uint32_t off = static_cast<uint32_t>(min(wave * 512 + i * 64 + lane, last_chunk)) * 16u;
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(t[i]) : "v"(off), "s"(input) : "memory");
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            x_requests_first();
+            request_weights();
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("s_waitcnt vmcnt(%8)"
+                         : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7])
+                         : "n"(kCols * kSteps + 1)
+                         : "memory");
+            if (kProbe & kProbeTimeline) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int g = i * 64 + lane, b = g >> 3, c = g & 7;
+                stage[b * 8 + (c ^ ((b >> 1) & 7))] = t[i];
+            }
+            float4 v[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const f32x4 got = stage[lane * 8 + (c ^ ((lane >> 1) & 7))];
+                v[c] = make_float4(got.x, got.y, got.z, got.w);
+            }
+            if (tid < x_blocks) {
+                const int r = tid / kb, b = tid - r * kb;
+                quantize_block_to_lds<kType, true>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+            }
+        } else {
+            const int xb = tid < x_blocks ? tid : x_blocks - 1;  // spare lanes of the last such wavefront repeat its last block
+            const bool two = !kCompact && x_blocks > threads;    // uniform: a second block per thread
+            const int xb1 = min(tid + threads, x_blocks - 1);
+            float4 v[8], v1[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb * 8 + i];
+            if (two) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) v1[i] = reinterpret_cast<const float4*>(input)[xb1 * 8 + i];
+            }
+            __builtin_amdgcn_sched_barrier(0);  // keep these requests ahead of the weight requests
+            x_requests_first();
+            request_weights();
+            __builtin_amdgcn_sched_barrier(0);
+            const int r = xb / kb, b = xb - r * kb;
+            quantize_block_to_lds<kType, true>(v, b, kb, qx + r * row_dwords, sx + r * kb, sumx + r * kb);
+            if (two) {
+                const int r1 = xb1 / kb, b1 = xb1 - r1 * kb;
+                quantize_block_to_lds<kType, true>(v1, b1, kb, qx + r1 * row_dwords, sx + r1 * kb, sumx + r1 * kb);
+            }
         }
         // more than two blocks per thread (not a shape the host sends here): these requests
         // queue behind the weights
         for (int xb2 = tid + 2 * threads; !kCompact && xb2 < x_blocks; xb2 += threads) {
+            float4 v[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) v[i] = reinterpret_cast<const float4*>(input)[xb2 * 8 + i];
             const int r2 = xb2 / kb, b2 = xb2 - r2 * kb;
             quantize_block_to_lds<kType, true>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
         }
+        if (kProbe & kProbeTimeline) stamp[6] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+        if (ready_counter) {  // this wavefront's blocks are in LDS: say so
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            if (lane == 0) __hip_atomic_fetch_add(ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+
     } else {
         // The requests of a unit's wavefronts queue at its one texture addresser.  Left alone
         // they interleave, every wavefront's last bytes arrive at the very end and all of them
         // finish their arithmetic at once; entering the queue one after the other, a wavefront
         // gets its bytes in a burst and only the last one still computes when the stream ends.
+        x_requests_first();
         for (int q = 0; q < wave * stagger; ++q) __builtin_amdgcn_s_sleep(1);
         request_weights();
     }
-    __syncthreads();
+    // No barrier here.  A wavefront is through its requests only when the memory pipeline has accepted them all,
+    // which for the last wavefronts of a unit is halfway through the stream; a barrier would hold the first ones,
+    // whose bytes are long there, until then, and all the arithmetic would be done in the second half.  Each
+    // wavefront waits for the quantizers alone (they depend on nobody: the loop ends).
+    if (!ready_counter) {
+        __syncthreads();
+    } else if (!(kProbe & kProbeNoPrologue)) {
+        const uint32_t quantizers = static_cast<uint32_t>(min(waves, (x_blocks + kWave - 1) / kWave));
+        // (bounded all the same: a wavefront that gave up would compute on what LDS holds and still end)
+        for (int spin = 0; spin < (1 << 22) && __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < quantizers; ++spin)
+            __builtin_amdgcn_s_sleep(2);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+    if (kProbe & kProbeTimeline) stamp[1] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     wd.exchange();
 
     // ---- 3. block dots and scaled accumulation (the weights stay packed in registers)
@@ -283,6 +377,10 @@ __device__ __forceinline__ void gemv_fused_body(
         }
     }
 
+    if (kProbe & kProbeTimeline) {
+        asm volatile("" : "+v"(acc[0][0]), "+v"(acc[kRows - 1][kCols - 1]));
+        stamp[2] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+    }
     // ---- 4. wavefront reduction (all rows x columns at once)
     constexpr int kPadded = pow2_at_least(kCells);
     static_assert(kCells <= 16, "at most 16 accumulators per lane and reduction");
@@ -305,6 +403,15 @@ __device__ __forceinline__ void gemv_fused_body(
         }
         float* dst = second ? dst_b : dst_a;
         if ((kProbe & kProbeNoStore) && red[0] != 1234.5f) return;  // (keeps the arithmetic alive)
+        if (kProbe & kProbeTimeline) {
+            stamp[3] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+            if (lane == 0 && red[0] != 1234.5f) {  // (keeps the arithmetic alive)
+                uint32_t* o = reinterpret_cast<uint32_t*>(extras.dots) + (static_cast<size_t>(blockIdx.x) * waves + wave) * 8;
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o[k] = stamp[k];
+            }
+            return;
+        }
         if (active && mine && o0 + cc < out_dim && dst) {
             const size_t at = static_cast<size_t>(cr) * out_dim + o0 + cc;
             float v = red[0];
@@ -632,6 +739,15 @@ hipError_t allow_large_lds(Kernel kernel, size_t lds, std::atomic<size_t>* limit
     return e;
 }
 
+// Whether a fused launch waits for its quantizing wavefronts through the LDS counter (kGemvReadyCounter) instead of a
+// barrier: only when some wavefront does not quantize, and for one row only when it is long (measured: a gain from
+// K = 6144 on, a small loss on one row of 4096 values, whose two quantizers are done before the barrier matters).
+bool use_ready_counter(int rows, int x_blocks, int waves) {
+    return waves > (x_blocks + 63) / 64 && (rows >= 2 || x_blocks >= 192);
+}
+// LDS behind the fused kernel's own: 16 bytes of counter, the f32 staging of X (8 KB per quantizing wavefront), alignment
+size_t ready_counter_lds_bytes(int x_blocks) { return 32 + static_cast<size_t>((x_blocks + 63) / 64) * 8192; }
+
 template <int kType, int kRows, bool kDots, bool kArgmax = false>
 hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, const float* input, int in_dim,
                         int out_dim, const GemvTuning& tune, unsigned long long* keys = nullptr, int* key_count = nullptr) {
@@ -649,7 +765,10 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
         (groups + waves / slices - 1) / (waves / slices) > compute_units() * 3)
         waves = workgroup_waves(512, 512, slices, groups, true);  // many rounds: nothing to balance
     const int groups_per_wg = waves / slices;
-    const size_t lds = gemv_fused_lds_bytes(kRows, in_dim);
+    // Several rows, or one long row, and wavefronts that do not quantize: those wait for the quantizers through a
+    // counter, not at a barrier (and X passes through 8 KB of LDS per quantizing wavefront on its way in).
+    const bool ready_counter = use_ready_counter(kRows, x_blocks, waves);
+    const size_t lds = gemv_fused_lds_bytes(kRows, in_dim) + (ready_counter ? ready_counter_lds_bytes(x_blocks) : 0);
     const bool compact = slices == 1 && tg.weight_b == nullptr && x_blocks <= waves * 64;
     auto kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true>
                           : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false>;
@@ -664,7 +783,7 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     const size_t tile_off = tile_scales_offset(kType, static_cast<size_t>(out_dim) * (in_dim / 32));
     if ((tile_off >> 4) > 0xFFFFFFFFull || slices > 255 || groups_per_wg > 255) return hipErrorInvalidValue;
     const uint32_t shape = static_cast<uint32_t>(slices) | static_cast<uint32_t>(groups_per_wg) << 8 |
-                           static_cast<uint32_t>(stagger) << 16 | (has_epilogue(tg.ep_a) ? kGemvHasEpilogueA : 0u) |
+                           static_cast<uint32_t>(stagger) << 16 | (ready_counter ? kGemvReadyCounter : 0u) | (has_epilogue(tg.ep_a) ? kGemvHasEpilogueA : 0u) |
                            (has_epilogue(tg.ep_b) ? kGemvHasEpilogueB : 0u);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * slices, groups_per_wg), lds, stream, tg.weight_a, tg.weight_b, input, tg.dst_a,
                        tg.dst_b, static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);
@@ -718,8 +837,8 @@ hipError_t launch_gemv_type(hipStream_t stream, const GemvTargets& tg, int* dots
 // quantized X (int8 + f32 scale + i32 sum per block) plus, for each of up to 16
 // wavefronts, one partial-sum slot per (row, column) it owns (at most 4 columns)
 size_t gemv_fused_lds_bytes(int rows, int in_dim) {
-    return static_cast<size_t>(rows) * in_dim + static_cast<size_t>(rows) * (in_dim / 32) * 8 +
-           static_cast<size_t>(16) * (rows < 4 ? 4 : rows) * 4 * 4;
+    const size_t x_blocks = static_cast<size_t>(rows) * (in_dim / 32);
+    return static_cast<size_t>(rows) * in_dim + x_blocks * 8 + static_cast<size_t>(16) * (rows < 4 ? 4 : rows) * 4 * 4;
 }
 
 int gemv_fused_max_in_dim() { return 16 * kSliceBlocks * 32; }
@@ -735,29 +854,55 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
     return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
 
-// Timing diagnostics on the one-row Q4_0 kernel (compact instantiation: in_dim <= 4096).
-hipError_t launch_gemv_probe(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
-                             int in_dim, int out_dim) {
+// Timing diagnostics on the Q4_0 decode kernel for one, two and four rows (compact instantiation: in_dim <= 4096).
+namespace {
+template <int kRows>
+hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
+                                  int in_dim, int out_dim, uint32_t* stamps, size_t stamps_bytes, int* grid_out, int* waves_out) {
     constexpr int kCols = 4;
-    if (in_dim > kSliceBlocks * 32 || probe < 0 || probe > 7) return hipErrorInvalidValue;
     const int groups = (out_dim + kCols - 1) / kCols;
-    const int waves = workgroup_waves(1024, 1024, 1, groups, false, 2);
+    const int x_blocks = kRows * (in_dim / 32);
+    const int waves = workgroup_waves(1024, 1024, 1, groups, false, (x_blocks + 127) / 128);
+    if (x_blocks > waves * 64) return hipErrorInvalidValue;  // the compact instantiation: one block of X per thread
     const int grid = (groups + waves - 1) / waves;
     const size_t tile_off = tile_scales_offset(2, static_cast<size_t>(out_dim) * (in_dim / 32));
-    const uint32_t shape = 1u | static_cast<uint32_t>(waves) << 8 | (grid <= compute_units() ? 1u << 16 : 0u);
-    const GemvExtras extras{nullptr, nullptr, Epilogue{}, Epilogue{}};
-    const size_t lds = gemv_fused_lds_bytes(1, in_dim);
+    const bool ready_counter = use_ready_counter(kRows, x_blocks, waves);
+    const uint32_t shape = 1u | static_cast<uint32_t>(waves) << 8 | (grid <= compute_units() ? 1u << 16 : 0u) |
+                           (ready_counter ? kGemvReadyCounter : 0u);
+    if (grid_out) *grid_out = grid;
+    if (waves_out) *waves_out = waves;
+    if (probe == kProbeTimeline && (stamps == nullptr || stamps_bytes < static_cast<size_t>(grid) * waves * 32)) return hipErrorInvalidValue;
+    const GemvExtras extras{reinterpret_cast<int*>(stamps), nullptr, Epilogue{}, Epilogue{}};
+    const size_t lds = gemv_fused_lds_bytes(kRows, in_dim) + (ready_counter ? ready_counter_lds_bytes(x_blocks) : 0);
+    static std::atomic<size_t> lds_limit[9] = {{64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024},
+                                               {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
 #define AFHIP_PROBE(P)                                                                                                  \
-    case P:                                                                                                             \
-        hipLaunchKernelGGL((gemv_fused_kernel<2, 1, kCols, false, false, true, P>), dim3(grid), dim3(64, waves), lds, stream, \
-                           weight_prepared, static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),     \
-                           static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);                   \
-        break;
+    case P: {                                                                                                           \
+        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, true, P>;                                        \
+        if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[P]); e != hipSuccess) return e;                      \
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(64, waves), lds, stream, weight_prepared,                           \
+                           static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),              \
+                           static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);                  \
+        break;                                                                                                          \
+    }
     switch (probe) {
-        AFHIP_PROBE(0) AFHIP_PROBE(1) AFHIP_PROBE(2) AFHIP_PROBE(3) AFHIP_PROBE(4) AFHIP_PROBE(5) AFHIP_PROBE(6) AFHIP_PROBE(7)
+        AFHIP_PROBE(0) AFHIP_PROBE(1) AFHIP_PROBE(2) AFHIP_PROBE(3) AFHIP_PROBE(4) AFHIP_PROBE(5) AFHIP_PROBE(6) AFHIP_PROBE(7) AFHIP_PROBE(8)
     }
 #undef AFHIP_PROBE
     return hipGetLastError();
+}
+}  // namespace
+
+hipError_t launch_gemv_probe(hipStream_t stream, int probe, int rows, float* dst, const float* input,
+                             const uint8_t* weight_prepared, int in_dim, int out_dim, uint32_t* stamps, size_t stamps_bytes,
+                             int* grid_out, int* waves_out) {
+    if (in_dim > kSliceBlocks * 32 || probe < 0 || probe > 8) return hipErrorInvalidValue;
+    switch (rows) {
+        case 1: return launch_gemv_probe_rows<1>(stream, probe, dst, input, weight_prepared, in_dim, out_dim, stamps, stamps_bytes, grid_out, waves_out);
+        case 2: return launch_gemv_probe_rows<2>(stream, probe, dst, input, weight_prepared, in_dim, out_dim, stamps, stamps_bytes, grid_out, waves_out);
+        case 4: return launch_gemv_probe_rows<4>(stream, probe, dst, input, weight_prepared, in_dim, out_dim, stamps, stamps_bytes, grid_out, waves_out);
+        default: return hipErrorInvalidValue;
+    }
 }
 
 hipError_t launch_gemv_argmax_keys(hipStream_t stream, int tensor_type, unsigned long long* keys, int* key_count,

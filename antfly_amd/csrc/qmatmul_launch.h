@@ -196,10 +196,12 @@ hipError_t launch_gemm_q4k_tiled(hipStream_t stream, float* dst, const float* x,
 hipError_t launch_dequantize_q4k_tiled_rows(hipStream_t stream, float* dst, const uint8_t* weight, const long long* ids,
                                             size_t rows, int dim, size_t weight_rows);
 
-// The one-row Q4_0 decode kernel with parts left out (bit 0: the block dots, bit 1: the store of Y,
-// bit 2: the activation prologue): timing diagnostics, results meaningless.  in_dim <= 4096.
-hipError_t launch_gemv_probe(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
-                             int in_dim, int out_dim);
+// The Q4_0 decode kernel (one, two or four rows, in_dim <= 4096) with parts left out (bit 0: the block dots, bit 1: the
+// store of Y, bit 2: the activation prologue; results meaningless), or, probe 8, complete but storing eight 100 MHz
+// clock readings per wavefront into `stamps` (32 bytes per wavefront of the launch) instead of Y.
+hipError_t launch_gemv_probe(hipStream_t stream, int probe, int rows, float* dst, const float* input, const uint8_t* weight_prepared,
+                             int in_dim, int out_dim, uint32_t* stamps = nullptr, size_t stamps_bytes = 0, int* grid_out = nullptr,
+                             int* waves_out = nullptr);
 
 hipError_t launch_stream_read(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes);
 hipError_t launch_stream_read_shaped(hipStream_t stream, const uint8_t* src, uint32_t* sink, size_t bytes, int threads,

@@ -32,6 +32,8 @@ typedef float rate_v32f __attribute__((ext_vector_type(32)));
     asm volatile("v_cvt_f32_i32 %1, %3\n\tv_fma_f32 %0, %2, %1, %0" : "+v"(ACC), "+v"(TMP) : "v"(T), "v"(SRC))
 #define RATE_SUB_FMA(ACC, T, SRC, TMP) \
     asm volatile("v_sub_f32 %1, %3, %4\n\tv_fma_f32 %0, %2, %1, %0" : "+v"(ACC), "+v"(TMP) : "v"(T), "v"(SRC), "v"(fb))
+#define RATE_DOT8(ACC, A, B) asm volatile("v_dot8_i32_i4 %0, %1, %2, %0" : "+v"(ACC) : "v"(A), "v"(B))
+#define RATE_DOT4(ACC, A, B) asm volatile("v_dot4_i32_i8 %0, %1, %2, %0" : "+v"(ACC) : "v"(A), "v"(B))
 #define RATE_MFMA_I8(ACC) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, %0" : "+v"(ACC) : "v"(ma), "v"(mb))
 #define RATE_MFMA_I8_FRESH(ACC) asm volatile("v_mfma_i32_32x32x32_i8 %0, %1, %2, 0" : "=v"(ACC) : "v"(ma), "v"(mb))
 #define RATE_MFMA_F32(ACC) asm volatile("v_mfma_f32_32x32x1_2b_f32 %0, %1, %2, %0" : "+v"(ACC) : "v"(fa), "v"(fb))
@@ -65,6 +67,8 @@ typedef float rate_v32f __attribute__((ext_vector_type(32)));
 //     comes from L2), waited for together
 // 20  8 global_load_dwordx4 into registers, waited for, then 8 ds_write_b128: the same bytes as 17 by way
 //     of the register file
+// 21  32 v_dot8_i32_i4 into 32 accumulators     22  8 chains of 4 v_dot8_i32_i4 into one accumulator each
+//     (the decode kernel's block dot)            23  32 v_dot4_i32_i8 into 32 accumulators
 template <int kPattern, int kThreads>
 __global__ __launch_bounds__(kThreads) void rate_probe_kernel(uint32_t* __restrict__ stamps, int* __restrict__ sink,
                                                           int iterations, int seed) {
@@ -110,6 +114,15 @@ __global__ __launch_bounds__(kThreads) void rate_probe_kernel(uint32_t* __restri
         } else if (kPattern == 2) {
 #pragma unroll
             for (int i = 0; i < 32; ++i) RATE_SUB(facc[i], iacc[i]);
+        } else if (kPattern == 21) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) RATE_DOT8(iacc[i], a, b);
+        } else if (kPattern == 22) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) RATE_DOT8(iacc[i / 4], a, b);
+        } else if (kPattern == 23) {
+#pragma unroll
+            for (int i = 0; i < 32; ++i) RATE_DOT4(iacc[i], a, b);
         } else if (kPattern == 3) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -266,7 +279,7 @@ hipError_t launch_rate_probe(hipStream_t stream, int pattern, int wavefronts_per
         AFHIP_RATE_CASE(0) AFHIP_RATE_CASE(1) AFHIP_RATE_CASE(2) AFHIP_RATE_CASE(3) AFHIP_RATE_CASE(4) AFHIP_RATE_CASE(5)
         AFHIP_RATE_CASE(6) AFHIP_RATE_CASE(7) AFHIP_RATE_CASE(8) AFHIP_RATE_CASE(9) AFHIP_RATE_CASE(10) AFHIP_RATE_CASE(11)
         AFHIP_RATE_CASE(12) AFHIP_RATE_CASE(13) AFHIP_RATE_CASE(14) AFHIP_RATE_CASE(15) AFHIP_RATE_CASE(16) AFHIP_RATE_CASE(17) AFHIP_RATE_CASE(18)
-        AFHIP_RATE_CASE(19) AFHIP_RATE_CASE(20)
+        AFHIP_RATE_CASE(19) AFHIP_RATE_CASE(20) AFHIP_RATE_CASE(21) AFHIP_RATE_CASE(22) AFHIP_RATE_CASE(23)
         default: return hipErrorInvalidValue;
     }
 #undef AFHIP_RATE_CASE

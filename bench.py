@@ -109,9 +109,11 @@ def main() -> int:
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k; q4p / q8p: pair calls): time only these calls, print one line each, exit")
-    ap.add_argument("--probe", choices=["gemv", "rates", "gemm", "read"], default=None,
-                    help="read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+    ap.add_argument("--probe", choices=["gemv", "rates", "gemm", "read", "timeline"], default=None,
+                    help="timeline: the Q4_0 decode kernel's wavefronts read the 100 MHz clock at their phases (afhip_launch_gemv_timeline; --probe-rows 1, 2 or 4): when the quantized activations are ready, when a wavefront's block dots are done; read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
+    ap.add_argument("--probe-rows", type=int, choices=[1, 2, 4], default=1,
+                    help="--probe gemv: rows of X (the decode kernel's instantiation for that many rows)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -420,6 +422,9 @@ def main() -> int:
             (1, "32 v_cvt_f32_i32", 32, (1, 2, 4)),
             (2, "32 v_sub_f32", 32, (1, 2, 4)),
             (3, "16 x (v_cvt_f32_i32 -> v_fma_f32 that consumes it)", 32, (1, 2, 4)),
+            (21, "32 v_dot8_i32_i4, 32 accumulators", 32, (1, 2, 4)),
+            (22, "32 v_dot8_i32_i4, 8 chains of 4 (the decode kernel's block dot)", 32, (1, 2, 4)),
+            (23, "32 v_dot4_i32_i8, 32 accumulators", 32, (1, 2, 4)),
             (4, "4 v_mfma_i32_32x32x32_i8", 4, (1, 2, 4)),
             (5, "2 v_mfma_f32_32x32x1_2b_f32", 2, (1, 2, 4)),
             (6, "4 x (int8 MFMA + 8 v_fma_f32), one wavefront", 4, (1, 2, 4)),
@@ -575,11 +580,46 @@ def main() -> int:
                           "barrier_cycles_median": int(np.median(st[:, :, 3])), "load_wait_cycles_median": int(np.median(st[:, :, 2]))}))
         return 0
 
+    if args.probe == "timeline":
+        import ctypes
+        lib = _lib.lib()
+        in_dim, out_dim, copies, prows = 4096, 14336, args.copies, args.probe_rows
+        ws = prepared_copies(Q4, out_dim, in_dim, copies, 2024)
+        x = torch.from_numpy(synth.activations(2025, prows, in_dim)).to(dev)
+        stamps = torch.zeros(1 << 18, dtype=torch.int32, device=dev)
+        groups, waves = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        for i in range(64):  # back to back, weights rotating; the last launch's readings are the ones looked at
+            rc = lib.afhip_launch_gemv_timeline(stream, prows, buf(stamps), buf(x), buf(ws[i % copies]), in_dim, out_dim,
+                                                ctypes.byref(groups), ctypes.byref(waves))
+            if rc != 0:
+                raise RuntimeError(f"timeline probe failed: {rc}")
+        torch.cuda.synchronize()
+        g, w = groups.value, waves.value
+        st = stamps.cpu().numpy().view(np.uint32)[: g * w * 8].reshape(g, w, 8).astype(np.int64)
+        t0 = st[:, :, 0].min()
+        ns = (st - t0) * 10
+        ns[st == 0] = -1  # a reading that wavefront does not take
+        print(f"Q4_0 decode kernel, {prows} row(s), K={in_dim}, N={out_dim}: {g} workgroups x {w} wavefronts; ns after the launch's first wavefront began, median over workgroups")
+        print("| wavefront | begins | activations ready | block dots done | reduction done | (quantizer) past the barrier behind its requests for X | X arrived | blocks quantized |")
+        print("|---|---|---|---|---|---|---|---|")
+        for wv in range(w):
+            cells = []
+            for k in (0, 1, 2, 3, 4, 5, 6):
+                col = ns[:, wv, k]
+                cells.append("" if (col < 0).all() else str(int(np.median(col[col >= 0]))))
+            print(f"| {wv} | " + " | ".join(cells) + " |")
+        first = ns[:, :, 0].min(axis=1)
+        print(f"workgroups begin {int(first.min())} .. {int(first.max())} ns (median {int(np.median(first))}); the last wavefront of the launch ends at {int(ns[:, :, 3].max())} ns")
+        print(json.dumps({"probe": "timeline", "rows": prows, "workgroups": g, "wavefronts": w, "activations_ready_ns_median": int(np.median(ns[:, :, 1])),
+                          "launch_ends_ns": int(ns[:, :, 3].max())}))
+        return 0
+
     if args.probe == "gemv":
         in_dim, out_dim, copies, per_graph, replays = 4096, 14336, args.copies, 100, 10
         ws = prepared_copies(Q4, out_dim, in_dim, copies, 2024)
-        x = torch.from_numpy(synth.activations(2025, 1, in_dim)).to(dev)
-        y = torch.empty((1, out_dim), dtype=torch.float32, device=dev)
+        prows = args.probe_rows
+        x = torch.from_numpy(synth.activations(2025, prows, in_dim)).to(dev)
+        y = torch.empty((prows, out_dim), dtype=torch.float32, device=dev)
         sink = torch.zeros(4, dtype=torch.int32, device=dev)
         w_bytes = out_dim * (in_dim // 32) * 18
         lib = _lib.lib()
@@ -614,16 +654,17 @@ def main() -> int:
                  5: "without prologue and dots", 6: "without prologue and store", 7: "loads and the wavefront reduction only"}
         for probe in range(8):
             def call(i, st, probe=probe):
-                rc = lib.afhip_launch_gemv_probe(st, probe, buf(y), buf(x), buf(ws[i % copies]), in_dim, out_dim)
+                rc = lib.afhip_launch_gemv_probe_rows(st, probe, prows, buf(y), buf(x), buf(ws[i % copies]), in_dim, out_dim)
                 if rc != 0:
                     raise RuntimeError(f"probe failed: {rc}")
             rows_out.append((f"probe {probe}: {names[probe]}", timed(call)))
-        nbytes = gemv_bytes(Q4, 1, in_dim, out_dim)
+        nbytes = gemv_bytes(Q4, prows, in_dim, out_dim)
+        print(f"rows of X: {prows}")
         print("| variant | us per launch | GB/s | % of 8 TB/s |")
         print("|---|---|---|---|")
         for name, us in rows_out:
             print(f"| {name} | {us:.3f} | {nbytes / us / 1e3:.0f} | {nbytes / us / 1e3 / 80:.1f} |")
-        print(json.dumps({"probe": "gemv", "us_per_launch": {n: round(u, 3) for n, u in rows_out}}))
+        print(json.dumps({"probe": "gemv", "rows": prows, "us_per_launch": {n: round(u, 3) for n, u in rows_out}}))
         return 0
 
     if args.counter_probe:

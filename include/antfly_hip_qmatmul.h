@@ -615,6 +615,19 @@ afhip_status afhip_launch_stream_copy(void *stream, afhip_buffer src, afhip_buff
  * --probe gemv times the eight variants to show where a launch's time goes. */
 afhip_status afhip_launch_gemv_probe(void *stream, int probe, afhip_buffer dst, afhip_buffer input,
                                      afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* The same for `rows` = 1, 2 or 4 rows of X (input [rows][in_dim], dst [rows][out_dim]): the decode kernel's
+ * instantiations that quantize two and four rows in their prologue. */
+afhip_status afhip_launch_gemv_probe_rows(void *stream, int probe, size_t rows, afhip_buffer dst, afhip_buffer input,
+                                          afhip_buffer weight_prepared, size_t in_dim, size_t out_dim);
+/* The same kernel, complete, but storing instead of Y eight 32-bit readings of the 100 MHz clock per wavefront at
+ * stamps[8 * (workgroup * wavefronts_per_workgroup + wavefront)]: [0] entry, [1] past the wait for the quantized
+ * activations (a barrier, or for several rows a counter in LDS), [2] block dots done, [3] wavefront reduction done; the
+ * quantizing wavefronts of a counter launch also [4] past the barrier behind their requests for X, [5] X arrived,
+ * [6] their blocks quantized.  The launch geometry comes back through the two pointers; `stamps` too small for it
+ * (32 bytes per wavefront) is refused.  `bench.py --probe timeline` prints the table. */
+afhip_status afhip_launch_gemv_timeline(void *stream, size_t rows, afhip_buffer stamps, afhip_buffer input,
+                                        afhip_buffer weight_prepared, size_t in_dim, size_t out_dim, size_t *workgroups,
+                                        size_t *wavefronts_per_workgroup);
 /* Tuning, process-wide, no counterpart in the reference: the largest grid (workgroups) for which 9 .. 64 rows on a
  * wide matrix take the 32-row MFMA kernel on 64-column tiles; negative restores the default (one workgroup per
  * compute unit), 0 switches that kernel off.  Tests lift the bound to reach the kernel's K shares and pair launches. */
@@ -629,7 +642,7 @@ afhip_status afhip_launch_gemm_stamps(void *stream, afhip_buffer stamps, afhip_b
                                       afhip_buffer weight_prepared, size_t rows, size_t in_dim, size_t out_dim);
 /* Diagnostic with no counterpart in the reference: what instruction patterns cost a SIMD, timed
  * by the wavefronts themselves.  One workgroup of 256 x `wavefronts_per_simd` (1, 2 or 4) threads
- * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 20, listed in
+ * per compute unit; every wavefront runs `iterations` rounds of `pattern` (0 .. 23, listed in
  * csrc/rate_probe_kernels.hip: vector-ALU instructions, int8 and f32 MFMAs, their mixes inside one
  * wavefront and side by side in two) and stores four 32-bit words into `stamps`
  * [wavefront][4]: shader-clock cycles of its loop, 100 MHz reference ticks of its loop, the
