@@ -136,7 +136,7 @@ struct GemvExtras {
     Epilogue ep_b;  // ops/ops.zig:1728, :915)
 };
 constexpr uint32_t kGemvHasEpilogueA = 1u << 24, kGemvHasEpilogueB = 1u << 25;
-constexpr uint32_t kGemvReadyCounter = 1u << 26;  // several rows: wait for the quantizing wavefronts through a counter in LDS
+constexpr uint32_t kGemvReadyCounter = 1u << 26;  // wait for the quantizing wavefronts through a counter in LDS, not at a barrier
 
 
 // Compute units of the current device (cached).

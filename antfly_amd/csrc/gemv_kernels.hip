@@ -183,36 +183,43 @@ __device__ __forceinline__ void gemv_fused_body(
     if (!(kProbe & kProbeNoPrologue) && wave * kWave < x_blocks) {  // wave-uniform
         if (ready_counter) {
             // (The host sets the counter bit only when some wavefront does not quantize: one block a thread at most.)
-            // A thread quantizes block `tid` but does not fetch it itself: the wavefront reads its 64 blocks as eight
-            // contiguous kilobytes (lane l takes 16-byte chunk 64 i + l), passes them through 8 KB of LDS of its own
-            // (chunk c of block b in slot c ^ ((b >> 1) & 7) of the block's eight: the per-thread reads that follow are
-            // conflict-free) and each thread picks up its block.  No other wavefront touches that region: no barrier.
-            // The requests are inline assembly so that they leave here, ahead of every weight request, whatever the
-            // compiler would make of loads whose values are first needed much later; it does not count them, hence
-            // the wait by hand: all but the weight requests issued in between.
+            // A thread quantizes block `tid` but does not fetch it itself: the wavefront's 64 blocks come in as eight
+            // contiguous kilobytes, straight into 8 KB of LDS of its own (global_load_lds: the bytes never are values
+            // the compiler could touch before they have arrived), and each thread then picks up its block.  LDS slot
+            // 64 i + l of load i is chunk slot l % 8 of block 8 i + l / 8; it receives that block's 16-byte chunk
+            // (l % 8) ^ ((block >> 1) & 7), so that the per-thread reads that follow are conflict-free.  No other
+            // wavefront touches the region: no barrier.  Then X alone is waited for (nothing else is outstanding: the
+            // wait does not depend on where the compiler puts its own loads), the weights are requested, and the
+            // quantization runs while they come.
             typedef float f32x4 __attribute__((ext_vector_type(4)));
-            f32x4* stage = reinterpret_cast<f32x4*>(lds + flag_off + 16) + wave * 512;
+            const uint32_t stage_byte = flag_off + 16 + static_cast<uint32_t>(wave) * 8192;
+            const uint32_t stage_lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + stage_byte);
             const int last_chunk = x_blocks * 8 - 1;
-            f32x4 t[8];
+            uint32_t off[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const uint32_t off = static_cast<uint32_t>(min(wave * 512 + i * 64 + lane, last_chunk)) * 16u;
-                asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(t[i]) : "v"(off), "s"(input) : "memory");
+                const int b = wave * 64 + i * 8 + (lane >> 3), c = (lane & 7) ^ ((b >> 1) & 7);
+                off[i] = static_cast<uint32_t>(min(b * 8 + c, last_chunk)) * 16u;
             }
+            // (all eight offsets first, then nothing but the requests: the compiler does not count these loads, and a
+            // wait it places for reasons of its own between them -- before a vector register is overwritten, say --
+            // would wait for them)
+            asm volatile("" : "+v"(off[0]), "+v"(off[1]), "+v"(off[2]), "+v"(off[3]), "+v"(off[4]), "+v"(off[5]), "+v"(off[6]), "+v"(off[7]));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             :
+                             : "s"(stage_lds + i * 1024), "v"(off[i]), "s"(input)
+                             : "memory", "m0");
             __builtin_amdgcn_sched_barrier(0);
             x_requests_first();
+            asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+            if (kProbe & kProbeTimeline) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+            __builtin_amdgcn_sched_barrier(0);
             request_weights();
             __builtin_amdgcn_sched_barrier(0);
-            asm volatile("s_waitcnt vmcnt(%8)"
-                         : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7])
-                         : "n"(kCols * kSteps + 1)
-                         : "memory");
-            if (kProbe & kProbeTimeline) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const int g = i * 64 + lane, b = g >> 3, c = g & 7;
-                stage[b * 8 + (c ^ ((b >> 1) & 7))] = t[i];
-            }
+            const f32x4* stage = reinterpret_cast<const f32x4*>(lds + stage_byte);
             float4 v[8];
 #pragma unroll
             for (int c = 0; c < 8; ++c) {
@@ -255,10 +262,13 @@ __device__ __forceinline__ void gemv_fused_body(
             quantize_block_to_lds<kType, true>(v, b2, kb, qx + r2 * row_dwords, sx + r2 * kb, sumx + r2 * kb);
         }
         if (kProbe & kProbeTimeline) stamp[6] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
-        if (ready_counter) {  // this wavefront's blocks are in LDS: say so
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        if (ready_counter) {
+            // This wavefront's blocks are in LDS: say so.  The fence names LDS only -- a general release would also
+            // wait for the wavefront's own weight requests to complete before the counter moves.
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
             if (lane == 0) __hip_atomic_fetch_add(ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         }
+
 
     } else {
         // The requests of a unit's wavefronts queue at its one texture addresser.  Left alone
@@ -280,7 +290,7 @@ __device__ __forceinline__ void gemv_fused_body(
         // (bounded all the same: a wavefront that gave up would compute on what LDS holds and still end)
         for (int spin = 0; spin < (1 << 22) && __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < quantizers; ++spin)
             __builtin_amdgcn_s_sleep(2);
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
     }
     if (kProbe & kProbeTimeline) stamp[1] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     wd.exchange();

@@ -120,6 +120,11 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (33, 96, 513), (64, 1056, 640), (130, 256, 1030), (257, 512, 512),
     (16, 14336, 512), (70, 8224, 520),  # long K on the MFMA kernel: many ring stages, a one-block last stage
     (8, 14336, 516), (7, 9216, 512),    # small batch with a long K: one launch with more than 128 KB of LDS
+    # the decode kernel with the quantized activations awaited through a counter (several rows, or one long row, and
+    # wavefronts that do not quantize): quantizers with a ragged last block set, every row count, one long row in
+    # two and four K slices, a wide matrix (full-size workgroups)
+    (2, 4096, 4100), (3, 4096, 2052), (4, 4096, 6144), (2, 1120, 3000), (4, 992, 8200), (1, 6144, 1030), (1, 14336, 2050),
+    (2, 2080, 14336),
     # the single-shot MFMA kernel (5..64 rows): every count of live result registers, two row tiles, a K
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
