@@ -82,6 +82,7 @@ __device__ __forceinline__ void quantize_block_image(const float4 (&v)[8], int b
 }
 
 constexpr uint32_t kBatchHasEpilogueA = 1u << 28, kBatchHasEpilogueB = 1u << 29;
+constexpr uint32_t kBatchReadyCounter = 1u << 30;  // wait for the quantizing wavefronts through a counter in LDS (below)
 
 // blockDim = (64, waves); grid = (column chunks, K slices).
 //   shape: waves | stagger << 8 | kBatchHasEpilogue*
@@ -126,21 +127,65 @@ __global__ __launch_bounds__(1024) void gemv_batch_kernel(
     const TileScales* tile_scales = reinterpret_cast<const TileScales*>(weight + (static_cast<size_t>(tile_off16) << 4)) +
                                     (static_cast<size_t>(min(group, groups_each - 1)) * ((kb + kSliceBlocks - 1) / kSliceBlocks) + slice) * kWave;
 
-    // ---- 1. requests: this wavefront's share of the X slice (coalesced), then its weights
-    // staging units: unit q = row (q >> 4), 64 chunks [64 (q & 15), +64) of that row's slice
+    // ---- 1. requests: X (coalesced), then the weights.
+    // Two forms.  With the counter (kBatchReadyCounter: the host sets it when the workgroup has wavefronts that do not
+    // quantize and LDS holds image and staging side by side, up to seven rows) the first 2 * kRows wavefronts are the
+    // quantizers: wavefront w takes the 64 blocks [64 w, +64) of the slice's kRows x 128 (half a row: 8 KB contiguous)
+    // straight into 8 KB of LDS of its own with eight global_load_lds (slot 64 i + l of load i = chunk slot l % 8 of
+    // block 8 i + l / 8, which receives chunk (l % 8) ^ ((block >> 1) & 7): conflict-free per-thread reads later);
+    // one early barrier puts every request for X ahead of every weight request in the memory pipeline's queue (and
+    // publishes the cleared counter); the quantizers wait for X alone, then everybody requests weights.  Nobody waits
+    // at a barrier behind the weight requests: a wavefront is through those only when the pipeline has accepted them,
+    // for the last wavefronts of a unit halfway into the stream.
+    // Without the counter: every wavefront fetches a share of X into registers, and three barriers follow (staging
+    // written, staging read, image written: the image lies over the staging area).
+    const bool ready_counter = (shape & kBatchReadyCounter) != 0;  // wave-uniform
+    constexpr uint32_t kCounterOff = kRows * (kQRowBytes + kSliceBlocks * 8);
+    uint32_t* ready = reinterpret_cast<uint32_t*>(lds + kCounterOff);
+    const bool quantizer = ready_counter && wave < 2 * kRows;
+    const uint32_t stage_byte = kCounterOff + 16 + static_cast<uint32_t>(wave) * 8192;
+    // staging units of the other form: unit q = row (q >> 4), 64 chunks [64 (q & 15), +64) of that row's slice
     constexpr int kUnits = kRows * 16;
     constexpr int kXPre = 8;  // units per wavefront requested ahead of the weights
     const u32x4* x4 = reinterpret_cast<const u32x4*>(input);
     u32x4 xv[kXPre];
     int xpos[kXPre];
+    if (ready_counter) {
+        if (tid == 0) *ready = 0;
+        if (quantizer) {
+            const int r = wave >> 1;
+            uint32_t off[8];
 #pragma unroll
-    for (int i = 0; i < kXPre; ++i) {
-        const int q = wave + i * waves;  // wave-uniform
-        if (q < kUnits) {
-            const int r = q >> 4, p = ((q & 15) << 6) + lane;  // chunk position p inside the row's staging area
-            const int b = p >> 3, c = (p & 7) ^ (b & 7);      // block, 16-byte chunk of it that lives at p
-            xpos[i] = r * kRawRowBytes + p * 16;
-            xv[i] = x4[(static_cast<size_t>(r) * in_dim + (slice * kSliceBlocks + min(b, kb_s - 1)) * 32) / 4 + c];
+            for (int i = 0; i < 8; ++i) {
+                const int b = (wave & 1) * 64 + i * 8 + (lane >> 3), c = (lane & 7) ^ ((b >> 1) & 7);
+                off[i] = static_cast<uint32_t>((static_cast<size_t>(r) * in_dim + (slice * kSliceBlocks + min(b, kb_s - 1)) * 32) * 4 + c * 16);
+            }
+            // (all offsets first, then nothing but the requests: the compiler does not count these loads, and a wait it
+            // places for reasons of its own between them would wait for them)
+            asm volatile("" : "+v"(off[0]), "+v"(off[1]), "+v"(off[2]), "+v"(off[3]), "+v"(off[4]), "+v"(off[5]), "+v"(off[6]), "+v"(off[7]));
+            const uint32_t stage_lds = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(reinterpret_cast<uintptr_t>(lds)) + stage_byte);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             :
+                             : "s"(stage_lds + i * 1024), "v"(off[i]), "s"(input)
+                             : "memory", "m0");
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if (quantizer) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+    } else {
+#pragma unroll
+        for (int i = 0; i < kXPre; ++i) {
+            const int q = wave + i * waves;  // wave-uniform
+            if (q < kUnits) {
+                const int r = q >> 4, p = ((q & 15) << 6) + lane;  // chunk position p inside the row's staging area
+                const int b = p >> 3, c = (p & 7) ^ (b & 7);      // block, 16-byte chunk of it that lives at p
+                xpos[i] = r * kRawRowBytes + p * 16;
+                xv[i] = x4[(static_cast<size_t>(r) * in_dim + (slice * kSliceBlocks + min(b, kb_s - 1)) * 32) / 4 + c];
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0);  // the activation requests stay ahead of the weight requests
@@ -173,36 +218,59 @@ __global__ __launch_bounds__(1024) void gemv_batch_kernel(
     unsigned char* qimg = lds;                                                         // [kRows][4096]
     float* sx = reinterpret_cast<float*>(lds + kRows * kQRowBytes);                     // [kRows][128]
     int* sumx = reinterpret_cast<int*>(lds + kRows * kQRowBytes + kRows * kSliceBlocks * 4);  // [kRows][128]
+    if (ready_counter) {
+        if (quantizer) {
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const f32x4* stage = reinterpret_cast<const f32x4*>(lds + stage_byte);
+            float4 v[8];
 #pragma unroll
-    for (int i = 0; i < kXPre; ++i)
-        if (wave + i * waves < kUnits) *reinterpret_cast<u32x4*>(lds + xpos[i]) = xv[i];
-    for (int q = wave + kXPre * waves; q < kUnits; q += waves) {  // small workgroups: the rest queues behind the weights
-        const int r = q >> 4, p = ((q & 15) << 6) + lane;
-        const int b = p >> 3, c = (p & 7) ^ (b & 7);
-        *reinterpret_cast<u32x4*>(lds + r * kRawRowBytes + p * 16) =
-            x4[(static_cast<size_t>(r) * in_dim + (slice * kSliceBlocks + min(b, kb_s - 1)) * 32) / 4 + c];
+            for (int c = 0; c < 8; ++c) {
+                const f32x4 got = stage[lane * 8 + (c ^ ((lane >> 1) & 7))];
+                v[c] = make_float4(got.x, got.y, got.z, got.w);
+            }
+            const int r = wave >> 1, b = (wave & 1) * 64 + lane;
+            quantize_block_image<kType>(v, b, qimg + r * kQRowBytes, sx + r * kSliceBlocks, sumx + r * kSliceBlocks);
+            // this wavefront's blocks are in LDS: say so (the fence names LDS only -- a general release would also wait
+            // for the wavefront's own weight requests)
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            if (lane == 0) __hip_atomic_fetch_add(ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+        // (bounded all the same; the quantizers depend on nobody)
+        for (int spin = 0; spin < (1 << 22) && __hip_atomic_load(ready, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) < 2u * kRows; ++spin)
+            __builtin_amdgcn_s_sleep(2);
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    } else {
+#pragma unroll
+        for (int i = 0; i < kXPre; ++i)
+            if (wave + i * waves < kUnits) *reinterpret_cast<u32x4*>(lds + xpos[i]) = xv[i];
+        for (int q = wave + kXPre * waves; q < kUnits; q += waves) {  // small workgroups: the rest queues behind the weights
+            const int r = q >> 4, p = ((q & 15) << 6) + lane;
+            const int b = p >> 3, c = (p & 7) ^ (b & 7);
+            *reinterpret_cast<u32x4*>(lds + r * kRawRowBytes + p * 16) =
+                x4[(static_cast<size_t>(r) * in_dim + (slice * kSliceBlocks + min(b, kb_s - 1)) * 32) / 4 + c];
+        }
+        __syncthreads();
+        constexpr int kXBlocks = kRows * kSliceBlocks;
+        float4 raw0[8], raw1[8];
+        const int id1 = tid + threads;
+        const bool two = id1 < kXBlocks;
+        auto read_block = [&](int id, float4 (&v)[8]) {
+            const int r = id >> 7, b = id & (kSliceBlocks - 1);
+            const unsigned char* base = lds + r * kRawRowBytes + b * 128;
+#pragma unroll
+            for (int c = 0; c < 8; ++c) v[c] = *reinterpret_cast<const float4*>(base + ((c ^ (b & 7)) << 4));
+        };
+        if (tid < kXBlocks) read_block(tid, raw0);
+        if (two) read_block(id1, raw1);
+        __syncthreads();
+        auto quantize = [&](int id, const float4 (&v)[8]) {
+            const int r = id >> 7, b = id & (kSliceBlocks - 1);
+            quantize_block_image<kType>(v, b, qimg + r * kQRowBytes, sx + r * kSliceBlocks, sumx + r * kSliceBlocks);
+        };
+        if (tid < kXBlocks) quantize(tid, raw0);
+        if (two) quantize(id1, raw1);
+        __syncthreads();
     }
-    __syncthreads();
-    constexpr int kXBlocks = kRows * kSliceBlocks;
-    float4 raw0[8], raw1[8];
-    const int id1 = tid + threads;
-    const bool two = id1 < kXBlocks;
-    auto read_block = [&](int id, float4 (&v)[8]) {
-        const int r = id >> 7, b = id & (kSliceBlocks - 1);
-        const unsigned char* base = lds + r * kRawRowBytes + b * 128;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) v[c] = *reinterpret_cast<const float4*>(base + ((c ^ (b & 7)) << 4));
-    };
-    if (tid < kXBlocks) read_block(tid, raw0);
-    if (two) read_block(id1, raw1);
-    __syncthreads();
-    auto quantize = [&](int id, const float4 (&v)[8]) {
-        const int r = id >> 7, b = id & (kSliceBlocks - 1);
-        quantize_block_image<kType>(v, b, qimg + r * kQRowBytes, sx + r * kSliceBlocks, sumx + r * kSliceBlocks);
-    };
-    if (tid < kXBlocks) quantize(tid, raw0);
-    if (two) quantize(id1, raw1);
-    __syncthreads();
     wd.exchange();
 
     // ---- 3. block dots and scaled accumulation
@@ -323,7 +391,10 @@ hipError_t launch_rows(hipStream_t stream, float* dst_a, float* dst_b, int* dots
     const int groups = (out_dim + kCols - 1) / kCols * (weight_b ? 2 : 1);
     const int waves = gemv_batch_waves(kRows, in_dim, groups);
     const int chunks = (groups + waves - 1) / waves;
-    const size_t lds = static_cast<size_t>(kRows) * kRawRowBytes;
+    // the counter form: wavefronts that do not quantize, and LDS for image, scales, counter and staging side by side
+    const bool ready_counter = kRows >= 2 && kRows <= 7 && waves > 2 * kRows;
+    const size_t lds = ready_counter ? static_cast<size_t>(kRows) * (kQRowBytes + kSliceBlocks * 8 + kRawRowBytes) + 16
+                                     : static_cast<size_t>(kRows) * kRawRowBytes;
     auto kernel = gemv_batch_kernel<kType, kRows, kDots>;
     static std::atomic<size_t> lds_limit{64 * 1024};
     if (hipError_t e = allow_lds(kernel, lds, &lds_limit); e != hipSuccess) return e;
@@ -333,7 +404,7 @@ hipError_t launch_rows(hipStream_t stream, float* dst_a, float* dst_b, int* dots
     const bool split = slices > 1 && !kDots;
     if (split && partial == nullptr) return hipErrorInvalidValue;
     const int stagger = static_cast<long>(chunks) * slices <= gemv_compute_units() ? 1 : 0;
-    const uint32_t shape = static_cast<uint32_t>(waves) | static_cast<uint32_t>(stagger) << 8 |
+    const uint32_t shape = static_cast<uint32_t>(waves) | static_cast<uint32_t>(stagger) << 8 | (ready_counter ? kBatchReadyCounter : 0u) |
                            (!split && has_epilogue(ep_a) ? kBatchHasEpilogueA : 0u) | (!split && has_epilogue(ep_b) ? kBatchHasEpilogueB : 0u);
     const GemvExtras extras{dots, nullptr, ep_a, ep_b};
     hipLaunchKernelGGL(kernel, dim3(chunks, slices), dim3(64, waves), lds, stream, weight_a, weight_b, input, dst_a, dst_b,

@@ -125,6 +125,9 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # two and four K slices, a wide matrix (full-size workgroups)
     (2, 4096, 4100), (3, 4096, 2052), (4, 4096, 6144), (2, 1120, 3000), (4, 992, 8200), (1, 6144, 1030), (1, 14336, 2050),
     (2, 2080, 14336),
+    # ... and the long-K kernel (K > 4096, two to seven rows, sixteen-wavefront workgroups): full and ragged last slice,
+    # ragged columns, the most rows the counter form takes
+    (2, 8192, 2048), (4, 9216, 4100), (3, 14336, 4096), (7, 8192, 4096), (5, 4128, 2100),
     # the single-shot MFMA kernel (5..64 rows): every count of live result registers, two row tiles, a K
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
