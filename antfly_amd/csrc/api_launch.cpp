@@ -462,7 +462,7 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
         // workgroup would repeat too much of that work, so X is quantized once by its own
         // kernel into the caller's scratch.  (AFHIP_GEMV_FUSED_ROWS caps the rows for tuning runs.)
         static const int env_fused_rows = env_int("AFHIP_GEMV_FUSED_ROWS");
-        const size_t type_rows = tensor_type == AFHIP_TYPE_Q4_0 ? 4 : 2;
+        const size_t type_rows = 4;  // both formats
         const size_t fused_rows = env_fused_rows >= 1 && env_fused_rows <= 4 ? size_t(env_fused_rows) : type_rows;
         const bool prequantize = rows > fused_rows || (rows > 2 && rows * kb > kGemvFusedQuantBlocks);
         const WorkspaceView ws = workspace_view(workspace.ptr, rows, in_dim);
