@@ -298,7 +298,7 @@ def main() -> int:
                        "one set of random weights repacked into 32 distinct device copies; matmuls only, gate and up as "
                        "one pair call (shared X)",
                "weight_bytes_per_token": weight_bytes}
-        for m in (1, 5):
+        for m in (1, 2, 4, 5):
             xs = {k: torch.from_numpy(synth.activations(900 + k, m, k)).to(dev) for k in (4096, 14336)}
             ys = {n: torch.empty((m, n), dtype=torch.float32, device=dev) for n in (6144, 4096, 14336)}
             y_up = torch.empty((m, 14336), dtype=torch.float32, device=dev)
@@ -800,7 +800,12 @@ def main() -> int:
             ("q8_gemv_m1_k4096_n4096", Q8, 1, 4096, 4096),
             ("q8_gemv_m1_k4096_n14336", Q8, 1, 4096, 14336),
             ("q4_gemv_m2_k4096_n14336", Q4, 2, 4096, 14336),
+            ("q4_gemv_m3_k4096_n14336", Q4, 3, 4096, 14336),
             ("q4_gemv_m4_k4096_n14336", Q4, 4, 4096, 14336),
+            ("q8_gemv_m2_k4096_n14336", Q8, 2, 4096, 14336),
+            ("q8_gemv_m4_k4096_n14336", Q8, 4, 4096, 14336),
+            ("q4_gemv_m2_k14336_n4096", Q4, 2, 14336, 4096),    # long K, few rows: K shared out over workgroups + reduce kernel
+            ("q4_gemv_m4_k14336_n4096", Q4, 4, 14336, 4096),
             ("q4_batch_m8_k4096_n14336", Q4, 8, 4096, 14336),   # speculative verify: compact-fragment quantizer + eight-row MFMA kernel
             ("q4_gemv_m1_k14336_n4096", Q4, 1, 14336, 4096),
             ("q4_batch_m5_k14336_n4096", Q4, 5, 14336, 4096),
