@@ -522,8 +522,13 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
 #pragma unroll
     for (int k = 0; k < kSpares; ++k) spare[k] = __builtin_nontemporal_load(qa8 + k * 32 + (lane & 31));  // inside the first pair's entries
     constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
+    // Q4_0 asks for the second stage only when the first one and the register loads are there (below); Q8_0, whose
+    // stages are half as many blocks, measured better with the second stage requested up front.
+    constexpr bool kStartupAlone = kType == 2;
+    if (!kStartupAlone) {
 #pragma unroll
-    for (int st = 1; st < kAheadStages; ++st) issue_stage(st);
+        for (int st = 1; st < kAheadStages; ++st) issue_stage(st);
+    }
 
     // this lane's B operand: column 16 * cg + l16, block 2p + par, k half kh.  Q8_0: bytes
     // [16 kh, +16) of the block.  Q4_0: bytes [8 kh, +8), low nibbles and high nibbles dword by
@@ -574,13 +579,20 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
             if (it % kHalfPairs == 0) {
                 const int st = stage_of(it), hb = st / kCG, cg = st % kCG;
                 if (st == 0) {
-                    // everything older than the second stage: the first stage and all the register loads
-                    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * (kAheadStages - 1)) : "memory");
+                    // the first stage and all the register loads, waited for while nothing else of this wavefront is
+                    // outstanding: behind the second stage's requests the wait would also have to see those accepted by
+                    // the memory pipeline, which for the last wavefronts of a unit is well into the stream
+                    if (kStartupAlone) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
+                    else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * (kAheadStages - 1)) : "memory");
 #pragma unroll
                     for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(packed[q]));
 #pragma unroll
                     for (int c = 0; c < kCG; ++c) asm volatile("" : "+v"(tb_part[c][0]), "+v"(tb_part[c][kWpl - 1]));
                     asm volatile("" : "+v"(sx_part[0]), "+v"(sx_part[kScaleLoads - 1]));
+                }
+                if (kStartupAlone && st == 0) {
+#pragma unroll
+                    for (int ahead = 1; ahead < kAheadStages; ++ahead) issue_stage(ahead);
                 }
                 if (st + kAheadStages < kStages) issue_stage(st + kAheadStages);
                 // operands of this stage's scale products (in the shadow of the wait below).
