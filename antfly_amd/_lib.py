@@ -117,6 +117,7 @@ SIGNATURES = {
     "afhip_launch_gemv_probe": (_st, [_vp, _i, Buffer, Buffer, Buffer, _sz, _sz]),
     "afhip_launch_gemv_probe_rows": (_st, [_vp, _i, _sz, Buffer, Buffer, Buffer, _sz, _sz]),
     "afhip_launch_gemv_timeline": (_st, [_vp, _sz, Buffer, Buffer, Buffer, _sz, _sz, C.POINTER(_sz), C.POINTER(_sz)]),
+    "afhip_launch_rows8_timeline": (_st, [_vp, _sz, Buffer, Buffer, Buffer, _sz, _sz, Buffer, C.POINTER(_sz), C.POINTER(_sz)]),
     "afhip_static_scratch_init": (_st, []),
     "afhip_launch_linear_f32_static": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, _sz, _sz, _sz, _i]),
     "afhip_launch_linear_pair_f32": (_st, [_vp, _i, _i, Buffer, Buffer, Buffer, Buffer, Buffer, _sz, _sz, _sz, Buffer, _i]),

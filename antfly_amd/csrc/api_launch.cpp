@@ -996,6 +996,27 @@ afhip_status afhip_launch_gemv_timeline(void* stream, size_t rows, afhip_buffer 
     return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
 }
 
+afhip_status afhip_launch_rows8_timeline(void* stream, size_t rows, afhip_buffer stamps, afhip_buffer input, afhip_buffer weight,
+                                         size_t in_dim, size_t out_dim, afhip_buffer workspace, size_t* workgroups,
+                                         size_t* columns_per_workgroup) {
+    if (rows < 1 || rows > 8) return AFHIP_ERR_INVALID_ARGUMENT;
+    if (in_dim == 0 || in_dim % 256 != 0 || in_dim > 4096 || out_dim == 0 || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
+    const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q4_0, out_dim, in_dim);
+    const size_t ws = batch_mfma_workspace_bytes(AFHIP_TYPE_Q4_0, rows, in_dim, out_dim);
+    if (need == 0 || weight.len < need || input.len < rows * in_dim * 4 || ws == 0 || workspace.len < ws) return AFHIP_ERR_INVALID_STATE;
+    if (stamps.ptr == 0 || stamps.ptr % 4 != 0 || input.ptr == 0 || weight.ptr == 0 || workspace.ptr == 0 || input.ptr % 16 != 0 ||
+        weight.ptr % 16 != 0 || workspace.ptr % 16 != 0)
+        return AFHIP_ERR_INVALID_STATE;
+    int groups = 0, cols = 0;
+    hipError_t e = launch_batch8_timeline(static_cast<hipStream_t>(stream), reinterpret_cast<uint32_t*>(stamps.ptr), stamps.len,
+                                          reinterpret_cast<const float*>(input.ptr), reinterpret_cast<const uint8_t*>(weight.ptr),
+                                          static_cast<int>(rows), static_cast<int>(in_dim), static_cast<int>(out_dim),
+                                          reinterpret_cast<uint8_t*>(workspace.ptr), &groups, &cols);
+    if (workgroups) *workgroups = static_cast<size_t>(groups);
+    if (columns_per_workgroup) *columns_per_workgroup = static_cast<size_t>(cols);
+    return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
+}
+
 afhip_status afhip_launch_gemv_probe(void* stream, int probe, afhip_buffer dst, afhip_buffer input, afhip_buffer weight,
                                      size_t in_dim, size_t out_dim) {
     return afhip_launch_gemv_probe_rows(stream, probe, 1, dst, input, weight, in_dim, out_dim);

@@ -424,11 +424,17 @@ __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* _
     }
 }
 
-template <int kType, int kCG>
+// kStamps (bench.py --probe timeline8): the same code, but instead of results every wavefront stores eight readings of the
+// 100 MHz clock at dst_a[8 * (8 * workgroup + wavefront)]: [0] entry, [1] .. [4] the first four stages' bytes there, [5] the last
+// stage's, [6] K loop done, [7] after the workgroup's reduction.
+// kFullCols: a workgroup takes all 16 kCG columns (`cols` is not looked at).
+template <int kType, int kCG, bool kStamps = false, bool kFullCols = false>
 __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                      const uint32_t* __restrict__ qa8, const float* __restrict__ sa8,
                                                                      const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
-                                                                     int share_blocks, Epilogue ep_a, BmSecond second) {
+                                                                     int share_blocks, int cols_arg, Epilogue ep_a, BmSecond second) {
+    uint32_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (kStamps) stamp[0] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     using F = BmFormat<kType>;
     const bool is_b = blockIdx.z != 0;
     float* dst = is_b ? second.dst : dst_a;
@@ -441,7 +447,10 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l16 = lane & 15, g = lane >> 4, par = g >> 1, kh = g & 1;  // column, lane group, block parity, k half
-    const int n0 = blockIdx.x * kCols;
+    // a workgroup's columns: `cols` of them, a multiple of 8 in (16 kCG - 16, 16 kCG] (the host picks what spreads the matrix
+    // evenly over the compute units); the arithmetic runs on all 16 kCG, the last ones on a copy of column cols - 1
+    const int cols = kFullCols ? 16 * kCG : cols_arg;
+    const int n0 = blockIdx.x * cols;
     const int share_begin = static_cast<int>(blockIdx.y) * share_blocks;  // a multiple of kWB: even
     const int share_end = min(share_begin + share_blocks, kb_full);
     const int blk0 = share_begin + wave * kWB;
@@ -473,7 +482,7 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         for (int u = 0; u < 2; ++u) {
             const int c = 16 * cg + 8 * u + c8;
             const int chunk = slot ^ ((c >> 1) & 7);
-            const int cc = min(n0 + c, out_dim - 1) - n0;
+            const int cc = min(n0 + min(c, cols - 1), out_dim - 1) - n0;
             uint32_t off;
             if (kType == 2) {
                 off = (static_cast<uint32_t>(cc) * kb_full + clamp_blk(8 * hb + chunk)) * 16u;
@@ -498,7 +507,7 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     uint32_t tb_part[kCG][kWpl];
 #pragma unroll
     for (int cg = 0; cg < kCG; ++cg) {
-        const int cc = min(n0 + 16 * cg + l16, out_dim - 1);
+        const int cc = min(n0 + min(16 * cg + l16, cols - 1), out_dim - 1);
         const uint16_t* sw = reinterpret_cast<const uint16_t*>(weight + blocks_total * kQB) + static_cast<size_t>(cc) * kb_full;
         const uint32_t* run = reinterpret_cast<const uint32_t*>(sw + min(blk0, kb_full - 8)) + g * kWpl;
         if constexpr (kWpl == 2) {
@@ -633,6 +642,8 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
                     else asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
                 }
                 fetch_weights(it);
+                if (kStamps && st < 4) stamp[1 + st] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+                if (kStamps && st == kStages - 1) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
             }
             __builtin_amdgcn_sched_barrier(0);
             if (it + 1 < kSteps && (it + 1) % kHalfPairs != 0) fetch_weights(it + 1);
@@ -656,6 +667,7 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
             __builtin_amdgcn_sched_barrier(0);
         }
         scale(kSteps - 1);
+        if (kStamps) stamp[6] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     } else {
         asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // nothing may still be writing LDS when the region is reused
     }
@@ -676,10 +688,21 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
 #pragma unroll
         for (int w = 0; w < kBmWaves; ++w) sum += red[w * kCG * 256 + item] + red[w * kCG * 256 + item + 32];
         const int n = n0 + c;
-        if (m < rows && n < out_dim) {
+        if (kStamps) {
+            asm volatile("" : : "v"(sum));  // (keeps the arithmetic alive)
+        } else if (m < rows && c < cols && n < out_dim) {
             const size_t at = static_cast<size_t>(m) * out_dim + n;
             if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
             else dst[at] = finish_output(ep, n, at, sum);
+        }
+    }
+    if (kStamps) {
+        __syncthreads();
+        stamp[7] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+        if (lane == 0) {
+            uint32_t* o = reinterpret_cast<uint32_t*>(dst_a) + (static_cast<size_t>(blockIdx.x) * kBmWaves + wave) * 8;
+#pragma unroll
+            for (int q = 0; q < 8; ++q) o[q] = stamp[q];
         }
     }
 }
@@ -938,12 +961,17 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
 
 template <int kType, int kCG>
 hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
-                      int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
-    const dim3 grid(static_cast<unsigned>((out_dim + 16 * kCG - 1) / (16 * kCG)), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
-    hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows,
-                       in_dim, out_dim, share_blocks, ep, second);
+                      int in_dim, int out_dim, int shares, int share_blocks, int cols, const Epilogue& ep, const BmSecond& second) {
+    const dim3 grid(static_cast<unsigned>((out_dim + cols - 1) / cols), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
+    if (cols == 16 * kCG)
+        hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG, false, true>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa,
+                           weight, rows, in_dim, out_dim, share_blocks, cols, ep, second);
+    else
+        hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight,
+                           rows, in_dim, out_dim, share_blocks, cols, ep, second);
     return hipGetLastError();
 }
+
 
 // Column groups of sixteen a workgroup takes: four (64 columns: the activations' share of a
 // workgroup's traffic and a wavefront's set-up halve) where that still gives most compute units a
@@ -962,6 +990,24 @@ bool bm8_one_column_group(int tensor_type, size_t in_dim, size_t out_dim) {
     const size_t shares = static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim))), units = static_cast<size_t>(gemv_compute_units());
     const size_t narrow = (out_dim + 15) / 16 * shares;
     return (out_dim + 31) / 32 * shares < units && narrow >= units && narrow <= units + units / 8;
+}
+
+// Columns a workgroup of the eight-row kernel takes (a multiple of 8 up to 64).  Where some column count gives a grid of
+// no more workgroups than compute units, the smallest such count: every unit gets one workgroup, or nearly every
+// one, and none two.  Measured at five and eight rows against the rule below: 11008 columns (K = 4096) 10.6 us on 230
+// workgroups of 48 columns against 12.2 on 344 of 32 (172 of 64: 11.6); K = 14336 x 4096 columns 14.7 on 64 x 4 K
+// shares against 15.6 on 128 x 4; K = 8192 x 8192 columns 14.4 on 128 x 2 against 15.3 on 256 x 2; Q8_0 6144 columns
+// 11.5 on 128 x 2 of 48 against 12.2 on 192 x 2; 14336 columns 12.1 .. 12.3 on 256 of 56 against 12.4 on 224 of 64.
+// (A column count that is not a multiple of 16 leaves part of a workgroup's last column group idle.)
+// Else the grid takes several rounds whatever the tile, and fewer, larger workgroups fetch the operand fragments less
+// often: 64 columns from 12288 columns on, 16 where that is one round and a bit, else 32 (Q8_0, 14336 columns, two
+// K shares: 18.0 us on 448 workgroups of 64 against 18.9 on 598 of 48; a pair of those 30.2 against 32.2).
+int bm8_columns(int tensor_type, int in_dim, int out_dim, bool pair) {
+    const long units = gemv_compute_units(), shares = bm_shares(tensor_type, in_dim);
+    for (long cols = 8; cols <= 64; cols += 8)
+        if ((out_dim + cols - 1) / cols * shares * (pair ? 2 : 1) <= units) return static_cast<int>(cols);
+    if (bm8_column_groups(out_dim) == 4) return 64;
+    return bm8_one_column_group(tensor_type, static_cast<size_t>(in_dim), static_cast<size_t>(out_dim)) ? 16 : 32;
 }
 
 template <int kType>
@@ -1067,10 +1113,10 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const BmSecond second{dst_b, weight_b_prepared, ep_b};
     hipError_t e;
     if (eight) {
-        const bool wide = bm8_column_groups(out_dim) == 4;
-#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
-        const bool one = bm8_one_column_group(tensor_type, static_cast<size_t>(in_dim), static_cast<size_t>(out_dim));
-        e = tensor_type == 2 ? (wide ? AFHIP_BM8(2, 4) : (one ? AFHIP_BM8(2, 1) : AFHIP_BM8(2, 2))) : (wide ? AFHIP_BM8(8, 4) : (one ? AFHIP_BM8(8, 1) : AFHIP_BM8(8, 2)));
+        const int cols = bm8_columns(tensor_type, in_dim, out_dim, weight_b_prepared != nullptr), cg = (cols + 15) / 16;
+#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, ep, second)
+        if (tensor_type == 2) e = cg == 4 ? AFHIP_BM8(2, 4) : (cg == 3 ? AFHIP_BM8(2, 3) : (cg == 2 ? AFHIP_BM8(2, 2) : AFHIP_BM8(2, 1)));
+        else e = cg == 4 ? AFHIP_BM8(8, 4) : (cg == 3 ? AFHIP_BM8(8, 3) : (cg == 2 ? AFHIP_BM8(8, 2) : AFHIP_BM8(8, 1)));
 #undef AFHIP_BM8
     }
     else if (thirty_two)
@@ -1090,6 +1136,34 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
         }
     }
     return hipSuccess;
+}
+
+// The eight-row kernel's own timeline (Q4_0, one K share, a matrix the kernel takes in tiles of 49 .. 64 columns): the
+// compact-fragment quantizer, then the kernel template with its stamps flag, which stores clock readings (32 bytes per
+// wavefront, eight wavefronts a workgroup) into `stamps` instead of results.
+hipError_t launch_batch8_timeline(hipStream_t stream, uint32_t* stamps, size_t stamps_bytes, const float* input,
+                                  const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, uint8_t* workspace, int* workgroups,
+                                  int* columns) {
+    const int kb = in_dim / 32;
+    if (rows < 1 || rows > 8 || in_dim % 256 != 0 || kb > BmFormat<2>::kShareBlocks || workspace == nullptr || stamps == nullptr) return hipErrorInvalidValue;
+    if (!batch_mfma_supports(2, rows, in_dim, out_dim)) return hipErrorInvalidValue;
+    const int cols = bm8_columns(2, in_dim, out_dim, false);
+    if (cols <= 48) return hipErrorInvalidValue;
+    const int groups = (out_dim + cols - 1) / cols;
+    if (workgroups) *workgroups = groups;
+    if (columns) *columns = cols;
+    if (stamps_bytes < static_cast<size_t>(groups) * kBmWaves * 32) return hipErrorInvalidValue;
+    uint32_t* qa = reinterpret_cast<uint32_t*>(workspace);
+    const int pairs = (kb + 1) / 2;
+    float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
+    const int units = 8 * (2 * pairs) * 8;
+    hipLaunchKernelGGL(quantize_fragments8_kernel<2>, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+    if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+    int share_blocks = (kb + BmFormat<2>::kWaveBlocks - 1) / BmFormat<2>::kWaveBlocks * BmFormat<2>::kWaveBlocks;
+    hipLaunchKernelGGL((batch8_mfma_kernel<2, 4, true>), dim3(static_cast<unsigned>(groups), 1, 1), dim3(kBmThreads), kBmLdsBytes, stream,
+                       reinterpret_cast<float*>(stamps), static_cast<float*>(nullptr), qa, sa, weight_prepared, rows, in_dim, out_dim, share_blocks,
+                       cols, Epilogue{}, BmSecond{nullptr, nullptr, Epilogue{}});
+    return hipGetLastError();
 }
 
 }  // namespace afhip

@@ -109,10 +109,10 @@ def main() -> int:
                     help="launch only this configuration 200 times (for a kernel trace of one shape) and exit")
     ap.add_argument("--shapes", default=None,
                     help="comma-separated fmt:rows:in_dim:out_dim (fmt q4 / q8 / q4k; q4p / q8p: pair calls): time only these calls, print one line each, exit")
-    ap.add_argument("--probe", choices=["gemv", "rates", "gemm", "read", "timeline"], default=None,
-                    help="timeline: the Q4_0 decode kernel's wavefronts read the 100 MHz clock at their phases (afhip_launch_gemv_timeline; --probe-rows 1, 2 or 4): when the quantized activations are ready, when a wavefront's block dots are done; read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
+    ap.add_argument("--probe", choices=["gemv", "rates", "gemm", "read", "timeline", "timeline8"], default=None,
+                    help="timeline8: the same for the eight-row MFMA kernel (afhip_launch_rows8_timeline; --probe-rows 5 or 8): when a wavefront's weight stages are there, when its K loop ends; timeline: the Q4_0 decode kernel's wavefronts read the 100 MHz clock at their phases (afhip_launch_gemv_timeline; --probe-rows 1, 2 or 4): when the quantized activations are ready, when a wavefront's block dots are done; read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
-    ap.add_argument("--probe-rows", type=int, choices=[1, 2, 4], default=1,
+    ap.add_argument("--probe-rows", type=int, choices=[1, 2, 4, 5, 8], default=1,
                     help="--probe gemv: rows of X (the decode kernel's instantiation for that many rows)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -612,6 +612,48 @@ def main() -> int:
         print(f"workgroups begin {int(first.min())} .. {int(first.max())} ns (median {int(np.median(first))}); the last wavefront of the launch ends at {int(ns[:, :, 3].max())} ns")
         print(json.dumps({"probe": "timeline", "rows": prows, "workgroups": g, "wavefronts": w, "activations_ready_ns_median": int(np.median(ns[:, :, 1])),
                           "launch_ends_ns": int(ns[:, :, 3].max())}))
+        return 0
+
+    if args.probe == "timeline8":
+        import ctypes
+        lib = _lib.lib()
+        in_dim, out_dim, copies = 4096, 14336, args.copies
+        prows = args.probe_rows if args.probe_rows >= 5 else 8
+        ws = prepared_copies(Q4, out_dim, in_dim, copies, 2024)
+        x = torch.from_numpy(synth.activations(2025, prows, in_dim)).to(dev)
+        stamps = torch.zeros(1 << 18, dtype=torch.int32, device=dev)
+        work = torch.empty(kernels.workspaceBytes(Q4, 8, in_dim, out_dim), dtype=torch.uint8, device=dev)
+        groups, cols = ctypes.c_size_t(0), ctypes.c_size_t(0)
+        takes = []  # five runs of 64 launches back to back, weights rotating; each run's last launch is read
+        for take in range(5):
+            for i in range(64):
+                rc = lib.afhip_launch_rows8_timeline(stream, prows, buf(stamps), buf(x), buf(ws[i % copies]), in_dim, out_dim, buf(work),
+                                                     ctypes.byref(groups), ctypes.byref(cols))
+                if rc != 0:
+                    raise RuntimeError(f"timeline8 probe failed: {rc}")
+            torch.cuda.synchronize()
+            g, w = groups.value, 8
+            st = stamps.cpu().numpy().view(np.uint32)[: g * w * 8].reshape(g, w, 8).astype(np.int64)
+            takes.append((st - st[:, :, 0].min()) * 10)
+        ns = np.median(np.stack(takes), axis=0)  # per reading, the median of the five runs
+        print(f"Q4_0 eight-row MFMA kernel, {prows} rows, K={in_dim}, N={out_dim}: {g} workgroups of {cols.value} columns x {w} wavefronts; "
+              "ns after the launch's first wavefront began, median over workgroups (each reading: median of five runs)")
+        print("| wavefront | begins | stage 0 there | stage 1 | stage 2 | stage 3 | last stage | K loop done | workgroup reduced |")
+        print("|---|---|---|---|---|---|---|---|---|")
+        for wv in range(w):
+            print(f"| {wv} | " + " | ".join(str(int(np.median(ns[:, wv, k]))) for k in range(8)) + " |")
+        first = ns[:, :, 0].min(axis=1)
+        print(f"workgroups begin {int(first.min())} .. {int(first.max())} ns (median {int(np.median(first))}); the last wavefront of the launch ends at {int(ns[:, :, 7].max())} ns")
+        print("| per workgroup, ns | median | min | max |")
+        print("|---|---|---|---|")
+        for name, v in (("entry to the first stage there (slowest wavefront)", (ns[:, :, 1] - ns[:, :, 0]).max(axis=1)),
+                        ("first stage there to the last stage there", (ns[:, :, 5] - ns[:, :, 1]).max(axis=1)),
+                        ("last stage there to K loop done", (ns[:, :, 6] - ns[:, :, 5]).max(axis=1)),
+                        ("K loop done to reduced", (ns[:, :, 7] - ns[:, :, 6]).min(axis=1)),
+                        ("whole workgroup", ns[:, :, 7].max(axis=1) - first)):
+            print(f"| {name} | {int(np.median(v))} | {int(v.min())} | {int(v.max())} |")
+        print(json.dumps({"probe": "timeline8", "rows": prows, "workgroups": g, "columns_per_workgroup": cols.value,
+                          "first_stage_there_ns_median": int(np.median(ns[:, :, 1])), "launch_ends_ns": int(ns[:, :, 7].max())}))
         return 0
 
     if args.probe == "gemv":

@@ -628,6 +628,14 @@ afhip_status afhip_launch_gemv_probe_rows(void *stream, int probe, size_t rows, 
 afhip_status afhip_launch_gemv_timeline(void *stream, size_t rows, afhip_buffer stamps, afhip_buffer input,
                                         afhip_buffer weight_prepared, size_t in_dim, size_t out_dim, size_t *workgroups,
                                         size_t *wavefronts_per_workgroup);
+/* The same for the eight-row MFMA kernel (Q4_0, 1 .. 8 rows, in_dim a multiple of 256 up to 4096, a matrix the kernel
+ * takes in tiles of more than 48 columns): the compact-fragment quantizer runs, then the kernel with its stamps flag;
+ * eight wavefronts a workgroup, stamps[8 * (8 * workgroup + wavefront)]: [0] entry, [1] .. [4] the bytes of the first
+ * four weight stages there, [5] the last stage's, [6] K loop done, [7] after the workgroup's reduction.
+ * `workspace`: afhip_linear_workspace_bytes(Q4_0, 8, in_dim, out_dim) bytes.  `bench.py --probe timeline8`. */
+afhip_status afhip_launch_rows8_timeline(void *stream, size_t rows, afhip_buffer stamps, afhip_buffer input,
+                                         afhip_buffer weight_prepared, size_t in_dim, size_t out_dim, afhip_buffer workspace,
+                                         size_t *workgroups, size_t *columns_per_workgroup);
 /* Tuning, process-wide, no counterpart in the reference: the largest grid (workgroups) for which 9 .. 64 rows on a
  * wide matrix take the 32-row MFMA kernel on 64-column tiles; negative restores the default (one workgroup per
  * compute unit), 0 switches that kernel off.  Tests lift the bound to reach the kernel's K shares and pair launches. */

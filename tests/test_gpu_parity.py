@@ -138,6 +138,9 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (8, 512, 8200), (5, 4096, 12290), (7, 9216, 4112), (6, 256, 16416),
     # ... on 16-column tiles (4096 to 4608 columns and one K share): full, ragged last tile, one live wavefront
     (5, 4096, 4096), (8, 1024, 4600), (6, 256, 4100),
+    # ... with the column count of a workgroup picked to spread the matrix evenly over the compute units: 56 of a
+    # workgroup's 64 columns live (14336), 48 and 40 (three column groups; ragged last tile), 24 (two groups, 6144)
+    (8, 512, 14336), (6, 1024, 11008), (5, 256, 10000), (7, 2048, 6144), (8, 256, 9000),
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
@@ -359,3 +362,4 @@ def test_thirty_two_row_kernel_with_k_shares_and_pairs(fmt, rows, in_dim, out_di
             assert np.array_equal(got[1], G.linear(fmt, PREP, x, db, rows, in_dim, out_dim))
         finally:
             _lib.lib().afhip_tune_batch32_max_workgroups(-1)
+
