@@ -141,6 +141,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # ... with the column count of a workgroup picked to spread the matrix evenly over the compute units: 56 of a
     # workgroup's 64 columns live (14336), 48 and 40 (three column groups; ragged last tile), 24 (two groups, 6144)
     (8, 512, 14336), (6, 1024, 11008), (5, 256, 10000), (7, 2048, 6144), (8, 256, 9000),
+    (5, 8192, 7168),  # ... 56 columns with two K shares (Q4_0)
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
