@@ -29,7 +29,7 @@
 //     block-ascending partial sums); K shares of a long K go to partial[share][rows][out_dim]
 //     and splitk_reduce_kernel adds them in share order.
 //   * Up to eight rows on a grid that fills the chip take batch8_mfma_kernel (further down): the
-//     16x16x64 MFMA on two blocks at once, 32- or 64-column tiles, weights requested two stages
+//     16x16x64 MFMA on two blocks at once, tiles of 8 .. 64 columns, weights requested two stages
 //     ahead instead of all at once.
 //   * Nine to 64 rows on a wide matrix whose grid is one round of 64-column tiles take
 //     batch32_mfma_kernel (further down): this kernel's arithmetic, staged weight requests, one

@@ -92,7 +92,7 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
 bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 size_t batch_mfma_workspace_bytes(int tensor_type, size_t rows, size_t in_dim, size_t out_dim);
 void set_batch32_max_workgroups(long bound);
-// Timing diagnostics: the eight-row kernel (Q4_0, a matrix wide enough for its 64-column tiles, K of one share) storing
+// Timing diagnostics: the eight-row kernel (Q4_0, a matrix it takes in tiles of more than 48 columns, K of one share) storing
 // clock readings per wavefront into `stamps` instead of results; `workspace` as for launch_batch_mfma.
 hipError_t launch_batch8_timeline(hipStream_t stream, uint32_t* stamps, size_t stamps_bytes, const float* input,
                                   const uint8_t* weight_prepared, int rows, int in_dim, int out_dim, uint8_t* workspace, int* workgroups,
