@@ -465,10 +465,11 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     // the wavefront's 8 KB of LDS.  What a compute unit can keep in flight is a small part of what
     // its wavefronts want, and a wavefront that cannot issue a load cannot compute either, so a
     // wavefront requests two stages ahead of the one it works on, not everything at once.
-    // The first stage goes out first (a compute unit has one address unit and all its wavefronts
-    // queue there), then what goes to registers, kept small: one or two 4-byte loads for the row
-    // scales of the wavefront's pairs, an 8-byte load per column group for the weight scales, the
-    // operand fragments in their compact form (two pairs a load), two spares; then the second stage.
+    // Order of the requests (a compute unit has one address unit, all its wavefronts queue there and are
+    // served in order): what the quantizer's launch left in the L2 -- the operand fragments in their compact form
+    // (two pairs a load) and one or two 4-byte loads for the row scales of the wavefront's pairs -- for the whole
+    // workgroup, a barrier, then the first stage, an 8-byte load per column group for the weight scales, two
+    // spares; then the second stage.
     // A wavefront's loads complete in the order issued, so "all but the youngest n have completed"
     // says that a stage is there.  The compiler counts only its own loads when it waits for one of
     // them, which can only be too strict: it retires as many more of the oldest younger loads as
@@ -492,14 +493,39 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
             bm_lds_load16(wbase, off, lds_wave + ((st & 3) * 2 + u) * 1024);
         }
     };
-    issue_stage(0);
     const int pair0 = blk0 >> 1;
+    // What comes from the L2 goes first, for the whole workgroup: the operand fragments and row scales (written by the
+    // quantizer's launch, read by every workgroup) come back in a fraction of the time a weight byte takes, but a compute
+    // unit serves its requests in the order issued -- behind the first weight requests they would wait for HBM.  One
+    // barrier, reached within a few instructions, keeps every wavefront's weight requests behind all of these.
     // row scales: 64 bytes a pair; lane L of load q takes slot L % 16 of pair 4 q + L / 16
+    // operand fragments, compact: 512 bytes a pair, two pairs a load; lane L of load q holds entry
+    // L % 32 of pair 2 q + L / 32
+    // (Inline assembly: the compiler may move its own loads from read-only memory across the barrier; waited for by
+    // hand before the first stage is used.)
     constexpr int kScaleLoads = (kPairs + 3) / 4;
     float sx_part[kScaleLoads];
+    bm_v4i packed[kPairs / 2];
+    {
+        uint32_t frag_off[kPairs / 2], scale_off[kScaleLoads];
 #pragma unroll
-    for (int q = 0; q < kScaleLoads; ++q)
-        sx_part[q] = sa8[min(pair0 + 4 * q + g, pairs_total - 1) * 16 + l16];
+        for (int q = 0; q < kPairs / 2; ++q) frag_off[q] = static_cast<uint32_t>(min(pair0 + 2 * q + (lane >> 5), pairs_total - 1) * 32 + (lane & 31)) * 16u;
+#pragma unroll
+        for (int q = 0; q < kScaleLoads; ++q) scale_off[q] = static_cast<uint32_t>(min(pair0 + 4 * q + g, pairs_total - 1) * 16 + l16) * 4u;
+#pragma unroll
+        for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(frag_off[q]));
+#pragma unroll
+        for (int q = 0; q < kScaleLoads; ++q) asm volatile("" : "+v"(scale_off[q]));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < kPairs / 2; ++q) asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(packed[q]) : "v"(frag_off[q]), "s"(qa8) : "memory");
+#pragma unroll
+        for (int q = 0; q < kScaleLoads; ++q) asm volatile("global_load_dword %0, %1, %2" : "=v"(sx_part[q]) : "v"(scale_off[q]), "s"(sa8) : "memory");
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    issue_stage(0);
     // weight scales, fp16 in block order (rows of whole 16-byte runs: the host sends no other shape
     // here): word p of a column's run holds blocks 2p and 2p + 1; lane group g takes words
     // [g * kWpl, +kWpl) and the lane exchange hands word p out when its stage comes
@@ -517,14 +543,6 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         } else {
             tb_part[cg][0] = run[0];
         }
-    }
-    // operand fragments, compact: 512 bytes a pair, two pairs a load; lane L of load q holds entry
-    // L % 32 of pair 2 q + L / 32
-    const bm_v4i* qa4 = reinterpret_cast<const bm_v4i*>(qa8);
-    bm_v4i packed[kPairs / 2];
-#pragma unroll
-    for (int q = 0; q < kPairs / 2; ++q) {
-        packed[q] = qa4[static_cast<size_t>(min(pair0 + 2 * q + (lane >> 5), pairs_total - 1)) * 32 + (lane & 31)];
     }
     constexpr int kSpares = 2;
     uint32_t spare[kSpares];
