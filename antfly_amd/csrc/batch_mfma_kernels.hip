@@ -525,14 +525,63 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
     }
+    // Weight scales, fp16 in block order (rows of whole 16-byte runs: the host sends no other shape here): word p of a
+    // column's run holds blocks 2p and 2p + 1.
+    // Q4_0 on tiles of two column groups and more: the workgroup's scales of this K share -- up to 64 columns x 256 bytes
+    // -- go through LDS.  Thread t fetches sixteen bytes (eight blocks) per round, sixteen threads a column: whole
+    // 128-byte lines, each asked for once per workgroup and ahead of the first weight stage.  (A wavefront fetching its
+    // own sixteen blocks of every column asks for 64 pieces of 32 bytes; with the eight wavefronts' 512 requests per
+    // compute unit a launch on 14336 columns took 0.4 us longer, a pair of them 0.9.)  In LDS a column's sixteen chunks
+    // are stored at chunk ^ (column % 16): the sixteen columns a step reads one word of then sit in sixteen different
+    // banks.  (16-column tiles keep the register form: 7.14 against 7.26 us on 4096 columns.)
+    constexpr bool kScalesInLds = kType == 2 && kCG >= 2;
+    constexpr int kChunks = F::kShareBlocks / 8;
+    constexpr int kScaleRounds = (16 * kCG * kChunks + kBmThreads - 1) / kBmThreads;  // rounds of the workgroup's threads over the tile's columns
+    constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
+    unsigned char* lds_scales = bm_lds + kBmLdsBytes;
+    bm_v4i scale_run[kScaleRounds];
+    if (kScalesInLds) {
+        const uint8_t* sbase = weight + blocks_total * kQB + static_cast<size_t>(n0) * kb_full * 2;
+        uint32_t run_off[kScaleRounds];
+#pragma unroll
+        for (int r = 0; r < kScaleRounds; ++r) {
+            const int c = tid / kChunks + r * (kBmThreads / kChunks), chunk = tid % kChunks;
+            const int cc = min(n0 + min(c, cols - 1), out_dim - 1) - n0;
+            run_off[r] = static_cast<uint32_t>(cc * kb_full + min(share_begin + 8 * chunk, kb_full - 8)) * 2u;
+            asm volatile("" : "+v"(run_off[r]));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < kScaleRounds; ++r) {
+            scale_run[r] = bm_v4i{0, 0, 0, 0};
+            if (tid / kChunks + r * (kBmThreads / kChunks) < 16 * kCG)
+                asm volatile("global_load_dwordx4 %0, %1, %2" : "+v"(scale_run[r]) : "v"(run_off[r]), "s"(sbase) : "memory");
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     issue_stage(0);
-    // weight scales, fp16 in block order (rows of whole 16-byte runs: the host sends no other shape
-    // here): word p of a column's run holds blocks 2p and 2p + 1; lane group g takes words
-    // [g * kWpl, +kWpl) and the lane exchange hands word p out when its stage comes
+    if (kScalesInLds) {
+        // the scale runs are there when at most the first stage's two requests are in flight; the workgroup meets once they
+        // are in LDS (the first stage is waited for behind that, with nothing else of the wavefront outstanding: behind
+        // the second stage's requests the wait would also have to see those accepted by the memory pipeline, which for
+        // the last wavefronts of a unit is well into the stream)
+        asm volatile("s_waitcnt vmcnt(2)" : : : "memory");
+#pragma unroll
+        for (int r = 0; r < kScaleRounds; ++r) {
+            asm volatile("" : "+v"(scale_run[r]));
+            const int c = tid / kChunks + r * (kBmThreads / kChunks), chunk = tid % kChunks;
+            if (c < 16 * kCG) *reinterpret_cast<bm_v4i*>(lds_scales + c * (kChunks * 16) + ((chunk ^ (c & (kChunks - 1))) << 4)) = scale_run[r];
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    }
+    // Q8_0: lane group g takes words [g * kWpl, +kWpl) of its wavefront's blocks and the lane exchange hands word p
+    // out when its stage comes
     constexpr int kWpl = kPairs / 4;
     uint32_t tb_part[kCG][kWpl];
 #pragma unroll
-    for (int cg = 0; cg < kCG; ++cg) {
+    for (int cg = 0; cg < (kScalesInLds ? 0 : kCG); ++cg) {
         const int cc = min(n0 + min(16 * cg + l16, cols - 1), out_dim - 1);
         const uint16_t* sw = reinterpret_cast<const uint16_t*>(weight + blocks_total * kQB) + static_cast<size_t>(cc) * kb_full;
         const uint32_t* run = reinterpret_cast<const uint32_t*>(sw + min(blk0, kb_full - 8)) + g * kWpl;
@@ -545,10 +594,11 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         }
     }
     constexpr int kSpares = 2;
-    uint32_t spare[kSpares];
+    uint32_t spare[kSpares] = {0, 0};
+    if (!kScalesInLds) {  // (Q4_0 has no load of the compiler's left: nothing to keep its waits from)
 #pragma unroll
-    for (int k = 0; k < kSpares; ++k) spare[k] = __builtin_nontemporal_load(qa8 + k * 32 + (lane & 31));  // inside the first pair's entries
-    constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
+        for (int k = 0; k < kSpares; ++k) spare[k] = __builtin_nontemporal_load(qa8 + k * 32 + (lane & 31));  // inside the first pair's entries
+    }
     // Q4_0 asks for the second stage only when the first one and the register loads are there (below); Q8_0, whose
     // stages are half as many blocks, measured better with the second stage requested up front.
     constexpr bool kStartupAlone = kType == 2;
@@ -606,15 +656,12 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
             if (it % kHalfPairs == 0) {
                 const int st = stage_of(it), hb = st / kCG, cg = st % kCG;
                 if (st == 0) {
-                    // the first stage and all the register loads, waited for while nothing else of this wavefront is
-                    // outstanding: behind the second stage's requests the wait would also have to see those accepted by
-                    // the memory pipeline, which for the last wavefronts of a unit is well into the stream
                     if (kStartupAlone) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * (kAheadStages - 1)) : "memory");
 #pragma unroll
                     for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(packed[q]));
 #pragma unroll
-                    for (int c = 0; c < kCG; ++c) asm volatile("" : "+v"(tb_part[c][0]), "+v"(tb_part[c][kWpl - 1]));
+                    for (int c = 0; c < (kScalesInLds ? 0 : kCG); ++c) asm volatile("" : "+v"(tb_part[c][0]), "+v"(tb_part[c][kWpl - 1]));
                     asm volatile("" : "+v"(sx_part[0]), "+v"(sx_part[kScaleLoads - 1]));
                 }
                 if (kStartupAlone && st == 0) {
@@ -630,7 +677,13 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
 #pragma unroll
                 for (int q = 0; q < kHalfPairs; ++q) {
                     const int p = hb * kHalfPairs + q;
-                    const uint32_t word = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(4 * (16 * (p / kWpl) + l16), static_cast<int>(tb_part[cg][p % kWpl])));
+                    uint32_t word;
+                    if (kScalesInLds) {
+                        const int c = 16 * cg + l16, pw = wave * kPairs + p;  // column of the tile, pair of the share
+                        word = *reinterpret_cast<const uint32_t*>(lds_scales + c * (kChunks * 16) + (((pw >> 2) ^ (c & (kChunks - 1))) << 4) + ((pw & 3) << 2));
+                    } else {
+                        word = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(4 * (16 * (p / kWpl) + l16), static_cast<int>(tb_part[cg][p % kWpl])));
+                    }
                     const float sw = half_bits_to_f32(static_cast<uint16_t>(word >> (16 * kh))) * (kType == 2 ? 0.0625f : 1.0f);
                     tbm[q] = (g < 2 && 2 * p + g < nb) ? sw : 0.0f;
                 }
@@ -977,16 +1030,36 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
 #undef AFHIP_BM
 }
 
+// LDS of an eight-row launch: the wavefronts' rings, and for Q4_0 the workgroup's weight scales of one K share
+static size_t bm8_lds_bytes(int tensor_type, int column_groups) {
+    return kBmLdsBytes + (tensor_type == 2 && column_groups >= 2 ? 16 * column_groups * (BmFormat<2>::kShareBlocks / 8) * 16 : 0);
+}
+// (raising a kernel's limit is sticky: once per instantiation)
+template <typename Kernel>
+static hipError_t bm_allow_large_lds(Kernel kernel, size_t lds, std::atomic<size_t>* limit) {
+    if (lds <= limit->load(std::memory_order_acquire)) return hipSuccess;
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (e == hipSuccess) limit->store(160 * 1024, std::memory_order_release);
+    return e;
+}
+
 template <int kType, int kCG>
 hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
                       int in_dim, int out_dim, int shares, int share_blocks, int cols, const Epilogue& ep, const BmSecond& second) {
     const dim3 grid(static_cast<unsigned>((out_dim + cols - 1) / cols), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
-    if (cols == 16 * kCG)
-        hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG, false, true>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa,
-                           weight, rows, in_dim, out_dim, share_blocks, cols, ep, second);
-    else
-        hipLaunchKernelGGL((batch8_mfma_kernel<kType, kCG>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight,
-                           rows, in_dim, out_dim, share_blocks, cols, ep, second);
+    const size_t lds = bm8_lds_bytes(kType, kCG);
+    static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
+    if (cols == 16 * kCG) {
+        auto kernel = batch8_mfma_kernel<kType, kCG, false, true>;
+        if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[0]); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks,
+                           cols, ep, second);
+    } else {
+        auto kernel = batch8_mfma_kernel<kType, kCG>;
+        if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[1]); e != hipSuccess) return e;
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks,
+                           cols, ep, second);
+    }
     return hipGetLastError();
 }
 
@@ -1178,7 +1251,9 @@ hipError_t launch_batch8_timeline(hipStream_t stream, uint32_t* stamps, size_t s
     hipLaunchKernelGGL(quantize_fragments8_kernel<2>, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, stream, input, rows, in_dim, qa, sa);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     int share_blocks = (kb + BmFormat<2>::kWaveBlocks - 1) / BmFormat<2>::kWaveBlocks * BmFormat<2>::kWaveBlocks;
-    hipLaunchKernelGGL((batch8_mfma_kernel<2, 4, true>), dim3(static_cast<unsigned>(groups), 1, 1), dim3(kBmThreads), kBmLdsBytes, stream,
+    static std::atomic<size_t> lds_limit{64 * 1024};
+    if (hipError_t e = bm_allow_large_lds(batch8_mfma_kernel<2, 4, true>, bm8_lds_bytes(2, 4), &lds_limit); e != hipSuccess) return e;
+    hipLaunchKernelGGL((batch8_mfma_kernel<2, 4, true>), dim3(static_cast<unsigned>(groups), 1, 1), dim3(kBmThreads), bm8_lds_bytes(2, 4), stream,
                        reinterpret_cast<float*>(stamps), static_cast<float*>(nullptr), qa, sa, weight_prepared, rows, in_dim, out_dim, share_blocks,
                        cols, Epilogue{}, BmSecond{nullptr, nullptr, Epilogue{}});
     return hipGetLastError();
