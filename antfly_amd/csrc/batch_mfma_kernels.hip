@@ -527,14 +527,15 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     }
     // Weight scales, fp16 in block order (rows of whole 16-byte runs: the host sends no other shape here): word p of a
     // column's run holds blocks 2p and 2p + 1.
-    // Q4_0 on tiles of two column groups and more: the workgroup's scales of this K share -- up to 64 columns x 256 bytes
-    // -- go through LDS.  Thread t fetches sixteen bytes (eight blocks) per round, sixteen threads a column: whole
-    // 128-byte lines, each asked for once per workgroup and ahead of the first weight stage.  (A wavefront fetching its
-    // own sixteen blocks of every column asks for 64 pieces of 32 bytes; with the eight wavefronts' 512 requests per
-    // compute unit a launch on 14336 columns took 0.4 us longer, a pair of them 0.9.)  In LDS a column's sixteen chunks
-    // are stored at chunk ^ (column % 16): the sixteen columns a step reads one word of then sit in sixteen different
-    // banks.  (16-column tiles keep the register form: 7.14 against 7.26 us on 4096 columns.)
-    constexpr bool kScalesInLds = kType == 2 && kCG >= 2;
+    // Tiles of three column groups and more: the workgroup's scales of this K share -- up to 64 columns x 256 bytes (Q4_0;
+    // 128 for Q8_0) -- go through LDS.  Thread t fetches sixteen bytes (eight blocks) per round, sixteen (eight) threads a
+    // column: whole 128-byte lines, each asked for once per workgroup and ahead of the first weight stage.  (A wavefront
+    // fetching the scales of its own blocks of every column asks for 64 pieces of 32 (16) bytes; with the eight
+    // wavefronts' 512 requests per compute unit a Q4_0 launch on 14336 columns took 0.4 us longer, a pair of them 0.9,
+    // Q8_0 0.6.)  In LDS a column's chunks are stored at chunk ^ (column % chunks): the sixteen columns a step reads one
+    // word of then sit in different banks.  Smaller tiles keep the register form (Q4_0, 16 columns on 4096: 7.14
+    // against 7.26 us; Q8_0, 32 columns in 2.7 rounds on 11008: 15.6 against 16.1; Q4_0 24 columns on 6144: no difference).
+    constexpr bool kScalesInLds = kCG >= 3;
     constexpr int kChunks = F::kShareBlocks / 8;
     constexpr int kScaleRounds = (16 * kCG * kChunks + kBmThreads - 1) / kBmThreads;  // rounds of the workgroup's threads over the tile's columns
     constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
@@ -1032,7 +1033,8 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
 
 // LDS of an eight-row launch: the wavefronts' rings, and for Q4_0 the workgroup's weight scales of one K share
 static size_t bm8_lds_bytes(int tensor_type, int column_groups) {
-    return kBmLdsBytes + (tensor_type == 2 && column_groups >= 2 ? 16 * column_groups * (BmFormat<2>::kShareBlocks / 8) * 16 : 0);
+    const int share_blocks = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
+    return kBmLdsBytes + (column_groups >= 3 ? 16 * column_groups * (share_blocks / 8) * 16 : 0);
 }
 // (raising a kernel's limit is sticky: once per instantiation)
 template <typename Kernel>
