@@ -109,7 +109,7 @@ static int env_int(const char* name) {
 // (128 on wide Q4_0 matrices), and for Q8_0, whose K shares are half as long, only while all workgroups
 // of the launch are resident at once.  Five to eight rows on a grid that fills the chip always:
 // its eight-row kernel requests weights as it goes and needs neither condition.
-static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
+static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim, bool pair) {
     static const char* v = std::getenv("AFHIP_BATCH_MFMA_MIN_ROWS");
     static const long forced = v && *v ? std::atol(v) : -1;
     // up to 64 rows everywhere; up to 128 on a Q4_0 matrix wide enough to give every compute unit a
@@ -118,6 +118,15 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
     if (forced == 0 || rows > max_rows || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
     if (forced > 0) return rows >= static_cast<size_t>(forced);
     if (rows >= kBatchMfmaMinRows && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
+    // Three and four rows of Q4_0 on more columns than one round of the decode kernel's workgroups takes (64 columns a
+    // compute unit; both matrices of a pair count): the decode kernel's block dots, on the vector ALU, grow with rows
+    // and columns, the eight-row kernel's time does not.  Four rows: a pair of 14336 columns 18.3 -> 16.7 us, 28672
+    // columns 18.5 -> 16.9, 128256 columns 64.6 -> 50.8 (three rows 55.9 -> 49.8); on one round the decode kernel wins
+    // (14336 columns 9.9 against 10.9, a pair of 8192 10.2 against 11.3), and three rows on two rounds are even.
+    if (tensor_type == AFHIP_TYPE_Q4_0 && in_dim <= 4096 && (rows == 3 || rows == 4)) {
+        const size_t round = static_cast<size_t>(gemv_compute_units()) * 64, columns = out_dim * (pair ? 2 : 1);
+        if (columns > (rows == 4 ? round : 2 * round) && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
+    }
     if (rows < (in_dim > 4096 ? kBatchMfmaMinRows + 1 : kBatchMfmaMinRows)) return false;
     if (tensor_type == AFHIP_TYPE_Q8_0) {
         const size_t shares = (in_dim / 32 + 63) / 64, tiles = (out_dim + 31) / 32;
@@ -380,7 +389,10 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
     // Five to 64 (128) rows: the weights are read once, so the single-shot MFMA kernel (X quantized into
     // MFMA operand order first) beats both the row-by-row GEMV and the tiled GEMM.
     if (layout == AFHIP_LAYOUT_PREPARED && !want_dots && kind != AFHIP_DISPATCH_SCALAR &&
-        batch_mfma_preferred(tensor_type, rows, in_dim, out_dim)) {
+        batch_mfma_preferred(tensor_type, rows, in_dim, out_dim, pair) &&
+        // (below five rows the decode kernel, which needs no workspace, remains for a caller that lends none)
+        (rows >= kBatchMfmaMinRows || (workspace.ptr != 0 && workspace.ptr % 16 == 0 &&
+                                       workspace.len >= batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim)))) {
         const size_t need = batch_mfma_workspace_bytes(tensor_type, rows, in_dim, out_dim);
         if (workspace.ptr == 0 || workspace.len < need || workspace.ptr % 16 != 0) return AFHIP_ERR_INVALID_STATE;
         if (counters) {

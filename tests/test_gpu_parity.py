@@ -142,6 +142,8 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # workgroup's 64 columns live (14336), 48 and 40 (three column groups; ragged last tile), 24 (two groups, 6144)
     (8, 512, 14336), (6, 1024, 11008), (5, 256, 10000), (7, 2048, 6144), (8, 256, 9000),
     (5, 8192, 7168),  # ... 56 columns with two K shares (Q4_0)
+    # three and four rows on more columns than one round of the decode kernel's workgroups: Q4_0 takes the eight-row kernel
+    (4, 256, 16448), (3, 256, 33000), (4, 4096, 28672),
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
@@ -213,6 +215,7 @@ PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K sl
     (3, 64, 100), (20, 2048, 300),  # the last: MFMA GEMM with K shared out over workgroups, both matrices through one scratch
     (6, 512, 8200), (7, 9216, 4112),  # the eight-row MFMA kernel, one launch over both matrices; with K shares
     (20, 512, 12290),                 # the 32-row MFMA kernel on 64-column tiles, both matrices
+    (4, 512, 8200), (3, 256, 16500),  # four and three rows whose two matrices together exceed one (two) rounds of the decode kernel
 ]
 
 
@@ -220,8 +223,9 @@ PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K sl
 @pytest.mark.parametrize("layout", [RAW, PREP])
 @pytest.mark.parametrize("rows,in_dim,out_dim", PAIR_SHAPES)
 def test_pair_equals_two_single_ops(fmt, layout, rows, in_dim, out_dim):
-    """Each half of a pair is bit-identical to the single op on that matrix (and so to the
-    oracle within the single op's bound); the op is the engine's two-call fallback fused."""
+    """Each half of a pair is bit-identical to the single op on that matrix where both take the same kernel (and so
+    equal to the oracle within the single op's bound), within that bound of it otherwise; the op is the engine's
+    two-call fallback fused."""
     print(f"case: pair fmt={fmt} layout={layout} rows={rows} in={in_dim} out={out_dim}", flush=True)
     x = synth.activations(510 + rows, rows, in_dim)
     wa = synth.weights(fmt, 511, out_dim, in_dim)
@@ -229,8 +233,18 @@ def test_pair_equals_two_single_ops(fmt, layout, rows, in_dim, out_dim):
     da = G.prepare(fmt, wa, out_dim, in_dim) if layout == PREP else G.to_dev(wa)
     db = G.prepare(fmt, wb, out_dim, in_dim) if layout == PREP else G.to_dev(wb)
     ya, yb = G.linear_pair(fmt, layout, x, da, db, rows, in_dim, out_dim)
-    assert np.array_equal(ya, G.linear(fmt, layout, x, da, rows, in_dim, out_dim))
-    assert np.array_equal(yb, G.linear(fmt, layout, x, db, rows, in_dim, out_dim))
+    sa, sb = G.linear(fmt, layout, x, da, rows, in_dim, out_dim), G.linear(fmt, layout, x, db, rows, in_dim, out_dim)
+    # Three and four rows of Q4_0: the pair's two matrices together may exceed one (two) rounds of the decode kernel's
+    # workgroups (64 columns a compute unit, 256 units) where one matrix does not; the pair then runs on the eight-row
+    # MFMA kernel and a single op on the decode kernel -- the same block dots, another f32 summation order.
+    one_round = 256 * 64 * (1 if rows == 4 else 2)
+    routes_differ = (fmt == Q4 and layout == PREP and rows in (3, 4) and in_dim <= 4096 and in_dim % 256 == 0 and
+                     out_dim <= one_round < 2 * out_dim)
+    if routes_differ:
+        assert G.max_rel_err(ya, sa.astype(np.float64)) <= TIGHT and G.max_rel_err(yb, sb.astype(np.float64)) <= TIGHT
+    else:
+        assert np.array_equal(ya, sa)
+        assert np.array_equal(yb, sb)
     ref_b = O.linear_no_bias(fmt, x, wb, rows, in_dim, out_dim, workers=8)
     assert G.max_rel_err(yb, ref_b.astype(np.float64)) <= TIGHT
 
