@@ -441,7 +441,12 @@ static afhip_status linear_impl_body(void* stream_v, int tensor_type, int layout
         }
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
-    if (fused_ok && rows >= 2 && in_dim > 4096) {
+    // (Two rows up to K = 11008 stay on the decode kernel below: one launch, the K slices of a column group meet inside the
+    // workgroup.  Measured against this path's kernel + reduce launch: K = 6144 x N = 4096 6.0 against 7.2 us, K = N = 8192
+    // 8.7 against 10.5, a pair of K = 8192 x N = 4096 8.7 against 12.2, K = 11008 8.4 against 9.0, Q8_0 K = N = 8192 14.7
+    // against 19.2; from K = 12288 on this path wins -- 9.3 against 9.5, N = 8192 15.0 against 17.0 -- and with three and
+    // four rows it does from K = 6144 on.)
+    if (fused_ok && rows >= 2 && in_dim > 4096 && !(rows == 2 && in_dim <= 11008)) {
         // small batches on a K longer than 4096 (also when a plan forces them on more rows: slices
         // of eight rows): K is shared out over workgroups, each of which stages and quantizes only
         // its 4096-value slice of X; the slices' sums meet in the caller's scratch.

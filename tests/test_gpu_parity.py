@@ -128,6 +128,8 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # ... and the long-K kernel (K > 4096, two to seven rows, sixteen-wavefront workgroups): full and ragged last slice,
     # ragged columns, the most rows the counter form takes
     (2, 8192, 2048), (4, 9216, 4100), (3, 14336, 4096), (7, 8192, 4096), (5, 4128, 2100),
+    (2, 14336, 2048), (2, 12288, 4100),  # (two rows take that kernel from K = 12288 on; below, the decode kernel with K slices)
+    (2, 11008, 1030), (2, 6144, 4100),
     # the single-shot MFMA kernel (5..64 rows): every count of live result registers, two row tiles, a K
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
