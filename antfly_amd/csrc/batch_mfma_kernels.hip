@@ -398,11 +398,20 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
 // k order, lane half h = g % 2:  Q8_0: values [16 h, 16 h + 16).  Q4_0: dwords x[8h..8h+3],
 // x[16+8h..+3], x[8h+4..8h+7], x[16+8h+4..+7] -- the low and the high nibbles of bytes [8 h, 8 h + 8) of
 // the block, dword by dword, so that one lane unpacks whole bytes.
+// zero_a (and zero_b): result arrays of zero_count floats that the matmul launch behind this one adds its two K shares'
+// sums to; cleared here, by the launch that has to run first anyway.
 template <int kType>
 __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* __restrict__ x, int rows, int in_dim,
-                                                                   uint32_t* __restrict__ qa8, float* __restrict__ sa8) {
+                                                                   uint32_t* __restrict__ qa8, float* __restrict__ sa8,
+                                                                   float* __restrict__ zero_a, float* __restrict__ zero_b, int zero_count) {
     const int kb = in_dim >> 5, slots = ((kb + 1) >> 1) * 2;  // block slots: whole pairs
     const int units = 8 * slots * 8;                           // (row, block slot, eight lanes)
+    if (zero_a != nullptr) {
+        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < zero_count; i += gridDim.x * blockDim.x) {
+            zero_a[i] = 0.0f;
+            if (zero_b != nullptr) zero_b[i] = 0.0f;
+        }
+    }
     for (int u = blockIdx.x * blockDim.x + threadIdx.x; u < units; u += gridDim.x * blockDim.x) {
         const int j = u & 7, bs = (u >> 3) % slots, r = (u >> 3) / slots;
         const bool real = r < rows && bs < kb;
@@ -428,11 +437,13 @@ __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* _
 // 100 MHz clock at dst_a[8 * (8 * workgroup + wavefront)]: [0] entry, [1] .. [4] the first four stages' bytes there, [5] the last
 // stage's, [6] K loop done, [7] after the workgroup's reduction.
 // kFullCols: a workgroup takes all 16 kCG columns (`cols` is not looked at).
+// accumulate: the launch has exactly two K shares and no epilogue; the result array has been cleared (by the quantizer's
+// launch) and each share adds its sums with a float atomic -- no partial sums in scratch, no reduce launch behind.
 template <int kType, int kCG, bool kStamps = false, bool kFullCols = false>
 __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                      const uint32_t* __restrict__ qa8, const float* __restrict__ sa8,
                                                                      const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
-                                                                     int share_blocks, int cols_arg, Epilogue ep_a, BmSecond second) {
+                                                                     int share_blocks, int cols_arg, int accumulate, Epilogue ep_a, BmSecond second) {
     uint32_t stamp[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (kStamps) stamp[0] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     using F = BmFormat<kType>;
@@ -765,6 +776,8 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         } else if (m < rows && c < cols && n < out_dim) {
             const size_t at = static_cast<size_t>(m) * out_dim + n;
             if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+            // two K shares, no epilogue: both add to the zeroed result; 0 + a + b = 0 + b + a to the bit, whoever comes first
+            else if (accumulate) unsafeAtomicAdd(dst + at, sum);
             else dst[at] = finish_output(ep, n, at, sum);
         }
     }
@@ -1047,20 +1060,21 @@ static hipError_t bm_allow_large_lds(Kernel kernel, size_t lds, std::atomic<size
 
 template <int kType, int kCG>
 hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
-                      int in_dim, int out_dim, int shares, int share_blocks, int cols, const Epilogue& ep, const BmSecond& second) {
+                      int in_dim, int out_dim, int shares, int share_blocks, int cols, bool accumulate, const Epilogue& ep, const BmSecond& second) {
     const dim3 grid(static_cast<unsigned>((out_dim + cols - 1) / cols), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
+    if (accumulate || shares == 1) partial = nullptr;
     const size_t lds = bm8_lds_bytes(kType, kCG);
     static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
     if (cols == 16 * kCG) {
         auto kernel = batch8_mfma_kernel<kType, kCG, false, true>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[0]); e != hipSuccess) return e;
-        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks,
-                           cols, ep, second);
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
+                           accumulate ? 1 : 0, ep, second);
     } else {
         auto kernel = batch8_mfma_kernel<kType, kCG>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[1]); e != hipSuccess) return e;
-        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks,
-                           cols, ep, second);
+        hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
+                           accumulate ? 1 : 0, ep, second);
     }
     return hipGetLastError();
 }
@@ -1175,15 +1189,22 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const long bound = bound_set >= 0 ? bound_set : gemv_compute_units();
     const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
                             static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
+    // Two K shares and nothing to do to the sums but add them: the eight-row kernel's shares add to the result themselves
+    // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
+    auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
+    const bool accumulate = eight && real_shares == 2 && plain(ep) && (weight_b_prepared == nullptr || plain(ep_b));
     if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
         const int pairs = (kb + 1) / 2;
         sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
         const int units = 8 * (2 * pairs) * 8;
         const dim3 qgrid(static_cast<unsigned>((units + 255) / 256));
+        float* zero_a = accumulate ? dst : nullptr;
+        float* zero_b = accumulate && weight_b_prepared ? dst_b : nullptr;
+        const int zero_count = rows * out_dim;
         if (tensor_type == 2)
-            hipLaunchKernelGGL(quantize_fragments8_kernel<2>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+            hipLaunchKernelGGL(quantize_fragments8_kernel<2>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa, zero_a, zero_b, zero_count);
         else
-            hipLaunchKernelGGL(quantize_fragments8_kernel<8>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+            hipLaunchKernelGGL(quantize_fragments8_kernel<8>, qgrid, dim3(256), 0, stream, input, rows, in_dim, qa, sa, zero_a, zero_b, zero_count);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     } else {
         const size_t units = static_cast<size_t>(padded) * (in_dim / 4);
@@ -1205,7 +1226,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     hipError_t e;
     if (eight) {
         const int cols = bm8_columns(tensor_type, in_dim, out_dim, weight_b_prepared != nullptr), cg = (cols + 15) / 16;
-#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, ep, second)
+#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
         if (tensor_type == 2) e = cg == 4 ? AFHIP_BM8(2, 4) : (cg == 3 ? AFHIP_BM8(2, 3) : (cg == 2 ? AFHIP_BM8(2, 2) : AFHIP_BM8(2, 1)));
         else e = cg == 4 ? AFHIP_BM8(8, 4) : (cg == 3 ? AFHIP_BM8(8, 3) : (cg == 2 ? AFHIP_BM8(8, 2) : AFHIP_BM8(8, 1)));
 #undef AFHIP_BM8
@@ -1218,7 +1239,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
                        ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
                        : bm_launch_rows<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
     if (e != hipSuccess) return e;
-    if (real_shares > 1) {
+    if (real_shares > 1 && !accumulate) {
         e = launch_splitk_reduce(stream, dst, partial, count, out_dim, real_shares, ep);
         if (e != hipSuccess) return e;
         if (weight_b_prepared) {
@@ -1248,14 +1269,15 @@ hipError_t launch_batch8_timeline(hipStream_t stream, uint32_t* stamps, size_t s
     const int pairs = (kb + 1) / 2;
     float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
     const int units = 8 * (2 * pairs) * 8;
-    hipLaunchKernelGGL(quantize_fragments8_kernel<2>, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, stream, input, rows, in_dim, qa, sa);
+    hipLaunchKernelGGL(quantize_fragments8_kernel<2>, dim3(static_cast<unsigned>((units + 255) / 256)), dim3(256), 0, stream, input, rows, in_dim, qa, sa,
+                       static_cast<float*>(nullptr), static_cast<float*>(nullptr), 0);
     if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     int share_blocks = (kb + BmFormat<2>::kWaveBlocks - 1) / BmFormat<2>::kWaveBlocks * BmFormat<2>::kWaveBlocks;
     static std::atomic<size_t> lds_limit{64 * 1024};
     if (hipError_t e = bm_allow_large_lds(batch8_mfma_kernel<2, 4, true>, bm8_lds_bytes(2, 4), &lds_limit); e != hipSuccess) return e;
     hipLaunchKernelGGL((batch8_mfma_kernel<2, 4, true>), dim3(static_cast<unsigned>(groups), 1, 1), dim3(kBmThreads), bm8_lds_bytes(2, 4), stream,
                        reinterpret_cast<float*>(stamps), static_cast<float*>(nullptr), qa, sa, weight_prepared, rows, in_dim, out_dim, share_blocks,
-                       cols, Epilogue{}, BmSecond{nullptr, nullptr, Epilogue{}});
+                       cols, 0, Epilogue{}, BmSecond{nullptr, nullptr, Epilogue{}});
     return hipGetLastError();
 }
 
