@@ -108,11 +108,20 @@ __device__ __forceinline__ void fence_registers(float (&a)[16]) {
 // kByteOrder (Q4_0 operands of batch32_mfma_kernel): within a block the lane half h holds the dwords
 // x[8h..8h+3], x[16+8h..+3], x[8h+4..8h+7], x[16+8h+4..+7] instead of x[16h..16h+15] -- the values whose
 // nibbles share the bytes [8 h, 8 h + 8) of the weight block, so that a lane unpacks whole bytes.
+// zero_a (and zero_b): result arrays of zero_count floats that the matmul launch behind this one adds its two K shares'
+// sums to; cleared here, by the launch that has to run first anyway.
 template <bool kByteOrder>
 __global__ __launch_bounds__(256) void quantize_fragments_kernel(const float* __restrict__ x, int rows, int in_dim, int row_tiles,
-                                                                  uint32_t* __restrict__ qa, float* __restrict__ sa) {
+                                                                  uint32_t* __restrict__ qa, float* __restrict__ sa,
+                                                                  float* __restrict__ zero_a, float* __restrict__ zero_b, size_t zero_count) {
     const int units_per_row = in_dim >> 2, kb = in_dim >> 5, padded = row_tiles * 32;
     const size_t units = static_cast<size_t>(padded) * units_per_row;
+    if (zero_a != nullptr) {
+        for (size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; i < zero_count; i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+            zero_a[i] = 0.0f;
+            if (zero_b != nullptr) zero_b[i] = 0.0f;
+        }
+    }
     for (size_t u = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; u < units;
          u += static_cast<size_t>(gridDim.x) * blockDim.x) {
         const int r = static_cast<int>(u / units_per_row), c4 = static_cast<int>(u % units_per_row);
@@ -136,7 +145,7 @@ template <int kType, int kRowTiles, int kLive>
 __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                   const uint32_t* __restrict__ qa, const float* __restrict__ sa,
                                                                   const uint8_t* __restrict__ weight_a, int rows, int in_dim,
-                                                                  int out_dim, int share_blocks, Epilogue ep_a, BmSecond second) {
+                                                                  int out_dim, int share_blocks, Epilogue ep_a, BmSecond second, int accumulate) {
     using F = BmFormat<kType>;
     // blockIdx.z == 1: the second matrix of a pair (same X, same shape)
     const bool is_b = blockIdx.z != 0;
@@ -358,6 +367,7 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
             if (m < rows && n < out_dim) {
                 const size_t at = static_cast<size_t>(m) * out_dim + n;
                 if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                else if (accumulate) unsafeAtomicAdd(dst + at, sum);  // (two K shares, no epilogue, the result cleared beforehand: see batch8_mfma_kernel)
                 else dst[at] = finish_output(ep, n, at, sum);
             }
         }
@@ -816,7 +826,7 @@ template <int kType, int kRT, int kLive>
 __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                       const uint32_t* __restrict__ qa, const float* __restrict__ sa,
                                                                       const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
-                                                                      int share_blocks, Epilogue ep_a, BmSecond second) {
+                                                                      int share_blocks, Epilogue ep_a, BmSecond second, int accumulate) {
     using F = BmFormat<kType>;
     const bool is_b = blockIdx.z != 0;
     float* dst = is_b ? second.dst : dst_a;
@@ -1012,6 +1022,7 @@ __global__ __launch_bounds__(kBmThreads, 2) void batch32_mfma_kernel(float* __re
                 for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
                 const size_t at = static_cast<size_t>(m) * out_dim + n;
                 if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                else if (accumulate) unsafeAtomicAdd(dst + at, sum);  // (two K shares, no epilogue, the result cleared beforehand: see batch8_mfma_kernel)
                 else dst[at] = finish_output(ep, n, at, sum);
             }
         }
@@ -1022,18 +1033,18 @@ namespace {
 
 template <int kType, int kRowTiles, int kLive>
 hipError_t bm_launch(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
-                     int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+                     int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second, bool accumulate) {
     const dim3 grid(static_cast<unsigned>((out_dim + 31) / 32), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
     hipLaunchKernelGGL((batch_mfma_kernel<kType, kRowTiles, kLive>), grid, block, kBmLdsBytes, stream, dst,
-                       shares > 1 ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep, second);
+                       shares > 1 && !accumulate ? partial : nullptr, qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep, second, accumulate ? 1 : 0);
     return hipGetLastError();
 }
 
 template <int kType>
 hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight,
-                          int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+                          int rows, int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second, bool accumulate) {
 #define AFHIP_BM(TILES, LIVE) \
-    return bm_launch<kType, TILES, LIVE>(stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, shares, share_blocks, ep, second)
+    return bm_launch<kType, TILES, LIVE>(stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, shares, share_blocks, ep, second, accumulate)
     if (rows <= 8) AFHIP_BM(1, 4);
     if (rows <= 16) AFHIP_BM(1, 8);
     if (rows <= 24) AFHIP_BM(1, 12);
@@ -1119,11 +1130,11 @@ int bm8_columns(int tensor_type, int in_dim, int out_dim, bool pair) {
 
 template <int kType>
 hipError_t bm_launch32(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
-                       int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second) {
+                       int in_dim, int out_dim, int shares, int share_blocks, const Epilogue& ep, const BmSecond& second, bool accumulate) {
     const dim3 grid(static_cast<unsigned>((out_dim + 63) / 64), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
 #define AFHIP_BM32(RT, LIVE)                                                                                                                 \
-    hipLaunchKernelGGL((batch32_mfma_kernel<kType, RT, LIVE>), grid, block, kBmLdsBytes, stream, dst, shares > 1 ? partial : nullptr, qa, sa, \
-                       weight, rows, in_dim, out_dim, share_blocks, ep, second)
+    hipLaunchKernelGGL((batch32_mfma_kernel<kType, RT, LIVE>), grid, block, kBmLdsBytes, stream, dst, shares > 1 && !accumulate ? partial : nullptr, \
+                       qa, sa, weight, rows, in_dim, out_dim, share_blocks, ep, second, accumulate ? 1 : 0)
     if (rows <= 16) AFHIP_BM32(1, 8);
     else if (rows <= 24) AFHIP_BM32(1, 12);
     else if (rows <= 32) AFHIP_BM32(1, 16);
@@ -1189,10 +1200,10 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const long bound = bound_set >= 0 ? bound_set : gemv_compute_units();
     const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && bm8_column_groups(out_dim) == 4 &&
                             static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
-    // Two K shares and nothing to do to the sums but add them: the eight-row kernel's shares add to the result themselves
+    // Two K shares and nothing to do to the sums but add them: the kernel's shares add to the result themselves
     // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
     auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
-    const bool accumulate = eight && real_shares == 2 && plain(ep) && (weight_b_prepared == nullptr || plain(ep_b));
+    const bool accumulate = real_shares == 2 && plain(ep) && (weight_b_prepared == nullptr || plain(ep_b));
     if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
         const int pairs = (kb + 1) / 2;
         sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
@@ -1210,12 +1221,15 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
         const size_t units = static_cast<size_t>(padded) * (in_dim / 4);
         size_t grid = (units + 255) / 256;
         if (grid > 4096) grid = 4096;
+        float* zero_a = accumulate ? dst : nullptr;
+        float* zero_b = accumulate && weight_b_prepared ? dst_b : nullptr;
+        const size_t zero_count = static_cast<size_t>(rows) * out_dim;
         if (thirty_two && tensor_type == 2)
             hipLaunchKernelGGL(quantize_fragments_kernel<true>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
-                               row_tiles, qa, sa);
+                               row_tiles, qa, sa, zero_a, zero_b, zero_count);
         else
             hipLaunchKernelGGL(quantize_fragments_kernel<false>, dim3(static_cast<unsigned>(grid)), dim3(256), 0, stream, input, rows, in_dim,
-                               row_tiles, qa, sa);
+                               row_tiles, qa, sa, zero_a, zero_b, zero_count);
         if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
     }
     // (an op that is being timed: its activation-quantizer phase ends here)
@@ -1232,12 +1246,12 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
 #undef AFHIP_BM8
     }
     else if (thirty_two)
-        e = tensor_type == 2 ? bm_launch32<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
-                             : bm_launch32<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
+        e = tensor_type == 2 ? bm_launch32<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second, accumulate)
+                             : bm_launch32<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second, accumulate);
     else
         e = tensor_type == 2
-                       ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second)
-                       : bm_launch_rows<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second);
+                       ? bm_launch_rows<2>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second, accumulate)
+                       : bm_launch_rows<8>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, ep, second, accumulate);
     if (e != hipSuccess) return e;
     if (real_shares > 1 && !accumulate) {
         e = launch_splitk_reduce(stream, dst, partial, count, out_dim, real_shares, ep);
