@@ -127,6 +127,22 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
         const size_t round = static_cast<size_t>(gemv_compute_units()) * 64, columns = out_dim * (pair ? 2 : 1);
         if (columns > (rows == 4 ? round : 2 * round) && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
     }
+    // Two to four rows on a K beyond 4096, against the kernel that shares K out over workgroups and its reduce launch
+    // (us, that kernel first): Q4_0 four rows 6144 x 4096 columns 9.9 / 8.4, 8192 x 8192 12.5 / 11.3, 14336 x 4096
+    // 12.7 / 11.7, 14336 x 8192 21.0 / 16.5; three rows 6144 x 2048 8.6 / 6.7, 8192 x 4096 8.9 / 9.0, 14336 x 8192
+    // 18.9 / 16.5, but 11008 x 4096 10.7 / 11.4 and 14336 x 2048 8.9 / 9.7; two rows stay (8192 x 8192 8.4 / 11.3).
+    // Q8_0 three and four rows everywhere (8192 x 8192 20.0 / 15.0, 6144 x 2048 7.7 / 6.9); two rows on a long K or
+    // a wide matrix (14336 x 4096 15.7 / 14.3, 6144 x 16384 25.1 / 21.1, but 8192 x 4096 8.2 / 10.0).  (One matrix's
+    // columns also for a pair: both halves take the kernel the single op takes.)
+    if (in_dim > 4096 && rows >= 2 && rows <= 4 && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) {
+        if (tensor_type == AFHIP_TYPE_Q4_0) {
+            if (rows == 4) return true;
+            if (rows == 3) return in_dim <= 8192 || out_dim >= 8192;
+        } else {
+            if (rows >= 3) return true;
+            return (in_dim > 11008 && out_dim >= 4096) || out_dim > 8192;
+        }
+    }
     if (rows < (in_dim > 4096 ? kBatchMfmaMinRows + 1 : kBatchMfmaMinRows)) return false;
     if (tensor_type == AFHIP_TYPE_Q8_0) {
         const size_t shares = (in_dim / 32 + 63) / 64, tiles = (out_dim + 31) / 32;

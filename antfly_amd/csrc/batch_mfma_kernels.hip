@@ -449,7 +449,10 @@ __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* _
 // kFullCols: a workgroup takes all 16 kCG columns (`cols` is not looked at).
 // accumulate: the launch has exactly two K shares and no epilogue; the result array has been cleared (by the quantizer's
 // launch) and each share adds its sums with a float atomic -- no partial sums in scratch, no reduce launch behind.
-template <int kType, int kCG, bool kStamps = false, bool kFullCols = false>
+// kHalves: stage rounds of a wavefront -- it owns kHalves runs of eight (Q4_0; four Q8_0) consecutive blocks, and a K share
+// is 8 * kHalves of them: a longer K makes fewer shares (K = 14336 of Q4_0: two of 224 blocks at kHalves = 4 instead of
+// four of 112), and two shares need no reduce launch.
+template <int kType, int kCG, bool kStamps = false, bool kFullCols = false, int kHalves = 2>
 __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                      const uint32_t* __restrict__ qa8, const float* __restrict__ sa8,
                                                                      const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
@@ -462,8 +465,9 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     const uint8_t* weight = is_b ? second.weight : weight_a;
     const Epilogue ep = is_b ? second.ep : ep_a;
     float* partial = partial_a == nullptr ? nullptr : partial_a + (is_b ? static_cast<size_t>(gridDim.y) * rows * out_dim : 0);
-    constexpr int kQB = F::kQuantBytes, kWB = F::kWaveBlocks, kPairs = kWB / 2, kHalfPairs = kPairs / 2;
-    constexpr int kCols = 16 * kCG, kStages = 2 * kCG, kSteps = kStages * kHalfPairs;
+    constexpr int kQB = F::kQuantBytes, kStageBlocks = F::kWaveBlocks / 2, kWB = kHalves * kStageBlocks;
+    constexpr int kPairs = kWB / 2, kHalfPairs = kStageBlocks / 2;  // pairs of blocks: of the wavefront, of a stage
+    constexpr int kCols = 16 * kCG, kStages = kHalves * kCG, kSteps = kStages * kHalfPairs;
     const int kb_full = in_dim >> 5, pairs_total = (kb_full + 1) >> 1;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -556,8 +560,8 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     // Q8_0 0.6.)  In LDS a column's chunks are stored at chunk ^ (column % chunks): the sixteen columns a step reads one
     // word of then sit in different banks.  Smaller tiles keep the register form (Q4_0, 16 columns on 4096: 7.14
     // against 7.26 us; Q8_0, 32 columns in 2.7 rounds on 11008: 15.6 against 16.1; Q4_0 24 columns on 6144: no difference).
-    constexpr bool kScalesInLds = kCG >= 3;
-    constexpr int kChunks = F::kShareBlocks / 8;
+    constexpr bool kScalesInLds = kCG >= 3 || kHalves > 2;
+    constexpr int kChunks = kBmWaves * kWB / 8;
     constexpr int kScaleRounds = (16 * kCG * kChunks + kBmThreads - 1) / kBmThreads;  // rounds of the workgroup's threads over the tile's columns
     constexpr int kAheadStages = 2;  // requested beyond the stage being worked on (the ring has four slots)
     unsigned char* lds_scales = bm_lds + kBmLdsBytes;
@@ -1056,9 +1060,9 @@ hipError_t bm_launch_rows(hipStream_t stream, float* dst, float* partial, const 
 }
 
 // LDS of an eight-row launch: the wavefronts' rings, and for Q4_0 the workgroup's weight scales of one K share
-static size_t bm8_lds_bytes(int tensor_type, int column_groups) {
-    const int share_blocks = tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks;
-    return kBmLdsBytes + (column_groups >= 3 ? 16 * column_groups * (share_blocks / 8) * 16 : 0);
+static size_t bm8_lds_bytes(int tensor_type, int column_groups, int halves = 2) {
+    const int share_blocks = (tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks) / 2 * halves;
+    return kBmLdsBytes + (column_groups >= 3 || halves > 2 ? 16 * column_groups * (share_blocks / 8) * 16 : 0);
 }
 // (raising a kernel's limit is sticky: once per instantiation)
 template <typename Kernel>
@@ -1069,20 +1073,20 @@ static hipError_t bm_allow_large_lds(Kernel kernel, size_t lds, std::atomic<size
     return e;
 }
 
-template <int kType, int kCG>
+template <int kType, int kCG, int kHalves>
 hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
                       int in_dim, int out_dim, int shares, int share_blocks, int cols, bool accumulate, const Epilogue& ep, const BmSecond& second) {
     const dim3 grid(static_cast<unsigned>((out_dim + cols - 1) / cols), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
     if (accumulate || shares == 1) partial = nullptr;
-    const size_t lds = bm8_lds_bytes(kType, kCG);
+    const size_t lds = bm8_lds_bytes(kType, kCG, kHalves);
     static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
     if (cols == 16 * kCG) {
-        auto kernel = batch8_mfma_kernel<kType, kCG, false, true>;
+        auto kernel = batch8_mfma_kernel<kType, kCG, false, true, kHalves>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[0]); e != hipSuccess) return e;
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
                            accumulate ? 1 : 0, ep, second);
     } else {
-        auto kernel = batch8_mfma_kernel<kType, kCG>;
+        auto kernel = batch8_mfma_kernel<kType, kCG, false, false, kHalves>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[1]); e != hipSuccess) return e;
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
                            accumulate ? 1 : 0, ep, second);
@@ -1101,11 +1105,39 @@ int bm_shares(int tensor_type, int in_dim) {
     return (in_dim / 32 + share_max - 1) / share_max;
 }
 
+// The eight-row kernel's stage rounds per wavefront (its kHalves: 2 or 4, Q8_0 also 8) and the K shares that makes.
+// The fewest rounds that leave at most two shares (two add to the result themselves, more need a reduce launch; with
+// fewer, longer shares a workgroup takes fewer columns and fetches more operand fragments for them), else the most.
+// One share instead of two where the two shares' grid of 64-column tiles would not fit the compute units in one round
+// while a single share's may.  (A pair counts as one of its matrices and an epilogue does not enter: each half of a
+// pair stays bit-identical to the single op, and an op with a bias to the plain op plus the bias.)
+// Measured, five rows, against two rounds everywhere (us): Q4_0 K = 14336 x 4096 columns 11.7 against 13.8 (two shares
+// instead of four), 11008 x 4096 11.4 against 13.4, 8192 x 28672 29.3 against 31.2, 28672 x 4096 19.3 against 22.4;
+// Q8_0 4096 x 14336 (eight rows) 14.0 against 15.5 (one share in one round), 4096 x 11008 11.8 against 14.0,
+// 8192 x 8192 15.1 against 22.3 (16.0 as one share), 14336 x 4096 14.4 against 19.3 (16.7 at four rounds).  Where two
+// shares fit one round they stay: Q4_0 8192 x 8192 11.7 (12.6 as one share), 6144 x 4096 8.5 (9.4).
+int bm8_halves(int tensor_type, int in_dim, int out_dim) {
+    const long kb = in_dim / 32, base = (tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks) / 2;
+    const int most = tensor_type == 2 ? 4 : 8;
+    const long tiles = (out_dim + 63) / 64;
+    for (int h = 2; h <= most; h *= 2) {
+        const long shares = (kb + h * base - 1) / (h * base);
+        if (shares > 2) continue;
+        if (shares == 2 && h < most && 2 * tiles > gemv_compute_units()) continue;
+        return h;
+    }
+    return most;
+}
+int bm8_shares(int tensor_type, int in_dim, int halves) {
+    const int share_max = (tensor_type == 2 ? BmFormat<2>::kShareBlocks : BmFormat<8>::kShareBlocks) / 2 * halves;
+    return (in_dim / 32 + share_max - 1) / share_max;
+}
+
 // A single group of sixteen columns a workgroup: for a matrix whose 32-column tiles (times K shares) leave compute
 // units idle while its 16-column tiles fill them in one round -- 4096 columns at K = 4096: 7.9 against 9.0 us on
 // batch_mfma_kernel; with a second, partial round (6144 columns: 9.7 against 9.4) it does not pay.
-bool bm8_one_column_group(int tensor_type, size_t in_dim, size_t out_dim) {
-    const size_t shares = static_cast<size_t>(bm_shares(tensor_type, static_cast<int>(in_dim))), units = static_cast<size_t>(gemv_compute_units());
+bool bm8_one_column_group(size_t shares, size_t out_dim) {
+    const size_t units = static_cast<size_t>(gemv_compute_units());
     const size_t narrow = (out_dim + 15) / 16 * shares;
     return (out_dim + 31) / 32 * shares < units && narrow >= units && narrow <= units + units / 8;
 }
@@ -1120,12 +1152,12 @@ bool bm8_one_column_group(int tensor_type, size_t in_dim, size_t out_dim) {
 // Else the grid takes several rounds whatever the tile, and fewer, larger workgroups fetch the operand fragments less
 // often: 64 columns from 12288 columns on, 16 where that is one round and a bit, else 32 (Q8_0, 14336 columns, two
 // K shares: 18.0 us on 448 workgroups of 64 against 18.9 on 598 of 48; a pair of those 30.2 against 32.2).
-int bm8_columns(int tensor_type, int in_dim, int out_dim, bool pair) {
-    const long units = gemv_compute_units(), shares = bm_shares(tensor_type, in_dim);
+int bm8_columns(long shares, int out_dim, bool pair) {
+    const long units = gemv_compute_units();
     for (long cols = 8; cols <= 64; cols += 8)
         if ((out_dim + cols - 1) / cols * shares * (pair ? 2 : 1) <= units) return static_cast<int>(cols);
     if (bm8_column_groups(out_dim) == 4) return 64;
-    return bm8_one_column_group(tensor_type, static_cast<size_t>(in_dim), static_cast<size_t>(out_dim)) ? 16 : 32;
+    return bm8_one_column_group(static_cast<size_t>(shares), static_cast<size_t>(out_dim)) ? 16 : 32;
 }
 
 template <int kType>
@@ -1184,13 +1216,16 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     float* sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(padded) * in_dim);
     const size_t front = static_cast<size_t>(padded) * in_dim + static_cast<size_t>(kb) * padded * 4;
     float* partial = reinterpret_cast<float*>(workspace + (front + 255) / 256 * 256);
-    const int shares = bm_shares(tensor_type, in_dim);
+    const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);
+    auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
+    const bool both_plain = plain(ep) && (weight_b_prepared == nullptr || plain(ep_b));
+    const int halves = eight ? bm8_halves(tensor_type, in_dim, out_dim) : 2;
+    const int shares = eight ? bm8_shares(tensor_type, in_dim, halves) : bm_shares(tensor_type, in_dim);
     // equal shares, whole wavefront slices: a multiple of the blocks one wavefront owns
-    const int wave_blocks = tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks;
+    const int wave_blocks = (tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks) / 2 * halves;
     int share_blocks = (kb + shares - 1) / shares;
     share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
     const int real_shares = (kb + share_blocks - 1) / share_blocks;
-    const bool eight = batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim);
     // Nine to 64 rows on a matrix wide enough for 64-column tiles (and rows of whole 16-byte runs of
     // scales), with no more workgroups than compute units: batch32_mfma_kernel holds one workgroup per
     // unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
@@ -1202,8 +1237,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
                             static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1) <= bound;
     // Two K shares and nothing to do to the sums but add them: the kernel's shares add to the result themselves
     // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
-    auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
-    const bool accumulate = real_shares == 2 && plain(ep) && (weight_b_prepared == nullptr || plain(ep_b));
+    const bool accumulate = real_shares == 2 && both_plain;
     if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
         const int pairs = (kb + 1) / 2;
         sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
@@ -1239,10 +1273,12 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const BmSecond second{dst_b, weight_b_prepared, ep_b};
     hipError_t e;
     if (eight) {
-        const int cols = bm8_columns(tensor_type, in_dim, out_dim, weight_b_prepared != nullptr), cg = (cols + 15) / 16;
-#define AFHIP_BM8(T, CG) bm_launch8<T, CG>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
-        if (tensor_type == 2) e = cg == 4 ? AFHIP_BM8(2, 4) : (cg == 3 ? AFHIP_BM8(2, 3) : (cg == 2 ? AFHIP_BM8(2, 2) : AFHIP_BM8(2, 1)));
-        else e = cg == 4 ? AFHIP_BM8(8, 4) : (cg == 3 ? AFHIP_BM8(8, 3) : (cg == 2 ? AFHIP_BM8(8, 2) : AFHIP_BM8(8, 1)));
+        const int cols = bm8_columns(real_shares, out_dim, weight_b_prepared != nullptr), cg = (cols + 15) / 16;
+#define AFHIP_BM8(T, CG, H) bm_launch8<T, CG, H>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
+#define AFHIP_BM8_CG(T, H) (cg == 4 ? AFHIP_BM8(T, 4, H) : (cg == 3 ? AFHIP_BM8(T, 3, H) : (cg == 2 ? AFHIP_BM8(T, 2, H) : AFHIP_BM8(T, 1, H))))
+        if (tensor_type == 2) e = halves == 4 ? AFHIP_BM8_CG(2, 4) : AFHIP_BM8_CG(2, 2);
+        else e = halves == 8 ? AFHIP_BM8_CG(8, 8) : (halves == 4 ? AFHIP_BM8_CG(8, 4) : AFHIP_BM8_CG(8, 2));
+#undef AFHIP_BM8_CG
 #undef AFHIP_BM8
     }
     else if (thirty_two)
@@ -1273,7 +1309,7 @@ hipError_t launch_batch8_timeline(hipStream_t stream, uint32_t* stamps, size_t s
     const int kb = in_dim / 32;
     if (rows < 1 || rows > 8 || in_dim % 256 != 0 || kb > BmFormat<2>::kShareBlocks || workspace == nullptr || stamps == nullptr) return hipErrorInvalidValue;
     if (!batch_mfma_supports(2, rows, in_dim, out_dim)) return hipErrorInvalidValue;
-    const int cols = bm8_columns(2, in_dim, out_dim, false);
+    const int cols = bm8_columns(1, out_dim, false);
     if (cols <= 48) return hipErrorInvalidValue;
     const int groups = (out_dim + cols - 1) / cols;
     if (workgroups) *workgroups = groups;

@@ -130,6 +130,9 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (2, 8192, 2048), (4, 9216, 4100), (3, 14336, 4096), (7, 8192, 4096), (5, 4128, 2100),
     (2, 14336, 2048), (2, 12288, 4100),  # (two rows take that kernel from K = 12288 on; below, the decode kernel with K slices)
     (2, 11008, 1030), (2, 6144, 4100),
+    # (three and four rows on whole 256-value runs of K take the eight-row MFMA kernel where that measured faster; the
+    # long-K kernel keeps a K that is not such a multiple, and three rows of Q4_0 on a long K and few columns)
+    (4, 8224, 1030), (3, 6144, 2050), (4, 14336, 1030), (2, 14336, 4100), (3, 11008, 4096),
     # the single-shot MFMA kernel (5..64 rows): every count of live result registers, two row tiles, a K
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
