@@ -127,6 +127,13 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
         const size_t round = static_cast<size_t>(gemv_compute_units()) * 64, columns = out_dim * (pair ? 2 : 1);
         if (columns > (rows == 4 ? round : 2 * round) && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
     }
+    // Q8_0, K of 2048 to 4096 (one K share of the eight-row kernel in one round on a wide matrix): four rows from 11008
+    // columns on (11008 14.2 -> 12.3 us, 14336 16.0 -> 14.4, 28672 29.1 -> 23.8, a pair of 14336 30.1 -> 23.2; 8192 9.3
+    // against 10.0 stays), three rows beyond 14336 (28672 25.9 -> 23.5, K = 2048 x 16384 10.9 -> 9.9; 14336 is even);
+    // two rows stay on the decode kernel everywhere (14336 12.6 against 14.4).  One matrix's columns, also for a pair.
+    if (tensor_type == AFHIP_TYPE_Q8_0 && in_dim >= 2048 && in_dim <= 4096 &&
+        ((rows == 4 && out_dim >= 11008) || (rows == 3 && out_dim > 14336)) && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim))
+        return true;
     // Two to four rows on a K beyond 4096, against the kernel that shares K out over workgroups and its reduce launch
     // (us, that kernel first): Q4_0 four rows 6144 x 4096 columns 9.9 / 8.4, 8192 x 8192 12.5 / 11.3, 14336 x 4096
     // 12.7 / 11.7, 14336 x 8192 21.0 / 16.5; three rows 6144 x 2048 8.6 / 6.7, 8192 x 4096 8.9 / 9.0, 14336 x 8192

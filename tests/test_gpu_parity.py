@@ -149,6 +149,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (5, 8192, 7168),  # ... 56 columns with two K shares (Q4_0)
     # three and four rows on more columns than one round of the decode kernel's workgroups: Q4_0 takes the eight-row kernel
     (4, 256, 16448), (3, 256, 33000), (4, 4096, 28672),
+    (3, 2048, 14400), (4, 2048, 11040),  # ... and Q8_0 on wide matrices with K of 2048 to 4096
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
