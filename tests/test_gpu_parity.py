@@ -154,6 +154,9 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # wavefront with half its blocks, K shares with a short last share
     (9, 512, 12290), (16, 4096, 12288), (17, 256, 12300), (24, 1024, 12352), (32, 512, 12290), (29, 9216, 12288),
     (33, 1024, 12352), (48, 512, 12290), (64, 4096, 12288),  # ... and two row tiles
+    # ... on fewer columns, where the K shares fill the grid: four shares and the reduce launch, two shares adding to
+    # the result themselves with a ragged last tile (Q4_0), two shares of Q8_0
+    (16, 14336, 4096), (12, 8192, 8190), (20, 4096, 8192),
 ]
 
 
