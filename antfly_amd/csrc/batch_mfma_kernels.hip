@@ -1227,17 +1227,19 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
     const int real_shares = (kb + share_blocks - 1) / share_blocks;
     // Nine to 64 rows (rows of whole 16-byte runs of scales) where the 64-column tiles times the K shares (times two
-    // for a pair) make a grid of three quarters of the compute units up to all of them: batch32_mfma_kernel holds one
+    // for a pair) make a grid of five eighths of the compute units up to all of them: batch32_mfma_kernel holds one
     // workgroup per unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
     // unit (N = 20480: 21.1 against 18.5 us).  The grid counts, not the width: a long K on few columns qualifies through
     // its shares (sixteen rows, against batch_mfma_kernel: Q4_0 K = 14336 x 4096 columns 17.9 -> 17.0 us, 64 rows
     // 31.8 -> 27.6, K = N = 8192 15.7 -> 14.0, K = 8192 x 6144 columns 14.3 -> 13.0; Q8_0 K = 4096 x 8192 columns
-    // 12.7 -> 11.1, K = 8192 x 4096 columns 15.4 -> 14.4).  set_batch32_max_workgroups overrides the bound (tests
+    // 12.7 -> 11.1, K = 8192 x 4096 columns 15.4 -> 14.4).  Below: 160 and 172 workgroups (K = 4096, 10240 and 11008
+    // columns) 13.8 -> 12.7 and 13.9 -> 12.8, Q8_0 160 (5120 columns) 11.0 -> 9.9; 128 workgroups lose (8192 columns
+    // 10.6 -> 12.5).  set_batch32_max_workgroups overrides the bound (tests
     // reach the kernel's K shares and pair launches that way; 0 switches the kernel off).
     const long bound_set = batch32_bound.load(std::memory_order_relaxed);
     const long bound = bound_set >= 0 ? bound_set : gemv_compute_units();
     const long groups32 = static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1);
-    const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && groups32 >= gemv_compute_units() * 3 / 4 && groups32 <= bound;
+    const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && groups32 >= gemv_compute_units() * 5 / 8 && groups32 <= bound;
     // Two K shares and nothing to do to the sums but add them: the kernel's shares add to the result themselves
     // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
     const bool accumulate = real_shares == 2 && both_plain;

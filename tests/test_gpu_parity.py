@@ -156,7 +156,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (33, 1024, 12352), (48, 512, 12290), (64, 4096, 12288),  # ... and two row tiles
     # ... on fewer columns, where the K shares fill the grid: four shares and the reduce launch, two shares adding to
     # the result themselves with a ragged last tile (Q4_0), two shares of Q8_0
-    (16, 14336, 4096), (12, 8192, 8190), (20, 4096, 8192),
+    (16, 14336, 4096), (12, 8192, 8190), (20, 4096, 8192), (17, 512, 10250),
 ]
 
 
