@@ -416,7 +416,13 @@ __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* _
                                                                    float* __restrict__ zero_a, float* __restrict__ zero_b, int zero_count) {
     const int kb = in_dim >> 5, slots = ((kb + 1) >> 1) * 2;  // block slots: whole pairs
     const int units = 8 * slots * 8;                           // (row, block slot, eight lanes)
-    if (zero_a != nullptr) {
+    // blockIdx.y: the group of eight rows (rows 8 .. 15 of X make a second set of fragments and scales behind the first)
+    const int group = blockIdx.y;
+    x += static_cast<size_t>(group) * 8 * in_dim;
+    rows -= 8 * group;
+    qa8 += static_cast<size_t>(group) * (slots / 2) * 128;
+    sa8 += static_cast<size_t>(group) * (slots / 2) * 16;
+    if (zero_a != nullptr && group == 0) {
         for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < zero_count; i += gridDim.x * blockDim.x) {
             zero_a[i] = 0.0f;
             if (zero_b != nullptr) zero_b[i] = 0.0f;
@@ -452,8 +458,10 @@ __global__ __launch_bounds__(256) void quantize_fragments8_kernel(const float* _
 // kHalves: stage rounds of a wavefront -- it owns kHalves runs of eight (Q4_0; four Q8_0) consecutive blocks, and a K share
 // is 8 * kHalves of them: a longer K makes fewer shares (K = 14336 of Q4_0: two of 224 blocks at kHalves = 4 instead of
 // four of 112), and two shares need no reduce launch.
-template <int kType, int kCG, bool kStamps = false, bool kFullCols = false, int kHalves = 2>
-__global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
+// kGroups: groups of eight rows (one or two: nine to sixteen rows run every step's two MFMAs once per group on the same
+// weight operand; the second group's fragments and row scales lie behind the first's).
+template <int kType, int kCG, bool kStamps = false, bool kFullCols = false, int kHalves = 2, int kGroups = 1>
+__global__ __launch_bounds__(kBmThreads, kGroups > 1 ? 2 : 4) void batch8_mfma_kernel(float* __restrict__ dst_a, float* __restrict__ partial_a,
                                                                      const uint32_t* __restrict__ qa8, const float* __restrict__ sa8,
                                                                      const uint8_t* __restrict__ weight_a, int rows, int in_dim, int out_dim,
                                                                      int share_blocks, int cols_arg, int accumulate, Epilogue ep_a, BmSecond second) {
@@ -529,8 +537,8 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     // (Inline assembly: the compiler may move its own loads from read-only memory across the barrier; waited for by
     // hand before the first stage is used.)
     constexpr int kScaleLoads = (kPairs + 3) / 4;
-    float sx_part[kScaleLoads];
-    bm_v4i packed[kPairs / 2];
+    float sx_part[kGroups][kScaleLoads];
+    bm_v4i packed[kGroups][kPairs / 2];
     {
         uint32_t frag_off[kPairs / 2], scale_off[kScaleLoads];
 #pragma unroll
@@ -543,9 +551,14 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         for (int q = 0; q < kScaleLoads; ++q) asm volatile("" : "+v"(scale_off[q]));
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int q = 0; q < kPairs / 2; ++q) asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(packed[q]) : "v"(frag_off[q]), "s"(qa8) : "memory");
+        for (int grp = 0; grp < kGroups; ++grp) {
+            const uint32_t* qa_g = qa8 + static_cast<size_t>(grp) * pairs_total * 128;
+            const float* sa_g = sa8 + static_cast<size_t>(grp) * pairs_total * 16;
 #pragma unroll
-        for (int q = 0; q < kScaleLoads; ++q) asm volatile("global_load_dword %0, %1, %2" : "=v"(sx_part[q]) : "v"(scale_off[q]), "s"(sa8) : "memory");
+            for (int q = 0; q < kPairs / 2; ++q) asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(packed[grp][q]) : "v"(frag_off[q]), "s"(qa_g) : "memory");
+#pragma unroll
+            for (int q = 0; q < kScaleLoads; ++q) asm volatile("global_load_dword %0, %1, %2" : "=v"(sx_part[grp][q]) : "v"(scale_off[q]), "s"(sa_g) : "memory");
+        }
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
@@ -647,11 +660,13 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         baddr[q] = lds_wave + (unit * 64 + row + (chunk ^ swz)) * 16 + (kType == 2 ? 8 * kh : 0);
     }
 
-    float acc[kCG][4];
+    float acc[kGroups][kCG][4];
 #pragma unroll
-    for (int cg = 0; cg < kCG; ++cg)
+    for (int grp = 0; grp < kGroups; ++grp)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) acc[cg][v] = 0.0f;
+        for (int cg = 0; cg < kCG; ++cg)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) acc[grp][cg][v] = 0.0f;
 
     // ---- 2. the stages, software-pipelined by hand over the steps (one step = a pair of blocks,
     // sixteen columns: one int8 MFMA and one scale-product MFMA).  A step's weight bytes are
@@ -666,16 +681,19 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
         typedef float bm_v4f __attribute__((ext_vector_type(4)));
         typedef __attribute__((address_space(3))) const Raw LdsRaw;
         Raw raw[2];
-        bm_v4i afrag[kHalfPairs];
-        float sxm[kHalfPairs], tbm[kHalfPairs];
-        bm_v4i cres[2];
-        bm_v4f tres[2];
+        bm_v4i afrag[kGroups][kHalfPairs];
+        float sxm[kGroups][kHalfPairs], tbm[kHalfPairs];
+        bm_v4i cres[kGroups][2];
+        bm_v4f tres[kGroups][2];
         auto stage_of = [&](int it) { return it / kHalfPairs; };
         auto fetch_weights = [&](int it) { raw[it & 1] = *reinterpret_cast<LdsRaw*>(baddr[it % kHalfPairs] + (stage_of(it) & 3) * 2048); };
         auto scale = [&](int it) {
             const int cg = stage_of(it) % kCG;
 #pragma unroll
-            for (int v = 0; v < 4; ++v) acc[cg][v] = __builtin_fmaf(tres[it & 1][v], static_cast<float>(cres[it & 1][v]), acc[cg][v]);
+            for (int grp = 0; grp < kGroups; ++grp)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    acc[grp][cg][v] = __builtin_fmaf(tres[grp][it & 1][v], static_cast<float>(cres[grp][it & 1][v]), acc[grp][cg][v]);
         };
 #pragma unroll
         for (int it = 0; it < kSteps; ++it) {
@@ -685,10 +703,16 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
                     if (kStartupAlone) asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
                     else asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * (kAheadStages - 1)) : "memory");
 #pragma unroll
-                    for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(packed[q]));
+                    for (int grp = 0; grp < kGroups; ++grp) {
 #pragma unroll
-                    for (int c = 0; c < (kScalesInLds ? 0 : kCG); ++c) asm volatile("" : "+v"(tb_part[c][0]), "+v"(tb_part[c][kWpl - 1]));
-                    asm volatile("" : "+v"(sx_part[0]), "+v"(sx_part[kScaleLoads - 1]));
+                        for (int q = 0; q < kPairs / 2; ++q) asm volatile("" : "+v"(packed[grp][q]));
+#pragma unroll
+                        for (int q = 0; q < kScaleLoads; ++q) asm volatile("" : "+v"(sx_part[grp][q]));  // (one operand a statement: never the same register twice)
+                    }
+#pragma unroll
+                    for (int c = 0; c < (kScalesInLds ? 0 : kCG); ++c)
+#pragma unroll
+                        for (int q = 0; q < kWpl; ++q) asm volatile("" : "+v"(tb_part[c][q]));
                 }
                 if (kStartupAlone && st == 0) {
 #pragma unroll
@@ -718,17 +742,19 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
                     // entry 8 g + i % 8 of its pair through the lane exchange if the slot's block is the lane
                     // group's, else zeros
 #pragma unroll
-                    for (int q = 0; q < kHalfPairs; ++q) {
-                        const int p = hb * kHalfPairs + q;
-                        const float sx = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (16 * (p & 3) + l16), __float_as_int(sx_part[p >> 2])));
-                        sxm[q] = g == (l16 >> 3) ? sx : 0.0f;
-                        const int from = 4 * (32 * (p & 1) + 8 * g + (l16 & 7));
+                    for (int grp = 0; grp < kGroups; ++grp)
 #pragma unroll
-                        for (int d = 0; d < 4; ++d) {
-                            const int got = __builtin_amdgcn_ds_bpermute(from, packed[p >> 1][d]);
-                            afrag[q][d] = (l16 >> 3) == par ? got : 0;
+                        for (int q = 0; q < kHalfPairs; ++q) {
+                            const int p = hb * kHalfPairs + q;
+                            const float sx = __int_as_float(__builtin_amdgcn_ds_bpermute(4 * (16 * (p & 3) + l16), __float_as_int(sx_part[grp][p >> 2])));
+                            sxm[grp][q] = g == (l16 >> 3) ? sx : 0.0f;
+                            const int from = 4 * (32 * (p & 1) + 8 * g + (l16 & 7));
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) {
+                                const int got = __builtin_amdgcn_ds_bpermute(from, packed[grp][p >> 1][d]);
+                                afrag[grp][q][d] = (l16 >> 3) == par ? got : 0;
+                            }
                         }
-                    }
                 }
                 // this stage is there when at most the stages requested behind it are in flight
                 {
@@ -757,8 +783,11 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
             }
             __builtin_amdgcn_sched_barrier(0);
             const int q = it % kHalfPairs;
-            cres[it & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[q], b, bm_v4i{0, 0, 0, 0}, 0, 0, 0);
-            tres[it & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(sxm[q], tbm[q], bm_v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+#pragma unroll
+            for (int grp = 0; grp < kGroups; ++grp) {
+                cres[grp][it & 1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(afrag[grp][q], b, bm_v4i{0, 0, 0, 0}, 0, 0, 0);
+                tres[grp][it & 1] = __builtin_amdgcn_mfma_f32_16x16x4f32(sxm[grp][q], tbm[q], bm_v4f{0.0f, 0.0f, 0.0f, 0.0f}, 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
             if (it > 0) scale(it - 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -771,28 +800,31 @@ __global__ __launch_bounds__(kBmThreads, 4) void batch8_mfma_kernel(float* __res
     asm volatile("" : : "v"(spare[0]), "v"(spare[1]));
 
     // ---- 3. the wavefronts' sums (and the two block parities) meet in LDS
-    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][cg * 4 + v][lane]
-    __syncthreads();
+    float* red = reinterpret_cast<float*>(bm_lds);  // [wave][cg * 4 + v][lane], one group of rows at a time
 #pragma unroll
-    for (int cg = 0; cg < kCG; ++cg)
+    for (int grp = 0; grp < kGroups; ++grp) {
+        __syncthreads();
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[(wave * kCG * 4 + cg * 4 + v) * 64 + lane] = acc[cg][v];
-    __syncthreads();
-    if (tid < 8 * kCols) {
-        const int m = tid / kCols, c = tid % kCols;
-        const int item = ((c >> 4) * 4 + (m & 3)) * 64 + 16 * (m >> 2) + (c & 15);
-        float sum = 0.0f;
+        for (int cg = 0; cg < kCG; ++cg)
 #pragma unroll
-        for (int w = 0; w < kBmWaves; ++w) sum += red[w * kCG * 256 + item] + red[w * kCG * 256 + item + 32];
-        const int n = n0 + c;
-        if (kStamps) {
-            asm volatile("" : : "v"(sum));  // (keeps the arithmetic alive)
-        } else if (m < rows && c < cols && n < out_dim) {
-            const size_t at = static_cast<size_t>(m) * out_dim + n;
-            if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
-            // two K shares, no epilogue: both add to the zeroed result; 0 + a + b = 0 + b + a to the bit, whoever comes first
-            else if (accumulate) unsafeAtomicAdd(dst + at, sum);
-            else dst[at] = finish_output(ep, n, at, sum);
+            for (int v = 0; v < 4; ++v) red[(wave * kCG * 4 + cg * 4 + v) * 64 + lane] = acc[grp][cg][v];
+        __syncthreads();
+        if (tid < 8 * kCols) {
+            const int m8 = tid / kCols, c = tid % kCols, m = 8 * grp + m8;
+            const int item = ((c >> 4) * 4 + (m8 & 3)) * 64 + 16 * (m8 >> 2) + (c & 15);
+            float sum = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kBmWaves; ++w) sum += red[w * kCG * 256 + item] + red[w * kCG * 256 + item + 32];
+            const int n = n0 + c;
+            if (kStamps) {
+                asm volatile("" : : "v"(sum));  // (keeps the arithmetic alive)
+            } else if (m < rows && c < cols && n < out_dim) {
+                const size_t at = static_cast<size_t>(m) * out_dim + n;
+                if (partial != nullptr) partial[static_cast<size_t>(blockIdx.y) * rows * out_dim + at] = sum;
+                // two K shares, no epilogue: both add to the zeroed result; 0 + a + b = 0 + b + a to the bit, whoever comes first
+                else if (accumulate) unsafeAtomicAdd(dst + at, sum);
+                else dst[at] = finish_output(ep, n, at, sum);
+            }
         }
     }
     if (kStamps) {
@@ -1073,7 +1105,7 @@ static hipError_t bm_allow_large_lds(Kernel kernel, size_t lds, std::atomic<size
     return e;
 }
 
-template <int kType, int kCG, int kHalves>
+template <int kType, int kCG, int kHalves, int kGroups>
 hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint32_t* qa, const float* sa, const uint8_t* weight, int rows,
                       int in_dim, int out_dim, int shares, int share_blocks, int cols, bool accumulate, const Epilogue& ep, const BmSecond& second) {
     const dim3 grid(static_cast<unsigned>((out_dim + cols - 1) / cols), static_cast<unsigned>(shares), second.weight ? 2u : 1u), block(kBmThreads);
@@ -1081,12 +1113,12 @@ hipError_t bm_launch8(hipStream_t stream, float* dst, float* partial, const uint
     const size_t lds = bm8_lds_bytes(kType, kCG, kHalves);
     static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
     if (cols == 16 * kCG) {
-        auto kernel = batch8_mfma_kernel<kType, kCG, false, true, kHalves>;
+        auto kernel = batch8_mfma_kernel<kType, kCG, false, true, kHalves, kGroups>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[0]); e != hipSuccess) return e;
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
                            accumulate ? 1 : 0, ep, second);
     } else {
-        auto kernel = batch8_mfma_kernel<kType, kCG, false, false, kHalves>;
+        auto kernel = batch8_mfma_kernel<kType, kCG, false, false, kHalves, kGroups>;
         if (hipError_t e = bm_allow_large_lds(kernel, lds, &lds_limit[1]); e != hipSuccess) return e;
         hipLaunchKernelGGL(kernel, grid, block, lds, stream, dst, partial, qa, sa, weight, rows, in_dim, out_dim, share_blocks, cols,
                            accumulate ? 1 : 0, ep, second);
@@ -1185,13 +1217,20 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
     return true;
 }
 
-// The eight-row kernel: at most eight rows and rows of whole 16-byte runs of weight scales.  (It used to be kept to grids
+// The eight-row kernel: at most eight rows -- Q8_0 sixteen, as two groups of eight -- and rows of whole 16-byte runs of
+// weight scales.  Nine and sixteen rows against the 32-row kernels (us): Q8_0 K = 4096 x 14336 columns 18.7 -> 15.4,
+// 28672 columns 34.7 -> 26.4, K = 14336 x 4096 21.0 -> 16.1, K = N = 8192 23.5 -> 17.1, a pair of 14336 columns
+// 35.0 -> 27.1, 4096 x 4096 8.7 -> 8.9, K = 2048 x 8192 columns 8.3 -> 8.8.  Q4_0, whose 32-row kernels are better (half
+// the bytes per block, the same MFMA time), loses with two groups -- 14336 columns 13.3 -> 14.6, K = N = 8192
+// 13.8 -> 14.7, 128256 columns 74 -> 84; 4096 columns 9.8 -> 9.2 and K = 14336 x 4096 16.8 -> 15.8 are the only gains --
+// and keeps one: a step's MFMAs of two groups (2 x (16 + 32) cycles a SIMD) take as long as its bytes.
+// (It used to be kept to grids
 // of at least a workgroup per compute unit; with its tiles sized to the matrix and its first requests in order it also
 // wins below that: five rows, K = 4096, against batch_mfma_kernel: 6144 columns 8.5 against 9.6 us, 3072 6.8 against
 // 9.0, 1024 6.6 against 8.7.)
 bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
-    return rows <= 8 && (in_dim / 32) % 8 == 0;
+    return rows <= (tensor_type == 8 ? 16 : 8) && (in_dim / 32) % 8 == 0;
 }
 
 // Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares, for two matrices]
@@ -1243,11 +1282,12 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     // Two K shares and nothing to do to the sums but add them: the kernel's shares add to the result themselves
     // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
     const bool accumulate = real_shares == 2 && both_plain;
-    if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks, inside the same region
+    const int groups = rows > 8 ? 2 : 1;  // (eight-row kernel) groups of eight rows
+    if (eight) {  // its own operand layout: 512 + 64 bytes per pair of blocks and group of eight rows, inside the same region
         const int pairs = (kb + 1) / 2;
-        sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(pairs) * 512);
+        sa = reinterpret_cast<float*>(workspace + static_cast<size_t>(groups) * pairs * 512);
         const int units = 8 * (2 * pairs) * 8;
-        const dim3 qgrid(static_cast<unsigned>((units + 255) / 256));
+        const dim3 qgrid(static_cast<unsigned>((units + 255) / 256), static_cast<unsigned>(groups));
         float* zero_a = accumulate ? dst : nullptr;
         float* zero_b = accumulate && weight_b_prepared ? dst_b : nullptr;
         const int zero_count = rows * out_dim;
@@ -1279,10 +1319,12 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     hipError_t e;
     if (eight) {
         const int cols = bm8_columns(real_shares, out_dim, weight_b_prepared != nullptr), cg = (cols + 15) / 16;
-#define AFHIP_BM8(T, CG, H) bm_launch8<T, CG, H>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
-#define AFHIP_BM8_CG(T, H) (cg == 4 ? AFHIP_BM8(T, 4, H) : (cg == 3 ? AFHIP_BM8(T, 3, H) : (cg == 2 ? AFHIP_BM8(T, 2, H) : AFHIP_BM8(T, 1, H))))
-        if (tensor_type == 2) e = halves == 4 ? AFHIP_BM8_CG(2, 4) : AFHIP_BM8_CG(2, 2);
-        else e = halves == 8 ? AFHIP_BM8_CG(8, 8) : (halves == 4 ? AFHIP_BM8_CG(8, 4) : AFHIP_BM8_CG(8, 2));
+#define AFHIP_BM8(T, CG, H, G) bm_launch8<T, CG, H, G>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
+#define AFHIP_BM8_CG(T, H, G) (cg == 4 ? AFHIP_BM8(T, 4, H, G) : (cg == 3 ? AFHIP_BM8(T, 3, H, G) : (cg == 2 ? AFHIP_BM8(T, 2, H, G) : AFHIP_BM8(T, 1, H, G))))
+#define AFHIP_BM8_G(T, H) (groups == 2 ? AFHIP_BM8_CG(T, H, 2) : AFHIP_BM8_CG(T, H, 1))
+        if (tensor_type == 2) e = halves == 4 ? AFHIP_BM8_CG(2, 4, 1) : AFHIP_BM8_CG(2, 2, 1);  // (Q4_0: one group of rows only)
+        else e = halves == 8 ? AFHIP_BM8_G(8, 8) : (halves == 4 ? AFHIP_BM8_G(8, 4) : AFHIP_BM8_G(8, 2));
+#undef AFHIP_BM8_G
 #undef AFHIP_BM8_CG
 #undef AFHIP_BM8
     }

@@ -388,7 +388,8 @@ __device__ __forceinline__ void gemv_fused_body(
     }
 
     if (kProbe & kProbeTimeline) {
-        asm volatile("" : "+v"(acc[0][0]), "+v"(acc[kRows - 1][kCols - 1]));
+        asm volatile("" : "+v"(acc[0][0]));
+        if (kRows * kCols > 1) asm volatile("" : "+v"(acc[kRows - 1][kCols - 1]));  // (never the same register twice in one statement)
         stamp[2] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
     }
     // ---- 4. wavefront reduction (all rows x columns at once)
