@@ -240,8 +240,12 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
     static const int env_no_planes = env_int("AFHIP_Q4K_NO_DIGIT_PLANES");
     if (tiled && env_no_planes == 0 && q4k_i8_rows_supports(rows, in_dim) && workspace.ptr != 0 && workspace.ptr % 16 == 0 &&
         workspace.len >= q4k_i8_rows_workspace_bytes(in_dim)) {
+        // (few column tiles: two workgroups a tile with half of K each add to the results, which the planes' launch clears)
+        const bool two_shares = q4k_i8_rows_two_shares(rows, in_dim, out_dim, pair, ep, ep_b);
         hipError_t e = launch_q4k_digit_planes(stream, reinterpret_cast<const float*>(input.ptr), static_cast<int>(rows),
-                                               static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr));
+                                               static_cast<int>(in_dim), reinterpret_cast<void*>(workspace.ptr),
+                                               two_shares ? reinterpret_cast<float*>(dst.ptr) : nullptr,
+                                               two_shares && pair ? reinterpret_cast<float*>(dst_b.ptr) : nullptr, rows * out_dim);
         if (counters) {
             for (int i = 0; i < (pair ? 2 : 1); ++i) {
                 if (kind == AFHIP_DISPATCH_MMV) counters->mmv++;
@@ -253,7 +257,7 @@ static afhip_status linear_q4k_impl(hipStream_t stream, int layout, afhip_buffer
             e = launch_gemv_q4k_i8_rows(stream, reinterpret_cast<float*>(dst.ptr), reinterpret_cast<const void*>(workspace.ptr),
                                         reinterpret_cast<const uint8_t*>(weight.ptr), static_cast<int>(rows), static_cast<int>(in_dim),
                                         static_cast<int>(out_dim), ep, pair ? reinterpret_cast<float*>(dst_b.ptr) : nullptr,
-                                        pair ? reinterpret_cast<const uint8_t*>(weight_b.ptr) : nullptr, ep_b);
+                                        pair ? reinterpret_cast<const uint8_t*>(weight_b.ptr) : nullptr, ep_b, two_shares);
         return e == hipSuccess ? AFHIP_OK : static_cast<afhip_status>(e);
     }
     // more rows than one GEMV launch holds: X split once into the caller's scratch, then the

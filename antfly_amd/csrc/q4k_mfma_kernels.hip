@@ -440,9 +440,18 @@ __device__ __forceinline__ Q4kDigits q4k_digit_planes(const float4 v) {
 // operand order -- 1 KB per (super-block, sub-block): lane (MFMA row c = 4 * row + digit, half g) holds
 // its 16 bytes (K = 16 g .. 16 g + 15 of the sub-block) at 16 * (32 g + c) -- so a wavefront's operand is
 // one contiguous load; then -s per (row, super-block) and the sub-block sums.  One wavefront per item.
+// zero_a (and zero_b): result arrays of zero_count floats that the matmul launch behind this one adds its two K shares'
+// sums to; cleared here, by the launch that has to run first anyway.
 __global__ __launch_bounds__(256) void q4k_digit_planes_kernel(const float* __restrict__ x, int rows, int in_dim,
                                                                uint8_t* __restrict__ frag, float* __restrict__ minus_s,
-                                                               float* __restrict__ sub_sums) {
+                                                               float* __restrict__ sub_sums, float* __restrict__ zero_a,
+                                                               float* __restrict__ zero_b, int zero_count) {
+    if (zero_a != nullptr) {
+        for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < zero_count; i += gridDim.x * blockDim.x) {
+            zero_a[i] = 0.0f;
+            if (zero_b != nullptr) zero_b[i] = 0.0f;
+        }
+    }
     const int kb = in_dim >> 8, lane = threadIdx.x & 63;
     const int item = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (item >= rows * kb) return;
@@ -456,11 +465,22 @@ __global__ __launch_bounds__(256) void q4k_digit_planes_kernel(const float* __re
     if (lane == 0) minus_s[r * kb + sb] = dg.minus_s;
 }
 
+// Clears result arrays ahead of a launch whose two K shares add to them (one or two rows: no launch of its own precedes).
+__global__ __launch_bounds__(256) void q4k_zero_results_kernel(float* __restrict__ a, float* __restrict__ b, int count) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < count; i += gridDim.x * blockDim.x) {
+        a[i] = 0.0f;
+        if (b != nullptr) b[i] = 0.0f;
+    }
+}
+
 // kGroups = ceil(rows / 2) row groups: row r sits in lane half r % 2, D registers 4 (r / 2) + digit.
 // kPlanesGiven: the digit planes, -s and the sub-block sums come from q4k_digit_planes_kernel (`frag`, `frag_scale`,
 // `frag_sums`) instead of being made here from `x`: the MFMA operand is then a 16-byte load per lane and sub-block,
 // requested with the weights, and nothing of X passes through LDS but the few floats of the wavefront's own slice.
 // A second matrix of the same shape on the same X (gate and up: grid.y = 2): one launch for both.
+// K shares (grid.z = 2, `accumulate`): a matrix with so few column tiles that half the compute units would stay idle
+// gives each tile to two workgroups, each with half of K; both add their sums to the result array, cleared beforehand,
+// with a float atomic -- two addends on a zero give the same float in either order.  No epilogue then.
 struct Q4kSecond {
     float* dst;
     const uint8_t* weight;
@@ -472,7 +492,7 @@ __global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 
                                                                   const uint8_t* __restrict__ weight_a, int rows, int in_dim,
                                                                   int out_dim, int slices, int sb_per_slice, Epilogue ep_a,
                                                                   const uint8_t* __restrict__ frag, const float* __restrict__ frag_scale,
-                                                                  const float* __restrict__ frag_sums, Q4kSecond second) {
+                                                                  const float* __restrict__ frag_sums, Q4kSecond second, int accumulate) {
     const bool is_b = blockIdx.y != 0;
     float* dst = is_b ? second.dst : dst_a;
     const uint8_t* weight = is_b ? second.weight : weight_a;
@@ -489,7 +509,7 @@ __global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 
 
     const int n_tiles = (out_dim + kTileCols - 1) >> 5;
     const int tile = blockIdx.x < static_cast<unsigned>(n_tiles) ? blockIdx.x : n_tiles - 1;
-    const int slice = wave;  // one tile per workgroup: blockDim.x = 64 * slices
+    const int slice = static_cast<int>(blockIdx.z) * slices + wave;  // one tile per workgroup and K share: blockDim.x = 64 * slices
     const int sb_begin = slice * sb_per_slice;
     const int sb_end = min(kb, sb_begin + sb_per_slice);
     const uint8_t* tile_base = weight + static_cast<size_t>(tile) * kb * kTileBytes;
@@ -661,7 +681,8 @@ __global__ __launch_bounds__(kMaxThreads, kMaxThreads == 1024 && kFlight == 1 ? 
         const int o = static_cast<int>(blockIdx.x) * kTileCols + (ln & 31);
         if (row < rows && o < out_dim) {
             const size_t idx = static_cast<size_t>(row) * out_dim + o;
-            dst[idx] = finish_output(ep, o, idx, total);
+            if (accumulate) unsafeAtomicAdd(dst + idx, total);
+            else dst[idx] = finish_output(ep, o, idx, total);
         }
     }
 }
@@ -971,7 +992,14 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     while (slices > kb) slices /= 2;
     static const int env_slices = tuning_int("AFHIP_Q4K_SLICES"), env_tiles = tuning_int("AFHIP_Q4K_TILES_PER_WG");
     if (env_slices >= 1 && env_slices <= max_waves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
-    const int sb_per_slice = (kb + slices - 1) / slices;
+    // The int8 kernel at one or two rows on a matrix whose column tiles (of both matrices of a pair) occupy at most half
+    // the compute units, K long enough for a super-block per wavefront of two workgroups, no epilogue: two K shares
+    // (K = 14336 x 4096 columns: 128 tiles, one row 12.7 us on half the chip).
+    auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
+    const bool two_shares = kGroups == 1 && use_i8 && env_slices == 0 && slices == 16 && kb >= 32 && plain(ep) &&
+                            (second == nullptr || plain(second->ep)) &&
+                            2 * n_tiles * (second ? 2 : 1) <= gemv_compute_units();
+    const int sb_per_slice = (kb + (two_shares ? 2 : 1) * slices - 1) / ((two_shares ? 2 : 1) * slices);
     int tiles_per_wg = use_i8 ? 1 : (slices > 8 ? 16 : 8) / slices;  // (the int8 kernel: its wavefronts partition K, nothing else)
     if (!use_i8 && env_tiles >= 1 && env_tiles * slices <= max_waves) tiles_per_wg = env_tiles;
     const int waves = slices * tiles_per_wg;
@@ -985,7 +1013,7 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     if constexpr (kGroups <= 2) {
         if (use_i8) {
             if (tiles_per_wg != 1) return hipErrorInvalidValue;  // (a tuning knob asked for a shape this kernel does not have)
-            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue, const uint8_t*, const float*, const float*, Q4kSecond) = nullptr;
+            void (*k8)(float*, const float*, const uint8_t*, int, int, int, int, int, Epilogue, const uint8_t*, const float*, const float*, Q4kSecond, int) = nullptr;
             if constexpr (kGroups == 1) {
                 switch (variant) {
                     case 0:
@@ -1006,9 +1034,15 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
                     return e;
                 large_lds8[variant] = true;
             }
-            hipLaunchKernelGGL(k8, dim3(grid, second ? 2 : 1), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim, out_dim, slices,
-                               sb_per_slice, ep, static_cast<const uint8_t*>(nullptr), static_cast<const float*>(nullptr),
-                               static_cast<const float*>(nullptr), second ? *second : Q4kSecond{nullptr, nullptr, Epilogue{}});
+            if (two_shares) {
+                const int count = rows * out_dim;
+                hipLaunchKernelGGL(q4k_zero_results_kernel, dim3((count + 1023) / 1024), dim3(256), 0, stream, dst,
+                                   second ? second->dst : static_cast<float*>(nullptr), count);
+                if (hipError_t e = hipGetLastError(); e != hipSuccess) return e;
+            }
+            hipLaunchKernelGGL(k8, dim3(grid, second ? 2 : 1, two_shares ? 2 : 1), dim3(waves * 64), lds8, stream, dst, x, weight, rows, in_dim,
+                               out_dim, slices, sb_per_slice, ep, static_cast<const uint8_t*>(nullptr), static_cast<const float*>(nullptr),
+                               static_cast<const float*>(nullptr), second ? *second : Q4kSecond{nullptr, nullptr, Epilogue{}}, two_shares ? 1 : 0);
             return hipGetLastError();
         }
     }
@@ -1174,19 +1208,32 @@ size_t q4k_i8_rows_workspace_bytes(size_t in_dim) {
     return kb * 8192 + kb * 8 * 4 + kb * 8 * 8 * 4;
 }
 
-hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace) {
+// Whether launch_gemv_q4k_i8_rows shares K out over two workgroups per column tile, which add to the result arrays: then
+// launch_q4k_digit_planes has to clear them.  Column tiles (of both matrices of a pair) that occupy at most half of the
+// two workgroups a compute unit holds, a super-block per wavefront of both shares, no epilogue.
+bool q4k_i8_rows_two_shares(size_t rows, size_t in_dim, size_t out_dim, bool pair, const Epilogue& ep, const Epilogue& ep_b) {
+    auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
+    if (!q4k_i8_rows_supports(rows, in_dim) || !plain(ep) || (pair && !plain(ep_b))) return false;
+    const size_t n_tiles = (out_dim + kTileCols - 1) / kTileCols;
+    return in_dim / kQ4kBlockValues >= 16 && n_tiles * (pair ? 2 : 1) <= static_cast<size_t>(gemv_compute_units());
+}
+
+hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace, float* zero_a,
+                                   float* zero_b, size_t zero_count) {
     if (!q4k_i8_rows_supports(static_cast<size_t>(rows), static_cast<size_t>(in_dim)) || workspace == nullptr) return hipErrorInvalidValue;
     const int kb = in_dim / kQ4kBlockValues;
     uint8_t* frag = static_cast<uint8_t*>(workspace);
     float* minus_s = reinterpret_cast<float*>(frag + static_cast<size_t>(kb) * 8192);
     float* sums = minus_s + static_cast<size_t>(kb) * 8;
     const int items = rows * kb;
-    hipLaunchKernelGGL(q4k_digit_planes_kernel, dim3((items + 3) / 4), dim3(256), 0, stream, x, rows, in_dim, frag, minus_s, sums);
+    hipLaunchKernelGGL(q4k_digit_planes_kernel, dim3((items + 3) / 4), dim3(256), 0, stream, x, rows, in_dim, frag, minus_s, sums, zero_a,
+                       zero_b, static_cast<int>(zero_count));
     return hipGetLastError();
 }
 
 hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, int rows, int in_dim,
-                                   int out_dim, const Epilogue& ep, float* dst_b, const uint8_t* weight_b, const Epilogue& ep_b) {
+                                   int out_dim, const Epilogue& ep, float* dst_b, const uint8_t* weight_b, const Epilogue& ep_b,
+                                   bool results_cleared) {
     if (!q4k_i8_rows_supports(static_cast<size_t>(rows), static_cast<size_t>(in_dim)) || workspace == nullptr) return hipErrorInvalidValue;
     if (out_dim == 0) return hipSuccess;
     const int kb = in_dim / kQ4kBlockValues;
@@ -1195,24 +1242,28 @@ hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* w
     const float* sums = minus_s + static_cast<size_t>(kb) * 8;
     int slices = 8;
     while (slices > kb) slices /= 2;
-    const int sb_per_slice = (kb + slices - 1) / slices;
+    // (two K shares only when the caller had the result arrays cleared by the digit planes' launch)
+    const bool two_shares = results_cleared && q4k_i8_rows_two_shares(static_cast<size_t>(rows), static_cast<size_t>(in_dim),
+                                                                      static_cast<size_t>(out_dim), weight_b != nullptr, ep, ep_b);
+    const int shares = two_shares ? 2 : 1, accumulate = two_shares ? 1 : 0;
+    const int sb_per_slice = (kb + shares * slices - 1) / (shares * slices);
     const int n_tiles = (out_dim + kTileCols - 1) / kTileCols;
     const size_t lds = q4k_i8_rows_lds_bytes(rows, in_dim, slices);
     const float* no_x = nullptr;
     const Q4kSecond second{dst_b, weight_b, ep_b};
-    const dim3 grid(n_tiles, weight_b != nullptr ? 2 : 1);
+    const dim3 grid(n_tiles, weight_b != nullptr ? 2 : 1, shares);
     switch ((rows + 1) / 2) {
         case 2:
             hipLaunchKernelGGL((gemv_q4k_i8_kernel<2, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second, accumulate);
             break;
         case 3:
             hipLaunchKernelGGL((gemv_q4k_i8_kernel<3, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second, accumulate);
             break;
         default:
             hipLaunchKernelGGL((gemv_q4k_i8_kernel<4, 1, 512, true>), grid, dim3(64 * slices), lds, stream, dst, no_x, weight, rows, in_dim,
-                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second);
+                               out_dim, slices, sb_per_slice, ep, frag, minus_s, sums, second, accumulate);
             break;
     }
     return hipGetLastError();

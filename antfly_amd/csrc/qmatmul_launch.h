@@ -184,10 +184,15 @@ hipError_t launch_gemv_q4k_tiled(hipStream_t stream, float* dst, const float* x,
 // launch_gemv_q4k_i8_rows multiplies one matrix, or a pair of them in one launch, by them.
 bool q4k_i8_rows_supports(size_t rows, size_t in_dim);
 size_t q4k_i8_rows_workspace_bytes(size_t in_dim);
-hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace);
+// q4k_i8_rows_two_shares: the matmul launch would give every column tile to two workgroups with half of K each, which add
+// to the result arrays -- the caller then has launch_q4k_digit_planes clear them (zero_a, zero_b, zero_count floats each)
+// and says so to launch_gemv_q4k_i8_rows (results_cleared); otherwise one workgroup per tile, as without.
+bool q4k_i8_rows_two_shares(size_t rows, size_t in_dim, size_t out_dim, bool pair, const Epilogue& ep, const Epilogue& ep_b);
+hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace, float* zero_a = nullptr,
+                                   float* zero_b = nullptr, size_t zero_count = 0);
 hipError_t launch_gemv_q4k_i8_rows(hipStream_t stream, float* dst, const void* workspace, const uint8_t* weight, int rows, int in_dim,
                                    int out_dim, const Epilogue& ep, float* dst_b = nullptr, const uint8_t* weight_b = nullptr,
-                                   const Epilogue& ep_b = Epilogue{});
+                                   const Epilogue& ep_b = Epilogue{}, bool results_cleared = false);
 // More rows than one launch of the kernel above holds (gemv_q4k_tiled_rows_per_launch): X is split
 // once into `workspace` (gemm_q4k_workspace_bytes, 16-byte aligned; it also holds the partial sums when a
 // small problem splits K over several workgroups) and a GEMM walks K for 32 rows

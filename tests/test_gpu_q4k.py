@@ -171,7 +171,9 @@ SHAPES = [(1, 256, 1), (1, 256, 7), (2, 512, 33), (1, 4096, 64), (2, 4096, 130),
 
 TILED_SHAPES = SHAPES + [(1, 1024, 300), (6, 4096, 70), (7, 1024, 257), (8, 2048, 96), (9, 1024, 64), (17, 512, 40),
                         (2, 4096, 1000), (4, 4096, 96), (3, 8192, 200), (4, 1024, 8192), (3, 4096, 8200),
-                        (1, 4096, 14336), (2, 14336, 4096), (1, 4096, 32064)]  # the last three: full FFN and vocabulary-sized matrices
+                        (1, 4096, 14336), (2, 14336, 4096), (1, 4096, 32064),  # these three: full FFN and vocabulary-sized matrices
+                        # few column tiles on a long K: two workgroups a tile, half of K each (a last share with idle wavefronts)
+                        (1, 11008, 100), (2, 8192, 2048), (5, 11008, 260), (8, 4096, 4096)]
 
 
 @pytest.mark.parametrize("layout,rows,in_dim,out_dim", [(RAW, *s) for s in SHAPES] + [(PREP, *s) for s in TILED_SHAPES])
