@@ -107,8 +107,9 @@ static int env_int(const char* name) {
 // AFHIP_BATCH_MFMA_MIN_ROWS overrides the lower row bound for tuning runs, 0 switches the kernel off):
 // from five rows on (six on a K longer than 4096, where the split-K GEMV still wins at five) up to 64
 // (128 on wide Q4_0 matrices), and for Q8_0, whose K shares are half as long, only while all workgroups
-// of the launch are resident at once.  Five to eight rows on a grid that fills the chip always:
-// its eight-row kernel requests weights as it goes and needs neither condition.
+// of the launch are resident at once.  Five to eight rows (Q8_0: sixteen) on a K of whole 256-value runs always:
+// the eight-row kernel requests weights as it goes and needs neither condition.  Two to four rows where measured
+// faster than the decode kernels (the rules below).
 static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, size_t out_dim, bool pair) {
     static const char* v = std::getenv("AFHIP_BATCH_MFMA_MIN_ROWS");
     static const long forced = v && *v ? std::atol(v) : -1;

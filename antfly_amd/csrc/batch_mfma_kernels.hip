@@ -28,12 +28,13 @@
 //   * The eight wavefronts' sums meet in LDS in wavefront order (y is a fixed-order sum of eight
 //     block-ascending partial sums); K shares of a long K go to partial[share][rows][out_dim]
 //     and splitk_reduce_kernel adds them in share order.
-//   * Up to eight rows on a grid that fills the chip take batch8_mfma_kernel (further down): the
-//     16x16x64 MFMA on two blocks at once, tiles of 8 .. 64 columns, weights requested two stages
-//     ahead instead of all at once.
-//   * Nine to 64 rows on a wide matrix whose grid is one round of 64-column tiles take
-//     batch32_mfma_kernel (further down): this kernel's arithmetic, staged weight requests, one
-//     workgroup per compute unit.
+//   * Up to eight rows (Q8_0: sixteen, as two groups of eight) on a K of whole 256-value runs take
+//     batch8_mfma_kernel (further down): the 16x16x64 MFMA on two blocks at once, tiles of 8 .. 64
+//     columns, weights requested two stages ahead instead of all at once, a long K in at most two
+//     shares where that is possible.
+//   * Nine to 64 rows whose 64-column tiles times K shares make a grid of five eighths to all of
+//     the compute units take batch32_mfma_kernel (further down): this kernel's arithmetic, staged
+//     weight requests, one workgroup per compute unit.
 #include <hip/hip_runtime.h>
 
 #include <atomic>

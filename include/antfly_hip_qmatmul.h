@@ -182,8 +182,12 @@ afhip_status afhip_launch_linear_f32_static(void *stream, int tensor_type, int l
 /* Two matmuls of the same shape, format and layout that share X (what the engine's
  * linearNoBiasPair computes for gate + up, ops/ops.zig:909, CPU op
  * ops/native_compute.zig:6262-6307): Ya = X * Wa^T, Yb = X * Wb^T.  Each result is
- * exactly what afhip_launch_linear_f32 gives for that matrix; X is quantized once,
- * and up to 8 rows both matrices are served by one kernel launch. */
+ * bit for bit what afhip_launch_linear_f32 gives for that matrix wherever the pair and the
+ * single call take the same kernel -- everywhere but three and four rows of Q4_0 with
+ * in_dim <= 4096 whose two matrices together exceed one (three rows: two) rounds of the decode
+ * kernel's workgroups while one of them does not: there the same block dots are summed in
+ * another order (equal within the op's tolerance).  X is quantized once, and up to 8 rows
+ * (Q8_0: 16) both matrices are served by one kernel launch. */
 afhip_status afhip_launch_linear_pair_f32(void *stream, int tensor_type, int layout, afhip_buffer dst_a,
                                           afhip_buffer dst_b, afhip_buffer input, afhip_buffer weight_a,
                                           afhip_buffer weight_b, size_t rows, size_t in_dim,
