@@ -359,9 +359,16 @@ __global__ __launch_bounds__(kBmThreads, kRowTiles == 1 ? 4 : 2) void batch_mfma
         for (int v = 0; v < kLive; ++v) red[(wave * kLive + v) * 64 + lane] = acc[rt][v];
         __syncthreads();
         for (int i = tid; i < kItems; i += kBmThreads) {
-            float sum = red[i];
+            // the first four wavefronts' sums, the last four's, then both: what two K shares of four wavefronts each
+            // add up to (launch_batch_mfma splits a single share there where that is faster, to the same bits)
+            float half[2];
 #pragma unroll
-            for (int w = 1; w < kBmWaves; ++w) sum += red[w * kItems + i];
+            for (int h = 0; h < 2; ++h) {
+                half[h] = red[(kBmWaves / 2) * h * kItems + i];
+#pragma unroll
+                for (int w = 1; w < kBmWaves / 2; ++w) half[h] += red[((kBmWaves / 2) * h + w) * kItems + i];
+            }
+            const float sum = half[0] + half[1];
             const int l = i & 63, v = i >> 6;
             const int m = rt * 32 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3);
             const int n = n0 + (l & 31);
@@ -1265,7 +1272,7 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const int wave_blocks = (tensor_type == 2 ? BmFormat<2>::kWaveBlocks : BmFormat<8>::kWaveBlocks) / 2 * halves;
     int share_blocks = (kb + shares - 1) / shares;
     share_blocks = (share_blocks + wave_blocks - 1) / wave_blocks * wave_blocks;
-    const int real_shares = (kb + share_blocks - 1) / share_blocks;
+    int real_shares = (kb + share_blocks - 1) / share_blocks;
     // Nine to 64 rows (rows of whole 16-byte runs of scales) where the 64-column tiles times the K shares (times two
     // for a pair) make a grid of five eighths of the compute units up to all of them: batch32_mfma_kernel holds one
     // workgroup per unit, and a second round of them costs more than batch_mfma_kernel's two resident workgroups per
@@ -1280,6 +1287,18 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
     const long bound = bound_set >= 0 ? bound_set : gemv_compute_units();
     const long groups32 = static_cast<long>((out_dim + 63) / 64) * real_shares * (weight_b_prepared ? 2 : 1);
     const bool thirty_two = !eight && rows <= 64 && kb % 8 == 0 && groups32 >= gemv_compute_units() * 5 / 8 && groups32 <= bound;
+    // batch_mfma_kernel on a K of one share that more than four of its wavefronts work on, few column tiles (at most
+    // half the compute units' worth, one matrix counted) and no epilogue: two shares of four wavefronts each.  The
+    // kernel adds its wavefronts' sums as (first four) + (last four), so the two shares' sums are exactly those halves
+    // and the result has the same bits as the single share's (which a call with an epilogue keeps: no reduce launch
+    // for it).  Four wavefronts a workgroup on twice the workgroups, sixteen rows: 4096 x 4096 columns 9.8 -> 8.8 us,
+    // 2048 columns 9.3 -> 8.2, 48 rows 14.5 -> 12.8.  (Beyond one workgroup per compute unit it loses: 6144 columns
+    // 10.1 -> 11.8, 8192 columns at 64 rows 15.7 -> 22.4.)
+    if (!eight && !thirty_two && real_shares == 1 && both_plain && kb > (kBmWaves / 2) * wave_blocks &&
+        2 * static_cast<long>((out_dim + 31) / 32) <= gemv_compute_units()) {
+        share_blocks = (kBmWaves / 2) * wave_blocks;
+        real_shares = 2;
+    }
     // Two K shares and nothing to do to the sums but add them: the kernel's shares add to the result themselves
     // (cleared by the quantizer's launch), which saves the reduce launch -- two of them for a pair.
     const bool accumulate = real_shares == 2 && both_plain;
