@@ -115,7 +115,13 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
     static const long forced = v && *v ? std::atol(v) : -1;
     // up to 64 rows everywhere; up to 128 on a Q4_0 matrix wide enough to give every compute unit a
     // column tile (there the tiled GEMM, whose 64 x 128 workgroup tiles re-read X per tile, is slower)
-    const size_t max_rows = tensor_type == AFHIP_TYPE_Q4_0 && (out_dim + 31) / 32 >= static_cast<size_t>(gemv_compute_units()) ? 128 : 64;
+    // ... and where the tiled GEMM's grid of 32 x 64 tiles would not fit the compute units in one round while its
+    // 64 x 128 tiles leave most of them idle (65 .. 128 rows on 4608 .. 8160 columns: 128 rows x 4608 columns 31.5 -> 24.1 us,
+    // 65 rows x 6144 columns 31.0 -> 19.9, 100 rows of K = 8192 x 6144 columns 56.6 -> 43.8; one round of the GEMM stays
+    // faster: 128 rows x 4096 columns 17.8 against 21.2, 96 rows x 5120 columns 17.7 against 20.1)
+    const size_t units = static_cast<size_t>(gemv_compute_units());
+    const bool wide = (out_dim + 31) / 32 >= units || (rows + 31) / 32 * ((out_dim + 63) / 64) > units;
+    const size_t max_rows = tensor_type == AFHIP_TYPE_Q4_0 && wide ? 128 : 64;
     if (forced == 0 || rows > max_rows || !batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
     if (forced > 0) return rows >= static_cast<size_t>(forced);
     if (rows >= kBatchMfmaMinRows && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;

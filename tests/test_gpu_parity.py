@@ -137,6 +137,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     # that ends inside a wavefront's run of blocks, a second K share of one block, ragged columns
     (24, 4096, 544), (25, 2048, 512), (32, 4128, 513), (48, 320, 520), (12, 3072, 1000),
     (70, 512, 8200), (128, 1056, 8192), (97, 256, 8224),  # three and four row tiles (Q4_0 on a wide matrix)
+    (100, 512, 4700), (66, 1024, 6150),  # ... and on a matrix whose tiled-GEMM grid would take a second round
     # the eight-row MFMA kernel (5..8 rows on a grid of at least a workgroup per compute unit): one live
     # wavefront and a ragged last tile; 64-column tiles, ragged; K shares with a short last share; a
     # wavefront with half its blocks
