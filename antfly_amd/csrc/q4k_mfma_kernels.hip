@@ -992,13 +992,14 @@ hipError_t launch_q4k_mfma_rows(hipStream_t stream, float* dst, const float* x, 
     while (slices > kb) slices /= 2;
     static const int env_slices = tuning_int("AFHIP_Q4K_SLICES"), env_tiles = tuning_int("AFHIP_Q4K_TILES_PER_WG");
     if (env_slices >= 1 && env_slices <= max_waves && (env_slices & (env_slices - 1)) == 0 && env_slices <= kb) slices = env_slices;
-    // The int8 kernel at one or two rows on a matrix whose column tiles (of both matrices of a pair) occupy at most half
-    // the compute units, K long enough for a super-block per wavefront of two workgroups, no epilogue: two K shares
-    // (K = 14336 x 4096 columns: 128 tiles, one row 12.7 us on half the chip).
+    // The int8 kernel at one or two rows on a matrix whose column tiles occupy at most half the compute units (one
+    // matrix counted, so that each half of a pair takes the single op's path and has its bits), K long enough for a
+    // super-block per wavefront of two workgroups, no epilogue: two K shares (K = 14336 x 4096 columns: 128 tiles, one
+    // row 12.7 us on half the chip).  A call with an epilogue keeps one share and sums in another order.
     auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
     const bool two_shares = kGroups == 1 && use_i8 && env_slices == 0 && slices == 16 && kb >= 32 && plain(ep) &&
                             (second == nullptr || plain(second->ep)) &&
-                            2 * n_tiles * (second ? 2 : 1) <= gemv_compute_units();
+                            2 * n_tiles <= gemv_compute_units();
     const int sb_per_slice = (kb + (two_shares ? 2 : 1) * slices - 1) / ((two_shares ? 2 : 1) * slices);
     int tiles_per_wg = use_i8 ? 1 : (slices > 8 ? 16 : 8) / slices;  // (the int8 kernel: its wavefronts partition K, nothing else)
     if (!use_i8 && env_tiles >= 1 && env_tiles * slices <= max_waves) tiles_per_wg = env_tiles;
@@ -1209,13 +1210,13 @@ size_t q4k_i8_rows_workspace_bytes(size_t in_dim) {
 }
 
 // Whether launch_gemv_q4k_i8_rows shares K out over two workgroups per column tile, which add to the result arrays: then
-// launch_q4k_digit_planes has to clear them.  Column tiles (of both matrices of a pair) that occupy at most half of the
-// two workgroups a compute unit holds, a super-block per wavefront of both shares, no epilogue.
+// launch_q4k_digit_planes has to clear them.  Column tiles that occupy at most half the compute units (one matrix
+// counted: each half of a pair then has the single op's bits), a super-block per wavefront of both shares, no epilogue.
 bool q4k_i8_rows_two_shares(size_t rows, size_t in_dim, size_t out_dim, bool pair, const Epilogue& ep, const Epilogue& ep_b) {
     auto plain = [](const Epilogue& e) { return e.bias == nullptr && e.residual == nullptr && e.activation == kActNone; };
     if (!q4k_i8_rows_supports(rows, in_dim) || !plain(ep) || (pair && !plain(ep_b))) return false;
     const size_t n_tiles = (out_dim + kTileCols - 1) / kTileCols;
-    return in_dim / kQ4kBlockValues >= 16 && n_tiles * (pair ? 2 : 1) <= static_cast<size_t>(gemv_compute_units());
+    return in_dim / kQ4kBlockValues >= 16 && 2 * n_tiles <= static_cast<size_t>(gemv_compute_units());
 }
 
 hipError_t launch_q4k_digit_planes(hipStream_t stream, const float* x, int rows, int in_dim, void* workspace, float* zero_a,

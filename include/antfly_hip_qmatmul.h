@@ -196,7 +196,10 @@ afhip_status afhip_launch_linear_pair_f32(void *stream, int tensor_type, int lay
  * kernel that writes Y (the engine's `linear`, ops/ops.zig:1728; the CUDA backend's biased
  * launchers, ops/cuda/kernels.zig:339ff and cuda_compute.zig:544-575; the CPU op adds the
  * bias rows after the no-bias product, ops/native_compute.zig:5065-5077 and :5197-5203).
- * Each element is exactly afhip_launch_linear_f32's value plus its bias in f32. */
+ * Each element is exactly afhip_launch_linear_f32's value plus its bias in f32 -- one exception:
+ * Q4_K on a matrix of at most 32 x (compute units / 2) columns with a long K, where the plain op
+ * gives each column tile to two workgroups with half of K each and the biased one keeps one
+ * workgroup a tile: the same products summed in another order (equal within the op's tolerance). */
 afhip_status afhip_launch_linear_bias_f32(void *stream, int tensor_type, int layout, afhip_buffer dst,
                                           afhip_buffer input, afhip_buffer weight, afhip_buffer bias,
                                           size_t rows, size_t in_dim, size_t out_dim,

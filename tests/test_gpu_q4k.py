@@ -258,6 +258,26 @@ def test_digit_plane_rows_pair_and_bias():
     assert np.array_equal(G.linear_bias(Q4K, PREP, x, da, bias, rows, in_dim, out_dim), ya + bias[None, :])
 
 
+@pytest.mark.parametrize("rows,in_dim,out_dim", [(1, 8192, 640), (2, 14336, 300), (5, 4096, 640), (8, 11008, 1000)])
+def test_two_k_shares_pair_and_bias(rows, in_dim, out_dim):
+    """Few column tiles on a long K: the plain op gives each tile to two workgroups with half of K each.  Each half of a
+    pair still equals the single op bit for bit (the rule counts one matrix); a call with a bias keeps one workgroup a
+    tile and sums in another order: the plain value plus the bias within the op's bound."""
+    print(f"case: q4_k two K shares rows={rows} in={in_dim} out={out_dim}", flush=True)
+    wa, wb = synth.weights(Q4K, 197, out_dim, in_dim), synth.weights(Q4K, 198, out_dim, in_dim)
+    x = synth.activations(199, rows, in_dim)
+    da, db = device_weight(PREP, wa, out_dim, in_dim), device_weight(PREP, wb, out_dim, in_dim)
+    ya, yb = G.linear_pair(Q4K, PREP, x, da, db, rows, in_dim, out_dim)
+    assert np.array_equal(ya, G.linear(Q4K, PREP, x, da, rows, in_dim, out_dim))
+    assert np.array_equal(yb, G.linear(Q4K, PREP, x, db, rows, in_dim, out_dim))
+    ref = O.linear_q4_k(x, wa, rows, in_dim, out_dim, f64=True)
+    assert G.max_rel_err(ya, ref) <= TIGHT
+    bias = synth.activations(200, 1, out_dim).reshape(-1)
+    yb_ = G.linear_bias(Q4K, PREP, x, da, bias, rows, in_dim, out_dim)
+    assert G.max_rel_err(yb_ - bias[None, :], ref) <= TIGHT
+    assert G.max_rel_err(yb_, (ya + bias[None, :]).astype(np.float64)) <= TIGHT
+
+
 Q8K_SHAPES = [(1, 2048, 512), (1, 3072, 2048), (2, 3072, 600), (4, 512, 1000), (9, 768, 513), (64, 1536, 512), (77, 2048, 520)]
 
 
