@@ -264,6 +264,74 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(uint8_t* __restrict_
     }
 }
 
+typedef uint32_t stream_u32x4 __attribute__((ext_vector_type(4)));
+
+// The same quantizer for rows of whole 1024-value runs and a 16-byte aligned destination: a workgroup's 32 blocks of an
+// iteration are then 576 (Q8_0: 1088) contiguous bytes of one destination row, starting on a 16-byte boundary.  They are
+// put together in LDS (the 2-byte pieces a lane has to write -- blocks are 18 and 34 bytes long -- cost nothing there)
+// and leave as whole 16-byte stores; the kernel above sends every piece to memory as a 16-bit store.
+template <int kType>
+__global__ __launch_bounds__(256) void quantize_rows_runs_kernel(uint8_t* __restrict__ dst, const float* __restrict__ x,
+                                                                 const long long* __restrict__ ids, size_t rows, int dim,
+                                                                 size_t dst_rows) {
+    constexpr int kRawBytes = kType == 2 ? 18 : 34, kRunBytes = 32 * kRawBytes, kChunks = kRunBytes / 16;
+    constexpr int kRuns = 4;  // runs a workgroup takes per iteration: four loads in flight per thread
+    __shared__ __align__(16) unsigned char image[kRuns * kRunBytes];
+    const size_t kb = static_cast<size_t>(dim >> 5), runs_per_row = kb >> 5;
+    const size_t runs = rows * runs_per_row;  // a run: 32 consecutive blocks of one row
+    const int tid = threadIdx.x, j = tid & 7, bl = tid >> 3;
+    for (size_t run0 = static_cast<size_t>(blockIdx.x) * kRuns; run0 < runs; run0 += static_cast<size_t>(gridDim.x) * kRuns) {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+        float4 v[kRuns];
+#pragma unroll
+        for (int r = 0; r < kRuns; ++r) {
+            const f32x4 in = run0 + r < runs ? __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(x) + (run0 + r) * 256 + tid)
+                                             : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            v[r] = float4{in[0], in[1], in[2], in[3]};
+        }
+#pragma unroll
+        for (int r = 0; r < kRuns; ++r) {
+            float m = fmaxf(fmaxf(fabsf(v[r].x), fabsf(v[r].y)), fmaxf(fabsf(v[r].z), fabsf(v[r].w)));
+            m = max_over_8(m);
+            const float scale = m == 0.0f ? 1.0f : m / (kType == 2 ? 8.0f : 127.0f);
+            const float inv = m == 0.0f ? 0.0f : 1.0f / scale;
+            uint32_t packed;
+            if (kType == 2) {
+                auto nib = [&](float a) {
+                    const float tq = a * inv;
+                    const float rq = tq + __builtin_copysignf(0x1.fffffep-2f, tq);
+                    return static_cast<uint32_t>(min(max(static_cast<int>(rq) + 8, 0), 15));
+                };
+                const uint32_t mine = nib(v[r].x) | (nib(v[r].y) << 8) | (nib(v[r].z) << 16) | (nib(v[r].w) << 24);
+                const uint32_t other = static_cast<uint32_t>(__shfl_xor(static_cast<int>(mine), 4));
+                packed = mine | (other << 4);  // meaningful on lanes j < 4 (other = lane j + 4)
+            } else {
+                const int q0 = act_quant(v[r].x, inv), q1 = act_quant(v[r].y, inv), q2 = act_quant(v[r].z, inv), q3 = act_quant(v[r].w, inv);
+                packed = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | (static_cast<uint32_t>(q3 & 0xFF) << 24);
+            }
+            unsigned char* out = image + r * kRunBytes + bl * kRawBytes;
+            if (j == 0) *reinterpret_cast<uint16_t*>(out) = __builtin_bit_cast(uint16_t, static_cast<_Float16>(scale));
+            if (kType != 2 || j < 4) {
+                uint16_t* q = reinterpret_cast<uint16_t*>(out + 2 + 4 * j);
+                q[0] = static_cast<uint16_t>(packed & 0xFFFF);
+                q[1] = static_cast<uint16_t>(packed >> 16);
+            }
+        }
+        __syncthreads();
+        for (int c = tid; c < kRuns * kChunks; c += 256) {
+            const int r = c / kChunks, piece = c - r * kChunks;
+            const size_t run = run0 + r;
+            if (run >= runs) continue;
+            const size_t t = run / runs_per_row, r32 = run - t * runs_per_row;
+            const long long row = ids ? ids[t] : static_cast<long long>(t);
+            if (row < 0 || static_cast<size_t>(row) >= dst_rows) continue;  // a row id outside the destination writes nothing
+            stream_u32x4* to = reinterpret_cast<stream_u32x4*>(dst + (static_cast<size_t>(row) * kb + r32 * 32) * kRawBytes);
+            __builtin_nontemporal_store(reinterpret_cast<const stream_u32x4*>(image + r * kRunBytes)[piece], to + piece);
+        }
+        __syncthreads();
+    }
+}
+
 __global__ __launch_bounds__(256) void decode_fp16_kernel(float* __restrict__ dst, const uint16_t* __restrict__ src,
                                                           size_t n) {
     const size_t i = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x;
@@ -273,7 +341,6 @@ __global__ __launch_bounds__(256) void decode_fp16_kernel(float* __restrict__ ds
 // Plain streaming read of `n16` 16-byte units (nothing else): the reference
 // point for what one launch of a given size can draw from HBM, and the kernel of
 // known traffic that hardware byte counters are scaled against.
-typedef uint32_t stream_u32x4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(256) void stream_read_kernel(const stream_u32x4* __restrict__ src, uint32_t* __restrict__ sink,
                                                           size_t n16) {
     const size_t i = blockIdx.x * static_cast<size_t>(256) + threadIdx.x;
@@ -560,6 +627,13 @@ hipError_t launch_dequantize_rows(hipStream_t stream, int tensor_type, int layou
 hipError_t launch_quantize_rows(hipStream_t stream, int tensor_type, uint8_t* dst_raw, const float* x, const long long* ids,
                                 size_t rows, int dim, size_t dst_rows) {
     if (rows == 0 || dim == 0) return hipSuccess;
+    if (dim % 1024 == 0 && reinterpret_cast<uintptr_t>(dst_raw) % 16 == 0) {  // whole runs of 32 blocks, aligned: 16-byte stores
+        const size_t groups = (rows * static_cast<size_t>(dim >> 10) + 3) / 4;  // four runs a workgroup and iteration
+        const dim3 run_grid(static_cast<unsigned>(groups < 65536 ? groups : 65536));
+        if (tensor_type == 2) hipLaunchKernelGGL(quantize_rows_runs_kernel<2>, run_grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+        else hipLaunchKernelGGL(quantize_rows_runs_kernel<8>, run_grid, dim3(256), 0, stream, dst_raw, x, ids, rows, dim, dst_rows);
+        return launch_status();
+    }
     const dim3 grid(grid_for(rows * static_cast<size_t>(dim >> 2)));
     const bool narrow = rows * static_cast<size_t>(dim >> 5) <= 0xFFFFFFFFull;
     if (tensor_type == 2) {

@@ -99,7 +99,7 @@ def rows_for_quantizer(seed, rows, dim):
 
 
 @pytest.mark.parametrize("fmt", [Q8, Q4])
-@pytest.mark.parametrize("rows,dim", [(1, 32), (4, 256), (9, 4096)])
+@pytest.mark.parametrize("rows,dim", [(1, 32), (4, 256), (9, 4096), (5, 1024), (7, 3072), (1, 2048)])  # (the last three: a ragged last group of 1024-value runs)
 def test_quantize_rows_matches_weight_quantizers(fmt, rows, dim):
     print(f"case: cpy_f32_to_q fmt={fmt} rows={rows} dim={dim}", flush=True)
     x = rows_for_quantizer(6, rows, dim) if rows * dim >= 256 else synth.activations(6, rows, dim)
@@ -130,6 +130,27 @@ def test_set_rows_scatters_whole_rows(fmt):
         assert np.array_equal(got[r], want[t])
     untouched = [r for r in range(dst_rows) if r not in ids]
     assert (got[untouched] == 0xEE).all()
+
+
+@pytest.mark.parametrize("fmt", [Q8, Q4])
+def test_set_rows_on_whole_runs_aligned_and_not(fmt):
+    """Rows of whole 1024-value runs take the kernel that stores 16 bytes at a time: scattered rows, row ids outside the
+    destination, and a destination that is not 16-byte aligned (which falls back to the piecewise kernel) give the same bytes."""
+    dst_rows, dim = 7, 2048
+    x = rows_for_quantizer(18, 5, dim)
+    ids = np.array([6, -1, 2, dst_rows, 0], dtype=np.int64)
+    row_bytes = dim // 32 * O.BLOCK_BYTES[fmt]
+    want = O.quantize_weights(fmt, x).reshape(5, row_bytes)
+    xd, idd = G.to_dev(x), G.to_dev(ids)
+    for shift in (0, 2):
+        print(f"case: set_rows on runs fmt={fmt} destination offset {shift}", flush=True)
+        canvas = torch.full((16 + (dst_rows + 2) * row_bytes,), 0xC3, dtype=torch.uint8, device=G.DEV)
+        dst = canvas[shift + row_bytes : shift + (dst_rows + 1) * row_bytes]
+        kernels.launchQuantizeRows(G.stream(), fmt, G.buf(dst), G.buf(xd), 5, dim, row_ids_i64=G.buf(idd), dst_rows=dst_rows)
+        torch.cuda.synchronize()
+        got = canvas.cpu().numpy()[shift : shift + (dst_rows + 2) * row_bytes].reshape(dst_rows + 2, row_bytes)
+        assert np.array_equal(got[1 + 6], want[0]) and np.array_equal(got[1 + 2], want[2]) and np.array_equal(got[1 + 0], want[4])
+        assert (got[[0, 2, 4, 5, 6, dst_rows + 1]] == 0xC3).all()  # canaries and the rows nobody addressed
 
 
 def test_quantize_then_dequantize_full_size_properties():
