@@ -1032,7 +1032,10 @@ afhip_status afhip_launch_gemv_probe_rows(void* stream, int probe, size_t rows, 
 afhip_status afhip_launch_gemv_timeline(void* stream, size_t rows, afhip_buffer stamps, afhip_buffer input, afhip_buffer weight,
                                         size_t in_dim, size_t out_dim, size_t* workgroups, size_t* wavefronts_per_workgroup) {
     if (rows != 1 && rows != 2 && rows != 4) return AFHIP_ERR_INVALID_ARGUMENT;
-    if (in_dim == 0 || in_dim % 32 != 0 || in_dim > 4096 || out_dim == 0 || out_dim > 0x7fffffff) return AFHIP_ERR_INVALID_STATE;
+    // (one row also on a K of several slices, as the decode kernel takes it)
+    if (in_dim == 0 || in_dim % 32 != 0 || in_dim > (rows == 1 ? static_cast<size_t>(gemv_fused_max_in_dim()) : 4096) || out_dim == 0 ||
+        out_dim > 0x7fffffff)
+        return AFHIP_ERR_INVALID_STATE;
     const size_t need = afhip_prepared_weight_bytes(AFHIP_TYPE_Q4_0, out_dim, in_dim);
     if (need == 0 || weight.len < need || input.len < rows * in_dim * 4) return AFHIP_ERR_INVALID_STATE;
     if (stamps.ptr == 0 || stamps.ptr % 4 != 0 || input.ptr == 0 || weight.ptr == 0 || input.ptr % 16 != 0 || weight.ptr % 16 != 0)

@@ -462,6 +462,14 @@ __device__ __forceinline__ void gemv_fused_body(
         key = workgroup_max_key(key, reinterpret_cast<unsigned long long*>(partial), tid, waves);
         if (tid == 0) extras.keys[blockIdx.x] = key;
     }
+    if (kProbe & kProbeTimeline) {  // (several K slices: the probe passes no result array, the readings go out here)
+        stamp[3] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
+        if (lane == 0) {
+            uint32_t* o = reinterpret_cast<uint32_t*>(extras.dots) + (static_cast<size_t>(blockIdx.x) * waves + wave) * 8;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) o[k] = stamp[k];
+        }
+    }
 }
 
 template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
@@ -873,6 +881,30 @@ hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, con
     constexpr int kCols = 4;
     const int groups = (out_dim + kCols - 1) / kCols;
     const int x_blocks = kRows * (in_dim / 32);
+    if (in_dim > kSliceBlocks * 32) {
+        // the timeline of a row longer than one K slice: launch_fused's shape for one matrix, the kernel's general
+        // instantiation (K slices side by side in a workgroup, their sums meeting in LDS)
+        if (probe != kProbeTimeline || stamps == nullptr) return hipErrorInvalidValue;
+        const int slices = (in_dim / 32 + kSliceBlocks - 1) / kSliceBlocks;
+        const int waves = workgroup_waves(1024, 1024, slices, groups, false, (x_blocks + 127) / 128);
+        const int groups_per_wg = waves / slices, grid = (groups + groups_per_wg - 1) / groups_per_wg;
+        const bool ready_counter = use_ready_counter(kRows, x_blocks, waves);
+        const size_t lds = gemv_fused_lds_bytes(kRows, in_dim) + (ready_counter ? ready_counter_lds_bytes(x_blocks) : 0);
+        const size_t tile_off = tile_scales_offset(2, static_cast<size_t>(out_dim) * (in_dim / 32));
+        if (grid_out) *grid_out = grid;
+        if (waves_out) *waves_out = waves;
+        if (stamps_bytes < static_cast<size_t>(grid) * waves * 32 || slices > 255 || groups_per_wg > 255) return hipErrorInvalidValue;
+        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, false, kProbeTimeline>;
+        static std::atomic<size_t> long_lds_limit{64 * 1024};
+        if (hipError_t e = allow_large_lds(kernel, lds, &long_lds_limit); e != hipSuccess) return e;
+        const uint32_t shape = static_cast<uint32_t>(slices) | static_cast<uint32_t>(groups_per_wg) << 8 |
+                               (grid <= compute_units() ? 1u << 16 : 0u) | (ready_counter ? kGemvReadyCounter : 0u);
+        const GemvExtras extras{reinterpret_cast<int*>(stamps), nullptr, Epilogue{}, Epilogue{}};
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * slices, groups_per_wg), lds, stream, weight_prepared,
+                           static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),
+                           static_cast<uint32_t>(tile_off >> 4), in_dim / 32, out_dim, shape, extras);
+        return hipGetLastError();
+    }
     const int waves = workgroup_waves(1024, 1024, 1, groups, false, (x_blocks + 127) / 128);
     if (x_blocks > waves * 64) return hipErrorInvalidValue;  // the compact instantiation: one block of X per thread
     const int grid = (groups + waves - 1) / waves;
@@ -907,7 +939,7 @@ hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, con
 hipError_t launch_gemv_probe(hipStream_t stream, int probe, int rows, float* dst, const float* input,
                              const uint8_t* weight_prepared, int in_dim, int out_dim, uint32_t* stamps, size_t stamps_bytes,
                              int* grid_out, int* waves_out) {
-    if (in_dim > kSliceBlocks * 32 || probe < 0 || probe > 8) return hipErrorInvalidValue;
+    if (in_dim > gemv_fused_max_in_dim() || probe < 0 || probe > 8) return hipErrorInvalidValue;
     switch (rows) {
         case 1: return launch_gemv_probe_rows<1>(stream, probe, dst, input, weight_prepared, in_dim, out_dim, stamps, stamps_bytes, grid_out, waves_out);
         case 2: return launch_gemv_probe_rows<2>(stream, probe, dst, input, weight_prepared, in_dim, out_dim, stamps, stamps_bytes, grid_out, waves_out);

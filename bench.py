@@ -113,7 +113,7 @@ def main() -> int:
                     help="timeline8: the same for the eight-row MFMA kernel (afhip_launch_rows8_timeline; --probe-rows 5 or 8): when a wavefront's weight stages are there, when its K loop ends; timeline: the Q4_0 decode kernel's wavefronts read the 100 MHz clock at their phases (afhip_launch_gemv_timeline; --probe-rows 1, 2 or 4): when the quantized activations are ready, when a wavefront's block dots are done; read: a kernel that only reads the headline matrix's 33 MB, swept over workgroup size, loads in flight per lane and load hint (afhip_launch_stream_read_shaped); gemm: the Q8_0 M=512 prefill kernel's own clock readings (afhip_launch_gemm_stamps): cycles in the K loop, waiting for loads and at barriers, and the clock the chip held; rates: instruction issue rates of a SIMD (afhip_launch_rate_probe), print a table, exit; gemv: time the one-row Q4_0 decode kernel with parts left out (afhip_launch_gemv_probe) next to "
                          "a kernel that only reads the same bytes, print a table, exit")
     ap.add_argument("--probe-shape", default="4096:14336",
-                    help="--probe timeline: K:N of the matrix, K at most 4096 (default: the headline's 4096:14336)")
+                    help="--probe timeline: K:N of the matrix, K at most 4096 (one row: 16384; default: the headline's 4096:14336)")
     ap.add_argument("--probe-rows", type=int, choices=[1, 2, 4, 5, 8], default=1,
                     help="--probe gemv: rows of X (the decode kernel's instantiation for that many rows)")
     args = ap.parse_args()

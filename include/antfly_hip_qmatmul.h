@@ -631,7 +631,9 @@ afhip_status afhip_launch_gemv_probe_rows(void *stream, int probe, size_t rows, 
  * activations (a barrier, or for several rows a counter in LDS), [2] block dots done, [3] wavefront reduction done; the
  * quantizing wavefronts of a counter launch also [4] past the barrier behind their requests for X, [5] X arrived,
  * [6] their blocks quantized.  The launch geometry comes back through the two pointers; `stamps` too small for it
- * (32 bytes per wavefront) is refused.  `bench.py --probe timeline` prints the table. */
+ * (32 bytes per wavefront) is refused.  in_dim up to 4096; one row up to 16384 (several K slices side by side in a
+ * workgroup, as the decode kernel takes such a row: [3] is then read behind the slices' sums).
+ * `bench.py --probe timeline [--probe-shape K:N]` prints the table. */
 afhip_status afhip_launch_gemv_timeline(void *stream, size_t rows, afhip_buffer stamps, afhip_buffer input,
                                         afhip_buffer weight_prepared, size_t in_dim, size_t out_dim, size_t *workgroups,
                                         size_t *wavefronts_per_workgroup);
