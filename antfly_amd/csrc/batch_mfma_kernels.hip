@@ -1231,14 +1231,19 @@ bool batch_mfma_supports(int tensor_type, size_t rows, size_t in_dim, size_t out
 // 35.0 -> 27.1, 4096 x 4096 8.7 -> 8.9, K = 2048 x 8192 columns 8.3 -> 8.8.  Q4_0, whose 32-row kernels are better (half
 // the bytes per block, the same MFMA time), loses with two groups -- 14336 columns 13.3 -> 14.6, K = N = 8192
 // 13.8 -> 14.7, 128256 columns 74 -> 84; 4096 columns 9.8 -> 9.2 and K = 14336 x 4096 16.8 -> 15.8 are the only gains --
-// and keeps one: a step's MFMAs of two groups (2 x (16 + 32) cycles a SIMD) take as long as its bytes.
+// and keeps one there: a step's MFMAs of two groups (2 x (16 + 32) cycles a SIMD) take as long as its bytes.  On a K
+// beyond 8192 and up to 8192 columns Q4_0 takes two groups too -- there the other kernels need three and more K shares
+// and a reduce launch, this one two shares that add to the result themselves: sixteen rows, K = 14336 x 4096 columns
+// 17.0 -> 15.9 us, 6144 columns 22.7 -> 19.3, 8192 columns 26.5 -> 22.7, a pair of 4096 columns 29.1 -> 22.8, K = 11008
+// x 4096 15.9 -> 15.4, K = 28672 x 4096 27.2 -> 26.2 (14336 x 14336 columns loses: 39.3 -> 41.0).
 // (It used to be kept to grids
 // of at least a workgroup per compute unit; with its tiles sized to the matrix and its first requests in order it also
 // wins below that: five rows, K = 4096, against batch_mfma_kernel: 6144 columns 8.5 against 9.6 us, 3072 6.8 against
 // 9.0, 1024 6.6 against 8.7.)
 bool batch_mfma_eight_rows(int tensor_type, size_t rows, size_t in_dim, size_t out_dim) {
     if (!batch_mfma_supports(tensor_type, rows, in_dim, out_dim)) return false;
-    return rows <= (tensor_type == 8 ? 16 : 8) && (in_dim / 32) % 8 == 0;
+    const bool sixteen = tensor_type == 8 || (in_dim > 8192 && out_dim <= 8192);
+    return rows <= (sixteen ? 16u : 8u) && (in_dim / 32) % 8 == 0;
 }
 
 // Workspace: [qa: 32 * row_tiles * in_dim bytes][sa: (in_dim / 32) * 32 * row_tiles floats][partial sums of K shares, for two matrices]
@@ -1342,7 +1347,8 @@ hipError_t launch_batch_mfma(hipStream_t stream, int tensor_type, float* dst, co
 #define AFHIP_BM8(T, CG, H, G) bm_launch8<T, CG, H, G>(stream, dst, partial, qa, sa, weight_prepared, rows, in_dim, out_dim, real_shares, share_blocks, cols, accumulate, ep, second)
 #define AFHIP_BM8_CG(T, H, G) (cg == 4 ? AFHIP_BM8(T, 4, H, G) : (cg == 3 ? AFHIP_BM8(T, 3, H, G) : (cg == 2 ? AFHIP_BM8(T, 2, H, G) : AFHIP_BM8(T, 1, H, G))))
 #define AFHIP_BM8_G(T, H) (groups == 2 ? AFHIP_BM8_CG(T, H, 2) : AFHIP_BM8_CG(T, H, 1))
-        if (tensor_type == 2) e = halves == 4 ? AFHIP_BM8_CG(2, 4, 1) : AFHIP_BM8_CG(2, 2, 1);  // (Q4_0: one group of rows only)
+        // (Q4_0: two groups of rows only on a long K, which runs four stage rounds)
+        if (tensor_type == 2) e = halves == 4 ? AFHIP_BM8_G(2, 4) : AFHIP_BM8_CG(2, 2, 1);
         else e = halves == 8 ? AFHIP_BM8_G(8, 8) : (halves == 4 ? AFHIP_BM8_G(8, 4) : AFHIP_BM8_G(8, 2));
 #undef AFHIP_BM8_G
 #undef AFHIP_BM8_CG

@@ -26,7 +26,8 @@ SHAPES = [(1, 4096, 1024), (1, 512, 514), (2, 2048, 640), (4, 1024, 600), (5, 82
           (20, 2048, 300), (33, 8224, 200),  # MFMA GEMM with K shared out over workgroups: the reduce kernel adds the bias
           (7, 512, 8200), (5, 9216, 4112),  # the eight-row MFMA kernel; with K shares (the reduce kernel adds the bias)
           (18, 512, 12290),
-          (12, 4096, 520), (40, 3072, 300)]  # one K share that the plain op runs as two shares of four wavefronts each: the same bits  # the 32-row MFMA kernel on 64-column tiles
+          (12, 4096, 520), (40, 3072, 300),
+          (12, 9216, 300)]  # Q4_0 too as two groups of eight rows (long K): two K shares, the reduce kernel adds the bias  # one K share that the plain op runs as two shares of four wavefronts each: the same bits  # the 32-row MFMA kernel on 64-column tiles
 
 
 def bias_vector(seed, out_dim):

@@ -226,6 +226,7 @@ PAIR_SHAPES = [  # rows, in_dim, out_dim: fused GEMV, small-batch GEMV with K sl
     (6, 512, 8200), (7, 9216, 4112),  # the eight-row MFMA kernel, one launch over both matrices; with K shares
     (20, 512, 12290),                 # the 32-row MFMA kernel on 64-column tiles, both matrices
     (4, 512, 8200), (3, 256, 16500),  # four and three rows whose two matrices together exceed one (two) rounds of the decode kernel
+    (12, 9216, 520),                  # the eight-row kernel on two groups of eight rows (Q8_0; Q4_0 on a long K), both matrices
 ]
 
 
