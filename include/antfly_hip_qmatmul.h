@@ -149,7 +149,10 @@ int afhip_uses_q8k_activation_quant(int tensor_type, size_t rows, size_t in_dim,
  * Kernel launchers: ops/cuda/kernels.zig:1221-1289 (launchLinearQ8_0F32 /
  * launchLinearQ4_0F32).  Same checks: in_dim must be a non-zero multiple of 32
  * and every buffer long enough, else AFHIP_ERR_INVALID_STATE; rows*out_dim == 0
- * is a successful no-op.
+ * is a successful no-op.  The result buffers must not overlap the activations, the
+ * weights, the workspace or each other (every workgroup reads all of X while others
+ * already write Y, and some launches clear Y before they read X), as in the
+ * reference, whose launchers write a freshly allocated output.
  * ---------------------------------------------------------------------- */
 
 /* Bytes of device scratch a launch needs (quantized activations for the
