@@ -75,7 +75,7 @@ struct GemvTargets {
 //               wavefronts of a counter launch also [4] past the barrier behind the requests for X, [5] X there,
 //               [6] blocks quantized
 constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4, kProbeTimeline = 8;
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, bool kDefer = false>
 __device__ __forceinline__ void gemv_fused_body(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
@@ -217,7 +217,7 @@ __device__ __forceinline__ void gemv_fused_body(
             asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
             if (kProbe & kProbeTimeline) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
             __builtin_amdgcn_sched_barrier(0);
-            request_weights();
+            if (!kDefer) request_weights();
             __builtin_amdgcn_sched_barrier(0);
             const f32x4* stage = reinterpret_cast<const f32x4*>(lds + stage_byte);
             float4 v[8];
@@ -267,6 +267,14 @@ __device__ __forceinline__ void gemv_fused_body(
             // wait for the wavefront's own weight requests to complete before the counter moves.
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
             if (lane == 0) __hip_atomic_fetch_add(ready, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            // With two quantizers to a SIMD on a launch that streams for microseconds, a quantizer asks for its weights
+            // only now: a request is through when the memory pipeline has accepted it, and right after the barrier that
+            // pipeline is taking the requests of all sixteen wavefronts -- a quantizer that joined the queue first began to
+            // quantize up to a microsecond late, and every wavefront waits for the last quantizer.  Its own weights come
+            // later this way, but the quantizers were the first to finish by a wide margin.  (kDefer: an instantiation of
+            // its own, chosen by the host -- a flag tested here cost the launches that do not defer 3 %.)
+            __builtin_amdgcn_sched_barrier(0);
+            if (kDefer) request_weights();
         }
 
 
@@ -472,12 +480,12 @@ __device__ __forceinline__ void gemv_fused_body(
     }
 }
 
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0>
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, bool kDefer = false>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
     GemvExtras extras) {
-    gemv_fused_body<kType, kRows, kCols, kWriteDots, kArgmax, kCompact, kProbe>(weight_a, weight_b, input, dst_a, dst_b, tile_off16,
+    gemv_fused_body<kType, kRows, kCols, kWriteDots, kArgmax, kCompact, kProbe, kDefer>(weight_a, weight_b, input, dst_a, dst_b, tile_off16,
                                                                                  kb, out_dim, shape, extras);
 }
 
@@ -764,6 +772,18 @@ hipError_t allow_large_lds(Kernel kernel, size_t lds, std::atomic<size_t>* limit
 bool use_ready_counter(int rows, int x_blocks, int waves) {
     return waves > (x_blocks + 63) / 64 && (rows >= 2 || x_blocks >= 192);
 }
+// Whether the quantizing wavefronts of a counter launch ask for their weights behind their quantization (see the kernel):
+// where two of them share a SIMD (eight and more; Q8_0, whose wavefronts request twice the bytes, from six on) and the
+// launch streams at least 24 MB of weights.  Measured (us, before -> after): Q4_0 four rows x 14336 columns 9.65 -> 9.0,
+// two rows K = 11008 x 4096 columns 8.4 -> 7.8, Q8_0 three rows x 14336 columns 14.2 -> 13.45; below those bounds it
+// costs: three rows (six quantizers) 8.6 -> 9.0, four rows x 4096 columns 6.0 -> 6.2, one row of 14336 values 7.75 -> 8.1.
+bool defer_quantizer_weights(int tensor_type, bool ready_counter, int x_blocks, int waves, int in_dim, int out_dim, bool pair) {
+    if (!ready_counter) return false;
+    const int quantizers = std::min(waves, (x_blocks + 63) / 64);
+    const double bytes = static_cast<double>(out_dim) * (pair ? 2 : 1) * (in_dim / 32) * (tensor_type == 2 ? 18 : 34);
+    return quantizers >= (tensor_type == 8 ? 6 : 8) && bytes >= 24.0e6;
+}
+
 // LDS behind the fused kernel's own: 16 bytes of counter, the f32 staging of X (8 KB per quantizing wavefront), alignment
 size_t ready_counter_lds_bytes(int x_blocks) { return 32 + static_cast<size_t>((x_blocks + 63) / 64) * 8192; }
 
@@ -791,8 +811,15 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     const bool compact = slices == 1 && tg.weight_b == nullptr && x_blocks <= waves * 64;
     auto kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true>
                           : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false>;
-    static std::atomic<size_t> lds_limit[2] = {{64 * 1024}, {64 * 1024}};
-    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[compact ? 1 : 0]); e != hipSuccess) return e;
+    bool defer = false;
+    if constexpr (kRows >= 2 && !kDots && !kArgmax) {  // (the instantiations that request a quantizer's weights late)
+        defer = defer_quantizer_weights(kType, ready_counter, x_blocks, waves, in_dim, out_dim, tg.weight_b != nullptr);
+        if (defer)
+            kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true, 0, true>
+                             : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false, 0, true>;
+    }
+    static std::atomic<size_t> lds_limit[4] = {{64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
+    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[(compact ? 1 : 0) + (defer ? 2 : 0)]); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     if (key_count) *key_count = grid;
     // one round of workgroups: the wavefronts of a unit enter its load queue one after the other
@@ -873,7 +900,9 @@ hipError_t launch_gemv_fused(hipStream_t stream, int tensor_type, float* dst, in
     return launch_gemv_type<8>(stream, tg, dots, input, pre, rows, in_dim, out_dim, tune);
 }
 
-// Timing diagnostics on the Q4_0 decode kernel for one, two and four rows (compact instantiation: in_dim <= 4096).
+// Timing diagnostics on the Q4_0 decode kernel for one, two and four rows (compact instantiation: in_dim <= 4096; at
+// four rows the one whose quantizing wavefronts request their weights late, which launch_fused picks on a launch of
+// 24 MB of weights and more -- the probe's matrix).
 namespace {
 template <int kRows>
 hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, const float* input, const uint8_t* weight_prepared,
@@ -921,7 +950,7 @@ hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, con
                                                {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
 #define AFHIP_PROBE(P)                                                                                                  \
     case P: {                                                                                                           \
-        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, true, P>;                                        \
+        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, true, P, kRows >= 4>;                            \
         if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[P]); e != hipSuccess) return e;                      \
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(64, waves), lds, stream, weight_prepared,                           \
                            static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),              \
