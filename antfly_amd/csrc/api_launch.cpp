@@ -130,9 +130,13 @@ static bool batch_mfma_preferred(int tensor_type, size_t rows, size_t in_dim, si
     // and columns, the eight-row kernel's time does not.  Four rows: a pair of 14336 columns 18.3 -> 16.7 us, 28672
     // columns 18.5 -> 16.9, 128256 columns 64.6 -> 50.8 (three rows 55.9 -> 49.8); on one round the decode kernel wins
     // (14336 columns 9.9 against 10.9, a pair of 8192 10.2 against 11.3), and three rows on two rounds are even.
+    // (Four rows of 4096 values -- eight quantizing wavefronts, which then request their weights behind their
+    // quantization -- hold out for two rounds as well: 20480 columns 13.3 against 16.1, a pair of 11008 14.0 against 15.1,
+    // 28672 columns 16.5 against 17.0; 128256 columns 65.3 against 52.1.)
     if (tensor_type == AFHIP_TYPE_Q4_0 && in_dim <= 4096 && (rows == 3 || rows == 4)) {
         const size_t round = static_cast<size_t>(gemv_compute_units()) * 64, columns = out_dim * (pair ? 2 : 1);
-        if (columns > (rows == 4 ? round : 2 * round) && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
+        const size_t rounds = rows == 4 && rows * in_dim < 16384 ? 1 : 2;
+        if (columns > rounds * round && batch_mfma_eight_rows(tensor_type, rows, in_dim, out_dim)) return true;
     }
     // Q8_0, K of 2048 to 4096 (one K share of the eight-row kernel in one round on a wide matrix): four rows from 11008
     // columns on (11008 14.2 -> 12.3 us, 14336 16.0 -> 14.4, 28672 29.1 -> 23.8, a pair of 14336 30.1 -> 23.2; 8192 9.3

@@ -187,7 +187,7 @@ afhip_status afhip_launch_linear_f32_static(void *stream, int tensor_type, int l
  * ops/native_compute.zig:6262-6307): Ya = X * Wa^T, Yb = X * Wb^T.  Each result is
  * bit for bit what afhip_launch_linear_f32 gives for that matrix wherever the pair and the
  * single call take the same kernel -- everywhere but three and four rows of Q4_0 with
- * in_dim <= 4096 whose two matrices together exceed one (three rows: two) rounds of the decode
+ * in_dim <= 4096 whose two matrices together exceed two (four rows of fewer than 4096 values: one) rounds of the decode
  * kernel's workgroups while one of them does not: there the same block dots are summed in
  * another order (equal within the op's tolerance).  X is quantized once, and up to 8 rows
  * (Q8_0: 16) both matrices are served by one kernel launch. */

@@ -149,7 +149,7 @@ SHAPES_A = [  # (rows, in_dim, out_dim): all take the activation-quantized route
     (8, 512, 14336), (6, 1024, 11008), (5, 256, 10000), (7, 2048, 6144), (8, 256, 9000),
     (5, 8192, 7168),  # ... 56 columns with two K shares (Q4_0)
     # three and four rows on more columns than one round of the decode kernel's workgroups: Q4_0 takes the eight-row kernel
-    (4, 256, 16448), (3, 256, 33000), (4, 4096, 28672),
+    (4, 256, 16448), (3, 256, 33000), (4, 4096, 28672), (4, 4096, 33000),  # (four rows of 4096 values: from two rounds on)
     (3, 2048, 14400), (4, 2048, 11040),  # ... and Q8_0 on wide matrices with K of 2048 to 4096
     # nine to 32 rows on 64-column tiles: every count of live result registers, ragged columns, one live
     # wavefront with half its blocks, K shares with a short last share
@@ -248,7 +248,7 @@ def test_pair_equals_two_single_ops(fmt, layout, rows, in_dim, out_dim):
     # Three and four rows of Q4_0: the pair's two matrices together may exceed one (two) rounds of the decode kernel's
     # workgroups (64 columns a compute unit, 256 units) where one matrix does not; the pair then runs on the eight-row
     # MFMA kernel and a single op on the decode kernel -- the same block dots, another f32 summation order.
-    one_round = 256 * 64 * (1 if rows == 4 else 2)
+    one_round = 256 * 64 * (1 if rows == 4 and rows * in_dim < 16384 else 2)
     routes_differ = (fmt == Q4 and layout == PREP and rows in (3, 4) and in_dim <= 4096 and in_dim % 256 == 0 and
                      out_dim <= one_round < 2 * out_dim)
     if routes_differ:
