@@ -75,7 +75,7 @@ struct GemvTargets {
 //               wavefronts of a counter launch also [4] past the barrier behind the requests for X, [5] X there,
 //               [6] blocks quantized
 constexpr int kProbeNoDots = 1, kProbeNoStore = 2, kProbeNoPrologue = 4, kProbeTimeline = 8;
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, bool kDefer = false>
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, int kDefer = 0>
 __device__ __forceinline__ void gemv_fused_body(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
@@ -217,7 +217,7 @@ __device__ __forceinline__ void gemv_fused_body(
             asm volatile("s_waitcnt vmcnt(0)" : : : "memory");
             if (kProbe & kProbeTimeline) stamp[5] = static_cast<uint32_t>(__builtin_amdgcn_s_memrealtime());
             __builtin_amdgcn_sched_barrier(0);
-            if (!kDefer) request_weights();
+            if (kDefer == 0 || (kDefer == 1 && wave < 4)) request_weights();
             __builtin_amdgcn_sched_barrier(0);
             const f32x4* stage = reinterpret_cast<const f32x4*>(lds + stage_byte);
             float4 v[8];
@@ -272,9 +272,10 @@ __device__ __forceinline__ void gemv_fused_body(
             // pipeline is taking the requests of all sixteen wavefronts -- a quantizer that joined the queue first began to
             // quantize up to a microsecond late, and every wavefront waits for the last quantizer.  Its own weights come
             // later this way, but the quantizers were the first to finish by a wide margin.  (kDefer: an instantiation of
-            // its own, chosen by the host -- a flag tested here cost the launches that do not defer 3 %.)
+            // its own, chosen by the host -- a flag tested here cost the launches that do not defer 3 %.  kDefer = 2: all
+            // quantizers; 1, for five to seven of them: only those that are a SIMD's second one, wavefronts 4 and up.)
             __builtin_amdgcn_sched_barrier(0);
-            if (kDefer) request_weights();
+            if (kDefer == 2 || (kDefer == 1 && wave >= 4)) request_weights();
         }
 
 
@@ -480,7 +481,7 @@ __device__ __forceinline__ void gemv_fused_body(
     }
 }
 
-template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, bool kDefer = false>
+template <int kType, int kRows, int kCols, bool kWriteDots, bool kArgmax = false, bool kCompact = false, int kProbe = 0, int kDefer = 0>
 __global__ __launch_bounds__(1024) void gemv_fused_kernel(
     const uint8_t* __restrict__ weight_a, const uint8_t* __restrict__ weight_b, const float* __restrict__ input,
     float* __restrict__ dst_a, float* __restrict__ dst_b, uint32_t tile_off16, int kb, int out_dim, uint32_t shape,
@@ -777,11 +778,16 @@ bool use_ready_counter(int rows, int x_blocks, int waves) {
 // launch streams at least 24 MB of weights.  Measured (us, before -> after): Q4_0 four rows x 14336 columns 9.65 -> 9.0,
 // two rows K = 11008 x 4096 columns 8.4 -> 7.8, Q8_0 three rows x 14336 columns 14.2 -> 13.45; below those bounds it
 // costs: three rows (six quantizers) 8.6 -> 9.0, four rows x 4096 columns 6.0 -> 6.2, one row of 14336 values 7.75 -> 8.1.
-bool defer_quantizer_weights(int tensor_type, bool ready_counter, int x_blocks, int waves, int in_dim, int out_dim, bool pair) {
-    if (!ready_counter) return false;
+// 0: nobody; 1: a SIMD's second quantizer (wavefronts 4 and up) -- five to seven quantizers of Q4_0: three rows x 11008
+// columns 7.7 -> 7.15, 28672 columns 16.65 -> 15.9, a pair of 14336 16.9 -> 15.3, 14336 columns 8.7 -> 8.6 (all of them
+// late: 8.6 -> 9.0); 2: all quantizers.
+int defer_quantizer_weights(int tensor_type, bool ready_counter, int x_blocks, int waves, int in_dim, int out_dim, bool pair) {
+    if (!ready_counter) return 0;
     const int quantizers = std::min(waves, (x_blocks + 63) / 64);
     const double bytes = static_cast<double>(out_dim) * (pair ? 2 : 1) * (in_dim / 32) * (tensor_type == 2 ? 18 : 34);
-    return quantizers >= (tensor_type == 8 ? 6 : 8) && bytes >= 24.0e6;
+    if (bytes < 24.0e6) return 0;
+    if (quantizers >= (tensor_type == 8 ? 6 : 8)) return 2;
+    return tensor_type == 2 && quantizers >= 5 ? 1 : 0;
 }
 
 // LDS behind the fused kernel's own: 16 bytes of counter, the f32 staging of X (8 KB per quantizing wavefront), alignment
@@ -811,15 +817,20 @@ hipError_t launch_fused(hipStream_t stream, const GemvTargets& tg0, int* dots, c
     const bool compact = slices == 1 && tg.weight_b == nullptr && x_blocks <= waves * 64;
     auto kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true>
                           : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false>;
-    bool defer = false;
+    int defer = 0;
     if constexpr (kRows >= 2 && !kDots && !kArgmax) {  // (the instantiations that request a quantizer's weights late)
         defer = defer_quantizer_weights(kType, ready_counter, x_blocks, waves, in_dim, out_dim, tg.weight_b != nullptr);
-        if (defer)
-            kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true, 0, true>
-                             : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false, 0, true>;
+        if (defer == 2)
+            kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true, 0, 2>
+                             : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false, 0, 2>;
+        if constexpr (kType == 2) {
+            if (defer == 1)
+                kernel = compact ? gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, true, 0, 1>
+                                 : gemv_fused_kernel<kType, kRows, kCols, kDots, kArgmax, false, 0, 1>;
+        }
     }
-    static std::atomic<size_t> lds_limit[4] = {{64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
-    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[(compact ? 1 : 0) + (defer ? 2 : 0)]); e != hipSuccess) return e;
+    static std::atomic<size_t> lds_limit[6] = {{64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
+    if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[(compact ? 1 : 0) + 2 * defer]); e != hipSuccess) return e;
     const int grid = (groups + groups_per_wg - 1) / groups_per_wg;
     if (key_count) *key_count = grid;
     // one round of workgroups: the wavefronts of a unit enter its load queue one after the other
@@ -950,7 +961,7 @@ hipError_t launch_gemv_probe_rows(hipStream_t stream, int probe, float* dst, con
                                                {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}, {64 * 1024}};
 #define AFHIP_PROBE(P)                                                                                                  \
     case P: {                                                                                                           \
-        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, true, P, kRows >= 4>;                            \
+        auto kernel = gemv_fused_kernel<2, kRows, kCols, false, false, true, P, (kRows >= 4 ? 2 : 0)>;                  \
         if (hipError_t e = allow_large_lds(kernel, lds, &lds_limit[P]); e != hipSuccess) return e;                      \
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(64, waves), lds, stream, weight_prepared,                           \
                            static_cast<const uint8_t*>(nullptr), input, dst, static_cast<float*>(nullptr),              \
